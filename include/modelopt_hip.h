@@ -1,0 +1,114 @@
+/*
+ * modelopt_hip.h -- C ABI of libmodelopt_hip.so: gfx950 (MI355X) kernels for the ModelOpt
+ * quantization hot path.
+ *
+ * Contract shared by every entry point:
+ *   - plain C linkage, raw device pointers, sizes and enums only (no torch / C++ types);
+ *   - the caller owns every buffer (inputs, outputs, accumulators); nothing is allocated,
+ *     freed or synchronised inside the library; work is enqueued on `stream`
+ *     (a hipStream_t passed as void*, NULL = the default stream) and is stream ordered;
+ *   - return value 0 on success, a negative MO_ERR_* code otherwise (no exceptions cross the
+ *     ABI); mo_error_string() names a code;
+ *   - tensors are contiguous row-major; `dtype` selects the element type of x / y.
+ *
+ * Each function cites the reference interface it replaces (paths relative to the reference
+ * checkout; TQ = modelopt/torch/quantization).
+ */
+#ifndef MODELOPT_HIP_H_
+#define MODELOPT_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum mo_dtype { MO_F32 = 0, MO_F16 = 1, MO_BF16 = 2 };
+
+enum mo_status {
+    MO_OK = 0,
+    MO_ERR_ARG = -1,      /* null pointer, negative size, inconsistent shape */
+    MO_ERR_DTYPE = -2,    /* unsupported element type */
+    MO_ERR_UNSUPPORTED = -3, /* valid request the kernels do not cover (e.g. block size) */
+    MO_ERR_LAUNCH = -4    /* the HIP runtime rejected the launch */
+};
+
+int mo_version(void);
+const char* mo_error_string(int status);
+
+/* ------------------------------------------------------------------ abs-max reductions
+ * Replaces reduce_amax (TQ/utils.py:156-188) as used by MaxCalibrator.collect
+ * (TQ/calib/max.py:53-94) and TensorQuantizer._get_amax (TQ/nn/modules/tensor_quantizer.py
+ * :505-514).
+ *
+ * x is viewed as [outer, axis, inner]; acc[a] = max(acc[a], max over (o, i) of |x[o, a, i]|).
+ * acc holds fp32 values that must be non-negative (or NaN) on entry -- zero for a fresh
+ * reduction, the running maximum for a calibrator.  NaN inputs make the result NaN, as
+ * torch.max does.  Per-tensor: outer = 1, axis = 1, inner = numel.
+ */
+int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
+              float* acc, void* stream);
+
+/* ------------------------------------------------------------------ fake quantisation
+ * x and y are viewed as [outer, axis, inner]; amax has `axis` elements of type amax_dtype
+ * (axis = 1: per tensor).  y may alias x.
+ */
+
+/* FP8 E4M3 quantize-dequantize.  Replaces fake_e4m3fy / fake_e4m3fy_with_axis
+ * (TQ/src/tensor_quant_gpu_fp8.cu:66-108) with the numerics of the CPU path _fp8_eager
+ * (TQ/tensor_quant.py:45-59): scale = 448 / f32(amax), inv = 1 / scale,
+ * y = T(f32(e4m3_rne(f32(x) * scale)) * inv); amax == NULL is a plain cast.
+ * saturate = 0: magnitudes that round above 448 become NaN (CPU torch cast);
+ * saturate = 1: they clamp to 448 (the reference's CUDA kernel). */
+int mo_fp8_qdq(const void* x, void* y, int64_t outer, int64_t axis, int64_t inner, int dtype,
+               const void* amax, int amax_dtype, int saturate, void* stream);
+
+/* Integer quantize-dequantize.  Replaces fake_tensor_quant / fake_tensor_quant_with_axis
+ * (TQ/src/tensor_quant_gpu.cu:43-143) with the numerics of _tensor_quant
+ * (TQ/tensor_quant.py:574-612): bound = 2^(bits-1+unsigned)-1, scale = bound / f32(amax),
+ * amax <= 2^-24 gives 0, y = T(clamp(rne(f32(x) * scale), lo, bound) / scale). */
+int mo_int_qdq(const void* x, void* y, int64_t outer, int64_t axis, int64_t inner, int dtype,
+               const void* amax, int amax_dtype, int num_bits, int is_unsigned,
+               int narrow_range, void* stream);
+
+/* NVFP4 dynamic-block quantize-dequantize of x[rows, k] with blocks of `block_size` (8, 16 or
+ * 32) along k (zero padded).  Replaces fp4_fake_quant_block (TQ/triton/fp4_kernel.py:141-208)
+ * and fused_amax_convert for (E2M1, E4M3) (TQ/src/tensor_quant_mx.cu:355).
+ * amax: 1-element global amax.
+ * mode 0: the threshold-ladder formula of TQ/triton/fp4_kernel.py:86-134 (448 clamp of the
+ *         block scale, scale < 1e-5 -> 1, sign from x >= 0);
+ * mode 1: identical to NVFP4QTensor.quantize followed by dequantize
+ *         (TQ/qtensor/nvfp4_tensor.py:143-297), the reference's CPU path. */
+int mo_nvfp4_qdq(const void* x, void* y, int64_t rows, int64_t k, int dtype, const void* amax,
+                 int amax_dtype, int block_size, int mode, void* stream);
+
+/* ------------------------------------------------------------------ real quantize + pack */
+
+/* NVFP4 quantize + pack.  Replaces NVFP4QTensor.quantize and get_weights_scaling_factor
+ * (TQ/qtensor/nvfp4_tensor.py:63-92,143-232) as called by to_quantized_weight
+ * (modelopt/torch/export/quant_utils.py:822-834) and TensorQuantizer._real_quantize
+ * (TQ/nn/modules/tensor_quantizer.py:610-622).
+ * x[rows, k]; kp = k rounded up to a multiple of block_size (zero padded).
+ * amax: device fp32 scalar, the global abs-max of x (amax_is_wsf2 = 0) or the already divided
+ *       global scale wsf2 (amax_is_wsf2 = 1); wsf2 = f32(amax) / (6 * 448).
+ * wsf_in: optional [rows, kp / block_size] E4M3 block scales to use instead of computing
+ *       them (NULL to compute).
+ * Outputs: packed[rows, kp / 2] (byte i = code[2i] | code[2i+1] << 4, code = sign << 3 |
+ * ordinal), wsf_out[rows, kp / block_size] E4M3 bytes (may be NULL when wsf_in is given),
+ * wsf2_out (fp32 scalar, may be NULL). */
+int mo_nvfp4_quantize(const void* x, int64_t rows, int64_t k, int dtype, int block_size,
+                      const float* amax, int amax_is_wsf2, const uint8_t* wsf_in,
+                      uint8_t* packed, uint8_t* wsf_out, float* wsf2_out, void* stream);
+
+/* NVFP4 unpack + rescale.  Replaces NVFP4QTensor.dequantize (TQ/qtensor/nvfp4_tensor.py
+ * :234-297) and fp4_dequantize (TQ/triton/fp4_kernel.py:307):
+ * y[rows, kp] = T(LUT[code] * (f32(wsf) * wsf2)). */
+int mo_nvfp4_dequantize(const uint8_t* packed, const uint8_t* wsf, const float* wsf2,
+                        int64_t rows, int64_t kp, int block_size, void* y, int dtype,
+                        void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MODELOPT_HIP_H_ */

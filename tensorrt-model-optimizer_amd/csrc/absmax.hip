@@ -1,0 +1,259 @@
+// Abs-max reductions (per tensor, per channel, per block) for gfx950.
+//
+// HBM-bound: 2 bytes (bf16/fp16) or 4 bytes (fp32) read per element, nothing written but the
+// accumulator.  All variants fold |x| with integer max on the abs bit pattern so NaN
+// propagates, and finish with one atomicMax per (row worker | column | block) into the fp32
+// accumulator the caller owns.
+#include "common.h"
+
+namespace mo {
+
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    u16x2 x, y;
+    __builtin_memcpy(&x, &a, 4);
+    __builtin_memcpy(&y, &b, 4);
+    u16x2 r = __builtin_elementwise_max(x, y);
+    uint32_t o;
+    __builtin_memcpy(&o, &r, 4);
+    return o;
+}
+
+// Running max state of one lane.  16-bit inputs keep two packed 15-bit magnitudes per word.
+template <int DT> struct AbsAcc {
+    uint32_t m = 0;
+    __device__ __forceinline__ void chunk(const void* p, int64_t i) {
+        if constexpr (DT == MO_F32) {
+            const u32x4* q = (const u32x4*)((const float*)p + i);
+            u32x4 a = __builtin_nontemporal_load(q), b = __builtin_nontemporal_load(q + 1);
+            uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { uint32_t t = w[j] & 0x7FFFFFFFu; m = t > m ? t : m; }
+        } else {
+            u32x4 a = __builtin_nontemporal_load((const u32x4*)((const uint16_t*)p + i));
+            uint32_t t = pk_max_u16(pk_max_u16(a.x & 0x7FFF7FFFu, a.y & 0x7FFF7FFFu),
+                                    pk_max_u16(a.z & 0x7FFF7FFFu, a.w & 0x7FFF7FFFu));
+            m = pk_max_u16(m, t);
+        }
+    }
+    __device__ __forceinline__ void elem(const void* p, int64_t i) {
+        if constexpr (DT == MO_F32) {
+            uint32_t t = ((const uint32_t*)p)[i] & 0x7FFFFFFFu;
+            m = t > m ? t : m;
+        } else {
+            m = pk_max_u16(m, ((const uint16_t*)p)[i] & 0x7FFFu);
+        }
+    }
+    // fp32 bit pattern of the lane's maximum
+    __device__ __forceinline__ uint32_t bits() const {
+        if constexpr (DT == MO_F32) return m;
+        uint32_t h = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
+        if constexpr (DT == MO_BF16) return h << 16;
+        return f2u(f16_bits_to_f32(h));
+    }
+};
+
+// ------------------------------------------------------------------------------ per tensor
+template <int DT>
+__global__ __launch_bounds__(256) void absmax_flat_kernel(const void* __restrict__ x, int64_t n,
+                                                          uint32_t* __restrict__ acc) {
+    __shared__ uint32_t smem[4];
+    AbsAcc<DT> a;
+    const int64_t chunks = n >> 3;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; c + 3 * stride < chunks; c += 4 * stride) {
+        a.chunk(x, c << 3);
+        a.chunk(x, (c + stride) << 3);
+        a.chunk(x, (c + 2 * stride) << 3);
+        a.chunk(x, (c + 3 * stride) << 3);
+    }
+    for (; c < chunks; c += stride) a.chunk(x, c << 3);
+    if (blockIdx.x == 0 && threadIdx.x < (n & 7)) a.elem(x, (chunks << 3) + threadIdx.x);
+    uint32_t v = block_max_u32(a.bits(), smem);
+    if (threadIdx.x == 0 && v) atomicMax(acc, v);
+}
+
+// ------------------------------------------------------------------------------ rows
+// x viewed as [nrows, inner]; row r feeds acc[r % axis].  A row is handled by `L` adjacent
+// lanes (power of two, <= 64) that stride over its chunks; gridDim.y splits long rows.
+template <int DT, bool ALIGNED>
+__global__ __launch_bounds__(256) void absmax_rows_kernel(const void* __restrict__ x,
+                                                          int64_t nrows, int64_t inner,
+                                                          int64_t axis, int lg_l, int64_t seg_chunks,
+                                                          uint32_t* __restrict__ acc) {
+    const int L = 1 << lg_l;
+    const int sub = threadIdx.x & (L - 1);
+    const int64_t workers = ((int64_t)gridDim.x * blockDim.x) >> lg_l;
+    const int64_t row_chunks = (inner + 7) >> 3;
+    const int64_t c0 = (int64_t)blockIdx.y * seg_chunks;
+    int64_t c1 = c0 + seg_chunks;
+    if (c1 > row_chunks) c1 = row_chunks;
+    // every lane of a worker iterates the same number of rows, so the shuffles stay convergent
+    for (int64_t r = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> lg_l; r < nrows;
+         r += workers) {
+        AbsAcc<DT> a;
+        const int64_t base = r * inner;
+        for (int64_t c = c0 + sub; c < c1; c += L) {
+            const int64_t col = c << 3;
+            if (ALIGNED && col + 8 <= inner) {
+                a.chunk(x, base + col);
+            } else {
+                for (int j = 0; j < 8; ++j)
+                    if (col + j < inner) a.elem(x, base + col + j);
+            }
+        }
+        uint32_t v = a.bits();
+        for (int o = L >> 1; o > 0; o >>= 1) {
+            uint32_t t = (uint32_t)__shfl_xor((int)v, o, kWave);
+            v = t > v ? t : v;
+        }
+        if (sub == 0 && v) atomicMax(acc + (r % axis), v);
+    }
+}
+
+// ------------------------------------------------------------------------------ columns
+// x viewed as [outer, axis] (inner == 1); a thread owns VEC adjacent columns over a slab of
+// rows (gridDim.y slabs) and ends with VEC atomics.
+template <int DT, int VEC>
+__global__ __launch_bounds__(256) void absmax_cols_kernel(const void* __restrict__ x,
+                                                          int64_t outer, int64_t axis,
+                                                          int64_t slab,
+                                                          uint32_t* __restrict__ acc) {
+    const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+    if (col >= axis) return;
+    const int64_t r0 = (int64_t)blockIdx.y * slab;
+    int64_t r1 = r0 + slab;
+    if (r1 > outer) r1 = outer;
+    uint32_t m[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) m[j] = 0;
+    if constexpr (VEC == 8) {
+        if constexpr (DT == MO_F32) {
+            for (int64_t r = r0; r < r1; ++r) {
+                const u32x4* q = (const u32x4*)((const float*)x + r * axis + col);
+                u32x4 a = __builtin_nontemporal_load(q), b = __builtin_nontemporal_load(q + 1);
+                uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) { uint32_t t = w[j] & 0x7FFFFFFFu; m[j] = t > m[j] ? t : m[j]; }
+            }
+        } else {
+            uint32_t p[4] = {0, 0, 0, 0};  // packed pairs of columns
+            int64_t r = r0;
+            for (; r + 3 < r1; r += 4) {
+                u32x4 a[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    a[u] = __builtin_nontemporal_load(
+                        (const u32x4*)((const uint16_t*)x + (r + u) * axis + col));
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    p[0] = pk_max_u16(p[0], a[u].x & 0x7FFF7FFFu);
+                    p[1] = pk_max_u16(p[1], a[u].y & 0x7FFF7FFFu);
+                    p[2] = pk_max_u16(p[2], a[u].z & 0x7FFF7FFFu);
+                    p[3] = pk_max_u16(p[3], a[u].w & 0x7FFF7FFFu);
+                }
+            }
+            for (; r < r1; ++r) {
+                u32x4 a = __builtin_nontemporal_load(
+                    (const u32x4*)((const uint16_t*)x + r * axis + col));
+                p[0] = pk_max_u16(p[0], a.x & 0x7FFF7FFFu);
+                p[1] = pk_max_u16(p[1], a.y & 0x7FFF7FFFu);
+                p[2] = pk_max_u16(p[2], a.z & 0x7FFF7FFFu);
+                p[3] = pk_max_u16(p[3], a.w & 0x7FFF7FFFu);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                uint32_t lo = p[j] & 0xFFFFu, hi = p[j] >> 16;
+                m[2 * j] = DT == MO_BF16 ? lo << 16 : f2u(f16_bits_to_f32(lo));
+                m[2 * j + 1] = DT == MO_BF16 ? hi << 16 : f2u(f16_bits_to_f32(hi));
+            }
+        }
+    } else {
+        AbsAcc<DT> a;
+        for (int64_t r = r0; r < r1; ++r) a.elem(x, r * axis + col);
+        m[0] = a.bits();
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+        if (m[j]) atomicMax(acc + col + j, m[j]);
+}
+
+template <int DT>
+static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, uint32_t* acc,
+                         hipStream_t s) {
+    const bool base_ok = ((uintptr_t)x & 15u) == 0;
+    if (axis == 1) {  // per tensor
+        const int64_t n = outer * inner;
+        if (base_ok) {
+            int64_t blocks = ((n >> 3) + 1023) / 1024;
+            if (blocks < 1) blocks = 1;
+            if (blocks > 2048) blocks = 2048;
+            absmax_flat_kernel<DT><<<dim3((unsigned)blocks), 256, 0, s>>>(x, n, acc);
+            return MO_OK;
+        }
+        outer = 1; inner = n;  // unaligned base: guarded row path below
+    }
+    if (inner == 1) {  // per column
+        const bool vec = base_ok && (axis % 8 == 0);
+        const int64_t threads = vec ? axis / 8 : axis;
+        const int64_t gx = (threads + 255) / 256;
+        // enough slabs to fill the chip, at least 16 rows each
+        int64_t gy = (2048 + gx - 1) / gx;
+        int64_t slab = (outer + gy - 1) / gy;
+        if (slab < 16) slab = 16;
+        gy = (outer + slab - 1) / slab;
+        if (gy > 65535) { gy = 65535; slab = (outer + gy - 1) / gy; }
+        if (vec)
+            absmax_cols_kernel<DT, 8><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
+        else
+            absmax_cols_kernel<DT, 1><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
+        return MO_OK;
+    }
+    // rows of length `inner`
+    const int64_t nrows = outer * axis;
+    const int64_t row_chunks = (inner + 7) >> 3;
+    int lg = 0;
+    while ((1 << lg) < 64 && (int64_t(1) << lg) < row_chunks) ++lg;
+    const int64_t workers_per_block = 256 >> lg;
+    int64_t gx = (nrows + workers_per_block - 1) / workers_per_block;
+    if (gx > 4096) gx = 4096;
+    // split long rows when there are too few rows to fill the chip
+    int64_t gy = 1;
+    const int64_t per_worker_chunks = row_chunks >> lg;
+    if (gx < 1024 && per_worker_chunks > 16) {
+        gy = 1024 / gx;
+        if (gy > per_worker_chunks / 8) gy = per_worker_chunks / 8;
+        if (gy < 1) gy = 1;
+        if (gy > 65535) gy = 65535;
+    }
+    int64_t seg = (row_chunks + gy - 1) / gy;
+    seg = ((seg + (1 << lg) - 1) >> lg) << lg;  // whole strides per segment
+    gy = (row_chunks + seg - 1) / seg;
+    const bool aligned = base_ok && (inner % 8 == 0);
+    if (aligned)
+        absmax_rows_kernel<DT, true><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, nrows, inner, axis, lg, seg, acc);
+    else
+        absmax_rows_kernel<DT, false><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, nrows, inner, axis, lg, seg, acc);
+    return MO_OK;
+}
+
+}  // namespace mo
+
+extern "C" int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
+                         float* acc, void* stream) {
+    if (outer < 0 || axis < 0 || inner < 0) return MO_ERR_ARG;
+    if (outer == 0 || axis == 0 || inner == 0) return MO_OK;
+    if (!x || !acc) return MO_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    int rc;
+    switch (dtype) {
+        case MO_F32: rc = mo::launch_absmax<MO_F32>(x, outer, axis, inner, (uint32_t*)acc, s); break;
+        case MO_F16: rc = mo::launch_absmax<MO_F16>(x, outer, axis, inner, (uint32_t*)acc, s); break;
+        case MO_BF16: rc = mo::launch_absmax<MO_BF16>(x, outer, axis, inner, (uint32_t*)acc, s); break;
+        default: return MO_ERR_DTYPE;
+    }
+    if (rc != MO_OK) return rc;
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}

@@ -1,0 +1,241 @@
+// Shared device helpers for the gfx950 quantization kernels.
+//
+// Conventions used by every kernel in this directory:
+//  * one "chunk" = 8 consecutive elements of the innermost dimension; a lane loads a chunk with
+//    one 16-byte access for 16-bit inputs (two for fp32), so a wavefront instruction touches
+//    1 KiB of contiguous memory when the tensor is chunk aligned;
+//  * all rounding that decides an output bit is done in software on integer bit patterns or
+//    with IEEE fp32 operations (no approximate reciprocal decides a bit on its own);
+//  * abs-max values travel as the uint32 bit pattern of a non-negative fp32: unsigned integer
+//    order equals numeric order there and every NaN pattern sorts above +inf, so an integer max
+//    propagates NaN exactly like torch.max does.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/modelopt_hip.h"
+
+namespace mo {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
+__device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
+
+// ---------------------------------------------------------------- 16-bit float <-> fp32
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return u2f(h << 16); }
+
+// fp32 -> bf16 bits, round to nearest even; NaN -> quiet NaN keeping the sign.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = f2u(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return ((u >> 16) & 0x8000u) | 0x7FC0u;
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    _Float16 v;
+    uint16_t b = (uint16_t)h;
+    __builtin_memcpy(&v, &b, 2);
+    return (float)v;
+}
+
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    _Float16 v = (_Float16)f;  // v_cvt_f16_f32: IEEE round to nearest even
+    uint16_t b;
+    __builtin_memcpy(&b, &v, 2);
+    return b;
+}
+
+// ---------------------------------------------------------------- chunk load / store by dtype
+// A chunk is always presented to the math as 8 fp32 values.  `abs16` style tricks live in the
+// kernels that need them; these helpers are the generic path.
+
+template <int DT> struct Elem;
+template <> struct Elem<MO_F32> { static constexpr int bytes = 4; };
+template <> struct Elem<MO_F16> { static constexpr int bytes = 2; };
+template <> struct Elem<MO_BF16> { static constexpr int bytes = 2; };
+
+template <int DT>
+__device__ __forceinline__ float load_elem(const void* p, int64_t i) {
+    if constexpr (DT == MO_F32) return ((const float*)p)[i];
+    else if constexpr (DT == MO_F16) return f16_bits_to_f32(((const uint16_t*)p)[i]);
+    else return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+}
+
+template <int DT>
+__device__ __forceinline__ void store_elem(void* p, int64_t i, float v) {
+    if constexpr (DT == MO_F32) ((float*)p)[i] = v;
+    else if constexpr (DT == MO_F16) ((uint16_t*)p)[i] = (uint16_t)f32_to_f16_bits(v);
+    else ((uint16_t*)p)[i] = (uint16_t)f32_to_bf16_bits(v);
+}
+
+// Aligned chunk (8 elements starting at element index i, i % 8 == 0, base 16-byte aligned).
+template <int DT>
+__device__ __forceinline__ void load_chunk(const void* p, int64_t i, float (&v)[8]) {
+    if constexpr (DT == MO_F32) {
+        const f32x4* q = (const f32x4*)((const float*)p + i);
+        f32x4 a = __builtin_nontemporal_load(q), b = __builtin_nontemporal_load(q + 1);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        u32x4 w = __builtin_nontemporal_load((const u32x4*)((const uint16_t*)p + i));
+        uint32_t r[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (DT == MO_BF16) {
+                v[2 * j] = u2f(r[j] << 16);
+                v[2 * j + 1] = u2f(r[j] & 0xFFFF0000u);
+            } else {
+                v[2 * j] = f16_bits_to_f32(r[j] & 0xFFFFu);
+                v[2 * j + 1] = f16_bits_to_f32(r[j] >> 16);
+            }
+        }
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ void store_chunk(void* p, int64_t i, const float (&v)[8]) {
+    if constexpr (DT == MO_F32) {
+        f32x4* q = (f32x4*)((float*)p + i);
+        f32x4 a = {v[0], v[1], v[2], v[3]}, b = {v[4], v[5], v[6], v[7]};
+        __builtin_nontemporal_store(a, q);
+        __builtin_nontemporal_store(b, q + 1);
+    } else {
+        uint32_t r[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (DT == MO_BF16)
+                r[j] = f32_to_bf16_bits(v[2 * j]) | (f32_to_bf16_bits(v[2 * j + 1]) << 16);
+            else
+                r[j] = f32_to_f16_bits(v[2 * j]) | (f32_to_f16_bits(v[2 * j + 1]) << 16);
+        }
+        u32x4 w = {r[0], r[1], r[2], r[3]};
+        __builtin_nontemporal_store(w, (u32x4*)((uint16_t*)p + i));
+    }
+}
+
+// Guarded chunk: elements [i, i + 8) of a row of which only indices < limit exist; the rest
+// read as +0 and are not written.
+template <int DT>
+__device__ __forceinline__ void load_chunk_guarded(const void* p, int64_t base, int64_t col,
+                                                   int64_t limit, float (&v)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (col + j < limit) ? load_elem<DT>(p, base + col + j) : 0.0f;
+}
+
+template <int DT>
+__device__ __forceinline__ void store_chunk_guarded(void* p, int64_t base, int64_t col,
+                                                    int64_t limit, const float (&v)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+        if (col + j < limit) store_elem<DT>(p, base + col + j, v[j]);
+}
+
+// Scalar read of an amax / scale operand given in any of the three float dtypes.
+__device__ __forceinline__ float load_scalar(const void* p, int dtype, int64_t i) {
+    if (dtype == MO_F32) return ((const float*)p)[i];
+    if (dtype == MO_F16) return f16_bits_to_f32(((const uint16_t*)p)[i]);
+    return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+}
+
+// ---------------------------------------------------------------- E4M3 (OCP e4m3fn)
+
+// fp32 -> E4M3 byte, round to nearest even, subnormals kept.  Magnitudes that round above 448
+// (i.e. > 464), infinities and NaN give the NaN pattern 0x7F | sign -- the behaviour of
+// torch's CPU cast.  With SAT the result saturates at +-448 instead (NaN stays NaN).
+template <bool SAT = false>
+__device__ __forceinline__ uint32_t f32_to_e4m3(float f) {
+    uint32_t u = f2u(f);
+    uint32_t sign = (u >> 24) & 0x80u;
+    uint32_t a = u & 0x7FFFFFFFu;
+    uint32_t r;
+    if (a < 0x3C800000u) {                       // |f| < 2^-6: fixed quantum 2^-9
+        r = f2u(u2f(a) + 16384.0f) - 0x46800000u;  // 2^14 aligns the unit to mantissa bit 0
+    } else {
+        uint32_t t = a + 0x7FFFFu + ((a >> 20) & 1u);
+        r = (t - (120u << 23)) >> 20;
+        if (a > 0x7F800000u) r = 0x7F;            // NaN
+        else if (t >= 0x43F00000u) r = SAT ? 0x7E : 0x7F;  // rounds to >= 480
+    }
+    return r | sign;
+}
+
+__device__ __forceinline__ float e4m3_to_f32(uint32_t b) {
+    uint32_t sign = (b & 0x80u) << 24;
+    uint32_t e = (b >> 3) & 0xFu, m = b & 7u;
+    if ((b & 0x7Fu) == 0x7Fu) return u2f(sign | 0x7FC00000u);
+    if (e == 0) return u2f(sign | f2u((float)m * 0.001953125f));
+    return u2f(sign | ((e + 120u) << 23) | (m << 20));
+}
+
+// fp32 rounded to the E4M3 grid, returned as fp32 (value of the byte above, without packing).
+template <bool SAT = false>
+__device__ __forceinline__ float round_e4m3(float f) {
+    uint32_t u = f2u(f);
+    uint32_t sign = u & 0x80000000u;
+    uint32_t a = u & 0x7FFFFFFFu;
+    float r;
+    if (a < 0x3C800000u) {
+        r = (u2f(a) + 16384.0f) - 16384.0f;
+    } else {
+        uint32_t t = (a + 0x7FFFFu + ((a >> 20) & 1u)) & 0xFFF00000u;
+        r = u2f(t);
+        if (a > 0x7F800000u) r = u2f(0x7FC00000u);
+        else if (t > 0x43E00000u) r = SAT ? 448.0f : u2f(0x7FC00000u);
+    }
+    return u2f(f2u(r) | sign);
+}
+
+// ---------------------------------------------------------------- E2M1 (FP4)
+
+// fp32 -> 4-bit code = sign << 3 | ordinal, ties to the even code.  NaN and +-inf give
+// ordinal 7; the sign bit is (v < 0), so -0.0 and NaN are unsigned.
+__device__ __forceinline__ uint32_t f32_to_e2m1(float v) {
+    float a = __builtin_fabsf(v);
+    uint32_t c = (uint32_t)!(a <= 0.25f) + (uint32_t)!(a < 0.75f) + (uint32_t)!(a <= 1.25f) +
+                 (uint32_t)!(a < 1.75f) + (uint32_t)!(a <= 2.5f) + (uint32_t)!(a < 3.5f) +
+                 (uint32_t)!(a <= 5.0f);
+    return c | ((v < 0.0f) ? 8u : 0u);
+}
+
+// 4-bit code -> fp32 value; code 8 decodes to +0.
+__device__ __forceinline__ float e2m1_to_f32(uint32_t c) {
+    uint32_t m = c & 7u;
+    // 0, .5, 1, 1.5, 2, 3, 4, 6: ordinal m >= 2 is a normal number with exponent (m >> 1) - 1
+    float mag = (m < 2u) ? 0.5f * (float)m
+                         : u2f(((126u + (m >> 1)) << 23) | ((m & 1u) << 22));
+    return (c & 8u) && m ? -mag : mag;
+}
+
+// ---------------------------------------------------------------- reductions
+
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        uint32_t t = (uint32_t)__shfl_xor((int)v, o, kWave);
+        v = t > v ? t : v;
+    }
+    return v;
+}
+
+// Block-wide max; result valid in thread 0.  `smem` holds one word per wave.
+__device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* smem) {
+    v = wave_max_u32(v);
+    int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (lane == 0) smem[wave] = v;
+    __syncthreads();
+    if (wave == 0) {
+        int nw = (blockDim.x + kWave - 1) / kWave;
+        v = lane < nw ? smem[lane] : 0u;
+        v = wave_max_u32(v);
+    }
+    return v;
+}
+
+}  // namespace mo

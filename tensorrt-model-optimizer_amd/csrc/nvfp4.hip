@@ -1,0 +1,266 @@
+// NVFP4 (E2M1 codes, E4M3 block scales, fp32 global scale) kernels for gfx950:
+// quantize + pack, unpack + rescale, and the fused quantize-dequantize.
+//
+// Work decomposition: a lane owns one chunk (8 elements); a block of BS elements is owned by
+// G = BS / 8 adjacent lanes that combine their abs-max with in-wave shuffles, so a wavefront
+// load instruction reads 1 KiB (bf16) of contiguous memory and a wavefront store writes 256
+// contiguous bytes of codes.  No LDS, no cross-wave traffic.
+//
+// Algorithmic bytes per element (bf16 in): quantize 2 + 1/2 + 1/16; dequantize 1/2 + 1/16 + 2;
+// quantize-dequantize 2 + 2.
+#include "common.h"
+
+namespace mo {
+
+// E4M3 byte of a block scale bs = bmax / gs6 (0 -> 1.0).  When the quotient is NaN because of
+// an invalid operation (0/0, inf/inf) the x86 reference produces the negative default NaN and
+// therefore the byte 0xFF; a NaN that comes from a NaN operand keeps that operand's (positive)
+// sign and gives 0x7F.
+__device__ __forceinline__ uint32_t block_scale_byte(float bmax, float gs6) {
+    float bs = bmax / gs6;
+    if (bs == 0.0f) bs = 1.0f;
+    if (bs != bs) return (bmax != bmax || gs6 != gs6) ? 0x7Fu : 0xFFu;
+    return f32_to_e4m3<false>(bs);
+}
+
+template <int G>
+__device__ __forceinline__ uint32_t group_max(uint32_t m) {
+#pragma unroll
+    for (int o = G >> 1; o > 0; o >>= 1) {
+        uint32_t t = (uint32_t)__shfl_xor((int)m, o, kWave);
+        m = t > m ? t : m;
+    }
+    return m;
+}
+
+__device__ __forceinline__ uint32_t chunk_absmax_bits(const float (&v)[8]) {
+    uint32_t m = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        uint32_t t = f2u(v[j]) & 0x7FFFFFFFu;
+        m = t > m ? t : m;
+    }
+    return m;
+}
+
+// Chunk c of the zero-padded [rows, kp] view -> loads from the real [rows, k] tensor.
+template <int DT, bool FLAT>
+__device__ __forceinline__ void load_padded(const void* x, int64_t c, int64_t k, int64_t cpr,
+                                            float (&v)[8], int64_t& base, int64_t& col) {
+    if constexpr (FLAT) {
+        base = 0; col = c << 3;
+        load_chunk<DT>(x, col, v);
+    } else {
+        const int64_t row = c / cpr;
+        col = (c - row * cpr) << 3;
+        base = row * k;
+        load_chunk_guarded<DT>(x, base, col, k, v);
+    }
+}
+
+// ------------------------------------------------------------------------------ quantize
+template <int DT, int BS, bool FLAT>
+__global__ __launch_bounds__(256) void nvfp4_quantize_kernel(
+    const void* __restrict__ x, int64_t total_chunks, int64_t k, int64_t cpr,
+    const float* __restrict__ amax, int amax_is_wsf2, const uint8_t* __restrict__ wsf_in,
+    uint32_t* __restrict__ packed, uint8_t* __restrict__ wsf_out, float* __restrict__ wsf2_out) {
+    constexpr int G = BS / 8;
+    const float wsf2 = amax_is_wsf2 ? amax[0] : amax[0] / 2688.0f;  // 6 * 448
+    const float gs6 = 6.0f * wsf2;
+    if (wsf2_out && blockIdx.x == 0 && threadIdx.x == 0) wsf2_out[0] = wsf2;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < total_chunks;
+         c += stride) {
+        float v[8];
+        int64_t base, col;
+        load_padded<DT, FLAT>(x, c, k, cpr, v, base, col);
+        uint32_t byte;
+        if (wsf_in) {
+            byte = wsf_in[c / G];
+        } else {
+            const float bmax = u2f(group_max<G>(chunk_absmax_bits(v)));
+            byte = block_scale_byte(bmax, gs6);
+            if (wsf_out && (threadIdx.x & (G - 1)) == 0) wsf_out[c / G] = (uint8_t)byte;
+        }
+        const float s = e4m3_to_f32(byte) * wsf2;
+        uint32_t w = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w |= f32_to_e2m1(v[j] / s) << (4 * j);
+        __builtin_nontemporal_store(w, packed + c);
+    }
+}
+
+// ------------------------------------------------------------------------------ dequantize
+template <int DT, int BS>
+__global__ __launch_bounds__(256) void nvfp4_dequantize_kernel(
+    const uint32_t* __restrict__ packed, const uint8_t* __restrict__ wsf,
+    const float* __restrict__ wsf2p, int64_t total_chunks, void* __restrict__ y) {
+    constexpr int G = BS / 8;
+    const float wsf2 = wsf2p[0];
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < total_chunks;
+         c += stride) {
+        const uint32_t w = __builtin_nontemporal_load(packed + c);
+        const float s = e4m3_to_f32(wsf[c / G]) * wsf2;
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = e2m1_to_f32((w >> (4 * j)) & 0xFu) * s;
+        store_chunk<DT>(y, c << 3, v);
+    }
+}
+
+// ------------------------------------------------------------------------------ QDQ
+// MODE 0: threshold ladder with clamped block scale; MODE 1: quantize -> dequantize.
+template <int DT, int BS, int MODE, bool FLAT>
+__global__ __launch_bounds__(256) void nvfp4_qdq_kernel(const void* __restrict__ x,
+                                                        void* __restrict__ y,
+                                                        int64_t total_chunks, int64_t k,
+                                                        int64_t cpr, const void* amax,
+                                                        int amax_dtype) {
+    constexpr int G = BS / 8;
+    const float gs = load_scalar(amax, amax_dtype, 0) / 2688.0f;
+    const float gs_safe = gs > 0.0f ? gs : 1e-12f;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < total_chunks;
+         c += stride) {
+        float v[8];
+        int64_t base, col;
+        load_padded<DT, FLAT>(x, c, k, cpr, v, base, col);
+        const float bmax = u2f(group_max<G>(chunk_absmax_bits(v)));
+        float o[8];
+        if constexpr (MODE == 0) {
+            float sc = bmax / (6.0f * gs_safe);
+            if (sc == sc) sc = sc < 448.0f ? sc : 448.0f;
+            float q = round_e4m3<false>(sc) * gs;
+            q = q >= 1e-5f ? q : 1.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float r = __builtin_fabsf(v[j]) / q;
+                float lvl = 6.0f;
+                lvl = r <= 5.0f ? 4.0f : lvl;
+                lvl = r < 3.5f ? 3.0f : lvl;
+                lvl = r <= 2.5f ? 2.0f : lvl;
+                lvl = r < 1.75f ? 1.5f : lvl;
+                lvl = r <= 1.25f ? 1.0f : lvl;
+                lvl = r < 0.75f ? 0.5f : lvl;
+                lvl = r <= 0.25f ? 0.0f : lvl;
+                const float t = lvl * q;
+                o[j] = v[j] >= 0.0f ? t : -t;
+            }
+        } else {
+            const uint32_t byte = block_scale_byte(bmax, 6.0f * gs);
+            const float s = e4m3_to_f32(byte) * gs;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[j] = e2m1_to_f32(f32_to_e2m1(v[j] / s)) * s;
+        }
+        if constexpr (FLAT) store_chunk<DT>(y, col, o);
+        else store_chunk_guarded<DT>(y, base, col, k, o);
+    }
+}
+
+static inline unsigned grid_for(int64_t chunks) {
+    int64_t b = (chunks + 255) / 256;
+    if (b < 1) b = 1;
+    if (b > 16384) b = 16384;
+    return (unsigned)b;
+}
+
+template <int DT, int BS>
+static void launch_quantize(const void* x, int64_t rows, int64_t k, int64_t kp, const float* amax,
+                            int is_wsf2, const uint8_t* wsf_in, uint8_t* packed, uint8_t* wsf_out,
+                            float* wsf2_out, hipStream_t s) {
+    const int64_t cpr = kp / 8, total = rows * cpr;
+    const bool flat = (k == kp) && (((uintptr_t)x & 15u) == 0);
+    if (flat)
+        nvfp4_quantize_kernel<DT, BS, true><<<grid_for(total), 256, 0, s>>>(
+            x, total, k, cpr, amax, is_wsf2, wsf_in, (uint32_t*)packed, wsf_out, wsf2_out);
+    else
+        nvfp4_quantize_kernel<DT, BS, false><<<grid_for(total), 256, 0, s>>>(
+            x, total, k, cpr, amax, is_wsf2, wsf_in, (uint32_t*)packed, wsf_out, wsf2_out);
+}
+
+template <int DT, int BS>
+static void launch_qdq(const void* x, void* y, int64_t rows, int64_t k, int64_t kp,
+                       const void* amax, int amax_dtype, int mode, hipStream_t s) {
+    const int64_t cpr = kp / 8, total = rows * cpr;
+    const bool flat = (k == kp) && (((uintptr_t)x & 15u) == 0) && (((uintptr_t)y & 15u) == 0);
+    const unsigned g = grid_for(total);
+    if (mode == 0) {
+        if (flat) nvfp4_qdq_kernel<DT, BS, 0, true><<<g, 256, 0, s>>>(x, y, total, k, cpr, amax, amax_dtype);
+        else nvfp4_qdq_kernel<DT, BS, 0, false><<<g, 256, 0, s>>>(x, y, total, k, cpr, amax, amax_dtype);
+    } else {
+        if (flat) nvfp4_qdq_kernel<DT, BS, 1, true><<<g, 256, 0, s>>>(x, y, total, k, cpr, amax, amax_dtype);
+        else nvfp4_qdq_kernel<DT, BS, 1, false><<<g, 256, 0, s>>>(x, y, total, k, cpr, amax, amax_dtype);
+    }
+}
+
+}  // namespace mo
+
+#define MO_DISPATCH_DT_BS(dtype, bs, CALL)                                            \
+    switch (dtype) {                                                                  \
+        case MO_F32:                                                                  \
+            if (bs == 8) { CALL(MO_F32, 8); } else if (bs == 16) { CALL(MO_F32, 16); } \
+            else { CALL(MO_F32, 32); }                                                \
+            break;                                                                    \
+        case MO_F16:                                                                  \
+            if (bs == 8) { CALL(MO_F16, 8); } else if (bs == 16) { CALL(MO_F16, 16); } \
+            else { CALL(MO_F16, 32); }                                                \
+            break;                                                                    \
+        case MO_BF16:                                                                 \
+            if (bs == 8) { CALL(MO_BF16, 8); } else if (bs == 16) { CALL(MO_BF16, 16); } \
+            else { CALL(MO_BF16, 32); }                                               \
+            break;                                                                    \
+        default: return MO_ERR_DTYPE;                                                 \
+    }
+
+extern "C" int mo_nvfp4_quantize(const void* x, int64_t rows, int64_t k, int dtype, int block_size,
+                                 const float* amax, int amax_is_wsf2, const uint8_t* wsf_in,
+                                 uint8_t* packed, uint8_t* wsf_out, float* wsf2_out,
+                                 void* stream) {
+    if (rows < 0 || k < 0) return MO_ERR_ARG;
+    if (block_size != 8 && block_size != 16 && block_size != 32) return MO_ERR_UNSUPPORTED;
+    if (rows == 0 || k == 0) return MO_OK;
+    if (!x || !amax || !packed || (!wsf_in && !wsf_out)) return MO_ERR_ARG;
+    if ((uintptr_t)packed & 3u) return MO_ERR_ARG;
+    const int64_t kp = (k + block_size - 1) / block_size * block_size;
+    hipStream_t s = (hipStream_t)stream;
+#define CALL(DT, BS) \
+    mo::launch_quantize<DT, BS>(x, rows, k, kp, amax, amax_is_wsf2, wsf_in, packed, wsf_out, wsf2_out, s)
+    MO_DISPATCH_DT_BS(dtype, block_size, CALL)
+#undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_nvfp4_dequantize(const uint8_t* packed, const uint8_t* wsf, const float* wsf2,
+                                   int64_t rows, int64_t kp, int block_size, void* y, int dtype,
+                                   void* stream) {
+    if (rows < 0 || kp < 0) return MO_ERR_ARG;
+    if (block_size != 8 && block_size != 16 && block_size != 32) return MO_ERR_UNSUPPORTED;
+    if (rows == 0 || kp == 0) return MO_OK;
+    if (!packed || !wsf || !wsf2 || !y || kp % block_size) return MO_ERR_ARG;
+    if (((uintptr_t)packed & 3u) || ((uintptr_t)y & 15u)) return MO_ERR_ARG;
+    const int64_t total = rows * (kp / 8);
+    hipStream_t s = (hipStream_t)stream;
+#define CALL(DT, BS)                                                                      \
+    mo::nvfp4_dequantize_kernel<DT, BS><<<mo::grid_for(total), 256, 0, s>>>(              \
+        (const uint32_t*)packed, wsf, wsf2, total, y)
+    MO_DISPATCH_DT_BS(dtype, block_size, CALL)
+#undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_nvfp4_qdq(const void* x, void* y, int64_t rows, int64_t k, int dtype,
+                            const void* amax, int amax_dtype, int block_size, int mode,
+                            void* stream) {
+    if (rows < 0 || k < 0 || (mode != 0 && mode != 1)) return MO_ERR_ARG;
+    if (block_size != 8 && block_size != 16 && block_size != 32) return MO_ERR_UNSUPPORTED;
+    if (amax_dtype < MO_F32 || amax_dtype > MO_BF16) return MO_ERR_DTYPE;
+    if (rows == 0 || k == 0) return MO_OK;
+    if (!x || !y || !amax) return MO_ERR_ARG;
+    const int64_t kp = (k + block_size - 1) / block_size * block_size;
+    hipStream_t s = (hipStream_t)stream;
+#define CALL(DT, BS) mo::launch_qdq<DT, BS>(x, y, rows, k, kp, amax, amax_dtype, mode, s)
+    MO_DISPATCH_DT_BS(dtype, block_size, CALL)
+#undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}

@@ -1,0 +1,178 @@
+// Elementwise quantize-dequantize kernels (FP8 E4M3 and N-bit integer) for gfx950.
+//
+// HBM-bound: one read and one write of the tensor (4 bytes per bf16 element).  x and y are
+// viewed as [outer, axis, inner] with one amax per index of `axis`.  Three addressing modes:
+//   TENSOR  one scale for everything (axis == 1);
+//   CHUNK   inner % 8 == 0, so the 8 elements a lane holds share a scale;
+//   ELEM    anything else (e.g. scales along the innermost dim): per-element scale lookup.
+#include "common.h"
+
+namespace mo {
+
+enum { TENSOR = 0, CHUNK = 1, ELEM = 2 };
+
+struct Fp8Op {
+    bool has_amax;
+    struct Scale { float mul, inv; };
+    __device__ __forceinline__ Scale make(float amax) const {
+        Scale s;
+        s.mul = 448.0f / amax;
+        s.inv = 1.0f / s.mul;
+        return s;
+    }
+    template <bool SAT>
+    __device__ __forceinline__ float apply(float x, const Scale& s) const {
+        if (!has_amax) return round_e4m3<SAT>(x);
+        return round_e4m3<SAT>(x * s.mul) * s.inv;
+    }
+};
+
+struct IntOp {
+    float bound, lo;
+    struct Scale { float mul, div; };
+    __device__ __forceinline__ Scale make(float amax) const {
+        Scale s;
+        const bool dead = amax <= 5.9604644775390625e-8f;  // 2^-24
+        const float sc = bound / amax;
+        s.mul = dead ? 0.0f : sc;
+        s.div = dead ? 1.0f : sc;
+        return s;
+    }
+    template <bool>
+    __device__ __forceinline__ float apply(float x, const Scale& s) const {
+        float q = __builtin_rintf(x * s.mul);  // round half to even
+        // clamp the way torch.clamp does: NaN stays NaN
+        q = q < lo ? lo : q;
+        q = q > bound ? bound : q;
+        return q / s.div;
+    }
+};
+
+template <int DT, int KIND, bool FLAG, typename Op>
+__global__ __launch_bounds__(256) void qdq_kernel(const void* __restrict__ x, void* __restrict__ y,
+                                                  int64_t n, int64_t axis, int64_t inner,
+                                                  const void* __restrict__ amax, int amax_dtype,
+                                                  Op op) {
+    const int64_t chunks = n >> 3;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    typename Op::Scale s0 = {};
+    if (KIND == TENSOR && amax) s0 = op.make(load_scalar(amax, amax_dtype, 0));
+    for (int64_t c = tid; c < chunks; c += stride) {
+        float v[8];
+        load_chunk<DT>(x, c << 3, v);
+        if constexpr (KIND == TENSOR) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = op.template apply<FLAG>(v[j], s0);
+        } else if constexpr (KIND == CHUNK) {
+            const int64_t a = ((c << 3) / inner) % axis;
+            const typename Op::Scale s = op.make(load_scalar(amax, amax_dtype, a));
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = op.template apply<FLAG>(v[j], s);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int64_t a = (((c << 3) + j) / inner) % axis;
+                v[j] = op.template apply<FLAG>(v[j], op.make(load_scalar(amax, amax_dtype, a)));
+            }
+        }
+        store_chunk<DT>(y, c << 3, v);
+    }
+    // tail (n % 8 elements) and nothing else: handled by the first lanes of block 0
+    if (blockIdx.x == 0 && threadIdx.x < (n & 7)) {
+        const int64_t i = (chunks << 3) + threadIdx.x;
+        const int64_t a = KIND == TENSOR ? 0 : (i / inner) % axis;
+        typename Op::Scale s = {};
+        if (amax) s = op.make(load_scalar(amax, amax_dtype, a));
+        store_elem<DT>(y, i, op.template apply<FLAG>(load_elem<DT>(x, i), s));
+    }
+}
+
+// Unaligned base pointers: same math, scalar accesses.
+template <int DT, bool FLAG, typename Op>
+__global__ __launch_bounds__(256) void qdq_scalar_kernel(const void* __restrict__ x,
+                                                         void* __restrict__ y, int64_t n,
+                                                         int64_t axis, int64_t inner,
+                                                         const void* __restrict__ amax,
+                                                         int amax_dtype, Op op) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        typename Op::Scale s = {};
+        if (amax) s = op.make(load_scalar(amax, amax_dtype, (i / inner) % axis));
+        store_elem<DT>(y, i, op.template apply<FLAG>(load_elem<DT>(x, i), s));
+    }
+}
+
+template <int DT, bool FLAG, typename Op>
+static void launch_qdq(const void* x, void* y, int64_t outer, int64_t axis, int64_t inner,
+                       const void* amax, int amax_dtype, Op op, hipStream_t s) {
+    const int64_t n = outer * axis * inner;
+    const bool aligned = (((uintptr_t)x | (uintptr_t)y) & 15u) == 0;
+    if (!aligned) {
+        int64_t b = (n + 255) / 256;
+        if (b > 16384) b = 16384;
+        qdq_scalar_kernel<DT, FLAG, Op><<<(unsigned)b, 256, 0, s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
+        return;
+    }
+    int64_t b = ((n >> 3) + 255) / 256;
+    if (b < 1) b = 1;
+    if (b > 16384) b = 16384;
+    const unsigned g = (unsigned)b;
+    if (axis == 1 || !amax)
+        qdq_kernel<DT, TENSOR, FLAG, Op><<<g, 256, 0, s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
+    else if (inner % 8 == 0)
+        qdq_kernel<DT, CHUNK, FLAG, Op><<<g, 256, 0, s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
+    else
+        qdq_kernel<DT, ELEM, FLAG, Op><<<g, 256, 0, s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
+}
+
+}  // namespace mo
+
+static int check_common(const void* x, void* y, int64_t outer, int64_t axis, int64_t inner,
+                        int amax_dtype) {
+    if (outer < 0 || axis < 0 || inner < 0) return MO_ERR_ARG;
+    if (amax_dtype < MO_F32 || amax_dtype > MO_BF16) return MO_ERR_DTYPE;
+    if (outer && axis && inner && (!x || !y)) return MO_ERR_ARG;
+    return MO_OK;
+}
+
+extern "C" int mo_fp8_qdq(const void* x, void* y, int64_t outer, int64_t axis, int64_t inner,
+                          int dtype, const void* amax, int amax_dtype, int saturate,
+                          void* stream) {
+    int rc = check_common(x, y, outer, axis, inner, amax_dtype);
+    if (rc != MO_OK) return rc;
+    if (outer == 0 || axis == 0 || inner == 0) return MO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    mo::Fp8Op op{amax != nullptr};
+#define CALL(DT)                                                                                   \
+    if (saturate) mo::launch_qdq<DT, true>(x, y, outer, axis, inner, amax, amax_dtype, op, s);     \
+    else mo::launch_qdq<DT, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s)
+    switch (dtype) {
+        case MO_F32: CALL(MO_F32); break;
+        case MO_F16: CALL(MO_F16); break;
+        case MO_BF16: CALL(MO_BF16); break;
+        default: return MO_ERR_DTYPE;
+    }
+#undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_int_qdq(const void* x, void* y, int64_t outer, int64_t axis, int64_t inner,
+                          int dtype, const void* amax, int amax_dtype, int num_bits,
+                          int is_unsigned, int narrow_range, void* stream) {
+    int rc = check_common(x, y, outer, axis, inner, amax_dtype);
+    if (rc != MO_OK) return rc;
+    if (!amax || num_bits < 1 || num_bits > 24) return MO_ERR_ARG;
+    if (outer == 0 || axis == 0 || inner == 0) return MO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    mo::IntOp op;
+    op.bound = (float)((1 << (num_bits - 1 + (is_unsigned ? 1 : 0))) - 1);
+    op.lo = is_unsigned ? 0.0f : (narrow_range ? -op.bound : -op.bound - 1.0f);
+    switch (dtype) {
+        case MO_F32: mo::launch_qdq<MO_F32, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s); break;
+        case MO_F16: mo::launch_qdq<MO_F16, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s); break;
+        case MO_BF16: mo::launch_qdq<MO_BF16, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s); break;
+        default: return MO_ERR_DTYPE;
+    }
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}

@@ -1,0 +1,49 @@
+import os
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG_PARENT = os.path.join(ROOT, "tensorrt-model-optimizer_amd")
+for p in (ROOT, PKG_PARENT):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+def pytest_collection_modifyitems(config, items):
+    if torch.cuda.is_available():
+        return
+    skip = pytest.mark.skip(reason="no GPU in this environment")
+    for item in items:
+        if "gpu" in item.keywords:
+            item.add_marker(skip)
+
+
+def assert_bits_equal(actual: torch.Tensor, expected: torch.Tensor, what: str = ""):
+    """Bit-exact comparison of two tensors of the same dtype; any NaN matches any NaN."""
+    assert actual.shape == expected.shape, f"{what}: shape {actual.shape} vs {expected.shape}"
+    assert actual.dtype == expected.dtype, f"{what}: dtype {actual.dtype} vs {expected.dtype}"
+    a, e = actual.detach().cpu(), expected.detach().cpu()
+    if a.dtype.is_floating_point:
+        if a.dtype in (torch.float8_e4m3fn,):
+            a, e = a.view(torch.uint8), e.view(torch.uint8)
+            ok = a == e
+        else:
+            nan_both = torch.isnan(a) & torch.isnan(e)
+            width = {2: torch.int16, 4: torch.int32, 8: torch.int64}[a.element_size()]
+            ok = (a.view(width) == e.view(width)) | nan_both
+    else:
+        ok = a == e
+    if not bool(ok.all()):
+        bad = (~ok).nonzero()
+        first = tuple(bad[0].tolist())
+        raise AssertionError(
+            f"{what}: {bad.shape[0]} of {ok.numel()} elements differ; first at {first}: "
+            f"got {a[first].item()!r} expected {e[first].item()!r}")
