@@ -1,0 +1,191 @@
+#!/usr/bin/env python3
+"""Headline benchmark: NVFP4 quantize+pack of all Llama-3-8B-shaped linear weights on one MI355X.
+
+One "step" = one pass of the quantize+pack hot path over the 224 bf16 weight tensors of the
+model (32 layers x {q, k, v, o, gate, up, down}), inputs and per-tensor global amax already
+resident in HBM, all outputs (packed codes, E4M3 block scales, fp32 global scales) written.
+Prints ONE JSON line.  Synthetic weights: bf16 N(0, 0.02), generated on the device.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers 32] [--no-cpu-baseline]
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "tensorrt-model-optimizer_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+# Llama-3-8B linear shapes [out, in]
+LAYER_SHAPES = [("q_proj", 4096, 4096), ("k_proj", 1024, 4096), ("v_proj", 1024, 4096),
+                ("o_proj", 4096, 4096), ("gate_proj", 14336, 4096), ("up_proj", 14336, 4096),
+                ("down_proj", 4096, 14336)]
+QUANT_BYTES_PER_ELEM = 2.0 + 0.5 + 1.0 / 16.0   # bf16 read + codes + block scale
+AMAX_BYTES_PER_ELEM = 2.0
+DEQUANT_BYTES_PER_ELEM = 0.5 + 1.0 / 16.0 + 2.0
+
+
+def make_weights(torch, layers, device):
+    g = torch.Generator(device=device).manual_seed(2)
+    ws = []
+    for _ in range(layers):
+        for _, n, k in LAYER_SHAPES:
+            ws.append(torch.randn(n, k, generator=g, device=device, dtype=torch.bfloat16).mul_(0.02))
+    return ws
+
+
+def timed(torch, fn, steps, warmup):
+    """Wall time per step (ms) and mean per-launch device time (ms) from events on the stream
+    the kernels are launched on (torch's current stream)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        fn()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    dev_ms = sum(s.elapsed_time(e) for s, e in zip(starts, ends)) / steps
+    return wall_ms, dev_ms
+
+
+def cpu_baseline(torch, layers_sampled=1):
+    """The CPU oracle (= the reference's CPU torch path restated) on a bounded sample: the seven
+    weights of `layers_sampled` layer(s), block scales + codes from a given global amax."""
+    from oracle import export as oexport
+
+    g = torch.Generator().manual_seed(2)
+    elems, secs = 0, 0.0
+    for _ in range(layers_sampled):
+        for _, n, k in LAYER_SHAPES:
+            w = (0.02 * torch.randn(n, k, generator=g)).to(torch.bfloat16)
+            amax = w.abs().max()
+            t0 = time.perf_counter()
+            oexport.nvfp4_export(w, amax, 16)
+            secs += time.perf_counter() - t0
+            elems += w.numel()
+    return {
+        "value": round(elems * QUANT_BYTES_PER_ELEM / secs / 1e9, 4),
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{layers_sampled} of 32 layers (7 weights, {elems} elements), torch CPU oracle, "
+                  f"{secs:.2f} s, host has {os.cpu_count()} logical CPUs",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip amax / dequant side measurements")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print(f"bench.py measures one GPU only: this build has no multi-GPU path (got --gpus {a.gpus}); "
+              "the path shards by tensor with no exchange, see DESIGN.md", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from modelopt_amd import _hip
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
+        sys.exit(1)
+    _hip.load()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    weights = make_weights(torch, a.layers, dev)
+    elems = sum(w.numel() for w in weights)
+    aplan = _hip.AbsmaxPlan(weights)
+    amax = aplan.run().clone()                   # calibrated per-tensor amax, as export has it
+    qplan = _hip.Nvfp4QuantizePlan(weights, amax)
+    torch.cuda.synchronize()
+
+    wall_ms, dev_ms = timed(torch, qplan.run, a.steps, a.warmup)
+    quant_bytes = elems * QUANT_BYTES_PER_ELEM
+    value = quant_bytes / (wall_ms * 1e-3) / 1e9
+    achieved = quant_bytes / (dev_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "nvfp4_quantize_pack_throughput",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"NVFP4 quantize+pack of Llama-3-8B linear weights, {a.layers} layers x 7 "
+                        f"tensors ({len(weights)} tensors, {elems} elements), bf16 N(0,0.02), "
+                        "16-element blocks, E4M3 block scales, fp32 global scale from a given amax",
+            "elements": elems,
+            "algorithmic_bytes": int(quant_bytes),
+            "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "nvfp4_quantize_multi_kernel",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "launch_ms": round(dev_ms, 4),
+            "traffic": None,
+        },
+    }
+
+    if not a.no_extras:
+        extras = {}
+        w_ms, d_ms = timed(torch, aplan.run, a.steps, a.warmup)
+        extras["amax_pass"] = {"ms": round(d_ms, 4),
+                               "GBps": round(elems * AMAX_BYTES_PER_ELEM / d_ms / 1e6, 1)}
+
+        # amax -> quantize back to back, the quantize launch reading the freshly reduced amax
+        qplan_pipe = _hip.Nvfp4QuantizePlan(weights, aplan.acc)
+
+        def pipeline2():
+            aplan.run()
+            qplan_pipe.run()
+        w_ms, d_ms = timed(torch, pipeline2, a.steps, a.warmup)
+        extras["amax_plus_quantize_pipeline"] = {
+            "ms": round(w_ms, 4),
+            "GBps": round(elems * (AMAX_BYTES_PER_ELEM + QUANT_BYTES_PER_ELEM) / w_ms / 1e6, 1)}
+        # dequant round trip on the first layer's tensors
+        packed, wsf, wsf2 = qplan.run()
+        n1 = len(LAYER_SHAPES)
+        e1 = sum(w.numel() for w in weights[:n1])
+
+        def dequant():
+            for i in range(n1):
+                _hip.nvfp4_dequantize(packed[i], wsf[i], wsf2[i], 16, torch.bfloat16)
+        w_ms, d_ms = timed(torch, dequant, a.steps, a.warmup)
+        extras["dequantize_one_layer"] = {
+            "ms": round(d_ms, 4), "GBps": round(e1 * DEQUANT_BYTES_PER_ELEM / d_ms / 1e6, 1)}
+        out["extras"] = extras
+
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

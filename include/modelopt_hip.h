@@ -36,6 +36,14 @@ enum mo_status {
 int mo_version(void);
 const char* mo_error_string(int status);
 
+/* Process-wide switches (debug / verification aids; defaults are all 0).
+ * MO_OPT_FORCE_EXACT = 1 makes the NVFP4 quantize kernels divide every element by its block
+ * scale (the reference's literal arithmetic) instead of the multiply-and-verify fast path; the
+ * outputs are identical either way, which is what the switch exists to demonstrate. */
+enum mo_option { MO_OPT_FORCE_EXACT = 0, MO_OPT_COUNT_ = 1 };
+int mo_set_option(int key, int value);
+int mo_get_option(int key);
+
 /* ------------------------------------------------------------------ abs-max reductions
  * Replaces reduce_amax (TQ/utils.py:156-188) as used by MaxCalibrator.collect
  * (TQ/calib/max.py:53-94) and TensorQuantizer._get_amax (TQ/nn/modules/tensor_quantizer.py
@@ -48,6 +56,21 @@ const char* mo_error_string(int status);
  */
 int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
               float* acc, void* stream);
+
+/* Per-tensor abs-max of many tensors in ONE launch.  jobs_dev is a device-resident table sorted
+ * by tile_begin; job j owns tiles [tile_begin_j, tile_begin_j + ceil(elems_j /
+ * MO_ABSMAX_TILE_ELEMS)), total_tiles is the sum.  acc as for mo_absmax (one fp32 per job).
+ * Every x must be 16-byte aligned.  No counterpart in the reference, which loops over modules
+ * in Python (MaxCalibrator.collect per weight, TQ/nn/modules/quant_module.py:148-169). */
+#define MO_ABSMAX_TILE_ELEMS 32768
+typedef struct mo_absmax_job {
+    const void* x;
+    float* acc;
+    int64_t elems;
+    int64_t tile_begin;
+} mo_absmax_job;
+int mo_absmax_multi(const mo_absmax_job* jobs_dev, int njobs, int64_t total_tiles, int dtype,
+                    void* stream);
 
 /* ------------------------------------------------------------------ fake quantisation
  * x and y are viewed as [outer, axis, inner]; amax has `axis` elements of type amax_dtype
@@ -99,6 +122,26 @@ int mo_nvfp4_qdq(const void* x, void* y, int64_t rows, int64_t k, int dtype, con
 int mo_nvfp4_quantize(const void* x, int64_t rows, int64_t k, int dtype, int block_size,
                       const float* amax, int amax_is_wsf2, const uint8_t* wsf_in,
                       uint8_t* packed, uint8_t* wsf_out, float* wsf2_out, void* stream);
+
+/* NVFP4 quantize + pack of many tensors in ONE launch (the whole-model export pass of
+ * modelopt/torch/export/unified_export_hf.py:233-391, which calls to_quantized_weight once per
+ * linear).  jobs_dev: device-resident table sorted by tile_begin; job j owns tiles
+ * [tile_begin_j, tile_begin_j + ceil(elems_j / MO_NVFP4_TILE_ELEMS)).  Requirements per job:
+ * bf16, block size 16, last dim a multiple of 16 (so elems % 16 == 0 and no padding), x 16-byte
+ * and packed 8-byte aligned.  Outputs and amax as for mo_nvfp4_quantize. */
+#define MO_NVFP4_TILE_ELEMS 16384
+typedef struct mo_nvfp4_job {
+    const void* x;
+    uint8_t* packed;
+    uint8_t* wsf;
+    const float* amax;
+    float* wsf2_out;   /* may be NULL */
+    int64_t elems;
+    int64_t tile_begin;
+    int64_t reserved;
+} mo_nvfp4_job;
+int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs, int64_t total_tiles,
+                            int dtype, int block_size, int amax_is_wsf2, void* stream);
 
 /* NVFP4 unpack + rescale.  Replaces NVFP4QTensor.dequantize (TQ/qtensor/nvfp4_tensor.py
  * :234-297) and fp4_dequantize (TQ/triton/fp4_kernel.py:307):

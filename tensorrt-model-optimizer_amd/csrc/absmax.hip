@@ -8,18 +8,6 @@
 
 namespace mo {
 
-typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
-    u16x2 x, y;
-    __builtin_memcpy(&x, &a, 4);
-    __builtin_memcpy(&y, &b, 4);
-    u16x2 r = __builtin_elementwise_max(x, y);
-    uint32_t o;
-    __builtin_memcpy(&o, &r, 4);
-    return o;
-}
-
 // Running max state of one lane.  16-bit inputs keep two packed 15-bit magnitudes per word.
 template <int DT> struct AbsAcc {
     uint32_t m = 0;
@@ -180,6 +168,39 @@ __global__ __launch_bounds__(256) void absmax_cols_kernel(const void* __restrict
         if (m[j]) atomicMax(acc + col + j, m[j]);
 }
 
+// ------------------------------------------------------------------------------ many tensors
+template <int DT>
+__global__ __launch_bounds__(256) void absmax_multi_kernel(const mo_absmax_job* __restrict__ jobs,
+                                                           int njobs, int64_t total_tiles) {
+    __shared__ uint32_t smem[4];
+    constexpr int64_t kTileChunks = MO_ABSMAX_TILE_ELEMS / 8;
+    for (int64_t t = blockIdx.x; t < total_tiles; t += gridDim.x) {
+        int lo = 0, hi = njobs - 1;
+        while (lo < hi) {  // last job with tile_begin <= t
+            const int mid = (lo + hi + 1) >> 1;
+            if (jobs[mid].tile_begin <= t) lo = mid; else hi = mid - 1;
+        }
+        const mo_absmax_job jb = jobs[lo];
+        const int64_t chunks = jb.elems >> 3;
+        const int64_t c0 = (t - jb.tile_begin) * kTileChunks;
+        int64_t c1 = c0 + kTileChunks;
+        if (c1 > chunks) c1 = chunks;
+        AbsAcc<DT> a;
+        int64_t c = c0 + threadIdx.x;
+        for (; c + 768 < c1; c += 1024) {
+            a.chunk(jb.x, c << 3);
+            a.chunk(jb.x, (c + 256) << 3);
+            a.chunk(jb.x, (c + 512) << 3);
+            a.chunk(jb.x, (c + 768) << 3);
+        }
+        for (; c < c1; c += 256) a.chunk(jb.x, c << 3);
+        if (c1 == chunks && threadIdx.x < (jb.elems & 7)) a.elem(jb.x, (chunks << 3) + threadIdx.x);
+        __syncthreads();  // smem reuse across tiles
+        const uint32_t v = block_max_u32(a.bits(), smem);
+        if (threadIdx.x == 0 && v) atomicMax((uint32_t*)jb.acc, v);
+    }
+}
+
 template <int DT>
 static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, uint32_t* acc,
                          hipStream_t s) {
@@ -255,5 +276,21 @@ extern "C" int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
         default: return MO_ERR_DTYPE;
     }
     if (rc != MO_OK) return rc;
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_absmax_multi(const mo_absmax_job* jobs_dev, int njobs, int64_t total_tiles,
+                               int dtype, void* stream) {
+    if (njobs < 0 || total_tiles < 0) return MO_ERR_ARG;
+    if (njobs == 0 || total_tiles == 0) return MO_OK;
+    if (!jobs_dev) return MO_ERR_ARG;
+    const unsigned grid = (unsigned)(total_tiles < 4096 ? total_tiles : 4096);
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case MO_F32: mo::absmax_multi_kernel<MO_F32><<<grid, 256, 0, s>>>(jobs_dev, njobs, total_tiles); break;
+        case MO_F16: mo::absmax_multi_kernel<MO_F16><<<grid, 256, 0, s>>>(jobs_dev, njobs, total_tiles); break;
+        case MO_BF16: mo::absmax_multi_kernel<MO_BF16><<<grid, 256, 0, s>>>(jobs_dev, njobs, total_tiles); break;
+        default: return MO_ERR_DTYPE;
+    }
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

@@ -215,6 +215,19 @@ __device__ __forceinline__ float e2m1_to_f32(uint32_t c) {
 
 // ---------------------------------------------------------------- reductions
 
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+
+// max of two pairs of unsigned 16-bit values packed in a word (v_pk_max_u16)
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    u16x2 x, y;
+    __builtin_memcpy(&x, &a, 4);
+    __builtin_memcpy(&y, &b, 4);
+    u16x2 r = __builtin_elementwise_max(x, y);
+    uint32_t o;
+    __builtin_memcpy(&o, &r, 4);
+    return o;
+}
+
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {

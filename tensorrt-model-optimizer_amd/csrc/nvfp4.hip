@@ -158,6 +158,150 @@ __global__ __launch_bounds__(256) void nvfp4_qdq_kernel(const void* __restrict__
     }
 }
 
+// ------------------------------------------------------------------------------ fast path
+// bf16 input, 16-element blocks, chunk-aligned tensor: a lane owns a whole block (two 16-byte
+// loads, one 8-byte store of codes, one scale byte).
+//
+// The reference divides every element by the block's scale s with an IEEE fp32 division and
+// rounds the quotient to E2M1.  Here the per-element division is replaced by a multiply with
+// r4 = 4 / s (one IEEE division per block) and the result is *proved* equal before it is used:
+// with u = |x| * r4 the seven rounding boundaries of E2M1 sit at the integers 1, 3, 5, 7, 10,
+// 14, 20, and u differs from 4 * (x / s) by less than 2^-22 relative, while a correctly rounded
+// quotient can only change sides within 2^-24 relative of a boundary.  So whenever u is further
+// than u * 2^-21 from the nearest integer the code computed from u is the reference's code; the
+// (rare) lanes that fail that test, and blocks whose scale is outside [2^-64, 2^10] or whose
+// abs-max is not finite, recompute their block with the exact division.
+__device__ __forceinline__ uint32_t fp4_pair(uint32_t old, float a, float b, int sel) {
+    // v_cvt_scalef32_pk_fp4_f32: two fp32 -> two E2M1 codes (round to nearest even, saturating)
+    // written to byte `sel` of `old`; the inputs are divided by the (power of two) scale.
+    switch (sel) {
+        case 0: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 4.0f, 0);
+        case 1: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 4.0f, 1);
+        case 2: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 4.0f, 2);
+        default: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 4.0f, 3);
+    }
+}
+
+__device__ __forceinline__ uint32_t exact_codes8(const uint32_t (&w)[4], float s) {
+    uint32_t o = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        o |= f32_to_e2m1(u2f(w[j] << 16) / s) << (8 * j);
+        o |= f32_to_e2m1(u2f(w[j] & 0xFFFF0000u) / s) << (8 * j + 4);
+    }
+    return o;
+}
+
+// One 16-element bf16 block held as 8 packed words -> scale byte and 64 bits of codes.
+__device__ __forceinline__ void quantize_block16_bf16(const uint32_t (&w)[8], float wsf2, float gs6,
+                                                      bool force_exact, uint32_t& byte,
+                                                      uint32_t& c_lo, uint32_t& c_hi) {
+    uint32_t m = w[0] & 0x7FFF7FFFu;
+#pragma unroll
+    for (int j = 1; j < 8; ++j) m = pk_max_u16(m, w[j] & 0x7FFF7FFFu);
+    const uint32_t h = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
+    const float bmax = u2f(h << 16);
+    byte = block_scale_byte(bmax, gs6);
+    const float s = e4m3_to_f32(byte) * wsf2;
+    const uint32_t sb = f2u(s);
+    bool fast = !force_exact && sb >= 0x1F800000u && sb <= 0x44800000u && h < 0x7F80u;
+    const float r4 = 4.0f * (1.0f / s);
+    fast = fast && (bmax * r4 < 3.0e38f);
+    bool redo = !fast;
+    if (fast) {
+        float emin = 1.0f;
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            // + 0.0f turns a -0.0 product into +0.0, the reference's unsigned zero code
+            const float u0 = __builtin_fmaf(u2f(w[j] << 16), r4, 0.0f);
+            const float u1 = __builtin_fmaf(u2f(w[j] & 0xFFFF0000u), r4, 0.0f);
+            const float a0 = __builtin_fabsf(u0), a1 = __builtin_fabsf(u1);
+            const float d0 = __builtin_fabsf(a0 - __builtin_rintf(a0));
+            const float d1 = __builtin_fabsf(a1 - __builtin_rintf(a1));
+            const float e0 = __builtin_fmaf(a0, -4.76837158203125e-7f, d0);  // 2^-21
+            const float e1 = __builtin_fmaf(a1, -4.76837158203125e-7f, d1);
+            emin = __builtin_fminf(emin, __builtin_fminf(e0, e1));
+            if (j < 4) lo = fp4_pair(lo, u0, u1, j);
+            else hi = fp4_pair(hi, u0, u1, j - 4);
+        }
+        c_lo = lo; c_hi = hi;
+        // e == 0 only for u == 0 (exact zero, no boundary near); e < 0 means "too close"
+        redo = !(emin >= 0.0f);
+    }
+    if (redo) {
+        const uint32_t w0[4] = {w[0], w[1], w[2], w[3]}, w1[4] = {w[4], w[5], w[6], w[7]};
+        c_lo = exact_codes8(w0, s);
+        c_hi = exact_codes8(w1, s);
+    }
+}
+
+// Tiles of kTileBlocks 16-element blocks; a workgroup of 256 lanes handles a tile in
+// kTileBlocks / 256 rounds with all loads of a round issued before its math.
+constexpr int kTileBlocks = MO_NVFP4_TILE_ELEMS / 16;
+
+__device__ __forceinline__ void quantize_tile_bf16(const uint16_t* __restrict__ x,
+                                                   int64_t nblocks, int64_t tile, float wsf2,
+                                                   float gs6, bool force_exact,
+                                                   u32x2* __restrict__ packed,
+                                                   uint8_t* __restrict__ wsf) {
+    constexpr int R = kTileBlocks / 256;
+    const int64_t b0 = tile * kTileBlocks + threadIdx.x;
+    u32x4 a[R], b[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int64_t blk = b0 + r * 256;
+        if (blk < nblocks) {
+            const u32x4* p = (const u32x4*)(x + blk * 16);
+            a[r] = __builtin_nontemporal_load(p);
+            b[r] = __builtin_nontemporal_load(p + 1);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int64_t blk = b0 + r * 256;
+        if (blk < nblocks) {
+            const uint32_t w[8] = {a[r].x, a[r].y, a[r].z, a[r].w, b[r].x, b[r].y, b[r].z, b[r].w};
+            uint32_t byte, lo, hi;
+            quantize_block16_bf16(w, wsf2, gs6, force_exact, byte, lo, hi);
+            u32x2 o = {lo, hi};
+            __builtin_nontemporal_store(o, packed + blk);
+            wsf[blk] = (uint8_t)byte;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void nvfp4_quantize_fast_kernel(
+    const uint16_t* __restrict__ x, int64_t nblocks, int64_t tiles,
+    const float* __restrict__ amax, int amax_is_wsf2, int force_exact,
+    u32x2* __restrict__ packed, uint8_t* __restrict__ wsf_out, float* __restrict__ wsf2_out) {
+    const float wsf2 = amax_is_wsf2 ? amax[0] : amax[0] / 2688.0f;
+    const float gs6 = 6.0f * wsf2;
+    if (wsf2_out && blockIdx.x == 0 && threadIdx.x == 0) wsf2_out[0] = wsf2;
+    for (int64_t t = blockIdx.x; t < tiles; t += gridDim.x)
+        quantize_tile_bf16(x, nblocks, t, wsf2, gs6, force_exact != 0, packed, wsf_out);
+}
+
+// Many tensors, one launch: a device-resident job table (sorted by tile_begin) maps the global
+// tile index to (tensor, local tile).
+__global__ __launch_bounds__(256) void nvfp4_quantize_multi_kernel(
+    const mo_nvfp4_job* __restrict__ jobs, int njobs, int64_t total_tiles, int amax_is_wsf2,
+    int force_exact) {
+    for (int64_t t = blockIdx.x; t < total_tiles; t += gridDim.x) {
+        int lo = 0, hi = njobs - 1;
+        while (lo < hi) {  // last job with tile_begin <= t
+            const int mid = (lo + hi + 1) >> 1;
+            if (jobs[mid].tile_begin <= t) lo = mid; else hi = mid - 1;
+        }
+        const mo_nvfp4_job jb = jobs[lo];
+        const float a = jb.amax[0];
+        const float wsf2 = amax_is_wsf2 ? a : a / 2688.0f;
+        if (jb.wsf2_out && t == jb.tile_begin && threadIdx.x == 0) jb.wsf2_out[0] = wsf2;
+        quantize_tile_bf16((const uint16_t*)jb.x, jb.elems >> 4, t - jb.tile_begin, wsf2,
+                           6.0f * wsf2, force_exact != 0, (u32x2*)jb.packed, jb.wsf);
+    }
+}
+
 static inline unsigned grid_for(int64_t chunks) {
     int64_t b = (chunks + 255) / 256;
     if (b < 1) b = 1;
@@ -224,6 +368,16 @@ extern "C" int mo_nvfp4_quantize(const void* x, int64_t rows, int64_t k, int dty
     if ((uintptr_t)packed & 3u) return MO_ERR_ARG;
     const int64_t kp = (k + block_size - 1) / block_size * block_size;
     hipStream_t s = (hipStream_t)stream;
+    if (dtype == MO_BF16 && block_size == 16 && k == kp && !wsf_in &&
+        (((uintptr_t)x & 15u) == 0) && (((uintptr_t)packed & 7u) == 0)) {
+        const int64_t nblocks = rows * k / 16;
+        const int64_t tiles = (nblocks + mo::kTileBlocks - 1) / mo::kTileBlocks;
+        const unsigned grid = (unsigned)(tiles < 8192 ? tiles : 8192);
+        mo::nvfp4_quantize_fast_kernel<<<grid, 256, 0, s>>>(
+            (const uint16_t*)x, nblocks, tiles, amax, amax_is_wsf2, mo_get_option(MO_OPT_FORCE_EXACT),
+            (mo::u32x2*)packed, wsf_out, wsf2_out);
+        return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+    }
 #define CALL(DT, BS) \
     mo::launch_quantize<DT, BS>(x, rows, k, kp, amax, amax_is_wsf2, wsf_in, packed, wsf_out, wsf2_out, s)
     MO_DISPATCH_DT_BS(dtype, block_size, CALL)
@@ -262,5 +416,18 @@ extern "C" int mo_nvfp4_qdq(const void* x, void* y, int64_t rows, int64_t k, int
 #define CALL(DT, BS) mo::launch_qdq<DT, BS>(x, y, rows, k, kp, amax, amax_dtype, mode, s)
     MO_DISPATCH_DT_BS(dtype, block_size, CALL)
 #undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs, int64_t total_tiles,
+                                       int dtype, int block_size, int amax_is_wsf2,
+                                       void* stream) {
+    if (njobs < 0 || total_tiles < 0) return MO_ERR_ARG;
+    if (dtype != MO_BF16 || block_size != 16) return MO_ERR_UNSUPPORTED;
+    if (njobs == 0 || total_tiles == 0) return MO_OK;
+    if (!jobs_dev) return MO_ERR_ARG;
+    const unsigned grid = (unsigned)(total_tiles < 8192 ? total_tiles : 8192);
+    mo::nvfp4_quantize_multi_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(
+        jobs_dev, njobs, total_tiles, amax_is_wsf2, mo_get_option(MO_OPT_FORCE_EXACT));
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

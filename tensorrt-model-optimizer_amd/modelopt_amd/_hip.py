@@ -21,7 +21,11 @@ _P, _I64, _INT = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 SIGNATURES = {
     "mo_version": [],
     "mo_error_string": [_INT],
+    "mo_set_option": [_INT, _INT],
+    "mo_get_option": [_INT],
     "mo_absmax": [_P, _I64, _I64, _I64, _INT, _P, _P],
+    "mo_absmax_multi": [_P, _INT, _I64, _INT, _P],
+    "mo_nvfp4_quantize_multi": [_P, _INT, _I64, _INT, _INT, _INT, _P],
     "mo_fp8_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _P],
     "mo_int_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _INT, _P],
     "mo_nvfp4_qdq": [_P, _P, _I64, _I64, _INT, _P, _INT, _INT, _INT, _P],
@@ -162,3 +166,94 @@ def nvfp4_dequantize(packed, wsf, wsf2, block_size, dtype):
     call("mo_nvfp4_dequantize", packed, _ptr(packed), _ptr(wsf.view(torch.uint8)), _ptr(wsf2),
          rows, kp, block_size, _ptr(y), dtype_code(dtype), _stream(packed))
     return y
+
+
+# ----------------------------------------------------------------------------- options
+
+MO_OPT_FORCE_EXACT = 0
+
+
+def set_option(key: int, value: int):
+    rc = load().mo_set_option(key, value)
+    if rc != 0:
+        raise RuntimeError(f"mo_set_option({key}) failed with status {rc}")
+
+
+# ----------------------------------------------------------------------------- multi-tensor plans
+
+ABSMAX_TILE_ELEMS = 32768
+NVFP4_TILE_ELEMS = 16384
+
+
+def _job_table(rows, device):
+    """rows: list of equal-length int tuples -> device int64 tensor [n, len] (the job structs)."""
+    return torch.tensor(rows, dtype=torch.int64).to(device)
+
+
+class AbsmaxPlan:
+    """Per-tensor abs-max of a fixed list of tensors in one launch.
+
+    ``acc`` is a float32 vector with one running maximum per tensor (zero it for a fresh
+    reduction).  The plan keeps the tensors alive and must be rebuilt if any is reallocated.
+    """
+
+    def __init__(self, tensors):
+        assert len(tensors) > 0
+        dev, dt = tensors[0].device, tensors[0].dtype
+        self.tensors = list(tensors)
+        self.dtype = dtype_code(dt)
+        self.acc = torch.zeros(len(tensors), dtype=torch.float32, device=dev)
+        rows, tile = [], 0
+        for i, t in enumerate(tensors):
+            _require_device(t)
+            if t.device != dev or t.dtype != dt or not t.is_contiguous() or t.data_ptr() % 16:
+                raise ValueError("AbsmaxPlan needs contiguous, 16-byte aligned tensors of one dtype/device")
+            rows.append((t.data_ptr(), self.acc.data_ptr() + 4 * i, t.numel(), tile))
+            tile += -(-t.numel() // ABSMAX_TILE_ELEMS)
+        self.total_tiles = tile
+        self.jobs = _job_table(rows, dev)
+
+    def run(self, zero=True):
+        if zero:
+            self.acc.zero_()
+        call("mo_absmax_multi", self.acc, _ptr(self.jobs), len(self.tensors), self.total_tiles,
+             self.dtype, _stream(self.acc))
+        return self.acc
+
+
+class Nvfp4QuantizePlan:
+    """NVFP4 quantize + pack of a fixed list of bf16 tensors (last dim % 16 == 0) in one launch.
+
+    ``amax`` is a float32 device vector with one global amax (or wsf2 when ``amax_is_wsf2``) per
+    tensor.  Outputs are allocated once here: ``packed[i]`` uint8 [..., K/2], ``wsf[i]``
+    float8_e4m3fn [..., K/16], ``wsf2`` float32 [n].
+    """
+
+    def __init__(self, tensors, amax, amax_is_wsf2=False):
+        assert len(tensors) > 0 and amax.dtype == torch.float32 and amax.numel() == len(tensors)
+        dev = tensors[0].device
+        self.tensors, self.amax, self.amax_is_wsf2 = list(tensors), amax, bool(amax_is_wsf2)
+        self.wsf2 = torch.empty(len(tensors), dtype=torch.float32, device=dev)
+        self.packed, self._wsf_u8 = [], []
+        rows, tile = [], 0
+        for i, t in enumerate(tensors):
+            _require_device(t)
+            if (t.dtype != torch.bfloat16 or not t.is_contiguous() or t.shape[-1] % 16
+                    or t.data_ptr() % 16 or t.device != dev):
+                raise ValueError("Nvfp4QuantizePlan needs contiguous bf16 tensors with last dim % 16 == 0")
+            lead = tuple(t.shape[:-1])
+            p = torch.empty(lead + (t.shape[-1] // 2,), dtype=torch.uint8, device=dev)
+            w = torch.empty(lead + (t.shape[-1] // 16,), dtype=torch.uint8, device=dev)
+            self.packed.append(p)
+            self._wsf_u8.append(w)
+            rows.append((t.data_ptr(), p.data_ptr(), w.data_ptr(), amax.data_ptr() + 4 * i,
+                         self.wsf2.data_ptr() + 4 * i, t.numel(), tile, 0))
+            tile += -(-t.numel() // NVFP4_TILE_ELEMS)
+        self.total_tiles = tile
+        self.jobs = _job_table(rows, dev)
+        self.wsf = [w.view(torch.float8_e4m3fn) for w in self._wsf_u8]
+
+    def run(self):
+        call("mo_nvfp4_quantize_multi", self.amax, _ptr(self.jobs), len(self.tensors),
+             self.total_tiles, MO_BF16, 16, int(self.amax_is_wsf2), _stream(self.amax))
+        return self.packed, self.wsf, self.wsf2

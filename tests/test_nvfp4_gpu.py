@@ -57,3 +57,105 @@ def test_fake_quant_matches_oracle(dtype, mode, shape):
         kp = p.shape[-1] * 2
         y_o = qtensor.nvfp4_dequantize(p, wsf, wsf2, 16, (shape[0], kp), dtype)[:, : shape[1]]
     assert_bits_equal(y.cpu(), y_o.contiguous(), f"qdq mode {mode}")
+
+
+def _edge_tensor():
+    """bf16 [rows, 64] rows built to hit every E2M1 tie, zero blocks, signed zeros, tiny values."""
+    rows = []
+    ties = [0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0]
+    base = torch.tensor(ties + [-t for t in ties])
+    for s in (1.0, 0.5, 0.0234375, 3.0, 448.0, 2.0 ** -20):
+        rows.append(torch.cat([base * s, (base + 0.1) * s, (base - 0.1) * s, base * s * 1.5]))
+    rows.append(torch.zeros(64))
+    z = torch.zeros(64); z[0] = -0.0; z[5] = 1e-30; z[6] = -1e-30; z[17] = 6.0; z[18] = -2.0 ** -126
+    rows.append(z)
+    z2 = torch.full((64,), -0.0); rows.append(z2)
+    return torch.stack(rows).to(torch.bfloat16)
+
+
+def test_edge_cases_match_oracle():
+    x = _edge_tensor()
+    for bs in (16,):
+        po, wo, w2o = qtensor.nvfp4_quantize(x, bs)
+        xd = x.to(DEV)
+        p, w, w2 = _hip.nvfp4_quantize(xd, _gpu_amax(xd).reshape(()), bs)
+        assert_bits_equal(w.cpu(), wo, "wsf")
+        assert_bits_equal(p.cpu(), po, "packed")
+
+
+def test_all_zero_tensor_matches_x86_nan_sign():
+    x = torch.zeros(4, 32, dtype=torch.bfloat16)
+    po, wo, w2o = qtensor.nvfp4_quantize(x, 16)
+    xd = x.to(DEV)
+    p, w, w2 = _hip.nvfp4_quantize(xd, _gpu_amax(xd).reshape(()), 16)
+    assert_bits_equal(w.cpu(), wo, "wsf")
+    assert_bits_equal(p.cpu(), po, "packed")
+
+
+@pytest.mark.parametrize("special", [float("nan"), float("inf"), -float("inf")])
+def test_nonfinite_inputs(special):
+    x = _rand((8, 64), torch.bfloat16, 3)
+    x[1, 3] = special
+    amax = torch.tensor(0.1, dtype=torch.bfloat16)  # a calibrated amax, as the export path passes
+    wsf2 = amax.float() / (6.0 * 448.0)
+    wo, _ = qtensor.nvfp4_block_scales(x, 16, wsf2)
+    po, _, _ = qtensor.nvfp4_quantize(x, 16, wo, wsf2)
+    xd = x.to(DEV)
+    p, w, w2 = _hip.nvfp4_quantize(xd, amax.float().to(DEV), 16)
+    assert_bits_equal(w.cpu(), wo, "wsf")
+    assert_bits_equal(p.cpu(), po, "packed")
+
+
+def test_all_bf16_patterns_against_oracle():
+    """Every bf16 bit pattern as an element, in blocks whose scale is set by a pilot value."""
+    allv = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    finite = allv[torch.isfinite(allv.float())]
+    finite = finite[: finite.numel() // 15 * 15].reshape(-1, 15)
+    for pilot in (1.0, 0.013, 300.0):
+        col = torch.full((finite.shape[0], 1), pilot, dtype=torch.bfloat16)
+        x = torch.cat([col, finite], dim=1).contiguous()
+        # clip magnitudes so the pilot stays the block maximum for most rows; others are fine too
+        amax = torch.tensor(pilot * 4, dtype=torch.bfloat16)
+        wsf2 = amax.float() / (6.0 * 448.0)
+        wo, _ = qtensor.nvfp4_block_scales(x, 16, wsf2)
+        po, _, _ = qtensor.nvfp4_quantize(x, 16, wo, wsf2)
+        xd = x.to(DEV)
+        p, w, w2 = _hip.nvfp4_quantize(xd, amax.float().to(DEV), 16)
+        assert_bits_equal(w.cpu(), wo, f"wsf pilot={pilot}")
+        assert_bits_equal(p.cpu(), po, f"packed pilot={pilot}")
+
+
+def test_fast_path_equals_exact_division_on_large_input():
+    """Same GPU, same input: multiply-and-verify codes == literal per-element division codes."""
+    g = torch.Generator(device=DEV).manual_seed(11)
+    x = (0.02 * torch.randn(8192, 8192, generator=g, device=DEV)).to(torch.bfloat16)
+    amax = _gpu_amax(x).reshape(())
+    p_fast, w_fast, _ = _hip.nvfp4_quantize(x, amax, 16)
+    _hip.set_option(_hip.MO_OPT_FORCE_EXACT, 1)
+    try:
+        p_exact, w_exact, _ = _hip.nvfp4_quantize(x, amax, 16)
+    finally:
+        _hip.set_option(_hip.MO_OPT_FORCE_EXACT, 0)
+    assert torch.equal(w_fast.view(torch.uint8), w_exact.view(torch.uint8))
+    assert torch.equal(p_fast, p_exact)
+    # and against the oracle on a slice the CPU finishes quickly
+    po, wo, _ = qtensor.nvfp4_quantize(x[:512].cpu(), 16, wsf2=(amax.cpu() / 2688.0))
+    assert_bits_equal(p_fast[:512].cpu(), po, "packed slice")
+
+
+def test_multi_tensor_plan_matches_single_calls():
+    shapes = [(256, 512), (64, 4096), (1000, 48), (3, 16)]
+    xs = [_rand(s, torch.bfloat16, 20 + i).to(DEV) for i, s in enumerate(shapes)]
+    aplan = _hip.AbsmaxPlan(xs)
+    acc = aplan.run().clone()
+    for i, x in enumerate(xs):
+        assert_bits_equal(acc[i].cpu(), _gpu_amax(x).cpu().reshape(()), f"amax {i}")
+    qplan = _hip.Nvfp4QuantizePlan(xs, acc)
+    packed, wsf, wsf2 = qplan.run()
+    for i, x in enumerate(xs):
+        p, w, w2 = _hip.nvfp4_quantize(x, acc[i], 16)
+        assert torch.equal(packed[i], p) and torch.equal(wsf[i].view(torch.uint8), w.view(torch.uint8))
+        assert_bits_equal(wsf2[i].cpu(), w2.cpu(), "wsf2")
+        po, wo, w2o = qtensor.nvfp4_quantize(x.cpu(), 16)
+        assert_bits_equal(packed[i].cpu(), po, f"packed {i}")
+        assert_bits_equal(wsf[i].cpu(), wo, f"wsf {i}")
