@@ -163,23 +163,33 @@ __global__ __launch_bounds__(256) void nvfp4_qdq_kernel(const void* __restrict__
 // loads, one 8-byte store of codes, one scale byte).
 //
 // The reference divides every element by the block's scale s with an IEEE fp32 division and
-// rounds the quotient to E2M1.  Here the per-element division is replaced by a multiply with
-// r4 = 4 / s (one IEEE division per block) and the result is *proved* equal before it is used:
-// with u = |x| * r4 the seven rounding boundaries of E2M1 sit at the integers 1, 3, 5, 7, 10,
-// 14, 20, and u differs from 4 * (x / s) by less than 2^-22 relative, while a correctly rounded
-// quotient can only change sides within 2^-24 relative of a boundary.  So whenever u is further
-// than u * 2^-21 from the nearest integer the code computed from u is the reference's code; the
-// (rare) lanes that fail that test, and blocks whose scale is outside [2^-64, 2^10] or whose
-// abs-max is not finite, recompute their block with the exact division.
+// rounds the quotient to E2M1 (ties to even).  The quotient is reproduced exactly, without the
+// general division sequence, from one correctly rounded reciprocal per block:
+//     r  = RN(1 / s)                       (IEEE division, once per block)
+//     q0 = RN(x * r)                       error <= 1.5 ulp
+//     q1 = RN(q0 + RN(x - s * q0) * r)     faithful (the residual is exact in an FMA)
+//     q  = RN(q1 + RN(x - s * q1) * r)     = RN(x / s)   (Markstein's theorem: a faithful
+//                                          quotient and a correctly rounded reciprocal give the
+//                                          correctly rounded quotient after one FMA correction)
+// valid when nothing over- or underflows; blocks whose scale is outside [2^-64, 2^10], whose
+// abs-max is not finite or whose largest quotient would overflow take the general division.
+// The hardware E2M1 conversion (round to nearest even, saturating) of q then yields the
+// reference's code; a -0.0 input is the one place where the reference's sign rule (v < 0)
+// and the hardware's (sign bit) differ, and q is +0.0 there because x - s * q0 is +0.0.
 __device__ __forceinline__ uint32_t fp4_pair(uint32_t old, float a, float b, int sel) {
-    // v_cvt_scalef32_pk_fp4_f32: two fp32 -> two E2M1 codes (round to nearest even, saturating)
-    // written to byte `sel` of `old`; the inputs are divided by the (power of two) scale.
+    // v_cvt_scalef32_pk_fp4_f32: two fp32 -> two E2M1 codes written to byte `sel` of `old`
     switch (sel) {
-        case 0: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 4.0f, 0);
-        case 1: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 4.0f, 1);
-        case 2: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 4.0f, 2);
-        default: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 4.0f, 3);
+        case 0: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, 0);
+        case 1: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, 1);
+        case 2: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, 2);
+        default: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, 3);
     }
+}
+
+__device__ __forceinline__ float exact_quotient(float x, float s, float r) {
+    const float q0 = x * r;
+    const float q1 = __builtin_fmaf(__builtin_fmaf(-s, q0, x), r, q0);
+    return __builtin_fmaf(__builtin_fmaf(-s, q1, x), r, q1);
 }
 
 __device__ __forceinline__ uint32_t exact_codes8(const uint32_t (&w)[4], float s) {
@@ -204,32 +214,20 @@ __device__ __forceinline__ void quantize_block16_bf16(const uint32_t (&w)[8], fl
     byte = block_scale_byte(bmax, gs6);
     const float s = e4m3_to_f32(byte) * wsf2;
     const uint32_t sb = f2u(s);
-    bool fast = !force_exact && sb >= 0x1F800000u && sb <= 0x44800000u && h < 0x7F80u;
-    const float r4 = 4.0f * (1.0f / s);
-    fast = fast && (bmax * r4 < 3.0e38f);
-    bool redo = !fast;
+    const float r = 1.0f / s;
+    const bool fast = !force_exact && sb >= 0x1F800000u && sb <= 0x44800000u && h < 0x7F80u &&
+                      (bmax * r < 1.0e38f);
     if (fast) {
-        float emin = 1.0f;
         uint32_t lo = 0, hi = 0;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            // + 0.0f turns a -0.0 product into +0.0, the reference's unsigned zero code
-            const float u0 = __builtin_fmaf(u2f(w[j] << 16), r4, 0.0f);
-            const float u1 = __builtin_fmaf(u2f(w[j] & 0xFFFF0000u), r4, 0.0f);
-            const float a0 = __builtin_fabsf(u0), a1 = __builtin_fabsf(u1);
-            const float d0 = __builtin_fabsf(a0 - __builtin_rintf(a0));
-            const float d1 = __builtin_fabsf(a1 - __builtin_rintf(a1));
-            const float e0 = __builtin_fmaf(a0, -4.76837158203125e-7f, d0);  // 2^-21
-            const float e1 = __builtin_fmaf(a1, -4.76837158203125e-7f, d1);
-            emin = __builtin_fminf(emin, __builtin_fminf(e0, e1));
-            if (j < 4) lo = fp4_pair(lo, u0, u1, j);
-            else hi = fp4_pair(hi, u0, u1, j - 4);
+            const float q0 = exact_quotient(u2f(w[j] << 16), s, r);
+            const float q1 = exact_quotient(u2f(w[j] & 0xFFFF0000u), s, r);
+            if (j < 4) lo = fp4_pair(lo, q0, q1, j);
+            else hi = fp4_pair(hi, q0, q1, j - 4);
         }
         c_lo = lo; c_hi = hi;
-        // e == 0 only for u == 0 (exact zero, no boundary near); e < 0 means "too close"
-        redo = !(emin >= 0.0f);
-    }
-    if (redo) {
+    } else {
         const uint32_t w0[4] = {w[0], w[1], w[2], w[3]}, w1[4] = {w[4], w[5], w[6], w[7]};
         c_lo = exact_codes8(w0, s);
         c_hi = exact_codes8(w1, s);
