@@ -59,7 +59,9 @@ int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dty
 
 /* Per-tensor abs-max of many tensors in ONE launch.  jobs_dev is a device-resident table sorted
  * by tile_begin; job j owns tiles [tile_begin_j, tile_begin_j + ceil(elems_j /
- * MO_ABSMAX_TILE_ELEMS)), total_tiles is the sum.  acc as for mo_absmax (one fp32 per job).
+ * MO_ABSMAX_TILE_ELEMS)), total_tiles is the sum (< 2^31).  tile_job_dev[t] = index of the job
+ * that owns tile t (device int32[total_tiles]); NULL makes every workgroup binary-search the
+ * table instead.  acc as for mo_absmax (one fp32 per job).
  * Every x must be 16-byte aligned.  No counterpart in the reference, which loops over modules
  * in Python (MaxCalibrator.collect per weight, TQ/nn/modules/quant_module.py:148-169). */
 #define MO_ABSMAX_TILE_ELEMS 32768
@@ -69,8 +71,8 @@ typedef struct mo_absmax_job {
     int64_t elems;
     int64_t tile_begin;
 } mo_absmax_job;
-int mo_absmax_multi(const mo_absmax_job* jobs_dev, int njobs, int64_t total_tiles, int dtype,
-                    void* stream);
+int mo_absmax_multi(const mo_absmax_job* jobs_dev, int njobs, const int32_t* tile_job_dev,
+                    int64_t total_tiles, int dtype, void* stream);
 
 /* ------------------------------------------------------------------ fake quantisation
  * x and y are viewed as [outer, axis, inner]; amax has `axis` elements of type amax_dtype
@@ -126,7 +128,8 @@ int mo_nvfp4_quantize(const void* x, int64_t rows, int64_t k, int dtype, int blo
 /* NVFP4 quantize + pack of many tensors in ONE launch (the whole-model export pass of
  * modelopt/torch/export/unified_export_hf.py:233-391, which calls to_quantized_weight once per
  * linear).  jobs_dev: device-resident table sorted by tile_begin; job j owns tiles
- * [tile_begin_j, tile_begin_j + ceil(elems_j / MO_NVFP4_TILE_ELEMS)).  Requirements per job:
+ * [tile_begin_j, tile_begin_j + ceil(elems_j / MO_NVFP4_TILE_ELEMS)); tile_job_dev as for
+ * mo_absmax_multi (optional tile -> job index map).  Requirements per job:
  * bf16, block size 16, last dim a multiple of 16 (so elems % 16 == 0 and no padding), x 16-byte
  * and packed 8-byte aligned.  Outputs and amax as for mo_nvfp4_quantize. */
 #define MO_NVFP4_TILE_ELEMS 16384
@@ -140,8 +143,9 @@ typedef struct mo_nvfp4_job {
     int64_t tile_begin;
     int64_t reserved;
 } mo_nvfp4_job;
-int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs, int64_t total_tiles,
-                            int dtype, int block_size, int amax_is_wsf2, void* stream);
+int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs, const int32_t* tile_job_dev,
+                            int64_t total_tiles, int dtype, int block_size, int amax_is_wsf2,
+                            void* stream);
 
 /* NVFP4 unpack + rescale.  Replaces NVFP4QTensor.dequantize (TQ/qtensor/nvfp4_tensor.py
  * :234-297) and fp4_dequantize (TQ/triton/fp4_kernel.py:307):

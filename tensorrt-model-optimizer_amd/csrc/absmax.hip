@@ -171,34 +171,39 @@ __global__ __launch_bounds__(256) void absmax_cols_kernel(const void* __restrict
 // ------------------------------------------------------------------------------ many tensors
 template <int DT>
 __global__ __launch_bounds__(256) void absmax_multi_kernel(const mo_absmax_job* __restrict__ jobs,
-                                                           int njobs, int64_t total_tiles) {
+                                                           int njobs,
+                                                           const int32_t* __restrict__ tile_job) {
     __shared__ uint32_t smem[4];
     constexpr int64_t kTileChunks = MO_ABSMAX_TILE_ELEMS / 8;
-    for (int64_t t = blockIdx.x; t < total_tiles; t += gridDim.x) {
-        int lo = 0, hi = njobs - 1;
+    const int64_t t = blockIdx.x;  // one workgroup per tile, dispatched in tile order
+    int lo;
+    if (tile_job) {
+        lo = tile_job[t];
+    } else {
+        lo = 0;
+        int hi = njobs - 1;
         while (lo < hi) {  // last job with tile_begin <= t
             const int mid = (lo + hi + 1) >> 1;
             if (jobs[mid].tile_begin <= t) lo = mid; else hi = mid - 1;
         }
-        const mo_absmax_job jb = jobs[lo];
-        const int64_t chunks = jb.elems >> 3;
-        const int64_t c0 = (t - jb.tile_begin) * kTileChunks;
-        int64_t c1 = c0 + kTileChunks;
-        if (c1 > chunks) c1 = chunks;
-        AbsAcc<DT> a;
-        int64_t c = c0 + threadIdx.x;
-        for (; c + 768 < c1; c += 1024) {
-            a.chunk(jb.x, c << 3);
-            a.chunk(jb.x, (c + 256) << 3);
-            a.chunk(jb.x, (c + 512) << 3);
-            a.chunk(jb.x, (c + 768) << 3);
-        }
-        for (; c < c1; c += 256) a.chunk(jb.x, c << 3);
-        if (c1 == chunks && threadIdx.x < (jb.elems & 7)) a.elem(jb.x, (chunks << 3) + threadIdx.x);
-        __syncthreads();  // smem reuse across tiles
-        const uint32_t v = block_max_u32(a.bits(), smem);
-        if (threadIdx.x == 0 && v) atomicMax((uint32_t*)jb.acc, v);
     }
+    const mo_absmax_job jb = jobs[lo];
+    const int64_t chunks = jb.elems >> 3;
+    const int64_t c0 = (t - jb.tile_begin) * kTileChunks;
+    int64_t c1 = c0 + kTileChunks;
+    if (c1 > chunks) c1 = chunks;
+    AbsAcc<DT> a;
+    int64_t c = c0 + threadIdx.x;
+    for (; c + 768 < c1; c += 1024) {
+        a.chunk(jb.x, c << 3);
+        a.chunk(jb.x, (c + 256) << 3);
+        a.chunk(jb.x, (c + 512) << 3);
+        a.chunk(jb.x, (c + 768) << 3);
+    }
+    for (; c < c1; c += 256) a.chunk(jb.x, c << 3);
+    if (c1 == chunks && threadIdx.x < (jb.elems & 7)) a.elem(jb.x, (chunks << 3) + threadIdx.x);
+    const uint32_t v = block_max_u32(a.bits(), smem);
+    if (threadIdx.x == 0 && v) atomicMax((uint32_t*)jb.acc, v);
 }
 
 template <int DT>
@@ -279,17 +284,18 @@ extern "C" int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }
 
-extern "C" int mo_absmax_multi(const mo_absmax_job* jobs_dev, int njobs, int64_t total_tiles,
-                               int dtype, void* stream) {
-    if (njobs < 0 || total_tiles < 0) return MO_ERR_ARG;
+extern "C" int mo_absmax_multi(const mo_absmax_job* jobs_dev, int njobs,
+                               const int32_t* tile_job_dev, int64_t total_tiles, int dtype,
+                               void* stream) {
+    if (njobs < 0 || total_tiles < 0 || total_tiles > 0x7FFFFFFF) return MO_ERR_ARG;
     if (njobs == 0 || total_tiles == 0) return MO_OK;
     if (!jobs_dev) return MO_ERR_ARG;
-    const unsigned grid = (unsigned)(total_tiles < 4096 ? total_tiles : 4096);
+    const unsigned grid = (unsigned)total_tiles;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case MO_F32: mo::absmax_multi_kernel<MO_F32><<<grid, 256, 0, s>>>(jobs_dev, njobs, total_tiles); break;
-        case MO_F16: mo::absmax_multi_kernel<MO_F16><<<grid, 256, 0, s>>>(jobs_dev, njobs, total_tiles); break;
-        case MO_BF16: mo::absmax_multi_kernel<MO_BF16><<<grid, 256, 0, s>>>(jobs_dev, njobs, total_tiles); break;
+        case MO_F32: mo::absmax_multi_kernel<MO_F32><<<grid, 256, 0, s>>>(jobs_dev, njobs, tile_job_dev); break;
+        case MO_F16: mo::absmax_multi_kernel<MO_F16><<<grid, 256, 0, s>>>(jobs_dev, njobs, tile_job_dev); break;
+        case MO_BF16: mo::absmax_multi_kernel<MO_BF16><<<grid, 256, 0, s>>>(jobs_dev, njobs, tile_job_dev); break;
         default: return MO_ERR_DTYPE;
     }
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;

@@ -234,34 +234,55 @@ __device__ __forceinline__ void quantize_block16_bf16(const uint32_t (&w)[8], fl
     }
 }
 
-// Tiles of kTileBlocks 16-element blocks; a workgroup of 256 lanes handles a tile in
-// kTileBlocks / 256 rounds with all loads of a round issued before its math.
+// Tiles of kTileBlocks 16-element blocks handled by a workgroup of 256 lanes.
+//
+// Loads are fully coalesced (lane t of a round reads chunk t, so a wavefront instruction reads
+// 1 KiB of contiguous memory); a block's two chunks then sit in adjacent lanes.  Rounds are
+// processed in pairs (A, B): the even lane of each pair keeps its A chunk and takes its
+// neighbour's A chunk (it now owns a whole round-A block), the odd lane keeps B and takes the
+// neighbour's B chunk.  The swap is one DPP move per dword (no LDS).  Every lane therefore
+// does the per-block work once for 16 elements, and stores 8 bytes of codes + 1 scale byte.
 constexpr int kTileBlocks = MO_NVFP4_TILE_ELEMS / 16;
+
+__device__ __forceinline__ uint32_t swap_adjacent_lanes(uint32_t v) {
+    // quad_perm [1, 0, 3, 2]
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);
+}
 
 __device__ __forceinline__ void quantize_tile_bf16(const uint16_t* __restrict__ x,
                                                    int64_t nblocks, int64_t tile, float wsf2,
                                                    float gs6, bool force_exact,
                                                    u32x2* __restrict__ packed,
                                                    uint8_t* __restrict__ wsf) {
-    constexpr int R = kTileBlocks / 256;
-    const int64_t b0 = tile * kTileBlocks + threadIdx.x;
-    u32x4 a[R], b[R];
+    constexpr int RP = kTileBlocks / 256;  // round pairs
+    const int64_t nchunks = nblocks * 2;
+    const int64_t c0 = tile * (kTileBlocks * 2) + threadIdx.x;
+    const bool odd = threadIdx.x & 1;
+    u32x4 a[RP], b[RP];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int64_t blk = b0 + r * 256;
-        if (blk < nblocks) {
-            const u32x4* p = (const u32x4*)(x + blk * 16);
-            a[r] = __builtin_nontemporal_load(p);
-            b[r] = __builtin_nontemporal_load(p + 1);
-        }
+    for (int p = 0; p < RP; ++p) {
+        const int64_t ca = c0 + p * 512, cb = ca + 256;
+        const u32x4 zero = {0, 0, 0, 0};
+        a[p] = ca < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + ca * 8)) : zero;
+        b[p] = cb < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + cb * 8)) : zero;
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int64_t blk = b0 + r * 256;
-        if (blk < nblocks) {
-            const uint32_t w[8] = {a[r].x, a[r].y, a[r].z, a[r].w, b[r].x, b[r].y, b[r].z, b[r].w};
-            uint32_t byte, lo, hi;
-            quantize_block16_bf16(w, wsf2, gs6, force_exact, byte, lo, hi);
+    for (int p = 0; p < RP; ++p) {
+        const int64_t ca = c0 + p * 512, cb = ca + 256;
+        const u32x4 send = odd ? a[p] : b[p];
+        u32x4 recv;
+        recv.x = swap_adjacent_lanes(send.x);
+        recv.y = swap_adjacent_lanes(send.y);
+        recv.z = swap_adjacent_lanes(send.z);
+        recv.w = swap_adjacent_lanes(send.w);
+        const u32x4 first = odd ? recv : a[p], second = odd ? b[p] : recv;
+        const uint32_t w[8] = {first.x, first.y, first.z, first.w,
+                               second.x, second.y, second.z, second.w};
+        uint32_t byte, lo, hi;
+        quantize_block16_bf16(w, wsf2, gs6, force_exact, byte, lo, hi);
+        const int64_t mine = odd ? cb : ca;  // odd: chunks (cb - 1, cb); even: (ca, ca + 1)
+        if (mine < nchunks) {
+            const int64_t blk = mine >> 1;
             u32x2 o = {lo, hi};
             __builtin_nontemporal_store(o, packed + blk);
             wsf[blk] = (uint8_t)byte;
@@ -276,28 +297,34 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_fast_kernel(
     const float wsf2 = amax_is_wsf2 ? amax[0] : amax[0] / 2688.0f;
     const float gs6 = 6.0f * wsf2;
     if (wsf2_out && blockIdx.x == 0 && threadIdx.x == 0) wsf2_out[0] = wsf2;
-    for (int64_t t = blockIdx.x; t < tiles; t += gridDim.x)
-        quantize_tile_bf16(x, nblocks, t, wsf2, gs6, force_exact != 0, packed, wsf_out);
+    quantize_tile_bf16(x, nblocks, blockIdx.x, wsf2, gs6, force_exact != 0, packed, wsf_out);
 }
 
-// Many tensors, one launch: a device-resident job table (sorted by tile_begin) maps the global
-// tile index to (tensor, local tile).
+// Many tensors, one launch.  One workgroup per tile, dispatched in tile order so the set of
+// tiles in flight stays a compact window of memory (a persistent grid drifts apart over a
+// multi-gigabyte pass and loses ~10 % of the bandwidth).  tile_job[t] names the tensor of tile
+// t; without it the job is found by binary search over tile_begin.
 __global__ __launch_bounds__(256) void nvfp4_quantize_multi_kernel(
-    const mo_nvfp4_job* __restrict__ jobs, int njobs, int64_t total_tiles, int amax_is_wsf2,
-    int force_exact) {
-    for (int64_t t = blockIdx.x; t < total_tiles; t += gridDim.x) {
-        int lo = 0, hi = njobs - 1;
+    const mo_nvfp4_job* __restrict__ jobs, int njobs, const int32_t* __restrict__ tile_job,
+    int amax_is_wsf2, int force_exact) {
+    const int64_t t = blockIdx.x;
+    int lo;
+    if (tile_job) {
+        lo = tile_job[t];
+    } else {
+        lo = 0;
+        int hi = njobs - 1;
         while (lo < hi) {  // last job with tile_begin <= t
             const int mid = (lo + hi + 1) >> 1;
             if (jobs[mid].tile_begin <= t) lo = mid; else hi = mid - 1;
         }
-        const mo_nvfp4_job jb = jobs[lo];
-        const float a = jb.amax[0];
-        const float wsf2 = amax_is_wsf2 ? a : a / 2688.0f;
-        if (jb.wsf2_out && t == jb.tile_begin && threadIdx.x == 0) jb.wsf2_out[0] = wsf2;
-        quantize_tile_bf16((const uint16_t*)jb.x, jb.elems >> 4, t - jb.tile_begin, wsf2,
-                           6.0f * wsf2, force_exact != 0, (u32x2*)jb.packed, jb.wsf);
     }
+    const mo_nvfp4_job jb = jobs[lo];
+    const float a = jb.amax[0];
+    const float wsf2 = amax_is_wsf2 ? a : a / 2688.0f;
+    if (jb.wsf2_out && t == jb.tile_begin && threadIdx.x == 0) jb.wsf2_out[0] = wsf2;
+    quantize_tile_bf16((const uint16_t*)jb.x, jb.elems >> 4, t - jb.tile_begin, wsf2, 6.0f * wsf2,
+                       force_exact != 0, (u32x2*)jb.packed, jb.wsf);
 }
 
 static inline unsigned grid_for(int64_t chunks) {
@@ -370,8 +397,8 @@ extern "C" int mo_nvfp4_quantize(const void* x, int64_t rows, int64_t k, int dty
         (((uintptr_t)x & 15u) == 0) && (((uintptr_t)packed & 7u) == 0)) {
         const int64_t nblocks = rows * k / 16;
         const int64_t tiles = (nblocks + mo::kTileBlocks - 1) / mo::kTileBlocks;
-        const unsigned grid = (unsigned)(tiles < 8192 ? tiles : 8192);
-        mo::nvfp4_quantize_fast_kernel<<<grid, 256, 0, s>>>(
+        if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+        mo::nvfp4_quantize_fast_kernel<<<(unsigned)tiles, 256, 0, s>>>(
             (const uint16_t*)x, nblocks, tiles, amax, amax_is_wsf2, mo_get_option(MO_OPT_FORCE_EXACT),
             (mo::u32x2*)packed, wsf_out, wsf2_out);
         return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
@@ -417,15 +444,15 @@ extern "C" int mo_nvfp4_qdq(const void* x, void* y, int64_t rows, int64_t k, int
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }
 
-extern "C" int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs, int64_t total_tiles,
+extern "C" int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs,
+                                       const int32_t* tile_job_dev, int64_t total_tiles,
                                        int dtype, int block_size, int amax_is_wsf2,
                                        void* stream) {
-    if (njobs < 0 || total_tiles < 0) return MO_ERR_ARG;
+    if (njobs < 0 || total_tiles < 0 || total_tiles > 0x7FFFFFFF) return MO_ERR_ARG;
     if (dtype != MO_BF16 || block_size != 16) return MO_ERR_UNSUPPORTED;
     if (njobs == 0 || total_tiles == 0) return MO_OK;
     if (!jobs_dev) return MO_ERR_ARG;
-    const unsigned grid = (unsigned)(total_tiles < 8192 ? total_tiles : 8192);
-    mo::nvfp4_quantize_multi_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(
-        jobs_dev, njobs, total_tiles, amax_is_wsf2, mo_get_option(MO_OPT_FORCE_EXACT));
+    mo::nvfp4_quantize_multi_kernel<<<(unsigned)total_tiles, 256, 0, (hipStream_t)stream>>>(
+        jobs_dev, njobs, tile_job_dev, amax_is_wsf2, mo_get_option(MO_OPT_FORCE_EXACT));
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

@@ -24,8 +24,8 @@ SIGNATURES = {
     "mo_set_option": [_INT, _INT],
     "mo_get_option": [_INT],
     "mo_absmax": [_P, _I64, _I64, _I64, _INT, _P, _P],
-    "mo_absmax_multi": [_P, _INT, _I64, _INT, _P],
-    "mo_nvfp4_quantize_multi": [_P, _INT, _I64, _INT, _INT, _INT, _P],
+    "mo_absmax_multi": [_P, _INT, _P, _I64, _INT, _P],
+    "mo_nvfp4_quantize_multi": [_P, _INT, _P, _I64, _INT, _INT, _INT, _P],
     "mo_fp8_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _P],
     "mo_int_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _INT, _P],
     "mo_nvfp4_qdq": [_P, _P, _I64, _I64, _INT, _P, _INT, _INT, _INT, _P],
@@ -190,6 +190,12 @@ def _job_table(rows, device):
     return torch.tensor(rows, dtype=torch.int64).to(device)
 
 
+def _tile_job_map(tiles_per_job, device):
+    """int32[total_tiles]: index of the job that owns each tile."""
+    counts = torch.tensor(tiles_per_job, dtype=torch.int64)
+    return torch.repeat_interleave(torch.arange(len(tiles_per_job), dtype=torch.int32), counts).to(device)
+
+
 class AbsmaxPlan:
     """Per-tensor abs-max of a fixed list of tensors in one launch.
 
@@ -203,21 +209,23 @@ class AbsmaxPlan:
         self.tensors = list(tensors)
         self.dtype = dtype_code(dt)
         self.acc = torch.zeros(len(tensors), dtype=torch.float32, device=dev)
-        rows, tile = [], 0
+        rows, tile, per_job = [], 0, []
         for i, t in enumerate(tensors):
             _require_device(t)
             if t.device != dev or t.dtype != dt or not t.is_contiguous() or t.data_ptr() % 16:
                 raise ValueError("AbsmaxPlan needs contiguous, 16-byte aligned tensors of one dtype/device")
             rows.append((t.data_ptr(), self.acc.data_ptr() + 4 * i, t.numel(), tile))
-            tile += -(-t.numel() // ABSMAX_TILE_ELEMS)
+            per_job.append(-(-t.numel() // ABSMAX_TILE_ELEMS))
+            tile += per_job[-1]
         self.total_tiles = tile
         self.jobs = _job_table(rows, dev)
+        self.tile_job = _tile_job_map(per_job, dev)
 
     def run(self, zero=True):
         if zero:
             self.acc.zero_()
-        call("mo_absmax_multi", self.acc, _ptr(self.jobs), len(self.tensors), self.total_tiles,
-             self.dtype, _stream(self.acc))
+        call("mo_absmax_multi", self.acc, _ptr(self.jobs), len(self.tensors), _ptr(self.tile_job),
+             self.total_tiles, self.dtype, _stream(self.acc))
         return self.acc
 
 
@@ -235,7 +243,7 @@ class Nvfp4QuantizePlan:
         self.tensors, self.amax, self.amax_is_wsf2 = list(tensors), amax, bool(amax_is_wsf2)
         self.wsf2 = torch.empty(len(tensors), dtype=torch.float32, device=dev)
         self.packed, self._wsf_u8 = [], []
-        rows, tile = [], 0
+        rows, tile, per_job = [], 0, []
         for i, t in enumerate(tensors):
             _require_device(t)
             if (t.dtype != torch.bfloat16 or not t.is_contiguous() or t.shape[-1] % 16
@@ -248,12 +256,15 @@ class Nvfp4QuantizePlan:
             self._wsf_u8.append(w)
             rows.append((t.data_ptr(), p.data_ptr(), w.data_ptr(), amax.data_ptr() + 4 * i,
                          self.wsf2.data_ptr() + 4 * i, t.numel(), tile, 0))
-            tile += -(-t.numel() // NVFP4_TILE_ELEMS)
+            per_job.append(-(-t.numel() // NVFP4_TILE_ELEMS))
+            tile += per_job[-1]
         self.total_tiles = tile
         self.jobs = _job_table(rows, dev)
+        self.tile_job = _tile_job_map(per_job, dev)
         self.wsf = [w.view(torch.float8_e4m3fn) for w in self._wsf_u8]
 
     def run(self):
         call("mo_nvfp4_quantize_multi", self.amax, _ptr(self.jobs), len(self.tensors),
-             self.total_tiles, MO_BF16, 16, int(self.amax_is_wsf2), _stream(self.amax))
+             _ptr(self.tile_job), self.total_tiles, MO_BF16, 16, int(self.amax_is_wsf2),
+             _stream(self.amax))
         return self.packed, self.wsf, self.wsf2
