@@ -27,6 +27,11 @@ LAYER_SHAPES = [("q_proj", 4096, 4096), ("k_proj", 1024, 4096), ("v_proj", 1024,
 QUANT_BYTES_PER_ELEM = 2.0 + 0.5 + 1.0 / 16.0   # bf16 read + codes + block scale
 AMAX_BYTES_PER_ELEM = 2.0
 DEQUANT_BYTES_PER_ELEM = 0.5 + 1.0 / 16.0 + 2.0
+# HBM bytes per launch of nvfp4_quantize_multi_kernel on the default 32-layer workload, from
+# rocprofv3 --pmc FETCH_SIZE (6,829,310 KiB x 2.000) and WRITE_SIZE (3,833,868 KiB x 1.000); the
+# scale factors come from a 1 GiB device copy in the same runs
+# (profiles/nvfp4_quantize_multi_kernel__llama3_8b_weights.txt).
+MEASURED_TRAFFIC_BYTES_32_LAYERS = 17.912e9
 
 
 def make_weights(torch, layers, device):
@@ -90,6 +95,9 @@ def main():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip amax / dequant side measurements")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 1 GiB device copy (a kernel of known traffic for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU only: this build has no multi-GPU path (got --gpus {a.gpus}); "
@@ -147,9 +155,18 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "launch_ms": round(dev_ms, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES_32_LAYERS if a.layers == 32 else None,
         },
     }
+
+    if a.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        big = torch.empty(1 << 30, dtype=torch.uint8, device=dev).zero_()  # push src out of the caches
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst, big
 
     if not a.no_extras:
         extras = {}
