@@ -81,8 +81,9 @@ int mo_absmax_multi(const mo_absmax_job* jobs_dev, int njobs, const int32_t* til
 
 /* FP8 E4M3 quantize-dequantize.  Replaces fake_e4m3fy / fake_e4m3fy_with_axis
  * (TQ/src/tensor_quant_gpu_fp8.cu:66-108) with the numerics of the CPU path _fp8_eager
- * (TQ/tensor_quant.py:45-59): scale = 448 / f32(amax), inv = 1 / scale,
- * y = T(f32(e4m3_rne(f32(x) * scale)) * inv); amax == NULL is a plain cast.
+ * (TQ/tensor_quant.py:45-59): scale = RN(RN(1 / f32(amax)) * 448) (what torch computes for
+ * `448.0 / amax`), inv = RN(1 / scale), y = T(f32(e4m3_rne(f32(x) * scale)) * inv);
+ * amax == NULL is a plain cast.
  * saturate = 0: magnitudes that round above 448 become NaN (CPU torch cast);
  * saturate = 1: they clamp to 448 (the reference's CUDA kernel). */
 int mo_fp8_qdq(const void* x, void* y, int64_t outer, int64_t axis, int64_t inner, int dtype,

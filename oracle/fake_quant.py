@@ -12,8 +12,9 @@ E4M3_MAX = 448.0
 def fp8_eager(x: torch.Tensor, amax: torch.Tensor | None = None):
     """FP8 E4M3 QDQ.  Follows TQ/tensor_quant.py:45-59.
 
-    ``scale = 448 / f32(amax)`` and ``inv = 1 / scale`` are two separate fp32 divisions (not
-    ``amax / 448``).  The cast is torch's ``float8_e4m3fn`` (RNE, subnormals kept, magnitudes
+    ``scale = 448.0 / f32(amax)`` is ``float / tensor``, which torch evaluates as
+    ``reciprocal(amax) * 448.0`` (two roundings, not a true division); ``inv = 1 / scale`` is
+    ``reciprocal(scale)``.  The cast is torch's ``float8_e4m3fn`` (RNE, subnormals kept, magnitudes
     that round above 448 become NaN on CPU).  ``amax`` may be any shape broadcastable to ``x``.
     """
     dt = x.dtype

@@ -16,7 +16,9 @@ struct Fp8Op {
     struct Scale { float mul, inv; };
     __device__ __forceinline__ Scale make(float amax) const {
         Scale s;
-        s.mul = 448.0f / amax;
+        // the reference writes `448.0 / amax`, which torch evaluates as reciprocal(amax) * 448
+        // (two roundings), and `1 / scale`, which is reciprocal(scale)
+        s.mul = (1.0f / amax) * 448.0f;
         s.inv = 1.0f / s.mul;
         return s;
     }

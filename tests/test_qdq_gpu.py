@@ -1,0 +1,150 @@
+"""GPU parity of the FP8 / integer quantize-dequantize kernels against the CPU oracle."""
+
+import json
+import os
+
+import pytest
+import torch
+
+from conftest import GOLDEN, assert_bits_equal
+from modelopt_amd import _hip
+from oracle import fake_quant, reduce
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+with open(os.path.join(GOLDEN, "reference_vectors.json")) as f:
+    VEC = json.load(f)
+
+
+def _rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def _c1_tensor(n=1024):
+    """BASELINE config 1 shape in small: N(0, 0.02) with 0.1 % of entries scaled x50."""
+    g = torch.Generator().manual_seed(1)
+    x = 0.02 * torch.randn(n, n, generator=g)
+    idx = torch.randperm(x.numel(), generator=g)[: x.numel() // 1000]
+    x.view(-1)[idx] *= 50
+    return x.to(torch.bfloat16)
+
+
+# ----------------------------------------------------------------------------- FP8
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(64, 256), (33, 47), (5,), (4, 3, 130)])
+def test_fp8_per_tensor(dtype, shape):
+    x = _rand(shape, dtype, 11)
+    amax = reduce.reduce_amax(x)
+    y = _hip.fp8_qdq(x.to(DEV), amax.to(DEV), 1, 1, x.numel())
+    assert_bits_equal(y.cpu(), fake_quant.fp8_eager(x, amax), str(shape))
+
+
+def test_fp8_config1_pipeline():
+    x = _c1_tensor()
+    xd = x.to(DEV)
+    acc = torch.zeros(1, dtype=torch.float32, device=DEV)
+    _hip.absmax_into(xd, acc, 1, 1, xd.numel())
+    amax = acc.reshape(()).to(torch.bfloat16)
+    assert_bits_equal(amax.cpu(), reduce.reduce_amax(x), "amax")
+    y = _hip.fp8_qdq(xd, amax, 1, 1, xd.numel())
+    assert_bits_equal(y.cpu(), fake_quant.fp8_eager(x, reduce.reduce_amax(x)), "qdq")
+
+
+def test_fp8_clipping_gives_nan_like_cpu_and_saturates_on_request():
+    x = _rand((32, 64), torch.bfloat16, 12)
+    amax = reduce.reduce_amax(x) * 0.25  # amax smaller than the data
+    want = fake_quant.fp8_eager(x, amax)
+    assert torch.isnan(want).any()
+    y = _hip.fp8_qdq(x.to(DEV), amax.to(DEV), 1, 1, x.numel())
+    assert_bits_equal(y.cpu(), want, "NaN on overflow")
+    ys = _hip.fp8_qdq(x.to(DEV), amax.to(DEV), 1, 1, x.numel(), saturate=True).cpu()
+    assert not torch.isnan(ys).any()
+    keep = ~torch.isnan(want)
+    assert torch.equal(ys[keep], want[keep])
+    assert (ys[~keep].abs().float() == ys.abs().float().max()).all()
+
+
+def test_fp8_no_amax_is_plain_cast():
+    x = _rand((40, 50), torch.float32, 13, scale=30)
+    y = _hip.fp8_qdq(x.to(DEV), None, 1, 1, x.numel())
+    assert_bits_equal(y.cpu(), fake_quant.fp8_eager(x, None), "cast")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("axis", [0, 1, 2])
+def test_fp8_per_channel(dtype, axis):
+    x = _rand((6, 16, 24), dtype, 14)
+    dims = [d for d in range(3) if d != axis]
+    amax = reduce.reduce_amax(x, axis=dims, keepdims=True)
+    outer = int(torch.tensor(x.shape[:axis]).prod()) if axis else 1
+    inner = int(torch.tensor(x.shape[axis + 1:]).prod()) if axis < 2 else 1
+    y = _hip.fp8_qdq(x.to(DEV), amax.reshape(-1).contiguous().to(DEV), outer, x.shape[axis], inner)
+    assert_bits_equal(y.cpu(), fake_quant.fp8_eager(x, amax), f"axis {axis}")
+
+
+def test_fp8_all_bf16_patterns():
+    allv = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    for amax in (torch.tensor(1.0), torch.tensor(0.37), torch.tensor(3.0e4)):
+        amax = amax.to(torch.bfloat16)
+        y = _hip.fp8_qdq(allv.to(DEV), amax.to(DEV), 1, 1, allv.numel())
+        assert_bits_equal(y.cpu(), fake_quant.fp8_eager(allv, amax), f"amax {amax.item()}")
+
+
+# ----------------------------------------------------------------------------- integer
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("num_bits", VEC["int_qdq_grid"]["num_bits"])
+@pytest.mark.parametrize("unsigned", VEC["int_qdq_grid"]["unsigned"])
+def test_int_per_tensor_and_per_channel(dtype, num_bits, unsigned):
+    x = _rand((37, 48), dtype, num_bits)
+    if unsigned:
+        x = x.abs()
+    for narrow in (True, False):
+        amax = reduce.reduce_amax(x)
+        y = _hip.int_qdq(x.to(DEV), amax.to(DEV), 1, 1, x.numel(), num_bits, unsigned, narrow)
+        assert_bits_equal(y.cpu(), fake_quant.tensor_quant(x, amax, num_bits, unsigned, narrow),
+                          f"tensor narrow={narrow}")
+        a0 = reduce.reduce_amax(x, axis=[1], keepdims=True) * 0.8  # with clipping
+        y = _hip.int_qdq(x.to(DEV), a0.reshape(-1).contiguous().to(DEV), 1, 37, 48, num_bits,
+                         unsigned, narrow)
+        assert_bits_equal(y.cpu(), fake_quant.tensor_quant(x, a0, num_bits, unsigned, narrow),
+                          f"axis0 narrow={narrow}")
+        a1 = reduce.reduce_amax(x, axis=[0], keepdims=True)
+        y = _hip.int_qdq(x.to(DEV), a1.reshape(-1).contiguous().to(DEV), 37, 48, 1, num_bits,
+                         unsigned, narrow)
+        assert_bits_equal(y.cpu(), fake_quant.tensor_quant(x, a1, num_bits, unsigned, narrow),
+                          f"axis1 narrow={narrow}")
+
+
+def test_int_tiny_amax_channel_is_zero():
+    c = VEC["int_tiny_amax"]
+    g = torch.Generator().manual_seed(0)
+    x = torch.rand(*c["shape"], generator=g)
+    amax = torch.tensor(c["amax"])
+    y = _hip.int_qdq(x.to(DEV), amax.to(DEV), 2, 3, 4, 8, False, True).cpu()
+    assert y[:, 1, :].abs().sum() == 0
+    assert_bits_equal(y, fake_quant.tensor_quant(x, amax.reshape(1, 3, 1), 8, False, True), "tiny")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("k", [256, 200])
+def test_int4_static_block128_like_awq_weight(dtype, k):
+    x = _rand((24, k), dtype, 21, scale=0.02)
+    want = fake_quant.static_block_fake_quant(
+        x, 128, lambda x2, amax: fake_quant.tensor_quant(x2, amax, 4, False, False))
+    pad = (-k) % 128
+    xp = torch.nn.functional.pad(x, (0, pad)).to(DEV).contiguous()
+    rows = xp.numel() // 128
+    acc = torch.zeros(rows, dtype=torch.float32, device=DEV)
+    _hip.absmax_into(xp, acc, 1, rows, 128)
+    y = _hip.int_qdq(xp, acc.to(dtype), 1, rows, 128, 4, False, False).reshape(24, k + pad)[:, :k]
+    assert_bits_equal(y.cpu().contiguous(), want.contiguous(), "int4 block 128")
+
+
+def test_inplace_alias():
+    x = _rand((128, 64), torch.bfloat16, 30)
+    amax = reduce.reduce_amax(x)
+    xd = x.to(DEV)
+    _hip.int_qdq(xd, amax.to(DEV), 1, 1, xd.numel(), 8, False, True, out=xd)
+    assert_bits_equal(xd.cpu(), fake_quant.tensor_quant(x, amax, 8, False, True), "in place")
