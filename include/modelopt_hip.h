@@ -155,6 +155,74 @@ int mo_nvfp4_dequantize(const uint8_t* packed, const uint8_t* wsf, const float* 
                         int64_t rows, int64_t kp, int block_size, void* y, int dtype,
                         void* stream);
 
+/* ------------------------------------------------------------------ FP8 / INT8 storage casts
+ * x viewed as [outer, axis, inner], one scale per index of `axis` (axis = 1: per tensor).
+ * q = fmt( via( f32(x) / f32(scale) ) ): `via_dtype` is the dtype torch's type promotion gives
+ * the quotient (bf16 tensor / bf16 or 0-dim fp32 scale -> bf16: the quotient is rounded to bf16
+ * before the final cast; a dim >= 1 fp32 scale -> fp32).  format MO_FMT_E4M3: RNE cast, values
+ * that round above 448 become NaN (torch CPU); MO_FMT_INT8: rne, clamp [-128, 127].
+ * Replaces FP8QTensor.quantize / INT8QTensor.quantize (TQ/qtensor/fp8_tensor.py:41-113,
+ * TQ/qtensor/int8_tensor.py:36-95) and the FP8 / INT8 branches of to_quantized_weight
+ * (modelopt/torch/export/quant_utils.py:759-774). */
+enum mo_format { MO_FMT_E4M3 = 0, MO_FMT_INT8 = 1 };
+int mo_real_quantize(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
+                     const void* scale, int scale_dtype, int via_dtype, int format,
+                     uint8_t* out, void* stream);
+
+/* y = T( f32(T(q)) * f32(T(scale)) ).  Replaces FP8QTensor.dequantize / INT8QTensor.dequantize
+ * (TQ/qtensor/fp8_tensor.py:115-151, TQ/qtensor/int8_tensor.py:97-130). */
+int mo_real_dequantize(const uint8_t* q, int64_t outer, int64_t axis, int64_t inner, int format,
+                       const void* scale, int scale_dtype, void* y, int dtype, void* stream);
+
+/* ------------------------------------------------------------------ INT4 weight compression
+ * Flat blocks of block_size elements over the n elements of x (tail zero padded).
+ * scales[b] = T(f32(T(1 / amax_b)) * 7) (what torch computes for `7 / amax` in dtype T),
+ * q = clamp(rne(T(x * scale)), -8, 7) + 8, packed[i] = q[2i] << 4 | q[2i + 1].
+ * scales has ceil(n / block_size) elements of dtype T; packed has ceil(n / block_size) *
+ * block_size / 2 bytes.  Replaces INT4_quantize (TQ/src/tensor_quant_gpu.cu:311) with the CPU
+ * numerics of INT4QTensor.quantize (TQ/qtensor/int4_tensor.py:40-88). */
+int mo_int4_block_quantize(const void* x, int64_t n, int64_t block_size, int dtype, void* scales,
+                           uint8_t* packed, void* stream);
+
+/* y[2i] = T((packed[i] >> 4) - 8) / scale), y[2i + 1] = T(((packed[i] & 15) - 8) / scale).
+ * Replaces INT4_dequantize (TQ/src/tensor_quant_gpu.cu:262) / INT4QTensor.dequantize
+ * (TQ/qtensor/int4_tensor.py:90-130). */
+int mo_int4_block_dequantize(const uint8_t* packed, int64_t nbytes, int64_t block_size,
+                             const void* scales, void* y, int dtype, void* stream);
+
+/* INT4-AWQ export pack of w[batch, n_rows, k] with fp32 scales ws[batch, n_rows, k/block_size]:
+ * q = int8(clamp(rne(f32(w) / ws), -8, 7)); out[b, j, c] = (q[b, 2j, c] & 0xF) |
+ * (q[b, 2j+1, c] << 4), out is uint8 [batch, n_rows / 2, k].  Replaces pack_int4_in_uint8
+ * (modelopt/torch/export/quant_utils.py:697-738). */
+int mo_int4_pack_rows(const void* w, int64_t batch, int64_t n_rows, int64_t k, int64_t block_size,
+                      int dtype, const float* ws, uint8_t* out, void* stream);
+
+/* ------------------------------------------------------------------ AWQ-lite / SmoothQuant
+ * y[r, c] = T(f32(x[r, c]) * f32(s[c])): the pre_quant_scale multiply of
+ * TensorQuantizer.forward (TQ/nn/modules/tensor_quantizer.py:881-882) and the weight folding of
+ * _apply_weight_pre_quant_scale (TQ/model_calib.py:346-353).  y may alias x. */
+int mo_mul_cols(const void* x, int64_t rows, int64_t k, int dtype, const void* s, int s_dtype,
+                void* y, void* stream);
+
+/* Fused weight path of one AWQ-lite search step (TQ/model_calib.py:671-685 through
+ * TensorQuantizer.forward and _tensor_quant): xs = T(x * s[c]) (s may be NULL), per-block amax
+ * over `block_size` (8..512, power of two) columns, INT-N quantize-dequantize with that amax.
+ * y may alias x. */
+int mo_scale_block_int_qdq(const void* x, int64_t rows, int64_t k, int dtype, const void* s,
+                           int s_dtype, int64_t block_size, int num_bits, int is_unsigned,
+                           int narrow_range, void* y, void* stream);
+
+/* acc[c] += sum over rows of |x[r, c]| (blk_amax == NULL: get_act_scale numerator,
+ * TQ/model_calib.py:605-606) or of T(|x[r, c]| / T(blk_amax[r, c / block_size] + tiny))
+ * (get_weight_scale numerator, TQ/model_calib.py:588-603).  fp32 accumulation; the caller
+ * divides by the row count and rounds through T as the reference's `.mean(0)` does. */
+int mo_abs_colsum(const void* x, int64_t rows, int64_t k, int dtype, const float* blk_amax,
+                  int64_t block_size, float* acc, void* stream);
+
+/* acc[0] += sum of f32(T(a[i] - b[i]))^2 in double: the numerator of update_loss
+ * (TQ/model_calib.py:623-627). */
+int mo_sq_diff_sum(const void* a, const void* b, int64_t n, int dtype, double* acc, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

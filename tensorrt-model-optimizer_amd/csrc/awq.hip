@@ -1,0 +1,219 @@
+// Kernels behind AWQ-lite and SmoothQuant for gfx950: per-channel scaling, the fused
+// scale -> block amax -> INT-N quantize-dequantize of a weight, column statistics and the
+// squared-error loss.  All HBM-bound except the search GEMM, which is not in this file.
+#include "common.h"
+
+namespace mo {
+
+// y[r, c] = T( f32(x[r, c]) * f32(s[c]) )   (bf16 * bf16 -> bf16 and bf16 * fp32 -> fp32 -> bf16
+// both reduce to one fp32 product rounded once to T)
+template <int DT>
+__global__ __launch_bounds__(256) void mul_cols_kernel(const void* __restrict__ x, int64_t rows,
+                                                       int64_t k, const void* __restrict__ s,
+                                                       int s_dtype, void* __restrict__ y) {
+    const int64_t kc = (k + 7) >> 3, total = rows * kc;
+    const bool vec = (k % 8 == 0) && ((((uintptr_t)x | (uintptr_t)y) & 15u) == 0);
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
+        const int64_t r = t / kc, c0 = (t - r * kc) << 3;
+        float v[8];
+        if (vec) load_chunk<DT>(x, r * k + c0, v);
+        else load_chunk_guarded<DT>(x, r * k, c0, k, v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (c0 + j < k) v[j] *= load_scalar(s, s_dtype, c0 + j);
+        if (vec) store_chunk<DT>(y, r * k + c0, v);
+        else store_chunk_guarded<DT>(y, r * k, c0, k, v);
+    }
+}
+
+// Static block INT-N fake quantisation along the last axis with an optional per-column
+// pre-scale, fused:  xs = T(x * s[c]);  amax = max |xs| over each block of `bs` columns (zero
+// padded);  scale = bound / f32(amax) (amax <= 2^-24 -> output 0);
+// y = T( clamp(rne(f32(xs) * scale), lo, bound) / scale ).
+// A lane owns a chunk of 8 columns; the G = bs / 8 lanes of a block share the amax by shuffles.
+template <int DT>
+__global__ __launch_bounds__(256) void scale_block_int_qdq_kernel(
+    const void* __restrict__ x, int64_t rows, int64_t k, const void* __restrict__ s, int s_dtype,
+    int lg_g, float bound, float lo, void* __restrict__ y) {
+    const int G = 1 << lg_g;
+    const int64_t bs = (int64_t)G << 3;
+    const int64_t kp = (k + bs - 1) / bs * bs, kc = kp >> 3, total = rows * kc;
+    const bool vec = (k % 8 == 0) && ((((uintptr_t)x | (uintptr_t)y) & 15u) == 0);
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    // total is a multiple of G and the grid of 64, so a block's lanes enter the loop together
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
+        const int64_t r = t / kc, c0 = (t - r * kc) << 3;
+        float v[8];
+        if (vec && c0 + 8 <= k) load_chunk<DT>(x, r * k + c0, v);
+        else load_chunk_guarded<DT>(x, r * k, c0, k, v);
+        uint32_t m = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (s && c0 + j < k) {
+                const float p = v[j] * load_scalar(s, s_dtype, c0 + j);
+                if constexpr (DT == MO_BF16) v[j] = bf16_bits_to_f32(f32_to_bf16_bits(p));
+                else if constexpr (DT == MO_F16) v[j] = f16_bits_to_f32(f32_to_f16_bits(p));
+                else v[j] = p;
+            }
+            const uint32_t a = f2u(v[j]) & 0x7FFFFFFFu;
+            m = a > m ? a : m;
+        }
+        for (int o = G >> 1; o > 0; o >>= 1) {
+            const uint32_t u = (uint32_t)__shfl_xor((int)m, o, kWave);
+            m = u > m ? u : m;
+        }
+        const float amax = u2f(m);
+        const bool dead = amax <= 5.9604644775390625e-8f;
+        const float sc = bound / amax;
+        const float mul = dead ? 0.0f : sc, div = dead ? 1.0f : sc;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float q = __builtin_rintf(v[j] * mul);
+            q = q < lo ? lo : q;
+            q = q > bound ? bound : q;
+            v[j] = q / div;
+        }
+        if (vec && c0 + 8 <= k) store_chunk<DT>(y, r * k + c0, v);
+        else store_chunk_guarded<DT>(y, r * k, c0, k, v);
+    }
+}
+
+// acc[c] += sum over rows of f32( T( |x[r, c]| / T(f32(blk_amax[r, c / bs]) + tiny) ) ) when
+// blk_amax is given, else of |x[r, c]|.  One thread per column over a slab of rows.
+template <int DT>
+__global__ __launch_bounds__(256) void abs_colsum_kernel(const void* __restrict__ x, int64_t rows,
+                                                         int64_t k, const float* __restrict__ blk_amax,
+                                                         int64_t bs, int64_t slab,
+                                                         float* __restrict__ acc) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= k) return;
+    const int64_t r0 = (int64_t)blockIdx.y * slab;
+    int64_t r1 = r0 + slab;
+    if (r1 > rows) r1 = rows;
+    const int64_t nb = blk_amax ? (k + bs - 1) / bs : 0;
+    // smallest positive normal of T, as torch.finfo(T).tiny
+    const float tiny = DT == MO_F16 ? 6.103515625e-05f : 1.17549435e-38f;
+    float sum = 0.0f;
+    for (int64_t r = r0; r < r1; ++r) {
+        float v = __builtin_fabsf(load_elem<DT>(x, r * k + c));
+        if (blk_amax) {
+            float d = blk_amax[r * nb + c / bs] + tiny;
+            if constexpr (DT == MO_BF16) d = bf16_bits_to_f32(f32_to_bf16_bits(d));
+            else if constexpr (DT == MO_F16) d = f16_bits_to_f32(f32_to_f16_bits(d));
+            v = v / d;
+            if constexpr (DT == MO_BF16) v = bf16_bits_to_f32(f32_to_bf16_bits(v));
+            else if constexpr (DT == MO_F16) v = f16_bits_to_f32(f32_to_f16_bits(v));
+        }
+        sum += v;
+    }
+    atomicAdd(acc + c, sum);
+}
+
+// acc[0] += sum of f32( T(a[i] - b[i]) )^2, accumulated in double across the grid.
+template <int DT>
+__global__ __launch_bounds__(256) void sq_diff_sum_kernel(const void* __restrict__ a,
+                                                          const void* __restrict__ b, int64_t n,
+                                                          double* __restrict__ acc) {
+    __shared__ double smem[4];
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    float part = 0.0f;
+    double sum = 0.0;
+    int cnt = 0;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        float d = load_elem<DT>(a, i) - load_elem<DT>(b, i);
+        if constexpr (DT == MO_BF16) d = bf16_bits_to_f32(f32_to_bf16_bits(d));
+        else if constexpr (DT == MO_F16) d = f16_bits_to_f32(f32_to_f16_bits(d));
+        part += d * d;
+        if (++cnt == 64) { sum += part; part = 0.0f; cnt = 0; }
+    }
+    sum += part;
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) smem[wave] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicAdd(acc, smem[0] + smem[1] + smem[2] + smem[3]);
+}
+
+static inline unsigned blocks_for_awq(int64_t items, int64_t cap = 16384) {
+    int64_t b = (items + 255) / 256;
+    if (b < 1) b = 1;
+    if (b > cap) b = cap;
+    return (unsigned)b;
+}
+
+}  // namespace mo
+
+#define DISPATCH_DT(dtype, CALL)          \
+    switch (dtype) {                      \
+        case MO_F32: CALL(MO_F32); break; \
+        case MO_F16: CALL(MO_F16); break; \
+        case MO_BF16: CALL(MO_BF16); break; \
+        default: return MO_ERR_DTYPE;     \
+    }
+
+extern "C" int mo_mul_cols(const void* x, int64_t rows, int64_t k, int dtype, const void* s,
+                           int s_dtype, void* y, void* stream) {
+    if (rows < 0 || k < 0) return MO_ERR_ARG;
+    if (s_dtype < MO_F32 || s_dtype > MO_BF16) return MO_ERR_DTYPE;
+    if (rows == 0 || k == 0) return MO_OK;
+    if (!x || !s || !y) return MO_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned g = mo::blocks_for_awq(rows * ((k + 7) >> 3));
+#define CALL(DT) mo::mul_cols_kernel<DT><<<g, 256, 0, st>>>(x, rows, k, s, s_dtype, y)
+    DISPATCH_DT(dtype, CALL)
+#undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_scale_block_int_qdq(const void* x, int64_t rows, int64_t k, int dtype,
+                                      const void* s, int s_dtype, int64_t block_size, int num_bits,
+                                      int is_unsigned, int narrow_range, void* y, void* stream) {
+    if (rows < 0 || k < 0 || num_bits < 1 || num_bits > 24) return MO_ERR_ARG;
+    if (s_dtype < MO_F32 || s_dtype > MO_BF16) return MO_ERR_DTYPE;
+    int lg = 0;
+    while ((8 << lg) < block_size && lg < 6) ++lg;
+    if ((8 << lg) != block_size) return MO_ERR_UNSUPPORTED;  // 8, 16, ..., 512
+    if (rows == 0 || k == 0) return MO_OK;
+    if (!x || !y) return MO_ERR_ARG;
+    const float bound = (float)((1 << (num_bits - 1 + (is_unsigned ? 1 : 0))) - 1);
+    const float lo = is_unsigned ? 0.0f : (narrow_range ? -bound : -bound - 1.0f);
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t kp = (k + block_size - 1) / block_size * block_size;
+    const unsigned g = mo::blocks_for_awq(rows * (kp >> 3));
+#define CALL(DT) mo::scale_block_int_qdq_kernel<DT><<<g, 256, 0, st>>>(x, rows, k, s, s_dtype, lg, bound, lo, y)
+    DISPATCH_DT(dtype, CALL)
+#undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_abs_colsum(const void* x, int64_t rows, int64_t k, int dtype,
+                             const float* blk_amax, int64_t block_size, float* acc, void* stream) {
+    if (rows < 0 || k < 0 || (blk_amax && block_size <= 0)) return MO_ERR_ARG;
+    if (rows == 0 || k == 0) return MO_OK;
+    if (!x || !acc) return MO_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t gx = (k + 255) / 256;
+    int64_t gy = (1024 + gx - 1) / gx;
+    int64_t slab = (rows + gy - 1) / gy;
+    if (slab < 8) slab = 8;
+    gy = (rows + slab - 1) / slab;
+    dim3 grid((unsigned)gx, (unsigned)gy);
+#define CALL(DT) mo::abs_colsum_kernel<DT><<<grid, 256, 0, st>>>(x, rows, k, blk_amax, block_size, slab, acc)
+    DISPATCH_DT(dtype, CALL)
+#undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_sq_diff_sum(const void* a, const void* b, int64_t n, int dtype, double* acc,
+                              void* stream) {
+    if (n < 0) return MO_ERR_ARG;
+    if (n == 0) return MO_OK;
+    if (!a || !b || !acc) return MO_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned g = mo::blocks_for_awq(n, 2048);
+#define CALL(DT) mo::sq_diff_sum_kernel<DT><<<g, 256, 0, st>>>(a, b, n, acc)
+    DISPATCH_DT(dtype, CALL)
+#undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}

@@ -31,6 +31,15 @@ SIGNATURES = {
     "mo_nvfp4_qdq": [_P, _P, _I64, _I64, _INT, _P, _INT, _INT, _INT, _P],
     "mo_nvfp4_quantize": [_P, _I64, _I64, _INT, _INT, _P, _INT, _P, _P, _P, _P, _P],
     "mo_nvfp4_dequantize": [_P, _P, _P, _I64, _I64, _INT, _P, _INT, _P],
+    "mo_real_quantize": [_P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _P, _P],
+    "mo_real_dequantize": [_P, _I64, _I64, _I64, _INT, _P, _INT, _P, _INT, _P],
+    "mo_int4_block_quantize": [_P, _I64, _I64, _INT, _P, _P, _P],
+    "mo_int4_block_dequantize": [_P, _I64, _I64, _P, _P, _INT, _P],
+    "mo_int4_pack_rows": [_P, _I64, _I64, _I64, _I64, _INT, _P, _P, _P],
+    "mo_mul_cols": [_P, _I64, _I64, _INT, _P, _INT, _P, _P],
+    "mo_scale_block_int_qdq": [_P, _I64, _I64, _INT, _P, _INT, _I64, _INT, _INT, _INT, _P, _P],
+    "mo_abs_colsum": [_P, _I64, _I64, _INT, _P, _I64, _P, _P],
+    "mo_sq_diff_sum": [_P, _P, _I64, _INT, _P, _P],
 }
 
 _lib = None
@@ -166,6 +175,102 @@ def nvfp4_dequantize(packed, wsf, wsf2, block_size, dtype):
     call("mo_nvfp4_dequantize", packed, _ptr(packed), _ptr(wsf.view(torch.uint8)), _ptr(wsf2),
          rows, kp, block_size, _ptr(y), dtype_code(dtype), _stream(packed))
     return y
+
+
+MO_FMT_E4M3, MO_FMT_INT8 = 0, 1
+
+
+def real_quantize(x, scale, outer, axis, inner, via_dtype, fmt):
+    """q = fmt(via(x / scale)); returns float8_e4m3fn or int8 tensor of x's shape."""
+    _require_device(x, scale)
+    assert x.is_contiguous() and scale.is_contiguous() and scale.numel() == axis
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    call("mo_real_quantize", x, _ptr(x), outer, axis, inner, dtype_code(x.dtype), _ptr(scale),
+         dtype_code(scale.dtype), dtype_code(via_dtype), fmt, _ptr(out), _stream(x))
+    return out.view(torch.float8_e4m3fn if fmt == MO_FMT_E4M3 else torch.int8)
+
+
+def real_dequantize(q, scale, outer, axis, inner, fmt, dtype):
+    _require_device(q, scale)
+    assert q.is_contiguous() and scale.is_contiguous() and scale.numel() == axis
+    y = torch.empty(q.shape, dtype=dtype, device=q.device)
+    call("mo_real_dequantize", q, _ptr(q.view(torch.uint8)), outer, axis, inner, fmt, _ptr(scale),
+         dtype_code(scale.dtype), _ptr(y), dtype_code(dtype), _stream(q))
+    return y
+
+
+def int4_block_quantize(x, block_size):
+    """Flat-block INT4 quantize + pack: returns (packed uint8 [padded_numel / 2], scales [nblocks, 1])."""
+    _require_device(x)
+    assert x.is_contiguous()
+    n = x.numel()
+    nblocks = -(-n // block_size)
+    scales = torch.empty((nblocks, 1), dtype=x.dtype, device=x.device)
+    packed = torch.empty(nblocks * block_size // 2, dtype=torch.uint8, device=x.device)
+    call("mo_int4_block_quantize", x, _ptr(x), n, block_size, dtype_code(x.dtype), _ptr(scales),
+         _ptr(packed), _stream(x))
+    return packed, scales
+
+
+def int4_block_dequantize(packed, scales, block_size):
+    _require_device(packed, scales)
+    assert packed.is_contiguous() and scales.is_contiguous()
+    y = torch.empty(packed.numel() * 2, dtype=scales.dtype, device=packed.device)
+    call("mo_int4_block_dequantize", packed, _ptr(packed), packed.numel(), block_size, _ptr(scales),
+         _ptr(y), dtype_code(scales.dtype), _stream(packed))
+    return y
+
+
+def int4_pack_rows(w, ws):
+    """INT4-AWQ export pack: w [..., N, K], ws fp32 [..., N, K / bs] -> uint8 [..., N / 2, K]."""
+    _require_device(w, ws)
+    assert w.is_contiguous() and ws.is_contiguous() and ws.dtype == torch.float32
+    n, k = w.shape[-2], w.shape[-1]
+    batch = w.numel() // (n * k) if n * k else 0
+    bs = k // ws.shape[-1]
+    out = torch.empty(tuple(w.shape[:-2]) + (n // 2, k), dtype=torch.uint8, device=w.device)
+    call("mo_int4_pack_rows", w, _ptr(w), batch, n, k, bs, dtype_code(w.dtype), _ptr(ws), _ptr(out),
+         _stream(w))
+    return out
+
+
+def mul_cols(x, s, out=None):
+    """y[..., c] = T(x[..., c] * s[c])."""
+    _require_device(x, s)
+    assert x.is_contiguous() and s.is_contiguous() and s.numel() == x.shape[-1]
+    k = x.shape[-1]
+    y = torch.empty_like(x) if out is None else out
+    call("mo_mul_cols", x, _ptr(x), x.numel() // k if k else 0, k, dtype_code(x.dtype), _ptr(s),
+         dtype_code(s.dtype), _ptr(y), _stream(x))
+    return y
+
+
+def scale_block_int_qdq(x, s, block_size, num_bits=4, unsigned=False, narrow_range=False, out=None):
+    _require_device(x, s)
+    assert x.is_contiguous() and (s is None or (s.is_contiguous() and s.numel() == x.shape[-1]))
+    k = x.shape[-1]
+    y = torch.empty_like(x) if out is None else out
+    call("mo_scale_block_int_qdq", x, _ptr(x), x.numel() // k if k else 0, k, dtype_code(x.dtype),
+         _ptr(s), dtype_code(s.dtype) if s is not None else MO_F32, block_size, num_bits,
+         int(bool(unsigned)), int(bool(narrow_range)), _ptr(y), _stream(x))
+    return y
+
+
+def abs_colsum_into(x, acc, blk_amax=None, block_size=0):
+    _require_device(x, acc, blk_amax)
+    k = x.shape[-1]
+    assert x.is_contiguous() and acc.dtype == torch.float32 and acc.numel() == k
+    call("mo_abs_colsum", x, _ptr(x), x.numel() // k if k else 0, k, dtype_code(x.dtype),
+         _ptr(blk_amax), block_size, _ptr(acc), _stream(x))
+    return acc
+
+
+def sq_diff_sum_into(a, b, acc):
+    _require_device(a, b, acc)
+    assert a.is_contiguous() and b.is_contiguous() and a.shape == b.shape and a.dtype == b.dtype
+    assert acc.dtype == torch.float64
+    call("mo_sq_diff_sum", a, _ptr(a), _ptr(b), a.numel(), dtype_code(a.dtype), _ptr(acc), _stream(a))
+    return acc
 
 
 # ----------------------------------------------------------------------------- options

@@ -1,0 +1,176 @@
+"""GPU parity of the storage-format kernels (FP8 / INT8 casts, INT4 packs) and the AWQ helpers."""
+
+import json
+import os
+
+import pytest
+import torch
+
+from conftest import GOLDEN, assert_bits_equal
+from modelopt_amd import _hip
+from oracle import awq, export, fake_quant, qtensor, reduce
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+with open(os.path.join(GOLDEN, "reference_vectors.json")) as f:
+    VEC = json.load(f)
+
+
+def _rand(shape, dtype, seed, scale=0.02):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+# ----------------------------------------------------------------------------- FP8
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_fp8_compress_path_per_tensor_and_channel(dtype):
+    x = _rand((48, 96), dtype, 1)
+    q_o, s_o = qtensor.fp8_quantize(x)  # scales = amax / 448 in the input dtype
+    q = _hip.real_quantize(x.to(DEV), s_o.reshape(1).to(DEV), 1, 1, x.numel(), dtype, _hip.MO_FMT_E4M3)
+    assert_bits_equal(q.cpu(), q_o, "per tensor")
+    y = _hip.real_dequantize(q, s_o.reshape(1).to(DEV), 1, 1, x.numel(), _hip.MO_FMT_E4M3, dtype)
+    assert_bits_equal(y.cpu(), qtensor.fp8_dequantize(q_o, s_o, x.shape, dtype), "dequant")
+    q_o, s_o = qtensor.fp8_quantize(x, axis=0)
+    q = _hip.real_quantize(x.to(DEV), s_o.reshape(-1).contiguous().to(DEV), 1, 48, 96, dtype,
+                           _hip.MO_FMT_E4M3)
+    assert_bits_equal(q.cpu(), q_o, "per channel")
+    y = _hip.real_dequantize(q, s_o.reshape(-1).contiguous().to(DEV), 1, 48, 96, _hip.MO_FMT_E4M3, dtype)
+    assert_bits_equal(y.cpu(), qtensor.fp8_dequantize(q_o, s_o, x.shape, dtype), "dequant channel")
+
+
+def test_fp8_export_cast_double_and_single_rounding():
+    w = _rand((512, 512), torch.bfloat16, 2)
+    wsf = reduce.reduce_amax(w).float() / 448.0
+    # 0-dim fp32 scale: quotient rounded to bf16 first
+    q = _hip.real_quantize(w.to(DEV), wsf.reshape(1).to(DEV), 1, 1, w.numel(), torch.bfloat16,
+                           _hip.MO_FMT_E4M3)
+    assert_bits_equal(q.cpu(), export.fp8_export_cast(w, wsf), "double rounding")
+    # 1-element fp32 scale: fp32 quotient, rounded once
+    q1 = _hip.real_quantize(w.to(DEV), wsf.reshape(1).to(DEV), 1, 1, w.numel(), torch.float32,
+                            _hip.MO_FMT_E4M3)
+    assert_bits_equal(q1.cpu(), export.fp8_export_cast(w, wsf.reshape(1)), "single rounding")
+    assert (q.view(torch.uint8) != q1.view(torch.uint8)).any()
+
+
+@pytest.mark.parametrize("case", [c for c in VEC["qtensor_roundtrip"]
+                                  if c["block_sizes"] is None or len(c["block_sizes"]) == 1],
+                         ids=lambda c: c["name"])
+def test_qtensor_golden_vectors_through_kernels(case):
+    """The reference's own golden round trips (tests/gpu/torch/quantization/test_qtensor_cuda.py
+    :133-241), computed by the HIP kernels."""
+    x = torch.tensor(case["input"], dtype=torch.bfloat16)
+    want = torch.tensor(case["output"], dtype=torch.bfloat16)
+    xd = x.to(DEV)
+    bits, bs, axis = case["num_bits"], case["block_sizes"], case["axis"]
+    if bits == 4:
+        b = bs["-1"]
+        packed, scales = _hip.int4_block_quantize(xd, b)
+        y = _hip.int4_block_dequantize(packed, scales, b)[: x.numel()].reshape(x.shape)
+    else:
+        fmt = _hip.MO_FMT_INT8 if bits == 8 else _hip.MO_FMT_E4M3
+        bound = 127.0 if bits == 8 else 448.0
+        if bs:  # 1-D blocks along the last dim: rows of length block
+            b = bs["-1"]
+            nblk = x.numel() // b
+            acc = torch.zeros(nblk, dtype=torch.float32, device=DEV)
+            _hip.absmax_into(xd, acc, 1, nblk, b)
+            outer, ax, inner = 1, nblk, b
+        elif axis is None:
+            acc = torch.zeros(1, dtype=torch.float32, device=DEV)
+            _hip.absmax_into(xd, acc, 1, 1, x.numel())
+            outer, ax, inner = 1, 1, x.numel()
+        else:
+            acc = torch.zeros(x.shape[0], dtype=torch.float32, device=DEV)
+            _hip.absmax_into(xd, acc, 1, x.shape[0], x.shape[1])
+            outer, ax, inner = 1, x.shape[0], x.shape[1]
+        scales = acc.to(torch.bfloat16) / bound
+        q = _hip.real_quantize(xd, scales, outer, ax, inner, torch.bfloat16, fmt)
+        y = _hip.real_dequantize(q, scales, outer, ax, inner, fmt, torch.bfloat16)
+    assert torch.allclose(y.cpu(), want), (y.cpu(), want)
+
+
+# ----------------------------------------------------------------------------- INT8 / INT4
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_int8_quantize_dequantize(dtype):
+    x = _rand((40, 64), dtype, 3, scale=1.0)
+    q_o, s_o = qtensor.int8_quantize(x, axis=0)
+    s = s_o.reshape(-1).contiguous().to(DEV)
+    q = _hip.real_quantize(x.to(DEV), s, 1, 40, 64, dtype, _hip.MO_FMT_INT8)
+    assert_bits_equal(q.cpu(), q_o, "int8 codes")
+    y = _hip.real_dequantize(q, s, 1, 40, 64, _hip.MO_FMT_INT8, dtype)
+    assert_bits_equal(y.cpu(), qtensor.int8_dequantize(q_o, s_o, x.shape, dtype), "int8 dequant")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape,bs", [((64, 256), 128), ((32, 64), 64), ((1, 10), 4), ((16, 48), 32)])
+def test_int4_block_quantize(dtype, shape, bs):
+    x = _rand(shape, dtype, 4, scale=1.0)
+    p_o, s_o = qtensor.int4_quantize(x, bs)
+    packed, scales = _hip.int4_block_quantize(x.to(DEV), bs)
+    assert_bits_equal(scales.cpu(), s_o, "scales")
+    assert torch.equal(packed.cpu(), p_o.reshape(-1))  # includes the zero-padded tail block
+    y = _hip.int4_block_dequantize(packed, scales, bs)[: x.numel()].reshape(shape)
+    y_o = qtensor.int4_dequantize(p_o, s_o, bs, shape, dtype)
+    assert_bits_equal(y.cpu(), y_o, "dequant")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(64, 256), (2, 8, 128), (130, 384)])
+def test_int4_awq_export_pack(dtype, shape):
+    w = _rand(shape, dtype, 5)
+    bs = 128
+    amax = reduce.reduce_block_amax(w, {-1: bs})
+    ws = amax.float() / 7.0
+    want = export.pack_int4_in_uint8(w, ws)
+    got = _hip.int4_pack_rows(w.to(DEV), ws.to(DEV))
+    assert_bits_equal(got.cpu(), want, "packed rows")
+
+
+# ----------------------------------------------------------------------------- AWQ helpers
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mul_cols_both_scale_dtypes(dtype):
+    x = _rand((33, 72), dtype, 6, scale=1.0)
+    s = (torch.rand(72) + 0.5)
+    y = _hip.mul_cols(x.to(DEV), s.to(dtype).to(DEV))
+    assert_bits_equal(y.cpu(), x * s.to(dtype), "T * T")
+    y = _hip.mul_cols(x.to(DEV), s.to(DEV))
+    assert_bits_equal(y.cpu(), (x * s[None, :]).to(dtype), "T * fp32 row")
+
+
+@pytest.mark.parametrize("k", [512, 200])
+def test_fused_scale_block_int4_qdq(k):
+    w = _rand((96, k), torch.bfloat16, 7)
+    s = (torch.rand(k) * 2 + 0.25).to(torch.bfloat16)
+    want = awq.int4_block_qdq(w * s, 128)
+    got = _hip.scale_block_int_qdq(w.to(DEV), s.to(DEV), 128, 4, False, False)
+    assert_bits_equal(got.cpu(), want.contiguous(), "fused scale + block qdq")
+    got = _hip.scale_block_int_qdq(w.to(DEV), None, 128, 4, False, False)
+    assert_bits_equal(got.cpu(), awq.int4_block_qdq(w, 128).contiguous(), "no scale")
+
+
+def test_awq_column_statistics_close_to_oracle():
+    x = _rand((512, 256), torch.bfloat16, 8, scale=1.0)
+    acc = torch.zeros(256, dtype=torch.float32, device=DEV)
+    _hip.abs_colsum_into(x.to(DEV), acc)
+    got = (acc / 512).to(torch.bfloat16).float().cpu()
+    want = awq.awq_act_scale(x)
+    assert torch.allclose(got, want, rtol=2 ** -7, atol=0)  # at most one bf16 ulp (summation order)
+    assert (got == want).float().mean() > 0.95
+    w = _rand((128, 256), torch.bfloat16, 9)
+    blk = torch.zeros(128 * 2, dtype=torch.float32, device=DEV)
+    _hip.absmax_into(w.to(DEV), blk, 1, 256, 128)
+    acc = torch.zeros(256, dtype=torch.float32, device=DEV)
+    _hip.abs_colsum_into(w.to(DEV), acc, blk, 128)
+    got = (acc / 128).to(torch.bfloat16).float().cpu()
+    want = awq.awq_weight_scale(w, 128)
+    assert torch.allclose(got, want, rtol=2 ** -7, atol=0)
+    assert (got == want).float().mean() > 0.95
+
+
+def test_sq_diff_loss():
+    a, b = _rand((256, 512), torch.bfloat16, 10, 1.0), _rand((256, 512), torch.bfloat16, 11, 1.0)
+    acc = torch.zeros(1, dtype=torch.float64, device=DEV)
+    _hip.sq_diff_sum_into(a.to(DEV), b.to(DEV), acc)
+    want = (a - b).float().pow(2).mean().item()
+    assert acc.item() / a.numel() == pytest.approx(want, rel=1e-5)
