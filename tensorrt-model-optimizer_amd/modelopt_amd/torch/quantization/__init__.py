@@ -1,0 +1,13 @@
+"""``modelopt_amd.torch.quantization`` -- import as ``mtq``.
+
+Same entry points as ``modelopt.torch.quantization``: ``quantize``, ``calibrate``, the named
+configs (``NVFP4_DEFAULT_CFG`` ...), ``TensorQuantizer`` under ``nn``.
+"""
+
+from . import calib, config, conversion, kernels, model_calib, nn, qtensor, tensor_quant, utils
+from .config import *  # noqa: F401,F403
+from .conversion import (register, replace_quant_module, set_quantizer_attribute,
+                         set_quantizer_by_cfg, set_quantizer_by_cfg_context, unregister)
+from .model_quant import (calibrate, disable_quantizer, enable_quantizer, fold_weight,
+                          postprocess_amax, print_quant_summary, quantize)
+from .plugins import attention as _attention_plugin  # noqa: F401  (registers KV quantizers)

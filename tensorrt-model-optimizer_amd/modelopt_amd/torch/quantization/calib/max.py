@@ -1,0 +1,113 @@
+"""Max calibrator with a device-resident running maximum.
+
+Same interface and result as the reference's ``MaxCalibrator`` (modelopt/torch/quantization/
+calib/max.py:26-94).  ``collect`` is one kernel launch that folds |x| into a persistent fp32
+accumulator with integer atomic max -- no temporaries and no host synchronisation.  The three
+sanity checks the reference runs (and blocks on) at every ``collect`` -- non-negative, no inf, no
+NaN -- are evaluated once, in ``compute_amax``; NaN and inf survive the running max, so nothing
+is lost by deferring them.
+"""
+
+import torch
+
+from .. import kernels
+from ..utils import convert_quantization_axis_to_reduce_axis
+
+__all__ = ["MaxCalibrator"]
+
+
+class _Calibrator:
+    def __init__(self, num_bits=8, axis=None, unsigned=False):
+        self._num_bits = num_bits
+        self._axis = axis
+        self._unsigned = unsigned
+
+    def collect(self, x):
+        raise NotImplementedError
+
+    def reset(self):
+        raise NotImplementedError
+
+    def compute_amax(self, *args, **kwargs):
+        raise NotImplementedError
+
+
+class MaxCalibrator(_Calibrator):
+    """Tracks the running abs-max of every tensor it is shown."""
+
+    def __init__(self, num_bits=8, axis=None, unsigned=False, track_amax=False):
+        super().__init__(num_bits, axis, unsigned)
+        self._track_amax = track_amax
+        if track_amax:
+            self._amaxs = []
+        self._acc = None             # fp32 running max, one element per kept channel
+        self._shape = None           # amax shape with the reduced dims kept as 1
+        self._dtype = None
+        self._calib_amax = None      # meta-device shortcut only
+        self._validated = False
+        self._seen_parameter = None  # identity of the last nn.Parameter folded in
+
+    @property
+    def amaxs(self):
+        return self._amaxs
+
+    @staticmethod
+    def _amax_shape(x, reduce_axis):
+        if reduce_axis is None:
+            return torch.Size(())
+        shape = torch.Size(1 if d in reduce_axis else x.shape[d] for d in range(x.dim()))
+        # the reference squeezes a one-element result to a scalar
+        return torch.Size(()) if shape.numel() == 1 else shape
+
+    @torch.no_grad()
+    def collect(self, x):
+        """Fold the abs-max of ``x`` (over everything but ``axis``) into the running maximum.
+
+        Raises ``RuntimeError`` when the amax shape differs from what was collected before.
+        """
+        reduce_axis = convert_quantization_axis_to_reduce_axis(x, self._axis)
+        shape = self._amax_shape(x, reduce_axis)
+        if x.device.type == "meta":
+            self._calib_amax = torch.empty(shape, dtype=x.dtype, device="meta")
+            return
+        keep = [] if reduce_axis is None else [d for d in range(x.dim()) if d not in reduce_axis]
+        layout = kernels.amax_layout(tuple(x.shape), keep)
+        if layout is None:
+            raise NotImplementedError("max calibration over non-adjacent kept dims is not covered")
+        if self._acc is None:
+            self._acc = torch.zeros(layout[1], dtype=torch.float32, device=x.device)
+            self._shape, self._dtype = shape, x.dtype
+        elif shape != self._shape:
+            raise RuntimeError("amax shape changed!")
+        if not self._track_amax:
+            kernels.absmax_accumulate(x, self._acc, layout)
+        else:
+            local = torch.zeros_like(self._acc)
+            kernels.absmax_accumulate(x, local, layout)
+            self._acc = torch.maximum(self._acc, local)
+            self._amaxs.append(local.reshape(shape).to(x.dtype).float().cpu().numpy())
+        self._validated = False
+
+    def reset(self):
+        self._seen_parameter = None
+        self._acc = None
+        self._shape = None
+        self._calib_amax = None
+        self._validated = False
+
+    def compute_amax(self):
+        """Running abs-max in the dtype of the collected tensors, or None if nothing was seen."""
+        if self._acc is None:
+            return self._calib_amax
+        amax = self._acc.to(self._dtype).reshape(self._shape)
+        if not self._validated:
+            bad = torch.stack([(self._acc < 0).any(), torch.isinf(self._acc).any(),
+                               torch.isnan(self._acc).any()]).tolist()  # one host sync
+            assert not bad[0], "detected negative values after abs, could be torch or cuda bug"
+            assert not bad[1], "detected inf values in amax"
+            assert not bad[2], "detected nan values in amax"
+            self._validated = True
+        return amax
+
+    def __str__(self):
+        return f"MaxCalibrator(track_amax={self._track_amax})"

@@ -1,0 +1,130 @@
+"""Model conversion: swap modules for their quantised versions and apply a ``quant_cfg``.
+
+Reference: modelopt/torch/quantization/conversion.py:56-67 (``convert_to_quantized_model``),
+:176 (``replace_quant_module``), :207 (``set_quantizer_by_cfg``), :241
+(``set_quantizer_attribute``).  The mode / state-manager machinery of the reference is not
+reproduced; conversion acts on the model in place.
+"""
+
+import fnmatch
+from contextlib import contextmanager
+from typing import Any
+
+from torch import nn
+
+from .config import QuantizeConfig, QuantizerAttributeConfig
+from .nn import QuantModuleRegistry, SequentialQuantizer, TensorQuantizer
+
+__all__ = ["replace_quant_module", "set_quantizer_by_cfg", "set_quantizer_attribute",
+           "set_quantizer_by_cfg_context", "register", "unregister"]
+
+
+def replace_quant_module(model: nn.Module):
+    """Recursively convert every registered module type found in ``model`` (in place)."""
+    assert not is_converted(model), "Model must not be quantized!"
+    for name, child in list(model.named_modules()):
+        if type(child) in QuantModuleRegistry:
+            QuantModuleRegistry.convert(child)
+    return model
+
+
+def is_converted(model: nn.Module) -> bool:
+    return any(isinstance(m, TensorQuantizer) for m in model.modules())
+
+
+def set_quantizer_by_cfg(quant_model: nn.Module, quant_cfg: dict | QuantizeConfig):
+    """Apply ``{wildcard or filter: attributes}`` to the quantizers of ``quant_model``.
+
+    ``"default"`` is applied first to every quantizer; then each pattern in insertion order, so
+    later entries win.  Keys that name a ``nn`` class (``"nn.BatchNorm1d"``) hold a nested
+    ``{pattern: attributes}`` dict applied only under modules of that class.
+    """
+    quant_cfg = dict(quant_cfg)
+    if "default" in quant_cfg:
+        set_quantizer_attribute(quant_model, "*", quant_cfg["default"])
+    for pattern, cfg in quant_cfg.items():
+        if pattern == "default":
+            continue
+        if isinstance(pattern, str) and pattern.startswith("nn.") and isinstance(cfg, dict) and all(
+                isinstance(v, (dict, list, QuantizerAttributeConfig)) for v in cfg.values()):
+            cls = getattr(nn, pattern[3:], None)
+            if cls is None:
+                continue
+            for sub_pattern, sub_cfg in cfg.items():
+                set_quantizer_attribute(quant_model, sub_pattern, sub_cfg, parent_class=cls)
+            continue
+        set_quantizer_attribute(quant_model, pattern, cfg)
+
+
+def _matches(name: str, wildcard_or_filter) -> bool:
+    if isinstance(wildcard_or_filter, str):
+        return fnmatch.fnmatch(name, wildcard_or_filter)
+    if callable(wildcard_or_filter):
+        return bool(wildcard_or_filter(name))
+    raise NotImplementedError(f"Unsupported type {type(wildcard_or_filter)}")
+
+
+def set_quantizer_attribute(quant_model: nn.Module, wildcard_or_filter_func, attribute,
+                            parent_class: type | None = None):
+    """Set attributes on every quantizer whose qualified name matches.  A list of attribute
+    dicts turns the matched ``TensorQuantizer`` into a ``SequentialQuantizer``."""
+    for name, module in list(quant_model.named_modules()):
+        if not isinstance(module, (TensorQuantizer, SequentialQuantizer)):
+            continue
+        if not _matches(name, wildcard_or_filter_func):
+            continue
+        parent_name, _, leaf = name.rpartition(".")
+        parent = quant_model.get_submodule(parent_name)
+        if isinstance(parent, SequentialQuantizer):
+            continue  # members are configured through their container
+        if parent_class is not None and not isinstance(parent, parent_class):
+            continue
+        if isinstance(attribute, (list, tuple)):
+            if not isinstance(module, SequentialQuantizer):
+                device = next((b.device for b in module.buffers()), None)
+                module = SequentialQuantizer(*(TensorQuantizer() for _ in attribute))
+                if device is not None:
+                    module.to(device)
+                setattr(parent, leaf, module)
+            elif len(attribute) != len(module):
+                raise ValueError("number of attributes does not match the SequentialQuantizer")
+            module.set_from_attribute_config([_as_cfg(a) for a in attribute])
+        else:
+            if isinstance(module, SequentialQuantizer):
+                module = TensorQuantizer()
+                setattr(parent, leaf, module)
+            module.set_from_attribute_config(_as_cfg(attribute))
+
+
+def _as_cfg(attribute):
+    """Validate a user dict through ``QuantizerAttributeConfig`` but keep only the keys given,
+    so a partial dict (``{"enable": False}``) leaves the other attributes alone."""
+    if isinstance(attribute, QuantizerAttributeConfig):
+        return attribute
+    full = QuantizerAttributeConfig(**attribute)
+    return {k: full[k] for k in attribute}
+
+
+@contextmanager
+def set_quantizer_by_cfg_context(quant_model: nn.Module, quant_cfg: dict[str, Any]):
+    """Temporarily apply ``quant_cfg``; the previous python-side attributes come back on exit."""
+    saved = {}
+    for name, module in quant_model.named_modules():
+        if isinstance(module, TensorQuantizer):
+            saved[module] = module.get_modelopt_state(properties_only=True)
+    set_quantizer_by_cfg(quant_model, quant_cfg)
+    try:
+        yield
+    finally:
+        for module, state in saved.items():
+            module.set_from_modelopt_state(state, properties_only=True)
+
+
+def register(original_cls: type, quantized_cls: type):
+    """Register a user module class for conversion (reference: conversion.py:340-380)."""
+    assert issubclass(original_cls, nn.Module) and issubclass(quantized_cls, nn.Module)
+    QuantModuleRegistry.register({original_cls: original_cls.__name__})(quantized_cls)
+
+
+def unregister(original_cls: type):
+    QuantModuleRegistry.unregister(original_cls)

@@ -1,0 +1,121 @@
+"""Shape logic between torch tensors and the HIP C ABI (``modelopt_amd._hip``).
+
+Everything here runs on the GPU through ``libmodelopt_hip.so``; CPU tensors are rejected.  The
+functions take and return torch tensors and never synchronise with the host.
+"""
+
+import math
+
+import torch
+
+from ... import _hip
+
+__all__ = [
+    "amax_layout", "absmax_accumulate", "reduce_amax_gpu", "fake_quant_int", "fake_quant_fp8",
+    "fake_quant_nvfp4", "mul_last_dim",
+]
+
+
+def _prod(xs):
+    return int(math.prod(xs))
+
+
+def amax_layout(shape, keep_dims):
+    """View a tensor of ``shape`` as [outer, axis, inner] such that the dims in ``keep_dims``
+    (a contiguous run of dims, or none) form ``axis``.  Returns (outer, axis, inner) or None
+    when the kept dims are not one contiguous run."""
+    nd = len(shape)
+    keep = sorted(d % nd for d in keep_dims if shape[d % nd] != 1)
+    if not keep:
+        return 1, 1, _prod(shape)
+    if keep != list(range(keep[0], keep[-1] + 1)):
+        # unit dims between kept dims do not break contiguity
+        for d in range(keep[0], keep[-1] + 1):
+            if d not in keep and shape[d] != 1:
+                return None
+    lo, hi = keep[0], keep[-1]
+    return _prod(shape[:lo]), _prod(shape[lo:hi + 1]), _prod(shape[hi + 1:])
+
+
+def layout_from_amax_shape(x_shape, amax_shape):
+    """[outer, axis, inner] for an amax whose shape broadcasts against ``x_shape`` (per-tensor,
+    or equal to x on a contiguous run of dims and 1 elsewhere)."""
+    n = _prod(amax_shape)
+    if n == 1:
+        return 1, 1, _prod(x_shape)
+    a = list(amax_shape)
+    if len(a) == 1 and len(x_shape) >= 1:
+        # squeezed per-channel amax: the reference matches it to the dim of equal length
+        if a[0] in list(x_shape):
+            d = list(x_shape).index(a[0])
+            return amax_layout(x_shape, [d])
+        return None
+    if len(a) != len(x_shape):
+        return None
+    keep = [d for d in range(len(a)) if a[d] != 1]
+    if any(a[d] != x_shape[d] for d in keep):
+        return None
+    return amax_layout(x_shape, keep)
+
+
+def absmax_accumulate(x: torch.Tensor, acc: torch.Tensor, layout):
+    """acc (fp32, ``axis`` elements) = max(acc, abs-max of x over the reduced dims)."""
+    outer, axis, inner = layout
+    return _hip.absmax_into(x if x.is_contiguous() else x.contiguous(), acc, outer, axis, inner)
+
+
+def reduce_amax_gpu(x: torch.Tensor, reduce_dims, keepdims=True):
+    """``reduce_amax`` on the device: abs-max over ``reduce_dims`` (None = all) in x.dtype."""
+    nd = x.dim()
+    if reduce_dims is None:
+        keep, out_shape = [], ()
+    else:
+        red = {d % nd for d in ([reduce_dims] if isinstance(reduce_dims, int) else reduce_dims)}
+        keep = [d for d in range(nd) if d not in red]
+        out_shape = tuple(1 if d in red else x.shape[d] for d in range(nd)) if keepdims else tuple(
+            x.shape[d] for d in keep)
+    layout = amax_layout(tuple(x.shape), keep)
+    if layout is None:
+        raise NotImplementedError(
+            "abs-max that keeps non-adjacent dims is not covered by the kernels (amax with more "
+            "than one non-unit run of dims)")
+    acc = torch.zeros(layout[1], dtype=torch.float32, device=x.device)
+    absmax_accumulate(x, acc, layout)
+    return acc.to(x.dtype).reshape(out_shape)
+
+
+def _qdq_layout(x, amax):
+    layout = layout_from_amax_shape(tuple(x.shape), tuple(amax.shape))
+    if layout is None:
+        raise NotImplementedError(
+            f"amax of shape {tuple(amax.shape)} against input {tuple(x.shape)}: scales on more than "
+            "one non-adjacent dim are not covered by the kernels")
+    return layout
+
+
+def fake_quant_int(x, amax, num_bits=8, unsigned=False, narrow_range=True):
+    x = x if x.is_contiguous() else x.contiguous()
+    outer, axis, inner = _qdq_layout(x, amax)
+    return _hip.int_qdq(x, amax.reshape(-1).contiguous(), outer, axis, inner, num_bits, unsigned,
+                        narrow_range)
+
+
+def fake_quant_fp8(x, amax=None, saturate=False):
+    x = x if x.is_contiguous() else x.contiguous()
+    if amax is None:
+        return _hip.fp8_qdq(x, None, 1, 1, x.numel(), saturate)
+    outer, axis, inner = _qdq_layout(x, amax)
+    return _hip.fp8_qdq(x, amax.reshape(-1).contiguous(), outer, axis, inner, saturate)
+
+
+def fake_quant_nvfp4(x, global_amax, block_size=16, mode=0):
+    x = x if x.is_contiguous() else x.contiguous()
+    if global_amax.numel() != 1:
+        global_amax = global_amax.amax()
+    return _hip.nvfp4_qdq(x, global_amax.reshape(1), block_size, mode)
+
+
+def mul_last_dim(x, scale):
+    """``x * scale`` for a scale that spans the last dim only."""
+    x = x if x.is_contiguous() else x.contiguous()
+    return _hip.mul_cols(x, scale.reshape(-1).contiguous())

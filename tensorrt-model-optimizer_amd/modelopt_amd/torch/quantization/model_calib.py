@@ -1,0 +1,402 @@
+"""Calibration algorithms: max, SmoothQuant and AWQ-lite.
+
+Reference: modelopt/torch/quantization/model_calib.py:66-185 (``max_calibrate``), :272-306
+(stats collection), :346-408 (pre-quant-scale folding), :412-496 (``smoothquant``), :530-786
+(``awq_lite``).  Single GPU: every distributed synchronisation of the reference is a no-op here.
+The per-element work (abs-max, scaling, quantize-dequantize, column statistics, squared error)
+runs in the HIP kernels; the search GEMM is a plain library GEMM (``F.linear``).
+"""
+
+import types
+import warnings
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from ... import _hip
+from .conversion import set_quantizer_by_cfg_context
+from .nn import QuantModule, SequentialQuantizer, TensorQuantizer
+from .utils import is_quantized_linear
+
+__all__ = ["max_calibrate", "smoothquant", "awq", "awq_lite", "enable_stats_collection",
+           "finish_stats_collection", "apply_pre_quant_scale_and_smooth"]
+
+
+# ----------------------------------------------------------------------------- max
+def weight_only_quantize(model: nn.Module):
+    """Show every weight to its quantizer once (no activations involved)."""
+    seen = set()
+    for module in model.modules():
+        if module in seen:
+            continue
+        if isinstance(module, QuantModule) and hasattr(module, "weight_quantizer") and getattr(
+                module, "weight", None) is not None:
+            module.weight_quantizer(module.weight)
+        seen.add(module)
+
+
+def enable_stats_collection(model: nn.Module):
+    """Switch every enabled quantizer to calibration (quantisation off, statistics on)."""
+    for module in model.modules():
+        if isinstance(module, TensorQuantizer) and not module._disabled:
+            if module._calibrator is not None:
+                module.disable_quant()
+                module.enable_calib()
+            else:
+                module.disable()
+
+
+def finish_stats_collection(model: nn.Module, method: str | None = None):
+    """Load the collected amax into ``_amax`` and switch quantisation back on."""
+    for module in model.modules():
+        if not isinstance(module, TensorQuantizer) or module._disabled:
+            continue
+        cal = getattr(module, "_calibrator", None)
+        if cal and not getattr(module, "_dynamic", False) and cal.compute_amax() is not None:
+            module.load_calib_amax()
+        module.enable_quant()
+        module.disable_calib()
+
+
+@torch.no_grad()
+def max_calibrate(model: nn.Module, forward_loop=None, distributed_sync=True):
+    """Max calibration: run ``forward_loop(model)`` with statistics collection on."""
+    enable_stats_collection(model)
+    if forward_loop is None:
+        weight_only_quantize(model)
+    else:
+        forward_loop(model)
+    finish_stats_collection(model)
+
+
+# ----------------------------------------------------------------------------- pre-quant scale
+_ENABLE_FOLDING_PQS_TO_WEIGHTS = True
+
+
+@torch.no_grad()
+def _apply_weight_pre_quant_scale(linear, pre_quant_scale):
+    """``W <- dtype(W * s[None, :])`` with an fp32 ``s`` (one product, one rounding), then
+    recalibrate the weight amax."""
+    if _ENABLE_FOLDING_PQS_TO_WEIGHTS:
+        s = pre_quant_scale.to(linear.weight.device).squeeze().to(torch.float32).contiguous()
+        _hip.mul_cols(linear.weight.data, s, out=linear.weight.data)
+    else:
+        linear.weight_quantizer._enable_pre_quant_scale = True
+        linear.weight_quantizer.pre_quant_scale = pre_quant_scale.squeeze()[None, :].to(
+            linear.weight.dtype)
+    linear.weight_quantizer.reset_amax()
+    max_calibrate(linear, lambda lin: lin.weight_quantizer(lin.weight))
+
+
+@torch.no_grad()
+def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.Tensor | None = None):
+    """Set the input ``pre_quant_scale`` and fold its inverse into the weight."""
+    assert is_quantized_linear(linear), "Only quantized linear modules are supported"
+    assert linear.input_quantizer.pre_quant_scale is None, "pre_quant_scale should be None first!"
+    if pre_quant_scale is None:
+        pre_quant_scale = getattr(linear.input_quantizer, "_pre_quant_scale", None)
+    assert pre_quant_scale is not None, "pre_quant_scale should be provided or already set"
+    assert torch.all(pre_quant_scale > 0), "pre_quant_scale should be positive"
+    pre_quant_scale = pre_quant_scale.to(torch.float32)  # fp32 keeps the scaling maths safe
+
+    linear.input_quantizer._enable_pre_quant_scale = True
+    linear.input_quantizer.pre_quant_scale = pre_quant_scale.to(linear.weight.dtype)
+    _apply_weight_pre_quant_scale(linear, 1.0 / pre_quant_scale)
+
+    if linear.input_quantizer.amax is not None:
+        assert hasattr(linear.input_quantizer, "_amax_for_smoothing")
+        device, dtype = linear.weight.device, linear.weight.dtype
+        smoothing = linear.input_quantizer._amax_for_smoothing.to(device=device, dtype=dtype)
+        linear.input_quantizer.amax = (smoothing * pre_quant_scale.to(device)).amax().to(dtype)
+
+
+# ----------------------------------------------------------------------------- SmoothQuant
+@torch.no_grad()
+def smoothquant(model: nn.Module, forward_loop=None, alpha=1.0):
+    """SmoothQuant with per-channel weight scaling for INT8 linears."""
+    assert forward_loop is not None, "forward_loop must be provided for smoothquant"
+    for module in model.modules():
+        if (is_quantized_linear(module) and module.input_quantizer.is_enabled
+                and module.input_quantizer.axis is None):
+            module.input_quantizer.axis = -1
+    max_calibrate(model, forward_loop)
+
+    def postprocess(module):
+        act_amax = module.input_quantizer.amax.float()
+        w = module.weight
+        device, dtype = w.device, w.dtype
+        col = torch.zeros(w.shape[1], dtype=torch.float32, device=device)
+        _hip.absmax_into(w.data.contiguous(), col, w.shape[0], w.shape[1], 1)
+        weight_scale = col.to(dtype).reshape(1, -1)  # == w.abs().amax(dim=0, keepdim=True)
+        scale_a = (weight_scale.pow(1 - alpha) / act_amax.pow(alpha)).squeeze()
+        module.input_quantizer._amax_for_smoothing = act_amax.cpu()
+        module.input_quantizer.reset_amax()
+        module.input_quantizer.axis = None
+        module.input_quantizer.amax = act_amax.amax().to(dtype=dtype, device=device)
+        eps = 1.0 / (1 << 31)
+        if scale_a.min() <= eps:  # channels that never fired would make scale_a overflow
+            scale_a[act_amax.reshape(-1) <= eps] = 1
+        scale_a = scale_a.clamp(min=1e-4, max=1e4)
+        apply_pre_quant_scale_and_smooth(module, scale_a)
+
+    smoothed = 0
+    for name, module in model.named_modules():
+        if not is_quantized_linear(module):
+            continue
+        if not hasattr(module.input_quantizer, "_amax"):
+            warnings.warn(f"{name} is not calibrated, skip smoothing")
+            continue
+        if module.input_quantizer.num_bits != 8 or module.weight_quantizer.num_bits != 8:
+            warnings.warn(f"Only int8 smoothing is supported, skip {name}")
+            continue
+        if module.input_quantizer.axis != -1:
+            warnings.warn(f"Only per-channel smoothing is supported, skip {name}")
+            continue
+        assert module.input_quantizer._amax.numel() > 1, f"Error: {name} has only one channel to smooth"
+        postprocess(module)
+        smoothed += 1
+    print(f"Smoothed {smoothed} modules")
+
+
+# ----------------------------------------------------------------------------- AWQ-lite
+def awq(model: nn.Module, forward_loop=None, algorithm: str = "awq_lite", **kwargs):
+    with SequentialQuantizer.convert_to_single_quantizer(model):
+        if algorithm in ("awq_full", "awq_lite"):
+            awq_lite(model, forward_loop, **kwargs)
+        if algorithm in ("awq_full", "awq_clip"):
+            raise NotImplementedError("awq_clip is outside the hot path built here")
+    for module in model.modules():
+        if is_quantized_linear(module) and isinstance(module.weight_quantizer, SequentialQuantizer):
+            max_calibrate(module, lambda lin: lin.weight_quantizer(lin.weight))
+
+
+def _awq_block_size(weight, quantizer):
+    if quantizer.block_sizes is None:
+        return None
+    return quantizer.block_sizes.get(-1) or quantizer.block_sizes.get(weight.dim() - 1)
+
+
+def get_weight_scale(weight, block_size=None):
+    """fp32 [K]: column mean of ``|w| / (block amax + tiny)``, every step rounded in the weight
+    dtype like the reference's tensor expression."""
+    n, k = weight.shape
+    w = weight.data.contiguous()
+    dev = w.device
+    if block_size:
+        nb = -(-k // block_size)
+        if k % block_size:
+            w_blk = F.pad(w, (0, nb * block_size - k))
+        else:
+            w_blk = w
+        blk_amax = torch.zeros(n * nb, dtype=torch.float32, device=dev)
+        _hip.absmax_into(w_blk, blk_amax, 1, n * nb, block_size)
+        bs = block_size
+    else:
+        blk_amax = torch.zeros(n, dtype=torch.float32, device=dev)
+        _hip.absmax_into(w, blk_amax, 1, n, k)
+        bs = k
+    acc = torch.zeros(k, dtype=torch.float32, device=dev)
+    _hip.abs_colsum_into(w, acc, blk_amax, bs)
+    return (acc / n).to(weight.dtype).to(torch.float32)
+
+
+def get_act_scale(x):
+    """fp32 [K]: mean over tokens of ``|x|`` rounded in the activation dtype."""
+    x2 = x.contiguous().view(-1, x.shape[-1])
+    acc = torch.zeros(x2.shape[1], dtype=torch.float32, device=x.device)
+    _hip.abs_colsum_into(x2, acc)
+    return (acc / x2.shape[0]).to(x.dtype).to(torch.float32)
+
+
+def get_scale(x_max, w_max, alpha):
+    scales = (x_max.pow(alpha) / (w_max.to(x_max.device).pow(1 - alpha)
+                                  + torch.finfo(torch.float32).tiny)).clamp(min=1e-4, max=1e4).view(-1)
+    return (scales / (scales.max() * scales.min()).sqrt()).view(-1)
+
+
+class _AWQLiteHelper:
+    cache_mode: bool = False
+
+    def __init__(self, module, name, alpha_step):
+        self.name = name
+        self.act_scale = 0.0
+        self.num_cache_steps = 0
+        self.num_search_steps = 0
+        self.block_size = _awq_block_size(module.weight, module.weight_quantizer)
+        self.weight_scale = get_weight_scale(module.weight, self.block_size)
+        dev = module.weight.device
+        self.alphas = [k.item() for k in torch.arange(0, 1.0 + alpha_step, alpha_step)]
+        self.sq_err_steps = []  # per search step: (float64 [n_alphas] sums of squared error, numel)
+        self.loss = {a: 0.0 for a in self.alphas}
+        self.best_scale = None
+        self.best_alpha = None
+        self.is_input_quantized = module.input_quantizer.is_enabled
+        self.num_tokens = 0
+        self.module = module
+        self.is_enabled = True
+
+    def setup(self):
+        m = self.module
+        m._forward_no_awq = m.forward
+        m.forward = types.MethodType(_awq_forward, m)
+        if m.input_quantizer.is_enabled:
+            m.input_quantizer.disable()
+            if m.input_quantizer.axis not in (None, -1):
+                self.is_enabled = False
+                return
+            m.input_quantizer.axis = -1
+
+    def cleanup(self):
+        m = self.module
+        if hasattr(m, "_if_calib"):
+            delattr(m, "_if_calib")
+        if "forward" in m.__dict__:
+            del m.__dict__["forward"]
+        if hasattr(m, "_forward_no_awq"):
+            del m.__dict__["_forward_no_awq"]
+
+
+def _fused_weight_path(module):
+    """True when the weight quantizer is a plain static last-axis INT block quantizer, so the
+    per-alpha weight path can run as one fused kernel."""
+    q = module.weight_quantizer
+    if not isinstance(q, TensorQuantizer) or not isinstance(q._num_bits, int):
+        return False
+    bs = q.block_sizes
+    if not bs or bs.get("type", "static") == "dynamic" or not q.fake_quant or hasattr(q, "_amax"):
+        return False
+    axes = {k: v for k, v in bs.items() if isinstance(k, int)}
+    if list(axes) not in ([-1], [module.weight.dim() - 1]):
+        return False
+    b = next(iter(axes.values()))
+    return b in (8, 16, 32, 64, 128, 256, 512) and module.weight.dtype in (
+        torch.bfloat16, torch.float16, torch.float32)
+
+
+def _awq_forward(self, input, *args, **kwargs):
+    """Replacement ``forward`` of a quantised linear during AWQ-lite (cache pass, then search)."""
+    helper = self.awq_lite
+    self.weight_quantizer.disable()
+    for q in (self.input_quantizer, self.weight_quantizer):
+        if hasattr(q, "_pre_quant_scale"):
+            delattr(q, "_pre_quant_scale")
+    out_actual = self._forward_no_awq(input, *args, **kwargs)
+    self.weight_quantizer.enable()
+    if input.numel() == 0 or not helper.is_enabled:
+        return out_actual
+
+    if _AWQLiteHelper.cache_mode:
+        helper.act_scale += get_act_scale(self.input_quantizer(input))
+        helper.num_cache_steps += 1
+        helper.num_tokens += input.numel() / input.shape[-1]
+        if helper.is_input_quantized:
+            with set_quantizer_by_cfg_context(self.input_quantizer, {"*": {"enable": True}}):
+                max_calibrate(self.input_quantizer, lambda quantizer: quantizer(input), False)
+        return out_actual
+
+    ref = out_actual[0] if isinstance(out_actual, tuple) else out_actual
+    ref = ref.contiguous()
+    dtype = self.weight.dtype
+    fused = _fused_weight_path(self) and not args and not kwargs
+    sq_err = torch.zeros(len(helper.alphas), dtype=torch.float64, device=ref.device)
+    for i, alpha in enumerate(helper.alphas):
+        awq_scale = get_scale(helper.act_scale, helper.weight_scale, alpha)
+        if fused:
+            q = self.weight_quantizer
+            xs = self.input_quantizer(_hip.mul_cols(input.contiguous(), (1 / awq_scale).to(dtype)))
+            wq = _hip.scale_block_int_qdq(self.weight.data.contiguous(), awq_scale.to(dtype),
+                                          _awq_block_size(self.weight, q), q._num_bits, q._unsigned,
+                                          q._narrow_range)
+            out = self.output_quantizer(F.linear(xs, wq, self.bias))
+        else:
+            self.input_quantizer.pre_quant_scale = (1 / awq_scale).to(dtype)
+            self.weight_quantizer.pre_quant_scale = awq_scale.to(dtype)
+            out = self._forward_no_awq(input, *args, **kwargs)
+            out = out[0] if isinstance(out, tuple) else out
+        _hip.sq_diff_sum_into(out.contiguous(), ref, sq_err[i:i + 1])
+    helper.sq_err_steps.append((sq_err, ref.numel()))
+    helper.num_search_steps += 1
+    return out_actual
+
+
+def _finalize_losses(helper):
+    """loss[alpha] = sum over search steps of that step's mean squared error.  The kernel leaves
+    per-step sums of squares on the device; this is the one host synchronisation of the search."""
+    if not helper.sq_err_steps:
+        return {a: 0.0 for a in helper.alphas}
+    sums = torch.stack([s for s, _ in helper.sq_err_steps])
+    sizes = torch.tensor([n for _, n in helper.sq_err_steps], dtype=torch.float64,
+                         device=sums.device)
+    total = (sums / sizes[:, None]).sum(0).cpu().tolist()
+    return dict(zip(helper.alphas, total))
+
+
+@torch.no_grad()
+def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: bool = False, **kwargs):
+    """AWQ-lite: per linear, search ``alpha`` of the scale ``s = act^alpha / w^(1-alpha)`` that
+    minimises the output error of the quantised layer, then fold the best scale."""
+    if forward_loop is None:
+        warnings.warn("forward_loop must be provided for awq_lite; skipping awq_lite")
+        return
+
+    for name, module in model.named_modules():
+        if is_quantized_linear(module) and module.weight_quantizer.is_enabled:
+            module.awq_lite = _AWQLiteHelper(module, name, alpha_step)
+            module.awq_lite.setup()
+
+    _AWQLiteHelper.cache_mode = True
+    print("awq_lite: Caching activation statistics...")
+    enable_stats_collection(model)
+    forward_loop(model)
+    max_calibrate(model, lambda model: None)
+
+    for name, module in model.named_modules():
+        if is_quantized_linear(module) and hasattr(module, "awq_lite") and module.awq_lite.num_cache_steps > 0:
+            module._if_calib = True
+            h = module.awq_lite
+            h.act_scale = h.act_scale / h.num_cache_steps
+            if bool(torch.any(torch.isnan(h.act_scale)) or torch.any(torch.isnan(h.weight_scale))):
+                h.is_enabled = False
+
+    _AWQLiteHelper.cache_mode = False
+    print("awq_lite: Searching parameters...")
+    forward_loop(model)
+
+    def postprocess(module, name):
+        h = module.awq_lite
+        if h.is_enabled:
+            h.loss = _finalize_losses(h)
+            h.best_alpha = min(h.loss, key=h.loss.get)
+            h.best_scale = get_scale(h.act_scale, h.weight_scale, h.best_alpha)
+        for q in (module.weight_quantizer, module.input_quantizer):
+            if hasattr(q, "_pre_quant_scale"):
+                delattr(q, "_pre_quant_scale")
+        if h.is_input_quantized and module.input_quantizer.amax is not None:
+            act_amax = module.input_quantizer.amax
+            module.input_quantizer._amax_for_smoothing = act_amax.cpu()
+            module.input_quantizer.reset_amax()
+            module.input_quantizer.axis = None
+            module.input_quantizer.amax = act_amax.amax()
+            module.input_quantizer.enable()
+        if h.is_enabled:
+            apply_pre_quant_scale_and_smooth(module, 1.0 / h.best_scale)
+        else:
+            warnings.warn(f"awq_lite: Disabling for {name}, quantizing with max calibration.")
+            max_calibrate(module, lambda module: module.weight_quantizer(module.weight))
+
+    for name, module in model.named_modules():
+        if hasattr(module, "awq_lite"):
+            h = module.awq_lite
+            if h.num_cache_steps == 0:
+                h.is_enabled = False
+            elif h.num_search_steps == 0:
+                h.is_enabled = False
+                warnings.warn(
+                    "awq_lite: Calling `forward_loop(model)` the second time did not forward data "
+                    f"through the {name}. Please provide a valid `forward_loop` function that can "
+                    "be used to forward data through the model many times.")
+            postprocess(module, name)
+            h.cleanup()
+            if not debug:
+                delattr(module, "awq_lite")

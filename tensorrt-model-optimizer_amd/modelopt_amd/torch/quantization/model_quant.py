@@ -1,0 +1,118 @@
+"""User-facing API: ``quantize``, ``calibrate`` and helpers.
+
+Reference: modelopt/torch/quantization/model_quant.py:53-118 (``calibrate``), :136-231
+(``quantize``).  ``quantize(model, config, forward_loop)`` converts the model in place (module
+swap + quantizer attributes) and runs the configured calibration algorithm; the reference's
+mode registry / state manager (``apply_mode``) is not reproduced.
+"""
+
+import copy
+import fnmatch
+import warnings
+from collections.abc import Callable
+
+import torch
+from torch import nn
+
+from . import model_calib
+from .config import QuantizeConfig, QuantizerAttributeConfig, normalize_algorithm
+from .conversion import is_converted, replace_quant_module, set_quantizer_attribute, set_quantizer_by_cfg
+from .nn import SequentialQuantizer, TensorQuantizer
+
+__all__ = ["quantize", "calibrate", "disable_quantizer", "enable_quantizer", "print_quant_summary",
+           "fold_weight", "postprocess_amax"]
+
+ForwardLoop = Callable[[nn.Module], None]
+
+
+def _full_attribute_cfg(cfg):
+    """What pydantic validation of the reference's ``QuantizeConfig`` does to an attribute dict:
+    it becomes a complete ``QuantizerAttributeConfig`` (unspecified fields take their defaults),
+    so a later pattern replaces, rather than patches, what an earlier one set."""
+    if isinstance(cfg, QuantizerAttributeConfig):
+        return cfg
+    if isinstance(cfg, (list, tuple)):
+        return [_full_attribute_cfg(c) for c in cfg]
+    if isinstance(cfg, dict):
+        try:
+            return QuantizerAttributeConfig(**cfg)
+        except Exception:
+            # class-scoped entry such as "nn.BatchNorm1d": {"*": {...}}
+            if all(isinstance(v, (dict, list, QuantizerAttributeConfig)) for v in cfg.values()):
+                return {k: _full_attribute_cfg(v) for k, v in cfg.items()}
+            raise
+    raise TypeError(f"unsupported quantizer config entry: {cfg!r}")
+
+
+def _validated(config):
+    config = config if isinstance(config, QuantizeConfig) else QuantizeConfig(**dict(config))
+    quant_cfg = {k: _full_attribute_cfg(v) for k, v in config.quant_cfg.items()}
+    return quant_cfg, config.algorithm
+
+
+def calibrate(model: nn.Module, algorithm="max", forward_loop: ForwardLoop | None = None) -> nn.Module:
+    """Run a calibration algorithm (``"max"``, ``"smoothquant"``, ``"awq_lite"``, a dict with
+    ``"method"``, or ``None``) on a converted model."""
+    method, kwargs = normalize_algorithm(algorithm)
+    if method is None:
+        return model
+    training = model.training
+    model.eval()
+    try:
+        if method == "max":
+            model_calib.max_calibrate(model, forward_loop, kwargs.get("distributed_sync", True))
+        elif method == "smoothquant":
+            model_calib.smoothquant(model, forward_loop, alpha=kwargs.get("alpha", 1.0))
+        elif method == "awq_lite":
+            model_calib.awq(model, forward_loop, "awq_lite", alpha_step=kwargs.get("alpha_step", 0.1),
+                            debug=kwargs.get("debug", False))
+        for name, module in model.named_modules():
+            if isinstance(module, TensorQuantizer):
+                for attr in ("_amax", "_pre_quant_scale"):
+                    module.validate_attr(attr_name=attr, warn_error=True, name=name)
+    finally:
+        model.train(training)
+    return model
+
+
+def quantize(model: nn.Module, config, forward_loop: ForwardLoop | None = None) -> nn.Module:
+    """Quantise and calibrate ``model`` in place and return it.
+
+    ``config`` is ``{"quant_cfg": {wildcard: quantizer attributes, ...}, "algorithm": ...}`` (for
+    instance ``NVFP4_DEFAULT_CFG``); ``forward_loop(model)`` feeds the calibration data.
+    """
+    quant_cfg, algorithm = _validated(config)
+    if not is_converted(model):
+        replace_quant_module(model)
+    set_quantizer_by_cfg(model, quant_cfg)
+    return calibrate(model, algorithm, forward_loop=forward_loop)
+
+
+def disable_quantizer(model: nn.Module, wildcard_or_filter_func):
+    set_quantizer_attribute(model, wildcard_or_filter_func, {"enable": False})
+
+
+def enable_quantizer(model: nn.Module, wildcard_or_filter_func):
+    set_quantizer_attribute(model, wildcard_or_filter_func, {"enable": True})
+
+
+def print_quant_summary(model: nn.Module):
+    count = 0
+    for name, mod in model.named_modules():
+        if isinstance(mod, TensorQuantizer):
+            print(f"{name:80} {mod}")
+            count += 1
+    print(f"{count} TensorQuantizers found in model")
+
+
+def fold_weight(model: nn.Module):
+    for module in model.modules():
+        if hasattr(module, "fold_weight") and hasattr(module, "weight_quantizer"):
+            module.fold_weight()
+
+
+def postprocess_amax(model: nn.Module, key: str, post_process_fn) -> None:
+    """Apply ``post_process_fn`` to the amax of every quantizer whose name matches ``key``."""
+    for name, module in model.named_modules():
+        if isinstance(module, TensorQuantizer) and fnmatch.fnmatch(name, key) and module.amax is not None:
+            module.amax = post_process_fn(module.amax)

@@ -1,0 +1,103 @@
+"""NVFP4 real quantisation (reference: qtensor/nvfp4_tensor.py:31-297) on the HIP kernels.
+
+Layout: ``packed`` uint8 [..., K/2] with byte i = code[2i] | code[2i+1] << 4 (code = sign << 3 |
+E2M1 ordinal); per-block scales ``float8_e4m3fn`` [..., K/block]; one fp32 global scale
+``amax / (6 * 448)``.  The last dim is zero padded to a multiple of the block.
+"""
+
+import torch
+
+from .... import _hip
+from ..utils import reduce_amax, reduce_block_amax
+from .base_qtensor import BaseQuantizedTensor
+
+__all__ = ["NVFP4QTensor"]
+
+e2m1_bounds = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5])
+e2m1_values = torch.tensor([0, 0.5, 1, 1.5, 2, 3, 4, 6, 0, -0.5, -1, -1.5, -2, -3, -4, -6])
+
+
+def _f32_scalar(t: torch.Tensor):
+    return t.detach().reshape(()).to(torch.float32)
+
+
+class NVFP4QTensor(BaseQuantizedTensor):
+    """Packed NVFP4 tensor."""
+
+    @classmethod
+    def get_weights_scaling_factor_2_from_quantizer(cls, weight_quantizer):
+        assert hasattr(weight_quantizer, "_amax"), "Weight quantizer does not have attribute amax"
+        return weight_quantizer._amax.float() / (6.0 * 448.0)
+
+    @classmethod
+    def get_weights_scaling_factor_2(cls, input: torch.Tensor):
+        return reduce_amax(input).float() / (6.0 * 448.0)
+
+    @classmethod
+    def get_weights_scaling_factor(cls, input, block_size, weights_scaling_factor_2=None,
+                                   keep_high_precision=False):
+        """Per-block scale (E4M3 unless ``keep_high_precision``) and the global scale."""
+        if weights_scaling_factor_2 is None:
+            weights_scaling_factor_2 = cls.get_weights_scaling_factor_2(input)
+        assert block_size != 0, "Block size is zero. Cannot return per_block amax for given input."
+        assert input.shape[-1] % block_size == 0, (
+            "Weight shape is not divisible for block size for block quantization.")
+        wsf2 = weights_scaling_factor_2.to(input.device)
+        if keep_high_precision:
+            bamax = reduce_block_amax(input, {-1: block_size}).float()
+            scale = bamax / (6.0 * wsf2)
+            scale[scale == 0] = 1.0
+            return scale, weights_scaling_factor_2
+        _, wsf, _ = _hip.nvfp4_quantize(input.contiguous(), _f32_scalar(wsf2), block_size,
+                                        amax_is_wsf2=True)
+        return wsf, weights_scaling_factor_2
+
+    @classmethod
+    def get_activation_scaling_factor(cls, quantizer):
+        if not quantizer.is_enabled:
+            return None
+        amax = quantizer.export_amax()
+        if amax is None:
+            return None
+        sf = amax.float() / (quantizer.maxbound * 448.0)
+        assert torch.all(sf > 0), f" activation scaling factor {sf} not positive."
+        return sf
+
+    @classmethod
+    def quantize(cls, input, block_size, weights_scaling_factor=None, weights_scaling_factor_2=None,
+                 keep_high_precision=False, try_tensorrt=False):
+        """Returns (NVFP4QTensor, per-block E4M3 scales, fp32 global scale) in one kernel pass
+        (plus one abs-max pass when the global scale is not given)."""
+        if keep_high_precision:
+            raise NotImplementedError("keep_high_precision=True (un-rounded scaled weights) is not built")
+        shape, dtype = input.shape, input.dtype
+        x = input.contiguous()
+        if weights_scaling_factor_2 is None:
+            acc = torch.zeros(1, dtype=torch.float32, device=x.device)
+            _hip.absmax_into(x, acc, 1, 1, x.numel())
+            scalar, is_wsf2 = acc.reshape(()), False
+        else:
+            scalar, is_wsf2 = _f32_scalar(weights_scaling_factor_2.to(x.device)), True
+        wsf_in = None
+        if weights_scaling_factor is not None:
+            wsf_in = weights_scaling_factor.to(x.device).contiguous()
+            assert wsf_in.dtype == torch.float8_e4m3fn, "block scales must be float8_e4m3fn"
+        packed, wsf, wsf2 = _hip.nvfp4_quantize(x, scalar, block_size, is_wsf2, wsf_in)
+        if weights_scaling_factor is not None:
+            wsf = weights_scaling_factor
+        if weights_scaling_factor_2 is not None:
+            wsf2 = weights_scaling_factor_2
+        return cls(shape, dtype, packed), wsf, wsf2
+
+    def dequantize(self, dtype: torch.dtype = None, fast=False, **kwarg):
+        """``dtype(LUT[code] * (f32(scale) * double_scale))`` reshaped to the original shape."""
+        if dtype is None:
+            dtype = self.metadata["dtype"]
+        scale, wsf2 = kwarg["scale"], kwarg["double_scale"]
+        block = kwarg["block_sizes"][-1]
+        if scale.dtype != torch.float8_e4m3fn:
+            raise NotImplementedError("NVFP4 dequantize needs float8_e4m3fn block scales")
+        packed = self._quantized_data
+        y = _hip.nvfp4_dequantize(packed.contiguous(), scale.to(packed.device).contiguous(),
+                                  _f32_scalar(wsf2.to(packed.device)), block, dtype)
+        return y.reshape(self.metadata["shape"])

@@ -1,0 +1,112 @@
+"""Quantization utilities with the reference's names (modelopt/torch/quantization/utils.py),
+backed by the HIP abs-max kernels."""
+
+import torch
+import torch.nn.functional as F
+
+from . import kernels
+
+__all__ = [
+    "convert_quantization_axis_to_reduce_axis", "reduce_amax", "reduce_block_amax",
+    "reduce_block_padding", "is_quantized", "is_quantized_linear",
+    "update_quant_cfg_with_kv_cache_quant", "quantizer_attr_names", "weight_attr_names",
+]
+
+
+def convert_quantization_axis_to_reduce_axis(input, axis):
+    """Quantization axis -> dims to reduce (reference: utils.py:137-152)."""
+    if axis is None:
+        return None
+    kept = list(axis) if isinstance(axis, (list, tuple)) else [axis]
+    nd = input.dim()
+    return [d for d in range(nd) if d not in kept and (d - nd) not in kept]
+
+
+@torch.no_grad()
+def reduce_amax(input, axis=None, keepdims=True, squeeze_scalar=True):
+    """Abs-max over ``axis`` (None = everything) in the input dtype (reference: utils.py:156-188).
+
+    One kernel pass (the reference reads the tensor twice: max and min); NaN propagates.
+    """
+    if axis is None:
+        return kernels.reduce_amax_gpu(input, None)
+    out = kernels.reduce_amax_gpu(input, axis, keepdims=keepdims)
+    if squeeze_scalar and out.numel() == 1:
+        out = out.squeeze()
+    return out
+
+
+@torch.no_grad()
+def reduce_block_padding(input, block_sizes: dict, pad_value: float = 0):
+    """Right-pad the listed dims to multiples of their block (reference: utils.py:101-134)."""
+    nd = input.dim()
+    for dim, blk in block_sizes.items():
+        d = dim if dim >= 0 else nd + dim
+        rem = input.size(d) % blk
+        if rem:
+            spec = [0] * (2 * nd)
+            spec[(nd - 1 - d) * 2 + 1] = blk - rem
+            input = F.pad(input, spec, value=pad_value)
+    return input
+
+
+@torch.no_grad()
+def reduce_block_amax(input_tensor, block_sizes: dict):
+    """Blockwise abs-max, one listed dim at a time (reference: utils.py:52-98)."""
+    out = input_tensor
+    for dim, blk in block_sizes.items():
+        d = dim if dim >= 0 else out.dim() + dim
+        assert out.shape[d] % blk == 0, (
+            f"Tensor dimension {out.shape[d]} is not divisible by {blk}")
+        shape = list(out.shape)
+        shape[d:d + 1] = [shape[d] // blk, blk]
+        out = reduce_amax(out.reshape(shape), d + 1, keepdims=False, squeeze_scalar=False)
+    return out
+
+
+def is_quantized(module):
+    from .nn import TensorQuantizer
+
+    return any(isinstance(m, TensorQuantizer) for m in module.modules())
+
+
+def is_quantized_linear(module):
+    """A module with input/weight quantizers and a 2-D weight (reference: utils.py:222-232)."""
+    from .nn import SequentialQuantizer, TensorQuantizer
+
+    return (
+        hasattr(module, "input_quantizer") and hasattr(module, "weight_quantizer")
+        and isinstance(module.input_quantizer, (TensorQuantizer, SequentialQuantizer))
+        and isinstance(module.weight_quantizer, (TensorQuantizer, SequentialQuantizer))
+        and getattr(module, "weight", None) is not None and module.weight.dim() == 2
+    )
+
+
+class _QuantizerNames:
+    def __init__(self, weight_name="weight"):
+        prefix = "" if weight_name == "weight" else weight_name + "_"
+        self.weight_quantizer = prefix + "weight_quantizer"
+        self.input_quantizer = prefix + "input_quantizer"
+        self.output_quantizer = prefix + "output_quantizer"
+
+
+def quantizer_attr_names(weight_name="weight"):
+    return _QuantizerNames(weight_name)
+
+
+def weight_attr_names(module):
+    if hasattr(module, "weight_quantizer") and getattr(module, "weight", None) is not None:
+        yield "weight"
+
+
+def update_quant_cfg_with_kv_cache_quant(quant_cfg: dict, kv_cache_quant_cfg: dict) -> dict:
+    """Merge KV-cache quantizer entries into a config (reference: utils.py:769-781)."""
+    import copy
+
+    quant_cfg = copy.deepcopy(quant_cfg)
+    inner = quant_cfg.get("quant_cfg", {"default": {"enable": False}})
+    inner.update(kv_cache_quant_cfg)
+    quant_cfg["quant_cfg"] = inner
+    if not quant_cfg.get("algorithm"):
+        quant_cfg["algorithm"] = "max"
+    return quant_cfg

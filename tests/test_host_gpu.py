@@ -1,0 +1,349 @@
+"""GPU tests of the host layer (TensorQuantizer, calibrators, mtq.quantize, SmoothQuant,
+AWQ-lite) against the CPU oracle."""
+
+import copy
+import json
+import os
+
+import pytest
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+import modelopt_amd.torch.quantization as mtq
+from conftest import GOLDEN, assert_bits_equal
+from modelopt_amd.torch.quantization import calib
+from modelopt_amd.torch.quantization.config import QuantizerAttributeConfig
+from modelopt_amd.torch.quantization.nn import TensorQuantizer
+from modelopt_amd.torch.quantization.qtensor import NVFP4QTensor
+from oracle import awq as oawq
+from oracle import fake_quant, qtensor, reduce
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+with open(os.path.join(GOLDEN, "reference_vectors.json")) as f:
+    VEC = json.load(f)
+
+
+def _rand(shape, dtype=torch.bfloat16, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+# ----------------------------------------------------------------------------- calibrator
+def test_max_calibrator_like_reference_tests():
+    c = calib.MaxCalibrator(8, None, False)
+    a, b = _rand((16,), torch.float32, 1).abs(), _rand((16,), torch.float32, 2).abs()
+    c.collect(a.to(DEV)); c.collect(b.to(DEV))
+    assert torch.equal(c.compute_amax().cpu(), torch.max(a.max(), b.max()))
+    for axis in (0, -4):
+        c = calib.MaxCalibrator(8, axis, False)
+        a, b = _rand((3, 4, 2, 2), torch.float32, 3), _rand((3, 4, 2, 2), torch.float32, 4)
+        c.collect(a.to(DEV)); c.collect(b.to(DEV))
+        o = reduce.MaxCalibrator(8, axis, False)
+        o.collect(a); o.collect(b)
+        assert c.compute_amax().shape == o.compute_amax().shape
+        assert torch.equal(c.compute_amax().cpu(), o.compute_amax())
+        c.reset()
+        assert c.compute_amax() is None
+    c = calib.MaxCalibrator(8, 0, False)
+    c.collect(_rand((3, 4, 2, 2), torch.float32, 5).to(DEV))
+    with pytest.raises(RuntimeError, match="shape changed"):
+        c.collect(_rand((4, 4, 2, 2), torch.float32, 6).to(DEV))
+
+
+def test_max_calibrator_flags_nan_and_inf_at_compute():
+    c = calib.MaxCalibrator(8, None, False)
+    x = _rand((64,), torch.float32, 7)
+    x[3] = float("nan")
+    c.collect(x.to(DEV))
+    with pytest.raises(AssertionError, match="nan"):
+        c.compute_amax()
+    c = calib.MaxCalibrator(8, None, False)
+    x[3] = float("inf")
+    c.collect(x.to(DEV))
+    with pytest.raises(AssertionError, match="inf"):
+        c.compute_amax()
+
+
+# ----------------------------------------------------------------------------- TensorQuantizer
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_quantizer_int8_per_tensor_and_channel(dtype):
+    x = _rand((32, 64), dtype, 10)
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=8)).to(DEV)
+    y = q(x.to(DEV))  # dynamic amax
+    assert_bits_equal(y.cpu(), fake_quant.tensor_quant(x, reduce.reduce_amax(x), 8, False, False), "dynamic")
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=8, axis=0), amax=None).to(DEV)
+    q.enable_calib(); q.disable_quant()
+    q(x.to(DEV)); q(2 * x.to(DEV))
+    q.load_calib_amax(); q.enable_quant(); q.disable_calib()
+    want_amax = reduce.reduce_amax(2 * x, axis=[1])
+    assert_bits_equal(q.amax.cpu(), want_amax, "calibrated per-channel amax")
+    y = q(x.to(DEV))
+    assert_bits_equal(y.cpu(), fake_quant.tensor_quant(x, want_amax, 8, False, False), "per channel")
+
+
+def test_quantizer_fp8_and_noncontiguous():
+    x = _rand((48, 40), torch.bfloat16, 11)
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=(4, 3)), amax=3.0).to(DEV)
+    y = q(x.to(DEV))
+    assert_bits_equal(y.cpu(), fake_quant.fp8_eager(x, torch.tensor(3.0)), "fp8 static amax")
+    xt = x.to(DEV).t()  # non-contiguous view
+    y = q(xt)
+    assert_bits_equal(y.cpu(), fake_quant.fp8_eager(x.t().contiguous(), torch.tensor(3.0)), "transposed")
+
+
+@pytest.mark.parametrize("k", [256, 200])
+def test_quantizer_int4_static_block(k):
+    x = _rand((24, k), torch.bfloat16, 12, 0.02)
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=4, block_sizes={-1: 128})).to(DEV)
+    y = q(x.to(DEV))
+    assert y.shape == x.shape
+    assert_bits_equal(y.cpu().contiguous(), oawq.int4_block_qdq(x, 128).contiguous(), "block 128 dynamic amax")
+    # calibrated: amax buffer [rows, 1], export shape [N, K/128]
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=4, block_sizes={-1: 128})).to(DEV)
+    q.enable_calib(); q.disable_quant(); q(x.to(DEV)); q.load_calib_amax()
+    q.enable_quant(); q.disable_calib()
+    assert q.amax.shape == (24 * (-(-k // 128)), 1)
+    assert q.export_amax().shape == (24, -(-k // 128))
+    assert_bits_equal(q(x.to(DEV)).cpu().contiguous(), oawq.int4_block_qdq(x, 128).contiguous(), "calibrated")
+
+
+def test_quantizer_nvfp4_dynamic_and_pre_quant_scale():
+    cfg = QuantizerAttributeConfig(num_bits=(2, 1),
+                                   block_sizes={-1: 16, "type": "dynamic", "scale_bits": (4, 3)})
+    x = _rand((4, 8, 64), torch.bfloat16, 13)
+    q = TensorQuantizer(cfg).to(DEV)
+    y = q(x.to(DEV))  # global amax computed on the fly
+    assert_bits_equal(y.cpu(), fake_quant.nvfp4_fake_quant(x, reduce.reduce_amax(x), 16), "dynamic amax")
+    q.amax = torch.tensor(2.5, dtype=torch.bfloat16)
+    assert_bits_equal(q(x.to(DEV)).cpu(), fake_quant.nvfp4_fake_quant(x, torch.tensor(2.5), 16), "static amax")
+    s = (torch.rand(64) + 0.5).to(torch.bfloat16)
+    q.pre_quant_scale = s.to(DEV)
+    assert_bits_equal(q(x.to(DEV)).cpu(), fake_quant.nvfp4_fake_quant(x * s, torch.tensor(2.5), 16), "pqs")
+    q.disable()
+    assert_bits_equal(q(x.to(DEV)).cpu(), x * s, "pre_quant_scale still applied when disabled")
+
+
+@pytest.mark.parametrize("case", [c for c in VEC["qtensor_roundtrip"]
+                                  if c["block_sizes"] is None or len(c["block_sizes"]) == 1],
+                         ids=lambda c: c["name"])
+def test_real_quantize_golden_through_tensor_quantizer(case):
+    """tests/gpu/torch/quantization/test_qtensor_cuda.py:243-262 with the reference's vectors."""
+    bits = tuple(case["num_bits"]) if isinstance(case["num_bits"], list) else case["num_bits"]
+    bs = None if case["block_sizes"] is None else {int(k): v for k, v in case["block_sizes"].items()}
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=bits, block_sizes=bs, fake_quant=False,
+                                                 axis=case["axis"])).to(DEV)
+    x = torch.tensor(case["input"], dtype=torch.bfloat16).to(DEV)
+    packed = q(x)
+    deq = q(packed)
+    assert torch.allclose(deq.cpu(), torch.tensor(case["output"], dtype=torch.bfloat16))
+
+
+def test_nvfp4_real_quantize_uses_quantizer_amax():
+    cfg = QuantizerAttributeConfig(num_bits=(2, 1), fake_quant=False,
+                                   block_sizes={-1: 16, "type": "dynamic", "scale_bits": (4, 3)})
+    q = TensorQuantizer(cfg).to(DEV)
+    q.amax = torch.tensor(1.1)
+    x = torch.rand(32, 32, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    out = q(x.to(DEV))
+    assert torch.allclose(q._double_scale.cpu(), torch.tensor(1.1) / 448.0 / 6.0)
+    wsf2 = torch.tensor(1.1).float() / (448.0 * 6.0)
+    wsf_o, _ = qtensor.nvfp4_block_scales(x, 16, wsf2)
+    p_o, _, _ = qtensor.nvfp4_quantize(x, 16, wsf_o, wsf2)
+    assert_bits_equal(out._quantized_data.cpu(), p_o, "packed")
+    assert_bits_equal(q._scale.cpu(), wsf_o, "block scales")
+    deq = q(out)
+    assert_bits_equal(deq.cpu(), qtensor.nvfp4_dequantize(p_o, wsf_o, wsf2, 16, x.shape, torch.bfloat16), "deq")
+
+
+def test_nvfp4_qtensor_classmethods():
+    x = _rand((16, 64), torch.bfloat16, 14, 0.02)
+    xd = x.to(DEV)
+    assert_bits_equal(NVFP4QTensor.get_weights_scaling_factor_2(xd).cpu(), qtensor.nvfp4_global_scale(x), "wsf2")
+    wsf, wsf2 = NVFP4QTensor.get_weights_scaling_factor(xd, 16)
+    wsf_o, wsf2_o = qtensor.nvfp4_block_scales(x, 16)
+    assert_bits_equal(wsf.cpu(), wsf_o, "wsf")
+    qt, wsf_b, wsf2_b = NVFP4QTensor.quantize(xd, 16, wsf, wsf2)
+    p_o, _, _ = qtensor.nvfp4_quantize(x, 16, wsf_o, wsf2_o)
+    assert_bits_equal(qt._quantized_data.cpu(), p_o, "packed with given scales")
+    hp, _ = NVFP4QTensor.get_weights_scaling_factor(xd, 16, keep_high_precision=True)
+    hp_o, _ = qtensor.nvfp4_block_scales(x, 16, keep_high_precision=True)
+    assert_bits_equal(hp.cpu(), hp_o, "high precision scales")
+
+
+# ----------------------------------------------------------------------------- mtq.quantize
+class _MLP(nn.Module):
+    def __init__(self, d=64, h=128, dtype=torch.bfloat16, seed=0):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+        self.fc1 = nn.Linear(d, h, bias=True)
+        self.fc2 = nn.Linear(h, d, bias=False)
+        self.lm_head = nn.Linear(d, 32, bias=False)
+        for p in self.parameters():
+            p.data = (torch.randn(p.shape, generator=g) * 0.1)
+        self.to(dtype)
+
+    def forward(self, x):
+        return self.lm_head(self.fc2(F.relu(self.fc1(x))))
+
+
+def _batches(n=3, d=64, dtype=torch.bfloat16):
+    return [_rand((8, 16, d), dtype, 100 + i) for i in range(n)]
+
+
+def _oracle_linear_inputs(model, batches):
+    """CPU activations seen by fc1 / fc2 / lm_head with quantisation off (calibration mode)."""
+    acts = {"fc1": [], "fc2": [], "lm_head": []}
+    for x in batches:
+        acts["fc1"].append(x)
+        h = F.relu(F.linear(x, model.fc1.weight, model.fc1.bias))
+        acts["fc2"].append(h)
+        y = F.linear(h, model.fc2.weight)
+        acts["lm_head"].append(y)
+    return acts
+
+
+@pytest.mark.parametrize("cfg_name", ["INT8_DEFAULT_CFG", "FP8_DEFAULT_CFG", "NVFP4_DEFAULT_CFG"])
+def test_quantize_max_calibration_amax_matches_oracle(cfg_name):
+    ref = _MLP()
+    model = copy.deepcopy(ref).to(DEV)
+    batches = _batches()
+    mtq.quantize(model, getattr(mtq, cfg_name), lambda m: [m(b.to(DEV)) for b in batches])
+    assert not model.lm_head.input_quantizer.is_enabled and not model.lm_head.weight_quantizer.is_enabled
+    # calibration runs with quantisation off, so GPU activations equal CPU ones up to GEMM
+    # rounding; the weight amax is exact, the input amax is compared on GPU-side activations
+    w_axis = [1] if cfg_name == "INT8_DEFAULT_CFG" else None
+    for name in ("fc1", "fc2"):
+        lin = getattr(model, name)
+        want = reduce.reduce_amax(getattr(ref, name).weight.data, axis=w_axis)
+        assert_bits_equal(lin.weight_quantizer.amax.cpu().reshape(want.shape), want, f"{name} weight amax")
+    assert_bits_equal(model.fc1.input_quantizer.amax.cpu(),
+                      torch.stack([reduce.reduce_amax(b) for b in batches]).max(), "fc1 input amax")
+    assert model.fc2.input_quantizer.amax.numel() == 1 and model.fc2.input_quantizer.amax > 0
+    out = model(batches[0].to(DEV))
+    assert out.shape == (8, 16, 32) and torch.isfinite(out.float()).all()
+
+
+def test_quantized_linear_forward_equals_oracle_composition():
+    ref = _MLP()
+    model = copy.deepcopy(ref).to(DEV)
+    batches = _batches()
+    mtq.quantize(model, mtq.INT8_DEFAULT_CFG, lambda m: [m(b.to(DEV)) for b in batches])
+    x = batches[1]
+    lin = model.fc1
+    xq = fake_quant.tensor_quant(x, lin.input_quantizer.amax.cpu(), 8, False, False)
+    wq = fake_quant.tensor_quant(ref.fc1.weight.data, lin.weight_quantizer.amax.cpu(), 8, False, False)
+    got_x = lin.input_quantizer(x.to(DEV))
+    got_w = lin.weight_quantizer(lin.weight)
+    assert_bits_equal(got_x.cpu(), xq, "input fake quant")
+    assert_bits_equal(got_w.cpu(), wq, "weight fake quant")
+    y = lin(x.to(DEV))
+    assert torch.allclose(y.cpu().float(), F.linear(xq, wq, ref.fc1.bias).float(), rtol=2e-2, atol=2e-2)
+
+
+def test_weight_amax_is_cached_across_forwards():
+    model = _MLP().to(DEV)
+    mtq.replace_quant_module(model)
+    mtq.set_quantizer_by_cfg(model, mtq.model_quant._validated(mtq.INT8_DEFAULT_CFG)[0])
+    from modelopt_amd.torch.quantization import model_calib
+    model_calib.enable_stats_collection(model)
+    calls = []
+    cal = model.fc1.weight_quantizer._calibrator
+    orig = cal.collect
+    cal.collect = lambda x: (calls.append(1), orig(x))[1]
+    for b in _batches(4):
+        model(b.to(DEV))
+    assert len(calls) == 1  # the unchanged weight was reduced once, not once per forward
+    model.fc1.weight.data.mul_(2)  # touching .data does not bump the version ...
+    model.fc1.weight_quantizer.reset_amax()  # ... so callers reset, as the reference's folding does
+    model(_batches(1)[0].to(DEV))
+    assert len(calls) == 2
+    with torch.no_grad():
+        model.fc1.weight.mul_(0.5)  # an in-place update bumps the version
+    model(_batches(1)[0].to(DEV))
+    assert len(calls) == 3
+    model_calib.finish_stats_collection(model)
+
+
+# ----------------------------------------------------------------------------- SmoothQuant
+def test_smoothquant_matches_oracle():
+    ref = _MLP()
+    model = copy.deepcopy(ref).to(DEV)
+    batches = _batches()
+    cfg = copy.deepcopy(mtq.INT8_SMOOTHQUANT_CFG)
+    cfg["algorithm"] = {"method": "smoothquant", "alpha": 0.5}
+    mtq.quantize(model, cfg, lambda m: [m(b.to(DEV)) for b in batches])
+    act_amax = torch.stack([reduce.reduce_amax(b, axis=[0, 1]) for b in batches]).amax(0)  # [1,1,K]
+    pqs, w_new, in_amax, w_amax = oawq.smoothquant_linear(ref.fc1.weight.data, act_amax, alpha=0.5)
+    lin = model.fc1
+    assert_bits_equal(lin.input_quantizer._pre_quant_scale.cpu().reshape(-1), pqs.reshape(-1), "pre_quant_scale")
+    assert_bits_equal(lin.weight.data.cpu(), w_new, "smoothed weight")
+    assert_bits_equal(lin.input_quantizer.amax.cpu().reshape(()), in_amax.reshape(()), "input amax")
+    assert_bits_equal(lin.weight_quantizer.amax.cpu().reshape(w_amax.shape), w_amax, "weight amax")
+
+
+# ----------------------------------------------------------------------------- AWQ-lite
+class _OneLinear(nn.Module):
+    def __init__(self, n=128, k=256, seed=0):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+        self.proj = nn.Linear(k, n, bias=False)
+        self.proj.weight.data = (0.02 * torch.randn(n, k, generator=g))
+        self.to(torch.bfloat16)
+
+    def forward(self, x):
+        return self.proj(x)
+
+
+def _awq_batches(k=256, n=2, tokens=64):
+    g = torch.Generator().manual_seed(3)
+    c = torch.exp(torch.randn(k, generator=g))
+    hot = torch.randperm(k, generator=g)[: max(1, k // 100)]
+    c[hot] *= 20
+    return [(torch.randn(tokens, k, generator=g) * c).to(torch.bfloat16) for _ in range(n)]
+
+
+@pytest.mark.parametrize("alpha_step", [0.1, 0.05])
+def test_awq_lite_matches_oracle(alpha_step):
+    ref = _OneLinear()
+    model = copy.deepcopy(ref).to(DEV)
+    batches = _awq_batches()
+    cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
+    cfg["algorithm"] = {"method": "awq_lite", "alpha_step": alpha_step, "debug": True}
+    mtq.quantize(model, cfg, lambda m: [m(b.to(DEV)) for b in batches])
+    losses, best_alpha, best_scale, act_scale, weight_scale = oawq.awq_lite_search(
+        ref.proj.weight.data, batches, alpha_step, 128)
+    h = model.proj.awq_lite
+    assert list(h.loss) == list(losses)  # identical fp32 alpha keys
+    assert len(h.loss) == (21 if alpha_step == 0.05 else 11)
+    for a in losses:
+        assert h.loss[a] == pytest.approx(losses[a], rel=1e-3), f"alpha {a}"
+    assert h.best_alpha == best_alpha
+    assert torch.allclose(h.act_scale.cpu(), act_scale, rtol=2 ** -7)
+    assert torch.allclose(h.weight_scale.cpu(), weight_scale, rtol=2 ** -7)
+    # folding: input pre_quant_scale and smoothed weight from the oracle's formula on the
+    # GPU's own best_scale (the statistics may differ from the CPU's in the last bf16 bit)
+    pqs, w_new = oawq.fold_pre_quant_scale(ref.proj.weight.data, 1.0 / h.best_scale.cpu())
+    assert_bits_equal(model.proj.input_quantizer._pre_quant_scale.cpu(), pqs, "pre_quant_scale")
+    assert_bits_equal(model.proj.weight.data.cpu(), w_new, "folded weight")
+    want_amax = reduce.reduce_amax(w_new.reshape(-1, 128), axis=[1], keepdims=True)
+    assert_bits_equal(model.proj.weight_quantizer.amax.cpu(), want_amax, "recalibrated block amax")
+    assert "forward" not in model.proj.__dict__  # patch removed
+
+
+def test_awq_generic_path_equals_fused_path(monkeypatch):
+    from modelopt_amd.torch.quantization import model_calib
+
+    batches = _awq_batches()
+    results = []
+    for fused in (True, False):
+        model = _OneLinear().to(DEV)
+        if not fused:
+            monkeypatch.setattr(model_calib, "_fused_weight_path", lambda m: False)
+        cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
+        cfg["algorithm"] = {"method": "awq_lite", "alpha_step": 0.1, "debug": True}
+        mtq.quantize(model, cfg, lambda m: [m(b.to(DEV)) for b in batches])
+        results.append((model.proj.awq_lite.loss, model.proj.weight.data.clone()))
+    assert results[0][0] == results[1][0]
+    assert torch.equal(results[0][1], results[1][1])
