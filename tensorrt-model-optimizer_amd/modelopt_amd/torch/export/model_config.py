@@ -1,0 +1,17 @@
+"""Format names used in exported configs (reference: export/model_config.py:29-47)."""
+
+QUANTIZATION_NONE = None
+QUANTIZATION_FP8 = "fp8"
+QUANTIZATION_INT8_SQ = "int8_sq"
+QUANTIZATION_INT8_WO = "int8_wo"
+QUANTIZATION_INT4_AWQ = "int4_awq"
+QUANTIZATION_W4A8_AWQ = "w4a8_awq"
+QUANTIZATION_NVFP4 = "nvfp4"
+QUANTIZATION_NVFP4_AWQ = "nvfp4_awq"
+QUANTIZATION_FP8_PC_PT = "fp8_pc_pt"
+
+KV_CACHE_FP8 = "FP8"
+KV_CACHE_INT8 = "INT8"
+KV_CACHE_NVFP4 = "NVFP4"
+
+__all__ = [n for n in dir() if n.startswith(("QUANTIZATION_", "KV_CACHE_"))]

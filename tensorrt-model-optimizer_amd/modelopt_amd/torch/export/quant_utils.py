@@ -1,0 +1,405 @@
+"""Scaling factors, packed weights and state-dict post-processing for export.
+
+Reference: modelopt/torch/export/quant_utils.py (:68-91, :214-320, :373-534, :602-738, :741-834,
+:860-983, :1132-1185, :1190-1288).  The packing itself runs in the HIP kernels.
+"""
+
+import fnmatch
+from types import SimpleNamespace
+from typing import Any
+
+import torch
+from torch import nn
+
+from ... import __version__, _hip
+from ..quantization.nn import SequentialQuantizer, TensorQuantizer
+from ..quantization.qtensor import NVFP4QTensor, QTensorWrapper
+from ..quantization.utils import (quantizer_attr_names, reduce_block_amax, true_divide,
+                                  weight_attr_names)
+from .model_config import *  # noqa: F403
+
+__all__ = [
+    "get_scaling_factor_from_weight", "get_scaling_factor", "get_activation_scaling_factor",
+    "get_weight_scaling_factor", "get_weight_scaling_factor_2", "get_prequant_scaling_factor",
+    "get_kv_cache_dtype", "get_weight_block_size", "get_quantization_format",
+    "process_layer_quant_config", "pack_int4_in_uint8", "to_quantized_weight",
+    "postprocess_state_dict", "preprocess_linear_fusion", "get_quant_config", "all_items_same",
+]
+
+
+def get_scaling_factor_from_weight(weight, group_size) -> torch.Tensor:
+    """``max|w| / 7`` per group of ``group_size`` input channels (``/127`` per row when 0)."""
+    n, k = weight.shape
+    if group_size != 0:
+        if k % group_size != 0:
+            raise NotImplementedError("Weight shape is not divisible for block size for block quantization.")
+        amax = reduce_block_amax(weight.contiguous(), {-1: group_size}).float()
+        bound = 7.0
+    else:
+        acc = torch.zeros(n, dtype=torch.float32, device=weight.device)
+        _hip.absmax_into(weight.contiguous(), acc, 1, n, k)
+        amax, bound = acc, 127.0
+    sf = true_divide(amax, bound)
+    sf[sf == 0] = 1.0
+    return sf
+
+
+def get_scaling_factor(quantizer: TensorQuantizer) -> torch.Tensor | None:
+    if not quantizer.is_enabled:
+        return None
+    amax = quantizer.export_amax()
+    if amax is None:
+        return None
+    if quantizer.num_bits == (2, 1):
+        sf = NVFP4QTensor.get_weights_scaling_factor_2_from_quantizer(quantizer)
+    else:
+        sf = true_divide(amax.float(), quantizer.maxbound)
+    assert torch.all(sf > 0), f"scaling factor {sf} not positive."
+    return sf
+
+
+def get_activation_scaling_factor(module: nn.Module, input_quantizer_name: str = "input_quantizer"):
+    q = getattr(module, input_quantizer_name, None)
+    if q is None:
+        return None
+    if get_quantization_format(module) in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
+        return NVFP4QTensor.get_activation_scaling_factor(q)
+    return get_scaling_factor(q)
+
+
+def get_weight_scaling_factor(module: nn.Module, weight_name: str = "weight"):
+    weight = getattr(module, weight_name)
+    wq = getattr(module, quantizer_attr_names(weight_name).weight_quantizer, None)
+    if wq is None:
+        return None
+    if isinstance(wq, SequentialQuantizer):
+        return get_scaling_factor(wq[0])
+    if get_quantization_format(module) in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
+        wsf2 = NVFP4QTensor.get_weights_scaling_factor_2_from_quantizer(wq)
+        return NVFP4QTensor.get_weights_scaling_factor(weight, wq.block_sizes[-1],
+                                                       wsf2.to(weight.device))[0]
+    return get_scaling_factor(wq)
+
+
+def get_weight_scaling_factor_2(module: nn.Module, weight_name: str = "weight"):
+    wq = getattr(module, quantizer_attr_names(weight_name).weight_quantizer, None)
+    if wq is None:
+        return None
+    if get_quantization_format(module) in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
+        return NVFP4QTensor.get_weights_scaling_factor_2_from_quantizer(wq)
+    if not isinstance(wq, SequentialQuantizer) or not wq[-1].is_enabled:
+        return None
+    assert len(wq) == 2, "modelopt only supports 2 sequential quantization layers for now"
+    return get_scaling_factor(wq[-1])
+
+
+def get_prequant_scaling_factor(module: nn.Module):
+    q = getattr(module, "input_quantizer", None)
+    if q is not None and hasattr(q, "_pre_quant_scale"):
+        return q._pre_quant_scale.squeeze()
+    return None
+
+
+def get_kv_cache_dtype(modules) -> str | None:
+    if isinstance(modules, nn.Module):
+        modules = [modules]
+    bits = []
+    for module in modules:
+        for name in ("k_bmm_quantizer", "v_bmm_quantizer", "output_quantizer"):
+            q = getattr(module, name, None)
+            if q is not None and q.is_enabled:
+                bits.append(q.num_bits)
+    if (4, 3) in bits:
+        return KV_CACHE_FP8
+    if 8 in bits:
+        return KV_CACHE_INT8
+    if (2, 1) in bits:
+        return KV_CACHE_NVFP4
+    return QUANTIZATION_NONE
+
+
+def get_weight_block_size(module: nn.Module, weight_name: str = "weight") -> int:
+    wq = getattr(module, quantizer_attr_names(weight_name).weight_quantizer, None)
+    if wq is None:
+        return 0
+    if isinstance(wq, SequentialQuantizer):
+        wq = wq[0]
+    if not wq.is_enabled:
+        return 0
+    return wq.block_sizes[-1] if wq.block_sizes else 0
+
+
+def get_quantization_format(module) -> str | None:
+    """Format string of the first quantised weight found in ``module`` or its children."""
+
+    def of_layer(layer, names):
+        wq = getattr(layer, names.weight_quantizer, None)
+        iq = getattr(layer, names.input_quantizer, None)
+        if wq is None or not wq.is_enabled:
+            return QUANTIZATION_NONE
+        if isinstance(wq, SequentialQuantizer):
+            assert len(wq) == 2 and wq[0].num_bits == 4 and wq[1].num_bits == (4, 3), (
+                "Unsupported SequentialQuantizer configuration")
+            return QUANTIZATION_W4A8_AWQ
+        if wq.num_bits == 4:
+            assert wq.block_sizes and wq.block_sizes[-1] > 0, "Invalid block_sizes for INT4 quantizer"
+            return QUANTIZATION_INT4_AWQ
+        if wq.num_bits == 8:
+            return QUANTIZATION_INT8_SQ if iq is not None and iq.is_enabled else QUANTIZATION_INT8_WO
+        if wq.num_bits == (4, 3):
+            if wq.block_sizes:
+                raise NotImplementedError("FP8 block-scaled export is outside the path built here")
+            return QUANTIZATION_FP8_PC_PT if wq.axis == 0 else QUANTIZATION_FP8
+        if wq.num_bits == (2, 1):
+            if iq is not None and hasattr(iq, "_pre_quant_scale"):
+                return QUANTIZATION_NVFP4_AWQ
+            if wq.block_sizes.get("scale_bits") == (4, 3):
+                return QUANTIZATION_NVFP4
+        raise NotImplementedError(f"Unsupported quantizer with num_bits: {wq.num_bits}")
+
+    for weight_name in weight_attr_names(module):
+        fmt = of_layer(module, quantizer_attr_names(weight_name))
+        if fmt != QUANTIZATION_NONE:
+            return fmt
+    for _, child in module.named_children():
+        fmt = get_quantization_format(child)
+        if fmt != QUANTIZATION_NONE:
+            return fmt
+    return QUANTIZATION_NONE
+
+
+def _summarize_exclude_modules(unquantized, quantized):
+    """Shortest dot-boundary prefix wildcards that cover every unquantised layer and no quantised
+    one (``a.b.c`` -> ``a*`` if nothing quantised starts with ``a``, else ``{a.b, a.b.*}`` ...)."""
+    quantized = list(quantized)
+
+    def hits_quantized(pattern):
+        return any(fnmatch.fnmatchcase(q, pattern) for q in quantized)
+
+    result: set[str] = set()
+    for layer in unquantized:
+        chosen = [layer]
+        for i, ch in enumerate(layer):
+            if ch != ".":
+                continue
+            single = [layer[:i] + "*"]
+            pair = [layer[:i], layer[:i] + ".*"]
+            done = False
+            for cand in (single, pair):
+                if any(hits_quantized(p) for p in cand):
+                    continue
+                chosen, done = cand, True
+                break
+            if done:
+                break
+        if all(c in result for c in chosen):
+            continue
+        result.update(chosen)
+    return result
+
+
+_LAYER_CONFIGS = {
+    "fp8": lambda b: {"quant_algo": "FP8"},
+    "fp8_pc_pt": lambda b: {"quant_algo": "FP8_PER_CHANNEL_PER_TOKEN"},
+    "int4_awq": lambda b: {"quant_algo": "W4A16_AWQ", "group_size": b, "has_zero_point": False,
+                           "pre_quant_scale": True},
+    "w4a8_awq": lambda b: {"quant_algo": "W4A8_AWQ", "group_size": b, "has_zero_point": False,
+                           "pre_quant_scale": True},
+    "int8_wo": lambda b: {"quant_algo": "W8A16"},
+    "int8_sq": lambda b: {"quant_algo": "W8A8_SQ_PER_CHANNEL"},
+    "nvfp4": lambda b: {"quant_algo": "NVFP4", "group_size": b},
+    "nvfp4_awq": lambda b: {"quant_algo": "NVFP4_AWQ", "group_size": b, "has_zero_point": False,
+                            "pre_quant_scale": True},
+}
+
+
+def process_layer_quant_config(layer_config_dict):
+    """Per-layer ``{name.quantization, name.awq_block_size}`` entries -> the ``quantization``
+    section of ``hf_quant_config.json``."""
+    out: dict[str, Any] = {"quant_algo": None, "kv_cache_quant_algo": None, "quantized_layers": {}}
+    formats, last, excluded = set(), None, []
+    for key, fmt in layer_config_dict.items():
+        if "awq_block_size" in key:
+            continue
+        prefix = ".".join(key.rsplit(".", 1)[:-1])
+        block = layer_config_dict.get(prefix + ".awq_block_size", 0)
+        cfg = _LAYER_CONFIGS[fmt](block) if fmt in _LAYER_CONFIGS else {"quant_algo": fmt}
+        if cfg["quant_algo"] != QUANTIZATION_NONE:
+            formats.add(str(cfg))
+            last = cfg
+            out["quantized_layers"][prefix] = cfg
+        else:
+            excluded.append(prefix)
+    if len(formats) > 1:
+        out["quant_algo"] = "MIXED_PRECISION"
+    elif len(formats) == 1 and last is not None:
+        out.update(last)
+        out["exclude_modules"] = sorted(_summarize_exclude_modules(excluded, out["quantized_layers"].keys()))
+        out.pop("quantized_layers")
+    return out
+
+
+def pack_int4_in_uint8(weight, weights_scaling_factor):
+    """INT4-AWQ export pack: two's-complement nibbles, adjacent output rows share a byte;
+    ``[.., N, K]`` -> uint8 ``[.., N / 2, K]``."""
+    out_dim = weight.shape[-2]
+    assert out_dim % 2 == 0, f"Cannot pack weight. Out dimension {out_dim} is not an even number."
+    return _hip.int4_pack_rows(weight.contiguous(),
+                               weights_scaling_factor.to(torch.float32).contiguous())
+
+
+def to_quantized_weight(weight, weights_scaling_factor, quantization: str,
+                        weights_scaling_factor2=None, block_size=None):
+    """Weight -> packed / cast storage for ``quantization``."""
+    if weights_scaling_factor is not None:
+        weights_scaling_factor = weights_scaling_factor.to(weight.device)
+    if weights_scaling_factor2 is not None:
+        weights_scaling_factor2 = weights_scaling_factor2.to(weight.device)
+    if isinstance(weight, QTensorWrapper):
+        return weight.data
+    w = weight.contiguous()
+    if quantization == QUANTIZATION_FP8:
+        if weight.dtype == torch.float8_e4m3fn:
+            return weight
+        s = weights_scaling_factor
+        if weight.dim() == 3:
+            s = s.unsqueeze(-1)
+        via = torch.result_type(w, s)  # 0-dim fp32 scale: the quotient is a tensor of w.dtype
+        if s.numel() == 1:
+            return _hip.real_quantize(w, s.reshape(1).contiguous(), 1, 1, w.numel(), via,
+                                      _hip.MO_FMT_E4M3)
+        return _hip.real_quantize(w, s.reshape(-1).contiguous(), 1, w.shape[0],
+                                  w.numel() // w.shape[0], via, _hip.MO_FMT_E4M3)
+    if quantization in (QUANTIZATION_INT8_SQ, QUANTIZATION_INT8_WO):
+        s = weights_scaling_factor.reshape(-1).contiguous()
+        return _hip.real_quantize(w, s, 1, w.shape[0], w.shape[1], torch.result_type(w, s[:, None]),
+                                  _hip.MO_FMT_INT8)
+    if quantization == QUANTIZATION_FP8_PC_PT:
+        s = weights_scaling_factor.reshape(-1).contiguous()
+        return _hip.real_quantize(w, s, 1, w.shape[0], w.shape[1], torch.result_type(w, s[:, None]),
+                                  _hip.MO_FMT_E4M3)
+    if quantization in (QUANTIZATION_INT4_AWQ, QUANTIZATION_W4A8_AWQ):
+        return pack_int4_in_uint8(weight, weights_scaling_factor)
+    if quantization in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
+        assert block_size is not None, "Block size not passed. Unable to quantize to NVFP4 format."
+        assert weights_scaling_factor2 is not None, (
+            "Weights scaling factor 2 not passed. Unable to quantize to NVFP4 format")
+        return NVFP4QTensor.quantize(weight, block_size, weights_scaling_factor,
+                                     weights_scaling_factor2)[0]._quantized_data
+    raise NotImplementedError(f"quantization format {quantization} not supported")
+
+
+def postprocess_state_dict(state_dict: dict, maxbound: float, quantization: str | None) -> dict:
+    """Drop quantizer internals, rename KV amax to ``k_proj.k_scale`` / ``v_proj.v_scale``
+    (``amax / maxbound``, at least 1 for FP8) and input ``_pre_quant_scale`` to
+    ``pre_quant_scale``."""
+    replacements = {
+        "k_bmm_quantizer._amax": "k_proj.k_scale",
+        "v_bmm_quantizer._amax": "v_proj.v_scale",
+        "input_quantizer._pre_quant_scale": "pre_quant_scale",
+    }
+    skip_keys = ["output_quantizer", "_amax", "_bias_value", "input_quantizer._pre_quant_scale"]
+    out = {}
+    for key, value in state_dict.items():
+        if all(s not in key for s in skip_keys):
+            out[key] = value
+            continue
+        for old, new in replacements.items():
+            if key.endswith(old):
+                prefix = key[: -len(old)]
+                if "_amax" in key:
+                    assert quantization in (KV_CACHE_FP8, KV_CACHE_NVFP4), "Invalid KV cache quantization format."
+                    assert maxbound > 0, "Maxbound must be greater than zero."
+                    value = true_divide(value.float(), maxbound)
+                    if quantization == KV_CACHE_FP8:
+                        value.clamp_(min=1.0)
+                out[prefix + new] = value
+                break
+    for key, value in out.items():
+        if "scale" in key and isinstance(value, torch.Tensor) and value.dim() == 3 and value.shape[0] == 1:
+            out[key] = value.squeeze(0)
+    drop = [k for k in out if any(k.endswith("weight_quantizer." + q)
+                                  for q in ("_scale", "_double_scale", "_scale_zeros"))]
+    seen = {}
+    for key, value in out.items():
+        if isinstance(value, torch.Tensor) and value.numel() > 0:
+            ptr = value.data_ptr()
+            if ptr in seen:
+                drop.append(key)  # tied weight: keep the first name only
+            else:
+                seen[ptr] = key
+    for key in drop:
+        out.pop(key, None)
+    return out
+
+
+def all_items_same(items):
+    return all(x == items[0] for x in items)
+
+
+def _update_pre_quant_scale(module, new_pre_quant_scale):
+    """Re-smooth one linear to a new input scale: ``W <- dtype(f32(W) * old / new)`` (fp32), then
+    recalibrate the weight amax (reference: export/quant_utils.py:991-1008)."""
+    from ..quantization.model_calib import enable_stats_collection, finish_stats_collection
+
+    old = module.input_quantizer._pre_quant_scale
+    dtype, dev = module.weight.dtype, module.weight.device
+    ratio_num = old.to(dtype=torch.float32, device=dev)
+    ratio_den = new_pre_quant_scale.to(dtype=torch.float32, device=dev)
+    module.weight = nn.Parameter((module.weight.to(torch.float32) * ratio_num / ratio_den).to(dtype),
+                                 requires_grad=False)
+    module.input_quantizer.pre_quant_scale = new_pre_quant_scale
+    module.weight_quantizer.reset_amax()
+    enable_stats_collection(module.weight_quantizer)
+    module.weight_quantizer(module.weight)
+    finish_stats_collection(module.weight_quantizer)
+
+
+def preprocess_linear_fusion(modules: list[nn.Module], resmooth_only=False):
+    """Give linears that an engine will fuse (q/k/v, gate/up) one shared input amax and one
+    shared per-tensor weight amax."""
+    assert all_items_same([get_quantization_format(m) for m in modules]), (
+        "Modules have different quantization formats")
+    first = modules[0]
+    if hasattr(first, "input_quantizer"):
+        if first.input_quantizer.pre_quant_scale is not None:
+            avg = torch.mean(torch.stack([m.input_quantizer.pre_quant_scale for m in modules]), dim=0)
+            for m in modules:
+                if not torch.equal(m.input_quantizer.pre_quant_scale, avg):
+                    _update_pre_quant_scale(m, avg)
+        if resmooth_only:
+            return
+        if first.input_quantizer.is_enabled and first.input_quantizer.amax is not None:
+            assert first.input_quantizer.amax.numel() == 1, "Only support scalar input quant amax"
+            amax = torch.max(torch.stack([m.input_quantizer.amax for m in modules]))
+            for m in modules:
+                m.input_quantizer.amax = amax
+    if hasattr(first, "weight_quantizer") and not isinstance(first.weight_quantizer, SequentialQuantizer):
+        wq = first.weight_quantizer
+        if wq.is_enabled and wq.amax is not None and wq.amax.numel() == 1:
+            amax = torch.max(torch.stack([m.weight_quantizer.amax for m in modules]))
+            for m in modules:
+                m.weight_quantizer.amax = amax
+
+
+def get_quant_config(model: nn.Module) -> dict[str, Any]:
+    """The ``hf_quant_config.json`` dictionary of a quantised model."""
+    config: dict[str, Any] = {"producer": {"name": "modelopt", "version": __version__},
+                              "quantization": {"quant_algo": None, "kv_cache_quant_algo": None}}
+    layers = {}
+    kv_format = QUANTIZATION_NONE
+    off = SimpleNamespace(is_enabled=False)
+    for name, module in dict(model.named_modules()).items():
+        names = list(weight_attr_names(module))
+        if any(hasattr(module, quantizer_attr_names(w).weight_quantizer) for w in names):
+            layers[name + ".quantization"] = get_quantization_format(module)
+            layers[name + ".awq_block_size"] = get_weight_block_size(module)
+        if (getattr(module, "k_bmm_quantizer", off).is_enabled
+                or getattr(module, "v_bmm_quantizer", off).is_enabled):
+            fmt = get_kv_cache_dtype(module)
+            assert kv_format in (QUANTIZATION_NONE, fmt), "Do not support mixed precision kv cache quantization"
+            kv_format = fmt
+    config["quantization"].update(process_layer_quant_config(layers))
+    if kv_format is not None:
+        config["quantization"]["kv_cache_quant_algo"] = kv_format
+    return config

@@ -1,0 +1,172 @@
+"""Unified HF-layout export: packed weights + scales in safetensors, ``hf_quant_config.json``
+and ``config.json["quantization_config"]``.
+
+Reference: modelopt/torch/export/unified_export_hf.py:233-391 (``_export_quantized_weight``),
+:394-553 (``_export_hf_checkpoint``), :556-620 (``export_hf_checkpoint``).  NVFP4 linears are
+packed in ONE multi-tensor kernel launch over the whole model instead of module by module.
+"""
+
+import json
+import os
+import warnings
+from pathlib import Path
+from typing import Any
+
+import torch
+from torch import nn
+
+from ... import _hip
+from ..quantization.nn import SequentialQuantizer, TensorQuantizer
+from ..quantization.qtensor import NVFP4QTensor
+from ..quantization.utils import is_quantized_linear, true_divide
+from .model_config import *  # noqa: F403
+from .quant_utils import (get_activation_scaling_factor, get_quant_config, get_quantization_format,
+                          get_weight_block_size, get_weight_scaling_factor,
+                          get_weight_scaling_factor_2, postprocess_state_dict,
+                          preprocess_linear_fusion, to_quantized_weight)
+
+__all__ = ["export_hf_checkpoint", "convert_hf_quant_config_format"]
+
+
+def _register_input_scale(module, input_quantizer):
+    if (input_quantizer is not None and "disabled" not in repr(input_quantizer)
+            and input_quantizer.amax is not None):
+        module.register_buffer("input_scale", get_activation_scaling_factor(module).squeeze())
+
+
+def _export_quantized_weight(module: nn.Module, dtype: torch.dtype):
+    """Replace ``module.weight`` by its packed form and register ``weight_scale``,
+    ``weight_scale_2`` and ``input_scale`` buffers."""
+    fmt = get_quantization_format(module)
+    if fmt == QUANTIZATION_NONE:
+        return
+    block = get_weight_block_size(module)
+    wq, iq = module.weight_quantizer, getattr(module, "input_quantizer", None)
+    weight = module.weight
+    if fmt == QUANTIZATION_FP8:
+        wq._amax = wq._amax.to(torch.float32)
+        if wq._amax.dim() == 1:
+            wsf = torch.tensor(wq.amax.item() / wq.maxbound)
+        else:
+            wsf = true_divide(wq.amax, wq.maxbound).clone().detach()
+        module.register_buffer("weight_scale", wsf)
+        if iq is not None and hasattr(iq, "_amax"):
+            iq._amax = iq._amax.to(torch.float32)
+            module.register_buffer("input_scale", get_activation_scaling_factor(module).squeeze())
+    else:
+        if fmt not in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
+            module.register_buffer("weight_scale", get_weight_scaling_factor(module))
+        _register_input_scale(module, iq)
+    if fmt in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ, QUANTIZATION_W4A8_AWQ):
+        module.register_buffer("weight_scale_2", get_weight_scaling_factor_2(module).squeeze())
+
+    weight_scale = getattr(module, "weight_scale", None)
+    weight_scale_2 = getattr(module, "weight_scale_2", None)
+    if fmt in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
+        # block scales and codes from one pass over the weight
+        qt, weight_scale, _ = NVFP4QTensor.quantize(weight.data.to(dtype), block,
+                                                    weights_scaling_factor_2=weight_scale_2)
+        quantized = qt._quantized_data
+    else:
+        quantized = to_quantized_weight(weight.data.to(dtype), weight_scale, fmt, weight_scale_2, block)
+    module.weight = nn.Parameter(quantized, requires_grad=False)
+    if weight_scale is not None:
+        module.register_buffer("weight_scale", weight_scale)
+
+
+def _export_nvfp4_batched(modules: list[nn.Module], dtype: torch.dtype):
+    """All NVFP4 linears of the model in one launch (bf16 weights, K % 16 == 0)."""
+    weights = [m.weight.data for m in modules]
+    amax = torch.stack([m.weight_quantizer._amax.reshape(()).float() for m in modules]).to(
+        weights[0].device)
+    plan = _hip.Nvfp4QuantizePlan(weights, amax)  # the kernel derives wsf2 = amax / (6 * 448)
+    packed, wsf, wsf2 = plan.run()
+    for i, m in enumerate(modules):
+        _register_input_scale(m, getattr(m, "input_quantizer", None))
+        m.register_buffer("weight_scale_2", wsf2[i].clone())
+        m.weight = nn.Parameter(packed[i], requires_grad=False)
+        m.register_buffer("weight_scale", wsf[i])
+
+
+def _fusable_groups(model: nn.Module):
+    """(q, k, v) and (gate, up) projections that share an input."""
+    for module in model.modules():
+        for names in (("q_proj", "k_proj", "v_proj"), ("gate_proj", "up_proj")):
+            group = [getattr(module, n, None) for n in names]
+            if all(g is not None and is_quantized_linear(g) for g in group):
+                yield group
+
+
+def _export_hf_checkpoint(model: nn.Module, dtype: torch.dtype | None = None):
+    if dtype is None:
+        dtype = next(model.parameters()).dtype
+    for group in _fusable_groups(model):
+        if get_quantization_format(group[0]) != QUANTIZATION_NONE:
+            preprocess_linear_fusion(group)
+    quant_config = get_quant_config(model)
+    kv_format = quant_config["quantization"]["kv_cache_quant_algo"]
+    kv_bound = {KV_CACHE_NVFP4: 6 * 448, KV_CACHE_FP8: 448}.get(kv_format, 0)
+
+    linears = [m for m in model.modules()
+               if is_quantized_linear(m) and get_quantization_format(m) != QUANTIZATION_NONE]
+    batched = [m for m in linears
+               if get_quantization_format(m) == QUANTIZATION_NVFP4 and m.weight.dtype == torch.bfloat16
+               and dtype == torch.bfloat16 and m.weight.shape[-1] % 16 == 0 and m.weight.is_cuda
+               and get_weight_block_size(m) == 16 and m.weight.is_contiguous()]
+    if batched:
+        _export_nvfp4_batched(batched, dtype)
+    done = set(map(id, batched))
+    for m in linears:
+        if id(m) not in done:
+            _export_quantized_weight(m, dtype)
+    state = postprocess_state_dict(model.state_dict(), kv_bound, kv_format)
+    return state, quant_config
+
+
+def convert_hf_quant_config_format(input_config: dict[str, Any]) -> dict[str, Any]:
+    """``hf_quant_config.json`` -> the ``quantization_config`` block written into config.json
+    (reference: export/convert_hf_config.py:21-130)."""
+    q = input_config.get("quantization", {})
+    algo = q.get("quant_algo")
+    out: dict[str, Any] = {}
+    group = None
+    if algo == "FP8":
+        group = {"input_activations": {"dynamic": False, "num_bits": 8, "type": "float"},
+                 "weights": {"dynamic": False, "num_bits": 8, "type": "float"}, "targets": ["Linear"]}
+    elif algo == "NVFP4":
+        gs = q.get("group_size")
+        group = {"input_activations": {"dynamic": False, "num_bits": 4, "type": "float", "group_size": gs},
+                 "weights": {"dynamic": False, "num_bits": 4, "type": "float", "group_size": gs},
+                 "targets": ["Linear"]}
+    if group is not None:
+        out["config_groups"] = {"group_0": group}
+    out["ignore"] = q.get("exclude_modules", [])
+    out["quant_algo"] = algo
+    if q.get("kv_cache_quant_algo"):
+        out["kv_cache_scheme"] = {"dynamic": False, "num_bits": 8, "type": "float"} if q[
+            "kv_cache_quant_algo"] == "FP8" else q["kv_cache_quant_algo"]
+    out["producer"] = input_config.get("producer", {})
+    out["quant_method"] = "modelopt"
+    return out
+
+
+def export_hf_checkpoint(model: nn.Module, dtype: torch.dtype | None = None,
+                         export_dir: Path | str = "/tmp", save_modelopt_state: bool = False):
+    """Write ``model.safetensors``, ``hf_quant_config.json`` and ``config.json`` to
+    ``export_dir``.  ``model.config`` (a dict or an object with ``to_dict``) is used for
+    ``config.json`` when present."""
+    from safetensors.torch import save_file
+
+    export_dir = Path(export_dir)
+    export_dir.mkdir(parents=True, exist_ok=True)
+    state, hf_quant_config = _export_hf_checkpoint(model, dtype)
+    with open(export_dir / "hf_quant_config.json", "w") as f:
+        json.dump(hf_quant_config, f, indent=4)
+    tensors = {k: v.detach().contiguous().cpu() for k, v in state.items() if isinstance(v, torch.Tensor)}
+    save_file(tensors, str(export_dir / "model.safetensors"))
+    cfg = getattr(model, "config", {})
+    cfg = cfg.to_dict() if hasattr(cfg, "to_dict") else dict(cfg) if isinstance(cfg, dict) else {}
+    cfg["quantization_config"] = convert_hf_quant_config_format(hf_quant_config)
+    with open(export_dir / "config.json", "w") as f:
+        json.dump(cfg, f, indent=4, default=str)
+    return state, hf_quant_config

@@ -171,7 +171,7 @@ class TensorQuantizer(nn.Module):
             warnings.warn("step_size is undefined under dynamic amax mode!")
             return None
         assert isinstance(self._num_bits, int), "Step size is not defined for non-integer quantization."
-        return self._amax / (2.0 ** (self._num_bits - 1 + int(self._unsigned)) - 1.0)
+        return quant_utils.true_divide(self._amax, 2.0 ** (self._num_bits - 1 + int(self._unsigned)) - 1.0)
 
     @property
     def axis(self):
@@ -319,7 +319,7 @@ class TensorQuantizer(nn.Module):
         if self._num_bits == (4, 3):
             use_amax = self.amax is not None and not (bs and self.amax.numel() == 1)
             outputs, scale = FP8QTensor.quantize(inputs, axis=self._axis, block_sizes=bs,
-                                                 scales=self.amax / 448.0 if use_amax else None)
+                                                 scales=quant_utils.true_divide(self.amax, 448.0) if use_amax else None)
             buffers["_scale"] = scale
         elif self._num_bits == 8:
             outputs, scale = INT8QTensor.quantize(inputs, axis=self._axis, block_sizes=bs)
@@ -331,7 +331,8 @@ class TensorQuantizer(nn.Module):
         elif bs.get("scale_bits") == (4, 3):
             if self.amax is not None and self._amax.device != inputs.device:
                 self._amax = self._amax.to(inputs.device)
-            wsf2 = self.amax.float() / (448.0 * 6.0) if self.amax is not None else None
+            wsf2 = (quant_utils.true_divide(self.amax.float(), 448.0 * 6.0)
+                    if self.amax is not None else None)
             outputs, wsf, wsf2 = NVFP4QTensor.quantize(inputs, bs[-1], weights_scaling_factor_2=wsf2)
             buffers["_scale"], buffers["_double_scale"] = wsf, wsf2
         else:

@@ -4,7 +4,8 @@ import torch
 
 from .... import _hip
 from .. import kernels
-from ..utils import convert_quantization_axis_to_reduce_axis, reduce_amax, reduce_block_amax
+from ..utils import (convert_quantization_axis_to_reduce_axis, reduce_amax, reduce_block_amax,
+                     true_divide)
 from .base_qtensor import BaseQuantizedTensor
 from .fp8_tensor import _block_layout
 
@@ -22,7 +23,7 @@ class INT8QTensor(BaseQuantizedTensor):
                 amax = reduce_block_amax(x, block_sizes)
             else:
                 amax = reduce_amax(x, axis=convert_quantization_axis_to_reduce_axis(x, axis))
-            scales = amax / 127.0
+            scales = true_divide(amax, 127.0)
         if block_sizes:
             layout = _block_layout(x, scales, block_sizes)
         else:

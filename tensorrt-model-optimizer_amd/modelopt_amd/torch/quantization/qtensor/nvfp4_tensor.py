@@ -8,7 +8,7 @@ E2M1 ordinal); per-block scales ``float8_e4m3fn`` [..., K/block]; one fp32 globa
 import torch
 
 from .... import _hip
-from ..utils import reduce_amax, reduce_block_amax
+from ..utils import reduce_amax, reduce_block_amax, true_divide
 from .base_qtensor import BaseQuantizedTensor
 
 __all__ = ["NVFP4QTensor"]
@@ -27,11 +27,11 @@ class NVFP4QTensor(BaseQuantizedTensor):
     @classmethod
     def get_weights_scaling_factor_2_from_quantizer(cls, weight_quantizer):
         assert hasattr(weight_quantizer, "_amax"), "Weight quantizer does not have attribute amax"
-        return weight_quantizer._amax.float() / (6.0 * 448.0)
+        return true_divide(weight_quantizer._amax.float(), 6.0 * 448.0)
 
     @classmethod
     def get_weights_scaling_factor_2(cls, input: torch.Tensor):
-        return reduce_amax(input).float() / (6.0 * 448.0)
+        return true_divide(reduce_amax(input).float(), 6.0 * 448.0)
 
     @classmethod
     def get_weights_scaling_factor(cls, input, block_size, weights_scaling_factor_2=None,
@@ -59,7 +59,7 @@ class NVFP4QTensor(BaseQuantizedTensor):
         amax = quantizer.export_amax()
         if amax is None:
             return None
-        sf = amax.float() / (quantizer.maxbound * 448.0)
+        sf = true_divide(amax.float(), quantizer.maxbound * 448.0)
         assert torch.all(sf > 0), f" activation scaling factor {sf} not positive."
         return sf
 

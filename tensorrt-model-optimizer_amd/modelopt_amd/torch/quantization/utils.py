@@ -7,10 +7,21 @@ import torch.nn.functional as F
 from . import kernels
 
 __all__ = [
-    "convert_quantization_axis_to_reduce_axis", "reduce_amax", "reduce_block_amax",
+    "true_divide", "convert_quantization_axis_to_reduce_axis", "reduce_amax", "reduce_block_amax",
     "reduce_block_padding", "is_quantized", "is_quantized_linear",
     "update_quant_cfg_with_kv_cache_quant", "quantizer_attr_names", "weight_attr_names",
 ]
+
+
+def true_divide(t: torch.Tensor, divisor: float) -> torch.Tensor:
+    """``t / divisor`` as one correctly rounded division.
+
+    torch's GPU kernels evaluate ``tensor / python_scalar`` as ``tensor * (1 / scalar)`` (two
+    roundings) while the CPU kernels divide; every scale the reference derives that way
+    (``amax / 448``, ``amax / (6 * 448)``, ``amax / 7`` ...) is therefore computed here as a
+    tensor / tensor division, which is a true division on both devices.
+    """
+    return torch.div(t, torch.full((), float(divisor), dtype=t.dtype, device=t.device))
 
 
 def convert_quantization_axis_to_reduce_axis(input, axis):

@@ -347,3 +347,17 @@ def test_awq_generic_path_equals_fused_path(monkeypatch):
         results.append((model.proj.awq_lite.loss, model.proj.weight.data.clone()))
     assert results[0][0] == results[1][0]
     assert torch.equal(results[0][1], results[1][1])
+
+
+def test_true_divide_is_one_rounding_on_the_gpu():
+    """The helper behind every ``amax / constant`` scale equals the CPU's true division."""
+    from modelopt_amd.torch.quantization.utils import true_divide
+
+    g = torch.Generator().manual_seed(0)
+    t = torch.rand(200000, generator=g) * 10 + 1e-3
+    for d in (448.0, 2688.0, 7.0, 127.0):
+        want = t / d  # CPU: true division
+        got = true_divide(t.to(DEV), d).cpu()
+        assert torch.equal(got, want), d
+    tb = t[:4096].to(torch.bfloat16)
+    assert torch.equal(true_divide(tb.to(DEV), 448.0).cpu(), tb / 448.0)
