@@ -87,6 +87,58 @@ def cpu_baseline(torch, layers_sampled=1):
     }
 
 
+def calib_sweep(torch, layers, n_seqs, batch, seq_len=512):
+    """BASELINE config 5: mtq.quantize (NVFP4 weights + inputs, FP8 KV cache, max calibration) on
+    a random-init Llama-3-8B-shaped decoder over n_seqs x 512 uniform-random token ids.  Reports
+    end-to-end seconds (the reference's own stopwatch brackets mtq.quantize the same way,
+    examples/llm_ptq/hf_ptq.py:214-232), the forward-only seconds of the same data with no
+    quantizers attached, and their difference = time attributable to the quantizer kernels."""
+    import dataclasses
+
+    import modelopt_amd.torch.quantization as mtq
+    from modelopt_amd.testing.llama_decoder import LLAMA3_8B, LlamaForCausalLM
+
+    dev = torch.device("cuda:0")
+    cfg = dataclasses.replace(LLAMA3_8B, num_hidden_layers=layers)
+    model = LlamaForCausalLM(cfg, device=dev, seed=5)
+    g = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, cfg.vocab_size, (n_seqs, seq_len), generator=g).to(dev)
+
+    @torch.no_grad()
+    def forward_loop(m):
+        for i in range(0, n_seqs, batch):
+            m(ids[i:i + batch])
+
+    forward_loop(model)  # warm-up (GEMM autotuning, allocator)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    forward_loop(model)
+    torch.cuda.synchronize()
+    plain_s = time.perf_counter() - t0
+
+    qcfg = mtq.utils.update_quant_cfg_with_kv_cache_quant(mtq.NVFP4_DEFAULT_CFG,
+                                                          mtq.FP8_KV_CFG["quant_cfg"])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    mtq.quantize(model, qcfg, forward_loop)
+    torch.cuda.synchronize()
+    calib_s = time.perf_counter() - t0
+    n_q = sum(1 for m in model.modules() if isinstance(m, mtq.nn.TensorQuantizer) and m.is_enabled)
+    tokens = n_seqs * seq_len
+    act_bytes = tokens * layers * (38912 * 2 + 2 * 1024 * 2)   # inputs of 7 linears + K and V
+    w_bytes = sum(m.weight.numel() * 2 for m in model.modules()
+                  if hasattr(m, "weight_quantizer") and m.weight_quantizer.is_enabled)
+    return {
+        "end_to_end_calib_s": round(calib_s, 3),
+        "forward_only_s": round(plain_s, 3),
+        "quantizer_overhead_s": round(calib_s - plain_s, 3),
+        "enabled_quantizers": n_q,
+        "tokens": tokens,
+        "amax_bytes_read": {"activations_and_kv": act_bytes, "weights_once": w_bytes},
+        "config": f"{layers} layers, {n_seqs} seqs x {seq_len} tokens, batch {batch}, NVFP4 W+A, FP8 KV, max",
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -95,6 +147,10 @@ def main():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip amax / dequant side measurements")
+    ap.add_argument("--no-calib-sweep", action="store_true",
+                    help="skip the mtq.quantize calibration sweep on the Llama-3-8B-shaped decoder")
+    ap.add_argument("--calib-seqs", type=int, default=128)
+    ap.add_argument("--calib-batch", type=int, default=16)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device copy (a kernel of known traffic for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -196,6 +252,11 @@ def main():
         extras["dequantize_one_layer"] = {
             "ms": round(d_ms, 4), "GBps": round(e1 * DEQUANT_BYTES_PER_ELEM / d_ms / 1e6, 1)}
         out["extras"] = extras
+
+    if not a.no_calib_sweep:
+        del weights, aplan, qplan
+        torch.cuda.empty_cache()
+        out["calib_sweep"] = calib_sweep(torch, a.layers, a.calib_seqs, a.calib_batch)
 
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)

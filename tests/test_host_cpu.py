@@ -1,0 +1,295 @@
+"""Host-layer logic on CPU: configs, conversion, wildcards, block reshaping, export helpers.
+
+Orchestration tests swap the kernel facade for the CPU oracle (``oracle_backend`` fixture): the
+oracle is the stand-in for the HIP library here, exactly so that the Python control flow can be
+exercised without a GPU.  The product itself never does this -- see ``test_cpu_tensors_raise``.
+"""
+
+import copy
+
+import pytest
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+import modelopt_amd.torch.quantization as mtq
+from modelopt_amd.torch.export import quant_utils as equ
+from modelopt_amd.torch.quantization import kernels
+from modelopt_amd.torch.quantization.config import QuantizerAttributeConfig, normalize_algorithm
+from modelopt_amd.torch.quantization.nn import SequentialQuantizer, TensorQuantizer
+from oracle import fake_quant, reduce
+
+
+# ----------------------------------------------------------------------------- config
+def test_attribute_config_defaults_and_mapping_protocol():
+    c = QuantizerAttributeConfig()
+    assert c.num_bits == 8 and c.axis is None and c.fake_quant and not c.narrow_range and c.enable
+    assert dict(c.items())["calibrator"] == "max" and "block_sizes" in c
+    assert c["type"] == "static"
+
+
+@pytest.mark.parametrize("bad", [
+    {"enable": True},
+    {"num_bits": 0},
+    {"num_bits": (7, 7)},
+    {"num_bits": (2, 1)},                                    # FP4 needs dynamic block sizes
+    {"num_bits": 8, "axis": 0, "block_sizes": {-1: 128}},     # axis and block_sizes exclude each other
+    {"block_sizes": {-1: 16, -2: 16, "type": "dynamic"}},    # dynamic = last axis only
+    {"block_sizes": {"bogus": 1}},
+    {"type": "sometimes"},
+    {"bias": {"type": "static"}},
+])
+def test_attribute_config_rejects(bad):
+    with pytest.raises(Exception):
+        QuantizerAttributeConfig(**bad)
+
+
+def test_named_configs_validate():
+    for name in mtq.config.choices:
+        quant_cfg, algo = mtq.model_quant._validated(getattr(mtq, name))
+        assert "default" in quant_cfg and isinstance(quant_cfg["default"], QuantizerAttributeConfig)
+    assert normalize_algorithm("max") == ("max", {"distributed_sync": True})
+    assert normalize_algorithm({"method": "awq_lite", "alpha_step": 0.05})[1]["alpha_step"] == 0.05
+    assert normalize_algorithm(None) == (None, {})
+    with pytest.raises(NotImplementedError):
+        normalize_algorithm("svdquant")
+
+
+# ----------------------------------------------------------------------------- conversion
+class _Net(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.body = nn.Sequential(nn.Linear(16, 32), nn.ReLU(), nn.Linear(32, 16))
+        self.lm_head = nn.Linear(16, 8)
+
+    def forward(self, x):
+        return self.lm_head(self.body(x))
+
+
+def _converted(cfg):
+    m = _Net()
+    mtq.replace_quant_module(m)
+    mtq.set_quantizer_by_cfg(m, mtq.model_quant._validated(cfg)[0])
+    return m
+
+
+def test_conversion_adds_quantizers_and_keeps_parameters():
+    m = _Net()
+    w = m.body[0].weight
+    mtq.replace_quant_module(m)
+    assert m.body[0].weight is w and isinstance(m.body[0], nn.Linear)
+    assert type(m.body[0]).__name__ == "QuantLinear"
+    for lin in (m.body[0], m.body[2], m.lm_head):
+        assert {"input_quantizer", "weight_quantizer", "output_quantizer"} <= dict(lin.named_children()).keys()
+        assert not lin.output_quantizer.is_enabled
+    with pytest.raises(AssertionError):
+        mtq.replace_quant_module(m)
+
+
+def test_wildcards_and_lm_head_exclusion():
+    m = _converted(mtq.INT4_AWQ_CFG)
+    assert m.body[0].weight_quantizer.num_bits == 4 and m.body[0].weight_quantizer.block_sizes[-1] == 128
+    assert not m.body[0].input_quantizer.is_enabled
+    assert not m.lm_head.weight_quantizer.is_enabled and not m.lm_head.input_quantizer.is_enabled
+    mtq.set_quantizer_attribute(m, lambda n: n.endswith("body.2.weight_quantizer"), {"num_bits": 8, "axis": 0})
+    assert m.body[2].weight_quantizer.num_bits == 8 and m.body[2].weight_quantizer.axis == 0
+    assert m.body[0].weight_quantizer.num_bits == 4
+    mtq.disable_quantizer(m, "*body.0*")
+    assert not m.body[0].weight_quantizer.is_enabled and m.body[0].weight_quantizer.num_bits == 4
+
+
+def test_list_attribute_makes_sequential_quantizer():
+    m = _converted(mtq.W4A8_AWQ_BETA_CFG)
+    wq = m.body[0].weight_quantizer
+    assert isinstance(wq, SequentialQuantizer) and len(wq) == 2
+    assert wq[0].num_bits == 4 and wq[1].num_bits == (4, 3)
+    assert wq.is_enabled and wq.fake_quant
+    with SequentialQuantizer.convert_to_single_quantizer(m):
+        assert isinstance(m.body[0].weight_quantizer, TensorQuantizer)
+    assert isinstance(m.body[0].weight_quantizer, SequentialQuantizer)
+    assert equ.get_quantization_format(m.body[0]) == "w4a8_awq"
+
+
+def test_set_quantizer_by_cfg_context_restores():
+    m = _converted(mtq.INT8_DEFAULT_CFG)
+    q = m.body[0].input_quantizer
+    with mtq.set_quantizer_by_cfg_context(m, {"*input_quantizer": {"enable": False}}):
+        assert not q.is_enabled
+    assert q.is_enabled and q.num_bits == 8
+
+
+# ----------------------------------------------------------------------------- TensorQuantizer
+def test_quantizer_properties_and_state():
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=(4, 3)))
+    assert q.maxbound == 448.0 and q.amax is None and "per-tensor" in repr(q)
+    q.amax = 2.0
+    assert q.amax.item() == 2.0
+    with pytest.raises(RuntimeError, match="shape"):
+        q.amax = [1.0, 2.0]
+    q2 = TensorQuantizer(QuantizerAttributeConfig(
+        num_bits=(2, 1), block_sizes={-1: 16, "type": "dynamic", "scale_bits": (4, 3)}))
+    assert q2.maxbound == 6.0 and not q2.is_static_block_quant and not q2.is_mx_format
+    assert TensorQuantizer(QuantizerAttributeConfig(num_bits=4, block_sizes={-1: 128})).is_static_block_quant
+    assert TensorQuantizer(QuantizerAttributeConfig(num_bits=8, unsigned=True)).maxbound == 255
+    state = q.get_modelopt_state()
+    q3 = TensorQuantizer()
+    q3.set_from_modelopt_state(state)
+    assert q3.num_bits == (4, 3) and q3._amax.shape == ()
+    q.reset_amax()
+    assert q.amax is None
+    with pytest.raises(RuntimeError, match="Calibrator returned None"):
+        q.load_calib_amax()
+
+
+def test_cpu_tensors_raise_instead_of_falling_back():
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=8))
+    with pytest.raises(RuntimeError, match="GPU memory"):
+        q(torch.randn(4, 4))
+    with pytest.raises(RuntimeError, match="GPU memory"):
+        mtq.utils.reduce_amax(torch.randn(4, 4))
+
+
+def test_layout_helpers():
+    assert kernels.amax_layout((4, 5, 6), []) == (1, 1, 120)
+    assert kernels.amax_layout((4, 5, 6), [0]) == (1, 4, 30)
+    assert kernels.amax_layout((4, 5, 6), [-1]) == (20, 6, 1)
+    assert kernels.amax_layout((4, 5, 6), [1]) == (4, 5, 6)
+    assert kernels.amax_layout((4, 5, 6), [0, 1]) == (1, 20, 6)
+    assert kernels.amax_layout((4, 5, 6), [0, 2]) is None
+    assert kernels.amax_layout((4, 1, 6), [0, 2]) == (1, 24, 1)
+    assert kernels.layout_from_amax_shape((4, 5, 6), (1, 5, 1)) == (4, 5, 6)
+    assert kernels.layout_from_amax_shape((4, 5, 6), ()) == (1, 1, 120)
+    assert kernels.layout_from_amax_shape((8, 16), (8,)) == (1, 8, 16)
+    assert kernels.layout_from_amax_shape((4, 5, 6), (4, 1, 6)) is None
+
+
+@pytest.fixture
+def oracle_backend(monkeypatch):
+    """Route the kernel facade to the CPU oracle so host control flow runs without a GPU."""
+    def accumulate(x, acc, layout):
+        outer, axis, inner = layout
+        v = x.reshape(outer, axis, inner).abs().float().amax(dim=(0, 2))
+        acc.copy_(torch.maximum(acc, v))
+        return acc
+
+    def reduce_gpu(x, dims, keepdims=True):
+        return reduce.reduce_amax(x, axis=dims, keepdims=keepdims, squeeze_scalar=False) if dims is not None \
+            else reduce.reduce_amax(x)
+
+    monkeypatch.setattr(kernels, "absmax_accumulate", accumulate)
+    monkeypatch.setattr(kernels, "reduce_amax_gpu", reduce_gpu)
+    monkeypatch.setattr(kernels, "fake_quant_int", fake_quant.tensor_quant)
+    monkeypatch.setattr(kernels, "fake_quant_fp8", lambda x, amax=None, saturate=False: fake_quant.fp8_eager(x, amax))
+    monkeypatch.setattr(kernels, "fake_quant_nvfp4",
+                        lambda x, amax, bs=16, mode=0: fake_quant.nvfp4_fake_quant(x, amax, bs))
+    monkeypatch.setattr(kernels, "mul_last_dim", lambda x, s: x * s)
+
+
+@pytest.mark.parametrize("shape,block_sizes,amax_shape,export_shape", [
+    ((6, 256), {-1: 128}, (12, 1), (6, 2)),
+    ((6, 200), {-1: 128}, (12, 1), (6, 2)),          # padded to 256
+    ((2, 3, 64), {-1: 32}, (12, 1), (2, 3, 2)),
+])
+def test_static_block_reshape_and_amax_shapes(oracle_backend, shape, block_sizes, amax_shape, export_shape):
+    """Shapes follow tests/_test_utils/torch/quantization/tensor_quantizer_common.py:346-449."""
+    x = torch.randn(*shape)
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=4, block_sizes=block_sizes))
+    q.enable_calib(); q.disable_quant()
+    y = q(x)
+    assert y.shape == x.shape and torch.equal(y, x)
+    q.load_calib_amax()
+    assert tuple(q.amax.shape) == amax_shape
+    if export_shape is not None:
+        assert tuple(q.export_amax().shape) == export_shape
+        q.enable_quant(); q.disable_calib()
+        out = q(x)
+        want = fake_quant.static_block_fake_quant(
+            x, block_sizes[-1], lambda x2, a: fake_quant.tensor_quant(x2, a, 4, False, False))
+        assert torch.equal(out, want)
+    with pytest.raises(ValueError, match="shape has changed"):
+        q(torch.randn(shape[0] + 1, *shape[1:]))
+
+
+def test_two_axis_blocks_reshape_then_refuse(oracle_backend):
+    """2-D blocks take the general reshape ([2, 4, 2, 32], amax on dims 0 and 2); scales on two
+    non-adjacent dims are not covered by the kernels and must raise, not fall back."""
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=8, block_sizes={-1: 32, -2: 4}))
+    q.enable_calib(); q.disable_quant()
+    with pytest.raises(NotImplementedError):
+        q(torch.randn(8, 64))
+    assert tuple(q._block_reshape_size) == (2, 4, 2, 32) and q.axis == (0, 2)
+
+
+def test_block_sizes_none_means_per_channel(oracle_backend):
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=8, block_sizes={-1: None}))
+    x = torch.randn(5, 7)
+    y = q(x)
+    assert q.block_sizes is None and q.axis == (0,)
+    assert torch.equal(y, fake_quant.tensor_quant(x, reduce.reduce_amax(x, axis=[1]), 8, False, False))
+
+
+def test_quantize_flow_on_cpu_with_oracle_backend(oracle_backend):
+    m = _Net()
+    data = [torch.randn(4, 16) for _ in range(3)]
+    mtq.quantize(m, mtq.INT8_DEFAULT_CFG, lambda mod: [mod(d) for d in data])
+    lin = m.body[0]
+    assert torch.equal(lin.input_quantizer.amax, torch.stack([reduce.reduce_amax(d) for d in data]).max())
+    assert torch.equal(lin.weight_quantizer.amax, reduce.reduce_amax(lin.weight.data, axis=[1]))
+    assert lin.input_quantizer._if_quant and not lin.input_quantizer._if_calib
+    x = data[0]
+    want = F.linear(fake_quant.tensor_quant(x, lin.input_quantizer.amax, 8, False, False),
+                    fake_quant.tensor_quant(lin.weight.data, lin.weight_quantizer.amax, 8, False, False), lin.bias)
+    assert torch.allclose(lin(x), want)
+    # straight-through gradient with clipping
+    x = (data[0] * 3).requires_grad_()
+    lin.input_quantizer(x).sum().backward()
+    assert torch.equal(x.grad, (x.detach().abs() <= lin.input_quantizer.amax).float())
+
+
+# ----------------------------------------------------------------------------- export helpers
+def test_postprocess_state_dict_renames_like_reference():
+    """Key handling of tests/gpu/torch/export/test_export.py:199-253."""
+    sd = {
+        "layers.0.self_attn.k_bmm_quantizer._amax": torch.tensor(896.0),
+        "layers.0.self_attn.v_bmm_quantizer._amax": torch.tensor(4.48),
+        "layers.0.self_attn.q_proj.input_quantizer._pre_quant_scale": torch.ones(4),
+        "layers.0.self_attn.q_proj.input_quantizer._amax": torch.tensor(1.0),
+        "layers.0.self_attn.q_proj.weight_quantizer._amax": torch.tensor(1.0),
+        "layers.0.self_attn.q_proj.output_quantizer._amax": torch.tensor(1.0),
+        "layers.0.self_attn.q_proj.weight": torch.zeros(2, 2),
+        "layers.0.self_attn.q_proj.weight_scale": torch.ones(1, 2, 3),
+    }
+    out = equ.postprocess_state_dict(sd, 448, "FP8")
+    assert set(out) == {"layers.0.self_attn.k_proj.k_scale", "layers.0.self_attn.v_proj.v_scale",
+                        "layers.0.self_attn.q_proj.pre_quant_scale", "layers.0.self_attn.q_proj.weight",
+                        "layers.0.self_attn.q_proj.weight_scale"}
+    assert out["layers.0.self_attn.k_proj.k_scale"].item() == 2.0
+    assert out["layers.0.self_attn.v_proj.v_scale"].item() == 1.0       # clamped to at least 1
+    assert out["layers.0.self_attn.q_proj.weight_scale"].shape == (2, 3)  # leading 1 squeezed
+
+
+def test_hf_quant_config_sections():
+    layers = {"model.layers.0.q_proj.quantization": "nvfp4", "model.layers.0.q_proj.awq_block_size": 16,
+              "lm_head.quantization": None, "lm_head.awq_block_size": 0}
+    out = equ.process_layer_quant_config(layers)
+    assert out == {"quant_algo": "NVFP4", "kv_cache_quant_algo": None, "group_size": 16,
+                   "exclude_modules": ["lm_head"]}
+    layers["model.layers.0.k_proj.quantization"] = "fp8"
+    layers["model.layers.0.k_proj.awq_block_size"] = 0
+    out = equ.process_layer_quant_config(layers)
+    assert out["quant_algo"] == "MIXED_PRECISION" and set(out["quantized_layers"]) == {
+        "model.layers.0.q_proj", "model.layers.0.k_proj"}
+    awq = equ.process_layer_quant_config({"a.b.quantization": "int4_awq", "a.b.awq_block_size": 128})
+    assert awq["quant_algo"] == "W4A16_AWQ" and awq["group_size"] == 128 and awq["pre_quant_scale"] is True
+
+
+def test_quantization_format_detection():
+    for cfg, fmt in [(mtq.INT8_DEFAULT_CFG, "int8_sq"), (mtq.INT8_WEIGHT_ONLY_CFG, "int8_wo"),
+                     (mtq.FP8_DEFAULT_CFG, "fp8"), (mtq.INT4_AWQ_CFG, "int4_awq"),
+                     (mtq.NVFP4_DEFAULT_CFG, "nvfp4")]:
+        m = _converted(cfg)
+        assert equ.get_quantization_format(m.body[0]) == fmt
+        assert equ.get_quantization_format(m.lm_head) is None
+        assert equ.get_quantization_format(m) == fmt
+    m = _converted(mtq.NVFP4_DEFAULT_CFG)
+    assert equ.get_weight_block_size(m.body[0]) == 16 and equ.get_weight_block_size(m.lm_head) == 0
