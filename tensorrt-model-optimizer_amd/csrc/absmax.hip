@@ -42,25 +42,36 @@ template <int DT> struct AbsAcc {
     }
 };
 
+// Fold v into the running maximum.  The accumulator only ever grows, so a plain (possibly stale)
+// read that already shows a value >= v proves the atomic is unnecessary; thousands of
+// workgroups hitting one address then cost a handful of atomics instead of one each.
+__device__ __forceinline__ void fold_max(uint32_t* acc, uint32_t v) {
+    if (v && v > __builtin_nontemporal_load(acc)) atomicMax(acc, v);
+}
+
 // ------------------------------------------------------------------------------ per tensor
+// One workgroup per tile of MO_ABSMAX_TILE_ELEMS elements, dispatched in order.
 template <int DT>
 __global__ __launch_bounds__(256) void absmax_flat_kernel(const void* __restrict__ x, int64_t n,
                                                           uint32_t* __restrict__ acc) {
     __shared__ uint32_t smem[4];
+    constexpr int64_t kTileChunks = MO_ABSMAX_TILE_ELEMS / 8;
     AbsAcc<DT> a;
     const int64_t chunks = n >> 3;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    for (; c + 3 * stride < chunks; c += 4 * stride) {
+    const int64_t c0 = (int64_t)blockIdx.x * kTileChunks;
+    int64_t c1 = c0 + kTileChunks;
+    if (c1 > chunks) c1 = chunks;
+    int64_t c = c0 + threadIdx.x;
+    for (; c + 768 < c1; c += 1024) {
         a.chunk(x, c << 3);
-        a.chunk(x, (c + stride) << 3);
-        a.chunk(x, (c + 2 * stride) << 3);
-        a.chunk(x, (c + 3 * stride) << 3);
+        a.chunk(x, (c + 256) << 3);
+        a.chunk(x, (c + 512) << 3);
+        a.chunk(x, (c + 768) << 3);
     }
-    for (; c < chunks; c += stride) a.chunk(x, c << 3);
-    if (blockIdx.x == 0 && threadIdx.x < (n & 7)) a.elem(x, (chunks << 3) + threadIdx.x);
-    uint32_t v = block_max_u32(a.bits(), smem);
-    if (threadIdx.x == 0 && v) atomicMax(acc, v);
+    for (; c < c1; c += 256) a.chunk(x, c << 3);
+    if (c1 == chunks && threadIdx.x < (n & 7)) a.elem(x, (chunks << 3) + threadIdx.x);
+    const uint32_t v = block_max_u32(a.bits(), smem);
+    if (threadIdx.x == 0) fold_max(acc, v);
 }
 
 // ------------------------------------------------------------------------------ rows
@@ -97,29 +108,29 @@ __global__ __launch_bounds__(256) void absmax_rows_kernel(const void* __restrict
             uint32_t t = (uint32_t)__shfl_xor((int)v, o, kWave);
             v = t > v ? t : v;
         }
-        if (sub == 0 && v) atomicMax(acc + (r % axis), v);
+        if (sub == 0) fold_max(acc + (r % axis), v);
     }
 }
 
 // ------------------------------------------------------------------------------ columns
-// x viewed as [outer, axis] (inner == 1); a thread owns VEC adjacent columns over a slab of
-// rows (gridDim.y slabs) and ends with VEC atomics.
-template <int DT, int VEC>
-__global__ __launch_bounds__(256) void absmax_cols_kernel(const void* __restrict__ x,
-                                                          int64_t outer, int64_t axis,
-                                                          int64_t slab,
-                                                          uint32_t* __restrict__ acc) {
-    const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
-    if (col >= axis) return;
+// x viewed as [outer, axis] (inner == 1).  Vector path (axis % 8 == 0, aligned): a lane owns 8
+// adjacent columns, a wavefront 512; the four wavefronts of a workgroup take interleaved rows of
+// a slab, combine through LDS and fold once per column.  Scalar path: one column per lane.
+template <int DT>
+__global__ __launch_bounds__(256) void absmax_cols8_kernel(const void* __restrict__ x,
+                                                           int64_t outer, int64_t axis,
+                                                           int64_t slab,
+                                                           uint32_t* __restrict__ acc) {
+    __shared__ uint32_t smem[4][512];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t col = ((int64_t)blockIdx.x * 64 + lane) * 8;
     const int64_t r0 = (int64_t)blockIdx.y * slab;
     int64_t r1 = r0 + slab;
     if (r1 > outer) r1 = outer;
-    uint32_t m[VEC];
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) m[j] = 0;
-    if constexpr (VEC == 8) {
+    uint32_t m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (col < axis) {
         if constexpr (DT == MO_F32) {
-            for (int64_t r = r0; r < r1; ++r) {
+            for (int64_t r = r0 + wave; r < r1; r += 4) {
                 const u32x4* q = (const u32x4*)((const float*)x + r * axis + col);
                 u32x4 a = __builtin_nontemporal_load(q), b = __builtin_nontemporal_load(q + 1);
                 uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
@@ -128,13 +139,13 @@ __global__ __launch_bounds__(256) void absmax_cols_kernel(const void* __restrict
             }
         } else {
             uint32_t p[4] = {0, 0, 0, 0};  // packed pairs of columns
-            int64_t r = r0;
-            for (; r + 3 < r1; r += 4) {
+            int64_t r = r0 + wave;
+            for (; r + 12 < r1; r += 16) {
                 u32x4 a[4];
 #pragma unroll
                 for (int u = 0; u < 4; ++u)
                     a[u] = __builtin_nontemporal_load(
-                        (const u32x4*)((const uint16_t*)x + (r + u) * axis + col));
+                        (const u32x4*)((const uint16_t*)x + (r + 4 * u) * axis + col));
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     p[0] = pk_max_u16(p[0], a[u].x & 0x7FFF7FFFu);
@@ -143,7 +154,7 @@ __global__ __launch_bounds__(256) void absmax_cols_kernel(const void* __restrict
                     p[3] = pk_max_u16(p[3], a[u].w & 0x7FFF7FFFu);
                 }
             }
-            for (; r < r1; ++r) {
+            for (; r < r1; r += 4) {
                 u32x4 a = __builtin_nontemporal_load(
                     (const u32x4*)((const uint16_t*)x + r * axis + col));
                 p[0] = pk_max_u16(p[0], a.x & 0x7FFF7FFFu);
@@ -158,14 +169,35 @@ __global__ __launch_bounds__(256) void absmax_cols_kernel(const void* __restrict
                 m[2 * j + 1] = DT == MO_BF16 ? hi << 16 : f2u(f16_bits_to_f32(hi));
             }
         }
-    } else {
-        AbsAcc<DT> a;
-        for (int64_t r = r0; r < r1; ++r) a.elem(x, r * axis + col);
-        m[0] = a.bits();
     }
 #pragma unroll
-    for (int j = 0; j < VEC; ++j)
-        if (m[j]) atomicMax(acc + col + j, m[j]);
+    for (int j = 0; j < 8; ++j) smem[wave][lane * 8 + j] = m[j];
+    __syncthreads();
+    for (int t = threadIdx.x; t < 512; t += 256) {
+        const int64_t c = (int64_t)blockIdx.x * 512 + t;
+        if (c < axis) {
+            uint32_t v = smem[0][t];
+            v = smem[1][t] > v ? smem[1][t] : v;
+            v = smem[2][t] > v ? smem[2][t] : v;
+            v = smem[3][t] > v ? smem[3][t] : v;
+            fold_max(acc + c, v);
+        }
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void absmax_cols1_kernel(const void* __restrict__ x,
+                                                           int64_t outer, int64_t axis,
+                                                           int64_t slab,
+                                                           uint32_t* __restrict__ acc) {
+    const int64_t col = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (col >= axis) return;
+    const int64_t r0 = (int64_t)blockIdx.y * slab;
+    int64_t r1 = r0 + slab;
+    if (r1 > outer) r1 = outer;
+    AbsAcc<DT> a;
+    for (int64_t r = r0; r < r1; ++r) a.elem(x, r * axis + col);
+    fold_max(acc + col, a.bits());
 }
 
 // ------------------------------------------------------------------------------ many tensors
@@ -203,7 +235,7 @@ __global__ __launch_bounds__(256) void absmax_multi_kernel(const mo_absmax_job* 
     for (; c < c1; c += 256) a.chunk(jb.x, c << 3);
     if (c1 == chunks && threadIdx.x < (jb.elems & 7)) a.elem(jb.x, (chunks << 3) + threadIdx.x);
     const uint32_t v = block_max_u32(a.bits(), smem);
-    if (threadIdx.x == 0 && v) atomicMax((uint32_t*)jb.acc, v);
+    if (threadIdx.x == 0) fold_max((uint32_t*)jb.acc, v);
 }
 
 template <int DT>
@@ -213,28 +245,27 @@ static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
     if (axis == 1) {  // per tensor
         const int64_t n = outer * inner;
         if (base_ok) {
-            int64_t blocks = ((n >> 3) + 1023) / 1024;
-            if (blocks < 1) blocks = 1;
-            if (blocks > 2048) blocks = 2048;
-            absmax_flat_kernel<DT><<<dim3((unsigned)blocks), 256, 0, s>>>(x, n, acc);
+            const int64_t tiles = (n + MO_ABSMAX_TILE_ELEMS - 1) / MO_ABSMAX_TILE_ELEMS;
+            if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+            absmax_flat_kernel<DT><<<dim3((unsigned)tiles), 256, 0, s>>>(x, n, acc);
             return MO_OK;
         }
         outer = 1; inner = n;  // unaligned base: guarded row path below
     }
     if (inner == 1) {  // per column
         const bool vec = base_ok && (axis % 8 == 0);
-        const int64_t threads = vec ? axis / 8 : axis;
-        const int64_t gx = (threads + 255) / 256;
-        // enough slabs to fill the chip, at least 16 rows each
-        int64_t gy = (2048 + gx - 1) / gx;
+        const int64_t gx = vec ? (axis + 511) / 512 : (axis + 255) / 256;
+        // enough row slabs to fill the chip, each at least 16 rows (a multiple of 4)
+        int64_t gy = (4096 + gx - 1) / gx;
         int64_t slab = (outer + gy - 1) / gy;
         if (slab < 16) slab = 16;
+        slab = (slab + 3) / 4 * 4;
         gy = (outer + slab - 1) / slab;
-        if (gy > 65535) { gy = 65535; slab = (outer + gy - 1) / gy; }
+        if (gy > 65535) { gy = 65535; slab = ((outer + gy - 1) / gy + 3) / 4 * 4; gy = (outer + slab - 1) / slab; }
         if (vec)
-            absmax_cols_kernel<DT, 8><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
+            absmax_cols8_kernel<DT><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
         else
-            absmax_cols_kernel<DT, 1><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
+            absmax_cols1_kernel<DT><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
         return MO_OK;
     }
     // rows of length `inner`

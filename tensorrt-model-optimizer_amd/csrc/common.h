@@ -31,12 +31,27 @@ __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return u2f(h << 16); }
 
-// fp32 -> bf16 bits, round to nearest even; NaN -> quiet NaN keeping the sign.
+// fp32 -> bf16 bits, round to nearest even (v_cvt_pk_bf16_f32 on gfx950); NaN stays NaN.
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-    uint32_t u = f2u(f);
-    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return ((u >> 16) & 0x8000u) | 0x7FC0u;
-    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+    __bf16 h = (__bf16)f;
+    uint16_t b;
+    __builtin_memcpy(&b, &h, 2);
+    return b;
 }
+
+// two fp32 -> packed bf16 pair (lo in bits 0..15)
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    f32x2 v = {lo, hi};
+    bf16x2 h = __builtin_convertvector(v, bf16x2);
+    uint32_t b;
+    __builtin_memcpy(&b, &h, 4);
+    return b;
+}
+
+// fp32 rounded to the nearest bf16 / fp16 value, as fp32
+__device__ __forceinline__ float round_to_bf16(float f) { return u2f(f32_to_bf16_bits(f) << 16); }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
     _Float16 v;
@@ -111,7 +126,7 @@ __device__ __forceinline__ void store_chunk(void* p, int64_t i, const float (&v)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             if constexpr (DT == MO_BF16)
-                r[j] = f32_to_bf16_bits(v[2 * j]) | (f32_to_bf16_bits(v[2 * j + 1]) << 16);
+                r[j] = f32x2_to_bf16x2(v[2 * j], v[2 * j + 1]);
             else
                 r[j] = f32_to_f16_bits(v[2 * j]) | (f32_to_f16_bits(v[2 * j + 1]) << 16);
         }
@@ -211,6 +226,26 @@ __device__ __forceinline__ float e2m1_to_f32(uint32_t c) {
     float mag = (m < 2u) ? 0.5f * (float)m
                          : u2f(((126u + (m >> 1)) << 23) | ((m & 1u) << 22));
     return (c & 8u) && m ? -mag : mag;
+}
+
+// ---------------------------------------------------------------- exact division by a shared divisor
+// RN(x / s) from r = RN(1 / s) (one IEEE division shared by many x) and four FMAs:
+//   q0 = RN(x * r)                        within 1.5 ulp of x / s
+//   q1 = RN(q0 + RN(x - s * q0) * r)      faithful (the residual is exact in an FMA)
+//   q  = RN(q1 + RN(x - s * q1) * r)      correctly rounded: a faithful quotient and a correctly
+//                                         rounded reciprocal need one FMA correction (Markstein)
+// Valid when nothing over- or underflows (callers check the range of s and of the quotient).
+// A zero x gives +0 for either sign of x.
+__device__ __forceinline__ float exact_quotient(float x, float s, float r) {
+    const float q0 = x * r;
+    const float q1 = __builtin_fmaf(__builtin_fmaf(-s, q0, x), r, q0);
+    return __builtin_fmaf(__builtin_fmaf(-s, q1, x), r, q1);
+}
+
+// true when 2^-64 <= s <= 2^64 (normal, and far from the ends of the exponent range)
+__device__ __forceinline__ bool mid_range(float s) {
+    const uint32_t b = f2u(s);
+    return b >= 0x1F800000u && b <= 0x5F800000u;
 }
 
 // ---------------------------------------------------------------- reductions

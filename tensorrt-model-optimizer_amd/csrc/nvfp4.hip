@@ -186,12 +186,6 @@ __device__ __forceinline__ uint32_t fp4_pair(uint32_t old, float a, float b, int
     }
 }
 
-__device__ __forceinline__ float exact_quotient(float x, float s, float r) {
-    const float q0 = x * r;
-    const float q1 = __builtin_fmaf(__builtin_fmaf(-s, q0, x), r, q0);
-    return __builtin_fmaf(__builtin_fmaf(-s, q1, x), r, q1);
-}
-
 __device__ __forceinline__ uint32_t exact_codes8(const uint32_t (&w)[4], float s) {
     uint32_t o = 0;
 #pragma unroll

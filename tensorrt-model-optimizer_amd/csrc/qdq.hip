@@ -1,10 +1,14 @@
 // Elementwise quantize-dequantize kernels (FP8 E4M3 and N-bit integer) for gfx950.
 //
 // HBM-bound: one read and one write of the tensor (4 bytes per bf16 element).  x and y are
-// viewed as [outer, axis, inner] with one amax per index of `axis`.  Three addressing modes:
+// viewed as [outer, axis, inner] with one amax per index of `axis`.  Addressing modes:
 //   TENSOR  one scale for everything (axis == 1);
 //   CHUNK   inner % 8 == 0, so the 8 elements a lane holds share a scale;
-//   ELEM    anything else (e.g. scales along the innermost dim): per-element scale lookup.
+//   COLS    inner == 1 and axis % 8 == 0 (scales along the innermost dim): a lane keeps the 8
+//           scales of its columns in registers and walks down a slab of rows;
+//   ELEM    anything else: per-element scale lookup.
+// TENSOR / CHUNK / ELEM run one workgroup per tile of 1024 chunks (4 per lane, all loads issued
+// before the math), dispatched in tile order.
 #include "common.h"
 
 namespace mo {
@@ -31,13 +35,17 @@ struct Fp8Op {
 
 struct IntOp {
     float bound, lo;
-    struct Scale { float mul, div; };
+    // y = clamp(rne(x * mul), lo, bound) / div; when `fast`, the division is the exact
+    // reciprocal-and-FMA quotient (|q| <= 2^24 and div in [2^-64, 2^64] cannot over/underflow)
+    struct Scale { float mul, div, rdiv; bool fast; };
     __device__ __forceinline__ Scale make(float amax) const {
         Scale s;
         const bool dead = amax <= 5.9604644775390625e-8f;  // 2^-24
         const float sc = bound / amax;
         s.mul = dead ? 0.0f : sc;
         s.div = dead ? 1.0f : sc;
+        s.rdiv = 1.0f / s.div;
+        s.fast = mid_range(s.div);
         return s;
     }
     template <bool>
@@ -46,9 +54,12 @@ struct IntOp {
         // clamp the way torch.clamp does: NaN stays NaN
         q = q < lo ? lo : q;
         q = q > bound ? bound : q;
+        if (s.fast) return __builtin_copysignf(exact_quotient(q, s.div, s.rdiv), q);
         return q / s.div;
     }
 };
+
+constexpr int kTileChunks = 1024;
 
 template <int DT, int KIND, bool FLAG, typename Op>
 __global__ __launch_bounds__(256) void qdq_kernel(const void* __restrict__ x, void* __restrict__ y,
@@ -56,37 +67,83 @@ __global__ __launch_bounds__(256) void qdq_kernel(const void* __restrict__ x, vo
                                                   const void* __restrict__ amax, int amax_dtype,
                                                   Op op) {
     const int64_t chunks = n >> 3;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t c0 = (int64_t)blockIdx.x * kTileChunks + threadIdx.x;
     typename Op::Scale s0 = {};
     if (KIND == TENSOR && amax) s0 = op.make(load_scalar(amax, amax_dtype, 0));
-    for (int64_t c = tid; c < chunks; c += stride) {
-        float v[8];
-        load_chunk<DT>(x, c << 3, v);
+    float v[4][8];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        if (c < chunks) load_chunk<DT>(x, c << 3, v[u]);
+    }
+    const int64_t inner_chunks = KIND == CHUNK ? inner >> 3 : 1;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        if (c >= chunks) continue;
         if constexpr (KIND == TENSOR) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = op.template apply<FLAG>(v[j], s0);
+            for (int j = 0; j < 8; ++j) v[u][j] = op.template apply<FLAG>(v[u][j], s0);
         } else if constexpr (KIND == CHUNK) {
-            const int64_t a = ((c << 3) / inner) % axis;
+            int64_t row;
+            if (chunks <= 0xFFFFFFFFll) row = (uint32_t)c / (uint32_t)inner_chunks;
+            else row = c / inner_chunks;
+            const int64_t a = row < axis ? row : row % axis;
             const typename Op::Scale s = op.make(load_scalar(amax, amax_dtype, a));
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = op.template apply<FLAG>(v[j], s);
+            for (int j = 0; j < 8; ++j) v[u][j] = op.template apply<FLAG>(v[u][j], s);
         } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int64_t a = (((c << 3) + j) / inner) % axis;
-                v[j] = op.template apply<FLAG>(v[j], op.make(load_scalar(amax, amax_dtype, a)));
+                v[u][j] = op.template apply<FLAG>(v[u][j], op.make(load_scalar(amax, amax_dtype, a)));
             }
         }
-        store_chunk<DT>(y, c << 3, v);
+        store_chunk<DT>(y, c << 3, v[u]);
     }
-    // tail (n % 8 elements) and nothing else: handled by the first lanes of block 0
-    if (blockIdx.x == 0 && threadIdx.x < (n & 7)) {
+    // tail (n % 8 elements): the first lanes of the last workgroup
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x < (n & 7)) {
         const int64_t i = (chunks << 3) + threadIdx.x;
         const int64_t a = KIND == TENSOR ? 0 : (i / inner) % axis;
         typename Op::Scale s = {};
         if (amax) s = op.make(load_scalar(amax, amax_dtype, a));
         store_elem<DT>(y, i, op.template apply<FLAG>(load_elem<DT>(x, i), s));
+    }
+}
+
+// Scales along the innermost dim: x viewed as [rows, axis], axis % 8 == 0.
+template <int DT, bool FLAG, typename Op>
+__global__ __launch_bounds__(256) void qdq_cols_kernel(const void* __restrict__ x,
+                                                       void* __restrict__ y, int64_t rows,
+                                                       int64_t axis, int64_t slab,
+                                                       const void* __restrict__ amax,
+                                                       int amax_dtype, Op op) {
+    const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) << 3;
+    if (col >= axis) return;
+    typename Op::Scale s[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s[j] = op.make(load_scalar(amax, amax_dtype, col + j));
+    const int64_t r0 = (int64_t)blockIdx.y * slab;
+    int64_t r1 = r0 + slab;
+    if (r1 > rows) r1 = rows;
+    int64_t r = r0;
+    for (; r + 3 < r1; r += 4) {
+        float v[4][8];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) load_chunk<DT>(x, (r + u) * axis + col, v[u]);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[u][j] = op.template apply<FLAG>(v[u][j], s[j]);
+            store_chunk<DT>(y, (r + u) * axis + col, v[u]);
+        }
+    }
+    for (; r < r1; ++r) {
+        float v[8];
+        load_chunk<DT>(x, r * axis + col, v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = op.template apply<FLAG>(v[j], s[j]);
+        store_chunk<DT>(y, r * axis + col, v);
     }
 }
 
@@ -106,26 +163,38 @@ __global__ __launch_bounds__(256) void qdq_scalar_kernel(const void* __restrict_
 }
 
 template <int DT, bool FLAG, typename Op>
-static void launch_qdq(const void* x, void* y, int64_t outer, int64_t axis, int64_t inner,
-                       const void* amax, int amax_dtype, Op op, hipStream_t s) {
+static int launch_qdq(const void* x, void* y, int64_t outer, int64_t axis, int64_t inner,
+                      const void* amax, int amax_dtype, Op op, hipStream_t s) {
     const int64_t n = outer * axis * inner;
     const bool aligned = (((uintptr_t)x | (uintptr_t)y) & 15u) == 0;
     if (!aligned) {
         int64_t b = (n + 255) / 256;
         if (b > 16384) b = 16384;
         qdq_scalar_kernel<DT, FLAG, Op><<<(unsigned)b, 256, 0, s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
-        return;
+        return MO_OK;
     }
-    int64_t b = ((n >> 3) + 255) / 256;
-    if (b < 1) b = 1;
-    if (b > 16384) b = 16384;
-    const unsigned g = (unsigned)b;
+    if (amax && axis > 1 && inner == 1 && axis % 8 == 0 && axis >= 512) {
+        const int64_t gx = (axis / 8 + 255) / 256;
+        int64_t gy = (4096 + gx - 1) / gx;
+        int64_t slab = (outer + gy - 1) / gy;
+        if (slab < 8) slab = 8;
+        gy = (outer + slab - 1) / slab;
+        if (gy > 65535) { gy = 65535; slab = (outer + gy - 1) / gy; gy = (outer + slab - 1) / slab; }
+        qdq_cols_kernel<DT, FLAG, Op><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(
+            x, y, outer, axis, slab, amax, amax_dtype, op);
+        return MO_OK;
+    }
+    int64_t tiles = ((n >> 3) + kTileChunks - 1) / kTileChunks;
+    if (tiles < 1) tiles = 1;
+    if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+    const unsigned g = (unsigned)tiles;
     if (axis == 1 || !amax)
         qdq_kernel<DT, TENSOR, FLAG, Op><<<g, 256, 0, s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
     else if (inner % 8 == 0)
         qdq_kernel<DT, CHUNK, FLAG, Op><<<g, 256, 0, s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
     else
         qdq_kernel<DT, ELEM, FLAG, Op><<<g, 256, 0, s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
+    return MO_OK;
 }
 
 }  // namespace mo
@@ -146,9 +215,9 @@ extern "C" int mo_fp8_qdq(const void* x, void* y, int64_t outer, int64_t axis, i
     if (outer == 0 || axis == 0 || inner == 0) return MO_OK;
     hipStream_t s = (hipStream_t)stream;
     mo::Fp8Op op{amax != nullptr};
-#define CALL(DT)                                                                                   \
-    if (saturate) mo::launch_qdq<DT, true>(x, y, outer, axis, inner, amax, amax_dtype, op, s);     \
-    else mo::launch_qdq<DT, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s)
+#define CALL(DT)                                                                                       \
+    rc = saturate ? mo::launch_qdq<DT, true>(x, y, outer, axis, inner, amax, amax_dtype, op, s)        \
+                  : mo::launch_qdq<DT, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s)
     switch (dtype) {
         case MO_F32: CALL(MO_F32); break;
         case MO_F16: CALL(MO_F16); break;
@@ -156,6 +225,7 @@ extern "C" int mo_fp8_qdq(const void* x, void* y, int64_t outer, int64_t axis, i
         default: return MO_ERR_DTYPE;
     }
 #undef CALL
+    if (rc != MO_OK) return rc;
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }
 
@@ -171,10 +241,11 @@ extern "C" int mo_int_qdq(const void* x, void* y, int64_t outer, int64_t axis, i
     op.bound = (float)((1 << (num_bits - 1 + (is_unsigned ? 1 : 0))) - 1);
     op.lo = is_unsigned ? 0.0f : (narrow_range ? -op.bound : -op.bound - 1.0f);
     switch (dtype) {
-        case MO_F32: mo::launch_qdq<MO_F32, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s); break;
-        case MO_F16: mo::launch_qdq<MO_F16, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s); break;
-        case MO_BF16: mo::launch_qdq<MO_BF16, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s); break;
+        case MO_F32: rc = mo::launch_qdq<MO_F32, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s); break;
+        case MO_F16: rc = mo::launch_qdq<MO_F16, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s); break;
+        case MO_BF16: rc = mo::launch_qdq<MO_BF16, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s); break;
         default: return MO_ERR_DTYPE;
     }
+    if (rc != MO_OK) return rc;
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }
