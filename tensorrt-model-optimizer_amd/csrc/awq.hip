@@ -5,25 +5,71 @@
 
 namespace mo {
 
+template <int DT>
+__device__ __forceinline__ float round_to(float v) {
+    if constexpr (DT == MO_BF16) return round_to_bf16(v);
+    else if constexpr (DT == MO_F16) return f16_bits_to_f32(f32_to_f16_bits(v));
+    else return v;
+}
+
+// 8 consecutive scale values s[c0 .. c0 + 8) as fp32 (c0 % 8 == 0, s 16-byte aligned)
+__device__ __forceinline__ void load_scales8(const void* s, int s_dtype, int64_t c0, float (&f)[8]) {
+    if (s_dtype == MO_F32) load_chunk<MO_F32>(s, c0, f);
+    else if (s_dtype == MO_F16) load_chunk<MO_F16>(s, c0, f);
+    else load_chunk<MO_BF16>(s, c0, f);
+}
+
 // y[r, c] = T( f32(x[r, c]) * f32(s[c]) )   (bf16 * bf16 -> bf16 and bf16 * fp32 -> fp32 -> bf16
-// both reduce to one fp32 product rounded once to T)
+// both reduce to one fp32 product rounded once to T).
+// Vector path (k % 8 == 0, aligned): a lane keeps the scales of its 8 columns in registers and
+// walks down a slab of rows, 4 rows of loads in flight.
+template <int DT>
+__global__ __launch_bounds__(256) void mul_cols8_kernel(const void* __restrict__ x, int64_t rows,
+                                                        int64_t k, int64_t slab,
+                                                        const void* __restrict__ s, int s_dtype,
+                                                        void* __restrict__ y) {
+    const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) << 3;
+    if (col >= k) return;
+    float sc[8];
+    load_scales8(s, s_dtype, col, sc);
+    const int64_t r0 = (int64_t)blockIdx.y * slab;
+    int64_t r1 = r0 + slab;
+    if (r1 > rows) r1 = rows;
+    int64_t r = r0;
+    for (; r + 3 < r1; r += 4) {
+        float v[4][8];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) load_chunk<DT>(x, (r + u) * k + col, v[u]);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[u][j] *= sc[j];
+            store_chunk<DT>(y, (r + u) * k + col, v[u]);
+        }
+    }
+    for (; r < r1; ++r) {
+        float v[8];
+        load_chunk<DT>(x, r * k + col, v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] *= sc[j];
+        store_chunk<DT>(y, r * k + col, v);
+    }
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void mul_cols_kernel(const void* __restrict__ x, int64_t rows,
                                                        int64_t k, const void* __restrict__ s,
                                                        int s_dtype, void* __restrict__ y) {
     const int64_t kc = (k + 7) >> 3, total = rows * kc;
-    const bool vec = (k % 8 == 0) && ((((uintptr_t)x | (uintptr_t)y) & 15u) == 0);
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
         const int64_t r = t / kc, c0 = (t - r * kc) << 3;
         float v[8];
-        if (vec) load_chunk<DT>(x, r * k + c0, v);
-        else load_chunk_guarded<DT>(x, r * k, c0, k, v);
+        load_chunk_guarded<DT>(x, r * k, c0, k, v);
 #pragma unroll
         for (int j = 0; j < 8; ++j)
             if (c0 + j < k) v[j] *= load_scalar(s, s_dtype, c0 + j);
-        if (vec) store_chunk<DT>(y, r * k + c0, v);
-        else store_chunk_guarded<DT>(y, r * k, c0, k, v);
+        store_chunk_guarded<DT>(y, r * k, c0, k, v);
     }
 }
 
@@ -32,51 +78,63 @@ __global__ __launch_bounds__(256) void mul_cols_kernel(const void* __restrict__ 
 // padded);  scale = bound / f32(amax) (amax <= 2^-24 -> output 0);
 // y = T( clamp(rne(f32(xs) * scale), lo, bound) / scale ).
 // A lane owns a chunk of 8 columns; the G = bs / 8 lanes of a block share the amax by shuffles.
-template <int DT>
+// The division is the exact reciprocal-and-FMA quotient whenever the scale is mid-range.
+template <int DT, bool VEC>
 __global__ __launch_bounds__(256) void scale_block_int_qdq_kernel(
     const void* __restrict__ x, int64_t rows, int64_t k, const void* __restrict__ s, int s_dtype,
     int lg_g, float bound, float lo, void* __restrict__ y) {
     const int G = 1 << lg_g;
     const int64_t bs = (int64_t)G << 3;
     const int64_t kp = (k + bs - 1) / bs * bs, kc = kp >> 3, total = rows * kc;
-    const bool vec = (k % 8 == 0) && ((((uintptr_t)x | (uintptr_t)y) & 15u) == 0);
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    // total is a multiple of G and the grid of 64, so a block's lanes enter the loop together
-    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
-        const int64_t r = t / kc, c0 = (t - r * kc) << 3;
-        float v[8];
-        if (vec && c0 + 8 <= k) load_chunk<DT>(x, r * k + c0, v);
+    // one workgroup per 256 chunks; total is a multiple of G, so a block's lanes stay together
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const bool live = t < total;
+    int64_t r = 0, c0 = 0;
+    float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (live) {
+        if (total <= 0xFFFFFFFFll) r = (uint32_t)t / (uint32_t)kc; else r = t / kc;
+        c0 = (t - r * kc) << 3;
+        if (VEC) load_chunk<DT>(x, r * k + c0, v);
         else load_chunk_guarded<DT>(x, r * k, c0, k, v);
-        uint32_t m = 0;
+        if (s) {
+            if (VEC) {
+                float sc[8];
+                load_scales8(s, s_dtype, c0, sc);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            if (s && c0 + j < k) {
-                const float p = v[j] * load_scalar(s, s_dtype, c0 + j);
-                if constexpr (DT == MO_BF16) v[j] = bf16_bits_to_f32(f32_to_bf16_bits(p));
-                else if constexpr (DT == MO_F16) v[j] = f16_bits_to_f32(f32_to_f16_bits(p));
-                else v[j] = p;
+                for (int j = 0; j < 8; ++j) v[j] = round_to<DT>(v[j] * sc[j]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (c0 + j < k) v[j] = round_to<DT>(v[j] * load_scalar(s, s_dtype, c0 + j));
             }
-            const uint32_t a = f2u(v[j]) & 0x7FFFFFFFu;
-            m = a > m ? a : m;
         }
-        for (int o = G >> 1; o > 0; o >>= 1) {
-            const uint32_t u = (uint32_t)__shfl_xor((int)m, o, kWave);
-            m = u > m ? u : m;
-        }
-        const float amax = u2f(m);
-        const bool dead = amax <= 5.9604644775390625e-8f;
-        const float sc = bound / amax;
-        const float mul = dead ? 0.0f : sc, div = dead ? 1.0f : sc;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            float q = __builtin_rintf(v[j] * mul);
-            q = q < lo ? lo : q;
-            q = q > bound ? bound : q;
-            v[j] = q / div;
-        }
-        if (vec && c0 + 8 <= k) store_chunk<DT>(y, r * k + c0, v);
-        else store_chunk_guarded<DT>(y, r * k, c0, k, v);
     }
+    uint32_t m = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t a = f2u(v[j]) & 0x7FFFFFFFu;
+        m = a > m ? a : m;
+    }
+    for (int o = G >> 1; o > 0; o >>= 1) {
+        const uint32_t u = (uint32_t)__shfl_xor((int)m, o, kWave);
+        m = u > m ? u : m;
+    }
+    if (!live) return;
+    const float amax = u2f(m);
+    const bool dead = amax <= 5.9604644775390625e-8f;
+    const float sc = bound / amax;
+    const float mul = dead ? 0.0f : sc, div = dead ? 1.0f : sc;
+    const float rdiv = 1.0f / div;
+    const bool fast = mid_range(div);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        float q = __builtin_rintf(v[j] * mul);
+        q = q < lo ? lo : q;
+        q = q > bound ? bound : q;
+        v[j] = fast ? __builtin_copysignf(exact_quotient(q, div, rdiv), q) : q / div;
+    }
+    if (VEC) store_chunk<DT>(y, r * k + c0, v);
+    else store_chunk_guarded<DT>(y, r * k, c0, k, v);
 }
 
 // acc[c] += sum over rows of f32( T( |x[r, c]| / T(f32(blk_amax[r, c / bs]) + tiny) ) ) when
@@ -110,24 +168,41 @@ __global__ __launch_bounds__(256) void abs_colsum_kernel(const void* __restrict_
     atomicAdd(acc + c, sum);
 }
 
-// acc[0] += sum of f32( T(a[i] - b[i]) )^2, accumulated in double across the grid.
+// acc[0] += sum of f32( T(a[i] - b[i]) )^2.  Lanes sum 8-element chunks in fp32, the grid
+// combines in double (one atomic per workgroup).
 template <int DT>
 __global__ __launch_bounds__(256) void sq_diff_sum_kernel(const void* __restrict__ a,
                                                           const void* __restrict__ b, int64_t n,
-                                                          double* __restrict__ acc) {
+                                                          int vec, double* __restrict__ acc) {
     __shared__ double smem[4];
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    float part = 0.0f;
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     double sum = 0.0;
-    int cnt = 0;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        float d = load_elem<DT>(a, i) - load_elem<DT>(b, i);
-        if constexpr (DT == MO_BF16) d = bf16_bits_to_f32(f32_to_bf16_bits(d));
-        else if constexpr (DT == MO_F16) d = f16_bits_to_f32(f32_to_f16_bits(d));
-        part += d * d;
-        if (++cnt == 64) { sum += part; part = 0.0f; cnt = 0; }
+    if (vec) {
+        const int64_t chunks = n >> 3;
+        for (int64_t c = tid; c < chunks; c += stride) {
+            float va[8], vb[8];
+            load_chunk<DT>(a, c << 3, va);
+            load_chunk<DT>(b, c << 3, vb);
+            float part = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float d = round_to<DT>(va[j] - vb[j]);
+                part += d * d;
+            }
+            sum += part;
+        }
+        if (tid < (n & 7)) {
+            const int64_t i = (chunks << 3) + tid;
+            const float d = round_to<DT>(load_elem<DT>(a, i) - load_elem<DT>(b, i));
+            sum += d * d;
+        }
+    } else {
+        for (int64_t i = tid; i < n; i += stride) {
+            const float d = round_to<DT>(load_elem<DT>(a, i) - load_elem<DT>(b, i));
+            sum += d * d;
+        }
     }
-    sum += part;
     for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if (lane == 0) smem[wave] = sum;
@@ -159,10 +234,24 @@ extern "C" int mo_mul_cols(const void* x, int64_t rows, int64_t k, int dtype, co
     if (rows == 0 || k == 0) return MO_OK;
     if (!x || !s || !y) return MO_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
-    const unsigned g = mo::blocks_for_awq(rows * ((k + 7) >> 3));
-#define CALL(DT) mo::mul_cols_kernel<DT><<<g, 256, 0, st>>>(x, rows, k, s, s_dtype, y)
-    DISPATCH_DT(dtype, CALL)
+    const bool vec = (k % 8 == 0) && ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)s) & 15u) == 0);
+    if (vec) {
+        const int64_t gx = (k / 8 + 255) / 256;
+        int64_t gy = (4096 + gx - 1) / gx;
+        int64_t slab = (rows + gy - 1) / gy;
+        if (slab < 8) slab = 8;
+        gy = (rows + slab - 1) / slab;
+        if (gy > 65535) { gy = 65535; slab = (rows + gy - 1) / gy; gy = (rows + slab - 1) / slab; }
+        dim3 grid((unsigned)gx, (unsigned)gy);
+#define CALL(DT) mo::mul_cols8_kernel<DT><<<grid, 256, 0, st>>>(x, rows, k, slab, s, s_dtype, y)
+        DISPATCH_DT(dtype, CALL)
 #undef CALL
+    } else {
+        const unsigned g = mo::blocks_for_awq(rows * ((k + 7) >> 3));
+#define CALL(DT) mo::mul_cols_kernel<DT><<<g, 256, 0, st>>>(x, rows, k, s, s_dtype, y)
+        DISPATCH_DT(dtype, CALL)
+#undef CALL
+    }
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }
 
@@ -180,8 +269,15 @@ extern "C" int mo_scale_block_int_qdq(const void* x, int64_t rows, int64_t k, in
     const float lo = is_unsigned ? 0.0f : (narrow_range ? -bound : -bound - 1.0f);
     hipStream_t st = (hipStream_t)stream;
     const int64_t kp = (k + block_size - 1) / block_size * block_size;
-    const unsigned g = mo::blocks_for_awq(rows * (kp >> 3));
-#define CALL(DT) mo::scale_block_int_qdq_kernel<DT><<<g, 256, 0, st>>>(x, rows, k, s, s_dtype, lg, bound, lo, y)
+    const int64_t total = rows * (kp >> 3);
+    const int64_t blocks = (total + 255) / 256;
+    if (blocks > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+    const bool vec = (k % block_size == 0) &&
+                     ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)s) & 15u) == 0);
+    const unsigned g = (unsigned)blocks;
+#define CALL(DT)                                                                                      \
+    if (vec) mo::scale_block_int_qdq_kernel<DT, true><<<g, 256, 0, st>>>(x, rows, k, s, s_dtype, lg, bound, lo, y); \
+    else mo::scale_block_int_qdq_kernel<DT, false><<<g, 256, 0, st>>>(x, rows, k, s, s_dtype, lg, bound, lo, y)
     DISPATCH_DT(dtype, CALL)
 #undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
@@ -211,8 +307,9 @@ extern "C" int mo_sq_diff_sum(const void* a, const void* b, int64_t n, int dtype
     if (n == 0) return MO_OK;
     if (!a || !b || !acc) return MO_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
-    const unsigned g = mo::blocks_for_awq(n, 2048);
-#define CALL(DT) mo::sq_diff_sum_kernel<DT><<<g, 256, 0, st>>>(a, b, n, acc)
+    const unsigned g = mo::blocks_for_awq((n + 7) / 8, 4096);
+    const int vec = ((((uintptr_t)a | (uintptr_t)b) & 15u) == 0) ? 1 : 0;
+#define CALL(DT) mo::sq_diff_sum_kernel<DT><<<g, 256, 0, st>>>(a, b, n, vec, acc)
     DISPATCH_DT(dtype, CALL)
 #undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;

@@ -61,6 +61,9 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
 }
 
 __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    // The empty asm keeps the compiler from merging a preceding multiply into
+    // v_fma_mixlo_f16 a, b, 0 -- the +0 addend would turn a -0.0 product into +0.0.
+    asm volatile("" : "+v"(f));
     _Float16 v = (_Float16)f;  // v_cvt_f16_f32: IEEE round to nearest even
     uint16_t b;
     __builtin_memcpy(&b, &v, 2);

@@ -321,6 +321,169 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_multi_kernel(
                        force_exact != 0, (u32x2*)jb.packed, jb.wsf);
 }
 
+// ------------------------------------------------------------------------------ fast dequantize
+// bf16 output, 16-element blocks: a lane owns a block (8 bytes of codes, 1 scale byte in, 32
+// bytes out).  Codes are decoded by v_cvt_scalef32_pk_f32_fp4; "+ 0.0f" turns the hardware's
+// -0.0 for code 8 into the table's +0.0.
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void decode8(uint32_t codes, float s, float (&v)[8]) {
+#define MO_DEC(SEL)                                                                     \
+    {                                                                                   \
+        f32x2_t p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, SEL);         \
+        v[2 * SEL] = (p.x + 0.0f) * s;                                                  \
+        v[2 * SEL + 1] = (p.y + 0.0f) * s;                                              \
+    }
+    MO_DEC(0) MO_DEC(1) MO_DEC(2) MO_DEC(3)
+#undef MO_DEC
+}
+
+__global__ __launch_bounds__(256) void nvfp4_dequantize_fast_kernel(
+    const u32x2* __restrict__ packed, const uint8_t* __restrict__ wsf,
+    const float* __restrict__ wsf2p, int64_t nblocks, uint16_t* __restrict__ y) {
+    constexpr int R = 4;
+    const float wsf2 = wsf2p[0];
+    const int64_t b0 = (int64_t)blockIdx.x * (256 * R) + threadIdx.x;
+    u32x2 c[R];
+    uint32_t sb[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int64_t blk = b0 + r * 256;
+        if (blk < nblocks) {
+            c[r] = __builtin_nontemporal_load(packed + blk);
+            sb[r] = wsf[blk];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int64_t blk = b0 + r * 256;
+        if (blk < nblocks) {
+            const float s = e4m3_to_f32(sb[r]) * wsf2;
+            float lo[8], hi[8];
+            decode8(c[r].x, s, lo);
+            decode8(c[r].y, s, hi);
+            store_chunk<MO_BF16>(y, blk * 16, lo);
+            store_chunk<MO_BF16>(y, blk * 16 + 8, hi);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------ fast QDQ
+// bf16 in/out, 16-element blocks, aligned, no padding: same data movement as the quantize fast
+// path (coalesced chunk loads, lane-pair exchange so a lane owns a block), the quotient by the
+// exact reciprocal-and-FMA division, E2M1 rounding and decoding by the hardware converts.
+template <int MODE>
+__device__ __forceinline__ void qdq_block16_bf16(const uint32_t (&w)[8], float gs, float gs_safe,
+                                                 float (&lo)[8], float (&hi)[8]) {
+    uint32_t m = w[0] & 0x7FFF7FFFu;
+#pragma unroll
+    for (int j = 1; j < 8; ++j) m = pk_max_u16(m, w[j] & 0x7FFF7FFFu);
+    const uint32_t h = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
+    const float bmax = u2f(h << 16);
+    float x[16];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        x[2 * j] = u2f(w[j] << 16);
+        x[2 * j + 1] = u2f(w[j] & 0xFFFF0000u);
+    }
+    float s;  // the value one code unit stands for
+    if constexpr (MODE == 0) {
+        float sc = bmax / (6.0f * gs_safe);
+        if (sc == sc) sc = sc < 448.0f ? sc : 448.0f;
+        s = round_e4m3<false>(sc) * gs;
+        s = s >= 1e-5f ? s : 1.0f;
+    } else {
+        s = e4m3_to_f32(block_scale_byte(bmax, 6.0f * gs)) * gs;
+    }
+    const float r = 1.0f / s;
+    const uint32_t sb = f2u(s);
+    const bool fast = sb >= 0x1F800000u && sb <= 0x44800000u && h < 0x7F80u && (bmax * r < 1.0e38f);
+    float o[16];
+    if (fast) {
+        uint32_t c0 = 0, c1 = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float a = MODE == 0 ? __builtin_fabsf(x[2 * j]) : x[2 * j];
+            const float b = MODE == 0 ? __builtin_fabsf(x[2 * j + 1]) : x[2 * j + 1];
+            const float qa = exact_quotient(a, s, r), qb = exact_quotient(b, s, r);
+            if (j < 4) c0 = fp4_pair(c0, qa, qb, j);
+            else c1 = fp4_pair(c1, qa, qb, j - 4);
+        }
+        float d0[8], d1[8];
+        decode8(c0, s, d0);
+        decode8(c1, s, d1);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { o[j] = d0[j]; o[8 + j] = d1[j]; }
+        if constexpr (MODE == 0) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) o[j] = x[j] >= 0.0f ? o[j] : -o[j];
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            if constexpr (MODE == 0) {
+                const float q = __builtin_fabsf(x[j]) / s;
+                float lvl = 6.0f;
+                lvl = q <= 5.0f ? 4.0f : lvl;
+                lvl = q < 3.5f ? 3.0f : lvl;
+                lvl = q <= 2.5f ? 2.0f : lvl;
+                lvl = q < 1.75f ? 1.5f : lvl;
+                lvl = q <= 1.25f ? 1.0f : lvl;
+                lvl = q < 0.75f ? 0.5f : lvl;
+                lvl = q <= 0.25f ? 0.0f : lvl;
+                const float t = lvl * s;
+                o[j] = x[j] >= 0.0f ? t : -t;
+            } else {
+                o[j] = e2m1_to_f32(f32_to_e2m1(x[j] / s)) * s;
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { lo[j] = o[j]; hi[j] = o[8 + j]; }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void nvfp4_qdq_fast_kernel(const uint16_t* __restrict__ x,
+                                                             uint16_t* __restrict__ y,
+                                                             int64_t nblocks, const void* amax,
+                                                             int amax_dtype) {
+    constexpr int RP = kTileBlocks / 256;
+    const float gs = load_scalar(amax, amax_dtype, 0) / 2688.0f;
+    const float gs_safe = gs > 0.0f ? gs : 1e-12f;
+    const int64_t nchunks = nblocks * 2;
+    const int64_t c0 = (int64_t)blockIdx.x * (kTileBlocks * 2) + threadIdx.x;
+    const bool odd = threadIdx.x & 1;
+    u32x4 a[RP], b[RP];
+#pragma unroll
+    for (int p = 0; p < RP; ++p) {
+        const int64_t ca = c0 + p * 512, cb = ca + 256;
+        const u32x4 zero = {0, 0, 0, 0};
+        a[p] = ca < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + ca * 8)) : zero;
+        b[p] = cb < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + cb * 8)) : zero;
+    }
+#pragma unroll
+    for (int p = 0; p < RP; ++p) {
+        const int64_t ca = c0 + p * 512, cb = ca + 256;
+        const u32x4 send = odd ? a[p] : b[p];
+        u32x4 recv;
+        recv.x = swap_adjacent_lanes(send.x);
+        recv.y = swap_adjacent_lanes(send.y);
+        recv.z = swap_adjacent_lanes(send.z);
+        recv.w = swap_adjacent_lanes(send.w);
+        const u32x4 first = odd ? recv : a[p], second = odd ? b[p] : recv;
+        const uint32_t w[8] = {first.x, first.y, first.z, first.w,
+                               second.x, second.y, second.z, second.w};
+        float lo[8], hi[8];
+        qdq_block16_bf16<MODE>(w, gs, gs_safe, lo, hi);
+        const int64_t mine = odd ? cb : ca;
+        if (mine < nchunks) {
+            const int64_t blk = mine >> 1;
+            store_chunk<MO_BF16>(y, blk * 16, lo);
+            store_chunk<MO_BF16>(y, blk * 16 + 8, hi);
+        }
+    }
+}
+
 static inline unsigned grid_for(int64_t chunks) {
     int64_t b = (chunks + 255) / 256;
     if (b < 1) b = 1;
@@ -414,6 +577,14 @@ extern "C" int mo_nvfp4_dequantize(const uint8_t* packed, const uint8_t* wsf, co
     if (((uintptr_t)packed & 3u) || ((uintptr_t)y & 15u)) return MO_ERR_ARG;
     const int64_t total = rows * (kp / 8);
     hipStream_t s = (hipStream_t)stream;
+    if (dtype == MO_BF16 && block_size == 16 && (((uintptr_t)packed & 7u) == 0)) {
+        const int64_t nblocks = total / 2;
+        const int64_t tiles = (nblocks + 1023) / 1024;
+        if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+        mo::nvfp4_dequantize_fast_kernel<<<(unsigned)tiles, 256, 0, s>>>(
+            (const mo::u32x2*)packed, wsf, wsf2, nblocks, (uint16_t*)y);
+        return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+    }
 #define CALL(DT, BS)                                                                      \
     mo::nvfp4_dequantize_kernel<DT, BS><<<mo::grid_for(total), 256, 0, s>>>(              \
         (const uint32_t*)packed, wsf, wsf2, total, y)
@@ -432,6 +603,19 @@ extern "C" int mo_nvfp4_qdq(const void* x, void* y, int64_t rows, int64_t k, int
     if (!x || !y || !amax) return MO_ERR_ARG;
     const int64_t kp = (k + block_size - 1) / block_size * block_size;
     hipStream_t s = (hipStream_t)stream;
+    if (dtype == MO_BF16 && block_size == 16 && k == kp &&
+        ((((uintptr_t)x | (uintptr_t)y) & 15u) == 0)) {
+        const int64_t nblocks = rows * k / 16;
+        const int64_t tiles = (nblocks + mo::kTileBlocks - 1) / mo::kTileBlocks;
+        if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+        if (mode == 0)
+            mo::nvfp4_qdq_fast_kernel<0><<<(unsigned)tiles, 256, 0, s>>>(
+                (const uint16_t*)x, (uint16_t*)y, nblocks, amax, amax_dtype);
+        else
+            mo::nvfp4_qdq_fast_kernel<1><<<(unsigned)tiles, 256, 0, s>>>(
+                (const uint16_t*)x, (uint16_t*)y, nblocks, amax, amax_dtype);
+        return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+    }
 #define CALL(DT, BS) mo::launch_qdq<DT, BS>(x, y, rows, k, kp, amax, amax_dtype, mode, s)
     MO_DISPATCH_DT_BS(dtype, block_size, CALL)
 #undef CALL

@@ -159,3 +159,37 @@ def test_multi_tensor_plan_matches_single_calls():
         po, wo, w2o = qtensor.nvfp4_quantize(x.cpu(), 16)
         assert_bits_equal(packed[i].cpu(), po, f"packed {i}")
         assert_bits_equal(wsf[i].cpu(), wo, f"wsf {i}")
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_fake_quant_edge_cases_and_all_patterns(mode):
+    def want(x, amax):
+        if mode == 0:
+            return fake_quant.nvfp4_fake_quant(x, amax, 16)
+        wsf2 = amax.float() / 2688.0
+        wsf, _ = qtensor.nvfp4_block_scales(x, 16, wsf2)
+        p, _, _ = qtensor.nvfp4_quantize(x, 16, wsf, wsf2)
+        return qtensor.nvfp4_dequantize(p, wsf, wsf2, 16, x.shape, x.dtype)
+
+    x = _edge_tensor()
+    amax = reduce.reduce_amax(x)
+    assert_bits_equal(_hip.nvfp4_qdq(x.to(DEV), amax.to(DEV), 16, mode).cpu(), want(x, amax), "edge tensor")
+    allv = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    finite = allv[torch.isfinite(allv.float())]
+    finite = finite[: finite.numel() // 15 * 15].reshape(-1, 15)
+    for pilot in (1.0, 0.013):
+        col = torch.full((finite.shape[0], 1), pilot, dtype=torch.bfloat16)
+        x = torch.cat([col, finite], dim=1).contiguous()
+        amax = torch.tensor(pilot * 4, dtype=torch.bfloat16)
+        assert_bits_equal(_hip.nvfp4_qdq(x.to(DEV), amax.to(DEV), 16, mode).cpu(), want(x, amax),
+                          f"all patterns pilot={pilot}")
+
+
+def test_dequantize_every_code_and_scale():
+    codes = torch.arange(256, dtype=torch.uint8).repeat(8).reshape(-1, 8)          # 256 blocks
+    scales = torch.arange(256, dtype=torch.uint8)[: codes.shape[0]].view(torch.float8_e4m3fn).reshape(-1, 1)
+    wsf2 = torch.tensor(0.37)
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        y = _hip.nvfp4_dequantize(codes.to(DEV), scales.to(DEV), wsf2.to(DEV), 16, dtype)
+        y_o = qtensor.nvfp4_dequantize(codes, scales, wsf2, 16, (codes.shape[0], 16), dtype)
+        assert_bits_equal(y.cpu(), y_o, str(dtype))
