@@ -164,50 +164,50 @@ __device__ __forceinline__ float load_scalar(const void* p, int dtype, int64_t i
 
 // ---------------------------------------------------------------- E4M3 (OCP e4m3fn)
 
-// fp32 -> E4M3 byte, round to nearest even, subnormals kept.  Magnitudes that round above 448
-// (i.e. > 464), infinities and NaN give the NaN pattern 0x7F | sign -- the behaviour of
-// torch's CPU cast.  With SAT the result saturates at +-448 instead (NaN stays NaN).
+// gfx950's FP8 converts implement OCP E4M3: v_cvt_pk_fp8_f32 rounds to nearest even, keeps
+// subnormals and returns the NaN pattern 0x7F | sign for magnitudes that round above 448
+// (i.e. >= 464), for infinities and for NaN -- on every non-NaN fp32 input the same byte as
+// torch's CPU cast (a NaN input gives a NaN byte of unspecified sign).  v_cvt_f32_fp8 decodes
+// every byte exactly (both NaN bytes to a quiet NaN).
+typedef float f32pair __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float clamp448(float f) {
+    f = f > 448.0f ? 448.0f : f;  // NaN fails both comparisons and stays NaN
+    return f < -448.0f ? -448.0f : f;
+}
+
+// fp32 -> E4M3 byte.  With SAT the result saturates at +-448 instead of overflowing to NaN.
 template <bool SAT = false>
 __device__ __forceinline__ uint32_t f32_to_e4m3(float f) {
-    uint32_t u = f2u(f);
-    uint32_t sign = (u >> 24) & 0x80u;
-    uint32_t a = u & 0x7FFFFFFFu;
-    uint32_t r;
-    if (a < 0x3C800000u) {                       // |f| < 2^-6: fixed quantum 2^-9
-        r = f2u(u2f(a) + 16384.0f) - 0x46800000u;  // 2^14 aligns the unit to mantissa bit 0
-    } else {
-        uint32_t t = a + 0x7FFFFu + ((a >> 20) & 1u);
-        r = (t - (120u << 23)) >> 20;
-        if (a > 0x7F800000u) r = 0x7F;            // NaN
-        else if (t >= 0x43F00000u) r = SAT ? 0x7E : 0x7F;  // rounds to >= 480
-    }
-    return r | sign;
+    if constexpr (SAT) f = clamp448(f);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f, f, 0, false) & 0xFFu;
+}
+
+// two fp32 -> two E4M3 bytes in bits 0..15
+template <bool SAT = false>
+__device__ __forceinline__ uint32_t f32x2_to_e4m3x2(float a, float b) {
+    if constexpr (SAT) { a = clamp448(a); b = clamp448(b); }
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xFFFFu;
 }
 
 __device__ __forceinline__ float e4m3_to_f32(uint32_t b) {
-    uint32_t sign = (b & 0x80u) << 24;
-    uint32_t e = (b >> 3) & 0xFu, m = b & 7u;
-    if ((b & 0x7Fu) == 0x7Fu) return u2f(sign | 0x7FC00000u);
-    if (e == 0) return u2f(sign | f2u((float)m * 0.001953125f));
-    return u2f(sign | ((e + 120u) << 23) | (m << 20));
+    return __builtin_amdgcn_cvt_f32_fp8((int)b, 0);
 }
 
-// fp32 rounded to the E4M3 grid, returned as fp32 (value of the byte above, without packing).
+// fp32 rounded to the E4M3 grid, returned as fp32
 template <bool SAT = false>
 __device__ __forceinline__ float round_e4m3(float f) {
-    uint32_t u = f2u(f);
-    uint32_t sign = u & 0x80000000u;
-    uint32_t a = u & 0x7FFFFFFFu;
-    float r;
-    if (a < 0x3C800000u) {
-        r = (u2f(a) + 16384.0f) - 16384.0f;
-    } else {
-        uint32_t t = (a + 0x7FFFFu + ((a >> 20) & 1u)) & 0xFFF00000u;
-        r = u2f(t);
-        if (a > 0x7F800000u) r = u2f(0x7FC00000u);
-        else if (t > 0x43E00000u) r = SAT ? 448.0f : u2f(0x7FC00000u);
-    }
-    return u2f(f2u(r) | sign);
+    if constexpr (SAT) f = clamp448(f);
+    return __builtin_amdgcn_cvt_f32_fp8(__builtin_amdgcn_cvt_pk_fp8_f32(f, f, 0, false), 0);
+}
+
+template <bool SAT = false>
+__device__ __forceinline__ void round_e4m3_pair(float& a, float& b) {
+    if constexpr (SAT) { a = clamp448(a); b = clamp448(b); }
+    const f32pair p =
+        __builtin_amdgcn_cvt_pk_f32_fp8(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false), false);
+    a = p.x;
+    b = p.y;
 }
 
 // ---------------------------------------------------------------- E2M1 (FP4)

@@ -322,8 +322,9 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_multi_kernel(
 }
 
 // ------------------------------------------------------------------------------ fast dequantize
-// bf16 output, 16-element blocks: a lane owns a block (8 bytes of codes, 1 scale byte in, 32
-// bytes out).  Codes are decoded by v_cvt_scalef32_pk_f32_fp4; "+ 0.0f" turns the hardware's
+// bf16 output, 16-element blocks: a lane owns a chunk (4 bytes of codes in, 16 bytes out, the
+// scale byte shared with the neighbouring lane), so loads and stores of a wavefront are
+// contiguous.  Codes are decoded by v_cvt_scalef32_pk_f32_fp4; "+ 0.0f" turns the hardware's
 // -0.0 for code 8 into the table's +0.0.
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 
@@ -338,32 +339,30 @@ __device__ __forceinline__ void decode8(uint32_t codes, float s, float (&v)[8]) 
 #undef MO_DEC
 }
 
+constexpr int kDequantRounds = 8;  // chunks per lane
+
 __global__ __launch_bounds__(256) void nvfp4_dequantize_fast_kernel(
-    const u32x2* __restrict__ packed, const uint8_t* __restrict__ wsf,
-    const float* __restrict__ wsf2p, int64_t nblocks, uint16_t* __restrict__ y) {
-    constexpr int R = 4;
+    const uint32_t* __restrict__ packed, const uint8_t* __restrict__ wsf,
+    const float* __restrict__ wsf2p, int64_t nchunks, uint16_t* __restrict__ y) {
+    constexpr int R = kDequantRounds;
     const float wsf2 = wsf2p[0];
-    const int64_t b0 = (int64_t)blockIdx.x * (256 * R) + threadIdx.x;
-    u32x2 c[R];
-    uint32_t sb[R];
+    const int64_t c0 = (int64_t)blockIdx.x * (256 * R) + threadIdx.x;
+    uint32_t c[R], sb[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int64_t blk = b0 + r * 256;
-        if (blk < nblocks) {
-            c[r] = __builtin_nontemporal_load(packed + blk);
-            sb[r] = wsf[blk];
+        const int64_t ch = c0 + r * 256;
+        if (ch < nchunks) {
+            c[r] = __builtin_nontemporal_load(packed + ch);
+            sb[r] = wsf[ch >> 1];
         }
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int64_t blk = b0 + r * 256;
-        if (blk < nblocks) {
-            const float s = e4m3_to_f32(sb[r]) * wsf2;
-            float lo[8], hi[8];
-            decode8(c[r].x, s, lo);
-            decode8(c[r].y, s, hi);
-            store_chunk<MO_BF16>(y, blk * 16, lo);
-            store_chunk<MO_BF16>(y, blk * 16 + 8, hi);
+        const int64_t ch = c0 + r * 256;
+        if (ch < nchunks) {
+            float v[8];
+            decode8(c[r], e4m3_to_f32(sb[r]) * wsf2, v);
+            store_chunk<MO_BF16>(y, ch * 8, v);
         }
     }
 }
@@ -475,12 +474,23 @@ __global__ __launch_bounds__(256) void nvfp4_qdq_fast_kernel(const uint16_t* __r
                                second.x, second.y, second.z, second.w};
         float lo[8], hi[8];
         qdq_block16_bf16<MODE>(w, gs, gs_safe, lo, hi);
-        const int64_t mine = odd ? cb : ca;
-        if (mine < nchunks) {
-            const int64_t blk = mine >> 1;
-            store_chunk<MO_BF16>(y, blk * 16, lo);
-            store_chunk<MO_BF16>(y, blk * 16 + 8, hi);
-        }
+        // back to the load layout, so that the stores are contiguous across the wavefront:
+        // the even lane hands over the second chunk of its round-A block and receives the
+        // first chunk of the neighbour's round-B block; the odd lane the other way round.
+        u32x4 o0, o1;
+        o0.x = f32x2_to_bf16x2(lo[0], lo[1]); o0.y = f32x2_to_bf16x2(lo[2], lo[3]);
+        o0.z = f32x2_to_bf16x2(lo[4], lo[5]); o0.w = f32x2_to_bf16x2(lo[6], lo[7]);
+        o1.x = f32x2_to_bf16x2(hi[0], hi[1]); o1.y = f32x2_to_bf16x2(hi[2], hi[3]);
+        o1.z = f32x2_to_bf16x2(hi[4], hi[5]); o1.w = f32x2_to_bf16x2(hi[6], hi[7]);
+        const u32x4 give = odd ? o0 : o1;
+        u32x4 got;
+        got.x = swap_adjacent_lanes(give.x);
+        got.y = swap_adjacent_lanes(give.y);
+        got.z = swap_adjacent_lanes(give.z);
+        got.w = swap_adjacent_lanes(give.w);
+        const u32x4 out_a = odd ? got : o0, out_b = odd ? o1 : got;
+        if (ca < nchunks) __builtin_nontemporal_store(out_a, (u32x4*)(y + ca * 8));
+        if (cb < nchunks) __builtin_nontemporal_store(out_b, (u32x4*)(y + cb * 8));
     }
 }
 
@@ -577,12 +587,12 @@ extern "C" int mo_nvfp4_dequantize(const uint8_t* packed, const uint8_t* wsf, co
     if (((uintptr_t)packed & 3u) || ((uintptr_t)y & 15u)) return MO_ERR_ARG;
     const int64_t total = rows * (kp / 8);
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == MO_BF16 && block_size == 16 && (((uintptr_t)packed & 7u) == 0)) {
-        const int64_t nblocks = total / 2;
-        const int64_t tiles = (nblocks + 1023) / 1024;
+    if (dtype == MO_BF16 && block_size == 16) {
+        const int64_t per_tile = 256 * mo::kDequantRounds;
+        const int64_t tiles = (total + per_tile - 1) / per_tile;
         if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
         mo::nvfp4_dequantize_fast_kernel<<<(unsigned)tiles, 256, 0, s>>>(
-            (const mo::u32x2*)packed, wsf, wsf2, nblocks, (uint16_t*)y);
+            (const uint32_t*)packed, wsf, wsf2, total, (uint16_t*)y);
         return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
     }
 #define CALL(DT, BS)                                                                      \

@@ -31,6 +31,16 @@ struct Fp8Op {
         if (!has_amax) return round_e4m3<SAT>(x);
         return round_e4m3<SAT>(x * s.mul) * s.inv;
     }
+    // two elements per conversion instruction
+    template <bool SAT>
+    __device__ __forceinline__ void apply2(float& a, float& b, const Scale& sa, const Scale& sb) const {
+        if (!has_amax) { round_e4m3_pair<SAT>(a, b); return; }
+        a *= sa.mul;
+        b *= sb.mul;
+        round_e4m3_pair<SAT>(a, b);
+        a *= sa.inv;
+        b *= sb.inv;
+    }
 };
 
 struct IntOp {
@@ -56,6 +66,11 @@ struct IntOp {
         q = q > bound ? bound : q;
         if (s.fast) return __builtin_copysignf(exact_quotient(q, s.div, s.rdiv), q);
         return q / s.div;
+    }
+    template <bool F>
+    __device__ __forceinline__ void apply2(float& a, float& b, const Scale& sa, const Scale& sb) const {
+        a = apply<F>(a, sa);
+        b = apply<F>(b, sb);
     }
 };
 
@@ -83,7 +98,7 @@ __global__ __launch_bounds__(256) void qdq_kernel(const void* __restrict__ x, vo
         if (c >= chunks) continue;
         if constexpr (KIND == TENSOR) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[u][j] = op.template apply<FLAG>(v[u][j], s0);
+            for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[u][j], v[u][j + 1], s0, s0);
         } else if constexpr (KIND == CHUNK) {
             int64_t row;
             if (chunks <= 0xFFFFFFFFll) row = (uint32_t)c / (uint32_t)inner_chunks;
@@ -91,7 +106,7 @@ __global__ __launch_bounds__(256) void qdq_kernel(const void* __restrict__ x, vo
             const int64_t a = row < axis ? row : row % axis;
             const typename Op::Scale s = op.make(load_scalar(amax, amax_dtype, a));
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[u][j] = op.template apply<FLAG>(v[u][j], s);
+            for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[u][j], v[u][j + 1], s, s);
         } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
@@ -134,7 +149,8 @@ __global__ __launch_bounds__(256) void qdq_cols_kernel(const void* __restrict__ 
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[u][j] = op.template apply<FLAG>(v[u][j], s[j]);
+            for (int j = 0; j < 8; j += 2)
+                op.template apply2<FLAG>(v[u][j], v[u][j + 1], s[j], s[j + 1]);
             store_chunk<DT>(y, (r + u) * axis + col, v[u]);
         }
     }
@@ -142,7 +158,7 @@ __global__ __launch_bounds__(256) void qdq_cols_kernel(const void* __restrict__ 
         float v[8];
         load_chunk<DT>(x, r * axis + col, v);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = op.template apply<FLAG>(v[j], s[j]);
+        for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[j], v[j + 1], s[j], s[j + 1]);
         store_chunk<DT>(y, r * axis + col, v);
     }
 }

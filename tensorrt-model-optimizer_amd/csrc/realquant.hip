@@ -72,6 +72,119 @@ __global__ __launch_bounds__(256) void real_dequantize_kernel(const uint8_t* __r
     }
 }
 
+// ------------------------------------------------------------------------------ tiled fast paths
+// 16-byte aligned tensors whose scale is shared by the 8 elements of a chunk (per tensor, or
+// inner % 8 == 0).  One workgroup per tile of 1024 chunks, 4 per lane, loads issued before the
+// math.  The quotient x / s comes from one reciprocal per chunk and the exact FMA correction
+// whenever the scale is in range and the largest quotient of the chunk cannot overflow; the
+// sign of a zero quotient is restored from x (s is positive on that path).
+constexpr int kRealTileChunks = 1024;
+
+__device__ __forceinline__ int64_t chunk_scale_index(int64_t c, int64_t chunks,
+                                                     int64_t inner_chunks, int64_t axis) {
+    int64_t row;
+    if (chunks <= 0xFFFFFFFFll) row = (uint32_t)c / (uint32_t)inner_chunks;
+    else row = c / inner_chunks;
+    return row < axis ? row : row % axis;
+}
+
+template <int DT, int VIA, int FMT, bool UNIFORM>
+__global__ __launch_bounds__(256) void real_quantize_tile_kernel(
+    const void* __restrict__ x, int64_t chunks, int64_t axis, int64_t inner_chunks,
+    const void* __restrict__ scale, int scale_dtype, u32x2* __restrict__ out) {
+    const int64_t c0 = (int64_t)blockIdx.x * kRealTileChunks + threadIdx.x;
+    float v[4][8];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        if (c < chunks) load_chunk<DT>(x, c << 3, v[u]);
+    }
+    float s0 = 1.0f;
+    if (UNIFORM) s0 = load_scalar(scale, scale_dtype, 0);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        if (c >= chunks) continue;
+        const float s = UNIFORM ? s0
+                                : load_scalar(scale, scale_dtype,
+                                              chunk_scale_index(c, chunks, inner_chunks, axis));
+        const float r = 1.0f / s;
+        uint32_t m = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t t = f2u(v[u][j]) & 0x7FFFFFFFu;
+            m = t > m ? t : m;
+        }
+        float q[8];
+        if (mid_range(s) && u2f(m) * r < 1.0e38f) {  // a NaN element fails the comparison
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                q[j] = __builtin_copysignf(exact_quotient(v[u][j], s, r), v[u][j]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[j] = v[u][j] / s;
+        }
+        uint32_t lo = 0, hi = 0;
+        if constexpr (FMT == 0) {
+            lo = f32x2_to_e4m3x2(round_via<VIA>(q[0]), round_via<VIA>(q[1])) |
+                 (f32x2_to_e4m3x2(round_via<VIA>(q[2]), round_via<VIA>(q[3])) << 16);
+            hi = f32x2_to_e4m3x2(round_via<VIA>(q[4]), round_via<VIA>(q[5])) |
+                 (f32x2_to_e4m3x2(round_via<VIA>(q[6]), round_via<VIA>(q[7])) << 16);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                lo |= to_int8_byte(round_via<VIA>(q[j])) << (8 * j);
+                hi |= to_int8_byte(round_via<VIA>(q[4 + j])) << (8 * j);
+            }
+        }
+        const u32x2 o = {lo, hi};
+        __builtin_nontemporal_store(o, out + c);
+    }
+}
+
+template <int DT, int FMT, bool UNIFORM>
+__global__ __launch_bounds__(256) void real_dequantize_tile_kernel(
+    const u32x2* __restrict__ q, int64_t chunks, int64_t axis, int64_t inner_chunks,
+    const void* __restrict__ scale, int scale_dtype, void* __restrict__ y) {
+    const int64_t c0 = (int64_t)blockIdx.x * kRealTileChunks + threadIdx.x;
+    u32x2 w[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        if (c < chunks) w[u] = __builtin_nontemporal_load(q + c);
+    }
+    float s0 = 1.0f;
+    if (UNIFORM) s0 = round_via<DT>(load_scalar(scale, scale_dtype, 0));
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        if (c >= chunks) continue;
+        const float s = UNIFORM ? s0
+                                : round_via<DT>(load_scalar(
+                                      scale, scale_dtype,
+                                      chunk_scale_index(c, chunks, inner_chunks, axis)));
+        float v[8];
+        // every E4M3 value and every int8 value is exact in bf16, fp16 and fp32
+        if constexpr (FMT == 0) {
+            const f32pair p0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[u].x, false);
+            const f32pair p1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[u].x, true);
+            const f32pair p2 = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[u].y, false);
+            const f32pair p3 = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[u].y, true);
+            v[0] = p0.x; v[1] = p0.y; v[2] = p1.x; v[3] = p1.y;
+            v[4] = p2.x; v[5] = p2.y; v[6] = p3.x; v[7] = p3.y;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[j] = (float)(int8_t)(w[u].x >> (8 * j));
+                v[4 + j] = (float)(int8_t)(w[u].y >> (8 * j));
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] *= s;
+        store_chunk<DT>(y, c << 3, v);
+    }
+}
+
 // ------------------------------------------------------------------------------ INT4 compress
 // Flat blocks of `bs` elements (the tail block zero padded); one thread per block.
 //   scale = T( f32(T(1 / amax)) * 7 )            (torch evaluates `7 / amax` as reciprocal * 7)
@@ -154,6 +267,158 @@ __global__ __launch_bounds__(256) void int4_pack_rows_kernel(const void* __restr
     }
 }
 
+// ------------------------------------------------------------------------------ INT4 fast paths
+// Block sizes of 8 << k elements (k <= 6) on 16-byte aligned tensors: a lane owns a chunk, the
+// lanes of a block combine their abs-max with in-wave shuffles.
+__device__ __forceinline__ uint32_t int4_code(float v) {  // clamp(rne(v), -8, 7) + 8
+    float q = __builtin_rintf(v);
+    q = q < -8.0f ? -8.0f : q;
+    q = q > 7.0f ? 7.0f : q;
+    q += 8.0f;
+    return (q == q) ? ((uint32_t)(int)q & 0xFFu) : 0u;
+}
+
+__device__ __forceinline__ uint32_t int4_nibble(float v) {  // clamp(rne(v), -8, 7) & 0xF
+    float q = __builtin_rintf(v);
+    q = q < -8.0f ? -8.0f : q;
+    q = q > 7.0f ? 7.0f : q;
+    return (q == q) ? ((uint32_t)(int)q & 0xFu) : 0u;
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void int4_block_quantize_tile_kernel(
+    const void* __restrict__ x, int64_t chunks, int lanes_per_block, int shift,
+    void* __restrict__ scales, uint32_t* __restrict__ packed) {
+    const int64_t c0 = (int64_t)blockIdx.x * kRealTileChunks + threadIdx.x;
+    float v[4][8];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[u][j] = 0.0f;
+        if (c < chunks) load_chunk<DT>(x, c << 3, v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        uint32_t m = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t t = f2u(v[u][j]) & 0x7FFFFFFFu;
+            m = t > m ? t : m;
+        }
+        // chunks is a multiple of lanes_per_block, so the lanes of a block are all in or all out
+        for (int o = lanes_per_block >> 1; o > 0; o >>= 1) {
+            const uint32_t t = (uint32_t)__shfl_xor((int)m, o, kWave);
+            m = t > m ? t : m;
+        }
+        if (c >= chunks) continue;
+        const float scale = round_via<DT>(round_via<DT>(1.0f / u2f(m)) * 7.0f);
+        if ((threadIdx.x & (lanes_per_block - 1)) == 0) store_elem<DT>(scales, c >> shift, scale);
+        uint32_t w = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            const uint32_t hi = int4_code(round_via<DT>(v[u][j] * scale));
+            const uint32_t lo = int4_code(round_via<DT>(v[u][j + 1] * scale));
+            w |= (((hi << 4) | lo) & 0xFFu) << (4 * j);
+        }
+        __builtin_nontemporal_store(w, packed + c);
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void int4_block_dequantize_tile_kernel(
+    const uint32_t* __restrict__ packed, int64_t chunks, int shift,
+    const void* __restrict__ scales, void* __restrict__ y) {
+    const int64_t c0 = (int64_t)blockIdx.x * kRealTileChunks + threadIdx.x;
+    uint32_t w[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        if (c < chunks) w[u] = __builtin_nontemporal_load(packed + c);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        if (c >= chunks) continue;
+        const float s = load_elem<DT>(scales, c >> shift);
+        const float r = 1.0f / s;
+        const bool fast = mid_range(s);
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t b = (w[u] >> (8 * j)) & 0xFFu;
+            v[2 * j] = (float)(int)(b >> 4) - 8.0f;
+            v[2 * j + 1] = (float)(int)(b & 0xFu) - 8.0f;
+        }
+        if (fast) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = exact_quotient(v[j], s, r);  // 0 / s = +0, s > 0
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = v[j] / s;
+        }
+        store_chunk<DT>(y, c << 3, v);
+    }
+}
+
+// Row-pair pack with k % 8 == 0 and block_size % 8 == 0: a lane loads the same chunk of
+// columns from rows 2j and 2j + 1 and stores 8 bytes.
+template <int DT>
+__global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
+    const void* __restrict__ w, int64_t pairs, int64_t kc, int64_t chunks_per_scale,
+    const float* __restrict__ ws, u32x2* __restrict__ out) {
+    constexpr int R = 2;
+    const int64_t total = pairs * kc;
+    const int64_t t0 = (int64_t)blockIdx.x * (256 * R) + threadIdx.x;
+    const int64_t nsb = kc / chunks_per_scale;
+    float a[R][8], b[R][8], sa[R], sb[R];
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const int64_t t = t0 + u * 256;
+        if (t >= total) continue;
+        int64_t j, c;
+        if (total <= 0xFFFFFFFFll) { j = (uint32_t)t / (uint32_t)kc; c = (uint32_t)t - (uint32_t)j * (uint32_t)kc; }
+        else { j = t / kc; c = t - j * kc; }
+        load_chunk<DT>(w, ((2 * j) * kc + c) << 3, a[u]);
+        load_chunk<DT>(w, ((2 * j + 1) * kc + c) << 3, b[u]);
+        const int64_t sc = c / chunks_per_scale;
+        sa[u] = ws[(2 * j) * nsb + sc];
+        sb[u] = ws[(2 * j + 1) * nsb + sc];
+    }
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const int64_t t = t0 + u * 256;
+        if (t >= total) continue;
+        uint32_t m = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t ta = f2u(a[u][e]) & 0x7FFFFFFFu, tb = f2u(b[u][e]) & 0x7FFFFFFFu;
+            m = ta > m ? ta : m;
+            m = tb > m ? tb : m;
+        }
+        const float ra = 1.0f / sa[u], rb = 1.0f / sb[u];
+        const float big = u2f(m);
+        const bool fast = mid_range(sa[u]) && mid_range(sb[u]) && big * ra < 1.0e38f && big * rb < 1.0e38f;
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float qa, qb;
+            if (fast) {
+                qa = exact_quotient(a[u][e], sa[u], ra);
+                qb = exact_quotient(b[u][e], sb[u], rb);
+            } else {
+                qa = a[u][e] / sa[u];
+                qb = b[u][e] / sb[u];
+            }
+            const uint32_t byte = int4_nibble(qa) | (int4_nibble(qb) << 4);
+            if (e < 4) lo |= byte << (8 * e); else hi |= byte << (8 * (e - 4));
+        }
+        const u32x2 o = {lo, hi};
+        __builtin_nontemporal_store(o, out + t);
+    }
+}
+
 static inline unsigned blocks_for(int64_t items) {
     int64_t b = (items + 255) / 256;
     if (b < 1) b = 1;
@@ -182,6 +447,31 @@ extern "C" int mo_real_quantize(const void* x, int64_t outer, int64_t axis, int6
     if (n == 0) return MO_OK;
     if (!x || !scale || !out) return MO_ERR_ARG;
     hipStream_t s = (hipStream_t)stream;
+    const bool tiled = (n % 8 == 0) && (axis == 1 || inner % 8 == 0) &&
+                       (((uintptr_t)x & 15u) == 0) && (((uintptr_t)out & 7u) == 0) &&
+                       (n / 8 + mo::kRealTileChunks - 1) / mo::kRealTileChunks <= 0x7FFFFFFF;
+    if (tiled) {
+        const int64_t chunks = n / 8, ic = axis == 1 ? 1 : inner / 8;
+        const unsigned gt = (unsigned)((chunks + mo::kRealTileChunks - 1) / mo::kRealTileChunks);
+#define TILE4(DT, VIA, FMT)                                                                       \
+    if (axis == 1)                                                                                \
+        mo::real_quantize_tile_kernel<DT, VIA, FMT, true><<<gt, 256, 0, s>>>(                     \
+            x, chunks, axis, ic, scale, scale_dtype, (mo::u32x2*)out);                            \
+    else                                                                                          \
+        mo::real_quantize_tile_kernel<DT, VIA, FMT, false><<<gt, 256, 0, s>>>(                    \
+            x, chunks, axis, ic, scale, scale_dtype, (mo::u32x2*)out)
+#define TILE3(DT, VIA) \
+    if (format == MO_FMT_E4M3) { TILE4(DT, VIA, 0); } else { TILE4(DT, VIA, 1); }
+#define CALL(DT)                                           \
+    if (via_dtype == MO_F32) { TILE3(DT, MO_F32); }        \
+    else if (via_dtype == MO_F16) { TILE3(DT, MO_F16); }   \
+    else { TILE3(DT, MO_BF16); }
+        DISPATCH_DT(dtype, CALL)
+#undef CALL
+#undef TILE3
+#undef TILE4
+        return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+    }
     const unsigned g = mo::blocks_for((n + 7) / 8);
 #define CALL3(DT, VIA)                                                                             \
     if (format == MO_FMT_E4M3)                                                                     \
@@ -208,6 +498,26 @@ extern "C" int mo_real_dequantize(const uint8_t* q, int64_t outer, int64_t axis,
     if (n == 0) return MO_OK;
     if (!q || !scale || !y) return MO_ERR_ARG;
     hipStream_t s = (hipStream_t)stream;
+    const bool tiled = (n % 8 == 0) && (axis == 1 || inner % 8 == 0) &&
+                       (((uintptr_t)y & 15u) == 0) && (((uintptr_t)q & 7u) == 0) &&
+                       (n / 8 + mo::kRealTileChunks - 1) / mo::kRealTileChunks <= 0x7FFFFFFF;
+    if (tiled) {
+        const int64_t chunks = n / 8, ic = axis == 1 ? 1 : inner / 8;
+        const unsigned gt = (unsigned)((chunks + mo::kRealTileChunks - 1) / mo::kRealTileChunks);
+#define TILE3(DT, FMT)                                                                            \
+    if (axis == 1)                                                                                \
+        mo::real_dequantize_tile_kernel<DT, FMT, true><<<gt, 256, 0, s>>>(                        \
+            (const mo::u32x2*)q, chunks, axis, ic, scale, scale_dtype, y);                        \
+    else                                                                                          \
+        mo::real_dequantize_tile_kernel<DT, FMT, false><<<gt, 256, 0, s>>>(                       \
+            (const mo::u32x2*)q, chunks, axis, ic, scale, scale_dtype, y)
+#define CALL(DT) \
+    if (format == MO_FMT_E4M3) { TILE3(DT, 0); } else { TILE3(DT, 1); }
+        DISPATCH_DT(dtype, CALL)
+#undef CALL
+#undef TILE3
+        return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+    }
     const unsigned g = mo::blocks_for(n);
 #define CALL(DT)                                                                                      \
     if (format == MO_FMT_E4M3)                                                                        \
@@ -226,6 +536,19 @@ extern "C" int mo_int4_block_quantize(const void* x, int64_t n, int64_t block_si
     if (!x || !scales || !packed) return MO_ERR_ARG;
     const int64_t nblocks = (n + block_size - 1) / block_size;
     hipStream_t s = (hipStream_t)stream;
+    int shift = -1;  // block_size == 8 << shift
+    for (int k = 0; k <= 6; ++k)
+        if (block_size == (8ll << k)) shift = k;
+    const int64_t tiles = (n / 8 + mo::kRealTileChunks - 1) / mo::kRealTileChunks;
+    if (shift >= 0 && n % block_size == 0 && (((uintptr_t)x & 15u) == 0) &&
+        (((uintptr_t)packed & 3u) == 0) && tiles <= 0x7FFFFFFF) {
+#define CALL(DT)                                                                          \
+    mo::int4_block_quantize_tile_kernel<DT><<<(unsigned)tiles, 256, 0, s>>>(              \
+        x, n / 8, 1 << shift, shift, scales, (uint32_t*)packed)
+        DISPATCH_DT(dtype, CALL)
+#undef CALL
+        return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+    }
     const unsigned g = mo::blocks_for(nblocks);
 #define CALL(DT) mo::int4_block_quantize_kernel<DT><<<g, 256, 0, s>>>(x, n, block_size, nblocks, scales, packed)
     DISPATCH_DT(dtype, CALL)
@@ -239,6 +562,19 @@ extern "C" int mo_int4_block_dequantize(const uint8_t* packed, int64_t nbytes, i
     if (nbytes == 0) return MO_OK;
     if (!packed || !scales || !y) return MO_ERR_ARG;
     hipStream_t s = (hipStream_t)stream;
+    int shift = -1;
+    for (int k = 0; k <= 40; ++k)
+        if (block_size == (8ll << k)) shift = k;
+    const int64_t tiles = (nbytes / 4 + mo::kRealTileChunks - 1) / mo::kRealTileChunks;
+    if (shift >= 0 && nbytes % 4 == 0 && (((uintptr_t)y & 15u) == 0) &&
+        (((uintptr_t)packed & 3u) == 0) && tiles <= 0x7FFFFFFF) {
+#define CALL(DT)                                                                          \
+    mo::int4_block_dequantize_tile_kernel<DT><<<(unsigned)tiles, 256, 0, s>>>(            \
+        (const uint32_t*)packed, nbytes / 4, shift, scales, y)
+        DISPATCH_DT(dtype, CALL)
+#undef CALL
+        return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+    }
     const unsigned g = mo::blocks_for(nbytes);
 #define CALL(DT) mo::int4_block_dequantize_kernel<DT><<<g, 256, 0, s>>>(packed, nbytes, block_size, scales, y)
     DISPATCH_DT(dtype, CALL)
@@ -256,6 +592,18 @@ extern "C" int mo_int4_pack_rows(const void* w, int64_t batch, int64_t n_rows, i
     hipStream_t s = (hipStream_t)stream;
     // a stack of `batch` matrices is one matrix of batch * n_rows rows (n_rows is even)
     const int64_t rows = batch * n_rows;
+    if (k % 8 == 0 && block_size % 8 == 0 && (((uintptr_t)w & 15u) == 0) &&
+        (((uintptr_t)out & 7u) == 0)) {
+        const int64_t items = (rows >> 1) * (k / 8), tiles = (items + 511) / 512;
+        if (tiles <= 0x7FFFFFFF) {
+#define CALL(DT)                                                                      \
+    mo::int4_pack_rows_tile_kernel<DT><<<(unsigned)tiles, 256, 0, s>>>(               \
+        w, rows >> 1, k / 8, block_size / 8, ws, (mo::u32x2*)out)
+            DISPATCH_DT(dtype, CALL)
+#undef CALL
+            return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+        }
+    }
     const unsigned g = mo::blocks_for((rows >> 1) * ((k + 7) >> 3));
 #define CALL(DT) mo::int4_pack_rows_kernel<DT><<<g, 256, 0, s>>>(w, rows, k, block_size, ws, out)
     DISPATCH_DT(dtype, CALL)

@@ -127,6 +127,106 @@ def test_int4_awq_export_pack(dtype, shape):
     assert_bits_equal(got.cpu(), want, "packed rows")
 
 
+# ----------------------------------------------------------------------------- exhaustive / edge
+def _all_patterns(dtype):
+    """Every 16-bit pattern of a half-width dtype (NaNs, infinities, zeros, subnormals included);
+    for fp32 the bf16 patterns widened plus a few million random bit patterns."""
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    if dtype != torch.float32:
+        return bits.view(dtype)
+    wide = bits.view(torch.bfloat16).float()
+    g = torch.Generator().manual_seed(11)
+    rnd = torch.randint(-2**31, 2**31 - 1, (1 << 20,), generator=g, dtype=torch.int64).to(torch.int32)
+    return torch.cat([wide, rnd.view(torch.float32)])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("fmt", ["e4m3", "int8"])
+def test_storage_cast_every_pattern_and_extreme_scales(dtype, fmt):
+    x = _all_patterns(dtype)
+    code = _hip.MO_FMT_E4M3 if fmt == "e4m3" else _hip.MO_FMT_INT8
+    for sv in (1.0, 0.0123, 3.0e-5, 7.7e3, 2.0**-70, 2.0**70, 1.0e-30, 0.0, float("inf"), -0.5):
+        scale = torch.tensor([sv], dtype=torch.float32)
+        if fmt == "e4m3":
+            want = (x / scale).to(torch.float8_e4m3fn)
+        else:
+            want = (x / scale).round().clamp(-128, 127).to(torch.int8)
+        got = _hip.real_quantize(x.to(DEV), scale.to(DEV), 1, 1, x.numel(), torch.float32, code)
+        if fmt == "int8":
+            # a NaN quotient has no defined int8 value in the reference (float -> int cast of NaN)
+            ok = ~torch.isnan(x / scale)
+            assert torch.equal(got.cpu()[ok], want[ok]), f"scale {sv}"
+        else:
+            assert_bits_equal(got.cpu(), want, f"scale {sv}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_storage_cast_row_scales_and_unaligned_views(dtype):
+    g = torch.Generator().manual_seed(12)
+    x = (torch.randn((96, 264), generator=g) * 3).to(dtype)
+    x[5, 7] = float("inf"); x[6, :] = 0.0; x[9, 3] = float("nan"); x[11, 8] = -0.0
+    s = (x.float().abs().amax(dim=1).clamp(min=1e-3) / 448.0)
+    want = (x / s[:, None]).to(torch.float8_e4m3fn)        # fp32 [96, 1] scale -> fp32 quotient
+    got = _hip.real_quantize(x.to(DEV), s.to(DEV), 1, 96, 264, torch.float32, _hip.MO_FMT_E4M3)
+    assert_bits_equal(got.cpu(), want, "row scales, tiled path")
+    y = _hip.real_dequantize(got, s.to(DEV), 1, 96, 264, _hip.MO_FMT_E4M3, dtype)
+    assert_bits_equal(y.cpu(), want.to(dtype) * s[:, None].to(dtype), "row scales dequant")
+    # odd inner size and an odd element offset: the guarded path
+    xo = torch.zeros(96 * 263 + 1, dtype=dtype)
+    xo[1:] = x[:, :263].reshape(-1)
+    xd = xo.to(DEV)[1:].view(96, 263)
+    want = (x[:, :263] / s[:, None]).to(torch.float8_e4m3fn)
+    got = _hip.real_quantize(xd, s.to(DEV), 1, 96, 263, torch.float32, _hip.MO_FMT_E4M3)
+    assert_bits_equal(got.cpu(), want, "row scales, guarded path")
+    y = _hip.real_dequantize(got, s.to(DEV), 1, 96, 263, _hip.MO_FMT_E4M3, dtype)
+    assert_bits_equal(y.cpu(), want.to(dtype) * s[:, None].to(dtype), "guarded dequant")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bs", [8, 16, 128, 512, 24, 1024])
+def test_int4_block_quantize_special_blocks(dtype, bs):
+    """Zero blocks (scale = inf), huge and tiny magnitudes, infinities; power-of-two block sizes
+    take the tiled kernels, the others (and block sizes above 512) the general ones."""
+    g = torch.Generator().manual_seed(13)
+    nblk = 40
+    x = torch.randn((nblk, bs), generator=g)
+    x[0] = 0.0
+    x[1] *= 1e30
+    x[2] *= 1e-30
+    x[3, 1] = float("inf")
+    x[4, 0] = -0.0
+    x[5] = 7.0
+    x = x.to(dtype)
+    p_o, s_o = qtensor.int4_quantize(x, bs)
+    packed, scales = _hip.int4_block_quantize(x.to(DEV), bs)
+    assert_bits_equal(scales.cpu(), s_o, "scales")
+    finite = torch.isfinite(s_o.float()).reshape(-1) & (s_o.float().reshape(-1) != 0)
+    got = packed.cpu().reshape(nblk, -1)
+    assert torch.equal(got[finite], p_o.reshape(nblk, -1)[finite])
+    y = _hip.int4_block_dequantize(packed, scales, bs).reshape(nblk, bs)
+    y_o = qtensor.int4_dequantize(got.reshape(p_o.shape), s_o, bs, x.shape, dtype)
+    assert_bits_equal(y.cpu(), y_o, "dequant")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_int4_awq_export_pack_large_and_special(dtype):
+    g = torch.Generator().manual_seed(14)
+    w = (torch.randn((256, 1024), generator=g) * 0.05).to(dtype)
+    w[3, 130:140] = 0.0
+    w[4, 5] = -0.0
+    ws = reduce.reduce_block_amax(w, {-1: 64}).float() / 7.0
+    ws[7, 2] = 1e-30      # quotients far outside the clamp range
+    ws[8, 1] = 2.0**70    # scale outside the reciprocal path's range
+    want = export.pack_int4_in_uint8(w, ws)
+    got = _hip.int4_pack_rows(w.to(DEV), ws.to(DEV))
+    assert_bits_equal(got.cpu(), want, "packed rows")
+    # k not a multiple of 8 chunks per scale: general kernel
+    w2 = w[:, :1020].contiguous()
+    ws2 = reduce.reduce_block_amax(w2, {-1: 12}).float() / 7.0
+    assert_bits_equal(_hip.int4_pack_rows(w2.to(DEV), ws2.to(DEV)).cpu(),
+                      export.pack_int4_in_uint8(w2, ws2), "packed rows, block 12")
+
+
 # ----------------------------------------------------------------------------- AWQ helpers
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_mul_cols_both_scale_dtypes(dtype):
