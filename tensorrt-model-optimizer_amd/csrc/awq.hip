@@ -79,6 +79,8 @@ __global__ __launch_bounds__(256) void mul_cols_kernel(const void* __restrict__ 
 // y = T( clamp(rne(f32(xs) * scale), lo, bound) / scale ).
 // A lane owns a chunk of 8 columns; the G = bs / 8 lanes of a block share the amax by shuffles.
 // The division is the exact reciprocal-and-FMA quotient whenever the scale is mid-range.
+constexpr int kQdqTileChunks = 1024;
+
 template <int DT, bool VEC>
 __global__ __launch_bounds__(256) void scale_block_int_qdq_kernel(
     const void* __restrict__ x, int64_t rows, int64_t k, const void* __restrict__ s, int s_dtype,
@@ -86,55 +88,70 @@ __global__ __launch_bounds__(256) void scale_block_int_qdq_kernel(
     const int G = 1 << lg_g;
     const int64_t bs = (int64_t)G << 3;
     const int64_t kp = (k + bs - 1) / bs * bs, kc = kp >> 3, total = rows * kc;
-    // one workgroup per 256 chunks; total is a multiple of G, so a block's lanes stay together
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const bool live = t < total;
-    int64_t r = 0, c0 = 0;
-    float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (live) {
-        if (total <= 0xFFFFFFFFll) r = (uint32_t)t / (uint32_t)kc; else r = t / kc;
-        c0 = (t - r * kc) << 3;
-        if (VEC) load_chunk<DT>(x, r * k + c0, v);
-        else load_chunk_guarded<DT>(x, r * k, c0, k, v);
-        if (s) {
+    // one workgroup per tile of 1024 chunks, 4 per lane; total and the tile size are multiples
+    // of G, so the lanes of a block stay together and are all live or all idle
+    const int64_t t0 = (int64_t)blockIdx.x * kQdqTileChunks + threadIdx.x;
+    int64_t r[4], c0[4];
+    RawChunk<DT> raw[4];
+    float v[4][8];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t t = t0 + u * 256;
+        r[u] = c0[u] = 0;
+        zero_raw<DT>(raw[u]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[u][j] = 0.0f;
+        if (t < total) {
+            if (total <= 0xFFFFFFFFll) r[u] = (uint32_t)t / (uint32_t)kc; else r[u] = t / kc;
+            c0[u] = (t - r[u] * kc) << 3;
+            if (VEC) load_raw<DT>(x, r[u] * k + c0[u], raw[u]);
+            else load_chunk_guarded<DT>(x, r[u] * k, c0[u], k, v[u]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const bool live = t0 + u * 256 < total;
+        if (VEC) unpack_raw<DT>(raw[u], v[u]);
+        if (s && live) {
             if (VEC) {
                 float sc[8];
-                load_scales8(s, s_dtype, c0, sc);
+                load_scales8(s, s_dtype, c0[u], sc);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) v[j] = round_to<DT>(v[j] * sc[j]);
+                for (int j = 0; j < 8; ++j) v[u][j] = round_to<DT>(v[u][j] * sc[j]);
             } else {
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    if (c0 + j < k) v[j] = round_to<DT>(v[j] * load_scalar(s, s_dtype, c0 + j));
+                    if (c0[u] + j < k)
+                        v[u][j] = round_to<DT>(v[u][j] * load_scalar(s, s_dtype, c0[u] + j));
             }
         }
-    }
-    uint32_t m = 0;
+        uint32_t m = 0;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const uint32_t a = f2u(v[j]) & 0x7FFFFFFFu;
-        m = a > m ? a : m;
-    }
-    for (int o = G >> 1; o > 0; o >>= 1) {
-        const uint32_t u = (uint32_t)__shfl_xor((int)m, o, kWave);
-        m = u > m ? u : m;
-    }
-    if (!live) return;
-    const float amax = u2f(m);
-    const bool dead = amax <= 5.9604644775390625e-8f;
-    const float sc = bound / amax;
-    const float mul = dead ? 0.0f : sc, div = dead ? 1.0f : sc;
-    const float rdiv = 1.0f / div;
-    const bool fast = mid_range(div);
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t a = f2u(v[u][j]) & 0x7FFFFFFFu;
+            m = a > m ? a : m;
+        }
+        for (int o = G >> 1; o > 0; o >>= 1) {
+            const uint32_t w = (uint32_t)__shfl_xor((int)m, o, kWave);
+            m = w > m ? w : m;
+        }
+        if (!live) continue;
+        const float amax = u2f(m);
+        const bool dead = amax <= 5.9604644775390625e-8f;
+        const float sc = bound / amax;
+        const float mul = dead ? 0.0f : sc, div = dead ? 1.0f : sc;
+        const float rdiv = 1.0f / div;
+        const bool fast = mid_range(div);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        float q = __builtin_rintf(v[j] * mul);
-        q = q < lo ? lo : q;
-        q = q > bound ? bound : q;
-        v[j] = fast ? __builtin_copysignf(exact_quotient(q, div, rdiv), q) : q / div;
+        for (int j = 0; j < 8; ++j) {
+            float q = __builtin_rintf(v[u][j] * mul);
+            q = q < lo ? lo : q;
+            q = q > bound ? bound : q;
+            v[u][j] = fast ? __builtin_copysignf(exact_quotient(q, div, rdiv), q) : q / div;
+        }
+        if (VEC) store_chunk<DT>(y, r[u] * k + c0[u], v[u]);
+        else store_chunk_guarded<DT>(y, r[u] * k, c0[u], k, v[u]);
     }
-    if (VEC) store_chunk<DT>(y, r * k + c0, v);
-    else store_chunk_guarded<DT>(y, r * k, c0, k, v);
 }
 
 // acc[c] += sum over rows of f32( T( |x[r, c]| / T(f32(blk_amax[r, c / bs]) + tiny) ) ) when
@@ -180,15 +197,30 @@ __global__ __launch_bounds__(256) void sq_diff_sum_kernel(const void* __restrict
     double sum = 0.0;
     if (vec) {
         const int64_t chunks = n >> 3;
-        for (int64_t c = tid; c < chunks; c += stride) {
-            float va[8], vb[8];
-            load_chunk<DT>(a, c << 3, va);
-            load_chunk<DT>(b, c << 3, vb);
+        // 4 chunks of each operand in flight per lane
+        for (int64_t c = tid; c < chunks; c += 4 * stride) {
+            RawChunk<DT> ra[4], rb[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int64_t cu = c + u * stride;
+                zero_raw<DT>(ra[u]);
+                zero_raw<DT>(rb[u]);
+                if (cu < chunks) {
+                    load_raw<DT>(a, cu << 3, ra[u]);
+                    load_raw<DT>(b, cu << 3, rb[u]);
+                }
+            }
             float part = 0.0f;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float d = round_to<DT>(va[j] - vb[j]);
-                part += d * d;
+            for (int u = 0; u < 4; ++u) {
+                float va[8], vb[8];
+                unpack_raw<DT>(ra[u], va);
+                unpack_raw<DT>(rb[u], vb);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float d = round_to<DT>(va[j] - vb[j]);
+                    part += d * d;
+                }
             }
             sum += part;
         }
@@ -270,7 +302,7 @@ extern "C" int mo_scale_block_int_qdq(const void* x, int64_t rows, int64_t k, in
     hipStream_t st = (hipStream_t)stream;
     const int64_t kp = (k + block_size - 1) / block_size * block_size;
     const int64_t total = rows * (kp >> 3);
-    const int64_t blocks = (total + 255) / 256;
+    const int64_t blocks = (total + mo::kQdqTileChunks - 1) / mo::kQdqTileChunks;
     if (blocks > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
     const bool vec = (k % block_size == 0) &&
                      ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)s) & 15u) == 0);
@@ -307,7 +339,7 @@ extern "C" int mo_sq_diff_sum(const void* a, const void* b, int64_t n, int dtype
     if (n == 0) return MO_OK;
     if (!a || !b || !acc) return MO_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
-    const unsigned g = mo::blocks_for_awq((n + 7) / 8, 4096);
+    const unsigned g = mo::blocks_for_awq((n + 7) / 8, 1024);
     const int vec = ((((uintptr_t)a | (uintptr_t)b) & 15u) == 0) ? 1 : 0;
 #define CALL(DT) mo::sq_diff_sum_kernel<DT><<<g, 256, 0, st>>>(a, b, n, vec, acc)
     DISPATCH_DT(dtype, CALL)

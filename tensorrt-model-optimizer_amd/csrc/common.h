@@ -117,6 +117,49 @@ __device__ __forceinline__ void load_chunk(const void* p, int64_t i, float (&v)[
     }
 }
 
+// The same load split in two, so that a kernel can issue the loads of several chunks before
+// the first conversion has to wait for data: RawChunk holds the registers as loaded.
+template <int DT> struct RawChunk { u32x4 a; };
+template <> struct RawChunk<MO_F32> { u32x4 a, b; };
+
+template <int DT>
+__device__ __forceinline__ void load_raw(const void* p, int64_t i, RawChunk<DT>& r) {
+    if constexpr (DT == MO_F32) {
+        const u32x4* q = (const u32x4*)((const float*)p + i);
+        r.a = __builtin_nontemporal_load(q);
+        r.b = __builtin_nontemporal_load(q + 1);
+    } else {
+        r.a = __builtin_nontemporal_load((const u32x4*)((const uint16_t*)p + i));
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ void zero_raw(RawChunk<DT>& r) {
+    const u32x4 z = {0, 0, 0, 0};
+    r.a = z;
+    if constexpr (DT == MO_F32) r.b = z;
+}
+
+template <int DT>
+__device__ __forceinline__ void unpack_raw(const RawChunk<DT>& r, float (&v)[8]) {
+    if constexpr (DT == MO_F32) {
+        v[0] = u2f(r.a.x); v[1] = u2f(r.a.y); v[2] = u2f(r.a.z); v[3] = u2f(r.a.w);
+        v[4] = u2f(r.b.x); v[5] = u2f(r.b.y); v[6] = u2f(r.b.z); v[7] = u2f(r.b.w);
+    } else {
+        const uint32_t w[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (DT == MO_BF16) {
+                v[2 * j] = u2f(w[j] << 16);
+                v[2 * j + 1] = u2f(w[j] & 0xFFFF0000u);
+            } else {
+                v[2 * j] = f16_bits_to_f32(w[j] & 0xFFFFu);
+                v[2 * j + 1] = f16_bits_to_f32(w[j] >> 16);
+            }
+        }
+    }
+}
+
 template <int DT>
 __device__ __forceinline__ void store_chunk(void* p, int64_t i, const float (&v)[8]) {
     if constexpr (DT == MO_F32) {

@@ -15,8 +15,9 @@ namespace mo {
 
 enum { TENSOR = 0, CHUNK = 1, ELEM = 2 };
 
+template <bool HAS_AMAX>
 struct Fp8Op {
-    bool has_amax;
+    static constexpr bool has_amax = HAS_AMAX;
     struct Scale { float mul, inv; };
     __device__ __forceinline__ Scale make(float amax) const {
         Scale s;
@@ -85,17 +86,20 @@ __global__ __launch_bounds__(256) void qdq_kernel(const void* __restrict__ x, vo
     const int64_t c0 = (int64_t)blockIdx.x * kTileChunks + threadIdx.x;
     typename Op::Scale s0 = {};
     if (KIND == TENSOR && amax) s0 = op.make(load_scalar(amax, amax_dtype, 0));
+    RawChunk<DT> raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        zero_raw<DT>(raw[u]);
+        if (c < chunks) load_raw<DT>(x, c << 3, raw[u]);
+    }
+    const int64_t inner_chunks = KIND == CHUNK ? inner >> 3 : 1;
     float v[4][8];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int64_t c = c0 + u * 256;
-        if (c < chunks) load_chunk<DT>(x, c << 3, v[u]);
-    }
-    const int64_t inner_chunks = KIND == CHUNK ? inner >> 3 : 1;
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int64_t c = c0 + u * 256;
         if (c >= chunks) continue;
+        unpack_raw<DT>(raw[u], v[u]);
         if constexpr (KIND == TENSOR) {
 #pragma unroll
             for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[u][j], v[u][j + 1], s0, s0);
@@ -143,11 +147,13 @@ __global__ __launch_bounds__(256) void qdq_cols_kernel(const void* __restrict__ 
     if (r1 > rows) r1 = rows;
     int64_t r = r0;
     for (; r + 3 < r1; r += 4) {
+        RawChunk<DT> raw[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) load_raw<DT>(x, (r + u) * axis + col, raw[u]);
         float v[4][8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) load_chunk<DT>(x, (r + u) * axis + col, v[u]);
-#pragma unroll
         for (int u = 0; u < 4; ++u) {
+            unpack_raw<DT>(raw[u], v[u]);
 #pragma unroll
             for (int j = 0; j < 8; j += 2)
                 op.template apply2<FLAG>(v[u][j], v[u][j + 1], s[j], s[j + 1]);
@@ -230,10 +236,13 @@ extern "C" int mo_fp8_qdq(const void* x, void* y, int64_t outer, int64_t axis, i
     if (rc != MO_OK) return rc;
     if (outer == 0 || axis == 0 || inner == 0) return MO_OK;
     hipStream_t s = (hipStream_t)stream;
-    mo::Fp8Op op{amax != nullptr};
-#define CALL(DT)                                                                                       \
-    rc = saturate ? mo::launch_qdq<DT, true>(x, y, outer, axis, inner, amax, amax_dtype, op, s)        \
-                  : mo::launch_qdq<DT, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s)
+#define CALL2(DT, SAT)                                                                                 \
+    rc = amax ? mo::launch_qdq<DT, SAT>(x, y, outer, axis, inner, amax, amax_dtype,                    \
+                                        mo::Fp8Op<true>(), s)                                          \
+              : mo::launch_qdq<DT, SAT>(x, y, outer, axis, inner, amax, amax_dtype,                    \
+                                        mo::Fp8Op<false>(), s)
+#define CALL(DT) \
+    if (saturate) { CALL2(DT, true); } else { CALL2(DT, false); }
     switch (dtype) {
         case MO_F32: CALL(MO_F32); break;
         case MO_F16: CALL(MO_F16); break;
@@ -241,6 +250,7 @@ extern "C" int mo_fp8_qdq(const void* x, void* y, int64_t outer, int64_t axis, i
         default: return MO_ERR_DTYPE;
     }
 #undef CALL
+#undef CALL2
     if (rc != MO_OK) return rc;
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

@@ -93,18 +93,21 @@ __global__ __launch_bounds__(256) void real_quantize_tile_kernel(
     const void* __restrict__ x, int64_t chunks, int64_t axis, int64_t inner_chunks,
     const void* __restrict__ scale, int scale_dtype, u32x2* __restrict__ out) {
     const int64_t c0 = (int64_t)blockIdx.x * kRealTileChunks + threadIdx.x;
+    RawChunk<DT> raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        zero_raw<DT>(raw[u]);
+        if (c < chunks) load_raw<DT>(x, c << 3, raw[u]);
+    }
+    float s0 = 1.0f;
+    if (UNIFORM) s0 = load_scalar(scale, scale_dtype, 0);
     float v[4][8];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int64_t c = c0 + u * 256;
-        if (c < chunks) load_chunk<DT>(x, c << 3, v[u]);
-    }
-    float s0 = 1.0f;
-    if (UNIFORM) s0 = load_scalar(scale, scale_dtype, 0);
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int64_t c = c0 + u * 256;
         if (c >= chunks) continue;
+        unpack_raw<DT>(raw[u], v[u]);
         const float s = UNIFORM ? s0
                                 : load_scalar(scale, scale_dtype,
                                               chunk_scale_index(c, chunks, inner_chunks, axis));
@@ -290,17 +293,18 @@ __global__ __launch_bounds__(256) void int4_block_quantize_tile_kernel(
     const void* __restrict__ x, int64_t chunks, int lanes_per_block, int shift,
     void* __restrict__ scales, uint32_t* __restrict__ packed) {
     const int64_t c0 = (int64_t)blockIdx.x * kRealTileChunks + threadIdx.x;
+    RawChunk<DT> raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        zero_raw<DT>(raw[u]);
+        if (c < chunks) load_raw<DT>(x, c << 3, raw[u]);
+    }
     float v[4][8];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int64_t c = c0 + u * 256;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[u][j] = 0.0f;
-        if (c < chunks) load_chunk<DT>(x, c << 3, v[u]);
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int64_t c = c0 + u * 256;
+        unpack_raw<DT>(raw[u], v[u]);
         uint32_t m = 0;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -372,24 +376,31 @@ __global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
     const int64_t total = pairs * kc;
     const int64_t t0 = (int64_t)blockIdx.x * (256 * R) + threadIdx.x;
     const int64_t nsb = kc / chunks_per_scale;
-    float a[R][8], b[R][8], sa[R], sb[R];
+    RawChunk<DT> ra_[R], rb_[R];
+    float sa[R], sb[R];
 #pragma unroll
     for (int u = 0; u < R; ++u) {
         const int64_t t = t0 + u * 256;
+        zero_raw<DT>(ra_[u]);
+        zero_raw<DT>(rb_[u]);
+        sa[u] = sb[u] = 1.0f;
         if (t >= total) continue;
         int64_t j, c;
         if (total <= 0xFFFFFFFFll) { j = (uint32_t)t / (uint32_t)kc; c = (uint32_t)t - (uint32_t)j * (uint32_t)kc; }
         else { j = t / kc; c = t - j * kc; }
-        load_chunk<DT>(w, ((2 * j) * kc + c) << 3, a[u]);
-        load_chunk<DT>(w, ((2 * j + 1) * kc + c) << 3, b[u]);
+        load_raw<DT>(w, ((2 * j) * kc + c) << 3, ra_[u]);
+        load_raw<DT>(w, ((2 * j + 1) * kc + c) << 3, rb_[u]);
         const int64_t sc = c / chunks_per_scale;
         sa[u] = ws[(2 * j) * nsb + sc];
         sb[u] = ws[(2 * j + 1) * nsb + sc];
     }
+    float a[R][8], b[R][8];
 #pragma unroll
     for (int u = 0; u < R; ++u) {
         const int64_t t = t0 + u * 256;
         if (t >= total) continue;
+        unpack_raw<DT>(ra_[u], a[u]);
+        unpack_raw<DT>(rb_[u], b[u]);
         uint32_t m = 0;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
