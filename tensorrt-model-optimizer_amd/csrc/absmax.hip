@@ -25,6 +25,18 @@ template <int DT> struct AbsAcc {
             m = pk_max_u16(m, t);
         }
     }
+    // the same for a chunk loaded earlier
+    __device__ __forceinline__ void raw(const RawChunk<DT>& r) {
+        if constexpr (DT == MO_F32) {
+            const uint32_t w[8] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { uint32_t t = w[j] & 0x7FFFFFFFu; m = t > m ? t : m; }
+        } else {
+            uint32_t t = pk_max_u16(pk_max_u16(r.a.x & 0x7FFF7FFFu, r.a.y & 0x7FFF7FFFu),
+                                    pk_max_u16(r.a.z & 0x7FFF7FFFu, r.a.w & 0x7FFF7FFFu));
+            m = pk_max_u16(m, t);
+        }
+    }
     __device__ __forceinline__ void elem(const void* p, int64_t i) {
         if constexpr (DT == MO_F32) {
             uint32_t t = ((const uint32_t*)p)[i] & 0x7FFFFFFFu;
@@ -112,6 +124,43 @@ __global__ __launch_bounds__(256) void absmax_rows_kernel(const void* __restrict
     }
 }
 
+// Short aligned rows (inner % 8 == 0, inner / 8 a power of two <= 64): a row is exactly one chunk
+// per lane of its group, so a wavefront load covers 64 / L whole rows of contiguous memory.
+// One workgroup per tile of 1024 chunks, four chunks (of four different rows) per lane.  When
+// `exclusive` (every accumulator element is fed by one row only) the fold is a plain
+// read-modify-write instead of an atomic.
+template <int DT>
+__global__ __launch_bounds__(256) void absmax_short_rows_kernel(const void* __restrict__ x,
+                                                                int64_t nrows, int64_t axis,
+                                                                int lg_l, int exclusive,
+                                                                uint32_t* __restrict__ acc) {
+    const int64_t chunks = nrows << lg_l;
+    const int64_t c0 = (int64_t)blockIdx.x * 1024 + threadIdx.x;
+    RawChunk<DT> raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        zero_raw<DT>(raw[u]);
+        if (c < chunks) load_raw<DT>(x, c << 3, raw[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        AbsAcc<DT> a;
+        a.raw(raw[u]);
+        const uint32_t v = group_max_u32(a.bits(), lg_l);
+        if (c < chunks && (threadIdx.x & ((1 << lg_l) - 1)) == 0) {
+            const int64_t r = c >> lg_l;
+            uint32_t* dst = acc + (exclusive ? r : r % axis);
+            if (exclusive) {
+                if (v > *dst) *dst = v;
+            } else {
+                fold_max(dst, v);
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------ columns
 // x viewed as [outer, axis] (inner == 1).  Vector path (axis % 8 == 0, aligned): a lane owns 8
 // adjacent columns, a wavefront 512; the four wavefronts of a workgroup take interleaved rows of
@@ -183,6 +232,74 @@ __global__ __launch_bounds__(256) void absmax_cols8_kernel(const void* __restric
             fold_max(acc + c, v);
         }
     }
+}
+
+// Wide variant for axis >= 2048: a workgroup spans 2048 adjacent columns (4 KiB of a bf16 row per
+// load instruction round), every lane keeps its 8 columns for the whole slab of rows -- no LDS.
+template <int DT>
+__global__ __launch_bounds__(256) void absmax_cols8_wide_kernel(const void* __restrict__ x,
+                                                                int64_t outer, int64_t axis,
+                                                                int64_t slab,
+                                                                uint32_t* __restrict__ acc) {
+    const int64_t col = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (col >= axis) return;
+    const int64_t r0 = (int64_t)blockIdx.y * slab;
+    int64_t r1 = r0 + slab;
+    if (r1 > outer) r1 = outer;
+    uint32_t m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (DT == MO_F32) {
+        int64_t r = r0;
+        for (; r + 1 < r1; r += 2) {
+            const u32x4* q0 = (const u32x4*)((const float*)x + r * axis + col);
+            const u32x4* q1 = (const u32x4*)((const float*)x + (r + 1) * axis + col);
+            const u32x4 a = __builtin_nontemporal_load(q0), b = __builtin_nontemporal_load(q0 + 1);
+            const u32x4 c = __builtin_nontemporal_load(q1), d = __builtin_nontemporal_load(q1 + 1);
+            const uint32_t w[16] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w,
+                                    c.x, c.y, c.z, c.w, d.x, d.y, d.z, d.w};
+#pragma unroll
+            for (int j = 0; j < 16; ++j) { const uint32_t t = w[j] & 0x7FFFFFFFu; m[j & 7] = t > m[j & 7] ? t : m[j & 7]; }
+        }
+        for (; r < r1; ++r) {
+            const u32x4* q = (const u32x4*)((const float*)x + r * axis + col);
+            const u32x4 a = __builtin_nontemporal_load(q), b = __builtin_nontemporal_load(q + 1);
+            const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { const uint32_t t = w[j] & 0x7FFFFFFFu; m[j] = t > m[j] ? t : m[j]; }
+        }
+    } else {
+        uint32_t p[4] = {0, 0, 0, 0};  // packed pairs of columns
+        int64_t r = r0;
+        for (; r + 3 < r1; r += 4) {
+            u32x4 a[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                a[u] = __builtin_nontemporal_load(
+                    (const u32x4*)((const uint16_t*)x + (r + u) * axis + col));
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                p[0] = pk_max_u16(p[0], a[u].x & 0x7FFF7FFFu);
+                p[1] = pk_max_u16(p[1], a[u].y & 0x7FFF7FFFu);
+                p[2] = pk_max_u16(p[2], a[u].z & 0x7FFF7FFFu);
+                p[3] = pk_max_u16(p[3], a[u].w & 0x7FFF7FFFu);
+            }
+        }
+        for (; r < r1; ++r) {
+            const u32x4 a = __builtin_nontemporal_load(
+                (const u32x4*)((const uint16_t*)x + r * axis + col));
+            p[0] = pk_max_u16(p[0], a.x & 0x7FFF7FFFu);
+            p[1] = pk_max_u16(p[1], a.y & 0x7FFF7FFFu);
+            p[2] = pk_max_u16(p[2], a.z & 0x7FFF7FFFu);
+            p[3] = pk_max_u16(p[3], a.w & 0x7FFF7FFFu);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t lo = p[j] & 0xFFFFu, hi = p[j] >> 16;
+            m[2 * j] = DT == MO_BF16 ? lo << 16 : f2u(f16_bits_to_f32(lo));
+            m[2 * j + 1] = DT == MO_BF16 ? hi << 16 : f2u(f16_bits_to_f32(hi));
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) fold_max(acc + col + j, m[j]);
 }
 
 template <int DT>
@@ -262,7 +379,15 @@ static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
         slab = (slab + 3) / 4 * 4;
         gy = (outer + slab - 1) / slab;
         if (gy > 65535) { gy = 65535; slab = ((outer + gy - 1) / gy + 3) / 4 * 4; gy = (outer + slab - 1) / slab; }
-        if (vec)
+        if (vec && axis >= 2048) {
+            const int64_t wx = (axis + 2047) / 2048;
+            int64_t wy = (4096 + wx - 1) / wx;
+            int64_t ws = (outer + wy - 1) / wy;
+            if (ws < 16) ws = 16;
+            wy = (outer + ws - 1) / ws;
+            if (wy > 65535) { wy = 65535; ws = (outer + wy - 1) / wy; wy = (outer + ws - 1) / ws; }
+            absmax_cols8_wide_kernel<DT><<<dim3((unsigned)wx, (unsigned)wy), 256, 0, s>>>(x, outer, axis, ws, acc);
+        } else if (vec)
             absmax_cols8_kernel<DT><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
         else
             absmax_cols1_kernel<DT><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
@@ -271,6 +396,16 @@ static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
     // rows of length `inner`
     const int64_t nrows = outer * axis;
     const int64_t row_chunks = (inner + 7) >> 3;
+    if (base_ok && inner % 8 == 0 && row_chunks <= 64 && (row_chunks & (row_chunks - 1)) == 0) {
+        int lg_l = 0;
+        while ((int64_t(1) << lg_l) < row_chunks) ++lg_l;
+        const int64_t tiles = (nrows * row_chunks + 1023) / 1024;
+        if (tiles <= 0x7FFFFFFF) {
+            absmax_short_rows_kernel<DT><<<dim3((unsigned)tiles), 256, 0, s>>>(
+                x, nrows, axis, lg_l, outer == 1 ? 1 : 0, acc);
+            return MO_OK;
+        }
+    }
     int lg = 0;
     while ((1 << lg) < 64 && (int64_t(1) << lg) < row_chunks) ++lg;
     const int64_t workers_per_block = 256 >> lg;

@@ -131,10 +131,7 @@ __global__ __launch_bounds__(256) void scale_block_int_qdq_kernel(
             const uint32_t a = f2u(v[u][j]) & 0x7FFFFFFFu;
             m = a > m ? a : m;
         }
-        for (int o = G >> 1; o > 0; o >>= 1) {
-            const uint32_t w = (uint32_t)__shfl_xor((int)m, o, kWave);
-            m = w > m ? w : m;
-        }
+        m = group_max_u32(m, lg_g);
         if (!live) continue;
         const float amax = u2f(m);
         const bool dead = amax <= 5.9604644775390625e-8f;

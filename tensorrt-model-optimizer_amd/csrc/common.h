@@ -309,6 +309,27 @@ __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
     return o;
 }
 
+// Max over aligned groups of 1 << lg adjacent lanes (lg <= 6), every lane of a group getting
+// the result.  The steps up to 16 lanes are DPP moves (adjacent-lane swap, pair swap, mirror
+// within 8, mirror within 16); wider groups finish with cross-row shuffles.
+__device__ __forceinline__ uint32_t group_max_u32(uint32_t m, int lg) {
+#define MO_DPP_MAX(CTRL)                                                              \
+    {                                                                                 \
+        const uint32_t t = (uint32_t)__builtin_amdgcn_mov_dpp((int)m, CTRL, 0xF, 0xF, true); \
+        m = t > m ? t : m;                                                            \
+    }
+    if (lg >= 1) MO_DPP_MAX(0xB1)   // quad_perm [1, 0, 3, 2]
+    if (lg >= 2) MO_DPP_MAX(0x4E)   // quad_perm [2, 3, 0, 1]
+    if (lg >= 3) MO_DPP_MAX(0x141)  // row_half_mirror
+    if (lg >= 4) MO_DPP_MAX(0x140)  // row_mirror
+#undef MO_DPP_MAX
+    for (int o = 16; o < (1 << lg); o <<= 1) {
+        const uint32_t t = (uint32_t)__shfl_xor((int)m, o, kWave);
+        m = t > m ? t : m;
+    }
+    return m;
+}
+
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {

@@ -312,10 +312,7 @@ __global__ __launch_bounds__(256) void int4_block_quantize_tile_kernel(
             m = t > m ? t : m;
         }
         // chunks is a multiple of lanes_per_block, so the lanes of a block are all in or all out
-        for (int o = lanes_per_block >> 1; o > 0; o >>= 1) {
-            const uint32_t t = (uint32_t)__shfl_xor((int)m, o, kWave);
-            m = t > m ? t : m;
-        }
+        m = group_max_u32(m, shift);
         if (c >= chunks) continue;
         const float scale = round_via<DT>(round_via<DT>(1.0f / u2f(m)) * 7.0f);
         if ((threadIdx.x & (lanes_per_block - 1)) == 0) store_elem<DT>(scales, c >> shift, scale);
@@ -390,7 +387,7 @@ __global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
         else { j = t / kc; c = t - j * kc; }
         load_raw<DT>(w, ((2 * j) * kc + c) << 3, ra_[u]);
         load_raw<DT>(w, ((2 * j + 1) * kc + c) << 3, rb_[u]);
-        const int64_t sc = c / chunks_per_scale;
+        const int64_t sc = (uint32_t)c / (uint32_t)chunks_per_scale;  // both below 2^32
         sa[u] = ws[(2 * j) * nsb + sc];
         sb[u] = ws[(2 * j + 1) * nsb + sc];
     }
@@ -603,7 +600,7 @@ extern "C" int mo_int4_pack_rows(const void* w, int64_t batch, int64_t n_rows, i
     hipStream_t s = (hipStream_t)stream;
     // a stack of `batch` matrices is one matrix of batch * n_rows rows (n_rows is even)
     const int64_t rows = batch * n_rows;
-    if (k % 8 == 0 && block_size % 8 == 0 && (((uintptr_t)w & 15u) == 0) &&
+    if (k % 8 == 0 && block_size % 8 == 0 && k < (1ll << 34) && (((uintptr_t)w & 15u) == 0) &&
         (((uintptr_t)out & 7u) == 0)) {
         const int64_t items = (rows >> 1) * (k / 8), tiles = (items + 511) / 512;
         if (tiles <= 0x7FFFFFFF) {
