@@ -62,28 +62,42 @@ def timed(torch, fn, steps, warmup):
     return wall_ms, dev_ms
 
 
-def cpu_baseline(torch, layers_sampled=1):
-    """The CPU oracle (= the reference's CPU torch path restated) on a bounded sample: the seven
-    weights of `layers_sampled` layer(s), block scales + codes from a given global amax."""
+def cpu_baseline(torch, passes=8):
+    """The C restatement of the reference's NVFP4 quantize+pack (oracle/c, OpenMP over blocks) on
+    a bounded sample: the seven weights of one decoder layer, quantised `passes` times from a
+    given global amax.  The first weight is also run through the torch CPU restatement (the
+    reference's own CPU path) and must give the same bytes."""
+    from oracle import cref
     from oracle import export as oexport
 
     g = torch.Generator().manual_seed(2)
+    weights = []
+    for _, n, k in LAYER_SHAPES:
+        w = (0.02 * torch.randn(n, k, generator=g)).to(torch.bfloat16)
+        weights.append((w, float(w.abs().max())))
+    cref.nvfp4_quantize(*weights[0][:1], 16, weights[0][1])  # load the library, warm the threads
     elems, secs = 0, 0.0
-    for _ in range(layers_sampled):
-        for _, n, k in LAYER_SHAPES:
-            w = (0.02 * torch.randn(n, k, generator=g)).to(torch.bfloat16)
-            amax = w.abs().max()
+    for _ in range(passes):
+        for w, amax in weights:
             t0 = time.perf_counter()
-            oexport.nvfp4_export(w, amax, 16)
+            cref.nvfp4_quantize(w, 16, amax)
             secs += time.perf_counter() - t0
             elems += w.numel()
+    w, amax = weights[0]
+    t0 = time.perf_counter()
+    p_t, s_t, _ = oexport.nvfp4_export(w, torch.tensor(amax), 16)
+    torch_secs = time.perf_counter() - t0
+    p_c, s_c, _ = cref.nvfp4_quantize(w, 16, amax)
+    assert torch.equal(p_c, p_t) and torch.equal(s_c.view(torch.uint8), s_t.view(torch.uint8))
+    torch_rate = w.numel() * QUANT_BYTES_PER_ELEM / torch_secs / 1e9
     return {
         "value": round(elems * QUANT_BYTES_PER_ELEM / secs / 1e9, 4),
         "unit": "GB/s",
-        "cores": torch.get_num_threads(),
+        "cores": cref.threads(),
         "kind": "port",
-        "sample": f"{layers_sampled} of 32 layers (7 weights, {elems} elements), torch CPU oracle, "
-                  f"{secs:.2f} s, host has {os.cpu_count()} logical CPUs",
+        "sample": f"7 weights of one layer x {passes} passes ({elems} elements), C restatement with "
+                  f"OpenMP, {secs:.2f} s wall; the torch CPU path does {torch_rate:.3f} GB/s on "
+                  f"{torch.get_num_threads()} threads; host has {os.cpu_count()} logical CPUs",
     }
 
 

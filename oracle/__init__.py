@@ -10,9 +10,11 @@ computes (reference file:line is cited in each docstring; paths are relative to 
 checkout, ``modelopt/torch/quantization`` abbreviated ``TQ``).  The arithmetic primitives the
 reference itself calls on CPU (``Tensor.to(torch.float8_e4m3fn)``, ``torch.round``,
 ``torch.searchsorted``, IEEE fp32 ``/``) are called here too, so rounding behaviour is the
-library's, not a re-derivation.  ``oracle/c/`` holds an independent bit-level C restatement of
-the NVFP4 quantize+pack chain (software E4M3 / E2M1 rounding) that is cross-checked against the
-torch restatement.
+library's, not a re-derivation.  ``oracle/c/quant_ref.c`` (loaded through ``oracle/cref.py``) is
+an independent bit-level C restatement -- software E4M3 / E2M1 / bf16 / fp16 rounding, the NVFP4
+quantize+pack and dequantize chain, FP8 and integer fake quantisation, the INT4 block compress
+and the FP8 / INT8 storage casts -- that ``tests/test_oracle_c.py`` cross-checks bit for bit
+against the torch restatement; it is also the timed CPU baseline of ``bench.py``.
 
 What pins each function (checked by ``tests/test_oracle_golden.py`` against the fixtures in
 ``tests/golden/`` that were transcribed from the reference's own tests):

@@ -381,7 +381,7 @@ static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
         if (gy > 65535) { gy = 65535; slab = ((outer + gy - 1) / gy + 3) / 4 * 4; gy = (outer + slab - 1) / slab; }
         if (vec && axis >= 2048) {
             const int64_t wx = (axis + 2047) / 2048;
-            int64_t wy = (4096 + wx - 1) / wx;
+            int64_t wy = (2048 + wx - 1) / wx;
             int64_t ws = (outer + wy - 1) / wy;
             if (ws < 16) ws = 16;
             wy = (outer + ws - 1) / ws;

@@ -209,7 +209,7 @@ __device__ __forceinline__ float load_scalar(const void* p, int dtype, int64_t i
 
 // gfx950's FP8 converts implement OCP E4M3: v_cvt_pk_fp8_f32 rounds to nearest even, keeps
 // subnormals and returns the NaN pattern 0x7F | sign for magnitudes that round above 448
-// (i.e. >= 464), for infinities and for NaN -- on every non-NaN fp32 input the same byte as
+// (i.e. > 464; the tie at 464 goes to 448), for infinities and for NaN -- on every non-NaN fp32 input the same byte as
 // torch's CPU cast (a NaN input gives a NaN byte of unspecified sign).  v_cvt_f32_fp8 decodes
 // every byte exactly (both NaN bytes to a quiet NaN).
 typedef float f32pair __attribute__((ext_vector_type(2)));

@@ -193,3 +193,25 @@ def test_dequantize_every_code_and_scale():
         y = _hip.nvfp4_dequantize(codes.to(DEV), scales.to(DEV), wsf2.to(DEV), 16, dtype)
         y_o = qtensor.nvfp4_dequantize(codes, scales, wsf2, 16, (codes.shape[0], 16), dtype)
         assert_bits_equal(y.cpu(), y_o, str(dtype))
+
+
+@pytest.mark.parametrize("shape", [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)])
+def test_llama3_8b_weight_shapes_against_c_restatement(shape):
+    """Full-size Llama-3-8B linear weights: abs-max, global scale, block scales, packed codes and
+    the dequantised tensor, bit for bit against the C restatement of the reference arithmetic."""
+    from oracle import cref
+
+    g = torch.Generator(device=DEV).manual_seed(shape[0] * 31 + shape[1])
+    xd = (torch.randn(shape, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    acc = torch.zeros(1, dtype=torch.float32, device=DEV)
+    _hip.absmax_into(xd, acc, 1, 1, xd.numel())
+    packed, wsf, wsf2 = _hip.nvfp4_quantize(xd, acc.reshape(()), 16)
+    y = _hip.nvfp4_dequantize(packed, wsf, wsf2, 16, torch.bfloat16)
+    x = xd.cpu()
+    assert float(acc) == cref.absmax(x)
+    p_c, w_c, w2_c = cref.nvfp4_quantize(x, 16)
+    assert float(wsf2) == float(w2_c)
+    assert torch.equal(wsf.cpu().view(torch.uint8), w_c.view(torch.uint8))
+    assert torch.equal(packed.cpu(), p_c)
+    y_c = cref.nvfp4_dequantize(p_c, w_c, w2_c, 16, torch.bfloat16)
+    assert torch.equal(y.cpu().view(torch.int16), y_c.view(torch.int16))
