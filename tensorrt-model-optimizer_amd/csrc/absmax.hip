@@ -61,6 +61,14 @@ __device__ __forceinline__ void fold_max(uint32_t* acc, uint32_t v) {
     if (v && v > __builtin_nontemporal_load(acc)) atomicMax(acc, v);
 }
 
+// The same with a device-coherent read, which never returns a value older than the last atomic
+// but is itself served one request at a time per address: better when few workgroups share an
+// accumulator (the multi-tensor launch), worse when thousands do.
+__device__ __forceinline__ void fold_max_coherent(uint32_t* acc, uint32_t v) {
+    if (v && v > __hip_atomic_load(acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+        atomicMax(acc, v);
+}
+
 // ------------------------------------------------------------------------------ per tensor
 // One workgroup per tile of MO_ABSMAX_TILE_ELEMS elements, dispatched in order.
 template <int DT>
@@ -352,7 +360,7 @@ __global__ __launch_bounds__(256) void absmax_multi_kernel(const mo_absmax_job* 
     for (; c < c1; c += 256) a.chunk(jb.x, c << 3);
     if (c1 == chunks && threadIdx.x < (jb.elems & 7)) a.elem(jb.x, (chunks << 3) + threadIdx.x);
     const uint32_t v = block_max_u32(a.bits(), smem);
-    if (threadIdx.x == 0) fold_max((uint32_t*)jb.acc, v);
+    if (threadIdx.x == 0) fold_max_coherent((uint32_t*)jb.acc, v);
 }
 
 template <int DT>

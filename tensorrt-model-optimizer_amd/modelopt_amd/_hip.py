@@ -304,41 +304,57 @@ def _tile_job_map(tiles_per_job, device):
 class AbsmaxPlan:
     """Per-tensor abs-max of a fixed list of tensors in one launch.
 
-    ``acc`` is a float32 vector with one running maximum per tensor (zero it for a fresh
-    reduction).  The plan keeps the tensors alive and must be rebuilt if any is reallocated.
+    ``acc`` is a float32 vector with one running maximum per tensor, refreshed by ``run``.
+    Every tile folds into an accumulator with an atomic max, and atomics that hit one cache line
+    are served one after the other; so a tensor is cut into spans of ``SPAN_TILES`` tiles, each
+    span is a job with an accumulator of its own on a separate 256-byte line, and ``run`` ends
+    with a small reduction over the spans of each tensor.  The plan keeps the tensors alive and
+    must be rebuilt if any is reallocated.
     """
+
+    SPAN_TILES = 64
+    LINE = 64  # floats between two accumulators
 
     def __init__(self, tensors):
         assert len(tensors) > 0
         dev, dt = tensors[0].device, tensors[0].dtype
         self.tensors = list(tensors)
         self.dtype = dtype_code(dt)
+        esize = tensors[0].element_size()
+        span_elems = self.SPAN_TILES * ABSMAX_TILE_ELEMS
+        spans = [max(1, -(-t.numel() // span_elems)) for t in tensors]
+        self._lines = torch.zeros((len(tensors), max(spans), self.LINE), dtype=torch.float32, device=dev)
         self.acc = torch.zeros(len(tensors), dtype=torch.float32, device=dev)
         rows, tile, per_job = [], 0, []
         for i, t in enumerate(tensors):
             _require_device(t)
             if t.device != dev or t.dtype != dt or not t.is_contiguous() or t.data_ptr() % 16:
                 raise ValueError("AbsmaxPlan needs contiguous, 16-byte aligned tensors of one dtype/device")
-            rows.append((t.data_ptr(), self.acc.data_ptr() + 4 * i, t.numel(), tile))
-            per_job.append(-(-t.numel() // ABSMAX_TILE_ELEMS))
-            tile += per_job[-1]
+            for j in range(spans[i]):
+                n = min(span_elems, t.numel() - j * span_elems)
+                rows.append((t.data_ptr() + j * span_elems * esize, self._lines[i, j].data_ptr(),
+                             n, tile))
+                per_job.append(-(-n // ABSMAX_TILE_ELEMS))
+                tile += per_job[-1]
         self.total_tiles = tile
+        self.njobs = len(rows)
         self.jobs = _job_table(rows, dev)
         self.tile_job = _tile_job_map(per_job, dev)
 
     def run(self, zero=True):
         if zero:
-            self.acc.zero_()
-        call("mo_absmax_multi", self.acc, _ptr(self.jobs), len(self.tensors), _ptr(self.tile_job),
+            self._lines.zero_()
+        call("mo_absmax_multi", self.acc, _ptr(self.jobs), self.njobs, _ptr(self.tile_job),
              self.total_tiles, self.dtype, _stream(self.acc))
+        torch.amax(self._lines[:, :, 0], dim=1, out=self.acc)  # NaN propagates
         return self.acc
 
 
 class Nvfp4QuantizePlan:
     """NVFP4 quantize + pack of a fixed list of bf16 tensors (last dim % 16 == 0) in one launch.
 
-    ``amax`` is a float32 device vector with one global amax (or wsf2 when ``amax_is_wsf2``) per
-    tensor.  Outputs are allocated once here: ``packed[i]`` uint8 [..., K/2], ``wsf[i]``
+    ``amax`` is a float32 device vector (any stride) with one global amax (or wsf2 when
+    ``amax_is_wsf2``) per tensor.  Outputs are allocated once here: ``packed[i]`` uint8 [..., K/2], ``wsf[i]``
     float8_e4m3fn [..., K/16], ``wsf2`` float32 [n].
     """
 
@@ -359,7 +375,7 @@ class Nvfp4QuantizePlan:
             w = torch.empty(lead + (t.shape[-1] // 16,), dtype=torch.uint8, device=dev)
             self.packed.append(p)
             self._wsf_u8.append(w)
-            rows.append((t.data_ptr(), p.data_ptr(), w.data_ptr(), amax.data_ptr() + 4 * i,
+            rows.append((t.data_ptr(), p.data_ptr(), w.data_ptr(), amax[i].data_ptr(),
                          self.wsf2.data_ptr() + 4 * i, t.numel(), tile, 0))
             per_job.append(-(-t.numel() // NVFP4_TILE_ELEMS))
             tile += per_job[-1]
