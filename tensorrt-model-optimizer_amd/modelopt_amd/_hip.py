@@ -365,14 +365,24 @@ class Nvfp4QuantizePlan:
         self.wsf2 = torch.empty(len(tensors), dtype=torch.float32, device=dev)
         self.packed, self._wsf_u8 = [], []
         rows, tile, per_job = [], 0, []
-        for i, t in enumerate(tensors):
+        for t in tensors:
             _require_device(t)
             if (t.dtype != torch.bfloat16 or not t.is_contiguous() or t.shape[-1] % 16
                     or t.data_ptr() % 16 or t.device != dev):
                 raise ValueError("Nvfp4QuantizePlan needs contiguous bf16 tensors with last dim % 16 == 0")
+        # all outputs are carved from two slabs (codes, block scales), each view 256-byte aligned
+        def _pad(nbytes):
+            return (nbytes + 255) // 256 * 256
+        p_off, w_off = [0], [0]
+        for t in tensors:
+            p_off.append(p_off[-1] + _pad(t.numel() // 2))
+            w_off.append(w_off[-1] + _pad(t.numel() // 16))
+        self._packed_slab = torch.empty(max(p_off[-1], 1), dtype=torch.uint8, device=dev)
+        self._wsf_slab = torch.empty(max(w_off[-1], 1), dtype=torch.uint8, device=dev)
+        for i, t in enumerate(tensors):
             lead = tuple(t.shape[:-1])
-            p = torch.empty(lead + (t.shape[-1] // 2,), dtype=torch.uint8, device=dev)
-            w = torch.empty(lead + (t.shape[-1] // 16,), dtype=torch.uint8, device=dev)
+            p = self._packed_slab[p_off[i]:p_off[i] + t.numel() // 2].view(lead + (t.shape[-1] // 2,))
+            w = self._wsf_slab[w_off[i]:w_off[i] + t.numel() // 16].view(lead + (t.shape[-1] // 16,))
             self.packed.append(p)
             self._wsf_u8.append(w)
             rows.append((t.data_ptr(), p.data_ptr(), w.data_ptr(), amax[i].data_ptr(),
