@@ -40,8 +40,9 @@ def set_quantizer_by_cfg(quant_model: nn.Module, quant_cfg: dict | QuantizeConfi
     ``{pattern: attributes}`` dict applied only under modules of that class.
     """
     quant_cfg = dict(quant_cfg)
+    index = _quantizer_index(quant_model)  # walked once, shared by every pattern below
     if "default" in quant_cfg:
-        set_quantizer_attribute(quant_model, "*", quant_cfg["default"])
+        set_quantizer_attribute(quant_model, "*", quant_cfg["default"], _index=index)
     for pattern, cfg in quant_cfg.items():
         if pattern == "default":
             continue
@@ -51,9 +52,10 @@ def set_quantizer_by_cfg(quant_model: nn.Module, quant_cfg: dict | QuantizeConfi
             if cls is None:
                 continue
             for sub_pattern, sub_cfg in cfg.items():
-                set_quantizer_attribute(quant_model, sub_pattern, sub_cfg, parent_class=cls)
+                set_quantizer_attribute(quant_model, sub_pattern, sub_cfg, parent_class=cls,
+                                        _index=index)
             continue
-        set_quantizer_attribute(quant_model, pattern, cfg)
+        set_quantizer_attribute(quant_model, pattern, cfg, _index=index)
 
 
 def _matches(name: str, wildcard_or_filter) -> bool:
@@ -64,36 +66,50 @@ def _matches(name: str, wildcard_or_filter) -> bool:
     raise NotImplementedError(f"Unsupported type {type(wildcard_or_filter)}")
 
 
-def set_quantizer_attribute(quant_model: nn.Module, wildcard_or_filter_func, attribute,
-                            parent_class: type | None = None):
-    """Set attributes on every quantizer whose qualified name matches.  A list of attribute
-    dicts turns the matched ``TensorQuantizer`` into a ``SequentialQuantizer``."""
-    for name, module in list(quant_model.named_modules()):
+def _quantizer_index(quant_model: nn.Module):
+    """[name, quantizer, parent module, attribute name] of every quantizer that is configured on
+    its own (members of a ``SequentialQuantizer`` are configured through their container)."""
+    index = []
+    parents = dict(quant_model.named_modules())
+    for name, module in parents.items():
         if not isinstance(module, (TensorQuantizer, SequentialQuantizer)):
             continue
+        parent_name, _, leaf = name.rpartition(".")
+        parent = parents[parent_name]
+        if isinstance(parent, SequentialQuantizer):
+            continue
+        index.append([name, module, parent, leaf])
+    return index
+
+
+def set_quantizer_attribute(quant_model: nn.Module, wildcard_or_filter_func, attribute,
+                            parent_class: type | None = None, _index=None):
+    """Set attributes on every quantizer whose qualified name matches.  A list of attribute
+    dicts turns the matched ``TensorQuantizer`` into a ``SequentialQuantizer``."""
+    index = _quantizer_index(quant_model) if _index is None else _index
+    many = isinstance(attribute, (list, tuple))
+    cfg = [_as_cfg(a) for a in attribute] if many else _as_cfg(attribute)
+    for entry in index:
+        name, module, parent, leaf = entry
         if not _matches(name, wildcard_or_filter_func):
             continue
-        parent_name, _, leaf = name.rpartition(".")
-        parent = quant_model.get_submodule(parent_name)
-        if isinstance(parent, SequentialQuantizer):
-            continue  # members are configured through their container
         if parent_class is not None and not isinstance(parent, parent_class):
             continue
-        if isinstance(attribute, (list, tuple)):
+        if many:
             if not isinstance(module, SequentialQuantizer):
                 device = next((b.device for b in module.buffers()), None)
                 module = SequentialQuantizer(*(TensorQuantizer() for _ in attribute))
                 if device is not None:
                     module.to(device)
                 setattr(parent, leaf, module)
+                entry[1] = module
             elif len(attribute) != len(module):
                 raise ValueError("number of attributes does not match the SequentialQuantizer")
-            module.set_from_attribute_config([_as_cfg(a) for a in attribute])
-        else:
-            if isinstance(module, SequentialQuantizer):
-                module = TensorQuantizer()
-                setattr(parent, leaf, module)
-            module.set_from_attribute_config(_as_cfg(attribute))
+        elif isinstance(module, SequentialQuantizer):
+            module = TensorQuantizer()
+            setattr(parent, leaf, module)
+            entry[1] = module
+        module.set_from_attribute_config(cfg)
 
 
 def _as_cfg(attribute):

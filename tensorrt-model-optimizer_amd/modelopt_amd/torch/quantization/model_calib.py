@@ -17,7 +17,7 @@ from torch import nn
 from ... import _hip
 from .conversion import set_quantizer_by_cfg_context
 from .nn import QuantModule, SequentialQuantizer, TensorQuantizer
-from .utils import is_quantized_linear
+from .utils import all_valid_scales, is_quantized_linear
 
 __all__ = ["max_calibrate", "smoothquant", "awq", "awq_lite", "enable_stats_collection",
            "finish_stats_collection", "apply_pre_quant_scale_and_smooth"]
@@ -49,6 +49,15 @@ def enable_stats_collection(model: nn.Module):
 
 def finish_stats_collection(model: nn.Module, method: str | None = None):
     """Load the collected amax into ``_amax`` and switch quantisation back on."""
+    # the calibrators' deferred sanity checks, for all of them at once: one host synchronisation
+    # instead of one per quantizer (a calibrator that fails is left to raise its own message)
+    pending = [m._calibrator for m in model.modules()
+               if isinstance(m, TensorQuantizer) and not m._disabled
+               and getattr(m._calibrator, "_acc", None) is not None
+               and not m._calibrator._validated]
+    if pending and all_valid_scales([c._acc for c in pending]):
+        for c in pending:
+            c._validated = True
     for module in model.modules():
         if not isinstance(module, TensorQuantizer) or module._disabled:
             continue

@@ -18,6 +18,7 @@ from . import model_calib
 from .config import QuantizeConfig, QuantizerAttributeConfig, normalize_algorithm
 from .conversion import is_converted, replace_quant_module, set_quantizer_attribute, set_quantizer_by_cfg
 from .nn import SequentialQuantizer, TensorQuantizer
+from .utils import all_valid_scales
 
 __all__ = ["quantize", "calibrate", "disable_quantizer", "enable_quantizer", "print_quant_summary",
            "fold_weight", "postprocess_amax"]
@@ -66,9 +67,12 @@ def calibrate(model: nn.Module, algorithm="max", forward_loop: ForwardLoop | Non
         elif method == "awq_lite":
             model_calib.awq(model, forward_loop, "awq_lite", alpha_step=kwargs.get("alpha_step", 0.1),
                             debug=kwargs.get("debug", False))
-        for name, module in model.named_modules():
-            if isinstance(module, TensorQuantizer):
-                for attr in ("_amax", "_pre_quant_scale"):
+        quantizers = [(n, m) for n, m in model.named_modules() if isinstance(m, TensorQuantizer)]
+        attrs = ("_amax", "_pre_quant_scale")
+        # one check for all of them; only a failure is walked through to name the culprit
+        if not all_valid_scales([getattr(m, a, None) for _, m in quantizers for a in attrs]):
+            for name, module in quantizers:
+                for attr in attrs:
                     module.validate_attr(attr_name=attr, warn_error=True, name=name)
     finally:
         model.train(training)

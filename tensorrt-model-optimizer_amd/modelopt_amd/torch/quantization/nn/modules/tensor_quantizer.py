@@ -58,18 +58,21 @@ class TensorQuantizer(nn.Module):
         """Copy config fields onto ``_<field>`` attributes (``enable`` -> ``_disabled``,
         ``type`` -> ``_dynamic``, ``calibrator`` -> a calibrator instance)."""
         items = attribute_cfg.items()
+        fields = QuantizerAttributeConfig.model_fields
         for name, val in items:
-            assert name in QuantizerAttributeConfig.model_fields, (
-                f"{name} is not a valid `TensorQuantizer` attribute")
+            assert name in fields, f"{name} is not a valid `TensorQuantizer` attribute"
+        # the values are plain python objects (never tensors or modules), so they can skip
+        # nn.Module's attribute bookkeeping
+        plain = object.__setattr__
         for name, val in items:
             if name == "enable":
-                self._disabled = val is False
+                plain(self, "_disabled", val is False)
             elif name == "type":
-                self._dynamic = val == "dynamic"
+                plain(self, "_dynamic", val == "dynamic")
             elif name == "calibrator":
                 continue
             else:
-                setattr(self, f"_{name}", val)
+                plain(self, f"_{name}", val)
         for name, val in items:
             if name == "calibrator":
                 self._calibrator = self._make_calibrator(val)

@@ -121,3 +121,20 @@ def update_quant_cfg_with_kv_cache_quant(quant_cfg: dict, kv_cache_quant_cfg: di
     if not quant_cfg.get("algorithm"):
         quant_cfg["algorithm"] = "max"
     return quant_cfg
+
+
+def all_valid_scales(tensors) -> bool:
+    """True when every element of every tensor is finite and non-negative -- one device
+    reduction and one host synchronisation for the whole list."""
+    flat = [t.detach().reshape(-1).to(torch.float32) for t in tensors
+            if isinstance(t, torch.Tensor) and not t.is_meta and t.numel()]
+    if not flat:
+        return True
+    by_device = {}
+    for t in flat:
+        by_device.setdefault(t.device, []).append(t)
+    flags = []
+    for group in by_device.values():
+        v = torch.cat(group)
+        flags.append((torch.isfinite(v) & (v >= 0)).all())
+    return all(bool(f) for f in flags)
