@@ -11,6 +11,17 @@ from .fake_quant import static_block_fake_quant, tensor_quant
 from .reduce import reduce_amax
 
 
+def pow_ref(t: torch.Tensor, exponent: float):
+    """``t.pow(exponent)`` as the reference writes it, with one host dependence removed: torch's
+    CPU kernel evaluates ``pow(x, 0.5)`` as an fp32 square root, which is correctly rounded on
+    some hosts and one ulp off for about one input in six on others (seen between two x86 hosts
+    with the same torch build).  The oracle pins the correctly rounded root -- a double-precision
+    root rounded to fp32, then to ``t.dtype`` -- so that it gives one answer everywhere."""
+    if exponent == 0.5:
+        return t.double().sqrt().float().to(t.dtype)
+    return t.pow(exponent)
+
+
 def awq_weight_scale(w: torch.Tensor, block_size: int | None):
     """mean over rows of |w| / (block amax + tiny), in the weight dtype, then fp32 ``[K]``.
     Follows TQ/model_calib.py:588-603."""
@@ -38,7 +49,7 @@ def awq_act_scale(x: torch.Tensor):
 def awq_get_scale(x_max: torch.Tensor, w_max: torch.Tensor, alpha: float):
     """s = clamp(x^a / (w^(1-a) + tiny), 1e-4, 1e4); s /= sqrt(max(s) * min(s)).
     Follows TQ/model_calib.py:608-621."""
-    s = (x_max.pow(alpha) / (w_max.pow(1 - alpha) + torch.finfo(torch.float32).tiny)).clamp(
+    s = (pow_ref(x_max, alpha) / (pow_ref(w_max, 1 - alpha) + torch.finfo(torch.float32).tiny)).clamp(
         min=1e-4, max=1e4).view(-1)
     return (s / (s.max() * s.min()).sqrt()).view(-1)
 
@@ -104,7 +115,7 @@ def smoothquant_linear(w: torch.Tensor, act_amax: torch.Tensor, alpha: float = 1
     """
     a = act_amax.float()
     wcol = w.abs().amax(dim=0, keepdim=True)
-    scale_a = (wcol.pow(1 - alpha) / a.pow(alpha)).squeeze()
+    scale_a = (pow_ref(wcol, 1 - alpha) / pow_ref(a, alpha)).squeeze()
     eps = 1.0 / (1 << 31)
     if scale_a.min() <= eps:
         scale_a[a.reshape(-1) <= eps] = 1

@@ -120,6 +120,19 @@ def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.T
         linear.input_quantizer.amax = (smoothing * pre_quant_scale.to(device)).amax().to(dtype)
 
 
+def _pow(t: torch.Tensor, exponent: float) -> torch.Tensor:
+    """``t.pow(exponent)`` with the CPU result for the exponents the CPU evaluates exactly.
+
+    torch's CPU kernel turns ``pow(x, 0.5)`` into a correctly rounded fp32 square root; the GPU
+    kernel's square root is off by an ulp for about one input in six.  A double-precision root
+    rounded to fp32 is the correctly rounded fp32 root, so that is what is used here; other
+    exponents go through the device ``pow`` (within an ulp or two of the CPU's).
+    """
+    if exponent == 0.5:
+        return t.double().sqrt().float().to(t.dtype)
+    return t.pow(exponent)
+
+
 # ----------------------------------------------------------------------------- SmoothQuant
 @torch.no_grad()
 def smoothquant(model: nn.Module, forward_loop=None, alpha=1.0):
@@ -138,7 +151,7 @@ def smoothquant(model: nn.Module, forward_loop=None, alpha=1.0):
         col = torch.zeros(w.shape[1], dtype=torch.float32, device=device)
         _hip.absmax_into(w.data.contiguous(), col, w.shape[0], w.shape[1], 1)
         weight_scale = col.to(dtype).reshape(1, -1)  # == w.abs().amax(dim=0, keepdim=True)
-        scale_a = (weight_scale.pow(1 - alpha) / act_amax.pow(alpha)).squeeze()
+        scale_a = (_pow(weight_scale, 1 - alpha) / _pow(act_amax, alpha)).squeeze()
         module.input_quantizer._amax_for_smoothing = act_amax.cpu()
         module.input_quantizer.reset_amax()
         module.input_quantizer.axis = None
@@ -219,7 +232,7 @@ def get_act_scale(x):
 
 
 def get_scale(x_max, w_max, alpha):
-    scales = (x_max.pow(alpha) / (w_max.to(x_max.device).pow(1 - alpha)
+    scales = (_pow(x_max, alpha) / (_pow(w_max.to(x_max.device), 1 - alpha)
                                   + torch.finfo(torch.float32).tiny)).clamp(min=1e-4, max=1e4).view(-1)
     return (scales / (scales.max() * scales.min()).sqrt()).view(-1)
 
