@@ -10,6 +10,7 @@ Prints ONE JSON line.  Synthetic weights: bf16 N(0, 0.02), generated on the devi
 """
 
 import argparse
+import contextlib
 import json
 import os
 import sys
@@ -99,6 +100,95 @@ def cpu_baseline(torch, passes=8):
                   f"OpenMP, {secs:.2f} s wall; the torch CPU path does {torch_rate:.3f} GB/s on "
                   f"{torch.get_num_threads()} threads; host has {os.cpu_count()} logical CPUs",
     }
+
+
+def single_tensor_configs(torch, steps, warmup):
+    """BASELINE configs 1, 3 and 4 (one tensor / one linear each), device time per pass.
+
+    C1: FP8 abs-max + fake quant of a 4096 x 4096 weight with 0.1 % outliers (6 B / element).
+    C3: AWQ-lite search, 21 alphas, W 4096 x 4096, X 512 x 4096 (mtq.quantize end to end, and the
+        flop rate of its 22 GEMMs over that time).
+    C4: NVFP4 abs-max + dynamic-block fake quant of 8192 x 8192 activations (6 B / element), and
+        SmoothQuant (alpha 0.5) + INT8 on an 8192 x 8192 linear end to end.
+    """
+    import copy
+
+    from torch import nn
+
+    import modelopt_amd.torch.quantization as mtq
+    from modelopt_amd import _hip
+
+    dev = torch.device("cuda:0")
+    out = {}
+
+    g = torch.Generator().manual_seed(1)
+    w = 0.02 * torch.randn(4096, 4096, generator=g)
+    w.view(-1)[torch.randperm(w.numel(), generator=g)[:16777]] *= 50
+    w = w.to(torch.bfloat16).to(dev)
+    acc = torch.zeros(1, dtype=torch.float32, device=dev)
+    y = torch.empty_like(w)
+
+    def c1():
+        acc.zero_()
+        _hip.absmax_into(w, acc, 1, 1, w.numel())
+        _hip.fp8_qdq(w, acc, 1, 1, w.numel(), out=y)
+    _, ms = timed(torch, c1, steps, warmup)
+    out["c1_fp8_amax_plus_qdq_4096x4096"] = {"ms": round(ms, 4), "GBps": round(w.numel() * 6 / ms / 1e6, 1)}
+
+    g = torch.Generator().manual_seed(4)
+    x = (torch.randn(8192, 8192, generator=g) * torch.exp(1.5 * torch.randn(8192, generator=g))[None, :]
+         ).to(torch.bfloat16).to(dev)
+    y = torch.empty_like(x)
+
+    def c4():
+        acc.zero_()
+        _hip.absmax_into(x, acc, 1, 1, x.numel())
+        _hip.nvfp4_qdq(x, acc, 16, 0, out=y)
+    _, ms = timed(torch, c4, steps, warmup)
+    out["c4_nvfp4_amax_plus_qdq_8192x8192"] = {"ms": round(ms, 4), "GBps": round(x.numel() * 6 / ms / 1e6, 1)}
+
+    class OneLinear(nn.Module):
+        def __init__(self, weight):
+            super().__init__()
+            self.proj = nn.Linear(weight.shape[1], weight.shape[0], bias=False, device=dev,
+                                  dtype=torch.bfloat16)
+            self.proj.weight.data.copy_(weight)
+
+        def forward(self, t):
+            return self.proj(t)
+
+    def end_to_end(weight, acts, cfg, reps=3):
+        best = None
+        for _ in range(reps):          # the first repetition also pays GEMM autotuning
+            model = OneLinear(weight)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            mtq.quantize(model, cfg, lambda m: m(acts))
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        return best
+
+    g = torch.Generator().manual_seed(5)
+    w8 = (0.02 * torch.randn(8192, 8192, generator=g)).to(torch.bfloat16).to(dev)
+    cfg = copy.deepcopy(mtq.INT8_SMOOTHQUANT_CFG)
+    cfg["algorithm"] = {"method": "smoothquant", "alpha": 0.5}
+    out["c4_smoothquant_int8_8192x8192_end_to_end_ms"] = round(end_to_end(w8, x, cfg) * 1e3, 3)
+    del w8, x, y
+
+    g = torch.Generator().manual_seed(3)
+    w3 = (0.02 * torch.randn(4096, 4096, generator=g)).to(torch.bfloat16).to(dev)
+    c = torch.exp(torch.randn(4096, generator=g))
+    c[torch.randperm(4096, generator=g)[:41]] *= 20
+    x3 = (torch.randn(512, 4096, generator=g) * c).to(torch.bfloat16).to(dev)
+    cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
+    cfg["algorithm"] = {"method": "awq_lite", "alpha_step": 0.05}
+    secs = end_to_end(w3, x3, cfg)
+    flops = 2 * 512 * 4096 * 4096 * 22
+    out["c3_awq_lite_21_alphas_4096x4096"] = {
+        "end_to_end_ms": round(secs * 1e3, 3), "gemm_flops": flops,
+        "gemm_TFLOPs_over_end_to_end": round(flops / secs / 1e12, 1)}
+    return out
 
 
 def calib_sweep(torch, layers, n_seqs, batch, seq_len=512):
@@ -265,12 +355,15 @@ def main():
         w_ms, d_ms = timed(torch, dequant, a.steps, a.warmup)
         extras["dequantize_one_layer"] = {
             "ms": round(d_ms, 4), "GBps": round(e1 * DEQUANT_BYTES_PER_ELEM / d_ms / 1e6, 1)}
+        with contextlib.redirect_stdout(sys.stderr):   # the calibration algorithms print progress
+            extras["single_tensor_configs"] = single_tensor_configs(torch, a.steps, a.warmup)
         out["extras"] = extras
 
     if not a.no_calib_sweep:
         del weights, aplan, qplan
         torch.cuda.empty_cache()
-        out["calib_sweep"] = calib_sweep(torch, a.layers, a.calib_seqs, a.calib_batch)
+        with contextlib.redirect_stdout(sys.stderr):
+            out["calib_sweep"] = calib_sweep(torch, a.layers, a.calib_seqs, a.calib_batch)
 
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)

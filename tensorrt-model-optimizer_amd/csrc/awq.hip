@@ -336,7 +336,9 @@ extern "C" int mo_sq_diff_sum(const void* a, const void* b, int64_t n, int dtype
     if (n == 0) return MO_OK;
     if (!a || !b || !acc) return MO_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
-    const unsigned g = mo::blocks_for_awq((n + 7) / 8, 1024);
+    // every workgroup ends with one atomic on the same double: 8 chunks per lane before a second
+    // workgroup is worth its atomic, and never more than 1024 of them
+    const unsigned g = mo::blocks_for_awq((n + 63) / 64, 1024);
     const int vec = ((((uintptr_t)a | (uintptr_t)b) & 15u) == 0) ? 1 : 0;
 #define CALL(DT) mo::sq_diff_sum_kernel<DT><<<g, 256, 0, st>>>(a, b, n, vec, acc)
     DISPATCH_DT(dtype, CALL)

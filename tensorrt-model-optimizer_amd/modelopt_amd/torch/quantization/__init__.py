@@ -5,6 +5,7 @@ configs (``NVFP4_DEFAULT_CFG`` ...), ``TensorQuantizer`` under ``nn``.
 """
 
 from . import calib, config, conversion, kernels, model_calib, nn, qtensor, tensor_quant, utils
+from .compress import compress, is_real_quantized
 from .config import *  # noqa: F401,F403
 from .conversion import (register, replace_quant_module, set_quantizer_attribute,
                          set_quantizer_by_cfg, set_quantizer_by_cfg_context, unregister)

@@ -11,7 +11,7 @@ from typing import Any, Literal
 from pydantic import BaseModel, ConfigDict, ValidationInfo, field_validator, model_validator
 
 __all__ = [
-    "QuantizerAttributeConfig", "QuantizeConfig", "MaxCalibConfig", "SmoothQuantCalibConfig",
+    "QuantizerAttributeConfig", "QuantizeConfig", "CompressConfig", "MaxCalibConfig", "SmoothQuantCalibConfig",
     "AWQLiteCalibConfig", "INT8_DEFAULT_CFG", "INT8_SMOOTHQUANT_CFG", "INT8_WEIGHT_ONLY_CFG",
     "FP8_DEFAULT_CFG", "INT4_BLOCKWISE_WEIGHT_ONLY_CFG", "INT4_AWQ_CFG", "W4A8_AWQ_BETA_CFG",
     "FP8_KV_CFG", "NVFP4_DEFAULT_CFG", "NVFP4_AWQ_LITE_CFG", "NVFP4_KV_CFG", "choices",
@@ -209,6 +209,14 @@ class QuantizeConfig(_MappingConfig):
 
     quant_cfg: dict[str, Any] = {"default": {"num_bits": 8, "axis": None}}
     algorithm: Any = "max"
+
+
+class CompressConfig(_MappingConfig):
+    """``compress``: pattern -> compress or not; ``quant_gemm`` is accepted for compatibility
+    (no real-quant GEMM backend exists here).  Reference: config.py:1182-1195."""
+
+    compress: dict[str, bool] = {"*": True}
+    quant_gemm: bool = True
 
 
 _default_disabled_quantizer_cfg = {

@@ -1,10 +1,10 @@
 """Real-quantised tensor containers."""
 
-from .base_qtensor import BaseQuantizedTensor, QTensorWrapper
+from .base_qtensor import BaseQuantizedTensor, QTensorWrapper, pack_real_quantize_weight
 from .fp8_tensor import FP8QTensor
 from .int4_tensor import INT4QTensor
 from .int8_tensor import INT8QTensor
 from .nvfp4_tensor import NVFP4QTensor
 
-__all__ = ["BaseQuantizedTensor", "QTensorWrapper", "FP8QTensor", "INT4QTensor", "INT8QTensor",
+__all__ = ["BaseQuantizedTensor", "QTensorWrapper", "pack_real_quantize_weight", "FP8QTensor", "INT4QTensor", "INT8QTensor",
            "NVFP4QTensor"]

@@ -2,7 +2,7 @@
 
 import torch
 
-__all__ = ["BaseQuantizedTensor", "QTensorWrapper"]
+__all__ = ["BaseQuantizedTensor", "QTensorWrapper", "pack_real_quantize_weight"]
 
 
 class BaseQuantizedTensor:
@@ -50,3 +50,27 @@ class QTensorWrapper(torch.nn.Parameter):
     def get_state(self):
         return {"metadata": self.metadata, "quantized_data.shape": self.data.shape,
                 "quantized_data.dtype": self.data.dtype}
+
+
+def pack_real_quantize_weight(module, force_quantize: bool = False):
+    """Replace the weight of every sub-module whose weight quantizer is enabled and set to real
+    quantisation by its packed form (a ``QTensorWrapper``).  Reference: qtensor/base_qtensor.py
+    :196-229."""
+    from ..nn import SequentialQuantizer  # circular at import time
+
+    def compress(m):
+        w = getattr(m, "weight", None)
+        q = getattr(m, "weight_quantizer", None)
+        if w is None or w.is_meta or q is None:
+            return False
+        if q.is_enabled and not q._fake_quant and w.element_size() > 1:
+            if force_quantize:
+                q._dequantize = False
+            m.weight = QTensorWrapper(q(w))
+            return True
+        return False
+
+    with SequentialQuantizer.convert_to_single_quantizer(module), torch.no_grad():
+        for name, m in module.named_modules():
+            if name != "":
+                compress(m)

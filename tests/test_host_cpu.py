@@ -293,3 +293,15 @@ def test_quantization_format_detection():
         assert equ.get_quantization_format(m) == fmt
     m = _converted(mtq.NVFP4_DEFAULT_CFG)
     assert equ.get_weight_block_size(m.body[0]) == 16 and equ.get_weight_block_size(m.lm_head) == 0
+
+
+def test_compress_surface_without_a_gpu():
+    """Names and config handling of ``mtq.compress`` (the packing itself needs the GPU)."""
+    import modelopt_amd.torch.quantization as mtq
+
+    assert mtq.CompressConfig().compress == {"*": True} and mtq.CompressConfig().quant_gemm is True
+    model = torch.nn.Sequential(torch.nn.Linear(8, 8))
+    assert not mtq.is_real_quantized(model)
+    with pytest.raises(ValueError, match="expected a boolean"):
+        mtq.compress(model, {"*": "yes"})
+    assert issubclass(mtq.nn.RealQuantLinear, mtq.nn.QuantModule)
