@@ -23,7 +23,8 @@ __all__ = [
     "get_weight_scaling_factor", "get_weight_scaling_factor_2", "get_prequant_scaling_factor",
     "get_kv_cache_dtype", "get_weight_block_size", "get_quantization_format",
     "process_layer_quant_config", "pack_int4_in_uint8", "to_quantized_weight",
-    "postprocess_state_dict", "preprocess_linear_fusion", "get_quant_config", "all_items_same",
+    "postprocess_state_dict", "preprocess_linear_fusion", "fuse_prequant_layernorm",
+    "get_quant_config", "all_items_same",
 ]
 
 
@@ -380,6 +381,20 @@ def preprocess_linear_fusion(modules: list[nn.Module], resmooth_only=False):
             amax = torch.max(torch.stack([m.weight_quantizer.amax for m in modules]))
             for m in modules:
                 m.weight_quantizer.amax = amax
+
+
+def fuse_prequant_layernorm(layernorm_module: nn.Module, modules: list[nn.Module]):
+    """Fold the (already shared) input ``pre_quant_scale`` of ``modules`` into the weight and bias
+    of the layernorm that feeds them, and drop it from the modules so that it is not exported
+    (reference: export/quant_utils.py:1104-1129):
+    ``norm(x) * w * s == norm(x) * (w * s)``."""
+    scale = modules[0].input_quantizer._pre_quant_scale
+    layernorm_module.weight = nn.Parameter(layernorm_module.weight * scale)
+    if getattr(layernorm_module, "bias", None) is not None:
+        layernorm_module.bias = nn.Parameter(layernorm_module.bias * scale)
+    for module in modules:
+        delattr(module.input_quantizer, "_pre_quant_scale")
+        module.fused_with_prequant = True
 
 
 def get_quant_config(model: nn.Module) -> dict[str, Any]:

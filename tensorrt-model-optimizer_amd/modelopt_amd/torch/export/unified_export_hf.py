@@ -20,12 +20,15 @@ from ..quantization.nn import SequentialQuantizer, TensorQuantizer
 from ..quantization.qtensor import NVFP4QTensor
 from ..quantization.utils import is_quantized_linear, true_divide
 from .model_config import *  # noqa: F403
-from .quant_utils import (get_activation_scaling_factor, get_quant_config, get_quantization_format,
+from ..quantization.conversion import set_quantizer_by_cfg_context
+from .quant_utils import (fuse_prequant_layernorm, get_activation_scaling_factor, get_quant_config,
+                          get_quantization_format,
                           get_weight_block_size, get_weight_scaling_factor,
                           get_weight_scaling_factor_2, postprocess_state_dict,
                           preprocess_linear_fusion, to_quantized_weight)
 
-__all__ = ["export_hf_checkpoint", "convert_hf_quant_config_format"]
+__all__ = ["export_hf_checkpoint", "convert_hf_quant_config_format",
+           "requantize_resmooth_fused_llm_layers"]
 
 
 def _register_input_scale(module, input_quantizer):
@@ -97,12 +100,70 @@ def _fusable_groups(model: nn.Module):
                 yield group
 
 
+def _is_layernorm(module: nn.Module) -> bool:
+    return any(n in type(module).__name__ for n in ("LayerNorm", "RMSNorm"))
+
+
+def _quantizer_on(q) -> bool:
+    if isinstance(q, SequentialQuantizer):
+        return any(m.is_enabled for m in q)
+    return isinstance(q, TensorQuantizer) and q.is_enabled
+
+
+def requantize_resmooth_fused_llm_layers(model: nn.Module):
+    """Unify what an inference engine will fuse (reference: unified_export_hf.py:90-231).
+
+    Quantised linears that read the same tensor (q/k/v, gate/up) are found with forward hooks
+    during one two-token dummy forward with every quantizer switched off; each group gets one
+    averaged ``pre_quant_scale`` (weights re-smoothed), one input amax and one per-tensor weight
+    amax.  For AWQ formats, when the shared input is the output of a layernorm, the scale is
+    folded into the layernorm weight.  A model that cannot run on token ids falls back to
+    grouping by the usual projection names (no layernorm folding).
+    """
+    input_to_linear: dict = {}
+    output_to_layernorm: dict = {}
+
+    def linear_hook(module, args, output):
+        input_to_linear.setdefault(args[0], []).append(module)
+
+    def norm_hook(module, args, output):
+        output_to_layernorm[output] = module
+
+    handles = []
+    for module in model.modules():
+        if _is_layernorm(module):
+            handles.append(module.register_forward_hook(norm_hook))
+        elif is_quantized_linear(module) and (_quantizer_on(module.input_quantizer)
+                                              or _quantizer_on(module.weight_quantizer)):
+            handles.append(module.register_forward_hook(linear_hook))
+    groups = None
+    try:
+        device = next(model.parameters()).device
+        with torch.no_grad(), set_quantizer_by_cfg_context(model, {"*": {"enable": False}}):
+            model(torch.ones([1, 2], dtype=torch.long, device=device))
+        groups = list(input_to_linear.items())
+    except Exception as err:  # noqa: BLE001 -- any failure of a foreign forward means "not an LLM"
+        warnings.warn(f"dummy forward for layer fusion failed ({type(err).__name__}: {err}); "
+                      "grouping q/k/v and gate/up projections by name")
+    finally:
+        for h in handles:
+            h.remove()
+    if groups is None:
+        groups = [(None, g) for g in _fusable_groups(model)]
+    for tensor, modules in groups:
+        fmt = get_quantization_format(modules[0])
+        if len(modules) > 1 and fmt not in (QUANTIZATION_FP8, QUANTIZATION_NONE):
+            preprocess_linear_fusion(modules)
+        if (fmt is not QUANTIZATION_NONE and fmt is not None and "awq" in fmt and tensor is not None
+                and tensor in output_to_layernorm
+                and modules[0].input_quantizer.pre_quant_scale is not None):
+            fuse_prequant_layernorm(output_to_layernorm[tensor], modules)
+
+
 def _export_hf_checkpoint(model: nn.Module, dtype: torch.dtype | None = None):
     if dtype is None:
         dtype = next(model.parameters()).dtype
-    for group in _fusable_groups(model):
-        if get_quantization_format(group[0]) != QUANTIZATION_NONE:
-            preprocess_linear_fusion(group)
+    requantize_resmooth_fused_llm_layers(model)
     quant_config = get_quant_config(model)
     kv_format = quant_config["quantization"]["kv_cache_quant_algo"]
     kv_bound = {KV_CACHE_NVFP4: 6 * 448, KV_CACHE_FP8: 448}.get(kv_format, 0)

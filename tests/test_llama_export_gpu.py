@@ -109,10 +109,17 @@ def test_int4_awq_export(tmp_path):
     amax = lin.weight_quantizer.export_amax().cpu()
     assert amax.shape == (128, 2)
     state, qcfg = export_hf_checkpoint(model, export_dir=tmp_path)
-    # q/k/v (and gate/up) were re-smoothed to one shared input scale
-    attn = model.get_submodule("model.layers.0.self_attn")
-    assert torch.equal(attn.q_proj.input_quantizer._pre_quant_scale, attn.k_proj.input_quantizer._pre_quant_scale)
-    assert torch.equal(attn.q_proj.input_quantizer._pre_quant_scale, attn.v_proj.input_quantizer._pre_quant_scale)
+    # q/k/v (and gate/up) were re-smoothed to one shared input scale, which then went into the
+    # layernorm in front of them: no pre_quant_scale is exported for those five projections
+    layer = model.get_submodule("model.layers.0")
+    for lin_ in (layer.self_attn.q_proj, layer.self_attn.k_proj, layer.self_attn.v_proj,
+                 layer.mlp.gate_proj, layer.mlp.up_proj):
+        assert not hasattr(lin_.input_quantizer, "_pre_quant_scale") and lin_.fused_with_prequant
+    for proj in ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "mlp.gate_proj", "mlp.up_proj"):
+        assert f"model.layers.0.{proj}.pre_quant_scale" not in state
+    assert "model.layers.0.self_attn.o_proj.pre_quant_scale" in state
+    assert not torch.equal(state["model.layers.0.input_layernorm.weight"].cpu(),
+                           w["model.layers.0.input_layernorm.weight"])
     q = qcfg["quantization"]
     assert q["quant_algo"] == "W4A16_AWQ" and q["group_size"] == 128 and q["pre_quant_scale"] is True
     name = "model.layers.0.mlp.down_proj"
@@ -121,3 +128,32 @@ def test_int4_awq_export(tmp_path):
     assert_bits_equal(state[name + ".weight"].cpu(), oexport.pack_int4_in_uint8(w_folded, ws), "packed int4")
     assert state[name + ".weight"].shape == (64, 256)
     assert state[name + ".pre_quant_scale"].shape == (256,)
+
+
+def test_fusion_pre_pass_keeps_the_model_function():
+    """Shared scales, re-smoothed weights and the fold into the layernorm change how the
+    computation is written, not what it computes (up to bf16 rounding of the folded weights)."""
+    from modelopt_amd.torch.export import requantize_resmooth_fused_llm_layers
+
+    model, w = _quantized(copy.deepcopy(mtq.INT4_AWQ_CFG))
+    ids = _ids(1)[0].to(DEV)
+    attn = model.get_submodule("model.layers.1.self_attn")
+    pqs = [p.input_quantizer._pre_quant_scale.float().cpu() for p in (attn.q_proj, attn.k_proj, attn.v_proj)]
+    norm_w = model.get_submodule("model.layers.1.input_layernorm").weight.detach().float().cpu()
+    off = {"*": {"enable": False}}     # a disabled quantizer still applies its pre_quant_scale
+    with torch.no_grad(), mtq.set_quantizer_by_cfg_context(model, off):
+        before = model(ids).float()
+    requantize_resmooth_fused_llm_layers(model)
+    with torch.no_grad(), mtq.set_quantizer_by_cfg_context(model, off):
+        after = model(ids).float()
+    rel = (after - before).norm() / before.norm()
+    assert float(rel) < 0.02          # bf16 rounding of the re-smoothed and folded weights
+    avg = torch.stack(pqs).mean(0).to(torch.bfloat16).float()
+    got = model.get_submodule("model.layers.1.input_layernorm").weight.detach().float().cpu()
+    assert torch.allclose(got, (norm_w.to(torch.bfloat16) * avg.to(torch.bfloat16)).float(), rtol=2 ** -7)
+    # o_proj and down_proj read tensors no layernorm produced: their scales stay
+    assert hasattr(attn.o_proj.input_quantizer, "_pre_quant_scale")
+    # the block amax of a re-smoothed weight was recalibrated on the new weight
+    k = attn.k_proj
+    want = reduce.reduce_amax(k.weight.data.cpu().reshape(-1, 128), axis=[1], keepdims=True)
+    assert_bits_equal(k.weight_quantizer.amax.cpu().reshape(want.shape), want, "recalibrated amax")
