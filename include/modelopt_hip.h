@@ -110,6 +110,25 @@ int mo_nvfp4_qdq(const void* x, void* y, int64_t rows, int64_t k, int dtype, con
 
 /* ------------------------------------------------------------------ real quantize + pack */
 
+/* Block floating point quantize-dequantize of x[rows, k]: blocks of `block_size` (8, 16 or 32)
+ * along k (zero padded), one shared scale per block, every element
+ * sign(x) * format(|x| * scale) * unscale.  Replaces fused_amax_convert(inputs, block_size,
+ * format, scale_format, global_amax) (TQ/src/tensor_quant_mx.cu:355-386; arithmetic :35-57,
+ * :97-186; element tables TQ/src/tensor_quant_mx.h:38-178), the kernel behind the MXFP8 / MXFP6 /
+ * MXFP4 / MXINT8 configs (TQ/tensor_quant.py:158-198).  The enum follows the reference's Types.
+ *   scale_format MO_EF_E8M0, global_amax NULL: unscale = 2^ceil(log2(amax / format_max));
+ *   other scale_format, global_amax NULL: unscale = scale_format(amax / format_max), in double;
+ *   global_amax given (n_global_amax = 1, or = rows for one per row): the two-level scale of
+ *   compute_scale_with_global.  All fp32 steps are IEEE (the reference kernel is built with
+ *   --use_fast_math); zero and NaN inputs give a non-negative result. */
+enum mo_elem_format {
+    MO_EF_E4M3 = 0, MO_EF_E5M2 = 1, MO_EF_INT8 = 2, MO_EF_E0M3 = 3, MO_EF_E1M2 = 4,
+    MO_EF_E3M0 = 5, MO_EF_E2M1 = 6, MO_EF_E3M2 = 7, MO_EF_E2M3 = 8, MO_EF_E8M0 = 9
+};
+int mo_block_fp_qdq(const void* x, void* y, int64_t rows, int64_t k, int dtype, int block_size,
+                    int format, int scale_format, const float* global_amax,
+                    int64_t n_global_amax, void* stream);
+
 /* NVFP4 quantize + pack.  Replaces NVFP4QTensor.quantize and get_weights_scaling_factor
  * (TQ/qtensor/nvfp4_tensor.py:63-92,143-232) as called by to_quantized_weight
  * (modelopt/torch/export/quant_utils.py:822-834) and TensorQuantizer._real_quantize

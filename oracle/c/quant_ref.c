@@ -268,3 +268,134 @@ void qr_real_quantize(const void* x, int64_t n, int dtype, float scale, int via,
         }
     }
 }
+
+/* ------------------------------------------------------------------ block floating point (MX)
+ * fused_amax_convert, TQ/src/tensor_quant_mx.cu:35-57,97-186,243-297 with the tables and
+ * conversions of TQ/src/tensor_quant_mx.h:38-178, in IEEE fp32 / double (the reference kernel is
+ * built with --use_fast_math).  Format numbers follow the reference's enum Types. */
+enum { QR_E4M3 = 0, QR_E5M2, QR_INT8, QR_E0M3, QR_E1M2, QR_E3M0, QR_E2M1, QR_E3M2, QR_E2M3, QR_E8M0 };
+
+static const float t_e2m1[8] = {0, 0.5f, 1, 1.5f, 2, 3, 4, 6};
+static const float b_e2m1[7] = {0.25f, 0.75f, 1.25f, 1.75f, 2.5f, 3.5f, 5};
+static const float t_e1m2[8] = {0, 0.5f, 1, 1.5f, 2, 2.5f, 3, 3.5f};
+static const float b_e1m2[7] = {0.25f, 0.75f, 1.25f, 1.75f, 2.25f, 2.75f, 3.25f};
+static const float t_e0m3[8] = {0, 1, 2, 3, 4, 5, 6, 7};
+static const float b_e0m3[7] = {0.5f, 1.5f, 2.5f, 3.5f, 4.5f, 5.5f, 6.5f};
+static const float t_e3m0[8] = {0, 0.25f, 0.5f, 1, 2, 4, 8, 16};
+static const float b_e3m0[7] = {0.125f, 0.375f, 0.75f, 1.5f, 3, 6, 12};
+static const float t_e3m2[32] = {0, 0.0625f, 0.125f, 0.1875f, 0.25f, 0.3125f, 0.375f, 0.4375f,
+                                 0.5f, 0.625f, 0.75f, 0.875f, 1, 1.25f, 1.5f, 1.75f,
+                                 2, 2.5f, 3, 3.5f, 4, 5, 6, 7, 8, 10, 12, 14, 16, 20, 24, 28};
+static const float t_e2m3[32] = {0, 0.125f, 0.25f, 0.375f, 0.5f, 0.625f, 0.75f, 0.875f, 1, 1.125f,
+                                 1.25f, 1.375f, 1.5f, 1.625f, 1.75f, 1.875f, 2, 2.25f, 2.5f, 2.75f,
+                                 3, 3.25f, 3.5f, 3.75f, 4, 4.5f, 5, 5.5f, 6, 6.5f, 7, 7.5f};
+
+/* nearest table value; a tie goes to the value with the even index, or up when ties_away */
+static float table_round(float x, const float* values, const float* bounds, int n, int ties_away) {
+    float sign = 1.0f;
+    if (x < 0.0f) { sign = -1.0f; x = -x; }
+    if (isinf(x) || isnan(x)) return sign * values[n - 1];
+    for (int i = 0; i < n - 1; ++i) {
+        const float bound = bounds ? bounds[i] : 0.5f * (values[i] + values[i + 1]);
+        if (x < bound) return sign * values[i];
+        if (x == bound) return sign * ((ties_away || (i & 1)) ? values[i + 1] : values[i]);
+    }
+    return sign * values[n - 1];
+}
+
+/* fp32 -> E5M2 value (round to nearest even, subnormals kept, saturating at 57344) */
+static float round_e5m2_sat(float f) {
+    uint32_t u = f2u(f), sign = u & 0x80000000u, a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return f;
+    float m = u2f(a);
+    if (m > 57344.0f) m = 57344.0f;
+    if (m < 6.103515625e-05f) {                                  /* below 2^-14: quantum 2^-16 */
+        m = (m + 128.0f) - 128.0f;                               /* 2^7 aligns 2^-16 to bit 0 */
+    } else {
+        uint32_t b = f2u(m);
+        b = (b + 0xFFFFFu + ((b >> 21) & 1u)) & 0xFFE00000u;     /* keep 2 mantissa bits */
+        m = u2f(b);
+        if (m > 57344.0f) m = 57344.0f;
+    }
+    return u2f(f2u(m) | sign);
+}
+
+float qr_convert_to_types(float x, int fmt) {
+    switch (fmt) {
+        case QR_E4M3: {
+            if (x != x) return x;
+            float c = x > 448.0f ? 448.0f : (x < -448.0f ? -448.0f : x);
+            return qr_e4m3_to_f32(qr_f32_to_e4m3(c));
+        }
+        case QR_E5M2: return round_e5m2_sat(x);
+        case QR_INT8: {
+            float q = nearbyintf(x);
+            return q > 127.0f ? 127.0f : (q < -127.0f ? -127.0f : q);
+        }
+        case QR_E2M1: return table_round(x, t_e2m1, b_e2m1, 8, 0);
+        case QR_E0M3: return table_round(x, t_e0m3, b_e0m3, 8, 0);
+        case QR_E1M2: return table_round(x, t_e1m2, b_e1m2, 8, 0);
+        case QR_E3M0: return table_round(x, t_e3m0, b_e3m0, 8, 1);
+        case QR_E3M2: return table_round(x, t_e3m2, NULL, 32, 0);
+        case QR_E2M3: return table_round(x, t_e2m3, NULL, 32, 0);
+        default: return 0.0f;
+    }
+}
+
+static float format_max(int fmt) {
+    static const float m[9] = {448.0f, 57344.0f, 127.0f, 7.0f, 3.5f, 16.0f, 6.0f, 28.0f, 7.5f};
+    return fmt >= 0 && fmt < 9 ? m[fmt] : 0.0f;
+}
+
+/* x [rows, k]; blocks of `block` along k, zero padded; global_amax NULL, one value
+ * (n_global == 1) or one per row (n_global == rows). */
+void qr_block_fp_qdq(const void* x, int64_t rows, int64_t k, int dtype, int block, int fmt,
+                     int scale_fmt, const float* global_amax, int64_t n_global, void* y) {
+    const int64_t nb = (k + block - 1) / block;
+    for (int64_t r = 0; r < rows; ++r) {
+        for (int64_t b = 0; b < nb; ++b) {
+            float amax = 0.0f;
+            for (int j = 0; j < block; ++j) {
+                const int64_t c = b * block + j;
+                float a = c < k ? fabsf(load_as_f32(x, r * k + c, dtype)) : 0.0f;
+                if (a > 3.402823466e+38f) a = 3.402823466e+38f;      /* clamp, :192 */
+                amax = fmaxf(amax, a);                               /* drops NaN */
+            }
+            float scale = 1.0f, unscale = 1.0f;
+            const int bad_local = amax == 0.0f || isinf(amax) || isnan(amax);
+            if (global_amax) {
+                const float g = global_amax[n_global == rows && n_global > 1 ? r : 0];
+                if (!(bad_local || g == 0.0f || isinf(g) || isnan(g))) {
+                    const float fmax = format_max(fmt), smax = format_max(scale_fmt);
+                    const float local_unscale = amax / fmax;
+                    const double two_level = (double)smax * (double)(fmax / g);
+                    const double q = (double)qr_convert_to_types((float)(local_unscale * two_level),
+                                                                 scale_fmt) / two_level;
+                    scale = (float)(1.0 / q);
+                    unscale = (float)q;
+                }
+            } else if (!bad_local) {
+                if (scale_fmt == QR_E8M0) {
+                    const float ratio = amax / format_max(fmt);
+                    const uint32_t bits = f2u(ratio), ef = (bits >> 23) & 0xFFu, mant = bits & 0x7FFFFFu;
+                    const int e = (mant > 0 && ef != 0xFEu && !(ef == 0 && mant <= 0x400000u))
+                                      ? (int)ef - 126 : (int)ef - 127;
+                    scale = ldexpf(1.0f, -e);
+                    unscale = ldexpf(1.0f, e);
+                } else {
+                    double s = (double)format_max(fmt) / (double)amax;
+                    const double inv = (double)qr_convert_to_types((float)(1.0 / s), scale_fmt);
+                    scale = (float)(1.0 / inv);
+                    unscale = (float)inv;
+                }
+            }
+            for (int j = 0; j < block; ++j) {
+                const int64_t c = b * block + j;
+                if (c >= k) break;
+                const float v = load_as_f32(x, r * k + c, dtype);
+                const float q = qr_convert_to_types(fabsf(v) * scale, fmt) * unscale;
+                store_from_f32(y, r * k + c, dtype, v < 0.0f ? -q : q);
+            }
+        }
+    }
+}

@@ -40,6 +40,9 @@ def load():
         lib.qr_int_qdq.argtypes = [_P, _I64, _I, _F, _I, _I, _I, _P]
         lib.qr_int4_block_quantize.argtypes = [_P, _I64, _I, _I, _P, _P]
         lib.qr_real_quantize.argtypes = [_P, _I64, _I, _F, _I, _I, _P]
+        lib.qr_convert_to_types.argtypes, lib.qr_convert_to_types.restype = [_F, _I], _F
+        lib.qr_block_fp_qdq.argtypes = [_P, _I64, _I64, _I, _I, _I, _I, _P, _I64, _P]
+        lib.qr_block_fp_qdq.restype = None
         for name in ("qr_nvfp4_quantize", "qr_nvfp4_dequantize", "qr_fp8_qdq", "qr_int_qdq",
                      "qr_int4_block_quantize", "qr_real_quantize"):
             getattr(lib, name).restype = None
@@ -120,3 +123,19 @@ def real_quantize(x, scale, via_dtype, fmt):
     load().qr_real_quantize(x.data_ptr(), x.numel(), _DT[x.dtype], float(scale), _DT[via_dtype],
                             0 if fmt == "e4m3" else 1, out.data_ptr())
     return out.view(torch.float8_e4m3fn if fmt == "e4m3" else torch.int8)
+
+
+FORMATS = ["E4M3", "E5M2", "INT8", "E0M3", "E1M2", "E3M0", "E2M1", "E3M2", "E2M3", "E8M0"]
+
+
+def block_fp_fake_quant(x, block_size, fmt, scale_fmt="E8M0", global_amax=None):
+    """C twin of ``oracle.mx.block_fp_fake_quant``."""
+    x = _cpu(x)
+    k = x.shape[-1]
+    rows = x.numel() // k
+    y = torch.empty_like(x)
+    g = None if global_amax is None else global_amax.to(torch.float32).reshape(-1).contiguous()
+    load().qr_block_fp_qdq(x.data_ptr(), rows, k, _DT[x.dtype], block_size, FORMATS.index(fmt),
+                           FORMATS.index(scale_fmt), None if g is None else g.data_ptr(),
+                           0 if g is None else g.numel(), y.data_ptr())
+    return y

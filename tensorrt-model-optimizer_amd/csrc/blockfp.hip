@@ -1,0 +1,227 @@
+// Block floating point fake quantisation for gfx950: the MX formats (elements E4M3 / E5M2 / E3M2 /
+// E2M3 / E2M1 / INT8 ... with one shared power-of-two E8M0 scale per block) and the two-level
+// variant with a minifloat block scale under a global abs-max.
+//
+// HBM-bound: one read and one write of the tensor (4 bytes per bf16 element).  A lane owns a
+// chunk of 8 elements, the 1, 2 or 4 lanes of a block combine their abs-max with DPP moves; one
+// workgroup per tile of 1024 chunks, the loads of a lane's 4 chunks issued before the math.
+#include "common.h"
+
+namespace mo {
+
+// Nearest value of a small float format with M mantissa bits whose smallest normal number is
+// 2^EMIN (below it the quantum stays 2^(EMIN - M)), saturating at fmax; `a` is non-negative,
+// infinities and NaN give fmax.  Ties go to the even multiple of the quantum -- the value with
+// the even index in the reference's tables -- or away from zero when TIES_AWAY.
+template <int M, int EMIN, bool TIES_AWAY>
+__device__ __forceinline__ float round_minifloat(float a, float fmax) {
+    if (!(a < __builtin_inff())) return fmax;
+    int e = (int)(f2u(a) >> 23) - 127;
+    e = e > EMIN ? e : EMIN;
+    const float t = __builtin_ldexpf(a, M - e);
+    const float r = TIES_AWAY ? __builtin_floorf(t + 0.5f) : __builtin_rintf(t);
+    const float v = __builtin_ldexpf(r, e - M);
+    return v < fmax ? v : fmax;
+}
+
+// E5M2: round to nearest even with subnormals (quantum 2^-16), saturating at 57344; NaN stays.
+__device__ __forceinline__ float round_e5m2_sat(float a) {
+    if (a != a) return a;
+    a = a < 57344.0f ? a : 57344.0f;
+    int e = (int)(f2u(a) >> 23) - 127;
+    e = e > -14 ? e : -14;
+    const float v = __builtin_ldexpf(__builtin_rintf(__builtin_ldexpf(a, 2 - e)), e - 2);
+    return v < 57344.0f ? v : 57344.0f;
+}
+
+template <int FMT>
+__device__ __forceinline__ float convert_elem(float a) {  // a >= 0 (or NaN)
+    if constexpr (FMT == MO_EF_E4M3) return round_e4m3<true>(a);
+    else if constexpr (FMT == MO_EF_E5M2) return round_e5m2_sat(a);
+    else if constexpr (FMT == MO_EF_INT8) {
+        const float q = __builtin_rintf(a);
+        return q > 127.0f ? 127.0f : q;  // NaN stays NaN
+    }
+    else if constexpr (FMT == MO_EF_E0M3) return round_minifloat<3, 3, false>(a, 7.0f);
+    else if constexpr (FMT == MO_EF_E1M2) return round_minifloat<2, 1, false>(a, 3.5f);
+    else if constexpr (FMT == MO_EF_E3M0) return round_minifloat<0, -2, true>(a, 16.0f);
+    else if constexpr (FMT == MO_EF_E2M1) return round_minifloat<1, 0, false>(a, 6.0f);
+    else if constexpr (FMT == MO_EF_E3M2) return round_minifloat<2, -2, false>(a, 28.0f);
+    else return round_minifloat<3, 0, false>(a, 7.5f);  // E2M3
+}
+
+__device__ __forceinline__ float convert_runtime(float a, int fmt) {
+    switch (fmt) {
+        case MO_EF_E4M3: return convert_elem<MO_EF_E4M3>(a);
+        case MO_EF_E5M2: return convert_elem<MO_EF_E5M2>(a);
+        case MO_EF_INT8: return convert_elem<MO_EF_INT8>(a);
+        case MO_EF_E0M3: return convert_elem<MO_EF_E0M3>(a);
+        case MO_EF_E1M2: return convert_elem<MO_EF_E1M2>(a);
+        case MO_EF_E3M0: return convert_elem<MO_EF_E3M0>(a);
+        case MO_EF_E2M1: return convert_elem<MO_EF_E2M1>(a);
+        case MO_EF_E3M2: return convert_elem<MO_EF_E3M2>(a);
+        default: return convert_elem<MO_EF_E2M3>(a);
+    }
+}
+
+__host__ __device__ __forceinline__ float elem_format_max(int fmt) {
+    switch (fmt) {
+        case MO_EF_E4M3: return 448.0f;
+        case MO_EF_E5M2: return 57344.0f;
+        case MO_EF_INT8: return 127.0f;
+        case MO_EF_E0M3: return 7.0f;
+        case MO_EF_E1M2: return 3.5f;
+        case MO_EF_E3M0: return 16.0f;
+        case MO_EF_E2M1: return 6.0f;
+        case MO_EF_E3M2: return 28.0f;
+        default: return 7.5f;
+    }
+}
+
+struct BlockScale { float scale, unscale; };
+
+// amax: block abs-max with |x| clamped to FLT_MAX and NaN elements ignored.
+template <int FMT>
+__device__ __forceinline__ BlockScale block_scale(float amax, int scale_fmt, bool has_global,
+                                                  float global_amax) {
+    BlockScale s = {1.0f, 1.0f};
+    if (amax == 0.0f) return s;  // finite by construction
+    const float fmax = elem_format_max(FMT);
+    if (has_global) {
+        // two-level scale: the block's unscale, quantised to scale_fmt relative to the global amax
+        if (global_amax == 0.0f || !(__builtin_fabsf(global_amax) < __builtin_inff())) return s;
+        const float smax = elem_format_max(scale_fmt);
+        const float local_unscale = amax / fmax;
+        const double two_level = (double)smax * (double)(fmax / global_amax);
+        const double q = (double)convert_runtime((float)((double)local_unscale * two_level), scale_fmt) /
+                         two_level;
+        s.scale = (float)(1.0 / q);
+        s.unscale = (float)q;
+    } else if (scale_fmt == MO_EF_E8M0) {
+        // unscale = 2^ceil(log2(amax / fmax)), read off the bits of the fp32 quotient
+        const uint32_t bits = f2u(amax / fmax), ef = (bits >> 23) & 0xFFu, mant = bits & 0x7FFFFFu;
+        const int e = (mant > 0 && ef != 0xFEu && !(ef == 0 && mant <= 0x400000u)) ? (int)ef - 126
+                                                                                   : (int)ef - 127;
+        s.scale = __builtin_ldexpf(1.0f, -e);
+        s.unscale = __builtin_ldexpf(1.0f, e);
+    } else {
+        const double sc = (double)fmax / (double)amax;
+        const double inv = (double)convert_runtime((float)(1.0 / sc), scale_fmt);
+        s.scale = (float)(1.0 / inv);
+        s.unscale = (float)inv;
+    }
+    return s;
+}
+
+constexpr int kBlockFpTileChunks = 1024;
+
+// x viewed as [rows, kp] chunks with kp = k rounded up to whole blocks (zero padded).
+template <int DT, int FMT, bool FLAT>
+__global__ __launch_bounds__(256) void block_fp_qdq_kernel(
+    const void* __restrict__ x, void* __restrict__ y, int64_t total_chunks, int64_t k, int64_t cpr,
+    int lg_g, int scale_fmt, const float* __restrict__ global_amax, int per_row) {
+    const int64_t c0 = (int64_t)blockIdx.x * kBlockFpTileChunks + threadIdx.x;
+    float v[4][8];
+    int64_t base[4], col[4], row[4];
+    RawChunk<DT> raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        base[u] = col[u] = row[u] = 0;
+        zero_raw<DT>(raw[u]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[u][j] = 0.0f;
+        if (c < total_chunks) {
+            if (total_chunks <= 0xFFFFFFFFll) row[u] = (uint32_t)c / (uint32_t)cpr;
+            else row[u] = c / cpr;
+            if constexpr (FLAT) {
+                col[u] = c << 3;
+                load_raw<DT>(x, col[u], raw[u]);
+            } else {
+                col[u] = (c - row[u] * cpr) << 3;
+                base[u] = row[u] * k;
+                load_chunk_guarded<DT>(x, base[u], col[u], k, v[u]);
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const bool live = c0 + u * 256 < total_chunks;
+        if constexpr (FLAT) unpack_raw<DT>(raw[u], v[u]);
+        uint32_t m = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            uint32_t t = f2u(v[u][j]) & 0x7FFFFFFFu;
+            t = t > 0x7F800000u ? 0u : (t < 0x7F7FFFFFu ? t : 0x7F7FFFFFu);  // drop NaN, clamp inf
+            m = t > m ? t : m;
+        }
+        m = group_max_u32(m, lg_g);  // total_chunks is a multiple of the group size
+        if (!live) continue;
+        float g = 0.0f;
+        if (global_amax) g = global_amax[per_row ? row[u] : 0];
+        const BlockScale s = block_scale<FMT>(u2f(m), scale_fmt, global_amax != nullptr, g);
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float q = convert_elem<FMT>(__builtin_fabsf(v[u][j]) * s.scale) * s.unscale;
+            o[j] = v[u][j] < 0.0f ? -q : q;
+        }
+        if constexpr (FLAT) store_chunk<DT>(y, col[u], o);
+        else store_chunk_guarded<DT>(y, base[u], col[u], k, o);
+    }
+}
+
+template <int DT, int FMT>
+static void launch_block_fp(const void* x, void* y, int64_t rows, int64_t k, int64_t kp, int lg_g,
+                            int scale_fmt, const float* global_amax, int per_row, hipStream_t s) {
+    const int64_t cpr = kp / 8, total = rows * cpr;
+    const unsigned grid = (unsigned)((total + kBlockFpTileChunks - 1) / kBlockFpTileChunks);
+    const bool flat = (k == kp) && ((((uintptr_t)x | (uintptr_t)y) & 15u) == 0);
+    if (flat)
+        block_fp_qdq_kernel<DT, FMT, true><<<grid, 256, 0, s>>>(x, y, total, k, cpr, lg_g, scale_fmt,
+                                                                global_amax, per_row);
+    else
+        block_fp_qdq_kernel<DT, FMT, false><<<grid, 256, 0, s>>>(x, y, total, k, cpr, lg_g, scale_fmt,
+                                                                 global_amax, per_row);
+}
+
+}  // namespace mo
+
+extern "C" int mo_block_fp_qdq(const void* x, void* y, int64_t rows, int64_t k, int dtype,
+                               int block_size, int format, int scale_format,
+                               const float* global_amax, int64_t n_global_amax, void* stream) {
+    if (rows < 0 || k < 0) return MO_ERR_ARG;
+    if (block_size != 8 && block_size != 16 && block_size != 32) return MO_ERR_UNSUPPORTED;
+    if (format < MO_EF_E4M3 || format > MO_EF_E2M3) return MO_ERR_UNSUPPORTED;
+    if (scale_format < MO_EF_E4M3 || scale_format > MO_EF_E8M0) return MO_ERR_UNSUPPORTED;
+    if (global_amax && scale_format == MO_EF_E8M0) return MO_ERR_UNSUPPORTED;
+    if (global_amax && n_global_amax != 1 && n_global_amax != rows) return MO_ERR_ARG;
+    if (rows == 0 || k == 0) return MO_OK;
+    if (!x || !y) return MO_ERR_ARG;
+    const int64_t kp = (k + block_size - 1) / block_size * block_size;
+    if ((rows * (kp / 8) + mo::kBlockFpTileChunks - 1) / mo::kBlockFpTileChunks > 0x7FFFFFFF)
+        return MO_ERR_UNSUPPORTED;
+    const int lg_g = block_size == 8 ? 0 : (block_size == 16 ? 1 : 2);
+    const int per_row = global_amax && n_global_amax == rows && rows > 1;
+    hipStream_t s = (hipStream_t)stream;
+#define CALL_FMT(DT)                                                                                  \
+    switch (format) {                                                                                 \
+        case MO_EF_E4M3: mo::launch_block_fp<DT, MO_EF_E4M3>(x, y, rows, k, kp, lg_g, scale_format, global_amax, per_row, s); break; \
+        case MO_EF_E5M2: mo::launch_block_fp<DT, MO_EF_E5M2>(x, y, rows, k, kp, lg_g, scale_format, global_amax, per_row, s); break; \
+        case MO_EF_INT8: mo::launch_block_fp<DT, MO_EF_INT8>(x, y, rows, k, kp, lg_g, scale_format, global_amax, per_row, s); break; \
+        case MO_EF_E0M3: mo::launch_block_fp<DT, MO_EF_E0M3>(x, y, rows, k, kp, lg_g, scale_format, global_amax, per_row, s); break; \
+        case MO_EF_E1M2: mo::launch_block_fp<DT, MO_EF_E1M2>(x, y, rows, k, kp, lg_g, scale_format, global_amax, per_row, s); break; \
+        case MO_EF_E3M0: mo::launch_block_fp<DT, MO_EF_E3M0>(x, y, rows, k, kp, lg_g, scale_format, global_amax, per_row, s); break; \
+        case MO_EF_E2M1: mo::launch_block_fp<DT, MO_EF_E2M1>(x, y, rows, k, kp, lg_g, scale_format, global_amax, per_row, s); break; \
+        case MO_EF_E3M2: mo::launch_block_fp<DT, MO_EF_E3M2>(x, y, rows, k, kp, lg_g, scale_format, global_amax, per_row, s); break; \
+        default: mo::launch_block_fp<DT, MO_EF_E2M3>(x, y, rows, k, kp, lg_g, scale_format, global_amax, per_row, s); break;         \
+    }
+    switch (dtype) {
+        case MO_F32: CALL_FMT(MO_F32); break;
+        case MO_F16: CALL_FMT(MO_F16); break;
+        case MO_BF16: CALL_FMT(MO_BF16); break;
+        default: return MO_ERR_DTYPE;
+    }
+#undef CALL_FMT
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}

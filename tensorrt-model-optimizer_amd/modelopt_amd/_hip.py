@@ -29,6 +29,7 @@ SIGNATURES = {
     "mo_fp8_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _P],
     "mo_int_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _INT, _P],
     "mo_nvfp4_qdq": [_P, _P, _I64, _I64, _INT, _P, _INT, _INT, _INT, _P],
+    "mo_block_fp_qdq": [_P, _P, _I64, _I64, _INT, _INT, _INT, _INT, _P, _I64, _P],
     "mo_nvfp4_quantize": [_P, _I64, _I64, _INT, _INT, _P, _INT, _P, _P, _P, _P, _P],
     "mo_nvfp4_dequantize": [_P, _P, _P, _I64, _I64, _INT, _P, _INT, _P],
     "mo_real_quantize": [_P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _P, _P],
@@ -139,6 +140,31 @@ def nvfp4_qdq(x, amax, block_size=16, mode=0, out=None):
     y = torch.empty_like(x) if out is None else out
     call("mo_nvfp4_qdq", x, _ptr(x), _ptr(y), rows, k, dtype_code(x.dtype), _ptr(amax),
          dtype_code(amax.dtype), block_size, mode, _stream(x))
+    return y
+
+
+ELEM_FORMATS = ["E4M3", "E5M2", "INT8", "E0M3", "E1M2", "E3M0", "E2M1", "E3M2", "E2M3", "E8M0"]
+
+
+def block_fp_qdq(x, block_size, fmt, scale_fmt="E8M0", global_amax=None, out=None):
+    """Block floating point fake quantisation along the last dim (``fused_amax_convert``).
+    ``fmt`` / ``scale_fmt``: names or indices of ``ELEM_FORMATS``; ``global_amax``: None, one
+    fp32 element, or one per row of a 2-D ``x``."""
+    _require_device(x, global_amax)
+    assert x.is_contiguous()
+    fmt = ELEM_FORMATS.index(fmt) if isinstance(fmt, str) else int(fmt)
+    scale_fmt = ELEM_FORMATS.index(scale_fmt) if isinstance(scale_fmt, str) else int(scale_fmt)
+    k = x.shape[-1]
+    rows = x.numel() // k if k else 0
+    y = torch.empty_like(x) if out is None else out
+    n_global = 0
+    if global_amax is not None:
+        assert global_amax.dtype == torch.float32 and global_amax.is_contiguous()
+        n_global = global_amax.numel()
+        if not (n_global == 1 or (x.dim() == 2 and n_global == x.shape[0])):
+            raise ValueError("global_amax needs one element, or one per row of a 2-D input")
+    call("mo_block_fp_qdq", x, _ptr(x), _ptr(y), rows, k, dtype_code(x.dtype), block_size, fmt,
+         scale_fmt, _ptr(global_amax), n_global, _stream(x))
     return y
 
 

@@ -14,7 +14,8 @@ __all__ = [
     "QuantizerAttributeConfig", "QuantizeConfig", "CompressConfig", "MaxCalibConfig", "SmoothQuantCalibConfig",
     "AWQLiteCalibConfig", "INT8_DEFAULT_CFG", "INT8_SMOOTHQUANT_CFG", "INT8_WEIGHT_ONLY_CFG",
     "FP8_DEFAULT_CFG", "INT4_BLOCKWISE_WEIGHT_ONLY_CFG", "INT4_AWQ_CFG", "W4A8_AWQ_BETA_CFG",
-    "FP8_KV_CFG", "NVFP4_DEFAULT_CFG", "NVFP4_AWQ_LITE_CFG", "NVFP4_KV_CFG", "choices",
+    "FP8_KV_CFG", "NVFP4_DEFAULT_CFG", "NVFP4_AWQ_LITE_CFG", "NVFP4_KV_CFG", "MXFP8_DEFAULT_CFG",
+    "MXFP6_DEFAULT_CFG", "MXFP4_DEFAULT_CFG", "MXINT8_DEFAULT_CFG", "W4A8_MXFP4_FP8_CFG", "choices",
 ]
 
 _SPECIAL_BLOCK_KEYS = ("type", "scale_bits", "scale_block_sizes")
@@ -306,7 +307,31 @@ NVFP4_AWQ_LITE_CFG = {
     "algorithm": "awq_lite",
 }
 
+
+
+def _mx_cfg(num_bits):
+    q = {"num_bits": num_bits, "block_sizes": {-1: 32, "type": "dynamic", "scale_bits": (8, 0)},
+         "enable": True}
+    return {"quant_cfg": {"*weight_quantizer": dict(q), "*input_quantizer": dict(q),
+                          **_default_disabled_quantizer_cfg},
+            "algorithm": None}
+
+
+# reference: config.py:266-345 -- 32-element blocks, shared power-of-two scale, no calibration
+MXFP8_DEFAULT_CFG = _mx_cfg((4, 3))
+MXFP6_DEFAULT_CFG = _mx_cfg((3, 2))
+MXFP4_DEFAULT_CFG = _mx_cfg((2, 1))
+MXINT8_DEFAULT_CFG = _mx_cfg(8)
+W4A8_MXFP4_FP8_CFG = {
+    "quant_cfg": {"*weight_quantizer": dict(_mx_cfg((2, 1))["quant_cfg"]["*weight_quantizer"]),
+                  "*input_quantizer": {"num_bits": (4, 3), "axis": None},
+                  **_default_disabled_quantizer_cfg},
+    "algorithm": None,
+}
+
 choices = {
+    "MXFP8_DEFAULT_CFG", "MXFP6_DEFAULT_CFG", "MXFP4_DEFAULT_CFG", "MXINT8_DEFAULT_CFG",
+    "W4A8_MXFP4_FP8_CFG",
     "INT8_DEFAULT_CFG", "INT8_SMOOTHQUANT_CFG", "INT8_WEIGHT_ONLY_CFG", "FP8_DEFAULT_CFG",
     "INT4_BLOCKWISE_WEIGHT_ONLY_CFG", "INT4_AWQ_CFG", "W4A8_AWQ_BETA_CFG", "NVFP4_DEFAULT_CFG",
     "NVFP4_AWQ_LITE_CFG",

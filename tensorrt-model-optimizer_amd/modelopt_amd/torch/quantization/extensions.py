@@ -68,16 +68,17 @@ class _MxTypes:
 
 
 class _MxExt:
-    """Counterpart of ``modelopt_cuda_ext_mx`` (TQ/src/tensor_quant_mx.cu:393-411); only the
-    NVFP4 combination (E2M1 elements, E4M3 scales, global amax) is built."""
+    """Counterpart of ``modelopt_cuda_ext_mx`` (TQ/src/tensor_quant_mx.cu:393-411)."""
 
     Types = _MxTypes
+    _names = ["E4M3", "E5M2", "INT8", "E0M3", "E1M2", "E3M0", "E2M1", "E3M2", "E2M3", "E8M0"]
 
     @staticmethod
     def fused_amax_convert(inputs, block_size, format, scale_format, global_amax=None):
-        if format != _MxTypes.E2M1 or scale_format != _MxTypes.E4M3 or global_amax is None:
-            raise NotImplementedError("only (E2M1, E4M3, global amax) = NVFP4 is built")
-        return kernels.fake_quant_nvfp4(inputs, global_amax, block_size, mode=0)
+        if block_size not in (8, 16, 32):
+            raise ValueError("Blocksize for fused call must be one of {8, 16, 32}")
+        return kernels.fake_quant_block_fp(inputs, block_size, _MxExt._names[int(format)],
+                                           _MxExt._names[int(scale_format)], global_amax)
 
 
 def _loaded(raise_if_failed):

@@ -12,7 +12,7 @@ from ... import _hip
 
 __all__ = [
     "amax_layout", "absmax_accumulate", "reduce_amax_gpu", "fake_quant_int", "fake_quant_fp8",
-    "fake_quant_nvfp4", "mul_last_dim",
+    "fake_quant_nvfp4", "fake_quant_block_fp", "mul_last_dim",
 ]
 
 
@@ -113,6 +113,15 @@ def fake_quant_nvfp4(x, global_amax, block_size=16, mode=0):
     if global_amax.numel() != 1:
         global_amax = global_amax.amax()
     return _hip.nvfp4_qdq(x, global_amax.reshape(1), block_size, mode)
+
+
+def fake_quant_block_fp(x, block_size, fmt, scale_fmt="E8M0", global_amax=None):
+    """Block floating point fake quantisation along the last dim (``fused_amax_convert``):
+    ``fmt`` / ``scale_fmt`` are format names (``"E4M3"``, ``"E2M1"``, ``"E8M0"`` ...)."""
+    x = x if x.is_contiguous() else x.contiguous()
+    if global_amax is not None:
+        global_amax = global_amax.to(device=x.device, dtype=torch.float32).reshape(-1).contiguous()
+    return _hip.block_fp_qdq(x, block_size, fmt, scale_fmt, global_amax)
 
 
 def mul_last_dim(x, scale):

@@ -53,12 +53,20 @@ def _dynamic_block_quantize_impl(inputs, block_size, amax, num_bits, exponent_bi
     scale_bits = (scale_exponent_bits, scale_num_bits - scale_exponent_bits - 1)
     if exponent_bits != 0:
         num_bits = (exponent_bits, num_bits - exponent_bits - 1)
-    if num_bits == (2, 1) and scale_bits == (4, 3):
+    if num_bits not in mx_format_map:
+        raise NotImplementedError(f"Unsupported num_bits: {num_bits}, scale_bits: {scale_bits} "
+                                  "for dynamic block quantization.")
+    assert scale_bits in mx_format_map, f"Scale bits should be in {mx_format_map.keys()}"
+    if scale_bits != (8, 0):
         assert amax is not None and amax.is_cuda, "amax must be a GPU tensor for dynamic block quantization."
-        return kernels.fake_quant_nvfp4(inputs, amax, block_size, NVFP4_FAKE_QUANT_MODE)
-    raise NotImplementedError(
-        f"Unsupported num_bits: {num_bits}, scale_bits: {scale_bits} for dynamic block "
-        "quantization (only NVFP4 = E2M1 with E4M3 scales is built).")
+        if amax.numel() != 1:
+            amax = amax.amax()
+        if num_bits == (2, 1) and scale_bits == (4, 3):
+            return kernels.fake_quant_nvfp4(inputs, amax, block_size, NVFP4_FAKE_QUANT_MODE)
+    else:
+        amax = None      # a power-of-two block scale has no global level
+    return kernels.fake_quant_block_fp(inputs, block_size, mx_format_map[num_bits],
+                                       mx_format_map[scale_bits], amax)
 
 
 quantize_op = _quantize_impl
@@ -134,7 +142,7 @@ class ScaledE4M3Function(Function):
 
 
 class DynamicBlockQuantizationFunction(Function):
-    """Dynamic block quantisation (NVFP4) with pass-through backward by default."""
+    """Dynamic block quantisation (NVFP4, MX formats) with pass-through backward by default."""
 
     @staticmethod
     def forward(ctx, inputs, block_size, amax, bias, num_bits, scale_bits,

@@ -17,7 +17,7 @@ from modelopt_amd.torch.export import quant_utils as equ
 from modelopt_amd.torch.quantization import kernels
 from modelopt_amd.torch.quantization.config import QuantizerAttributeConfig, normalize_algorithm
 from modelopt_amd.torch.quantization.nn import SequentialQuantizer, TensorQuantizer
-from oracle import fake_quant, reduce
+from oracle import fake_quant, mx, reduce
 
 
 # ----------------------------------------------------------------------------- config
@@ -183,6 +183,7 @@ def oracle_backend(monkeypatch):
     monkeypatch.setattr(kernels, "fake_quant_nvfp4",
                         lambda x, amax, bs=16, mode=0: fake_quant.nvfp4_fake_quant(x, amax, bs))
     monkeypatch.setattr(kernels, "mul_last_dim", lambda x, s: x * s)
+    monkeypatch.setattr(kernels, "fake_quant_block_fp", mx.block_fp_fake_quant)
 
 
 @pytest.mark.parametrize("shape,block_sizes,amax_shape,export_shape", [
@@ -305,3 +306,16 @@ def test_compress_surface_without_a_gpu():
     with pytest.raises(ValueError, match="expected a boolean"):
         mtq.compress(model, {"*": "yes"})
     assert issubclass(mtq.nn.RealQuantLinear, mtq.nn.QuantModule)
+
+
+def test_mx_quantizer_control_flow(oracle_backend):
+    """An MX quantizer needs no amax, ignores calibration and pads the last block."""
+    cfg = mtq.MXFP4_DEFAULT_CFG["quant_cfg"]["*input_quantizer"]
+    q = TensorQuantizer(QuantizerAttributeConfig(**cfg))
+    assert q.is_mx_format
+    x = torch.randn(3, 5, 40).to(torch.bfloat16)
+    assert torch.equal(q(x), mx.block_fp_fake_quant(x, 32, "E2M1"))
+    q.enable_calib()
+    q(x)
+    assert q.amax is None
+    assert mtq.MXFP8_DEFAULT_CFG["algorithm"] is None
