@@ -110,6 +110,19 @@ int mo_nvfp4_qdq(const void* x, void* y, int64_t rows, int64_t k, int dtype, con
 
 /* ------------------------------------------------------------------ real quantize + pack */
 
+/* Squared fake-quantisation error for n_cand candidate amax values in one pass over x viewed
+ * as [outer, axis, inner]:
+ *   loss[k * axis + a] += sum over the elements of channel a of (f32(x) - QDQ(f32(x); cand[k * axis + a]))^2
+ * with QDQ the fp32 operator of mo_int_qdq (kind 0: num_bits / is_unsigned / narrow_range) or of
+ * mo_fp8_qdq (kind 1: saturate).  Replaces the candidate loop of MseCalibrator.collect
+ * (TQ/calib/mse.py:83-107: quant_func, F.mse_loss(reduction="none"), reduce_sum per candidate;
+ * driven by mse_calibrate, TQ/model_calib.py:189-262).  x 16-byte aligned; per-channel needs
+ * inner % 8 == 0; other layouts return MO_ERR_UNSUPPORTED (callers take the per-candidate path).
+ * The sums are fp32, accumulated in an order that differs from torch.sum. */
+int mo_qdq_sq_err(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
+                  const float* cand, int n_cand, int kind, int num_bits, int is_unsigned,
+                  int narrow_range, int saturate, float* loss, void* stream);
+
 /* Block floating point quantize-dequantize of x[rows, k]: blocks of `block_size` (8, 16 or 32)
  * along k (zero padded), one shared scale per block, every element
  * sign(x) * format(|x| * scale) * unscale.  Replaces fused_amax_convert(inputs, block_size,

@@ -10,70 +10,11 @@
 // TENSOR / CHUNK / ELEM run one workgroup per tile of 1024 chunks (4 per lane, all loads issued
 // before the math), dispatched in tile order.
 #include "common.h"
+#include "qdq_ops.h"
 
 namespace mo {
 
 enum { TENSOR = 0, CHUNK = 1, ELEM = 2 };
-
-template <bool HAS_AMAX>
-struct Fp8Op {
-    static constexpr bool has_amax = HAS_AMAX;
-    struct Scale { float mul, inv; };
-    __device__ __forceinline__ Scale make(float amax) const {
-        Scale s;
-        // the reference writes `448.0 / amax`, which torch evaluates as reciprocal(amax) * 448
-        // (two roundings), and `1 / scale`, which is reciprocal(scale)
-        s.mul = (1.0f / amax) * 448.0f;
-        s.inv = 1.0f / s.mul;
-        return s;
-    }
-    template <bool SAT>
-    __device__ __forceinline__ float apply(float x, const Scale& s) const {
-        if (!has_amax) return round_e4m3<SAT>(x);
-        return round_e4m3<SAT>(x * s.mul) * s.inv;
-    }
-    // two elements per conversion instruction
-    template <bool SAT>
-    __device__ __forceinline__ void apply2(float& a, float& b, const Scale& sa, const Scale& sb) const {
-        if (!has_amax) { round_e4m3_pair<SAT>(a, b); return; }
-        a *= sa.mul;
-        b *= sb.mul;
-        round_e4m3_pair<SAT>(a, b);
-        a *= sa.inv;
-        b *= sb.inv;
-    }
-};
-
-struct IntOp {
-    float bound, lo;
-    // y = clamp(rne(x * mul), lo, bound) / div; when `fast`, the division is the exact
-    // reciprocal-and-FMA quotient (|q| <= 2^24 and div in [2^-64, 2^64] cannot over/underflow)
-    struct Scale { float mul, div, rdiv; bool fast; };
-    __device__ __forceinline__ Scale make(float amax) const {
-        Scale s;
-        const bool dead = amax <= 5.9604644775390625e-8f;  // 2^-24
-        const float sc = bound / amax;
-        s.mul = dead ? 0.0f : sc;
-        s.div = dead ? 1.0f : sc;
-        s.rdiv = 1.0f / s.div;
-        s.fast = mid_range(s.div);
-        return s;
-    }
-    template <bool>
-    __device__ __forceinline__ float apply(float x, const Scale& s) const {
-        float q = __builtin_rintf(x * s.mul);  // round half to even
-        // clamp the way torch.clamp does: NaN stays NaN
-        q = q < lo ? lo : q;
-        q = q > bound ? bound : q;
-        if (s.fast) return __builtin_copysignf(exact_quotient(q, s.div, s.rdiv), q);
-        return q / s.div;
-    }
-    template <bool F>
-    __device__ __forceinline__ void apply2(float& a, float& b, const Scale& sa, const Scale& sb) const {
-        a = apply<F>(a, sa);
-        b = apply<F>(b, sb);
-    }
-};
 
 constexpr int kTileChunks = 1024;
 

@@ -13,6 +13,7 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_PKG_DIR), "libmodelopt_hip.so")
 
 MO_F32, MO_F16, MO_BF16 = 0, 1, 2
+MO_ERR_ARG, MO_ERR_DTYPE, MO_ERR_UNSUPPORTED, MO_ERR_LAUNCH = -1, -2, -3, -4
 _DTYPES = {torch.float32: MO_F32, torch.float16: MO_F16, torch.bfloat16: MO_BF16}
 
 _P, _I64, _INT = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
@@ -29,6 +30,7 @@ SIGNATURES = {
     "mo_fp8_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _P],
     "mo_int_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _INT, _P],
     "mo_nvfp4_qdq": [_P, _P, _I64, _I64, _INT, _P, _INT, _INT, _INT, _P],
+    "mo_qdq_sq_err": [_P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _INT, _INT, _INT, _P, _P],
     "mo_block_fp_qdq": [_P, _P, _I64, _I64, _INT, _INT, _INT, _INT, _P, _I64, _P],
     "mo_nvfp4_quantize": [_P, _I64, _I64, _INT, _INT, _P, _INT, _P, _P, _P, _P, _P],
     "mo_nvfp4_dequantize": [_P, _P, _P, _I64, _I64, _INT, _P, _INT, _P],
@@ -141,6 +143,25 @@ def nvfp4_qdq(x, amax, block_size=16, mode=0, out=None):
     call("mo_nvfp4_qdq", x, _ptr(x), _ptr(y), rows, k, dtype_code(x.dtype), _ptr(amax),
          dtype_code(amax.dtype), block_size, mode, _stream(x))
     return y
+
+
+def qdq_sq_err_into(x, cand, loss, outer, axis, inner, kind, num_bits=8, unsigned=False,
+                    narrow_range=False, saturate=False):
+    """loss[k, a] += sum (x - QDQ(x; cand[k, a]))^2 for every candidate k; ``cand`` and ``loss`` are
+    fp32 [n_cand, axis].  Returns False when the layout is not covered by the kernel."""
+    _require_device(x, cand, loss)
+    assert x.is_contiguous() and cand.is_contiguous() and loss.is_contiguous()
+    assert cand.dtype == torch.float32 and loss.dtype == torch.float32
+    assert cand.numel() == loss.numel() and cand.numel() % axis == 0
+    rc = load().mo_qdq_sq_err(_ptr(x), outer, axis, inner, dtype_code(x.dtype), _ptr(cand),
+                              cand.numel() // axis, 0 if kind == "int" else 1, int(num_bits),
+                              int(bool(unsigned)), int(bool(narrow_range)), int(bool(saturate)),
+                              _ptr(loss), _stream(x))
+    if rc == MO_ERR_UNSUPPORTED:
+        return False
+    if rc != 0:
+        raise RuntimeError(f"mo_qdq_sq_err failed: {load().mo_error_string(rc).decode()}")
+    return True
 
 
 ELEM_FORMATS = ["E4M3", "E5M2", "INT8", "E0M3", "E1M2", "E3M0", "E2M1", "E3M2", "E2M3", "E8M0"]

@@ -1,5 +1,6 @@
 """Calibrators."""
 
 from .max import MaxCalibrator, _Calibrator
+from .mse import MseCalibrator
 
-__all__ = ["MaxCalibrator"]
+__all__ = ["MaxCalibrator", "MseCalibrator"]

@@ -11,7 +11,7 @@ from typing import Any, Literal
 from pydantic import BaseModel, ConfigDict, ValidationInfo, field_validator, model_validator
 
 __all__ = [
-    "QuantizerAttributeConfig", "QuantizeConfig", "CompressConfig", "MaxCalibConfig", "SmoothQuantCalibConfig",
+    "QuantizerAttributeConfig", "QuantizeConfig", "CompressConfig", "MaxCalibConfig", "MseCalibConfig", "SmoothQuantCalibConfig",
     "AWQLiteCalibConfig", "INT8_DEFAULT_CFG", "INT8_SMOOTHQUANT_CFG", "INT8_WEIGHT_ONLY_CFG",
     "FP8_DEFAULT_CFG", "INT4_BLOCKWISE_WEIGHT_ONLY_CFG", "INT4_AWQ_CFG", "W4A8_AWQ_BETA_CFG",
     "FP8_KV_CFG", "NVFP4_DEFAULT_CFG", "NVFP4_AWQ_LITE_CFG", "NVFP4_KV_CFG", "MXFP8_DEFAULT_CFG",
@@ -177,8 +177,18 @@ class AWQLiteCalibConfig(_MappingConfig):
     debug: bool | None = False
 
 
+class MseCalibConfig(_MappingConfig):
+    """amax search minimising the quantisation error (reference: config.py:984-1020)."""
+
+    method: Literal["mse"] = "mse"
+    num_steps: int | None = 10
+    start_multiplier: float | None = 0.25
+    stop_multiplier: float | None = 4.0
+    distributed_sync: bool | None = True
+
+
 _ALGO_CONFIGS = {"max": MaxCalibConfig, "smoothquant": SmoothQuantCalibConfig,
-                 "awq_lite": AWQLiteCalibConfig}
+                 "awq_lite": AWQLiteCalibConfig, "mse": MseCalibConfig}
 
 
 def normalize_algorithm(algorithm):

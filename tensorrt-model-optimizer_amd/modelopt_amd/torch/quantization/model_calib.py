@@ -15,6 +15,8 @@ import torch.nn.functional as F
 from torch import nn
 
 from ... import _hip
+from . import calib
+from .calib.max import MaxCalibrator
 from .conversion import set_quantizer_by_cfg_context
 from .nn import QuantModule, SequentialQuantizer, TensorQuantizer
 from .utils import all_valid_scales, is_quantized_linear
@@ -62,8 +64,11 @@ def finish_stats_collection(model: nn.Module, method: str | None = None):
         if not isinstance(module, TensorQuantizer) or module._disabled:
             continue
         cal = getattr(module, "_calibrator", None)
-        if cal and not getattr(module, "_dynamic", False) and cal.compute_amax() is not None:
-            module.load_calib_amax()
+        if cal and not getattr(module, "_dynamic", False):
+            found = cal.compute_amax() if method != "mse" or isinstance(cal, MaxCalibrator) \
+                else cal.compute_amax(False)
+            if found is not None:
+                module.load_calib_amax()
         module.enable_quant()
         module.disable_calib()
 
@@ -77,6 +82,50 @@ def max_calibrate(model: nn.Module, forward_loop=None, distributed_sync=True):
     else:
         forward_loop(model)
     finish_stats_collection(model)
+
+
+@torch.no_grad()
+def mse_calibrate(model: nn.Module, forward_loop=None, distributed_sync=True, num_steps: int = 10,
+                  start_multiplier: float = 0.25, stop_multiplier: float = 4.0):
+    """Max calibration first, then an amax search per quantizer that minimises the squared error
+    between the tensors it sees and their fake-quantised versions (reference:
+    model_calib.py:189-262)."""
+    max_calibrate(model, forward_loop, distributed_sync)
+    for name, module in model.named_modules():
+        if not isinstance(module, TensorQuantizer) or module._disabled:
+            continue
+        if module.is_static_block_quant:
+            raise ValueError("MSE calibration does not support static block quantization. "
+                             f"Found static block quantization at {name}.")
+        if module._calibrator is None or module._dynamic or not hasattr(module, "_amax"):
+            continue
+        initial_amax = module._amax.clone().detach()
+
+        def quant_func(x, amax, quantizer=module):
+            saved = quantizer._amax.clone() if hasattr(quantizer, "_amax") else None
+            quantizer._amax = amax
+            state = (quantizer._if_quant, quantizer._if_calib, quantizer._fake_quant)
+            quantizer._if_quant, quantizer._if_calib, quantizer._fake_quant = True, False, True
+            try:
+                xq = quantizer(x)
+            finally:
+                quantizer._if_quant, quantizer._if_calib, quantizer._fake_quant = state
+                if saved is not None:
+                    quantizer._amax = saved
+                else:
+                    delattr(quantizer, "_amax")
+            return xq
+
+        module._calibrator = calib.MseCalibrator(
+            amax=initial_amax, axis=module._calibrator._axis, num_steps=num_steps,
+            start_multiplier=start_multiplier, stop_multiplier=stop_multiplier,
+            quant_func=quant_func, quantizer=module)
+    enable_stats_collection(model)
+    if forward_loop is None:
+        weight_only_quantize(model)
+    else:
+        forward_loop(model)
+    finish_stats_collection(model, method="mse")
 
 
 # ----------------------------------------------------------------------------- pre-quant scale

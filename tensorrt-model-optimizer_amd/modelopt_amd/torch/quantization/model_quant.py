@@ -62,6 +62,10 @@ def calibrate(model: nn.Module, algorithm="max", forward_loop: ForwardLoop | Non
     try:
         if method == "max":
             model_calib.max_calibrate(model, forward_loop, kwargs.get("distributed_sync", True))
+        elif method == "mse":
+            model_calib.mse_calibrate(model, forward_loop, kwargs.get("distributed_sync", True),
+                                      kwargs.get("num_steps", 10), kwargs.get("start_multiplier", 0.25),
+                                      kwargs.get("stop_multiplier", 4.0))
         elif method == "smoothquant":
             model_calib.smoothquant(model, forward_loop, alpha=kwargs.get("alpha", 1.0))
         elif method == "awq_lite":
