@@ -147,7 +147,7 @@ static void launch_sq_err(const void* x, int64_t outer, int64_t axis, int64_t in
     if (axis == 1) {
         int64_t g = ((n >> 3) + 511) / 512;
         if (g < 1) g = 1;
-        if (g > 512) g = 512;
+        if (g > 2048) g = 2048;
         sq_err_tensor_kernel<DT, KN, SAT, Op><<<(unsigned)g, 256, 0, s>>>(x, n, cand, K, op, loss);
     } else {
         const int64_t nrows = outer * axis;
