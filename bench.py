@@ -103,7 +103,7 @@ def cpu_baseline(torch, passes=8):
 
 
 def single_tensor_configs(torch, steps, warmup):
-    """BASELINE configs 1, 3 and 4 (one tensor / one linear each), device time per pass.
+    """The three single-tensor benchmark configurations (one tensor / one linear each), device time per pass.
 
     C1: FP8 abs-max + fake quant of a 4096 x 4096 weight with 0.1 % outliers (6 B / element).
     C3: AWQ-lite search, 21 alphas, W 4096 x 4096, X 512 x 4096 (mtq.quantize end to end, and the
@@ -192,7 +192,7 @@ def single_tensor_configs(torch, steps, warmup):
 
 
 def calib_sweep(torch, layers, n_seqs, batch, seq_len=512):
-    """BASELINE config 5: mtq.quantize (NVFP4 weights + inputs, FP8 KV cache, max calibration) on
+    """Calibration sweep configuration: mtq.quantize (NVFP4 weights + inputs, FP8 KV cache, max calibration) on
     a random-init Llama-3-8B-shaped decoder over n_seqs x 512 uniform-random token ids.  Reports
     end-to-end seconds (the reference's own stopwatch brackets mtq.quantize the same way,
     examples/llm_ptq/hf_ptq.py:214-232), the forward-only seconds of the same data with no
@@ -261,7 +261,7 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU only: this build has no multi-GPU path (got --gpus {a.gpus}); "
-              "the path shards by tensor with no exchange, see DESIGN.md", file=sys.stderr)
+              "the path shards by tensor with no exchange", file=sys.stderr)
         sys.exit(2)
 
     import torch

@@ -23,7 +23,7 @@ def _rand(shape, dtype, seed, scale=1.0):
 
 
 def _c1_tensor(n=1024):
-    """BASELINE config 1 shape in small: N(0, 0.02) with 0.1 % of entries scaled x50."""
+    """The FP8 benchmark input in small: N(0, 0.02) with 0.1 % of entries scaled x50."""
     g = torch.Generator().manual_seed(1)
     x = 0.02 * torch.randn(n, n, generator=g)
     idx = torch.randperm(x.numel(), generator=g)[: x.numel() // 1000]
