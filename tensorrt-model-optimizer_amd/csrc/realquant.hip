@@ -281,11 +281,12 @@ __device__ __forceinline__ uint32_t int4_code(float v) {  // clamp(rne(v), -8, 7
     return (q == q) ? ((uint32_t)(int)q & 0xFFu) : 0u;
 }
 
-__device__ __forceinline__ uint32_t int4_nibble(float v) {  // clamp(rne(v), -8, 7) & 0xF
-    float q = __builtin_rintf(v);
-    q = q < -8.0f ? -8.0f : q;
-    q = q > 7.0f ? 7.0f : q;
-    return (q == q) ? ((uint32_t)(int)q & 0xFu) : 0u;
+// clamp(rne(v), -8, 7) as an integer in three operations: v_med3_f32 clamps (and returns the
+// smallest operand, -8, for a NaN, which is the "NaN packs as code 0" rule of the kernels above),
+// adding 1.5 * 2^23 rounds to nearest even and leaves the integer in the low mantissa bits.
+__device__ __forceinline__ int int4_rne(float v) {
+    const float t = __builtin_amdgcn_fmed3f(v, -8.0f, 7.0f);
+    return (int)f2u(t + 12582912.0f) - 0x4B400000;
 }
 
 template <int DT>
@@ -316,14 +317,16 @@ __global__ __launch_bounds__(256) void int4_block_quantize_tile_kernel(
         if (c >= chunks) continue;
         const float scale = round_via<DT>(round_via<DT>(1.0f / u2f(m)) * 7.0f);
         if ((threadIdx.x & (lanes_per_block - 1)) == 0) store_elem<DT>(scales, c >> shift, scale);
-        uint32_t w = 0;
+        // byte = (hi + 8) << 4 | (lo + 8) = 16 * hi + lo + 0x88; the +8s of the four bytes are
+        // added once to the assembled word (the borrows of negative bytes cancel exactly)
+        int w = 0;
 #pragma unroll
         for (int j = 0; j < 8; j += 2) {
-            const uint32_t hi = int4_code(round_via<DT>(v[u][j] * scale));
-            const uint32_t lo = int4_code(round_via<DT>(v[u][j + 1] * scale));
-            w |= (((hi << 4) | lo) & 0xFFu) << (4 * j);
+            const int hi = int4_rne(round_via<DT>(v[u][j] * scale));
+            const int lo = int4_rne(round_via<DT>(v[u][j + 1] * scale));
+            w += (hi * 16 + lo) << (4 * j);
         }
-        __builtin_nontemporal_store(w, packed + c);
+        __builtin_nontemporal_store((uint32_t)w + 0x88888888u, packed + c);
     }
 }
 
@@ -419,7 +422,10 @@ __global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
                 qa = a[u][e] / sa[u];
                 qb = b[u][e] / sb[u];
             }
-            const uint32_t byte = int4_nibble(qa) | (int4_nibble(qb) << 4);
+            // a NaN quotient packs as 0 here (what the float -> int8 cast of the CPU path yields)
+            const uint32_t na = qa == qa ? (uint32_t)int4_rne(qa) & 0xFu : 0u;
+            const uint32_t nb = qb == qb ? (uint32_t)int4_rne(qb) & 0xFu : 0u;
+            const uint32_t byte = na | (nb << 4);
             if (e < 4) lo |= byte << (8 * e); else hi |= byte << (8 * (e - 4));
         }
         const u32x2 o = {lo, hi};

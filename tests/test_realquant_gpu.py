@@ -203,6 +203,7 @@ def test_int4_block_quantize_special_blocks(dtype, bs):
     finite = torch.isfinite(s_o.float()).reshape(-1) & (s_o.float().reshape(-1) != 0)
     got = packed.cpu().reshape(nblk, -1)
     assert torch.equal(got[finite], p_o.reshape(nblk, -1)[finite])
+    assert int(got[0].max()) == 0      # all-zero block: scale inf, 0 * inf = NaN packs as code 0
     y = _hip.int4_block_dequantize(packed, scales, bs).reshape(nblk, bs)
     y_o = qtensor.int4_dequantize(got.reshape(p_o.shape), s_o, bs, x.shape, dtype)
     assert_bits_equal(y.cpu(), y_o, "dequant")
