@@ -142,6 +142,19 @@ int mo_block_fp_qdq(const void* x, void* y, int64_t rows, int64_t k, int dtype, 
                     int format, int scale_format, const float* global_amax,
                     int64_t n_global_amax, void* stream);
 
+/* MXFP4 storage format over the n elements of x in flat blocks of block_size (8 << k, n a
+ * multiple of it).  Replaces MXFP4QTensor.quantize / dequantize (TQ/qtensor/mxfp4_tensor.py:38-83,
+ * :85-144):
+ *   scales[b] = uint8(127 + max(ceil(log2(f32(amax_b) / 6)), -127))   (E8M0)
+ *   v = f32(x) / 2^(scales[b] - 127); code = 8 * (v is not > 0) + #{E2M1 bounds < |v|}
+ *   (ties to the smaller magnitude, zero packs as code 8); packed[i] = code[2i] | code[2i+1] << 4.
+ * Dequantize: y = T((-1)^(code >> 3) * e2m1[code & 7] * 2^(scale - 127)).
+ * An infinite or NaN block amax has no defined scale byte in the reference; 255 is written. */
+int mo_mxfp4_quantize(const void* x, int64_t n, int dtype, int block_size, uint8_t* packed,
+                      uint8_t* scales, void* stream);
+int mo_mxfp4_dequantize(const uint8_t* packed, const uint8_t* scales, int64_t n, int block_size,
+                        void* y, int dtype, void* stream);
+
 /* NVFP4 quantize + pack.  Replaces NVFP4QTensor.quantize and get_weights_scaling_factor
  * (TQ/qtensor/nvfp4_tensor.py:63-92,143-232) as called by to_quantized_weight
  * (modelopt/torch/export/quant_utils.py:822-834) and TensorQuantizer._real_quantize

@@ -119,3 +119,36 @@ def block_fp_fake_quant(x: torch.Tensor, block_size: int, fmt: str, scale_fmt: s
     # the reference leaves the sign of a zero or NaN input undefined; +1 here
     y = torch.where(blocks < 0, -q, q)
     return y.reshape(rows, kp)[:, :k].reshape(shape).to(dtype)
+
+
+# --------------------------------------------------------------------------- packed MXFP4
+_E2M1_BOUNDS = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5])
+_E2M1_VALUES = torch.tensor([0, 0.5, 1, 1.5, 2, 3, 4, 6])
+
+
+def mxfp4_quantize(x: torch.Tensor, block_size: int = 32):
+    """MXFP4QTensor.quantize, TQ/qtensor/mxfp4_tensor.py:38-83, op for op: fp32 block amax,
+    ``e = ceil(max(log2(amax / 6), -127))``, ``x / exp2(e)``, code = sign bit (set unless the value
+    is positive) * 8 + number of E2M1 bounds strictly below the magnitude; two codes per byte, even
+    index in the low nibble.  Returns (packed uint8 [..., k / 2], scale bytes uint8 [nblocks, 1])."""
+    shape = x.shape
+    v = x.reshape(-1, block_size)
+    amax = v.float().abs().max(dim=-1, keepdim=True).values
+    descale = amax / 6.0
+    e = torch.ceil(torch.maximum(torch.log2(descale), torch.tensor(-127.0)))
+    v = (v / torch.exp2(e)).view(shape)
+    sign = torch.sign(v)
+    sign_bit = (2 - sign) // 2
+    ordinal = torch.sum((v.abs().unsqueeze(-1) - _E2M1_BOUNDS) > 0, dim=-1)
+    codes = (sign_bit * 0b1000 + ordinal).to(torch.uint8)
+    packed = (codes[..., 1::2] << 4) + codes[..., 0::2]
+    return packed, (e + 127).to(torch.uint8)
+
+
+def mxfp4_dequantize(packed: torch.Tensor, scales: torch.Tensor, block_size: int, shape, dtype):
+    """MXFP4QTensor.dequantize, :85-144."""
+    codes = torch.stack([packed & 0x0F, (packed >> 4) & 0x0F], dim=-1).reshape(*packed.shape[:-1], -1)
+    sign = 1 - 2 * ((codes & 0b1000) >> 3).to(torch.float32)
+    mag = _E2M1_VALUES[(codes & 0b0111).long().reshape(-1)].reshape(codes.shape)
+    v = (sign * mag).reshape(-1, block_size) * torch.exp2(scales.float() - 127).reshape(-1, 1)
+    return v.reshape(shape).to(dtype)

@@ -225,3 +225,155 @@ extern "C" int mo_block_fp_qdq(const void* x, void* y, int64_t rows, int64_t k, 
 #undef CALL_FMT
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }
+
+// ------------------------------------------------------------------------------ MXFP4 storage
+// Packed MXFP4: blocks of `block` elements share the E8M0 byte 127 + ceil(log2(amax / 6))
+// (clamped below at -127); codes are sign << 3 | ordinal with the ordinal = number of E2M1 bounds
+// strictly below |x / 2^e| (ties go to the smaller magnitude) and the sign bit set for every
+// element that is not positive -- zero packs as code 8; byte i = code[2i] | code[2i + 1] << 4.
+namespace mo {
+
+// ceil(log2(v)) clamped below at -127 for a positive finite fp32 v, read off the bits
+__device__ __forceinline__ int ceil_log2_clamped(float v) {
+    const uint32_t bits = f2u(v), ef = bits >> 23, mant = bits & 0x7FFFFFu;
+    if (ef == 0) return mant > 0x400000u ? -126 : -127;  // subnormal: above 2^-127 or not
+    return (int)ef - 127 + (mant != 0);
+}
+
+__device__ __forceinline__ uint32_t mxfp4_code(float v) {
+    const float a = __builtin_fabsf(v);
+    const uint32_t ord = (uint32_t)(a > 0.25f) + (uint32_t)(a > 0.75f) + (uint32_t)(a > 1.25f) +
+                         (uint32_t)(a > 1.75f) + (uint32_t)(a > 2.5f) + (uint32_t)(a > 3.5f) +
+                         (uint32_t)(a > 5.0f);
+    return ord | (v > 0.0f ? 0u : 8u);
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void mxfp4_quantize_kernel(const void* __restrict__ x,
+                                                             int64_t chunks, int lg_g,
+                                                             uint32_t* __restrict__ packed,
+                                                             uint8_t* __restrict__ scales) {
+    const int64_t c0 = (int64_t)blockIdx.x * kBlockFpTileChunks + threadIdx.x;
+    RawChunk<DT> raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        zero_raw<DT>(raw[u]);
+        if (c < chunks) load_raw<DT>(x, c << 3, raw[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        float v[8];
+        unpack_raw<DT>(raw[u], v);
+        uint32_t m = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t t = f2u(v[j]) & 0x7FFFFFFFu;
+            m = t > m ? t : m;
+        }
+        m = group_max_u32(m, lg_g);
+        if (c >= chunks) continue;
+        const float amax = u2f(m);
+        // amax == 0: log2(0) = -inf, clamped to -127.  Infinite or NaN amax has no defined byte in
+        // the reference (float -> uint8 of inf / NaN); 255 here.
+        int e = -127;
+        const bool finite = m < 0x7F800000u;
+        if (amax > 0.0f && finite) e = ceil_log2_clamped(amax / 6.0f);
+        if ((threadIdx.x & ((1 << lg_g) - 1)) == 0) scales[c >> lg_g] = finite ? (uint8_t)(e + 127) : 255;
+        const float inv = __builtin_ldexpf(1.0f, -e);  // x / 2^e is exact up to over / underflow
+        uint32_t w = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            // the reference divides: identical to the product unless 2^-e itself overflows
+            const float q = e >= -126 ? v[j] * inv : v[j] / __builtin_ldexpf(1.0f, e);
+            w |= mxfp4_code(q) << (4 * j);
+        }
+        __builtin_nontemporal_store(w, packed + c);
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void mxfp4_dequantize_kernel(const uint32_t* __restrict__ packed,
+                                                               const uint8_t* __restrict__ scales,
+                                                               int64_t chunks, int lg_g,
+                                                               void* __restrict__ y) {
+    const int64_t c0 = (int64_t)blockIdx.x * kBlockFpTileChunks + threadIdx.x;
+    uint32_t w[4], sb[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        w[u] = sb[u] = 0;
+        if (c < chunks) {
+            w[u] = __builtin_nontemporal_load(packed + c);
+            sb[u] = scales[c >> lg_g];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + u * 256;
+        if (c >= chunks) continue;
+        const float s = __builtin_ldexpf(1.0f, (int)sb[u] - 127);  // exp2(byte - 127) in fp32
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t code = (w[u] >> (4 * j)) & 0xFu;
+            const float mag = e2m1_to_f32(code & 7u);
+            v[j] = ((code & 8u) ? -mag : mag) * s;   // code 8 is -0
+        }
+        store_chunk<DT>(y, c << 3, v);
+    }
+}
+
+}  // namespace mo
+
+static int mxfp4_check(int64_t n, int block_size, int* lg_g) {
+    if (n < 0) return MO_ERR_ARG;
+    *lg_g = -1;
+    for (int k = 0; k <= 6; ++k)
+        if (block_size == (8 << k)) *lg_g = k;
+    if (*lg_g < 0) return MO_ERR_UNSUPPORTED;
+    if (n % block_size) return MO_ERR_ARG;
+    if ((n / 8 + mo::kBlockFpTileChunks - 1) / mo::kBlockFpTileChunks > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+    return MO_OK;
+}
+
+extern "C" int mo_mxfp4_quantize(const void* x, int64_t n, int dtype, int block_size,
+                                 uint8_t* packed, uint8_t* scales, void* stream) {
+    int lg_g;
+    const int rc = mxfp4_check(n, block_size, &lg_g);
+    if (rc != MO_OK) return rc;
+    if (n == 0) return MO_OK;
+    if (!x || !packed || !scales) return MO_ERR_ARG;
+    if (((uintptr_t)x & 15u) || ((uintptr_t)packed & 3u)) return MO_ERR_ARG;
+    const int64_t chunks = n / 8;
+    const unsigned grid = (unsigned)((chunks + mo::kBlockFpTileChunks - 1) / mo::kBlockFpTileChunks);
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case MO_F32: mo::mxfp4_quantize_kernel<MO_F32><<<grid, 256, 0, s>>>(x, chunks, lg_g, (uint32_t*)packed, scales); break;
+        case MO_F16: mo::mxfp4_quantize_kernel<MO_F16><<<grid, 256, 0, s>>>(x, chunks, lg_g, (uint32_t*)packed, scales); break;
+        case MO_BF16: mo::mxfp4_quantize_kernel<MO_BF16><<<grid, 256, 0, s>>>(x, chunks, lg_g, (uint32_t*)packed, scales); break;
+        default: return MO_ERR_DTYPE;
+    }
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_mxfp4_dequantize(const uint8_t* packed, const uint8_t* scales, int64_t n,
+                                   int block_size, void* y, int dtype, void* stream) {
+    int lg_g;
+    const int rc = mxfp4_check(n, block_size, &lg_g);
+    if (rc != MO_OK) return rc;
+    if (n == 0) return MO_OK;
+    if (!y || !packed || !scales) return MO_ERR_ARG;
+    if (((uintptr_t)y & 15u) || ((uintptr_t)packed & 3u)) return MO_ERR_ARG;
+    const int64_t chunks = n / 8;
+    const unsigned grid = (unsigned)((chunks + mo::kBlockFpTileChunks - 1) / mo::kBlockFpTileChunks);
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case MO_F32: mo::mxfp4_dequantize_kernel<MO_F32><<<grid, 256, 0, s>>>((const uint32_t*)packed, scales, chunks, lg_g, y); break;
+        case MO_F16: mo::mxfp4_dequantize_kernel<MO_F16><<<grid, 256, 0, s>>>((const uint32_t*)packed, scales, chunks, lg_g, y); break;
+        case MO_BF16: mo::mxfp4_dequantize_kernel<MO_BF16><<<grid, 256, 0, s>>>((const uint32_t*)packed, scales, chunks, lg_g, y); break;
+        default: return MO_ERR_DTYPE;
+    }
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}

@@ -31,6 +31,8 @@ SIGNATURES = {
     "mo_int_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _INT, _P],
     "mo_nvfp4_qdq": [_P, _P, _I64, _I64, _INT, _P, _INT, _INT, _INT, _P],
     "mo_qdq_sq_err": [_P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _INT, _INT, _INT, _P, _P],
+    "mo_mxfp4_quantize": [_P, _I64, _INT, _INT, _P, _P, _P],
+    "mo_mxfp4_dequantize": [_P, _P, _I64, _INT, _P, _INT, _P],
     "mo_block_fp_qdq": [_P, _P, _I64, _I64, _INT, _INT, _INT, _INT, _P, _I64, _P],
     "mo_nvfp4_quantize": [_P, _I64, _I64, _INT, _INT, _P, _INT, _P, _P, _P, _P, _P],
     "mo_nvfp4_dequantize": [_P, _P, _P, _I64, _I64, _INT, _P, _INT, _P],
@@ -186,6 +188,26 @@ def block_fp_qdq(x, block_size, fmt, scale_fmt="E8M0", global_amax=None, out=Non
             raise ValueError("global_amax needs one element, or one per row of a 2-D input")
     call("mo_block_fp_qdq", x, _ptr(x), _ptr(y), rows, k, dtype_code(x.dtype), block_size, fmt,
          scale_fmt, _ptr(global_amax), n_global, _stream(x))
+    return y
+
+
+def mxfp4_quantize(x, block_size=32):
+    """-> (packed uint8 [..., k / 2], E8M0 scale bytes uint8 [numel / block_size, 1])."""
+    _require_device(x)
+    assert x.is_contiguous() and x.numel() % block_size == 0 and x.shape[-1] % 2 == 0
+    packed = torch.empty(x.shape[:-1] + (x.shape[-1] // 2,), dtype=torch.uint8, device=x.device)
+    scales = torch.empty((x.numel() // block_size, 1), dtype=torch.uint8, device=x.device)
+    call("mo_mxfp4_quantize", x, _ptr(x), x.numel(), dtype_code(x.dtype), block_size, _ptr(packed),
+         _ptr(scales), _stream(x))
+    return packed, scales
+
+
+def mxfp4_dequantize(packed, scales, block_size, dtype):
+    _require_device(packed, scales)
+    assert packed.is_contiguous() and scales.is_contiguous() and scales.dtype == torch.uint8
+    y = torch.empty(packed.shape[:-1] + (packed.shape[-1] * 2,), dtype=dtype, device=packed.device)
+    call("mo_mxfp4_dequantize", packed, _ptr(packed), _ptr(scales), y.numel(), block_size, _ptr(y),
+         dtype_code(dtype), _stream(packed))
     return y
 
 

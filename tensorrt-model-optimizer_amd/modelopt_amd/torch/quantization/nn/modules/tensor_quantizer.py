@@ -19,8 +19,8 @@ from torch import nn
 from ... import calib, kernels
 from ... import utils as quant_utils
 from ...config import QuantizerAttributeConfig
-from ...qtensor import (BaseQuantizedTensor, FP8QTensor, INT4QTensor, INT8QTensor, NVFP4QTensor,
-                        QTensorWrapper)
+from ...qtensor import (BaseQuantizedTensor, FP8QTensor, INT4QTensor, INT8QTensor, MXFP4QTensor,
+                        NVFP4QTensor, QTensorWrapper)
 from ...tensor_quant import dynamic_block_quant, fake_tensor_quant, scaled_e4m3
 
 __all__ = ["SequentialQuantizer", "TensorQuantizer"]
@@ -330,7 +330,10 @@ class TensorQuantizer(nn.Module):
         elif bs.get("scale_bits", 0) == 8 and bs.get("scale_block_sizes"):
             raise NotImplementedError("NF4 double quantisation is outside the hot path built here")
         elif bs.get("scale_bits") == (8, 0) and bs.get("type") == "dynamic":
-            raise NotImplementedError("MX formats are outside the hot path built here")
+            if self._num_bits != (2, 1):
+                raise NotImplementedError("of the MX formats only MXFP4 has a packed tensor class")
+            outputs, scale = MXFP4QTensor.quantize(inputs, bs[-1])
+            buffers["_scale"] = scale
         elif bs.get("scale_bits") == (4, 3):
             if self.amax is not None and self._amax.device != inputs.device:
                 self._amax = self._amax.to(inputs.device)

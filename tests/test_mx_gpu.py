@@ -138,3 +138,50 @@ def test_extension_shim_matches_reference_call_shape():
                                                               mx_format_map[scale_bits]), str(num_bits))
     with pytest.raises(ValueError):
         ext.fused_amax_convert(x.to(DEV), 64, ext.Types.E2M1, ext.Types.E8M0, None)
+
+
+# ----------------------------------------------------------------------------- packed MXFP4
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("block", [32, 16])
+def test_mxfp4_pack_and_unpack_match_the_reference_qtensor(dtype, block):
+    g = torch.Generator().manual_seed(61)
+    x = (torch.randn((64, 256), generator=g) * torch.exp(3 * torch.randn((64, 1), generator=g))).to(dtype)
+    x[0, :64] = 0                                              # zero blocks: scale byte 0, code 8
+    x[1, :8] = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0]).to(dtype)   # exact bounds
+    x[1, 8:32] = 0.1
+    x[2, :32] = x[1, :32] * -4                                 # the same, negative, another scale
+    x[3, 5] = -0.0
+    x[4] *= 1e-30 if dtype != torch.float16 else 1e-4
+    packed, scales = _hip.mxfp4_quantize(x.to(DEV), block)
+    p_o, s_o = mx.mxfp4_quantize(x, block)
+    assert torch.equal(scales.cpu(), s_o)
+    assert torch.equal(packed.cpu(), p_o)
+    y = _hip.mxfp4_dequantize(packed, scales, block, dtype)
+    assert_bits_equal(y.cpu(), mx.mxfp4_dequantize(p_o, s_o, block, x.shape, dtype), "dequantised")
+
+
+def test_mxfp4_every_code_and_scale_byte_dequantizes_like_the_reference():
+    codes = torch.arange(256, dtype=torch.uint8).repeat(16).reshape(-1, 16)      # 256 blocks of 32
+    scales = torch.arange(256, dtype=torch.uint8).reshape(-1, 1)
+    for dtype in DTYPES:
+        y = _hip.mxfp4_dequantize(codes.to(DEV), scales.to(DEV), 32, dtype)
+        assert_bits_equal(y.cpu(), mx.mxfp4_dequantize(codes, scales, 32, (256, 32), dtype), str(dtype))
+
+
+def test_mxfp4_through_quantizer_and_compress():
+    import modelopt_amd.torch.quantization as mtq
+    from modelopt_amd.torch.quantization.qtensor import MXFP4QTensor, QTensorWrapper
+
+    lin = torch.nn.Sequential(torch.nn.Linear(128, 64, bias=False)).to(torch.bfloat16).to(DEV)
+    w = lin[0].weight.data.cpu().clone()
+    mtq.quantize(lin, mtq.MXFP4_DEFAULT_CFG, forward_loop=None)
+    with pytest.warns(UserWarning):
+        mtq.compress(lin)
+    assert isinstance(lin[0].weight, QTensorWrapper) and lin[0].weight.metadata["qtensor_class"] is MXFP4QTensor
+    p_o, s_o = mx.mxfp4_quantize(w, 32)
+    assert torch.equal(lin[0].weight.data.cpu(), p_o)
+    assert torch.equal(lin[0].weight_quantizer._scale.cpu(), s_o)
+    got = lin[0].weight_quantizer(lin[0].weight)
+    assert_bits_equal(got.cpu(), mx.mxfp4_dequantize(p_o, s_o, 32, w.shape, torch.bfloat16), "dequantised weight")
+    x = torch.randn(4, 128, dtype=torch.bfloat16, device=DEV)
+    assert torch.isfinite(lin(x).float()).all()
