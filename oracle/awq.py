@@ -125,3 +125,41 @@ def smoothquant_linear(w: torch.Tensor, act_amax: torch.Tensor, alpha: float = 1
     in_amax = (smoothing * scale_a.to(torch.float32)).amax().to(w.dtype)
     w_amax = reduce_amax(w_new, axis=[1], keepdims=True)
     return pqs, w_new, in_amax, w_amax
+
+
+@torch.no_grad()
+def awq_clip_search(w: torch.Tensor, batches, block_size: int = 128, num_bits: int = 4,
+                    max_co_batch_size: int = 1024, max_tokens_per_batch: int = 64,
+                    min_clip_ratio: float = 0.5, shrink_step: float = 0.05):
+    """AWQ clip for one ``[N, K]`` weight with static last-axis INT blocks.  Follows
+    TQ/model_calib.py:810-929,852-862: per clip ratio the weight is fake-quantised with
+    ``ratio * block amax``; the error is measured on the per-block partial outputs of up to
+    ``max_tokens_per_batch`` strided tokens of every batch, all elementwise arithmetic in the
+    weight dtype as the reference writes it.  Returns (losses {ratio: [N, K/bs]}, best clip amax
+    [N * K/bs, 1])."""
+    co, ci = w.shape
+    assert ci % block_size == 0
+    w_amax = reduce_amax(w.reshape(-1, block_size), axis=[1], keepdims=True)
+    ratios = [round(float(k), 2) for k in torch.arange(min_clip_ratio, 1.0, shrink_step)] + [1.0]
+    losses = {k: torch.zeros((co, ci // block_size)) for k in ratios}
+    w4 = w.reshape(co, 1, -1, block_size)
+    for x in batches:
+        x = x.reshape(-1, x.shape[-1])
+        x = x[0::max(1, x.shape[0] // max_tokens_per_batch)]
+        x4 = x.reshape(1, x.shape[0], -1, block_size)
+        for lo in range(0, co, max_co_batch_size):
+            hi = min(lo + max_co_batch_size, co)
+            org_out = (x4 * w4[lo:hi]).sum(dim=-1)
+            for shrink in ratios:
+                amax = w_amax * shrink
+                wq = tensor_quant(w.reshape(-1, block_size), amax, num_bits, False, False).reshape(w.shape)
+                cur_out = (x4 * wq[lo:hi].reshape(w4[lo:hi].shape)).sum(dim=-1)
+                losses[shrink][lo:hi] += (cur_out - org_out).float().pow(2).mean(dim=1)
+    best_loss = torch.ones_like(w_amax) * float("inf")
+    best = torch.zeros_like(w_amax)
+    for shrink, loss in losses.items():
+        loss = loss.view_as(w_amax)
+        better = loss < best_loss
+        best_loss = torch.where(better, loss, best_loss)
+        best = torch.where(better, w_amax * shrink, best)
+    return losses, best

@@ -177,6 +177,29 @@ class AWQLiteCalibConfig(_MappingConfig):
     debug: bool | None = False
 
 
+class AWQClipCalibConfig(_MappingConfig):
+    """Reference: config.py:1069-1115."""
+
+    method: Literal["awq_clip"] = "awq_clip"
+    max_co_batch_size: int | None = 1024
+    max_tokens_per_batch: int | None = 64
+    min_clip_ratio: float | None = 0.5
+    shrink_step: float | None = 0.05
+    debug: bool | None = False
+
+
+class AWQFullCalibConfig(_MappingConfig):
+    """awq_lite followed by awq_clip (reference: config.py:1118-1135)."""
+
+    method: Literal["awq_full"] = "awq_full"
+    alpha_step: float | None = 0.1
+    max_co_batch_size: int | None = 1024
+    max_tokens_per_batch: int | None = 64
+    min_clip_ratio: float | None = 0.5
+    shrink_step: float | None = 0.05
+    debug: bool | None = False
+
+
 class MseCalibConfig(_MappingConfig):
     """amax search minimising the quantisation error (reference: config.py:984-1020)."""
 
@@ -188,7 +211,8 @@ class MseCalibConfig(_MappingConfig):
 
 
 _ALGO_CONFIGS = {"max": MaxCalibConfig, "smoothquant": SmoothQuantCalibConfig,
-                 "awq_lite": AWQLiteCalibConfig, "mse": MseCalibConfig}
+                 "awq_lite": AWQLiteCalibConfig, "mse": MseCalibConfig,
+                 "awq_clip": AWQClipCalibConfig, "awq_full": AWQFullCalibConfig}
 
 
 def normalize_algorithm(algorithm):

@@ -7,6 +7,7 @@ The per-element work (abs-max, scaling, quantize-dequantize, column statistics, 
 runs in the HIP kernels; the search GEMM is a plain library GEMM (``F.linear``).
 """
 
+import math
 import types
 import warnings
 
@@ -230,13 +231,142 @@ def smoothquant(model: nn.Module, forward_loop=None, alpha=1.0):
     print(f"Smoothed {smoothed} modules")
 
 
+# ----------------------------------------------------------------------------- AWQ-clip
+class _AWQClipHelper:
+    """Per-linear state of the clip search (reference: model_calib.py:810-850)."""
+
+    def __init__(self, module, min_clip_ratio, shrink_step):
+        self.num_tokens = 0
+        self.block_size = _awq_block_size(module.weight, module.weight_quantizer)
+        q = module.weight_quantizer
+        q.reset_amax()
+        max_calibrate(q, lambda quantizer: quantizer(module.weight))
+        self.w_amax = q.amax.clone()
+        co, ci = module.weight.shape
+        ratios = [round(float(k), 2) for k in torch.arange(min_clip_ratio, 1.0, shrink_step)] + [1.0]
+        dev = module.weight.device
+        if self.is_per_tensor_clip(module):
+            self.loss = {k: torch.tensor(0.0, device=dev) for k in ratios}
+        else:
+            self.loss = {k: torch.zeros((co, math.ceil(ci / self.block_size)), device=dev) for k in ratios}
+        self.best_clip_val = None
+        self.best_loss = None
+        self.is_input_quantized = module.input_quantizer.is_enabled
+        q.disable()
+
+    @staticmethod
+    def is_per_tensor_clip(module):
+        q = module.weight_quantizer
+        dynamic_per_tensor = (q.block_sizes is not None and q.block_sizes.get("type") == "dynamic"
+                              and q.axis is None)
+        return dynamic_per_tensor or (q.axis is None and q.block_sizes is None)
+
+
+def _awq_clip_search(self, inputs, co_bsz, max_tokens):
+    """Accumulate, for every clip ratio, the error the clipped and fake-quantised weight makes on
+    the layer's partial (per input block) outputs (reference: model_calib.py:864-929).  The weight
+    is quantised once per ratio by the block fake-quant kernel; the partial sums are torch ops."""
+    helper, q = self.awq_clip, self.weight_quantizer
+    weight = self.weight
+    q.enable()
+    if helper.is_per_tensor_clip(self):
+        out_actual = inputs @ weight.T
+        original = q.amax.clone()
+        helper.num_tokens += inputs.shape[0]
+        for shrink in helper.loss:
+            q.amax = original * shrink
+            out = inputs @ q(weight).T
+            helper.loss[shrink] += (out - out_actual).float().pow(2).mean()
+        return
+    inputs = inputs.reshape(-1, inputs.shape[-1])
+    inputs = inputs[0::max(1, inputs.shape[0] // max_tokens)]
+    helper.num_tokens += inputs.shape[0]
+    bs = helper.block_size
+    co, ci = weight.shape
+    pad = (bs - ci % bs) % bs
+    if pad:
+        weight = F.pad(weight, (0, pad), "constant", 0)
+        inputs = F.pad(inputs, (0, pad), "constant", 0)
+    w4 = weight.reshape(co, 1, -1, bs)
+    x4 = inputs.reshape(1, inputs.shape[0], -1, bs)
+    quantized = {}
+    for shrink in helper.loss:           # one fake-quant pass over the weight per ratio
+        q.amax = helper.w_amax * shrink
+        wq = q(self.weight)
+        quantized[shrink] = F.pad(wq, (0, pad), "constant", 0) if pad else wq
+    for lo in range(0, co, co_bsz):
+        hi = min(lo + co_bsz, co)
+        org_out = (x4 * w4[lo:hi]).sum(dim=-1)
+        for shrink, wq in quantized.items():
+            cur_out = (x4 * wq[lo:hi].reshape(w4[lo:hi].shape)).sum(dim=-1)
+            helper.loss[shrink][lo:hi] += (cur_out - org_out).float().pow(2).mean(dim=1)
+
+
+def _awq_clip_forward(self, input, *args, **kwargs):
+    helper = self.awq_clip
+    if helper.is_input_quantized:
+        self.input_quantizer.enable()
+        max_calibrate(self.input_quantizer, lambda quantizer: quantizer(input))
+        self.input_quantizer.disable()
+    _awq_clip_search(self, self.input_quantizer(input), helper.max_co_batch_size,
+                     helper.max_tokens_per_batch)
+    self.weight_quantizer.disable()
+    return self._forward_no_awq(input, *args, **kwargs)
+
+
+@torch.no_grad()
+def awq_clip(model: nn.Module, forward_loop, max_co_batch_size: int = 1024,
+             max_tokens_per_batch: int = 64, min_clip_ratio: float = 0.5, shrink_step: float = 0.05,
+             debug: bool = False, **kwargs):
+    """AWQ clip: per weight block, the clipped amax (``ratio * block amax``) that minimises the
+    error of the block's contribution to the layer output on the calibration tokens (reference:
+    model_calib.py:789-997)."""
+    assert forward_loop is not None, "forward_loop must be provided for awq_clip"
+    patched = []
+    for name, module in model.named_modules():
+        if (is_quantized_linear(module) and module.weight_quantizer.is_enabled
+                and module.weight_quantizer.block_sizes is not None):
+            module._forward_no_awq = module.forward
+            module.forward = types.MethodType(_awq_clip_forward, module)
+            module.awq_clip = _AWQClipHelper(module, min_clip_ratio, shrink_step)
+            module.awq_clip.max_co_batch_size = max_co_batch_size
+            module.awq_clip.max_tokens_per_batch = max_tokens_per_batch
+            patched.append(module)
+    print("awq_clip: Estimating parameters...")
+    enable_stats_collection(model)
+    forward_loop(model)
+    max_calibrate(model, lambda m: None)
+    for module in patched:
+        helper = module.awq_clip
+        if helper.num_tokens > 0:
+            helper.best_loss = torch.ones_like(helper.w_amax) * float("inf")
+            helper.best_clip_val = torch.zeros_like(helper.w_amax)
+            for shrink, loss in helper.loss.items():
+                loss = loss.view_as(helper.w_amax)
+                better = loss < helper.best_loss
+                helper.best_loss = torch.where(better, loss, helper.best_loss)
+                helper.best_clip_val = torch.where(better, helper.w_amax * shrink, helper.best_clip_val)
+            module.weight_quantizer.amax = helper.best_clip_val
+            module.weight_quantizer.enable()
+            if helper.is_input_quantized:
+                module.input_quantizer.enable()
+        if not debug:
+            delattr(module, "awq_clip")
+        if "forward" in module.__dict__:
+            del module.__dict__["forward"]
+        if "_forward_no_awq" in module.__dict__:
+            del module.__dict__["_forward_no_awq"]
+
+
 # ----------------------------------------------------------------------------- AWQ-lite
 def awq(model: nn.Module, forward_loop=None, algorithm: str = "awq_lite", **kwargs):
     with SequentialQuantizer.convert_to_single_quantizer(model):
         if algorithm in ("awq_full", "awq_lite"):
             awq_lite(model, forward_loop, **kwargs)
         if algorithm in ("awq_full", "awq_clip"):
-            raise NotImplementedError("awq_clip is outside the hot path built here")
+            clip_args = {k: v for k, v in kwargs.items() if k in (
+                "max_co_batch_size", "max_tokens_per_batch", "min_clip_ratio", "shrink_step", "debug")}
+            awq_clip(model, forward_loop, **clip_args)
     for module in model.modules():
         if is_quantized_linear(module) and isinstance(module.weight_quantizer, SequentialQuantizer):
             max_calibrate(module, lambda lin: lin.weight_quantizer(lin.weight))

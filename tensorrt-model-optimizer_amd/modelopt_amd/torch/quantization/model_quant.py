@@ -68,6 +68,8 @@ def calibrate(model: nn.Module, algorithm="max", forward_loop: ForwardLoop | Non
                                       kwargs.get("stop_multiplier", 4.0))
         elif method == "smoothquant":
             model_calib.smoothquant(model, forward_loop, alpha=kwargs.get("alpha", 1.0))
+        elif method in ("awq_clip", "awq_full"):
+            model_calib.awq(model, forward_loop, method, **kwargs)
         elif method == "awq_lite":
             model_calib.awq(model, forward_loop, "awq_lite", alpha_step=kwargs.get("alpha_step", 0.1),
                             debug=kwargs.get("debug", False))

@@ -361,3 +361,44 @@ def test_true_divide_is_one_rounding_on_the_gpu():
         assert torch.equal(got, want), d
     tb = t[:4096].to(torch.bfloat16)
     assert torch.equal(true_divide(tb.to(DEV), 448.0).cpu(), tb / 448.0)
+
+
+# ----------------------------------------------------------------------------- AWQ-clip
+def test_awq_clip_matches_oracle():
+    ref = _OneLinear(n=64, k=256)
+    model = copy.deepcopy(ref).to(DEV)
+    batches = _awq_batches(k=256, n=2, tokens=96)
+    cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
+    cfg["algorithm"] = {"method": "awq_clip", "max_tokens_per_batch": 32, "debug": True}
+    mtq.quantize(model, cfg, lambda m: [m(b.to(DEV)) for b in batches])
+    losses, best = oawq.awq_clip_search(ref.proj.weight.data, batches, 128, 4, max_tokens_per_batch=32)
+    h = model.proj.awq_clip
+    assert list(h.loss) == list(losses) and len(losses) == 11
+    assert h.num_tokens == 64
+    w_amax = reduce.reduce_amax(ref.proj.weight.data.reshape(-1, 128), axis=[1], keepdims=True)
+    assert_bits_equal(h.w_amax.cpu(), w_amax, "block amax before clipping")
+    # the partial sums are bf16 torch reductions whose last bit can depend on the summation
+    # order; in practice the losses agree to 1e-8 and every block picks the same ratio
+    for r in losses:
+        got, want = h.loss[r].cpu(), losses[r]
+        rel = (got - want).abs().sum() / want.abs().sum().clamp(min=1e-30)
+        assert float(rel) < 1e-4, f"ratio {r}: {float(rel)}"
+    got_best = model.proj.weight_quantizer.amax.cpu()
+    same = (got_best == best).float().mean()
+    assert float(same) >= 0.99, float(same)
+    ratio = (got_best.float() / w_amax.float())
+    assert float(ratio.min()) >= 0.49 and float(ratio.max()) <= 1.0
+    assert model.proj.weight_quantizer.is_enabled and "forward" not in model.proj.__dict__
+    assert torch.isfinite(model(batches[0].to(DEV)).float()).all()
+
+
+def test_awq_full_runs_lite_then_clip():
+    model = _OneLinear(n=64, k=256).to(DEV)
+    batches = _awq_batches(k=256, n=2, tokens=64)
+    cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
+    cfg["algorithm"] = {"method": "awq_full", "alpha_step": 0.25, "debug": True}
+    mtq.quantize(model, cfg, lambda m: [m(b.to(DEV)) for b in batches])
+    assert hasattr(model.proj, "awq_lite") and hasattr(model.proj, "awq_clip")
+    assert model.proj.input_quantizer._pre_quant_scale is not None
+    assert model.proj.weight_quantizer.amax.shape == (64 * 2, 1)
+    assert torch.isfinite(model(batches[0].to(DEV)).float()).all()
