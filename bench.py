@@ -355,6 +355,35 @@ def main():
         w_ms, d_ms = timed(torch, dequant, a.steps, a.warmup)
         extras["dequantize_one_layer"] = {
             "ms": round(d_ms, 4), "GBps": round(e1 * DEQUANT_BYTES_PER_ELEM / d_ms / 1e6, 1)}
+        # what PyTorch-ROCm users get today: the reference's extensions refuse to build without
+        # CUDA, so its NVFP4 weight packing is the eager multi-pass torch code of its QTensor class
+        # run on the device; restated inline here on the first layer's seven weights
+        def eager_pack():
+            for i in range(n1):
+                w = weights[i]
+                wsf2 = amax[i] / (6.0 * 448.0)
+                blocks = w.reshape(*w.shape[:-1], -1, 16)
+                bs = blocks.abs().amax(dim=-1).float() / (6.0 * wsf2)
+                bs = torch.where(bs == 0, torch.ones_like(bs), bs).to(torch.float8_e4m3fn)
+                v = blocks.float() / (bs.float() * wsf2).unsqueeze(-1)
+                a = v.abs()
+                bounds = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0], device=w.device)
+                ordv = torch.searchsorted(bounds, a, out_int32=True)
+                odd = (a == 0.75) | (a == 1.75) | (a == 3.5)
+                codes = ((v < 0).to(torch.uint8) << 3) + (ordv + odd).to(torch.uint8)
+                codes = codes.reshape(*w.shape)
+                (codes[..., 1::2] << 4) | codes[..., 0::2]
+        w_ms, d_ms = timed(torch, eager_pack, 3, 1)
+        extras["eager_torch_pack_one_layer_on_gpu"] = {
+            "ms": round(d_ms, 4), "GBps": round(e1 * QUANT_BYTES_PER_ELEM / d_ms / 1e6, 1)}
+
+        # plain device copy of 4 GiB: the read + write rate the memory system sustains
+        src = torch.empty(1 << 32, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        w_ms, d_ms = timed(torch, lambda: dst.copy_(src), 5, 2)
+        extras["device_copy_4GiB"] = {"ms": round(d_ms, 4), "GBps": round(2 * src.numel() / d_ms / 1e6, 1)}
+        del src, dst
+
         with contextlib.redirect_stdout(sys.stderr):   # the calibration algorithms print progress
             extras["single_tensor_configs"] = single_tensor_configs(torch, a.steps, a.warmup)
         out["extras"] = extras

@@ -273,14 +273,6 @@ __global__ __launch_bounds__(256) void int4_pack_rows_kernel(const void* __restr
 // ------------------------------------------------------------------------------ INT4 fast paths
 // Block sizes of 8 << k elements (k <= 6) on 16-byte aligned tensors: a lane owns a chunk, the
 // lanes of a block combine their abs-max with in-wave shuffles.
-__device__ __forceinline__ uint32_t int4_code(float v) {  // clamp(rne(v), -8, 7) + 8
-    float q = __builtin_rintf(v);
-    q = q < -8.0f ? -8.0f : q;
-    q = q > 7.0f ? 7.0f : q;
-    q += 8.0f;
-    return (q == q) ? ((uint32_t)(int)q & 0xFFu) : 0u;
-}
-
 // clamp(rne(v), -8, 7) as an integer in three operations: v_med3_f32 clamps (and returns the
 // smallest operand, -8, for a NaN, which is the "NaN packs as code 0" rule of the kernels above),
 // adding 1.5 * 2^23 rounds to nearest even and leaves the integer in the low mantissa bits.
