@@ -410,10 +410,46 @@ def get_act_scale(x):
     return (acc / x2.shape[0]).to(x.dtype).to(torch.float32)
 
 
+def _exponent_columns(alphas, device):
+    """fp32 ``[A, 1]`` device columns of ``alpha`` and ``1 - alpha`` (the difference is taken in
+    double, as the scalar form of ``pow`` does before it narrows the exponent)."""
+    a = torch.tensor([float(v) for v in alphas], dtype=torch.float32)
+    b = torch.tensor([1 - float(v) for v in alphas], dtype=torch.float32)
+    return a.to(device)[:, None], b.to(device)[:, None]
+
+
+def _pow_rows(t, exponents, column):
+    """``[A, K]``: row i is ``_pow(t, exponents[i])``.  One broadcast ``pow`` over all rows; the
+    rows whose exponent the scalar form evaluates without calling ``pow`` (0, 1 and 0.5) are
+    then written the way it would write them."""
+    out = torch.pow(t.view(1, -1), column)
+    for i, e in enumerate(exponents):
+        if e == 0.0:
+            out[i].fill_(1.0)
+        elif e == 1.0:
+            out[i].copy_(t.view(-1))
+        elif e == 0.5:
+            out[i].copy_(_pow(t.view(-1), 0.5))
+    return out
+
+
+def get_scales(x_max, w_max, alphas, columns=None):
+    """fp32 ``[len(alphas), K]``: row i is the AWQ scale ``x^a / w^(1-a)`` for ``a = alphas[i]``,
+    clamped to [1e-4, 1e4] and normalised by ``sqrt(max * min)`` of its own row.  The whole
+    search grid takes a fixed number of launches instead of a dozen per alpha."""
+    dev = x_max.device
+    col_a, col_b = columns if columns is not None else _exponent_columns(alphas, dev)
+    num = _pow_rows(x_max.float(), [float(v) for v in alphas], col_a)
+    den = _pow_rows(w_max.to(dev).float(), [1 - float(v) for v in alphas], col_b)
+    scales = (num / (den + torch.finfo(torch.float32).tiny)).clamp_(min=1e-4, max=1e4)
+    norm = (scales.amax(1, keepdim=True) * scales.amin(1, keepdim=True)).sqrt_()
+    return scales.div_(norm)
+
+
 def get_scale(x_max, w_max, alpha):
-    scales = (_pow(x_max, alpha) / (_pow(w_max.to(x_max.device), 1 - alpha)
-                                  + torch.finfo(torch.float32).tiny)).clamp(min=1e-4, max=1e4).view(-1)
-    return (scales / (scales.max() * scales.min()).sqrt()).view(-1)
+    """fp32 ``[K]``: the AWQ scale for one ``alpha`` (a one-row ``get_scales``, so the folded
+    scale is bit for bit the one the search scored)."""
+    return get_scales(x_max, w_max, [alpha])[0]
 
 
 class _AWQLiteHelper:
@@ -432,6 +468,7 @@ class _AWQLiteHelper:
         self.loss = {a: 0.0 for a in self.alphas}
         self.best_scale = None
         self.best_alpha = None
+        self.exponent_columns = None  # device copies of alpha and 1 - alpha, made on first search step
         self.is_input_quantized = module.input_quantizer.is_enabled
         self.num_tokens = 0
         self.module = module
@@ -501,18 +538,25 @@ def _awq_forward(self, input, *args, **kwargs):
     dtype = self.weight.dtype
     fused = _fused_weight_path(self) and not args and not kwargs
     sq_err = torch.zeros(len(helper.alphas), dtype=torch.float64, device=ref.device)
-    for i, alpha in enumerate(helper.alphas):
-        awq_scale = get_scale(helper.act_scale, helper.weight_scale, alpha)
+    if helper.exponent_columns is None or helper.exponent_columns[0].device != ref.device:
+        helper.exponent_columns = _exponent_columns(helper.alphas, ref.device)
+    scales = get_scales(helper.act_scale, helper.weight_scale, helper.alphas, helper.exponent_columns)
+    w_scales = scales.to(dtype)
+    x_scales = (1 / scales).to(dtype)
+    if fused:
+        q = self.weight_quantizer
+        x_in = input.contiguous()
+        w_in = self.weight.data.contiguous()
+        block = _awq_block_size(self.weight, q)
+    for i in range(len(helper.alphas)):
         if fused:
-            q = self.weight_quantizer
-            xs = self.input_quantizer(_hip.mul_cols(input.contiguous(), (1 / awq_scale).to(dtype)))
-            wq = _hip.scale_block_int_qdq(self.weight.data.contiguous(), awq_scale.to(dtype),
-                                          _awq_block_size(self.weight, q), q._num_bits, q._unsigned,
+            xs = self.input_quantizer(_hip.mul_cols(x_in, x_scales[i]))
+            wq = _hip.scale_block_int_qdq(w_in, w_scales[i], block, q._num_bits, q._unsigned,
                                           q._narrow_range)
             out = self.output_quantizer(F.linear(xs, wq, self.bias))
         else:
-            self.input_quantizer.pre_quant_scale = (1 / awq_scale).to(dtype)
-            self.weight_quantizer.pre_quant_scale = awq_scale.to(dtype)
+            self.input_quantizer.pre_quant_scale = x_scales[i]
+            self.weight_quantizer.pre_quant_scale = w_scales[i]
             out = self._forward_no_awq(input, *args, **kwargs)
             out = out[0] if isinstance(out, tuple) else out
         _hip.sq_diff_sum_into(out.contiguous(), ref, sq_err[i:i + 1])
