@@ -235,6 +235,25 @@ int mo_int4_block_quantize(const void* x, int64_t n, int64_t block_size, int dty
 int mo_int4_block_dequantize(const uint8_t* packed, int64_t nbytes, int64_t block_size,
                              const void* scales, void* y, int dtype, void* stream);
 
+/* ------------------------------------------------------------------ NF4 weight compression
+ * Flat blocks of block_size elements over the n elements of x (tail zero padded).
+ * scales[b] = max |x| over block b (dtype T); v = T(f32(x) / f32(scales[b]));
+ * code = index of the entry of the bf16-rounded NF4 table nearest to v, distances T(|v - e|)
+ * compared after rounding to T, lowest index among equal distances, 0 for NaN;
+ * packed[i] = code[2i] << 4 | code[2i + 1].  scales has ceil(n / block_size) elements, packed
+ * ceil(n / block_size) * block_size / 2 bytes.  Replaces NF4_quantize
+ * (TQ/src/tensor_quant_gpu.cu:211-258) with the CPU numerics of NF4QTensor.quantize
+ * (TQ/qtensor/nf4_tensor.py:76-126); the block abs-max is computed here instead of by a
+ * separate reduce_amax pass. */
+int mo_nf4_quantize(const void* x, int64_t n, int64_t block_size, int dtype, void* scales,
+                    uint8_t* packed, void* stream);
+
+/* y[2i] = T(table[packed[i] >> 4] * f32(scales[2i / block_size])), y[2i + 1] likewise for the
+ * low nibble; scales and y have dtype T.  Replaces NF4_dequantize
+ * (TQ/src/tensor_quant_gpu.cu:146-197) / NF4QTensor.dequantize (TQ/qtensor/nf4_tensor.py:157-201). */
+int mo_nf4_dequantize(const uint8_t* packed, int64_t nbytes, int64_t block_size,
+                      const void* scales, void* y, int dtype, void* stream);
+
 /* INT4-AWQ export pack of w[batch, n_rows, k] with fp32 scales ws[batch, n_rows, k/block_size]:
  * q = int8(clamp(rne(f32(w) / ws), -8, 7)); out[b, j, c] = (q[b, 2j, c] & 0xF) |
  * (q[b, 2j+1, c] << 4), out is uint8 [batch, n_rows / 2, k].  Replaces pack_int4_in_uint8

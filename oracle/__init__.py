@@ -40,10 +40,12 @@ export.pack_int4_in_uint8              PARITY UNPINNED by reference tests (no go
                                        the unpack(pack(q)) == q invariant
 export.fp8_export_cast                 PARITY UNPINNED by reference tests; pinned by the torch
                                        type-promotion rule probed in tests (bf16 / 0-dim fp32)
+nf4.nf4_quantize / double_quantization golden round trips test_qtensor_cuda.py:111-131 (with and
+/ nf4_dequantize                       without padding), :30-68; per-element Python brute force
 awq.awq_lite / smoothquant             the reference's own independent oracle ``awq_lite_manual``
                                        tests/unit/torch/quantization/test_calib.py:53-118
                                        (restated in tests) + closed forms
 =====================================  =========================================================
 """
 
-from . import awq, export, fake_quant, qtensor, reduce  # noqa: F401
+from . import awq, export, fake_quant, nf4, qtensor, reduce  # noqa: F401

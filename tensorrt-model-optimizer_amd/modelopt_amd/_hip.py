@@ -41,6 +41,8 @@ SIGNATURES = {
     "mo_int4_block_quantize": [_P, _I64, _I64, _INT, _P, _P, _P],
     "mo_int4_block_dequantize": [_P, _I64, _I64, _P, _P, _INT, _P],
     "mo_int4_pack_rows": [_P, _I64, _I64, _I64, _I64, _INT, _P, _P, _P],
+    "mo_nf4_quantize": [_P, _I64, _I64, _INT, _P, _P, _P],
+    "mo_nf4_dequantize": [_P, _I64, _I64, _P, _P, _INT, _P],
     "mo_mul_cols": [_P, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_scale_block_int_qdq": [_P, _I64, _I64, _INT, _P, _INT, _I64, _INT, _INT, _INT, _P, _P],
     "mo_abs_colsum": [_P, _I64, _I64, _INT, _P, _I64, _P, _P],
@@ -286,6 +288,31 @@ def int4_block_dequantize(packed, scales, block_size):
     assert packed.is_contiguous() and scales.is_contiguous()
     y = torch.empty(packed.numel() * 2, dtype=scales.dtype, device=packed.device)
     call("mo_int4_block_dequantize", packed, _ptr(packed), packed.numel(), block_size, _ptr(scales),
+         _ptr(y), dtype_code(scales.dtype), _stream(packed))
+    return y
+
+
+def nf4_quantize(x, block_size):
+    """Flat-block NF4 quantize + pack: returns (packed uint8 [padded_numel / 2], per-block
+    abs-max [nblocks] in the dtype of x)."""
+    _require_device(x)
+    assert x.is_contiguous()
+    n = x.numel()
+    nblocks = -(-n // block_size)
+    scales = torch.empty(nblocks, dtype=x.dtype, device=x.device)
+    packed = torch.empty(nblocks * block_size // 2, dtype=torch.uint8, device=x.device)
+    call("mo_nf4_quantize", x, _ptr(x), n, block_size, dtype_code(x.dtype), _ptr(scales),
+         _ptr(packed), _stream(x))
+    return packed, scales
+
+
+def nf4_dequantize(packed, scales, block_size):
+    """``table[code] * scale`` in the dtype of ``scales``: [2 * packed.numel()]."""
+    _require_device(packed, scales)
+    assert packed.is_contiguous() and scales.is_contiguous()
+    assert scales.numel() * block_size >= packed.numel() * 2
+    y = torch.empty(packed.numel() * 2, dtype=scales.dtype, device=packed.device)
+    call("mo_nf4_dequantize", packed, _ptr(packed), packed.numel(), block_size, _ptr(scales),
          _ptr(y), dtype_code(scales.dtype), _stream(packed))
     return y
 

@@ -1,10 +1,9 @@
 """``TensorQuantizer`` and ``SequentialQuantizer``.
 
-Attribute names, buffers (``_amax``, ``_pre_quant_scale``, ``_scale``, ``_double_scale``), the
-order of operations in ``forward`` and the exported amax shapes follow the reference module
-(modelopt/torch/quantization/nn/modules/tensor_quantizer.py:65-1225); the arithmetic runs in the
-HIP kernels.  Not built: affine bias, Hadamard rotation, MX (E8M0-scaled) formats, NF4 double
-quantisation, ONNX export hooks.
+Attribute names, buffers (``_amax``, ``_pre_quant_scale``, ``_scale``, ``_double_scale``,
+``_scale_zeros``), the order of operations in ``forward`` and the exported amax shapes follow
+the reference module (modelopt/torch/quantization/nn/modules/tensor_quantizer.py:65-1225); the
+arithmetic runs in the HIP kernels.  Not built: affine bias, Hadamard rotation, ONNX export hooks.
 """
 
 import contextlib
@@ -20,7 +19,7 @@ from ... import calib, kernels
 from ... import utils as quant_utils
 from ...config import QuantizerAttributeConfig
 from ...qtensor import (BaseQuantizedTensor, FP8QTensor, INT4QTensor, INT8QTensor, MXFP4QTensor,
-                        NVFP4QTensor, QTensorWrapper)
+                        NF4QTensor, NVFP4QTensor, QTensorWrapper)
 from ...tensor_quant import dynamic_block_quant, fake_tensor_quant, scaled_e4m3
 
 __all__ = ["SequentialQuantizer", "TensorQuantizer"]
@@ -328,7 +327,10 @@ class TensorQuantizer(nn.Module):
             outputs, scale = INT8QTensor.quantize(inputs, axis=self._axis, block_sizes=bs)
             buffers["_scale"] = scale
         elif bs.get("scale_bits", 0) == 8 and bs.get("scale_block_sizes"):
-            raise NotImplementedError("NF4 double quantisation is outside the hot path built here")
+            sbs = bs["scale_block_sizes"][-1]
+            outputs, scales = NF4QTensor.quantize(inputs, bs[-1], sbs)
+            scale, double_scale, zeros = NF4QTensor.double_quantization(scales, sbs, bs["scale_bits"])
+            buffers["_scale"], buffers["_double_scale"], buffers["_scale_zeros"] = scale, double_scale, zeros
         elif bs.get("scale_bits") == (8, 0) and bs.get("type") == "dynamic":
             if self._num_bits != (2, 1):
                 raise NotImplementedError("of the MX formats only MXFP4 has a packed tensor class")

@@ -42,6 +42,18 @@ V["qtensor_roundtrip"] = [
      "output": [[0, 1, 2, 3], [4, 5, 6, 7]]},
 ]
 
+# tests/gpu/torch/quantization/test_qtensor_cuda.py:111-131 (test_qtensor_accuracy, NF4 rows): real
+# quantize through TensorQuantizer (4-bit table codes, int8 double-quantised scales) then
+# dequantize; bf16 in, expected bf16 out (torch.allclose), cpu and cuda.
+V["nf4_roundtrip"] = [
+    {"name": "nf4_block2", "block_size": 2, "scale_block_size": 4, "scale_bits": 8,
+     "input": [[0, 1, 2, 3, 4, 5, 6, 7]],
+     "output": [[0.0000, 1.0156, 2.1719, 3.0156, 3.6094, 5.0000, 5.0625, 7.0000]]},
+    {"name": "nf4_block2_padding", "block_size": 2, "scale_block_size": 4, "scale_bits": 8,
+     "input": [[0, 1, 2, 3, 4, 5, 7]],
+     "output": [[0.0000, 1.0156, 2.1719, 3.0156, 3.6094, 5.0000, 7.0000]]},
+]
+
 # tests/gpu/torch/quantization/test_qtensor_cuda.py:254-375 (test_nvfp4_quantize): block size 8,
 # dtypes fp32/fp16/bf16, cpu and cuda; dequantised values allclose(x, rtol=2e-1, atol=2e-1).
 V["nvfp4_quantize_inputs"] = [

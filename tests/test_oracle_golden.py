@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from conftest import GOLDEN, assert_bits_equal
-from oracle import export, fake_quant, qtensor, reduce
+from oracle import export, fake_quant, nf4, qtensor, reduce
 
 with open(os.path.join(GOLDEN, "reference_vectors.json")) as f:
     VEC = json.load(f)
@@ -264,3 +264,38 @@ def test_fp8_export_cast_double_rounding_rule():
     once = (w.float() / wsf).to(torch.float8_e4m3fn)
     assert_bits_equal(export.fp8_export_cast(w, wsf.reshape(1)), once, "1-elem scale")
     assert (twice.view(torch.uint8) != once.view(torch.uint8)).any()
+
+
+# ----------------------------------------------------------------------------- NF4
+def _nf4_roundtrip(x, block, sblock, bits, dtype=None):
+    packed, scales = nf4.nf4_quantize(x, block, sblock)
+    q, factor, zero = nf4.double_quantization(scales, sblock, bits)
+    return nf4.nf4_dequantize(packed, q, factor, zero, block, x.shape, dtype or x.dtype)
+
+
+@pytest.mark.parametrize("case", VEC["nf4_roundtrip"], ids=lambda c: c["name"])
+def test_nf4_roundtrip_golden(case):
+    x = torch.tensor(case["input"], dtype=torch.bfloat16)
+    want = torch.tensor(case["output"], dtype=torch.bfloat16)
+    got = _nf4_roundtrip(x, case["block_size"], case["scale_block_size"], case["scale_bits"])
+    assert torch.allclose(got, want), (got, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(256, 64), (256, 32)])
+def test_nf4_roundtrip_close(dtype, shape):
+    """tests/gpu/torch/quantization/test_qtensor_cuda.py:30-68: uniform [0, 1) input, block 64,
+    scale block 256, round trip within rtol = atol = 0.1."""
+    x = torch.rand(shape, generator=torch.Generator().manual_seed(0)).to(dtype)
+    got = _nf4_roundtrip(x, 64, 256, 8)
+    assert got.dtype == dtype and torch.allclose(got, x, rtol=1e-1, atol=1e-1)
+
+
+def test_nf4_nearest_index_brute_force():
+    """The table search against a per-element Python loop over the bf16 table (first minimum)."""
+    lut = nf4.NF4_TABLE
+    v = torch.linspace(-1, 1, 4001).to(torch.bfloat16)
+    got = nf4.nearest_table_index(v, lut)
+    for x, g in zip(v.tolist(), got.tolist()):
+        diffs = [abs(float((torch.tensor(x, dtype=torch.bfloat16) - e))) for e in lut]
+        assert g == diffs.index(min(diffs))
