@@ -57,6 +57,17 @@ int mo_get_option(int key);
 int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
               float* acc, void* stream);
 
+/* The per-column case of mo_absmax (x viewed as [outer, axis], inner == 1) in two passes through
+ * a caller-provided workspace: row slabs are reduced to partial[slabs, axis] with plain stores
+ * (slabs <= partial_rows, chosen by the library), then the columns of that matrix are folded
+ * into acc.  Same result as mo_absmax; it avoids the atomic traffic of a fresh accumulator
+ * (one atomic per column per workgroup), which dominates when outer * axis is large.
+ * partial: device buffer of partial_rows * axis 32-bit words, 16-byte aligned, contents
+ * ignored on entry.  Returns MO_ERR_UNSUPPORTED when axis % 8 != 0 or x is not 16-byte
+ * aligned (use mo_absmax then).  Replaces the same reference code as mo_absmax. */
+int mo_absmax_cols_staged(const void* x, int64_t outer, int64_t axis, int dtype, float* acc,
+                          void* partial, int64_t partial_rows, void* stream);
+
 /* Per-tensor abs-max of many tensors in ONE launch.  jobs_dev is a device-resident table sorted
  * by tile_begin; job j owns tiles [tile_begin_j, tile_begin_j + ceil(elems_j /
  * MO_ABSMAX_TILE_ELEMS)), total_tiles is the sum (< 2^31).  tile_job_dev[t] = index of the job

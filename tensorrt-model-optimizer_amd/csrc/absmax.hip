@@ -173,7 +173,11 @@ __global__ __launch_bounds__(256) void absmax_short_rows_kernel(const void* __re
 // x viewed as [outer, axis] (inner == 1).  Vector path (axis % 8 == 0, aligned): a lane owns 8
 // adjacent columns, a wavefront 512; the four wavefronts of a workgroup take interleaved rows of
 // a slab, combine through LDS and fold once per column.  Scalar path: one column per lane.
-template <int DT>
+// STAGED: instead of folding into acc[axis] with atomics, the workgroup of row slab blockIdx.y
+// stores its maxima to row blockIdx.y of acc[gridDim.y, axis] with plain stores (a second pass
+// reduces those rows).  With a fresh accumulator every workgroup of the first wave would
+// otherwise issue one atomic per column, millions in total, served a few per cache line at a time.
+template <int DT, bool STAGED>
 __global__ __launch_bounds__(256) void absmax_cols8_kernel(const void* __restrict__ x,
                                                            int64_t outer, int64_t axis,
                                                            int64_t slab,
@@ -237,14 +241,15 @@ __global__ __launch_bounds__(256) void absmax_cols8_kernel(const void* __restric
             v = smem[1][t] > v ? smem[1][t] : v;
             v = smem[2][t] > v ? smem[2][t] : v;
             v = smem[3][t] > v ? smem[3][t] : v;
-            fold_max(acc + c, v);
+            if constexpr (STAGED) acc[(int64_t)blockIdx.y * axis + c] = v;
+            else fold_max(acc + c, v);
         }
     }
 }
 
 // Wide variant for axis >= 2048: a workgroup spans 2048 adjacent columns (4 KiB of a bf16 row per
 // load instruction round), every lane keeps its 8 columns for the whole slab of rows -- no LDS.
-template <int DT>
+template <int DT, bool STAGED>
 __global__ __launch_bounds__(256) void absmax_cols8_wide_kernel(const void* __restrict__ x,
                                                                 int64_t outer, int64_t axis,
                                                                 int64_t slab,
@@ -306,8 +311,15 @@ __global__ __launch_bounds__(256) void absmax_cols8_wide_kernel(const void* __re
             m[2 * j + 1] = DT == MO_BF16 ? hi << 16 : f2u(f16_bits_to_f32(hi));
         }
     }
+    if constexpr (STAGED) {
+        u32x4* dst = (u32x4*)(acc + (int64_t)blockIdx.y * axis + col);
+        const u32x4 lo = {m[0], m[1], m[2], m[3]}, hi = {m[4], m[5], m[6], m[7]};
+        dst[0] = lo;
+        dst[1] = hi;
+    } else {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) fold_max(acc + col + j, m[j]);
+        for (int j = 0; j < 8; ++j) fold_max(acc + col + j, m[j]);
+    }
 }
 
 template <int DT>
@@ -394,9 +406,9 @@ static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
             if (ws < 16) ws = 16;
             wy = (outer + ws - 1) / ws;
             if (wy > 65535) { wy = 65535; ws = (outer + wy - 1) / wy; wy = (outer + ws - 1) / ws; }
-            absmax_cols8_wide_kernel<DT><<<dim3((unsigned)wx, (unsigned)wy), 256, 0, s>>>(x, outer, axis, ws, acc);
+            absmax_cols8_wide_kernel<DT, false><<<dim3((unsigned)wx, (unsigned)wy), 256, 0, s>>>(x, outer, axis, ws, acc);
         } else if (vec)
-            absmax_cols8_kernel<DT><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
+            absmax_cols8_kernel<DT, false><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
         else
             absmax_cols1_kernel<DT><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
         return MO_OK;
@@ -439,6 +451,62 @@ static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
     return MO_OK;
 }
 
+// Second pass of the staged per-column reduction: acc[c] = max(acc[c], max over rows of
+// partial[r, c]).  A workgroup owns 32 columns (eight lanes-groups take interleaved rows, then
+// combine through LDS), so the accumulator is updated by plain stores from its only writer.
+__global__ __launch_bounds__(256) void absmax_fold_partials_kernel(
+    const uint32_t* __restrict__ partial, int64_t rows, int64_t axis, uint32_t* __restrict__ acc) {
+    __shared__ uint32_t smem[8][32];
+    const int c = threadIdx.x & 31, g = threadIdx.x >> 5;
+    const int64_t col = (int64_t)blockIdx.x * 32 + c;
+    uint32_t m = 0;
+    if (col < axis) {
+        int64_t r = g;
+        for (; r + 24 < rows; r += 32) {
+            uint32_t v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = partial[(r + 8 * u) * axis + col];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) m = v[u] > m ? v[u] : m;
+        }
+        for (; r < rows; r += 8) {
+            const uint32_t v = partial[r * axis + col];
+            m = v > m ? v : m;
+        }
+    }
+    smem[g][c] = m;
+    __syncthreads();
+    if (g == 0 && col < axis) {
+#pragma unroll
+        for (int k = 1; k < 8; ++k) m = smem[k][c] > m ? smem[k][c] : m;
+        const uint32_t old = acc[col];
+        if (m > old) acc[col] = m;
+    }
+}
+
+// Per-column abs-max in two passes: row slabs -> partial[slabs, axis] (plain stores), then the
+// columns of that small matrix into acc.  No atomics.
+template <int DT>
+static int launch_absmax_cols_staged(const void* x, int64_t outer, int64_t axis, uint32_t* acc,
+                                     uint32_t* partial, int64_t partial_rows, hipStream_t s) {
+    if ((((uintptr_t)x | (uintptr_t)partial) & 15u) || (axis % 8)) return MO_ERR_UNSUPPORTED;
+    int64_t slabs = partial_rows < 65535 ? partial_rows : 65535;
+    int64_t rows = (outer + slabs - 1) / slabs;
+    rows = (rows + 3) / 4 * 4;  // the 16-bit paths take rows in groups of four
+    slabs = (outer + rows - 1) / rows;
+    if (axis >= 2048) {
+        const int64_t wx = (axis + 2047) / 2048;
+        absmax_cols8_wide_kernel<DT, true><<<dim3((unsigned)wx, (unsigned)slabs), 256, 0, s>>>(
+            x, outer, axis, rows, partial);
+    } else {
+        const int64_t gx = (axis + 511) / 512;
+        absmax_cols8_kernel<DT, true><<<dim3((unsigned)gx, (unsigned)slabs), 256, 0, s>>>(
+            x, outer, axis, rows, partial);
+    }
+    absmax_fold_partials_kernel<<<dim3((unsigned)((axis + 31) / 32)), 256, 0, s>>>(partial, slabs, axis, acc);
+    return MO_OK;
+}
+
 }  // namespace mo
 
 extern "C" int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
@@ -472,5 +540,23 @@ extern "C" int mo_absmax_multi(const mo_absmax_job* jobs_dev, int njobs,
         case MO_BF16: mo::absmax_multi_kernel<MO_BF16><<<grid, 256, 0, s>>>(jobs_dev, njobs, tile_job_dev); break;
         default: return MO_ERR_DTYPE;
     }
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_absmax_cols_staged(const void* x, int64_t outer, int64_t axis, int dtype,
+                                     float* acc, void* partial, int64_t partial_rows,
+                                     void* stream) {
+    if (outer < 0 || axis < 0 || partial_rows < 1) return MO_ERR_ARG;
+    if (outer == 0 || axis == 0) return MO_OK;
+    if (!x || !acc || !partial) return MO_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    int rc;
+    switch (dtype) {
+        case MO_F32: rc = mo::launch_absmax_cols_staged<MO_F32>(x, outer, axis, (uint32_t*)acc, (uint32_t*)partial, partial_rows, s); break;
+        case MO_F16: rc = mo::launch_absmax_cols_staged<MO_F16>(x, outer, axis, (uint32_t*)acc, (uint32_t*)partial, partial_rows, s); break;
+        case MO_BF16: rc = mo::launch_absmax_cols_staged<MO_BF16>(x, outer, axis, (uint32_t*)acc, (uint32_t*)partial, partial_rows, s); break;
+        default: return MO_ERR_DTYPE;
+    }
+    if (rc != MO_OK) return rc;
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

@@ -25,6 +25,7 @@ SIGNATURES = {
     "mo_set_option": [_INT, _INT],
     "mo_get_option": [_INT],
     "mo_absmax": [_P, _I64, _I64, _I64, _INT, _P, _P],
+    "mo_absmax_cols_staged": [_P, _I64, _I64, _INT, _P, _P, _I64, _P],
     "mo_absmax_multi": [_P, _INT, _P, _I64, _INT, _P],
     "mo_nvfp4_quantize_multi": [_P, _INT, _P, _I64, _INT, _INT, _INT, _P],
     "mo_fp8_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _P],
@@ -114,6 +115,15 @@ def absmax_into(x: torch.Tensor, acc: torch.Tensor, outer: int, axis: int, inner
     _require_device(x, acc)
     assert x.is_contiguous() and acc.dtype == torch.float32 and acc.numel() == axis
     assert outer * axis * inner == x.numel()
+    if inner == 1 and axis % 8 == 0 and outer >= 64 and x.data_ptr() % 16 == 0:
+        # per column over many rows: row slabs go to a small workspace first, so that a fresh
+        # accumulator is not hit by one atomic per column from every workgroup
+        across = -(-axis // 2048) if axis >= 2048 else -(-axis // 512)
+        slabs = max(1, min(-(-1024 // across), outer // 32))
+        partial = torch.empty((slabs, axis), dtype=torch.int32, device=x.device)
+        call("mo_absmax_cols_staged", x, _ptr(x), outer, axis, dtype_code(x.dtype), _ptr(acc),
+             _ptr(partial), slabs, _stream(x))
+        return acc
     call("mo_absmax", x, _ptr(x), outer, axis, inner, dtype_code(x.dtype), _ptr(acc), _stream(x))
     return acc
 

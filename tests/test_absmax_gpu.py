@@ -82,3 +82,31 @@ def test_unaligned_view():
     acc = torch.zeros(1, dtype=torch.float32, device=DEV)
     _hip.absmax_into(v, acc, 1, 1, v.numel())
     assert_bits_equal(acc.cpu().reshape(()).to(torch.bfloat16), reduce.reduce_amax(v.cpu()), "offset view")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(64, 8), (65, 2048), (1000, 4096), (333, 520), (8192, 8192), (4097, 2056)])
+def test_per_column_staged_path(dtype, shape):
+    """Tall matrices take the two-pass route (row slabs -> workspace -> columns); ragged row
+    counts, both column widths (LDS and wide kernel), NaN / inf columns, and a warm accumulator."""
+    x = _rand(shape, dtype, 11)
+    x[shape[0] // 2, 3] = float("nan")
+    x[shape[0] - 1, 5] = float("-inf")
+    want = reduce.reduce_amax(x, axis=[0], keepdims=False)
+    xd = x.to(DEV)
+    acc = torch.zeros(shape[1], dtype=torch.float32, device=DEV)
+    _hip.absmax_into(xd, acc, shape[0], shape[1], 1)
+    assert_bits_equal(acc.cpu().to(dtype), want, f"fresh {shape}")
+    # the single-pass entry point gives the same accumulator
+    direct = torch.zeros(shape[1], dtype=torch.float32, device=DEV)
+    _hip.call("mo_absmax", xd, xd.data_ptr(), shape[0], shape[1], 1, _hip.dtype_code(dtype),
+              direct.data_ptr(), _hip._stream(xd))
+    assert_bits_equal(acc.cpu(), direct.cpu(), f"staged vs direct {shape}")
+    # running maximum: a second, smaller tensor leaves it alone; a larger one raises it
+    _hip.absmax_into((xd * 0.5).nan_to_num(0.0, 0.0, 0.0), acc, shape[0], shape[1], 1)
+    assert_bits_equal(acc.cpu().to(dtype), want, f"warm, smaller {shape}")
+    big = _rand(shape, dtype, 12) * 4
+    _hip.absmax_into(big.to(DEV), acc, shape[0], shape[1], 1)
+    want2 = torch.maximum(want.float(), reduce.reduce_amax(big, axis=[0], keepdims=False).float())
+    want2[3] = float("nan")
+    assert_bits_equal(acc.cpu(), want2, f"warm, larger {shape}")
