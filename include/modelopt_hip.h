@@ -294,6 +294,25 @@ int mo_scale_block_int_qdq(const void* x, int64_t rows, int64_t k, int dtype, co
 int mo_abs_colsum(const void* x, int64_t rows, int64_t k, int dtype, const float* blk_amax,
                   int64_t block_size, float* acc, void* stream);
 
+/* AWQ-lite search step for a whole grid of alphas in one launch (bf16 only):
+ *   q_a = block INT-N quantise-dequantise (blocks of block_size along k, dynamic abs-max) of
+ *         bf16(w * s[a]);   out_a = bf16(xs[a] @ q_a^T)   (fp32 accumulation on the matrix cores)
+ *   loss[a] += sum over (t, n) of f32(bf16(out_a[t, n] - ref[t, n]))^2
+ * xs holds the activations already multiplied by 1 / s[a], chunk-major: [n_alpha][k / 8][tokens][8]
+ * (element (t, c) of alpha a at ((a * (k / 8) + c / 8) * tokens + t) * 8 + c % 8), so that the
+ * lanes of a matrix-core operand read adjacent memory; w [n, k]; s [n_alpha, k]; ref [tokens, n];
+ * loss: n_alpha doubles, accumulated into.  The quantised weights
+ * and the outputs never reach memory.  Returns MO_ERR_UNSUPPORTED unless dtype is bf16,
+ * tokens <= 512, n % 64 == 0, k % 128 == 0, block_size is 32, 64 or 128 and the buffers are
+ * 16-byte aligned (use mo_scale_block_int_qdq + a GEMM + mo_sq_diff_sum per alpha then).
+ * Replaces the per-alpha loop of the search forward, TQ/model_calib.py:645-690 (weight
+ * pre-quant scale, TQ/nn/modules/tensor_quantizer.py:881-882; dynamic block amax :505-514;
+ * _tensor_quant TQ/tensor_quant.py:574-612; update_loss TQ/model_calib.py:623-627). */
+int mo_awq_search_losses(const void* xs, const void* w, const void* s, const void* ref,
+                         int64_t n_alpha, int64_t tokens, int64_t n, int64_t k, int dtype,
+                         int64_t block_size, int num_bits, int is_unsigned, int narrow_range,
+                         double* loss, void* stream);
+
 /* acc[0] += sum of f32(T(a[i] - b[i]))^2 in double: the numerator of update_loss
  * (TQ/model_calib.py:623-627). */
 int mo_sq_diff_sum(const void* a, const void* b, int64_t n, int dtype, double* acc, void* stream);

@@ -46,6 +46,7 @@ SIGNATURES = {
     "mo_nf4_dequantize": [_P, _I64, _I64, _P, _P, _INT, _P],
     "mo_mul_cols": [_P, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_scale_block_int_qdq": [_P, _I64, _I64, _INT, _P, _INT, _I64, _INT, _INT, _INT, _P, _P],
+    "mo_awq_search_losses": [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _INT, _I64, _INT, _INT, _INT, _P, _P],
     "mo_abs_colsum": [_P, _I64, _I64, _INT, _P, _I64, _P, _P],
     "mo_sq_diff_sum": [_P, _P, _I64, _INT, _P, _P],
 }
@@ -338,6 +339,42 @@ def int4_pack_rows(w, ws):
     call("mo_int4_pack_rows", w, _ptr(w), batch, n, k, bs, dtype_code(w.dtype), _ptr(ws), _ptr(out),
          _stream(w))
     return out
+
+
+def awq_scaled_activations(x, inv_s):
+    """``T(x * inv_s[a])`` for every row a of ``inv_s`` in the layout the search kernel reads:
+    [n_alpha, K / 8, tokens, 8] (the 8-element chunks of a column group are contiguous over
+    tokens, so that the lanes of a matrix-core operand read adjacent memory)."""
+    n_alpha, k = inv_s.shape
+    tokens = x.shape[0]
+    xs = x[None] * inv_s[:, None, :]
+    return xs.view(n_alpha, tokens, k // 8, 8).transpose(1, 2).contiguous()
+
+
+def awq_search_losses_into(xs, w, s, ref, block_size, num_bits, unsigned, narrow_range, loss):
+    """loss[a] += squared error of ``bf16(x_a @ qdq(bf16(w * s[a]))^T)`` against ``ref``, all
+    alphas in one launch; ``xs`` = ``awq_scaled_activations(x, 1 / s)``.  Returns False (nothing
+    launched) when the shapes or dtype are outside what the kernel covers."""
+    _require_device(xs, w, s, ref, loss)
+    n_alpha, kc, tokens, eight = xs.shape
+    k = kc * 8
+    n = w.shape[0]
+    assert eight == 8
+    assert xs.is_contiguous() and w.is_contiguous() and s.is_contiguous() and ref.is_contiguous()
+    assert w.shape == (n, k) and s.shape == (n_alpha, k) and ref.shape == (tokens, n)
+    assert loss.dtype == torch.float64 and loss.numel() == n_alpha and loss.is_contiguous()
+    if not (xs.dtype == w.dtype == s.dtype == ref.dtype == torch.bfloat16):
+        return False
+    lib = load()
+    with torch.cuda.device(xs.device):
+        rc = lib.mo_awq_search_losses(_ptr(xs), _ptr(w), _ptr(s), _ptr(ref), n_alpha, tokens, n, k,
+                                      MO_BF16, block_size, int(num_bits), int(bool(unsigned)),
+                                      int(bool(narrow_range)), _ptr(loss), _stream(xs))
+    if rc == MO_ERR_UNSUPPORTED:
+        return False
+    if rc != 0:
+        raise RuntimeError(f"mo_awq_search_losses failed: {lib.mo_error_string(rc).decode()} (status {rc})")
+    return True
 
 
 def mul_cols(x, s, out=None):

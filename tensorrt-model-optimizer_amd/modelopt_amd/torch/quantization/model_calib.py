@@ -512,6 +512,28 @@ def _fused_weight_path(module):
         torch.bfloat16, torch.float16, torch.float32)
 
 
+def _one_launch_search(module, x, w, ref, x_scales, w_scales, block, sq_err) -> bool:
+    """All alphas of a search step in one kernel launch (weights quantised on the fly in front
+    of the matrix cores, the loss reduced in the epilogue): used when the layer is a plain bf16
+    linear without bias whose input and output quantizers are switched off and the batch has at
+    most 512 tokens -- the regime where per-alpha launches and the repeated weight pass dominate.
+    Returns False, with nothing launched and ``sq_err`` untouched, when that is not the case."""
+    if module.bias is not None or w.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
+        return False
+    for name in ("input_quantizer", "output_quantizer"):
+        quantizer = getattr(module, name, None)
+        if not isinstance(quantizer, TensorQuantizer) or quantizer.is_enabled:
+            return False
+    k = w.shape[1]
+    tokens = x.numel() // k
+    if tokens > 512 or k % 8:
+        return False
+    q = module.weight_quantizer
+    xs = _hip.awq_scaled_activations(x.view(tokens, k), x_scales)
+    return _hip.awq_search_losses_into(xs, w, w_scales, ref.view(tokens, -1), block, q._num_bits,
+                                       q._unsigned, q._narrow_range, sq_err)
+
+
 def _awq_forward(self, input, *args, **kwargs):
     """Replacement ``forward`` of a quantised linear during AWQ-lite (cache pass, then search)."""
     helper = self.awq_lite
@@ -548,6 +570,10 @@ def _awq_forward(self, input, *args, **kwargs):
         x_in = input.contiguous()
         w_in = self.weight.data.contiguous()
         block = _awq_block_size(self.weight, q)
+        if _one_launch_search(self, x_in, w_in, ref, x_scales, w_scales, block, sq_err):
+            helper.sq_err_steps.append((sq_err, ref.numel()))
+            helper.num_search_steps += 1
+            return out_actual
     for i in range(len(helper.alphas)):
         if fused:
             xs = self.input_quantizer(_hip.mul_cols(x_in, x_scales[i]))

@@ -1,0 +1,88 @@
+"""The one-launch AWQ-lite search kernel (matrix-core GEMM with the weight quantised on the fly)
+against (i) the same step done with separate kernels and a library GEMM on the device and (ii)
+the CPU restatement of the reference's search loop.  Losses are sums over a GEMM whose
+accumulation order differs between implementations, so they are compared to 1e-3 relative
+(the figure the selected alpha is required to be stable at); typical agreement is ~1e-5."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from modelopt_amd import _hip
+from oracle import awq as oawq
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _problem(tokens, n, k, n_alpha, seed):
+    g = torch.Generator().manual_seed(seed)
+    w = (0.02 * torch.randn(n, k, generator=g)).to(torch.bfloat16)
+    c = torch.exp(torch.randn(k, generator=g))
+    x = (torch.randn(tokens, k, generator=g) * c).to(torch.bfloat16)
+    s = torch.exp(0.5 * torch.randn(n_alpha, k, generator=g)).to(torch.bfloat16)
+    s[0] = 1.0
+    return x, w, s
+
+
+def _unfused_losses(x, w, s, ref, block, bits, unsigned, narrow):
+    out = torch.zeros(s.shape[0], dtype=torch.float64, device=DEV)
+    for i in range(s.shape[0]):
+        xs = _hip.mul_cols(x, (1 / s[i].float()).to(torch.bfloat16))
+        wq = _hip.scale_block_int_qdq(w, s[i].contiguous(), block, bits, unsigned, narrow)
+        _hip.sq_diff_sum_into(F.linear(xs, wq).contiguous(), ref, out[i:i + 1])
+    return out
+
+
+def _fused_losses(x, w, s, ref, block, bits, unsigned, narrow):
+    xs = _hip.awq_scaled_activations(x, (1 / s.float()).to(torch.bfloat16))
+    out = torch.zeros(s.shape[0], dtype=torch.float64, device=DEV)
+    assert _hip.awq_search_losses_into(xs, w, s.contiguous(), ref, block, bits, unsigned, narrow, out)
+    return out
+
+
+@pytest.mark.parametrize("tokens,n,k", [(512, 256, 512), (128, 64, 128), (100, 128, 256),
+                                        (300, 192, 384), (1, 64, 128), (512, 4096, 4096)])
+@pytest.mark.parametrize("block,bits,unsigned,narrow", [(128, 4, False, False), (64, 4, False, True),
+                                                         (32, 8, False, False)])
+def test_matches_unfused_device_path(tokens, n, k, block, bits, unsigned, narrow):
+    if n * k > 1 << 22 and block != 128:
+        pytest.skip("the large case runs once")
+    x, w, s = (t.to(DEV) for t in _problem(tokens, n, k, 5, tokens + n))
+    ref = F.linear(x, w).contiguous()
+    got = _fused_losses(x, w, s, ref, block, bits, unsigned, narrow)
+    want = _unfused_losses(x, w, s, ref, block, bits, unsigned, narrow)
+    assert torch.allclose(got, want, rtol=1e-3, atol=0), (got, want)
+    assert (got > 0).all()
+
+
+def test_accumulates_and_rejects_uncovered_shapes():
+    x, w, s = (t.to(DEV) for t in _problem(64, 64, 128, 2, 3))
+    ref = F.linear(x, w).contiguous()
+    first = _fused_losses(x, w, s, ref, 128, 4, False, False)
+    xs = _hip.awq_scaled_activations(x, (1 / s.float()).to(torch.bfloat16))
+    acc = first.clone()
+    assert _hip.awq_search_losses_into(xs, w, s, ref, 128, 4, False, False, acc)
+    assert torch.allclose(acc, 2 * first, rtol=1e-12)
+    # block size, feature count, token count outside the kernel's set: nothing is launched
+    assert not _hip.awq_search_losses_into(xs, w, s, ref, 256, 4, False, False, acc)
+    assert not _hip.awq_search_losses_into(xs[:, :8].contiguous(), w[:, :64].contiguous(),
+                                           s[:, :64].contiguous(), ref, 32, 4, False, False, acc)
+    big = torch.zeros(2, 16, 513, 8, dtype=torch.bfloat16, device=DEV)
+    assert not _hip.awq_search_losses_into(big, w, s, torch.zeros(513, 64, dtype=torch.bfloat16, device=DEV),
+                                           128, 4, False, False, acc)
+    assert torch.allclose(acc, 2 * first, rtol=1e-12)
+
+
+def test_matches_cpu_restatement_of_the_search_loop():
+    """losses of the reference's loop body (x * bf16(1/s)) @ QDQ(w * bf16(s))^T on the CPU"""
+    x, w, s = _problem(96, 128, 256, 4, 11)
+    ref = F.linear(x, w)
+    want = []
+    for i in range(s.shape[0]):
+        xs = x * (1 / s[i].float()).to(torch.bfloat16)
+        out = F.linear(xs, oawq.int4_block_qdq(w * s[i], 128))
+        want.append((out - ref).float().pow(2).sum().double())
+    want = torch.stack(want)
+    got = _fused_losses(x.to(DEV), w.to(DEV), s.to(DEV), ref.to(DEV).contiguous(), 128, 4, False, False)
+    assert torch.allclose(got.cpu(), want, rtol=1e-3), (got, want)

@@ -332,21 +332,33 @@ def test_awq_lite_matches_oracle(alpha_step):
     assert "forward" not in model.proj.__dict__  # patch removed
 
 
-def test_awq_generic_path_equals_fused_path(monkeypatch):
+def test_awq_search_paths_agree(monkeypatch):
+    """Three routes through a search step: (a) one launch for all alphas (weights quantised in
+    front of the matrix cores), (b) per alpha a fused weight kernel + library GEMM + loss kernel,
+    (c) per alpha through the quantizer modules.  (b) and (c) run the same GEMM on the same
+    operands and agree exactly; (a) accumulates in a different order, so its losses agree to
+    1e-4 relative -- with the same selected alpha, hence the same folded weight."""
     from modelopt_amd.torch.quantization import model_calib
 
     batches = _awq_batches()
-    results = []
-    for fused in (True, False):
+    results = {}
+    for route in "abc":
         model = _OneLinear().to(DEV)
-        if not fused:
+        if route != "a":
+            monkeypatch.setattr(model_calib, "_one_launch_search", lambda *a, **k: False)
+        if route == "c":
             monkeypatch.setattr(model_calib, "_fused_weight_path", lambda m: False)
         cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
         cfg["algorithm"] = {"method": "awq_lite", "alpha_step": 0.1, "debug": True}
         mtq.quantize(model, cfg, lambda m: [m(b.to(DEV)) for b in batches])
-        results.append((model.proj.awq_lite.loss, model.proj.weight.data.clone()))
-    assert results[0][0] == results[1][0]
-    assert torch.equal(results[0][1], results[1][1])
+        h = model.proj.awq_lite
+        results[route] = (h.loss, h.best_alpha, model.proj.weight.data.clone())
+    assert results["b"][0] == results["c"][0]
+    assert torch.equal(results["b"][2], results["c"][2])
+    for alpha, want in results["b"][0].items():
+        assert results["a"][0][alpha] == pytest.approx(want, rel=1e-4)
+    assert results["a"][1] == results["b"][1]
+    assert torch.equal(results["a"][2], results["b"][2])
 
 
 def test_true_divide_is_one_rounding_on_the_gpu():
