@@ -13,7 +13,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmodelopt_hip.so")
-HEADERS = [os.path.join(CSRC, "common.h"), os.path.join(HERE, "..", "include", "modelopt_hip.h")]
+HEADERS = [os.path.join(CSRC, h) for h in ("common.h", "qdq_ops.h", "awq_ops.h")] + [
+    os.path.join(HERE, "..", "include", "modelopt_hip.h")]
 
 # -ffp-contract=off: the rounding tricks rely on separately rounded fp32 multiplies and adds.
 # packed-fp32-ops is switched off on purpose (v_pk_*_f32 forms are not trusted on this target).

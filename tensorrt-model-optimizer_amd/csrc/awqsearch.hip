@@ -14,36 +14,13 @@
 // 70 % of this form's rate here), the activations are loaded straight into the A operand
 // registers from a chunk-major copy, in which the lanes of an operand read adjacent memory.  The output tile never leaves the registers: it is rounded
 // to bf16, compared with the reference output and reduced to one double per workgroup.
+#include "awq_ops.h"
 #include "common.h"
 
 namespace mo {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
-
-// defined in awq.hip's translation unit as well; kept identical (same arithmetic, same order)
-__device__ __forceinline__ void search_qdq_chunk(float (&v)[8], int lg_g, float bound, float lo) {
-    uint32_t m = 0;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const uint32_t a = f2u(v[j]) & 0x7FFFFFFFu;
-        m = a > m ? a : m;
-    }
-    m = group_max_u32(m, lg_g);
-    const float amax = u2f(m);
-    const bool dead = amax <= 5.9604644775390625e-8f;
-    const float sc = bound / amax;
-    const float mul = dead ? 0.0f : sc, div = dead ? 1.0f : sc;
-    const float rdiv = 1.0f / div;
-    const bool fast = mid_range(div);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        float q = __builtin_rintf(v[j] * mul);
-        q = q < lo ? lo : q;
-        q = q > bound ? bound : q;
-        v[j] = fast ? __builtin_copysignf(exact_quotient(q, div, rdiv), q) : q / div;
-    }
-}
 
 constexpr int kSearchTileN = 64;    // output features per workgroup
 constexpr int kSearchBlockK = 128;  // k elements per step: 16 chunks of 8
@@ -73,14 +50,11 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
     const int n0 = blockIdx.x * kSearchTileN;
     const int nkb = K / kSearchBlockK;
 
-    // roles alternate between neighbouring wavefronts (MO_SEARCH_ROLE_SHIFT picks the bit)
-#ifndef MO_SEARCH_ROLE_SHIFT
-#define MO_SEARCH_ROLE_SHIFT 0
-#endif
-    const bool producer = ((wave >> MO_SEARCH_ROLE_SHIFT) & 1) == 0;
-    // index of this wavefront within its role, 0..3
-    const int rw = MO_SEARCH_ROLE_SHIFT == 0 ? wave >> 1
-                 : MO_SEARCH_ROLE_SHIFT == 1 ? ((wave >> 2) << 1) | (wave & 1) : wave & 3;
+    // Wavefront w of a workgroup runs on SIMD w % 4: wavefronts 0-3 produce and 4-7 consume, so
+    // that every SIMD hosts one of each (with alternating roles two SIMDs would get both
+    // consumers and the matrix work would run at half rate).
+    const bool producer = wave < 4;
+    const int rw = wave & 3;  // index within the role
     if (producer) {
         // ------------------------------------------------------------------ producer
         const uint16_t* sa = s + (int64_t)a * K;
@@ -128,9 +102,7 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
             sb = *(const u32x4*)(sp + k2);
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-#ifndef MO_SEARCH_DBG_NO_QDQ
-                search_qdq_chunk(v[u], lg_g, bound, lo);
-#endif
+                block_int_qdq_chunk(v[u], lg_g, bound, lo);
                 u32x4 o;
                 o.x = f32x2_to_bf16x2(v[u][0], v[u][1]);
                 o.y = f32x2_to_bf16x2(v[u][2], v[u][3]);
@@ -209,23 +181,16 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
                     bf16x8_t afrag;
                     __builtin_memcpy(&afrag, &af[mb][j], 16);
 #pragma unroll
-                    for (int nb = 0; nb < 2; ++nb) {
-#ifndef MO_SEARCH_DBG_NO_MFMA
+                    for (int nb = 0; nb < 2; ++nb)
                         acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[nb],
                                                                               acc[mb][nb], 0, 0, 0);
-#else
-                        acc[mb][nb][0] += (float)afrag[0] + (float)bfrag[nb][0];
-#endif
-                    }
                 }
                 // keep the reloads behind the MFMAs that read the old fragments: hoisted above
                 // them they would need a second set of registers
                 __builtin_amdgcn_sched_barrier(0);
-#ifndef MO_SEARCH_DBG_NO_ALOAD
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
                     af[mb][j] = *(const u32x4*)(xa + aoff[mb] + (uint32_t)(nh * 4 + j) * step_stride);
-#endif
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
