@@ -12,3 +12,4 @@ from .conversion import (register, replace_quant_module, set_quantizer_attribute
 from .model_quant import (calibrate, disable_quantizer, enable_quantizer, fold_weight,
                           postprocess_amax, print_quant_summary, quantize)
 from .plugins import attention as _attention_plugin  # noqa: F401  (registers KV quantizers)
+from .tensor_quant import get_fp8_overflow_behavior, set_fp8_overflow_behavior

@@ -22,6 +22,10 @@ __all__ = ["replace_quant_module", "set_quantizer_by_cfg", "set_quantizer_attrib
 def replace_quant_module(model: nn.Module):
     """Recursively convert every registered module type found in ``model`` (in place)."""
     assert not is_converted(model), "Model must not be quantized!"
+    from .plugins import CUSTOM_MODEL_PLUGINS  # late: the plugins import the module registry
+
+    for plugin in CUSTOM_MODEL_PLUGINS:
+        plugin(model)
     for name, child in list(model.named_modules()):
         if type(child) in QuantModuleRegistry:
             QuantModuleRegistry.convert(child)

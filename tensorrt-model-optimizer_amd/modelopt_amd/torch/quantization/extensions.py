@@ -53,14 +53,15 @@ class _Fp8Ext:
 
     @staticmethod
     def fake_e4m3fy(inputs, amax):
-        return kernels.fake_quant_fp8(inputs, amax.reshape(()))
+        # the CUDA kernel this stands in for clamps to +-448 before the cast
+        return kernels.fake_quant_fp8(inputs, amax.reshape(()), saturate=True)
 
     @staticmethod
     def fake_e4m3fy_with_axis(inputs, amax, axis):
         x = inputs if inputs.is_contiguous() else inputs.contiguous()
         axis = axis % x.dim()
         outer, n, inner = kernels.amax_layout(tuple(x.shape), [axis])
-        return _hip.fp8_qdq(x, amax.reshape(-1).contiguous(), outer, x.shape[axis], inner)
+        return _hip.fp8_qdq(x, amax.reshape(-1).contiguous(), outer, x.shape[axis], inner, True)
 
 
 class _MxTypes:

@@ -27,9 +27,34 @@ mx_format_map = {(4, 3): "E4M3", (5, 2): "E5M2", (3, 2): "E3M2", (2, 3): "E2M3",
 NVFP4_FAKE_QUANT_MODE = 0
 
 
+# What FP8 fake quantisation does with a scaled value beyond the E4M3 range (|x| * 448 / amax
+# > 464, i.e. data above the calibrated amax).  The reference has both behaviours: its eager
+# torch path -- the only one that runs on a CPU -- casts with ``Tensor.to(float8_e4m3fn)``, which
+# gives NaN (tensor_quant.py:45-59), its CUDA kernel clamps to +-448 first
+# (src/tensor_quant_gpu_fp8.cu:43).  "nan" is the default here because results are held to the
+# CPU path bit for bit; "saturate" is what a deployment wants (a KV-cache value a hair above the
+# calibration maximum becomes the maximum instead of poisoning the attention output).
+_FP8_OVERFLOW = "nan"
+
+
+def set_fp8_overflow_behavior(mode: str) -> str:
+    """``"nan"`` (eager / CPU semantics, default) or ``"saturate"`` (the CUDA kernel's).  Returns
+    the previous mode."""
+    global _FP8_OVERFLOW
+    if mode not in ("nan", "saturate"):
+        raise ValueError(f"mode must be 'nan' or 'saturate', got {mode!r}")
+    previous, _FP8_OVERFLOW = _FP8_OVERFLOW, mode
+    return previous
+
+
+def get_fp8_overflow_behavior() -> str:
+    return _FP8_OVERFLOW
+
+
 def scaled_e4m3_impl(inputs: torch.Tensor, amax: torch.Tensor | None = None) -> torch.Tensor:
-    """FP8 E4M3 fake quantisation with the numerics of the reference's eager path."""
-    return kernels.fake_quant_fp8(inputs, amax)
+    """FP8 E4M3 fake quantisation with the numerics of the reference's eager path (or, after
+    ``set_fp8_overflow_behavior("saturate")``, of its CUDA kernel for out-of-range values)."""
+    return kernels.fake_quant_fp8(inputs, amax, saturate=_FP8_OVERFLOW == "saturate")
 
 
 fp8_eager = scaled_e4m3_impl
