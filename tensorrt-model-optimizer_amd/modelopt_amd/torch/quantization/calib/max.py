@@ -72,8 +72,8 @@ class MaxCalibrator(_Calibrator):
             return
         keep = [] if reduce_axis is None else [d for d in range(x.dim()) if d not in reduce_axis]
         layout = kernels.amax_layout(tuple(x.shape), keep)
-        if layout is None:
-            raise NotImplementedError("max calibration over non-adjacent kept dims is not covered")
+        if layout is None:  # kept dims apart (2-D blocks): reduce a copy with them in front
+            x, _, layout = kernels.kept_dims_first(x, keep)
         if self._acc is None:
             self._acc = torch.zeros(layout[1], dtype=torch.float32, device=x.device)
             self._shape, self._dtype = shape, x.dtype

@@ -15,7 +15,10 @@ __all__ = [
     "AWQLiteCalibConfig", "INT8_DEFAULT_CFG", "INT8_SMOOTHQUANT_CFG", "INT8_WEIGHT_ONLY_CFG",
     "FP8_DEFAULT_CFG", "INT4_BLOCKWISE_WEIGHT_ONLY_CFG", "INT4_AWQ_CFG", "W4A8_AWQ_BETA_CFG",
     "FP8_KV_CFG", "NVFP4_DEFAULT_CFG", "NVFP4_AWQ_LITE_CFG", "NVFP4_KV_CFG", "MXFP8_DEFAULT_CFG",
-    "MXFP6_DEFAULT_CFG", "MXFP4_DEFAULT_CFG", "MXINT8_DEFAULT_CFG", "W4A8_MXFP4_FP8_CFG", "choices",
+    "MXFP6_DEFAULT_CFG", "MXFP4_DEFAULT_CFG", "MXINT8_DEFAULT_CFG", "W4A8_MXFP4_FP8_CFG",
+    "NVFP4_AWQ_CLIP_CFG", "NVFP4_AWQ_FULL_CFG", "FP8_PER_CHANNEL_PER_TOKEN_CFG",
+    "FP8_2D_BLOCKWISE_WEIGHT_ONLY_CFG", "W4A8_NVFP4_FP8_CFG", "MXFP4_MLP_WEIGHT_ONLY_CFG",
+    "NVFP4_MLP_WEIGHT_ONLY_CFG", "NVFP4_MLP_ONLY_CFG", "choices",
 ]
 
 _SPECIAL_BLOCK_KEYS = ("type", "scale_bits", "scale_block_sizes")
@@ -340,6 +343,66 @@ NVFP4_AWQ_LITE_CFG = {
                   **_default_disabled_quantizer_cfg},
     "algorithm": "awq_lite",
 }
+# reference: config.py:410-447
+NVFP4_AWQ_CLIP_CFG = {
+    "quant_cfg": {"*weight_quantizer": dict(_NVFP4), "*input_quantizer": dict(_NVFP4),
+                  **_default_disabled_quantizer_cfg},
+    "algorithm": {"method": "awq_clip"},
+}
+NVFP4_AWQ_FULL_CFG = {
+    "quant_cfg": {"*weight_quantizer": dict(_NVFP4), "*input_quantizer": dict(_NVFP4),
+                  **_default_disabled_quantizer_cfg},
+    "algorithm": {"method": "awq_full", "alpha_step": 0.1},
+}
+# reference: config.py:201-212 -- per-channel weights, per-token dynamic activations
+FP8_PER_CHANNEL_PER_TOKEN_CFG = {
+    "quant_cfg": {"*weight_quantizer": {"num_bits": (4, 3), "axis": 0},
+                  "*input_quantizer": {"num_bits": (4, 3), "type": "dynamic",
+                                       "block_sizes": {-1: None}},
+                  **_default_disabled_quantizer_cfg},
+    "algorithm": "max",
+}
+# reference: config.py:215-226 -- 128 x 128 weight tiles (DeepSeek style)
+FP8_2D_BLOCKWISE_WEIGHT_ONLY_CFG = {
+    "quant_cfg": {"*weight_quantizer": {"num_bits": (4, 3), "block_sizes": {-1: 128, -2: 128},
+                                        "enable": True},
+                  "*input_quantizer": {"enable": False},
+                  **_default_disabled_quantizer_cfg},
+    "algorithm": "max",
+}
+# reference: config.py:559-575 -- NVFP4 weights in 32-element blocks, FP8 per-tensor activations
+W4A8_NVFP4_FP8_CFG = {
+    "quant_cfg": {"*weight_quantizer": {"num_bits": (2, 1),
+                                        "block_sizes": {-1: 32, "type": "dynamic",
+                                                        "scale_bits": (4, 3)},
+                                        "axis": None, "enable": True},
+                  "*input_quantizer": {"num_bits": (4, 3), "axis": None, "enable": True},
+                  **_default_disabled_quantizer_cfg},
+    "algorithm": "max",
+}
+# reference: config.py:577-620 -- MLP layers only
+MXFP4_MLP_WEIGHT_ONLY_CFG = {
+    "quant_cfg": {"*mlp*weight_quantizer": {"num_bits": (2, 1),
+                                            "block_sizes": {-1: 32, "type": "dynamic",
+                                                            "scale_bits": (8, 0)},
+                                            "enable": True, "pass_through_bwd": True},
+                  **_default_disabled_quantizer_cfg},
+    "algorithm": None,
+}
+NVFP4_MLP_WEIGHT_ONLY_CFG = {
+    "quant_cfg": {"*mlp*weight_quantizer": {"num_bits": (2, 1),
+                                            "block_sizes": {-1: 32, "type": "dynamic",
+                                                            "scale_bits": (4, 3)},
+                                            "enable": True, "pass_through_bwd": True},
+                  **_default_disabled_quantizer_cfg},
+    "algorithm": "max",
+}
+NVFP4_MLP_ONLY_CFG = {
+    "quant_cfg": {"*mlp*weight_quantizer": {**_NVFP4, "pass_through_bwd": True},
+                  "*mlp*input_quantizer": {**_NVFP4, "pass_through_bwd": True},
+                  **_default_disabled_quantizer_cfg},
+    "algorithm": "max",
+}
 
 
 
@@ -368,5 +431,7 @@ choices = {
     "W4A8_MXFP4_FP8_CFG",
     "INT8_DEFAULT_CFG", "INT8_SMOOTHQUANT_CFG", "INT8_WEIGHT_ONLY_CFG", "FP8_DEFAULT_CFG",
     "INT4_BLOCKWISE_WEIGHT_ONLY_CFG", "INT4_AWQ_CFG", "W4A8_AWQ_BETA_CFG", "NVFP4_DEFAULT_CFG",
-    "NVFP4_AWQ_LITE_CFG",
+    "NVFP4_AWQ_LITE_CFG", "NVFP4_AWQ_CLIP_CFG", "NVFP4_AWQ_FULL_CFG", "FP8_PER_CHANNEL_PER_TOKEN_CFG",
+    "FP8_2D_BLOCKWISE_WEIGHT_ONLY_CFG", "W4A8_NVFP4_FP8_CFG", "MXFP4_MLP_WEIGHT_ONLY_CFG",
+    "NVFP4_MLP_WEIGHT_ONLY_CFG", "NVFP4_MLP_ONLY_CFG", "FP8_KV_CFG", "NVFP4_KV_CFG",
 }

@@ -121,6 +121,10 @@ def _as_cfg(attribute):
     so a partial dict (``{"enable": False}``) leaves the other attributes alone."""
     if isinstance(attribute, QuantizerAttributeConfig):
         return attribute
+    if set(attribute) == {"enable"}:
+        # the "enable alone is not a config" rule is for user configs (checked when
+        # ``mtq.quantize`` parses them); internally this is how a quantizer is switched on
+        return {"enable": bool(attribute["enable"])}
     full = QuantizerAttributeConfig(**attribute)
     return {k: full[k] for k in attribute}
 

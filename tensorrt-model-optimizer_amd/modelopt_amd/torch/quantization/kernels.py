@@ -11,7 +11,7 @@ import torch
 from ... import _hip
 
 __all__ = [
-    "amax_layout", "absmax_accumulate", "reduce_amax_gpu", "fake_quant_int", "fake_quant_fp8",
+    "amax_layout", "kept_dims_first", "absmax_accumulate", "reduce_amax_gpu", "fake_quant_int", "fake_quant_fp8",
     "fake_quant_nvfp4", "fake_quant_block_fp", "mul_last_dim",
 ]
 
@@ -35,6 +35,25 @@ def amax_layout(shape, keep_dims):
                 return None
     lo, hi = keep[0], keep[-1]
     return _prod(shape[:lo]), _prod(shape[lo:hi + 1]), _prod(shape[hi + 1:])
+
+
+def kept_dims_first(x, keep_dims):
+    """For kept dims that are not one contiguous run (2-D blocks: dims 0 and 2 of
+    ``[N/b0, b0, K/b1, b1]``): a contiguous copy with the kept dims moved to the front, viewed by
+    the kernels as [1, prod(kept), prod(rest)], and the permutation that was applied.  Costs one
+    transposing copy each way; the common layouts never take this route."""
+    nd = x.dim()
+    keep = sorted({d % nd for d in keep_dims})
+    perm = keep + [d for d in range(nd) if d not in keep]
+    xp = x.permute(perm).contiguous()
+    return xp, perm, (1, _prod(x.shape[d] for d in keep), _prod(xp.shape[len(keep):]))
+
+
+def _undo_permutation(y, perm):
+    inverse = [0] * len(perm)
+    for i, d in enumerate(perm):
+        inverse[d] = i
+    return y.permute(inverse).contiguous()
 
 
 def layout_from_amax_shape(x_shape, amax_shape):
@@ -75,37 +94,45 @@ def reduce_amax_gpu(x: torch.Tensor, reduce_dims, keepdims=True):
         out_shape = tuple(1 if d in red else x.shape[d] for d in range(nd)) if keepdims else tuple(
             x.shape[d] for d in keep)
     layout = amax_layout(tuple(x.shape), keep)
+    src = x
     if layout is None:
-        raise NotImplementedError(
-            "abs-max that keeps non-adjacent dims is not covered by the kernels (amax with more "
-            "than one non-unit run of dims)")
+        src, _, layout = kept_dims_first(x, keep)
     acc = torch.zeros(layout[1], dtype=torch.float32, device=x.device)
-    absmax_accumulate(x, acc, layout)
+    absmax_accumulate(src, acc, layout)
     return acc.to(x.dtype).reshape(out_shape)
 
 
 def _qdq_layout(x, amax):
-    layout = layout_from_amax_shape(tuple(x.shape), tuple(amax.shape))
-    if layout is None:
+    return layout_from_amax_shape(tuple(x.shape), tuple(amax.shape))
+
+
+def _qdq(x, amax, run):
+    """``run(x2, amax_flat, outer, axis, inner)`` on ``x`` as it is when the amax spans one run
+    of dims, else on a copy with the amax dims moved to the front (and moved back afterwards)."""
+    x = x if x.is_contiguous() else x.contiguous()
+    layout = _qdq_layout(x, amax)
+    if layout is not None:
+        return run(x, amax.reshape(-1).contiguous(), *layout)
+    if amax.dim() != x.dim() or any(a not in (1, s) for a, s in zip(amax.shape, x.shape)):
         raise NotImplementedError(
-            f"amax of shape {tuple(amax.shape)} against input {tuple(x.shape)}: scales on more than "
-            "one non-adjacent dim are not covered by the kernels")
-    return layout
+            f"amax of shape {tuple(amax.shape)} does not broadcast against input {tuple(x.shape)}")
+    keep = [d for d in range(x.dim()) if amax.shape[d] != 1]
+    xp, perm, layout = kept_dims_first(x, keep)
+    y = run(xp, amax.reshape(-1).contiguous(), *layout)
+    return _undo_permutation(y.view(xp.shape), perm)
 
 
 def fake_quant_int(x, amax, num_bits=8, unsigned=False, narrow_range=True):
-    x = x if x.is_contiguous() else x.contiguous()
-    outer, axis, inner = _qdq_layout(x, amax)
-    return _hip.int_qdq(x, amax.reshape(-1).contiguous(), outer, axis, inner, num_bits, unsigned,
-                        narrow_range)
+    return _qdq(x, amax, lambda x2, a, outer, axis, inner: _hip.int_qdq(
+        x2, a, outer, axis, inner, num_bits, unsigned, narrow_range))
 
 
 def fake_quant_fp8(x, amax=None, saturate=False):
-    x = x if x.is_contiguous() else x.contiguous()
     if amax is None:
+        x = x if x.is_contiguous() else x.contiguous()
         return _hip.fp8_qdq(x, None, 1, 1, x.numel(), saturate)
-    outer, axis, inner = _qdq_layout(x, amax)
-    return _hip.fp8_qdq(x, amax.reshape(-1).contiguous(), outer, axis, inner, saturate)
+    return _qdq(x, amax, lambda x2, a, outer, axis, inner: _hip.fp8_qdq(
+        x2, a, outer, axis, inner, saturate))
 
 
 def fake_quant_nvfp4(x, global_amax, block_size=16, mode=0):

@@ -449,7 +449,7 @@ class TensorQuantizer(nn.Module):
     def _reset_to_original_shape(self, outputs: torch.Tensor):
         outputs = outputs.reshape(self._original_shape)
         if hasattr(self, "_slices"):
-            outputs = outputs[self._slices]
+            outputs = outputs[tuple(self._slices)]
         return outputs
 
     def _block_sizes_to_axis(self, x: torch.Tensor):

@@ -4,22 +4,38 @@ import torch
 
 from .... import _hip
 from .. import kernels
-from ..utils import (convert_quantization_axis_to_reduce_axis, reduce_amax, reduce_block_amax,
-                     true_divide)
+from ..utils import convert_quantization_axis_to_reduce_axis, reduce_amax, true_divide
+from ._blocks import BlockRows
 from .base_qtensor import BaseQuantizedTensor
 
 __all__ = ["FP8QTensor"]
 
 
-def _block_layout(x, scales, block_sizes):
-    """[outer, axis, inner] of a 1-D block layout along the last dim, or raise."""
-    dims = {d % x.dim() for d in block_sizes}
-    if dims != {x.dim() - 1}:
-        raise NotImplementedError("only block scales along the last dim are covered by the kernels")
-    blk = block_sizes[-1] if -1 in block_sizes else block_sizes[x.dim() - 1]
-    if x.shape[-1] % blk:
-        raise NotImplementedError("block scales with padding are not covered by the kernels")
-    return 1, x.numel() // blk, blk
+def _block_quantize(cls, input, scales, block_sizes, bound, fmt, crop=True):
+    """Shared by the FP8 and INT8 containers: block scales on any dims, zero padding.  The FP8
+    container stores the codes cropped to the input shape, the INT8 container stores them
+    padded (reference: fp8_tensor.py:108-112 against int8_tensor.py:86-88)."""
+    br = BlockRows(input.shape, block_sizes)
+    rows = br.to_rows(input)
+    if scales is None:
+        amax = reduce_amax(rows, axis=1, keepdims=False, squeeze_scalar=False)
+        scales = true_divide(amax, bound).reshape(br.scale_shape)
+    elif tuple(scales.shape) != br.scale_shape:
+        assert scales.numel() == br.rows, (
+            f"Mismatch in expected scale shape: {tuple(scales.shape)} vs {br.scale_shape}")
+        scales = scales.reshape(br.scale_shape)
+    via = torch.result_type(input, scales)
+    q = _hip.real_quantize(rows, scales.reshape(-1).contiguous(), 1, br.rows, br.block, via, fmt)
+    return cls(input.shape, input.dtype, br.from_rows(q, crop)), scales
+
+
+def _block_dequantize(q, shape, scales, block_sizes, fmt, dtype):
+    br = BlockRows(shape, block_sizes)
+    assert tuple(scales.shape) == br.scale_shape, (
+        f"Scales shape {tuple(scales.shape)} must match expected {br.scale_shape}.")
+    rows = br.to_rows(q.view(torch.uint8))
+    y = _hip.real_dequantize(rows, scales.reshape(-1).contiguous(), 1, br.rows, br.block, fmt, dtype)
+    return br.from_rows(y)
 
 
 class FP8QTensor(BaseQuantizedTensor):
@@ -27,19 +43,15 @@ class FP8QTensor(BaseQuantizedTensor):
 
     @classmethod
     def quantize(cls, input, scales=None, axis=None, block_sizes=None) -> tuple:
+        if block_sizes:
+            return _block_quantize(cls, input, scales, block_sizes, 448.0, _hip.MO_FMT_E4M3)
         x = input.contiguous()
         if scales is None:
-            if block_sizes:
-                amax = reduce_block_amax(x, block_sizes)
-            else:
-                amax = reduce_amax(x, axis=convert_quantization_axis_to_reduce_axis(x, axis))
+            amax = reduce_amax(x, axis=convert_quantization_axis_to_reduce_axis(x, axis))
             scales = true_divide(amax, 448.0)
-        if block_sizes:
-            layout = _block_layout(x, scales, block_sizes)
-        else:
-            layout = kernels.layout_from_amax_shape(tuple(x.shape), tuple(scales.shape))
-            if layout is None:
-                raise NotImplementedError("scale shape not covered by the kernels")
+        layout = kernels.layout_from_amax_shape(tuple(x.shape), tuple(scales.shape))
+        if layout is None:
+            raise NotImplementedError("scale shape not covered by the kernels")
         via = torch.result_type(x, scales)
         q = _hip.real_quantize(x, scales.reshape(-1).contiguous(), *layout, via, _hip.MO_FMT_E4M3)
         return cls(input.shape, input.dtype, q), scales
@@ -52,7 +64,7 @@ class FP8QTensor(BaseQuantizedTensor):
         q = self._quantized_data.contiguous()
         scales = scales.to(q.device)
         if block_sizes:
-            layout = _block_layout(q, scales, block_sizes)
-        else:
-            layout = kernels.layout_from_amax_shape(tuple(q.shape), tuple(scales.shape))
+            return _block_dequantize(q, self.metadata["shape"], scales, block_sizes,
+                                     _hip.MO_FMT_E4M3, dtype)
+        layout = kernels.layout_from_amax_shape(tuple(q.shape), tuple(scales.shape))
         return _hip.real_dequantize(q, scales.reshape(-1).contiguous(), *layout, _hip.MO_FMT_E4M3, dtype)

@@ -118,6 +118,26 @@ def test_set_quantizer_by_cfg_context_restores():
     assert q.is_enabled and q.num_bits == 8
 
 
+def test_enable_alone_is_internal_only():
+    """``{"enable": True}`` on its own switches a configured quantizer back on (enable_quantizer,
+    the AWQ cache pass: reference model_quant.py:enable_quantizer, model_calib.py:667), while a
+    user config that says nothing else is rejected when ``mtq.quantize`` parses it
+    (reference config.py:683-707)."""
+    m = _converted(mtq.INT8_DEFAULT_CFG)
+    q = m.body[0].input_quantizer
+    mtq.disable_quantizer(m, "*input_quantizer")
+    assert not q.is_enabled
+    mtq.enable_quantizer(m, "*input_quantizer")
+    assert q.is_enabled and q.num_bits == 8
+    q.disable()
+    with mtq.set_quantizer_by_cfg_context(q, {"*": {"enable": True}}):
+        assert q.is_enabled
+    assert not q.is_enabled
+    with pytest.raises(Exception, match="Cannot specify only"):
+        mtq.model_quant._validated({"quant_cfg": {"*weight_quantizer": {"enable": True}},
+                                    "algorithm": "max"})
+
+
 # ----------------------------------------------------------------------------- TensorQuantizer
 def test_quantizer_properties_and_state():
     q = TensorQuantizer(QuantizerAttributeConfig(num_bits=(4, 3)))
@@ -211,14 +231,21 @@ def test_static_block_reshape_and_amax_shapes(oracle_backend, shape, block_sizes
         q(torch.randn(shape[0] + 1, *shape[1:]))
 
 
-def test_two_axis_blocks_reshape_then_refuse(oracle_backend):
-    """2-D blocks take the general reshape ([2, 4, 2, 32], amax on dims 0 and 2); scales on two
-    non-adjacent dims are not covered by the kernels and must raise, not fall back."""
+def test_two_axis_blocks(oracle_backend):
+    """2-D blocks take the general reshape ([2, 4, 2, 32], amax on dims 0 and 2): calibration and
+    fake quantisation follow the reference's reshape -> quantise -> reshape back
+    (nn/modules/tensor_quantizer.py:755-800)."""
     q = TensorQuantizer(QuantizerAttributeConfig(num_bits=8, block_sizes={-1: 32, -2: 4}))
+    x = torch.randn(8, 64)
     q.enable_calib(); q.disable_quant()
-    with pytest.raises(NotImplementedError):
-        q(torch.randn(8, 64))
+    q(x)
     assert tuple(q._block_reshape_size) == (2, 4, 2, 32) and q.axis == (0, 2)
+    q.load_calib_amax()
+    blocks = x.reshape(2, 4, 2, 32)
+    assert torch.equal(q.amax, blocks.abs().amax(dim=(1, 3), keepdim=True))
+    q.enable_quant(); q.disable_calib()
+    want = fake_quant.tensor_quant(blocks, q.amax, 8, False, False).reshape(8, 64)
+    assert torch.equal(q(x), want)
 
 
 def test_block_sizes_none_means_per_channel(oracle_backend):

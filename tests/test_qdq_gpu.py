@@ -148,3 +148,37 @@ def test_inplace_alias():
     xd = x.to(DEV)
     _hip.int_qdq(xd, amax.to(DEV), 1, 1, xd.numel(), 8, False, True, out=xd)
     assert_bits_equal(xd.cpu(), fake_quant.tensor_quant(x, amax, 8, False, True), "in place")
+
+
+@pytest.mark.parametrize("num_bits", [(4, 3), 8])
+@pytest.mark.parametrize("shape,blocks", [((256, 384), {-1: 128, -2: 128}), ((8, 64), {-1: 32, -2: 4}),
+                                           ((100, 72), {-1: 16, -2: 8})])
+def test_two_axis_block_fake_quant_through_the_quantizer(num_bits, shape, blocks):
+    """2-D tiles (the FP8 128 x 128 weight-only config and smaller ones, with padding): the
+    quantizer reshapes to [N/b0, b0, K/b1, b1] and its amax keeps dims 0 and 2 -- two runs of
+    dims, which the kernels see through a transposing copy.  Against the same reshape on the CPU
+    (reference nn/modules/tensor_quantizer.py:755-800)."""
+    import torch.nn.functional as F
+
+    from modelopt_amd.torch.quantization.config import QuantizerAttributeConfig
+    from modelopt_amd.torch.quantization.nn import TensorQuantizer
+
+    x = _rand(shape, torch.bfloat16, 31)
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=num_bits, block_sizes=blocks)).to(DEV)
+    q.enable_calib(); q.disable_quant()
+    q(x.to(DEV))
+    q.load_calib_amax()
+    q.enable_quant(); q.disable_calib()
+    got = q(x.to(DEV)).cpu()
+
+    b0, b1 = blocks[-2], blocks[-1]
+    pad = F.pad(x, (0, -shape[1] % b1, 0, -shape[0] % b0))
+    tiles = pad.reshape(pad.shape[0] // b0, b0, pad.shape[1] // b1, b1)
+    amax = reduce.reduce_amax(tiles, axis=[1, 3], keepdims=True, squeeze_scalar=False)
+    assert_bits_equal(q.amax.cpu(), amax, "tile amax")
+    if num_bits == 8:
+        want = fake_quant.tensor_quant(tiles, amax, 8, False, False)
+    else:
+        want = fake_quant.fp8_eager(tiles, amax)
+    want = want.reshape(pad.shape)[: shape[0], : shape[1]]
+    assert_bits_equal(got, want, "2-D block fake quant")

@@ -90,6 +90,48 @@ def test_qtensor_golden_vectors_through_kernels(case):
     assert torch.allclose(y.cpu(), want), (y.cpu(), want)
 
 
+@pytest.mark.parametrize("case", VEC["qtensor_roundtrip"], ids=lambda c: c["name"])
+def test_qtensor_golden_vectors_through_the_quantizer(case):
+    """The same golden round trips the way the reference's test drives them: a real-quantising
+    ``TensorQuantizer`` (quantize on the first call, dequantize on the second), including the
+    2-D block and padded cases (tests/gpu/torch/quantization/test_qtensor_cuda.py:243-268)."""
+    from modelopt_amd.torch.quantization.config import QuantizerAttributeConfig
+    from modelopt_amd.torch.quantization.nn import TensorQuantizer
+
+    bits = tuple(case["num_bits"]) if isinstance(case["num_bits"], list) else case["num_bits"]
+    bs = None if case["block_sizes"] is None else {int(k): v for k, v in case["block_sizes"].items()}
+    q = TensorQuantizer(QuantizerAttributeConfig(num_bits=bits, block_sizes=bs, fake_quant=False,
+                                                 axis=case["axis"])).to(DEV)
+    x = torch.tensor(case["input"], dtype=torch.bfloat16, device=DEV)
+    packed = q(x)
+    out = q(packed)
+    want = torch.tensor(case["output"], dtype=torch.bfloat16)
+    assert out.shape == x.shape and torch.allclose(out.cpu(), want), (out.cpu(), want)
+
+
+@pytest.mark.parametrize("fmt", ["fp8", "int8"])
+@pytest.mark.parametrize("shape,blocks", [((256, 384), {-1: 128, -2: 128}), ((100, 200), {-1: 64, -2: 32}),
+                                           ((3, 40, 96), {-1: 32}), ((130, 70), {-1: 16})])
+def test_block_scales_on_any_dims_match_restatement(fmt, shape, blocks):
+    """2-D tiles, padding on either dim, 3-D inputs: codes, scales and dequantised values equal
+    the CPU restatement of the reference's pad / repeat_interleave formulation bit for bit."""
+    from modelopt_amd.torch.quantization.qtensor import FP8QTensor, INT8QTensor
+
+    x = _rand(shape, torch.bfloat16, 21, scale=1.0)
+    if fmt == "fp8":
+        q_o, s_o = qtensor.fp8_quantize(x, block_sizes=blocks)
+        want = qtensor.fp8_dequantize(q_o, s_o, x.shape, torch.bfloat16, blocks)
+        qt, s = FP8QTensor.quantize(x.to(DEV), block_sizes=blocks)
+    else:
+        q_o, s_o = qtensor.int8_quantize(x, block_sizes=blocks)
+        want = qtensor.int8_dequantize(q_o, s_o, x.shape, torch.bfloat16, blocks)
+        qt, s = INT8QTensor.quantize(x.to(DEV), block_sizes=blocks)
+    assert_bits_equal(s.cpu(), s_o, "scales")
+    assert_bits_equal(qt._quantized_data.cpu(), q_o, "codes")
+    got = qt.dequantize(scale=s, block_sizes=blocks)
+    assert_bits_equal(got.cpu(), want, "dequantised")
+
+
 # ----------------------------------------------------------------------------- INT8 / INT4
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_int8_quantize_dequantize(dtype):
