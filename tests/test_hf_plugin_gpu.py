@@ -134,3 +134,23 @@ def test_fp8_overflow_switch():
     assert torch.equal(sat, torch.tensor([0.5, 1.0, 1.0, 1.0, 1.0, -1.0], dtype=torch.bfloat16))
     with pytest.raises(ValueError):
         mtq.set_fp8_overflow_behavior("wrap")
+
+
+@pytest.mark.parametrize("name", sorted(n for n in mtq.config.choices if not n.endswith("KV_CFG")))
+def test_every_named_config_runs_on_the_hf_model(name):
+    """Each stock config (with the FP8 KV-cache quantizers merged in, as the reference's
+    llm_ptq example does) converts, calibrates and runs a forward on the tiny Llama; the
+    quantised logits stay within the error a 4- to 8-bit format gives on a random model."""
+    model, ids = _tiny_llama(), _ids()
+    ref = model(ids).logits
+    previous = mtq.set_fp8_overflow_behavior("saturate")
+    try:
+        mtq.quantize(model, _with_kv(getattr(mtq, name)), lambda m: m(ids))
+        out = model(ids).logits
+    finally:
+        mtq.set_fp8_overflow_behavior(previous)
+    assert torch.isfinite(out).all()
+    err = ((out.float() - ref.float()).norm() / ref.float().norm()).item()
+    assert err < 0.5, err
+    assert any(getattr(m, "is_enabled", False) for n, m in model.named_modules()
+               if n.endswith("weight_quantizer"))
