@@ -154,6 +154,94 @@ __global__ __launch_bounds__(256) void nf4_quantize_tile_kernel(
     }
 }
 
+// Table form for the 16-bit dtypes and large inputs.  The scaled value v is itself a 16-bit value
+// with |v| <= 1, so its code can be read from a table indexed by its bit pattern: 0x3F81
+// magnitudes for bf16 (0 .. 1.0), 0x3C01 for fp16, times two signs -- under 32 KiB of one-byte
+// codes.  A small kernel fills the table in device memory from the same thresholds (so the two
+// forms agree by construction); a workgroup copies it to LDS once and then converts
+// kNf4LutTiles tiles, which replaces the 19-instruction search per element by one LDS read.
+// Chunks whose block abs-max is zero, tiny or not finite take the threshold search.
+constexpr int kNf4LutBytes = 32768;
+constexpr int kNf4LutTiles = 8;
+template <int DT> struct Nf4Lut;
+template <> struct Nf4Lut<MO_BF16> { static constexpr int half = 0x3F81, slot = 0; };
+template <> struct Nf4Lut<MO_F16> { static constexpr int half = 0x3C01, slot = 1; };
+
+__device__ __align__(16) uint8_t g_nf4_lut[2][kNf4LutBytes];
+
+template <int DT>
+__global__ __launch_bounds__(256) void nf4_build_lut_kernel(Nf4Thresholds thresholds) {
+    const Nf4Regs th = nf4_regs(thresholds);
+    constexpr int half = Nf4Lut<DT>::half;
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= kNf4LutBytes) return;
+    uint32_t code = 0;
+    if (e < 2 * half) {
+        const uint32_t sign = e >= half ? 1u : 0u;
+        const uint32_t bits = (uint32_t)(e - (int)sign * half) | (sign << 15);
+        const float v = DT == MO_BF16 ? bf16_bits_to_f32(bits) : f16_bits_to_f32(bits);
+        code = nf4_code(v, th);
+    }
+    g_nf4_lut[Nf4Lut<DT>::slot][e] = (uint8_t)code;
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void nf4_quantize_lut_kernel(
+    const void* __restrict__ x, int64_t chunks, int lanes_per_block, int shift,
+    Nf4Thresholds thresholds, void* __restrict__ scales, uint32_t* __restrict__ packed) {
+    __shared__ __align__(16) uint8_t lut[kNf4LutBytes];
+    constexpr int half = Nf4Lut<DT>::half;
+    {
+        const u32x4* src = (const u32x4*)g_nf4_lut[Nf4Lut<DT>::slot];
+        u32x4* dst = (u32x4*)lut;
+#pragma unroll
+        for (int i = 0; i < kNf4LutBytes / 16 / 256; ++i) dst[threadIdx.x + i * 256] = src[threadIdx.x + i * 256];
+    }
+    __syncthreads();
+    const Nf4Regs th = nf4_regs(thresholds);
+    for (int t = 0; t < kNf4LutTiles; ++t) {
+        const int64_t c0 = ((int64_t)blockIdx.x * kNf4LutTiles + t) * kNf4TileChunks + threadIdx.x;
+        if (c0 - threadIdx.x >= chunks) break;  // uniform: the whole tile is past the end
+        RawChunk<DT> raw[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t c = c0 + u * 256;
+            zero_raw<DT>(raw[u]);
+            if (c < chunks) load_raw<DT>(x, c << 3, raw[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t c = c0 + u * 256;
+            float v[8];
+            unpack_raw<DT>(raw[u], v);
+            uint32_t m = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t a = f2u(v[j]) & 0x7FFFFFFFu;
+                m = a > m ? a : m;
+            }
+            m = group_max_u32(m, shift);
+            if (c >= chunks) continue;
+            const float amax = u2f(m);
+            if ((threadIdx.x & (lanes_per_block - 1)) == 0) store_elem<DT>(scales, c >> shift, amax);
+            uint32_t w = 0;
+            if (mid_range(amax)) {
+                const float r = 1.0f / amax;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float q = exact_quotient(v[j], amax, r);
+                    const uint32_t bits = DT == MO_BF16 ? f32_to_bf16_bits(q) : f32_to_f16_bits(q);
+                    const uint32_t entry = (bits & 0x7FFFu) + ((bits >> 15) & 1u) * (uint32_t)half;
+                    w |= (uint32_t)lut[entry] << (4 * (j ^ 1));
+                }
+            } else {
+                w = nf4_codes8<DT>(v, amax, th);
+            }
+            __builtin_nontemporal_store(w, packed + c);
+        }
+    }
+}
+
 // y[2i] = T(table[byte >> 4] * f32(scale[block])), y[2i + 1] = T(table[byte & 15] * ...)
 template <int DT>
 __global__ __launch_bounds__(256) void nf4_dequantize_kernel(const uint8_t* __restrict__ packed,
@@ -286,6 +374,19 @@ extern "C" int mo_nf4_quantize(const void* x, int64_t n, int64_t block_size, int
     const int64_t tiles = (n / 8 + mo::kNf4TileChunks - 1) / mo::kNf4TileChunks;
     if (shift >= 0 && n % block_size == 0 && (((uintptr_t)x & 15u) == 0) &&
         (((uintptr_t)packed & 3u) == 0) && tiles <= 0x7FFFFFFF) {
+        if (dtype != MO_F32 && tiles >= 64 * mo::kNf4LutTiles) {  // large 16-bit input: table form
+            const unsigned g = (unsigned)((tiles + mo::kNf4LutTiles - 1) / mo::kNf4LutTiles);
+            if (dtype == MO_BF16) {
+                mo::nf4_build_lut_kernel<MO_BF16><<<mo::kNf4LutBytes / 256, 256, 0, s>>>(th);
+                mo::nf4_quantize_lut_kernel<MO_BF16><<<g, 256, 0, s>>>(
+                    x, n / 8, 1 << shift, shift, th, scales, (uint32_t*)packed);
+            } else {
+                mo::nf4_build_lut_kernel<MO_F16><<<mo::kNf4LutBytes / 256, 256, 0, s>>>(th);
+                mo::nf4_quantize_lut_kernel<MO_F16><<<g, 256, 0, s>>>(
+                    x, n / 8, 1 << shift, shift, th, scales, (uint32_t*)packed);
+            }
+            return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+        }
 #define CALL(DT)                                                                    \
     mo::nf4_quantize_tile_kernel<DT><<<(unsigned)tiles, 256, 0, s>>>(               \
         x, n / 8, 1 << shift, shift, th, scales, (uint32_t*)packed)

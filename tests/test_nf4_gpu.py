@@ -69,6 +69,26 @@ def test_quantize_every_scaled_value(dtype):
     _check_quantize(blocks.flatten(), 8)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_quantize_every_scaled_value_on_the_table_path(dtype):
+    """Inputs of 4 M elements and more take the table-lookup kernel (16-bit dtypes): every
+    16-bit scaled value again, at block scales 2^-3 .. 2^4 (exact, so v stays the same value),
+    plus random blocks, all-zero and NaN blocks."""
+    v = _all_values_in_unit_range(dtype)
+    blocks = torch.ones(v.numel(), 8, dtype=dtype)
+    blocks[:, 1] = v
+    blocks[:, 5] = -v
+    parts = [blocks * (2.0 ** e) for e in range(-3, 5)]
+    g = torch.Generator().manual_seed(17)
+    rnd = (torch.randn(1 << 22, generator=g) * torch.exp(torch.randn(1 << 22, generator=g))).to(dtype)
+    x = torch.cat([p.flatten() for p in parts] + [rnd])
+    x = torch.cat([x, torch.zeros((-x.numel()) % (8192 * 8), dtype=dtype)])
+    x[-40:] = float("nan")
+    assert x.numel() >= 64 * 8 * 8192
+    _check_quantize(x, 8)
+    _check_quantize(x, 64)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_quantize_values_around_the_decision_points(dtype):
     """fp32 neighbours of every midpoint between table entries, at several block scales"""
