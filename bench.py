@@ -188,6 +188,23 @@ def single_tensor_configs(torch, steps, warmup):
     out["c3_awq_lite_21_alphas_4096x4096"] = {
         "end_to_end_ms": round(secs * 1e3, 3), "gemm_flops": flops,
         "gemm_TFLOPs_over_end_to_end": round(flops / secs / 1e12, 1)}
+
+    # the search step of that configuration on its own: one launch scores all 21 alphas (weights
+    # scaled and INT4 block-quantised on the fly, bf16 MFMA GEMM, loss in the epilogue); the
+    # MFMA roofline is MI355X's dense bf16 peak
+    import torch.nn.functional as F
+    scales = torch.exp(0.5 * torch.randn(21, 4096, generator=g)).to(torch.bfloat16).to(dev)
+    ref = F.linear(x3, w3).contiguous()
+    xs = _hip.awq_scaled_activations(x3, (1 / scales.float()).to(torch.bfloat16))
+    loss = torch.zeros(21, dtype=torch.float64, device=dev)
+
+    def search():
+        _hip.awq_search_losses_into(xs, w3, scales, ref, 128, 4, False, False, loss)
+    _, ms = timed(torch, search, steps, warmup)
+    kflops = 2 * 512 * 4096 * 4096 * 21
+    out["c3_awq_search_kernel_21_alphas"] = {
+        "ms": round(ms, 4), "TFLOPs": round(kflops / ms / 1e9, 1), "bound": "mfma",
+        "peak_TFLOPs": 2500.0, "frac": round(kflops / ms / 1e9 / 2500.0, 4)}
     return out
 
 
