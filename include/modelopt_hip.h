@@ -39,8 +39,13 @@ const char* mo_error_string(int status);
 /* Process-wide switches (debug / verification aids; defaults are all 0).
  * MO_OPT_FORCE_EXACT = 1 makes the NVFP4 quantize kernels divide every element by its block
  * scale (the reference's literal arithmetic) instead of the multiply-and-verify fast path; the
- * outputs are identical either way, which is what the switch exists to demonstrate. */
-enum mo_option { MO_OPT_FORCE_EXACT = 0, MO_OPT_COUNT_ = 1 };
+ * outputs are identical either way, which is what the switch exists to demonstrate.
+ * MO_OPT_SATURATE_BLOCK_SCALE = 1 makes the NVFP4 quantize kernels clamp a block scale at 448
+ * before its E4M3 cast.  The reference's cast (TQ/qtensor/nvfp4_tensor.py:84-91) is torch's
+ * non-saturating one: a block whose abs-max exceeds the per-tensor amax by more than 448/464
+ * (possible once awq_clip has shrunk that amax, TQ/model_calib.py:869-876) gets the NaN byte
+ * and dequantises to NaN.  0 keeps that behaviour. */
+enum mo_option { MO_OPT_FORCE_EXACT = 0, MO_OPT_SATURATE_BLOCK_SCALE = 1, MO_OPT_COUNT_ = 2 };
 int mo_set_option(int key, int value);
 int mo_get_option(int key);
 

@@ -15,12 +15,20 @@ namespace mo {
 // E4M3 byte of a block scale bs = bmax / gs6 (0 -> 1.0).  When the quotient is NaN because of
 // an invalid operation (0/0, inf/inf) the x86 reference produces the negative default NaN and
 // therefore the byte 0xFF; a NaN that comes from a NaN operand keeps that operand's (positive)
-// sign and gives 0x7F.
-__device__ __forceinline__ uint32_t block_scale_byte(float bmax, float gs6) {
+// sign and gives 0x7F.  `cap` is +inf for the reference's cast (a quotient above E4M3's range
+// becomes the NaN byte) or 448 to saturate instead (option MO_OPT_SATURATE_BLOCK_SCALE).
+__device__ __forceinline__ uint32_t block_scale_byte(float bmax, float gs6,
+                                                     float cap = __builtin_inff()) {
     float bs = bmax / gs6;
     if (bs == 0.0f) bs = 1.0f;
     if (bs != bs) return (bmax != bmax || gs6 != gs6) ? 0x7Fu : 0xFFu;
-    return f32_to_e4m3<false>(bs);
+    return f32_to_e4m3<false>(bs < cap ? bs : cap);
+}
+
+// bits of the `opts` kernel argument
+constexpr int kOptForceExact = 1, kOptSaturateScale = 2;
+__device__ __forceinline__ float scale_cap(int opts) {
+    return (opts & kOptSaturateScale) ? 448.0f : __builtin_inff();
 }
 
 template <int G>
@@ -63,10 +71,12 @@ template <int DT, int BS, bool FLAT>
 __global__ __launch_bounds__(256) void nvfp4_quantize_kernel(
     const void* __restrict__ x, int64_t total_chunks, int64_t k, int64_t cpr,
     const float* __restrict__ amax, int amax_is_wsf2, const uint8_t* __restrict__ wsf_in,
-    uint32_t* __restrict__ packed, uint8_t* __restrict__ wsf_out, float* __restrict__ wsf2_out) {
+    uint32_t* __restrict__ packed, uint8_t* __restrict__ wsf_out, float* __restrict__ wsf2_out,
+    int opts) {
     constexpr int G = BS / 8;
     const float wsf2 = amax_is_wsf2 ? amax[0] : amax[0] / 2688.0f;  // 6 * 448
     const float gs6 = 6.0f * wsf2;
+    const float cap = scale_cap(opts);
     if (wsf2_out && blockIdx.x == 0 && threadIdx.x == 0) wsf2_out[0] = wsf2;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < total_chunks;
@@ -79,7 +89,7 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_kernel(
             byte = wsf_in[c / G];
         } else {
             const float bmax = u2f(group_max<G>(chunk_absmax_bits(v)));
-            byte = block_scale_byte(bmax, gs6);
+            byte = block_scale_byte(bmax, gs6, cap);
             if (wsf_out && (threadIdx.x & (G - 1)) == 0) wsf_out[c / G] = (uint8_t)byte;
         }
         const float s = e4m3_to_f32(byte) * wsf2;
@@ -198,14 +208,15 @@ __device__ __forceinline__ uint32_t exact_codes8(const uint32_t (&w)[4], float s
 
 // One 16-element bf16 block held as 8 packed words -> scale byte and 64 bits of codes.
 __device__ __forceinline__ void quantize_block16_bf16(const uint32_t (&w)[8], float wsf2, float gs6,
-                                                      bool force_exact, uint32_t& byte,
+                                                      int opts, uint32_t& byte,
                                                       uint32_t& c_lo, uint32_t& c_hi) {
+    const bool force_exact = opts & kOptForceExact;
     uint32_t m = w[0] & 0x7FFF7FFFu;
 #pragma unroll
     for (int j = 1; j < 8; ++j) m = pk_max_u16(m, w[j] & 0x7FFF7FFFu);
     const uint32_t h = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
     const float bmax = u2f(h << 16);
-    byte = block_scale_byte(bmax, gs6);
+    byte = block_scale_byte(bmax, gs6, scale_cap(opts));
     const float s = e4m3_to_f32(byte) * wsf2;
     const uint32_t sb = f2u(s);
     const float r = 1.0f / s;
@@ -245,7 +256,7 @@ __device__ __forceinline__ uint32_t swap_adjacent_lanes(uint32_t v) {
 
 __device__ __forceinline__ void quantize_tile_bf16(const uint16_t* __restrict__ x,
                                                    int64_t nblocks, int64_t tile, float wsf2,
-                                                   float gs6, bool force_exact,
+                                                   float gs6, int opts,
                                                    u32x2* __restrict__ packed,
                                                    uint8_t* __restrict__ wsf) {
     constexpr int RP = kTileBlocks / 256;  // round pairs
@@ -273,7 +284,7 @@ __device__ __forceinline__ void quantize_tile_bf16(const uint16_t* __restrict__ 
         const uint32_t w[8] = {first.x, first.y, first.z, first.w,
                                second.x, second.y, second.z, second.w};
         uint32_t byte, lo, hi;
-        quantize_block16_bf16(w, wsf2, gs6, force_exact, byte, lo, hi);
+        quantize_block16_bf16(w, wsf2, gs6, opts, byte, lo, hi);
         const int64_t mine = odd ? cb : ca;  // odd: chunks (cb - 1, cb); even: (ca, ca + 1)
         if (mine < nchunks) {
             const int64_t blk = mine >> 1;
@@ -286,12 +297,12 @@ __device__ __forceinline__ void quantize_tile_bf16(const uint16_t* __restrict__ 
 
 __global__ __launch_bounds__(256) void nvfp4_quantize_fast_kernel(
     const uint16_t* __restrict__ x, int64_t nblocks, int64_t tiles,
-    const float* __restrict__ amax, int amax_is_wsf2, int force_exact,
+    const float* __restrict__ amax, int amax_is_wsf2, int opts,
     u32x2* __restrict__ packed, uint8_t* __restrict__ wsf_out, float* __restrict__ wsf2_out) {
     const float wsf2 = amax_is_wsf2 ? amax[0] : amax[0] / 2688.0f;
     const float gs6 = 6.0f * wsf2;
     if (wsf2_out && blockIdx.x == 0 && threadIdx.x == 0) wsf2_out[0] = wsf2;
-    quantize_tile_bf16(x, nblocks, blockIdx.x, wsf2, gs6, force_exact != 0, packed, wsf_out);
+    quantize_tile_bf16(x, nblocks, blockIdx.x, wsf2, gs6, opts, packed, wsf_out);
 }
 
 // Many tensors, one launch.  One workgroup per tile, dispatched in tile order so the set of
@@ -300,7 +311,7 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_fast_kernel(
 // t; without it the job is found by binary search over tile_begin.
 __global__ __launch_bounds__(256) void nvfp4_quantize_multi_kernel(
     const mo_nvfp4_job* __restrict__ jobs, int njobs, const int32_t* __restrict__ tile_job,
-    int amax_is_wsf2, int force_exact) {
+    int amax_is_wsf2, int opts) {
     const int64_t t = blockIdx.x;
     int lo;
     if (tile_job) {
@@ -318,7 +329,7 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_multi_kernel(
     const float wsf2 = amax_is_wsf2 ? a : a / 2688.0f;
     if (jb.wsf2_out && t == jb.tile_begin && threadIdx.x == 0) jb.wsf2_out[0] = wsf2;
     quantize_tile_bf16((const uint16_t*)jb.x, jb.elems >> 4, t - jb.tile_begin, wsf2, 6.0f * wsf2,
-                       force_exact != 0, (u32x2*)jb.packed, jb.wsf);
+                       opts, (u32x2*)jb.packed, jb.wsf);
 }
 
 // ------------------------------------------------------------------------------ fast dequantize
@@ -504,15 +515,15 @@ static inline unsigned grid_for(int64_t chunks) {
 template <int DT, int BS>
 static void launch_quantize(const void* x, int64_t rows, int64_t k, int64_t kp, const float* amax,
                             int is_wsf2, const uint8_t* wsf_in, uint8_t* packed, uint8_t* wsf_out,
-                            float* wsf2_out, hipStream_t s) {
+                            float* wsf2_out, int opts, hipStream_t s) {
     const int64_t cpr = kp / 8, total = rows * cpr;
     const bool flat = (k == kp) && (((uintptr_t)x & 15u) == 0);
     if (flat)
         nvfp4_quantize_kernel<DT, BS, true><<<grid_for(total), 256, 0, s>>>(
-            x, total, k, cpr, amax, is_wsf2, wsf_in, (uint32_t*)packed, wsf_out, wsf2_out);
+            x, total, k, cpr, amax, is_wsf2, wsf_in, (uint32_t*)packed, wsf_out, wsf2_out, opts);
     else
         nvfp4_quantize_kernel<DT, BS, false><<<grid_for(total), 256, 0, s>>>(
-            x, total, k, cpr, amax, is_wsf2, wsf_in, (uint32_t*)packed, wsf_out, wsf2_out);
+            x, total, k, cpr, amax, is_wsf2, wsf_in, (uint32_t*)packed, wsf_out, wsf2_out, opts);
 }
 
 template <int DT, int BS>
@@ -531,6 +542,12 @@ static void launch_qdq(const void* x, void* y, int64_t rows, int64_t k, int64_t 
 }
 
 }  // namespace mo
+
+// option bits handed to the quantize kernels
+static int quantize_opts() {
+    return (mo_get_option(MO_OPT_FORCE_EXACT) ? mo::kOptForceExact : 0) |
+           (mo_get_option(MO_OPT_SATURATE_BLOCK_SCALE) ? mo::kOptSaturateScale : 0);
+}
 
 #define MO_DISPATCH_DT_BS(dtype, bs, CALL)                                            \
     switch (dtype) {                                                                  \
@@ -566,12 +583,13 @@ extern "C" int mo_nvfp4_quantize(const void* x, int64_t rows, int64_t k, int dty
         const int64_t tiles = (nblocks + mo::kTileBlocks - 1) / mo::kTileBlocks;
         if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
         mo::nvfp4_quantize_fast_kernel<<<(unsigned)tiles, 256, 0, s>>>(
-            (const uint16_t*)x, nblocks, tiles, amax, amax_is_wsf2, mo_get_option(MO_OPT_FORCE_EXACT),
+            (const uint16_t*)x, nblocks, tiles, amax, amax_is_wsf2, quantize_opts(),
             (mo::u32x2*)packed, wsf_out, wsf2_out);
         return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
     }
 #define CALL(DT, BS) \
-    mo::launch_quantize<DT, BS>(x, rows, k, kp, amax, amax_is_wsf2, wsf_in, packed, wsf_out, wsf2_out, s)
+    mo::launch_quantize<DT, BS>(x, rows, k, kp, amax, amax_is_wsf2, wsf_in, packed, wsf_out, wsf2_out, \
+                                quantize_opts(), s)
     MO_DISPATCH_DT_BS(dtype, block_size, CALL)
 #undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
@@ -641,6 +659,6 @@ extern "C" int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs,
     if (njobs == 0 || total_tiles == 0) return MO_OK;
     if (!jobs_dev) return MO_ERR_ARG;
     mo::nvfp4_quantize_multi_kernel<<<(unsigned)total_tiles, 256, 0, (hipStream_t)stream>>>(
-        jobs_dev, njobs, tile_job_dev, amax_is_wsf2, mo_get_option(MO_OPT_FORCE_EXACT));
+        jobs_dev, njobs, tile_job_dev, amax_is_wsf2, quantize_opts());
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

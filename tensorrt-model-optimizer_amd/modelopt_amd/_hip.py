@@ -419,6 +419,7 @@ def sq_diff_sum_into(a, b, acc):
 # ----------------------------------------------------------------------------- options
 
 MO_OPT_FORCE_EXACT = 0
+MO_OPT_SATURATE_BLOCK_SCALE = 1
 
 
 def set_option(key: int, value: int):

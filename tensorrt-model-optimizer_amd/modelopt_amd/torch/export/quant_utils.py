@@ -13,10 +13,13 @@ from torch import nn
 
 from ... import __version__, _hip
 from ..quantization.nn import SequentialQuantizer, TensorQuantizer
-from ..quantization.qtensor import NVFP4QTensor, QTensorWrapper
+from ..quantization.qtensor import FP8QTensor, MXFP4QTensor, NVFP4QTensor, QTensorWrapper
 from ..quantization.utils import (quantizer_attr_names, reduce_block_amax, true_divide,
                                   weight_attr_names)
 from .model_config import *  # noqa: F403
+
+_NVFP4_FAMILY = (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ, QUANTIZATION_W4A8_NVFP4_FP8)
+_MXFP4_FAMILY = (QUANTIZATION_MXFP4, QUANTIZATION_W4A8_MXFP4_FP8)
 
 __all__ = [
     "get_scaling_factor_from_weight", "get_scaling_factor", "get_activation_scaling_factor",
@@ -75,10 +78,19 @@ def get_weight_scaling_factor(module: nn.Module, weight_name: str = "weight"):
         return None
     if isinstance(wq, SequentialQuantizer):
         return get_scaling_factor(wq[0])
-    if get_quantization_format(module) in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
-        wsf2 = NVFP4QTensor.get_weights_scaling_factor_2_from_quantizer(wq)
+    fmt = get_quantization_format(module)
+    if fmt in _NVFP4_FAMILY:
+        if fmt == QUANTIZATION_W4A8_NVFP4_FP8:
+            # the consumer dequantises the weight to FP8 (range 448), so the block scales are
+            # laid out against amax / 448 rather than amax / (6 * 448)
+            wsf2 = true_divide(wq._amax.float(), 448.0)
+        else:
+            wsf2 = NVFP4QTensor.get_weights_scaling_factor_2_from_quantizer(wq)
         return NVFP4QTensor.get_weights_scaling_factor(weight, wq.block_sizes[-1],
                                                        wsf2.to(weight.device))[0]
+    if fmt in _MXFP4_FAMILY:
+        return MXFP4QTensor.quantize(weight, block_size=wq.block_sizes[-1])[1].reshape(
+            *weight.shape[:-1], -1)
     return get_scaling_factor(wq)
 
 
@@ -86,8 +98,11 @@ def get_weight_scaling_factor_2(module: nn.Module, weight_name: str = "weight"):
     wq = getattr(module, quantizer_attr_names(weight_name).weight_quantizer, None)
     if wq is None:
         return None
-    if get_quantization_format(module) in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
+    fmt = get_quantization_format(module)
+    if fmt in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
         return NVFP4QTensor.get_weights_scaling_factor_2_from_quantizer(wq)
+    if fmt == QUANTIZATION_W4A8_NVFP4_FP8:
+        return true_divide(wq._amax.float(), 448.0)
     if not isinstance(wq, SequentialQuantizer) or not wq[-1].is_enabled:
         return None
     assert len(wq) == 2, "modelopt only supports 2 sequential quantization layers for now"
@@ -149,13 +164,27 @@ def get_quantization_format(module) -> str | None:
             return QUANTIZATION_INT8_SQ if iq is not None and iq.is_enabled else QUANTIZATION_INT8_WO
         if wq.num_bits == (4, 3):
             if wq.block_sizes:
-                raise NotImplementedError("FP8 block-scaled export is outside the path built here")
+                assert wq.block_sizes[-1] > 0, "Invalid block_sizes for FP8 quantizer"
+                return QUANTIZATION_FP8_PB_WO if wq.fake_quant else QUANTIZATION_FP8_PB_REAL
             return QUANTIZATION_FP8_PC_PT if wq.axis == 0 else QUANTIZATION_FP8
         if wq.num_bits == (2, 1):
+            blocks = wq.block_sizes
+            scale_bits = blocks.get("scale_bits")
             if iq is not None and hasattr(iq, "_pre_quant_scale"):
                 return QUANTIZATION_NVFP4_AWQ
-            if wq.block_sizes.get("scale_bits") == (4, 3):
+            if getattr(layer, "fused_with_prequant", False):
+                return QUANTIZATION_NVFP4_AWQ
+            assert iq is not None, f"input_quantizer is None for {names}"
+            fp8_input = (blocks.get("type", "static") == "dynamic" and iq.is_enabled
+                         and iq.num_bits == (4, 3) and iq.block_sizes is None)
+            if fp8_input and scale_bits == (8, 0):
+                return QUANTIZATION_W4A8_MXFP4_FP8
+            if fp8_input and scale_bits == (4, 3):
+                return QUANTIZATION_W4A8_NVFP4_FP8
+            if scale_bits == (4, 3):
                 return QUANTIZATION_NVFP4
+            if scale_bits == (8, 0):
+                return QUANTIZATION_MXFP4
         raise NotImplementedError(f"Unsupported quantizer with num_bits: {wq.num_bits}")
 
     for weight_name in weight_attr_names(module):
@@ -211,6 +240,9 @@ _LAYER_CONFIGS = {
     "nvfp4": lambda b: {"quant_algo": "NVFP4", "group_size": b},
     "nvfp4_awq": lambda b: {"quant_algo": "NVFP4_AWQ", "group_size": b, "has_zero_point": False,
                             "pre_quant_scale": True},
+    "w4a8_nvfp4_fp8": lambda b: {"quant_algo": "W4A8_NVFP4_FP8", "group_size": b,
+                                 "has_zero_point": False, "pre_quant_scale": True},
+    "w4a8_mxfp4_fp8": lambda b: {"quant_algo": "W4A8_MXFP4_FP8", "group_size": b},
 }
 
 
@@ -275,18 +307,23 @@ def to_quantized_weight(weight, weights_scaling_factor, quantization: str,
         s = weights_scaling_factor.reshape(-1).contiguous()
         return _hip.real_quantize(w, s, 1, w.shape[0], w.shape[1], torch.result_type(w, s[:, None]),
                                   _hip.MO_FMT_INT8)
+    if quantization == QUANTIZATION_FP8_PB_WO:
+        return FP8QTensor.quantize(weight, weights_scaling_factor.squeeze(),
+                                   block_sizes={-1: block_size, -2: block_size})[0]._quantized_data
     if quantization == QUANTIZATION_FP8_PC_PT:
         s = weights_scaling_factor.reshape(-1).contiguous()
         return _hip.real_quantize(w, s, 1, w.shape[0], w.shape[1], torch.result_type(w, s[:, None]),
                                   _hip.MO_FMT_E4M3)
     if quantization in (QUANTIZATION_INT4_AWQ, QUANTIZATION_W4A8_AWQ):
         return pack_int4_in_uint8(weight, weights_scaling_factor)
-    if quantization in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
+    if quantization in _NVFP4_FAMILY:
         assert block_size is not None, "Block size not passed. Unable to quantize to NVFP4 format."
         assert weights_scaling_factor2 is not None, (
             "Weights scaling factor 2 not passed. Unable to quantize to NVFP4 format")
         return NVFP4QTensor.quantize(weight, block_size, weights_scaling_factor,
                                      weights_scaling_factor2)[0]._quantized_data
+    if quantization in _MXFP4_FAMILY:
+        return MXFP4QTensor.quantize(weight, block_size=block_size)[0]._quantized_data
     raise NotImplementedError(f"quantization format {quantization} not supported")
 
 

@@ -17,7 +17,7 @@ from torch import nn
 
 from ... import _hip
 from ..quantization.nn import SequentialQuantizer, TensorQuantizer
-from ..quantization.qtensor import NVFP4QTensor
+from ..quantization.qtensor import NVFP4QTensor, QTensorWrapper
 from ..quantization.utils import is_quantized_linear, true_divide
 from .model_config import *  # noqa: F403
 from ..quantization.conversion import set_quantizer_by_cfg_context
@@ -57,15 +57,22 @@ def _export_quantized_weight(module: nn.Module, dtype: torch.dtype):
             iq._amax = iq._amax.to(torch.float32)
             module.register_buffer("input_scale", get_activation_scaling_factor(module).squeeze())
     else:
-        if fmt not in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
+        if fmt == QUANTIZATION_FP8_PB_REAL:
+            # already packed by ``compress``: the scales live on the quantizer
+            module.register_buffer("weight_scale", wq._scale.to(torch.float32))
+            del wq._scale
+        elif fmt not in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
             module.register_buffer("weight_scale", get_weight_scaling_factor(module))
         _register_input_scale(module, iq)
-    if fmt in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ, QUANTIZATION_W4A8_AWQ):
+    if fmt in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ, QUANTIZATION_W4A8_AWQ,
+               QUANTIZATION_W4A8_NVFP4_FP8):
         module.register_buffer("weight_scale_2", get_weight_scaling_factor_2(module).squeeze())
 
     weight_scale = getattr(module, "weight_scale", None)
     weight_scale_2 = getattr(module, "weight_scale_2", None)
-    if fmt in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
+    if isinstance(weight, QTensorWrapper):
+        quantized = weight.data                 # packed by ``compress`` already
+    elif fmt in (QUANTIZATION_NVFP4, QUANTIZATION_NVFP4_AWQ):
         # block scales and codes from one pass over the weight
         qt, weight_scale, _ = NVFP4QTensor.quantize(weight.data.to(dtype), block,
                                                     weights_scaling_factor_2=weight_scale_2)
@@ -152,7 +159,8 @@ def requantize_resmooth_fused_llm_layers(model: nn.Module):
         groups = [(None, g) for g in _fusable_groups(model)]
     for tensor, modules in groups:
         fmt = get_quantization_format(modules[0])
-        if len(modules) > 1 and fmt not in (QUANTIZATION_FP8, QUANTIZATION_NONE):
+        if len(modules) > 1 and fmt not in (QUANTIZATION_FP8, QUANTIZATION_NONE,
+                                            QUANTIZATION_FP8_PB_REAL):
             preprocess_linear_fusion(modules)
         if (fmt is not QUANTIZATION_NONE and fmt is not None and "awq" in fmt and tensor is not None
                 and tensor in output_to_layernorm
@@ -195,18 +203,20 @@ def convert_hf_quant_config_format(input_config: dict[str, Any]) -> dict[str, An
         group = {"input_activations": {"dynamic": False, "num_bits": 8, "type": "float"},
                  "weights": {"dynamic": False, "num_bits": 8, "type": "float"}, "targets": ["Linear"]}
     elif algo == "NVFP4":
-        gs = q.get("group_size")
+        gs = q.get("group_size", 16)
         group = {"input_activations": {"dynamic": False, "num_bits": 4, "type": "float", "group_size": gs},
                  "weights": {"dynamic": False, "num_bits": 4, "type": "float", "group_size": gs},
                  "targets": ["Linear"]}
     if group is not None:
         out["config_groups"] = {"group_0": group}
-    out["ignore"] = q.get("exclude_modules", [])
-    out["quant_algo"] = algo
+    out["ignore"] = q.get("exclude_modules") or []
+    if algo:
+        out["quant_algo"] = algo
     if q.get("kv_cache_quant_algo"):
         out["kv_cache_scheme"] = {"dynamic": False, "num_bits": 8, "type": "float"} if q[
             "kv_cache_quant_algo"] == "FP8" else q["kv_cache_quant_algo"]
-    out["producer"] = input_config.get("producer", {})
+    if input_config.get("producer"):
+        out["producer"] = input_config["producer"]
     out["quant_method"] = "modelopt"
     return out
 

@@ -7,6 +7,7 @@ reproduced; conversion acts on the model in place.
 """
 
 import fnmatch
+import warnings
 from contextlib import contextmanager
 from typing import Any
 
@@ -89,7 +90,9 @@ def _quantizer_index(quant_model: nn.Module):
 def set_quantizer_attribute(quant_model: nn.Module, wildcard_or_filter_func, attribute,
                             parent_class: type | None = None, _index=None):
     """Set attributes on every quantizer whose qualified name matches.  A list of attribute
-    dicts turns the matched ``TensorQuantizer`` into a ``SequentialQuantizer``."""
+    dicts turns the matched ``TensorQuantizer`` into a ``SequentialQuantizer``; a single dict on
+    a ``SequentialQuantizer`` is applied to each of its members (reference: conversion.py
+    :276-301)."""
     index = _quantizer_index(quant_model) if _index is None else _index
     many = isinstance(attribute, (list, tuple))
     cfg = [_as_cfg(a) for a in attribute] if many else _as_cfg(attribute)
@@ -108,11 +111,9 @@ def set_quantizer_attribute(quant_model: nn.Module, wildcard_or_filter_func, att
                 setattr(parent, leaf, module)
                 entry[1] = module
             elif len(attribute) != len(module):
-                raise ValueError("number of attributes does not match the SequentialQuantizer")
-        elif isinstance(module, SequentialQuantizer):
-            module = TensorQuantizer()
-            setattr(parent, leaf, module)
-            entry[1] = module
+                warnings.warn(f"The number of attributes ({len(attribute)}) does not match the number "
+                              f"of quantizers of {module} leading to partial assignment.")
+        # one dict on a SequentialQuantizer goes to every member
         module.set_from_attribute_config(cfg)
 
 

@@ -10,6 +10,7 @@ estimator that zeroes gradients where ``|x| > amax`` unless ``pass_through_bwd``
 import torch
 from torch.autograd import Function
 
+from ... import _hip
 from . import kernels
 from .config import QuantizerAttributeConfig
 
@@ -39,11 +40,19 @@ _FP8_OVERFLOW = "nan"
 
 def set_fp8_overflow_behavior(mode: str) -> str:
     """``"nan"`` (eager / CPU semantics, default) or ``"saturate"`` (the CUDA kernel's).  Returns
-    the previous mode."""
+    the previous mode.
+
+    The mode also governs the E4M3 cast of NVFP4 block scales in *real* quantisation (compress,
+    export): the reference casts with torch's non-saturating conversion
+    (qtensor/nvfp4_tensor.py:84-91), so a block whose abs-max lies above the per-tensor amax --
+    which ``awq_clip`` shrinks for NVFP4 (model_calib.py:869-876) -- stores the NaN byte;
+    ``"saturate"`` stores 448 instead, which is what the fake-quant kernel the clip search
+    itself ran on computes with."""
     global _FP8_OVERFLOW
     if mode not in ("nan", "saturate"):
         raise ValueError(f"mode must be 'nan' or 'saturate', got {mode!r}")
     previous, _FP8_OVERFLOW = _FP8_OVERFLOW, mode
+    _hip.set_option(_hip.MO_OPT_SATURATE_BLOCK_SCALE, int(mode == "saturate"))
     return previous
 
 

@@ -42,6 +42,7 @@ def test_version_and_error_strings_without_gpu():
     assert b"invalid argument" in lib.mo_error_string(-1)
     assert lib.mo_set_option(99, 1) == -1
     assert lib.mo_get_option(_hip.MO_OPT_FORCE_EXACT) == 0
+    assert lib.mo_get_option(_hip.MO_OPT_SATURATE_BLOCK_SCALE) == 0
 
 
 def test_missing_library_fails_loudly(monkeypatch):

@@ -110,6 +110,20 @@ def test_list_attribute_makes_sequential_quantizer():
     assert equ.get_quantization_format(m.body[0]) == "w4a8_awq"
 
 
+def test_one_dict_on_a_sequential_quantizer_goes_to_every_member():
+    """reference conversion.py:292-301, nn/modules/tensor_quantizer.py:1182-1196: the
+    SequentialQuantizer stays, each member takes the attributes; the export's dummy forward
+    relies on this to switch W4A8 quantizers off and back on."""
+    m = _converted(mtq.W4A8_AWQ_BETA_CFG)
+    with mtq.set_quantizer_by_cfg_context(m, {"*": {"enable": False}}):
+        wq = m.body[0].weight_quantizer
+        assert isinstance(wq, SequentialQuantizer) and not wq[0].is_enabled and not wq[1].is_enabled
+    wq = m.body[0].weight_quantizer
+    assert isinstance(wq, SequentialQuantizer) and wq[0].is_enabled and wq[1].is_enabled
+    assert wq[0].num_bits == 4 and wq[1].num_bits == (4, 3)
+    assert equ.get_quantization_format(m.body[0]) == "w4a8_awq"
+
+
 def test_set_quantizer_by_cfg_context_restores():
     m = _converted(mtq.INT8_DEFAULT_CFG)
     q = m.body[0].input_quantizer

@@ -157,3 +157,151 @@ def test_fusion_pre_pass_keeps_the_model_function():
     k = attn.k_proj
     want = reduce.reduce_amax(k.weight.data.cpu().reshape(-1, 128), axis=[1], keepdims=True)
     assert_bits_equal(k.weight_quantizer.amax.cpu().reshape(want.shape), want, "recalibrated amax")
+
+
+# ------------------------------------------------------------------ the remaining export formats
+from oracle import mx as omx          # noqa: E402
+from oracle import qtensor as oq      # noqa: E402
+
+
+def test_w4a8_nvfp4_fp8_export(tmp_path):
+    """reference export/quant_utils.py:275-287, :308-311: the per-tensor scale is amax / 448 (the
+    consumer dequantises to FP8), the block scales and codes follow from it; :660-666."""
+    model, w = _quantized(copy.deepcopy(mtq.W4A8_NVFP4_FP8_CFG))
+    state, qcfg = export_hf_checkpoint(model, export_dir=tmp_path)
+    q = qcfg["quantization"]
+    assert q["quant_algo"] == "W4A8_NVFP4_FP8" and q["group_size"] == 32
+    assert q["exclude_modules"] == ["lm_head"]
+    name = "model.layers.1.self_attn.o_proj"
+    wsf2 = reduce.reduce_amax(w[name + ".weight"]).float() / 448.0
+    packed, wsf, _ = oq.nvfp4_quantize(w[name + ".weight"], 32, wsf2=wsf2)
+    assert_bits_equal(state[name + ".weight_scale_2"].cpu().reshape(()), wsf2.reshape(()), "weight_scale_2")
+    assert_bits_equal(state[name + ".weight_scale"].cpu(), wsf, "weight_scale")
+    assert_bits_equal(state[name + ".weight"].cpu(), packed, "packed")
+    assert state[name + ".input_scale"].dtype == torch.float32 and state[name + ".input_scale"].numel() == 1
+    # fused projections share the weight amax
+    attn = "model.layers.0.self_attn."
+    shared = torch.stack([reduce.reduce_amax(w[attn + p + ".weight"]) for p in ("q_proj", "k_proj", "v_proj")]).max()
+    packed, wsf, _ = oq.nvfp4_quantize(w[attn + "k_proj.weight"], 32, wsf2=shared.float() / 448.0)
+    assert_bits_equal(state[attn + "k_proj.weight"].cpu(), packed, "k_proj packed")
+    assert_bits_equal(state[attn + "k_proj.weight_scale"].cpu(), wsf, "k_proj weight_scale")
+
+
+@pytest.mark.parametrize("cfg_name,algo", [("MXFP4_DEFAULT_CFG", "mxfp4"),
+                                           ("W4A8_MXFP4_FP8_CFG", "W4A8_MXFP4_FP8")])
+def test_mxfp4_exports(tmp_path, cfg_name, algo):
+    """reference export/quant_utils.py:289-292, :831-832, :667-671"""
+    model, w = _quantized(copy.deepcopy(getattr(mtq, cfg_name)))
+    state, qcfg = export_hf_checkpoint(model, export_dir=tmp_path)
+    assert qcfg["quantization"]["quant_algo"] == algo
+    if algo == "W4A8_MXFP4_FP8":
+        assert qcfg["quantization"]["group_size"] == 32
+    for name in ("model.layers.0.self_attn.k_proj", "model.layers.1.mlp.down_proj"):
+        weight = w[name + ".weight"]
+        packed, scales = omx.mxfp4_quantize(weight, 32)
+        assert_bits_equal(state[name + ".weight"].cpu(), packed, name + " packed")
+        assert_bits_equal(state[name + ".weight_scale"].cpu(), scales.reshape(weight.shape[0], -1),
+                          name + " weight_scale")
+        # both configs say ``"algorithm": None``: nothing is calibrated, so the FP8 input
+        # quantizer of the W4A8 variant has no amax to export either
+        assert name + ".input_scale" not in state
+        assert name + ".weight_scale_2" not in state
+
+
+def test_fp8_block_weight_only_export(tmp_path):
+    """reference export/quant_utils.py:474-480, :776-779: 128 x 128 blocks, scale = amax / 448"""
+    model, w = _quantized(copy.deepcopy(mtq.FP8_2D_BLOCKWISE_WEIGHT_ONLY_CFG))
+    state, qcfg = export_hf_checkpoint(model, export_dir=tmp_path)
+    assert qcfg["quantization"]["quant_algo"] == "fp8_pb_wo"
+    blocks = {-1: 128, -2: 128}
+    for name in ("model.layers.0.mlp.gate_proj", "model.layers.1.mlp.down_proj",
+                 "model.layers.0.self_attn.k_proj"):
+        weight = w[name + ".weight"]          # k_proj is 64 x 128: its rows are padded to a block
+        amax = reduce.reduce_block_amax(reduce.reduce_block_padding(weight, blocks), blocks)
+        if name.endswith("k_proj"):
+            # q, k and v are one block each here, which the fusion pre-pass takes for per-tensor
+            # scales and unifies (reference export/quant_utils.py:1056-1070)
+            attn = name.rsplit(".", 1)[0]
+            amax = torch.stack([reduce.reduce_amax(w[f"{attn}.{p}.weight"])
+                                for p in ("q_proj", "k_proj", "v_proj")]).max().reshape(amax.shape)
+        codes, scales = oq.fp8_quantize(weight, (amax.float() / 448.0).squeeze(), block_sizes=blocks)
+        assert state[name + ".weight"].dtype == torch.float8_e4m3fn
+        assert_bits_equal(state[name + ".weight"].cpu().view(torch.uint8), codes.view(torch.uint8), name)
+        got = state[name + ".weight_scale"].cpu()
+        assert got.dtype == torch.float32 and got.numel() == amax.numel()
+        assert_bits_equal(got.reshape(-1), (amax.float() / 448.0).reshape(-1), name + " weight_scale")
+        assert name + ".input_scale" not in state
+
+
+def test_fp8_block_real_export(tmp_path):
+    """A model packed by ``mtq.compress`` first (reference quant_utils.py:480, unified_export_hf
+    .py:292-297): the packed weight goes out as it is, the quantizer's scales as fp32."""
+    model, w = _quantized(copy.deepcopy(mtq.FP8_2D_BLOCKWISE_WEIGHT_ONLY_CFG))
+    mtq.compress(model)
+    name = "model.layers.1.mlp.down_proj"
+    lin = model.get_submodule(name)
+    codes = lin.weight.data.clone()
+    scales = lin.weight_quantizer._scale.clone()
+    state, qcfg = export_hf_checkpoint(model, export_dir=tmp_path)
+    assert qcfg["quantization"]["quant_algo"] == "fp8_pb_real"
+    assert_bits_equal(state[name + ".weight"].cpu().view(torch.uint8), codes.cpu().view(torch.uint8), name)
+    assert state[name + ".weight_scale"].dtype == torch.float32
+    assert torch.equal(state[name + ".weight_scale"].cpu(), scales.float().cpu())
+    want, _ = oq.fp8_quantize(w[name + ".weight"], block_sizes={-1: 128, -2: 128})
+    assert_bits_equal(codes.cpu().view(torch.uint8), want.view(torch.uint8), "compressed codes")
+
+
+def test_w4a8_awq_export(tmp_path):
+    """A SequentialQuantizer (INT4 blocks, then FP8 per tensor) survives the fusion pre-pass and
+    exports as W4A8_AWQ with both scales (reference export/quant_utils.py:446-459, :265-266,
+    :313-320)."""
+    model, w = _quantized(copy.deepcopy(mtq.W4A8_AWQ_BETA_CFG))
+    name = "model.layers.1.mlp.down_proj"
+    lin = model.get_submodule(name)
+    folded = lin.weight.data.cpu().clone()
+    amax4 = lin.weight_quantizer[0].export_amax().cpu()
+    amax8 = lin.weight_quantizer[1].export_amax().cpu()
+    state, qcfg = export_hf_checkpoint(model, export_dir=tmp_path)
+    q = qcfg["quantization"]
+    assert q["quant_algo"] == "W4A8_AWQ" and q["group_size"] == 128 and q["pre_quant_scale"] is True
+    ws = amax4.float() / 7.0
+    assert_bits_equal(state[name + ".weight_scale"].cpu(), ws, "weight_scale")
+    assert_bits_equal(state[name + ".weight_scale_2"].cpu().reshape(()), (amax8.float() / 448.0).reshape(()),
+                      "weight_scale_2")
+    assert_bits_equal(state[name + ".weight"].cpu(), oexport.pack_int4_in_uint8(folded, ws), "packed int4")
+    assert name + ".pre_quant_scale" in state and name + ".input_scale" in state
+
+
+def test_nvfp4_awq_clip_real_quantization_follows_the_overflow_mode(tmp_path):
+    """awq_clip shrinks the per-tensor amax of an NVFP4 weight (reference model_calib.py:869-876),
+    so block scales can exceed E4M3's range.  The reference's cast (qtensor/nvfp4_tensor.py:84-91)
+    then stores NaN; "saturate" stores 448, and the compressed model then computes what the
+    fake-quantised one does."""
+    ids = _ids(1)[0].to(DEV)
+    for mode in ("nan", "saturate"):
+        previous = mtq.set_fp8_overflow_behavior(mode)
+        try:
+            model, w = _quantized(copy.deepcopy(mtq.NVFP4_AWQ_CLIP_CFG))
+            lin = model.get_submodule("model.layers.0.self_attn.q_proj")
+            weight = lin.weight.data.cpu().clone()
+            # whether the search clips this particular layer depends on the data: apply the
+            # smallest shrink it considers, as model_calib.py:872 does when that one wins
+            lin.weight_quantizer.amax = lin.weight_quantizer.amax * 0.5
+            amax = lin.weight_quantizer.amax.float().cpu()
+            assert float(amax) < float(reduce.reduce_amax(weight))
+            fake = model(ids).float()
+            mtq.compress(model)
+            real = model(ids).float()
+            wsf = lin.weight_quantizer._scale.cpu()
+            want_scales, _ = oq.nvfp4_block_scales(weight, 16, amax / 2688.0, keep_high_precision=True)
+            if mode == "nan":
+                want = want_scales.to(torch.float8_e4m3fn)
+                assert_bits_equal(wsf.view(torch.uint8), want.view(torch.uint8), "block scales")
+                assert bool(torch.isnan(wsf.float()).any()) == bool((want_scales > 464).any())
+            else:
+                want = want_scales.clamp(max=448.0).to(torch.float8_e4m3fn)
+                assert_bits_equal(wsf.view(torch.uint8), want.view(torch.uint8), "saturated block scales")
+                assert torch.isfinite(real).all()
+                assert float((real - fake).norm() / fake.norm()) < 1e-2
+        finally:
+            mtq.set_fp8_overflow_behavior(previous)

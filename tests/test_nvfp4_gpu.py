@@ -143,6 +143,38 @@ def test_fast_path_equals_exact_division_on_large_input():
     assert_bits_equal(p_fast[:512].cpu(), po, "packed slice")
 
 
+@pytest.mark.parametrize("dtype,block", [(torch.bfloat16, 16), (torch.bfloat16, 32),
+                                         (torch.float16, 16), (torch.float32, 8)])
+def test_block_scale_overflow_follows_the_option(dtype, block):
+    """A per-tensor amax below the real maximum (awq_clip's doing, TQ/model_calib.py:869-876)
+    pushes block scales past E4M3's range: by default the scale byte is the NaN that torch's
+    cast gives (TQ/qtensor/nvfp4_tensor.py:84-91); with MO_OPT_SATURATE_BLOCK_SCALE it is 448,
+    and the codes follow from that scale.  Single-tensor (tile and generic kernels) and
+    multi-tensor launches."""
+    x = _rand((256, 512), dtype, 77)
+    amax = reduce.reduce_amax(x).float() * 0.4
+    wsf2 = amax / 2688.0
+    raw, _ = qtensor.nvfp4_block_scales(x, block, wsf2, keep_high_precision=True)
+    assert bool((raw > 464).any()) and bool((raw < 400).any())
+    xd = x.to(DEV)
+    for saturate in (0, 1):
+        wo = (raw.clamp(max=448.0) if saturate else raw).to(torch.float8_e4m3fn)
+        po, _, _ = qtensor.nvfp4_quantize(x, block, wo, wsf2)
+        _hip.set_option(_hip.MO_OPT_SATURATE_BLOCK_SCALE, saturate)
+        try:
+            p, w, _ = _hip.nvfp4_quantize(xd, amax.to(DEV), block)
+            if dtype == torch.bfloat16 and block == 16:
+                mp, mw, _ = _hip.Nvfp4QuantizePlan([xd], amax.to(DEV).reshape(1)).run()
+        finally:
+            _hip.set_option(_hip.MO_OPT_SATURATE_BLOCK_SCALE, 0)
+        assert_bits_equal(w.cpu(), wo, f"wsf saturate={saturate}")
+        assert bool(torch.isnan(w.float()).any()) == (not saturate)
+        ok = ~torch.isnan(wo.float()).repeat_interleave(block // 2, dim=-1)   # NaN scale: codes of NaN
+        assert torch.equal(p.cpu()[ok], po[ok])
+        if dtype == torch.bfloat16 and block == 16:
+            assert torch.equal(mp[0], p) and torch.equal(mw[0].view(torch.uint8), w.view(torch.uint8))
+
+
 def test_multi_tensor_plan_matches_single_calls():
     shapes = [(256, 512), (64, 4096), (1000, 48), (3, 16)]
     xs = [_rand(s, torch.bfloat16, 20 + i).to(DEV) for i, s in enumerate(shapes)]
