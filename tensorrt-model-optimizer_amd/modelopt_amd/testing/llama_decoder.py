@@ -68,6 +68,7 @@ def _rope(x, theta):
 class LlamaAttention(nn.Module):
     def __init__(self, cfg: LlamaConfig):
         super().__init__()
+        self.config = cfg
         self.h, self.hkv = cfg.num_attention_heads, cfg.num_key_value_heads
         self.d = cfg.hidden_size // cfg.num_attention_heads
         self.theta = cfg.rope_theta

@@ -5,6 +5,7 @@ Reference: modelopt/torch/export/quant_utils.py (:68-91, :214-320, :373-534, :60
 """
 
 import fnmatch
+import warnings
 from types import SimpleNamespace
 from typing import Any
 
@@ -27,6 +28,7 @@ __all__ = [
     "get_kv_cache_dtype", "get_weight_block_size", "get_quantization_format",
     "process_layer_quant_config", "pack_int4_in_uint8", "to_quantized_weight",
     "postprocess_state_dict", "preprocess_linear_fusion", "fuse_prequant_layernorm",
+    "fuse_prequant_to_linear",
     "get_quant_config", "all_items_same",
 ]
 
@@ -378,8 +380,6 @@ def all_items_same(items):
 def _update_pre_quant_scale(module, new_pre_quant_scale):
     """Re-smooth one linear to a new input scale: ``W <- dtype(f32(W) * old / new)`` (fp32), then
     recalibrate the weight amax (reference: export/quant_utils.py:991-1008)."""
-    from ..quantization.model_calib import enable_stats_collection, finish_stats_collection
-
     old = module.input_quantizer._pre_quant_scale
     dtype, dev = module.weight.dtype, module.weight.device
     ratio_num = old.to(dtype=torch.float32, device=dev)
@@ -387,10 +387,64 @@ def _update_pre_quant_scale(module, new_pre_quant_scale):
     module.weight = nn.Parameter((module.weight.to(torch.float32) * ratio_num / ratio_den).to(dtype),
                                  requires_grad=False)
     module.input_quantizer.pre_quant_scale = new_pre_quant_scale
+    _recalibrate_weight(module)
+
+
+def _recalibrate_weight(module):
+    from ..quantization.model_calib import enable_stats_collection, finish_stats_collection
+
     module.weight_quantizer.reset_amax()
     enable_stats_collection(module.weight_quantizer)
     module.weight_quantizer(module.weight)
     finish_stats_collection(module.weight_quantizer)
+
+
+# (classes whose name contains one of these, (linear that takes the scale, linear that gives it up))
+PQS_FUSE_MODULE_MAPPING = [
+    # attn @ (x @ Wv^T) * s == attn @ (x @ (s[:, None] * Wv)^T): o_proj's input scale moves into the
+    # output rows of v_proj
+    (["LlamaAttention", "Qwen3Attention", "Qwen3MoeAttention"], ("v_proj", "o_proj")),
+    # (act(gate(x)) * up(x)) * s == act(gate(x)) * (x @ (s[:, None] * Wup)^T): down_proj's into up_proj
+    (["LlamaMLP", "Qwen3MLP", "Qwen3MoeMLP"], ("up_proj", "down_proj")),
+]
+
+
+def fuse_prequant_to_linear(model: nn.Module, fuse_grouped_heads=False):
+    """Fold the input ``pre_quant_scale`` of ``o_proj`` / ``down_proj`` into the output rows of the
+    linear that produces their input (``v_proj`` / ``up_proj``), recalibrate that linear's weight
+    amax and drop the scale (reference: export/quant_utils.py:1011-1101).
+
+    With grouped-query attention ``o_proj`` has more input channels than ``v_proj`` has rows:
+    skipped with a warning, unless ``fuse_grouped_heads``, in which case the scale is first
+    averaged over the query heads of each KV head (and ``o_proj`` re-smoothed to that average).
+    """
+    for module in model.modules():
+        for class_names, (into_name, from_name) in PQS_FUSE_MODULE_MAPPING:
+            if not any(n in type(module).__name__ for n in class_names):
+                continue
+            into, source = module.get_submodule(into_name), module.get_submodule(from_name)
+            if not hasattr(getattr(source, "input_quantizer", None), "_pre_quant_scale"):
+                continue
+            scale = source.input_quantizer._pre_quant_scale
+            rows = into.weight.shape[-2]
+            if scale.numel() != rows:
+                if not fuse_grouped_heads or "attention" not in type(module).__name__.lower():
+                    warnings.warn(f"Skipping pattern fuse prequant for {type(module).__name__}"
+                                  f"pre_quant_scale dim {scale.numel()} != out_channel dim {rows}")
+                    continue
+                kv_heads = module.config.num_key_value_heads
+                head_dim = rows // kv_heads
+                n_rep = scale.numel() // kv_heads // head_dim
+                averaged = scale.view(kv_heads, n_rep, head_dim).mean(dim=1)
+                _update_pre_quant_scale(
+                    source, averaged.unsqueeze(1).expand(kv_heads, n_rep, head_dim).reshape(-1))
+                scale = averaged.reshape(-1)
+            into.weight = nn.Parameter(into.weight * scale.view(-1, 1))
+            if getattr(into, "bias", None) is not None:
+                into.bias = nn.Parameter(into.bias * scale)
+            _recalibrate_weight(into)
+            delattr(source.input_quantizer, "_pre_quant_scale")
+            source.fused_with_prequant = True
 
 
 def preprocess_linear_fusion(modules: list[nn.Module], resmooth_only=False):

@@ -21,7 +21,8 @@ from ..quantization.qtensor import NVFP4QTensor, QTensorWrapper
 from ..quantization.utils import is_quantized_linear, true_divide
 from .model_config import *  # noqa: F403
 from ..quantization.conversion import set_quantizer_by_cfg_context
-from .quant_utils import (fuse_prequant_layernorm, get_activation_scaling_factor, get_quant_config,
+from .quant_utils import (fuse_prequant_layernorm, fuse_prequant_to_linear,
+                          get_activation_scaling_factor, get_quant_config,
                           get_quantization_format,
                           get_weight_block_size, get_weight_scaling_factor,
                           get_weight_scaling_factor_2, postprocess_state_dict,
@@ -129,6 +130,9 @@ def requantize_resmooth_fused_llm_layers(model: nn.Module):
     """
     input_to_linear: dict = {}
     output_to_layernorm: dict = {}
+    model_format = get_quantization_format(model)
+    if model_format is not None and "nvfp4_awq" in model_format.lower():
+        fuse_prequant_to_linear(model)      # o_proj's scale into v_proj, down_proj's into up_proj
 
     def linear_hook(module, args, output):
         input_to_linear.setdefault(args[0], []).append(module)

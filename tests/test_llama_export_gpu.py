@@ -305,3 +305,53 @@ def test_nvfp4_awq_clip_real_quantization_follows_the_overflow_mode(tmp_path):
                 assert float((real - fake).norm() / fake.norm()) < 1e-2
         finally:
             mtq.set_fp8_overflow_behavior(previous)
+
+
+@pytest.mark.parametrize("cfg_name", ["INT4_AWQ_CFG", "NVFP4_AWQ_LITE_CFG"])
+@pytest.mark.parametrize("heads", [(4, 4), (4, 2), (4, 1)], ids=["mha", "gqa", "mqa"])
+def test_pattern_fuse_prequant(cfg_name, heads):
+    """tests/gpu/torch/export/test_quant_utils.py:43-103: o_proj's input scale goes into v_proj's
+    rows (averaged per KV head for grouped heads), down_proj's into up_proj's; the scales and the
+    model function stay."""
+    from modelopt_amd.torch.export.quant_utils import fuse_prequant_to_linear
+
+    cfg = LlamaConfig(vocab_size=256, hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                      num_attention_heads=heads[0], num_key_value_heads=heads[1])
+    model = LlamaForCausalLM(cfg, device=DEV, seed=3)
+    ids = torch.randint(0, 256, (1, 16), generator=torch.Generator().manual_seed(0)).to(DEV)
+    mtq.quantize(model, copy.deepcopy(getattr(mtq, cfg_name)), lambda m: m(ids))
+    off = {"*": {"enable": False}}
+    with torch.no_grad():
+        before = model(ids).float()
+        with mtq.set_quantizer_by_cfg_context(model, off):
+            before_exact = model(ids).float()
+    attn = model.get_submodule("model.layers.0.self_attn")
+    mlp = model.get_submodule("model.layers.0.mlp")
+    o_scale = attn.o_proj.input_quantizer._pre_quant_scale.detach().clone()
+    d_scale = mlp.down_proj.input_quantizer._pre_quant_scale.detach().clone()
+    v_w, up_w = attn.v_proj.weight.detach().clone(), mlp.up_proj.weight.detach().clone()
+
+    fuse_prequant_to_linear(model, fuse_grouped_heads=True)
+
+    for name in ("model.layers.0.self_attn.o_proj", "model.layers.0.mlp.down_proj",
+                 "model.layers.1.self_attn.o_proj", "model.layers.1.mlp.down_proj"):
+        lin = model.get_submodule(name)
+        assert not hasattr(lin.input_quantizer, "_pre_quant_scale"), name
+        assert lin.fused_with_prequant, name
+    # the arithmetic of the fold
+    kv, hd = heads[1], 64 // heads[0]
+    want_scale = o_scale.view(kv, heads[0] // kv, hd).mean(dim=1).reshape(-1)
+    assert torch.equal(attn.v_proj.weight.detach(), v_w * want_scale.view(-1, 1))
+    assert torch.equal(mlp.up_proj.weight.detach(), up_w * d_scale.view(-1, 1))
+    # and the weight amax of the scaled linears was taken again
+    wq = mlp.up_proj.weight_quantizer
+    if wq.amax.numel() == 1:
+        assert_bits_equal(wq.amax.cpu().reshape(()), reduce.reduce_amax(mlp.up_proj.weight.detach().cpu()).reshape(()))
+    with torch.no_grad():
+        after = model(ids).float()
+        with mtq.set_quantizer_by_cfg_context(model, off):
+            after_exact = model(ids).float()
+    assert torch.allclose(before, after, rtol=1e-1, atol=5e-1)
+    # without quantization error only the rounding of the folded weights (and, for grouped
+    # heads, of o_proj re-smoothed to the averaged scale) remains
+    assert float((after_exact - before_exact).norm() / before_exact.norm()) < 0.03
