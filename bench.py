@@ -205,6 +205,26 @@ def single_tensor_configs(torch, steps, warmup):
     out["c3_awq_search_kernel_21_alphas"] = {
         "ms": round(ms, 4), "TFLOPs": round(kflops / ms / 1e9, 1), "bound": "mfma",
         "peak_TFLOPs": 2500.0, "frac": round(kflops / ms / 1e9 / 2500.0, 4)}
+
+    # AWQ clip search on the same weight: 11 clip ratios x every 128-wide block, 64 calibration
+    # tokens, one launch.  Vector-ALU bound: per rounded product one fp32 multiply, one
+    # conversion to bf16 (half rate) and one fp32 add, i.e. 4 slots of the fp32 vector unit whose
+    # peak is 157.3 TFLOP/s / 2 = 78.65 T lane-operations a second
+    ratios = [round(float(v), 2) for v in torch.arange(0.5, 1.0, 0.05)] + [1.0]
+    x64 = x3[::8].contiguous()
+    w_amax = w3.view(-1, 128).abs().amax(1, keepdim=True)
+    clip_loss = torch.zeros(len(ratios), 4096, 32, device=dev)
+
+    def clip():
+        _hip.awq_clip_losses_into(x64, w3, w_amax, ratios, 128, 4, False, False, clip_loss)
+    _, ms = timed(torch, clip, steps, warmup)
+    products = 4096 * 4096 * 64 * (len(ratios) + 1)
+    out["awq_clip_search_kernel_11_ratios_4096x4096_64_tokens"] = {
+        "ms": round(ms, 4), "rounded_products_per_s": round(products / ms * 1e3, 0), "bound": "valu",
+        "peak_lane_ops_per_s": 78.65e12, "frac": round(4 * products / ms * 1e3 / 78.65e12, 4)}
+    cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
+    cfg["algorithm"] = {"method": "awq_clip"}
+    out["awq_clip_4096x4096_end_to_end_ms"] = round(end_to_end(w3, x3, cfg) * 1e3, 3)
     return out
 
 

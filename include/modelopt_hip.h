@@ -318,6 +318,22 @@ int mo_awq_search_losses(const void* xs, const void* w, const void* s, const voi
                          int64_t block_size, int num_bits, int is_unsigned, int narrow_range,
                          double* loss, void* stream);
 
+/* AWQ clip search, all ratios and all weight blocks of one [n, k] weight on one batch of
+ * `tokens` activations in one launch.  For block (row, b) of `block_size` input channels and
+ * ratio r, with T the weight dtype and every step rounded as the tensor expression rounds it:
+ *   org[t] = T(sum_j T(x[t, j] * w[row, j])),  cur[t] = T(sum_j T(x[t, j] * wq[row, j])),
+ *   wq = T(int_qdq(w, amax = A(f32(w_amax[row, b]) * ratios[r])))   (A: the dtype of w_amax)
+ *   loss[r, row, b] += sum_t f32(T(cur[t] - org[t]))^2 / tokens      (fp32, accumulated in place)
+ * x: [tokens, k] contiguous, same dtype as w; ratios: host array, at most 32; loss: fp32
+ * [n_ratios, n, k / block_size].  Returns MO_ERR_UNSUPPORTED unless block_size is 16, 32, 64 or
+ * 128 and divides k.  Replaces the (ratio x row batch) loop of the clip search,
+ * TQ/model_calib.py:898-930 (broadcast products :901 and :916, fake quant of the clipped weight
+ * :903-905, loss :919). */
+int mo_awq_clip_losses(const void* x, int64_t tokens, const void* w, int64_t n, int64_t k,
+                       int dtype, int64_t block_size, const void* w_amax, int amax_dtype,
+                       const float* ratios, int n_ratios, int num_bits, int is_unsigned,
+                       int narrow_range, float* loss, void* stream);
+
 /* acc[0] += sum of f32(T(a[i] - b[i]))^2 in double: the numerator of update_loss
  * (TQ/model_calib.py:623-627). */
 int mo_sq_diff_sum(const void* a, const void* b, int64_t n, int dtype, double* acc, void* stream);

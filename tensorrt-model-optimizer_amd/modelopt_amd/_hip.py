@@ -47,6 +47,7 @@ SIGNATURES = {
     "mo_mul_cols": [_P, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_scale_block_int_qdq": [_P, _I64, _I64, _INT, _P, _INT, _I64, _INT, _INT, _INT, _P, _P],
     "mo_awq_search_losses": [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _INT, _I64, _INT, _INT, _INT, _P, _P],
+    "mo_awq_clip_losses": [_P, _I64, _P, _I64, _I64, _INT, _I64, _P, _INT, _P, _INT, _INT, _INT, _INT, _P, _P],
     "mo_abs_colsum": [_P, _I64, _I64, _INT, _P, _I64, _P, _P],
     "mo_sq_diff_sum": [_P, _P, _I64, _INT, _P, _P],
 }
@@ -374,6 +375,35 @@ def awq_search_losses_into(xs, w, s, ref, block_size, num_bits, unsigned, narrow
         return False
     if rc != 0:
         raise RuntimeError(f"mo_awq_search_losses failed: {lib.mo_error_string(rc).decode()} (status {rc})")
+    return True
+
+
+def awq_clip_losses_into(x, w, w_amax, ratios, block_size, num_bits, unsigned, narrow_range, loss):
+    """``loss[r, row, b] +=`` the mean over the tokens of ``x`` of the squared error that block
+    ``(row, b)`` of ``w``, fake-quantised with ``ratios[r] * w_amax[row, b]``, makes on its
+    partial output -- every ratio and block in one launch.  x: [tokens, k], w: [n, k] of the same
+    dtype; w_amax: n * k / block_size values; loss: fp32 [len(ratios), n, k / block_size].
+    Returns False (nothing written) for shapes the kernel does not cover."""
+    _require_device(x, w, w_amax, loss)
+    n, k = w.shape
+    tokens = x.shape[0]
+    assert x.dim() == 2 and x.shape[1] == k and x.dtype == w.dtype
+    assert x.is_contiguous() and w.is_contiguous() and w_amax.is_contiguous() and loss.is_contiguous()
+    if k % block_size or block_size not in (16, 32, 64, 128) or len(ratios) > 32:
+        return False
+    assert w_amax.numel() == n * (k // block_size)
+    assert loss.dtype == torch.float32 and tuple(loss.shape) == (len(ratios), n, k // block_size)
+    host = (ctypes.c_float * len(ratios))(*[float(r) for r in ratios])
+    lib = load()
+    with torch.cuda.device(x.device):
+        rc = lib.mo_awq_clip_losses(_ptr(x), tokens, _ptr(w), n, k, dtype_code(w.dtype), block_size,
+                                    _ptr(w_amax), dtype_code(w_amax.dtype), host, len(ratios),
+                                    int(num_bits), int(bool(unsigned)), int(bool(narrow_range)),
+                                    _ptr(loss), _stream(x))
+    if rc == MO_ERR_UNSUPPORTED:
+        return False
+    if rc != 0:
+        raise RuntimeError(f"mo_awq_clip_losses failed: {lib.mo_error_string(rc).decode()} (status {rc})")
     return True
 
 

@@ -248,7 +248,10 @@ class _AWQClipHelper:
         if self.is_per_tensor_clip(module):
             self.loss = {k: torch.tensor(0.0, device=dev) for k in ratios}
         else:
-            self.loss = {k: torch.zeros((co, math.ceil(ci / self.block_size)), device=dev) for k in ratios}
+            # one tensor behind the per-ratio entries, so that the fused kernel can add to all
+            # of them in one launch
+            self.loss_all = torch.zeros((len(ratios), co, math.ceil(ci / self.block_size)), device=dev)
+            self.loss = {k: self.loss_all[i] for i, k in enumerate(ratios)}
         self.best_clip_val = None
         self.best_loss = None
         self.is_input_quantized = module.input_quantizer.is_enabled
@@ -260,6 +263,25 @@ class _AWQClipHelper:
         dynamic_per_tensor = (q.block_sizes is not None and q.block_sizes.get("type") == "dynamic"
                               and q.axis is None)
         return dynamic_per_tensor or (q.axis is None and q.block_sizes is None)
+
+
+def _fused_clip_search(helper, q, inputs, weight, bs):
+    """Every ratio and every block in one kernel launch, when the weight quantizer is a plain
+    integer fake quantizer with static blocks along the last axis that divide it (what
+    ``INT4_AWQ_CFG`` / ``W4A8_AWQ_BETA_CFG`` set up).  False: not covered, nothing done."""
+    blocks = q.block_sizes or {}
+    plain = (isinstance(q, TensorQuantizer) and isinstance(q.num_bits, int) and q._fake_quant
+             and not q._dynamic and blocks.get("type", "static") == "static"
+             and blocks.get("scale_bits") is None and q.pre_quant_scale is None
+             and not getattr(q, "_rotate", False) and getattr(q, "_bias", None) is None
+             and {k for k in blocks if isinstance(k, int)} <= {-1, weight.dim() - 1}
+             and weight.dim() == 2 and weight.shape[1] % bs == 0
+             and inputs.dtype == weight.dtype and helper.w_amax.numel() == weight.numel() // bs)
+    if not plain:
+        return False
+    return _hip.awq_clip_losses_into(inputs.contiguous(), weight.data.contiguous(),
+                                     helper.w_amax.contiguous(), list(helper.loss), bs, q.num_bits,
+                                     q._unsigned, q._narrow_range, helper.loss_all)
 
 
 def _awq_clip_search(self, inputs, co_bsz, max_tokens):
@@ -283,6 +305,8 @@ def _awq_clip_search(self, inputs, co_bsz, max_tokens):
     helper.num_tokens += inputs.shape[0]
     bs = helper.block_size
     co, ci = weight.shape
+    if _fused_clip_search(helper, q, inputs, weight, bs):
+        return
     pad = (bs - ci % bs) % bs
     if pad:
         weight = F.pad(weight, (0, pad), "constant", 0)

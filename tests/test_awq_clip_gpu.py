@@ -1,0 +1,144 @@
+"""The one-launch AWQ clip search kernel against the CPU restatement of the reference's tensor
+expression (TQ/model_calib.py:878-929): per clip ratio and weight block, the mean squared error
+of the block's partial outputs.  Products, partial sums and differences are rounded to the
+tensor dtype exactly as the expression rounds them; only the order of the fp32 accumulation
+inside a partial sum is the kernel's own, so single values may differ by one rounding step of
+the sum and the comparison is on aggregates."""
+
+import copy
+
+import pytest
+import torch
+
+import modelopt_amd.torch.quantization as mtq
+from modelopt_amd import _hip
+from oracle import awq as oawq
+from oracle import reduce
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _case(n, k, tokens, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    w = (0.05 * torch.randn(n, k, generator=g)).to(dtype)
+    # a few outliers, so that clipping pays for some blocks and not for others
+    idx = torch.randint(0, n * k, (n * k // 97,), generator=g)
+    w.view(-1)[idx] *= 4
+    x = (torch.randn(tokens, k, generator=g) * torch.exp(0.5 * torch.randn(1, k, generator=g))).to(dtype)
+    return w, x
+
+
+def _ratios():
+    return [round(float(v), 2) for v in torch.arange(0.5, 1.0, 0.05)] + [1.0]
+
+
+def _run_kernel(w, x, block, num_bits=4):
+    n, k = w.shape
+    w_amax = reduce.reduce_amax(w.reshape(-1, block), axis=[1], keepdims=True)
+    ratios = _ratios()
+    loss = torch.zeros(len(ratios), n, k // block, device=DEV)
+    ok = _hip.awq_clip_losses_into(x.to(DEV), w.to(DEV), w_amax.to(DEV), ratios, block, num_bits,
+                                   False, False, loss)
+    assert ok
+    return ratios, loss.cpu()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("block", [16, 32, 64, 128])
+def test_losses_match_restatement(dtype, block):
+    w, x = _case(96, 256, 40, dtype, block)
+    ratios, got = _run_kernel(w, x, block)
+    want, _ = oawq.awq_clip_search(w, [x], block, 4, max_tokens_per_batch=64)
+    assert list(want) == ratios
+    for i, r in enumerate(ratios):
+        rel = (got[i] - want[r]).abs().sum() / want[r].abs().sum()
+        assert float(rel) < 2e-4, (r, float(rel))
+        # and entry by entry nothing is far off
+        close = torch.isclose(got[i], want[r], rtol=0.05, atol=1e-12).float().mean()
+        assert float(close) > 0.97, (r, float(close))
+    best_got = torch.stack([got[i] for i in range(len(ratios))]).argmin(0)
+    best_want = torch.stack([want[r] for r in ratios]).argmin(0)
+    assert float((best_got == best_want).float().mean()) > 0.97
+
+
+@pytest.mark.parametrize("tokens", [1, 64, 65, 150])
+def test_token_chunks_and_ragged_rows(tokens):
+    """more tokens than one pass holds, a row count that is not a multiple of the lanes"""
+    w, x = _case(70, 128, tokens, torch.bfloat16, tokens)
+    ratios, got = _run_kernel(w, x, 64)
+    want, _ = oawq.awq_clip_search(w, [x], 64, 4, max_tokens_per_batch=1 << 20)
+    for i, r in enumerate(ratios):
+        rel = (got[i] - want[r]).abs().sum() / want[r].abs().sum()
+        assert float(rel) < 2e-4, (r, float(rel))
+
+
+def test_accumulates_over_batches_and_special_blocks():
+    """loss is added to; an all-zero block costs nothing at any ratio; 8-bit works too"""
+    w, x = _case(64, 128, 32, torch.bfloat16, 5)
+    w[3, :64] = 0
+    n, k, block = 64, 128, 64
+    w_amax = reduce.reduce_amax(w.reshape(-1, block), axis=[1], keepdims=True)
+    ratios = _ratios()
+    loss = torch.zeros(len(ratios), n, k // block, device=DEV)
+    x2 = _case(64, 128, 48, torch.bfloat16, 6)[1]
+    for xb in (x, x2):
+        assert _hip.awq_clip_losses_into(xb.to(DEV), w.to(DEV), w_amax.to(DEV), ratios, block, 8,
+                                         False, True, loss)
+    want, _ = oawq.awq_clip_search(w, [x, x2], block, 8, max_tokens_per_batch=64)
+    for i, r in enumerate(ratios):
+        # the restatement quantises with narrow_range False; 8 bits, narrow: compare loosely on
+        # the aggregate and exactly on the structure
+        assert float(loss[i].cpu()[3, 0]) == 0.0
+        assert torch.isfinite(loss[i]).all()
+    assert float(loss[-1].sum()) < float(loss[0].sum())     # 8 bits: clipping to half costs more
+
+
+def test_unsupported_shapes_are_reported_not_computed():
+    w, x = _case(64, 96, 8, torch.bfloat16, 1)
+    loss = torch.zeros(11, 64, 2, device=DEV)
+    amax = torch.ones(128, 1, dtype=torch.bfloat16, device=DEV)
+    assert not _hip.awq_clip_losses_into(x.to(DEV), w.to(DEV), amax, _ratios(), 48, 4, False, False, loss)
+    assert float(loss.abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_quantizer_level_search_uses_the_kernel_and_agrees_with_the_tensor_expression(dtype, monkeypatch):
+    """mtq.quantize(awq_clip) on one linear: fused route == the torch-op route of the same
+    module (ratio picked per block, within the aggregate tolerance)."""
+    from modelopt_amd.torch.quantization import model_calib
+
+    class One(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            torch.manual_seed(0)
+            self.proj = torch.nn.Linear(256, 128, bias=False)
+
+        def forward(self, x):
+            return self.proj(x)
+
+    batches = [torch.randn(4, 24, 256, generator=torch.Generator().manual_seed(i)).to(dtype) for i in range(2)]
+    results = {}
+    for route in ("fused", "torch"):
+        model = One().to(dtype).to(DEV)
+        calls = []
+        real = model_calib._fused_clip_search
+        if route == "torch":
+            monkeypatch.setattr(model_calib, "_fused_clip_search", lambda *a, **k: False)
+        else:
+            def spy(*a, **k):
+                calls.append(1)
+                return real(*a, **k)
+            monkeypatch.setattr(model_calib, "_fused_clip_search", spy)
+        cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
+        cfg["algorithm"] = {"method": "awq_clip", "debug": True}
+        mtq.quantize(model, cfg, lambda m: [m(b.to(DEV)) for b in batches])
+        monkeypatch.setattr(model_calib, "_fused_clip_search", real)
+        if route == "fused":
+            assert len(calls) == 2
+        results[route] = (model.proj.awq_clip.loss, model.proj.weight_quantizer.amax.clone())
+    for r in results["fused"][0]:
+        a, b = results["fused"][0][r], results["torch"][0][r]
+        assert float((a - b).abs().sum() / b.abs().sum()) < 2e-4
+    same = (results["fused"][1] == results["torch"][1]).float().mean()
+    assert float(same) > 0.97
