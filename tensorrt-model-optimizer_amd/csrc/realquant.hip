@@ -281,21 +281,24 @@ __device__ __forceinline__ int int4_rne(float v) {
     return (int)f2u(t + 12582912.0f) - 0x4B400000;
 }
 
+constexpr int kInt4QuantRounds = 8;   // chunks (16-byte loads in flight) per lane
+
 template <int DT>
 __global__ __launch_bounds__(256) void int4_block_quantize_tile_kernel(
     const void* __restrict__ x, int64_t chunks, int lanes_per_block, int shift,
     void* __restrict__ scales, uint32_t* __restrict__ packed) {
-    const int64_t c0 = (int64_t)blockIdx.x * kRealTileChunks + threadIdx.x;
-    RawChunk<DT> raw[4];
+    constexpr int U = kInt4QuantRounds;
+    const int64_t c0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+    RawChunk<DT> raw[U];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < U; ++u) {
         const int64_t c = c0 + u * 256;
         zero_raw<DT>(raw[u]);
         if (c < chunks) load_raw<DT>(x, c << 3, raw[u]);
     }
-    float v[4][8];
+    float v[U][8];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < U; ++u) {
         const int64_t c = c0 + u * 256;
         unpack_raw<DT>(raw[u], v[u]);
         uint32_t m = 0;
@@ -326,15 +329,16 @@ template <int DT>
 __global__ __launch_bounds__(256) void int4_block_dequantize_tile_kernel(
     const uint32_t* __restrict__ packed, int64_t chunks, int shift,
     const void* __restrict__ scales, void* __restrict__ y) {
-    const int64_t c0 = (int64_t)blockIdx.x * kRealTileChunks + threadIdx.x;
-    uint32_t w[4];
+    constexpr int U = kInt4QuantRounds;
+    const int64_t c0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+    uint32_t w[U];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < U; ++u) {
         const int64_t c = c0 + u * 256;
         if (c < chunks) w[u] = __builtin_nontemporal_load(packed + c);
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < U; ++u) {
         const int64_t c = c0 + u * 256;
         if (c >= chunks) continue;
         const float s = load_elem<DT>(scales, c >> shift);
@@ -360,26 +364,39 @@ __global__ __launch_bounds__(256) void int4_block_dequantize_tile_kernel(
 
 // Row-pair pack with k % 8 == 0 and block_size % 8 == 0: a lane loads the same chunk of
 // columns from rows 2j and 2j + 1 and stores 8 bytes.
+constexpr int kInt4PackRounds = 4;   // items per lane (two 16-byte loads in flight each)
 template <int DT>
 __global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
     const void* __restrict__ w, int64_t pairs, int64_t kc, int64_t chunks_per_scale,
     const float* __restrict__ ws, u32x2* __restrict__ out) {
-    constexpr int R = 2;
+    constexpr int R = kInt4PackRounds;
     const int64_t total = pairs * kc;
     const int64_t t0 = (int64_t)blockIdx.x * (256 * R) + threadIdx.x;
     const int64_t nsb = kc / chunks_per_scale;
     RawChunk<DT> ra_[R], rb_[R];
     float sa[R], sb[R];
+    // (row pair, chunk) of the lane's first item by one division, of the others by stepping
+    int64_t j0, cc0;
+    if (total <= 0xFFFFFFFFll) {
+        j0 = (uint32_t)t0 / (uint32_t)kc;
+        cc0 = (uint32_t)t0 - (uint32_t)j0 * (uint32_t)kc;
+    } else {
+        j0 = t0 / kc;
+        cc0 = t0 - j0 * kc;
+    }
+    const int64_t step_j = 256 / kc, step_c = 256 - step_j * kc;   // 256 = step_j * kc + step_c
 #pragma unroll
     for (int u = 0; u < R; ++u) {
         const int64_t t = t0 + u * 256;
         zero_raw<DT>(ra_[u]);
         zero_raw<DT>(rb_[u]);
         sa[u] = sb[u] = 1.0f;
+        int64_t j = j0 + u * step_j, c = cc0 + u * step_c;
+        // c < kc + u * step_c < (u + 1) * kc: at most u wraps
+#pragma unroll
+        for (int i = 0; i < u; ++i)
+            if (c >= kc) { c -= kc; ++j; }
         if (t >= total) continue;
-        int64_t j, c;
-        if (total <= 0xFFFFFFFFll) { j = (uint32_t)t / (uint32_t)kc; c = (uint32_t)t - (uint32_t)j * (uint32_t)kc; }
-        else { j = t / kc; c = t - j * kc; }
         load_raw<DT>(w, ((2 * j) * kc + c) << 3, ra_[u]);
         load_raw<DT>(w, ((2 * j + 1) * kc + c) << 3, rb_[u]);
         const int64_t sc = (uint32_t)c / (uint32_t)chunks_per_scale;  // both below 2^32
@@ -402,23 +419,28 @@ __global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
         }
         const float ra = 1.0f / sa[u], rb = 1.0f / sb[u];
         const float big = u2f(m);
+        // fast: both scales normal and mid-range, every element finite (a NaN or inf element
+        // makes `big` NaN or inf and fails the comparisons) -- no quotient can be NaN there
         const bool fast = mid_range(sa[u]) && mid_range(sb[u]) && big * ra < 1.0e38f && big * rb < 1.0e38f;
         uint32_t lo = 0, hi = 0;
+        if (fast) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            float qa, qb;
-            if (fast) {
-                qa = exact_quotient(a[u][e], sa[u], ra);
-                qb = exact_quotient(b[u][e], sb[u], rb);
-            } else {
-                qa = a[u][e] / sa[u];
-                qb = b[u][e] / sb[u];
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t na = (uint32_t)int4_rne(exact_quotient(a[u][e], sa[u], ra)) & 0xFu;
+                const uint32_t nb = (uint32_t)int4_rne(exact_quotient(b[u][e], sb[u], rb)) & 0xFu;
+                const uint32_t byte = na | (nb << 4);
+                if (e < 4) lo |= byte << (8 * e); else hi |= byte << (8 * (e - 4));
             }
-            // a NaN quotient packs as 0 here (what the float -> int8 cast of the CPU path yields)
-            const uint32_t na = qa == qa ? (uint32_t)int4_rne(qa) & 0xFu : 0u;
-            const uint32_t nb = qb == qb ? (uint32_t)int4_rne(qb) & 0xFu : 0u;
-            const uint32_t byte = na | (nb << 4);
-            if (e < 4) lo |= byte << (8 * e); else hi |= byte << (8 * (e - 4));
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float qa = a[u][e] / sa[u], qb = b[u][e] / sb[u];
+                // a NaN quotient packs as 0 here (what the float -> int8 cast of the CPU path yields)
+                const uint32_t na = qa == qa ? (uint32_t)int4_rne(qa) & 0xFu : 0u;
+                const uint32_t nb = qb == qb ? (uint32_t)int4_rne(qb) & 0xFu : 0u;
+                const uint32_t byte = na | (nb << 4);
+                if (e < 4) lo |= byte << (8 * e); else hi |= byte << (8 * (e - 4));
+            }
         }
         const u32x2 o = {lo, hi};
         __builtin_nontemporal_store(o, out + t);
@@ -545,7 +567,8 @@ extern "C" int mo_int4_block_quantize(const void* x, int64_t n, int64_t block_si
     int shift = -1;  // block_size == 8 << shift
     for (int k = 0; k <= 6; ++k)
         if (block_size == (8ll << k)) shift = k;
-    const int64_t tiles = (n / 8 + mo::kRealTileChunks - 1) / mo::kRealTileChunks;
+    const int64_t per_tile = 256 * mo::kInt4QuantRounds;
+    const int64_t tiles = (n / 8 + per_tile - 1) / per_tile;
     if (shift >= 0 && n % block_size == 0 && (((uintptr_t)x & 15u) == 0) &&
         (((uintptr_t)packed & 3u) == 0) && tiles <= 0x7FFFFFFF) {
 #define CALL(DT)                                                                          \
@@ -571,7 +594,8 @@ extern "C" int mo_int4_block_dequantize(const uint8_t* packed, int64_t nbytes, i
     int shift = -1;
     for (int k = 0; k <= 40; ++k)
         if (block_size == (8ll << k)) shift = k;
-    const int64_t tiles = (nbytes / 4 + mo::kRealTileChunks - 1) / mo::kRealTileChunks;
+    const int64_t per_tile = 256 * mo::kInt4QuantRounds;
+    const int64_t tiles = (nbytes / 4 + per_tile - 1) / per_tile;
     if (shift >= 0 && nbytes % 4 == 0 && (((uintptr_t)y & 15u) == 0) &&
         (((uintptr_t)packed & 3u) == 0) && tiles <= 0x7FFFFFFF) {
 #define CALL(DT)                                                                          \
@@ -600,7 +624,8 @@ extern "C" int mo_int4_pack_rows(const void* w, int64_t batch, int64_t n_rows, i
     const int64_t rows = batch * n_rows;
     if (k % 8 == 0 && block_size % 8 == 0 && k < (1ll << 34) && (((uintptr_t)w & 15u) == 0) &&
         (((uintptr_t)out & 7u) == 0)) {
-        const int64_t items = (rows >> 1) * (k / 8), tiles = (items + 511) / 512;
+        const int64_t per_tile = 256 * mo::kInt4PackRounds;
+        const int64_t items = (rows >> 1) * (k / 8), tiles = (items + per_tile - 1) / per_tile;
         if (tiles <= 0x7FFFFFFF) {
 #define CALL(DT)                                                                      \
     mo::int4_pack_rows_tile_kernel<DT><<<(unsigned)tiles, 256, 0, s>>>(               \
