@@ -17,7 +17,8 @@ and the FP8 / INT8 storage casts -- that ``tests/test_oracle_c.py`` cross-checks
 against the torch restatement; it is also the timed CPU baseline of ``bench.py``.
 
 What pins each function (checked by ``tests/test_oracle_golden.py`` against the fixtures in
-``tests/golden/`` that were transcribed from the reference's own tests):
+``tests/golden/`` that were transcribed from the reference's own tests; the search oracles by
+``tests/test_oracle_search.py``, the MX formats by ``tests/test_mx_oracle.py``):
 
 =====================================  =========================================================
 function                               pinned by
@@ -42,9 +43,25 @@ export.fp8_export_cast                 PARITY UNPINNED by reference tests; pinne
                                        type-promotion rule probed in tests (bf16 / 0-dim fp32)
 nf4.nf4_quantize / double_quantization golden round trips test_qtensor_cuda.py:111-131 (with and
 / nf4_dequantize                       without padding), :30-68; per-element Python brute force
-awq.awq_lite / smoothquant             the reference's own independent oracle ``awq_lite_manual``
-                                       tests/unit/torch/quantization/test_calib.py:53-118
-                                       (restated in tests) + closed forms
+awq.awq_lite_search / awq_get_scale /  tests/test_oracle_search.py: numpy float64 formulations written from
+awq_weight_scale / awq_act_scale       the mathematics (no shared code), on the case of the reference's
+                                       own test (16-32-16-16 MLP, seed 0, one randn(2, 64, 16) batch, INT4
+                                       blocks of 8: tests/unit/torch/quantization/test_calib.py:33-52,
+                                       :170-186, which that test checks against its own independent
+                                       implementation :72-116 with allclose) + closed forms (alpha 0 / 1,
+                                       max * min = 1)
+awq.awq_clip_search                    the same case against a float64 formulation of the per-block
+                                       clip error (reference's independent implementation
+                                       test_calib.py:120-167); token subsampling and batch accumulation
+awq.smoothquant_linear                 float64 formulation + the invariant (x * s) @ (w / s)^T == x @ w^T
+mse.mse_search / candidates            known-answer cases of tests/unit/torch/quantization/
+                                       test_mse_calibrator.py:40-186, :187-232, :321-479 (outlier tensors,
+                                       accumulation, independent channels) with the whole loss curve
+                                       equal to a float64 closed form
+mx.*                                   the reference's golden tables tests/gpu/torch/quantization/
+                                       test_quantize_mxformats_cuda.py (tests/golden/mx_vectors.json),
+                                       an independent C restatement, fixed points and tie rules
+                                       (tests/test_mx_oracle.py)
 =====================================  =========================================================
 """
 
