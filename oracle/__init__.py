@@ -41,6 +41,9 @@ export.pack_int4_in_uint8              PARITY UNPINNED by reference tests (no go
                                        the unpack(pack(q)) == q invariant
 export.fp8_export_cast                 PARITY UNPINNED by reference tests; pinned by the torch
                                        type-promotion rule probed in tests (bf16 / 0-dim fp32)
+export.int8_export_cast                PARITY UNPINNED by reference tests; float64 closed form
+export.nvfp4_export                    composition of the pinned qtensor.nvfp4_* functions
+fake_quant.static_block_fake_quant     float64 closed form (tests/test_oracle_search.py)
 nf4.nf4_quantize / double_quantization golden round trips test_qtensor_cuda.py:111-131 (with and
 / nf4_dequantize                       without padding), :30-68; per-element Python brute force
 awq.awq_lite_search / awq_get_scale /  tests/test_oracle_search.py: numpy float64 formulations written from
@@ -53,7 +56,8 @@ awq_weight_scale / awq_act_scale       the mathematics (no shared code), on the 
 awq.awq_clip_search                    the same case against a float64 formulation of the per-block
                                        clip error (reference's independent implementation
                                        test_calib.py:120-167); token subsampling and batch accumulation
-awq.smoothquant_linear                 float64 formulation + the invariant (x * s) @ (w / s)^T == x @ w^T
+awq.smoothquant_linear /               float64 formulation + the invariant (x * s) @ (w / s)^T == x @ w^T
+awq.fold_pre_quant_scale
 mse.mse_search / candidates            known-answer cases of tests/unit/torch/quantization/
                                        test_mse_calibrator.py:40-186, :187-232, :321-479 (outlier tensors,
                                        accumulation, independent channels) with the whole loss curve

@@ -231,3 +231,28 @@ def test_mse_oracle_accumulates_batches_and_optimises_channels_independently():
         assert float(best[c]) == pytest.approx(float(amax0[c]) * mult[int(np.argmin(want))], rel=1e-6)
     picked = (best / amax0).reshape(-1)
     assert float(picked[2]) < 1.0 and float(picked[5]) < 1.0       # the outlier channels clip
+
+
+# ----------------------------------------------------------------------------- small helpers
+def test_fold_pre_quant_scale_keeps_the_layer_function():
+    """the folded weight with the scaled input computes what the layer computed"""
+    g = torch.Generator().manual_seed(6)
+    w, x = torch.randn(12, 20, generator=g), torch.randn(7, 20, generator=g)
+    p = torch.rand(20, generator=g) + 0.5
+    pqs, w_new = oawq.fold_pre_quant_scale(w, p)
+    assert torch.allclose(pqs, p) and torch.allclose(w_new, w / p[None, :], rtol=1e-6)
+    assert torch.allclose((x * pqs) @ w_new.T, x @ w.T, rtol=1e-4, atol=1e-5)
+
+
+def test_int8_export_cast_and_block_fake_quant_closed_forms():
+    from oracle import export as oexport
+    from oracle.fake_quant import static_block_fake_quant
+
+    g = torch.Generator().manual_seed(7)
+    w = torch.randn(10, 24, generator=g) * 3
+    s = w.abs().amax(dim=1) / 127.0
+    want = np.clip(np.rint(w.double().numpy() / s.double().numpy()[:, None]), -128, 127)
+    got = oexport.int8_export_cast(w, s).numpy()
+    assert (got != want).mean() < 0.01 and np.abs(got - want).max() <= 1   # fp32 vs float64 quotient at a tie
+    got = static_block_fake_quant(w, 8, lambda x2, amax: tensor_quant(x2, amax, 4, False, False))
+    assert np.allclose(got.numpy(), _block_qdq64(w.double().numpy(), 8), rtol=1e-5, atol=1e-6)
