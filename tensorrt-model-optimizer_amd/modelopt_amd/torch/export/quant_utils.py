@@ -277,8 +277,16 @@ def process_layer_quant_config(layer_config_dict):
 def pack_int4_in_uint8(weight, weights_scaling_factor):
     """INT4-AWQ export pack: two's-complement nibbles, adjacent output rows share a byte;
     ``[.., N, K]`` -> uint8 ``[.., N / 2, K]``."""
-    out_dim = weight.shape[-2]
+    out_dim, in_dim = weight.shape[-2], weight.shape[-1]
     assert out_dim % 2 == 0, f"Cannot pack weight. Out dimension {out_dim} is not an even number."
+    # the reference takes the block size to be in_dim // (number of scales per row) and indexes
+    # the scales with column // block_size (export/quant_utils.py:701-706): when the blocks do
+    # not tile the row (padded last block) that index runs past the last scale and it raises
+    block_size = in_dim // weights_scaling_factor.shape[-1]
+    if block_size == 0 or (in_dim - 1) // block_size >= weights_scaling_factor.shape[-1]:
+        raise IndexError(
+            f"cannot pack INT4 weight: {weights_scaling_factor.shape[-1]} scales per row do not tile "
+            f"{in_dim} input channels (the last block is padded); the reference's pack fails the same way")
     return _hip.int4_pack_rows(weight.contiguous(),
                                weights_scaling_factor.to(torch.float32).contiguous())
 

@@ -270,6 +270,27 @@ def test_int4_awq_export_pack_large_and_special(dtype):
                       export.pack_int4_in_uint8(w2, ws2), "packed rows, block 12")
 
 
+def test_int4_awq_export_pack_with_a_padded_last_block():
+    """in_features that the 128-wide blocks do not tile (reference export/quant_utils.py:701-706:
+    block size = in_dim // scales per row, scale index = column // that).  192 columns with two
+    scales per row pack with 96-wide groups, as the reference's expression does; 320 columns
+    with three scales index past the last scale there, and raise here too."""
+    from modelopt_amd.torch.export.quant_utils import pack_int4_in_uint8
+
+    g = torch.Generator().manual_seed(15)
+    w = (torch.randn((64, 192), generator=g) * 0.05).to(torch.bfloat16)
+    ws = reduce.reduce_block_amax(reduce.reduce_block_padding(w, {-1: 128}), {-1: 128}).float() / 7.0
+    assert ws.shape == (64, 2)
+    assert_bits_equal(pack_int4_in_uint8(w.to(DEV), ws.to(DEV)).cpu(), export.pack_int4_in_uint8(w, ws),
+                      "96-wide groups")
+    w = (torch.randn((64, 320), generator=g) * 0.05).to(torch.bfloat16)
+    ws = reduce.reduce_block_amax(reduce.reduce_block_padding(w, {-1: 128}), {-1: 128}).float() / 7.0
+    with pytest.raises(IndexError):
+        export.pack_int4_in_uint8(w, ws)
+    with pytest.raises(IndexError):
+        pack_int4_in_uint8(w.to(DEV), ws.to(DEV))
+
+
 # ----------------------------------------------------------------------------- AWQ helpers
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_mul_cols_both_scale_dtypes(dtype):
