@@ -142,3 +142,36 @@ def test_quantizer_level_search_uses_the_kernel_and_agrees_with_the_tensor_expre
         assert float((a - b).abs().sum() / b.abs().sum()) < 2e-4
     same = (results["fused"][1] == results["torch"][1]).float().mean()
     assert float(same) > 0.97
+
+
+def test_full_size_layer_properties():
+    """4096 x 4096 bf16, 64 tokens, 11 ratios (an 8B model's attention projection), through
+    properties that need no CPU pass: scaling the activations by a power of two scales every
+    loss by its square *exactly* (every rounding in the chain commutes with a power of two);
+    the unrounded per-block errors from a plain einsum agree on aggregate; and clipping can only
+    be chosen where it does not lose against the unclipped block."""
+    g = torch.Generator(device=DEV).manual_seed(21)
+    n = k = 4096
+    w = (0.02 * torch.randn(n, k, generator=g, device=DEV)).to(torch.bfloat16)
+    x = torch.randn(64, k, generator=g, device=DEV).to(torch.bfloat16)
+    w_amax = w.view(-1, 128).abs().amax(1, keepdim=True)
+    ratios = _ratios()
+
+    def run(acts):
+        loss = torch.zeros(len(ratios), n, k // 128, device=DEV)
+        assert _hip.awq_clip_losses_into(acts, w, w_amax, ratios, 128, 4, False, False, loss)
+        return loss
+
+    base = run(x)
+    assert torch.isfinite(base).all() and float(base.min()) >= 0.0
+    assert torch.equal(run(x * 4), base * 16)
+    assert torch.equal(run(x * 0.5), base * 0.25)
+    # ratio 1.0 against unrounded fp32 partial sums of the plain block fake quantisation
+    wq = _hip.int_qdq(w, w_amax, 1, n * (k // 128), 128, 4, False, False)
+    err = (wq.float() - w.float()).view(n, k // 128, 128)
+    part = torch.einsum("tbj,nbj->tnb", x.float().view(64, k // 128, 128), err)
+    want = part.pow(2).mean(0)
+    rel = (base[-1] - want).abs().sum() / want.sum()
+    assert float(rel) < 0.05, float(rel)       # bf16 rounding of products and partial sums
+    best = base.argmin(0)
+    assert float((best == len(ratios) - 1).float().mean()) < 0.9     # some blocks do clip
