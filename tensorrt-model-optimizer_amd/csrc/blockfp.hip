@@ -281,13 +281,32 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_kernel(const void* __restr
         const bool finite = m < 0x7F800000u;
         if (amax > 0.0f && finite) e = ceil_log2_clamped(amax / 6.0f);
         if ((threadIdx.x & ((1 << lg_g) - 1)) == 0) scales[c >> lg_g] = finite ? (uint8_t)(e + 127) : 255;
-        const float inv = __builtin_ldexpf(1.0f, -e);  // x / 2^e is exact up to over / underflow
         uint32_t w = 0;
+        // the reference divides by 2^e: identical to the product with 2^-e unless 2^-e itself
+        // overflows (e = -127).  One branch per block, so that the common case carries no division
+        if (e >= -126 && finite && DT != MO_F32) {
+            // 16-bit inputs in a finite block: the hardware E2M1 conversion (round to nearest
+            // even, sign from the sign bit) gives the code once two differences are ironed out.
+            // Ties: the rule here sends a value that sits exactly on a bound to the smaller
+            // magnitude, so the magnitude is moved one fp32 ulp towards zero first -- x / 2^e
+            // carries at most 11 significant bits, so nothing sits one fp32 ulp *above* a bound
+            // and could be dragged onto it.  Zeros: +0 and -0 both pack as code 8, i.e. -0.
+            const float inv = __builtin_ldexpf(1.0f, -e);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            // the reference divides: identical to the product unless 2^-e itself overflows
-            const float q = e >= -126 ? v[j] * inv : v[j] / __builtin_ldexpf(1.0f, e);
-            w |= mxfp4_code(q) << (4 * j);
+            for (int j = 0; j < 8; j += 2) {
+                const uint32_t a = f2u(v[j] * inv), b = f2u(v[j + 1] * inv);
+                const float na = u2f((a << 1) == 0u ? 0x80000000u : a - 1u);
+                const float nb = u2f((b << 1) == 0u ? 0x80000000u : b - 1u);
+                w = fp4_pair(w, na, nb, j >> 1);
+            }
+        } else if (e >= -126) {
+            const float inv = __builtin_ldexpf(1.0f, -e);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) w |= mxfp4_code(v[j] * inv) << (4 * j);
+        } else {
+            const float d = __builtin_ldexpf(1.0f, e);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) w |= mxfp4_code(v[j] / d) << (4 * j);
         }
         __builtin_nontemporal_store(w, packed + c);
     }

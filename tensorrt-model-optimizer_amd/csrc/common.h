@@ -294,6 +294,18 @@ __device__ __forceinline__ bool mid_range(float s) {
     return b >= 0x1F800000u && b <= 0x5F800000u;
 }
 
+// Two fp32 values -> two E2M1 codes (hardware conversion: round to nearest even, saturating,
+// sign from the sign bit) written to byte `sel` of `old`, first value in the low nibble.
+__device__ __forceinline__ uint32_t fp4_pair(uint32_t old, float a, float b, int sel) {
+    // v_cvt_scalef32_pk_fp4_f32: two fp32 -> two E2M1 codes written to byte `sel` of `old`
+    switch (sel) {
+        case 0: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, 0);
+        case 1: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, 1);
+        case 2: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, 2);
+        default: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, 3);
+    }
+}
+
 // ---------------------------------------------------------------- reductions
 
 typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));

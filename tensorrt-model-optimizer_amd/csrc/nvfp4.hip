@@ -186,15 +186,6 @@ __global__ __launch_bounds__(256) void nvfp4_qdq_kernel(const void* __restrict__
 // The hardware E2M1 conversion (round to nearest even, saturating) of q then yields the
 // reference's code; a -0.0 input is the one place where the reference's sign rule (v < 0)
 // and the hardware's (sign bit) differ, and q is +0.0 there because x - s * q0 is +0.0.
-__device__ __forceinline__ uint32_t fp4_pair(uint32_t old, float a, float b, int sel) {
-    // v_cvt_scalef32_pk_fp4_f32: two fp32 -> two E2M1 codes written to byte `sel` of `old`
-    switch (sel) {
-        case 0: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, 0);
-        case 1: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, 1);
-        case 2: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, 2);
-        default: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, 3);
-    }
-}
 
 __device__ __forceinline__ uint32_t exact_codes8(const uint32_t (&w)[4], float s) {
     uint32_t o = 0;

@@ -160,6 +160,23 @@ def test_mxfp4_pack_and_unpack_match_the_reference_qtensor(dtype, block):
     assert_bits_equal(y.cpu(), mx.mxfp4_dequantize(p_o, s_o, block, x.shape, dtype), "dequantised")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mxfp4_pack_every_16_bit_value(dtype):
+    """Every finite 16-bit pattern as an element, 31 to a block behind a pilot value that sets
+    the block scale (values above the pilot move it, which is fine): all ties on the E2M1
+    bounds, both zeros, subnormals and the largest magnitudes, at four scales."""
+    allv = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+    finite = allv[torch.isfinite(allv.float())]
+    finite = finite[: finite.numel() // 31 * 31].reshape(-1, 31)
+    for pilot in (6.0, 4.0, 0.013, 300.0):
+        col = torch.full((finite.shape[0], 1), pilot, dtype=dtype)
+        x = torch.cat([col, finite], dim=1).contiguous()
+        packed, scales = _hip.mxfp4_quantize(x.to(DEV), 32)
+        p_o, s_o = mx.mxfp4_quantize(x, 32)
+        assert torch.equal(scales.cpu(), s_o), pilot
+        assert torch.equal(packed.cpu(), p_o), (pilot, (packed.cpu() != p_o).nonzero()[:4].tolist())
+
+
 def test_mxfp4_every_code_and_scale_byte_dequantizes_like_the_reference():
     codes = torch.arange(256, dtype=torch.uint8).repeat(16).reshape(-1, 16)      # 256 blocks of 32
     scales = torch.arange(256, dtype=torch.uint8).reshape(-1, 1)
