@@ -80,38 +80,95 @@ __global__ __launch_bounds__(256) void real_dequantize_kernel(const uint8_t* __r
 // sign of a zero quotient is restored from x (s is positive on that path).
 constexpr int kRealTileChunks = 1024;
 
-__device__ __forceinline__ int64_t chunk_scale_index(int64_t c, int64_t chunks,
-                                                     int64_t inner_chunks, int64_t axis) {
-    int64_t row;
-    if (chunks <= 0xFFFFFFFFll) row = (uint32_t)c / (uint32_t)inner_chunks;
-    else row = c / inner_chunks;
-    return row < axis ? row : row % axis;
+// Scale indices of the lane's chunks c0 + 256 u (u < U): one division for the first, the others
+// by stepping (256 = step_r * inner_chunks + step_c, at most u carries).
+template <int U>
+__device__ __forceinline__ void chunk_scale_indices(int64_t c0, int64_t chunks, int64_t inner_chunks,
+                                                    int64_t axis, int64_t (&idx)[U]) {
+    int64_t row0;
+    if (chunks <= 0xFFFFFFFFll) row0 = (uint32_t)c0 / (uint32_t)inner_chunks;
+    else row0 = c0 / inner_chunks;
+    const int64_t col0 = c0 - row0 * inner_chunks;
+    const int64_t step_r = 256 / inner_chunks, step_c = 256 - step_r * inner_chunks;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        int64_t row = row0 + u * step_r, col = col0 + u * step_c;
+#pragma unroll
+        for (int i = 0; i < u; ++i)
+            if (col >= inner_chunks) { col -= inner_chunks; ++row; }
+        idx[u] = row < axis ? row : row % axis;
+    }
 }
 
-template <int DT, int VIA, int FMT, bool UNIFORM>
+// Which scale a chunk takes, three ways (SCALES):
+//   kScalePerTensor  one scale; a tile is 1024 consecutive chunks of the flat tensor
+//   kScalePerRowTile rows of at least 2048 elements: a workgroup stays inside one row (the last
+//                    tile of a row may be short), so the scale, its reciprocal and the range
+//                    checks are wavefront-uniform (scalar) as in the per-tensor case
+//   kScalePerChunk   anything else: each lane finds the rows of its chunks
+constexpr int kScalePerTensor = 0, kScalePerRowTile = 1, kScalePerChunk = 2;
+
+// chunk index, validity and scale of the lane's 4 chunks
+template <int SCALES>
+__device__ __forceinline__ void tile_layout(int64_t chunks, int64_t axis, int64_t inner_chunks,
+                                            int64_t tiles_per_row, const void* scale,
+                                            int scale_dtype, int64_t (&c)[4], bool (&ok)[4],
+                                            float (&sv)[4]) {
+    if constexpr (SCALES == kScalePerRowTile) {
+        const int64_t row = (int64_t)blockIdx.x / tiles_per_row;
+        const int64_t tile = (int64_t)blockIdx.x - row * tiles_per_row;
+        const float s0 = load_scalar(scale, scale_dtype, row < axis ? row : row % axis);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t local = tile * kRealTileChunks + threadIdx.x + u * 256;
+            ok[u] = local < inner_chunks;
+            c[u] = row * inner_chunks + local;
+            sv[u] = s0;
+        }
+    } else {
+        const int64_t c0 = (int64_t)blockIdx.x * kRealTileChunks + threadIdx.x;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            c[u] = c0 + u * 256;
+            ok[u] = c[u] < chunks;
+        }
+        if constexpr (SCALES == kScalePerTensor) {
+            sv[0] = sv[1] = sv[2] = sv[3] = load_scalar(scale, scale_dtype, 0);
+        } else {
+            int64_t idx[4];
+            chunk_scale_indices<4>(c0, chunks, inner_chunks, axis, idx);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) sv[u] = ok[u] ? load_scalar(scale, scale_dtype, idx[u]) : 1.0f;
+        }
+    }
+}
+
+template <int DT, int VIA, int FMT, int SCALES>
 __global__ __launch_bounds__(256) void real_quantize_tile_kernel(
     const void* __restrict__ x, int64_t chunks, int64_t axis, int64_t inner_chunks,
-    const void* __restrict__ scale, int scale_dtype, u32x2* __restrict__ out) {
-    const int64_t c0 = (int64_t)blockIdx.x * kRealTileChunks + threadIdx.x;
+    int64_t tiles_per_row, const void* __restrict__ scale, int scale_dtype,
+    u32x2* __restrict__ out) {
+    int64_t cs[4];
+    bool ok[4];
+    float sv[4];
+    tile_layout<SCALES>(chunks, axis, inner_chunks, tiles_per_row, scale, scale_dtype, cs, ok, sv);
     RawChunk<DT> raw[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-        const int64_t c = c0 + u * 256;
         zero_raw<DT>(raw[u]);
-        if (c < chunks) load_raw<DT>(x, c << 3, raw[u]);
+        if (ok[u]) load_raw<DT>(x, cs[u] << 3, raw[u]);
     }
-    float s0 = 1.0f;
-    if (UNIFORM) s0 = load_scalar(scale, scale_dtype, 0);
     float v[4][8];
+    float rv = 1.0f;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-        const int64_t c = c0 + u * 256;
-        if (c >= chunks) continue;
+        const int64_t c = cs[u];
+        if (!ok[u]) continue;
         unpack_raw<DT>(raw[u], v[u]);
-        const float s = UNIFORM ? s0
-                                : load_scalar(scale, scale_dtype,
-                                              chunk_scale_index(c, chunks, inner_chunks, axis));
-        const float r = 1.0f / s;
+        const float s = sv[u];
+        // the reciprocal (an IEEE division) is taken again only when the scale changes
+        if (SCALES != kScalePerChunk || u == 0 || f2u(s) != f2u(sv[u - 1])) rv = 1.0f / s;
+        const float r = rv;
         uint32_t m = 0;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -119,7 +176,8 @@ __global__ __launch_bounds__(256) void real_quantize_tile_kernel(
             m = t > m ? t : m;
         }
         float q[8];
-        if (mid_range(s) && u2f(m) * r < 1.0e38f) {  // a NaN element fails the comparison
+        const bool fast = mid_range(s) && u2f(m) * r < 1.0e38f;  // a NaN element fails the comparison
+        if (fast) {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
                 q[j] = __builtin_copysignf(exact_quotient(v[u][j], s, r), v[u][j]);
@@ -128,7 +186,17 @@ __global__ __launch_bounds__(256) void real_quantize_tile_kernel(
             for (int j = 0; j < 8; ++j) q[j] = v[u][j] / s;
         }
         uint32_t lo = 0, hi = 0;
-        if constexpr (FMT == 0) {
+        if (FMT == 1 && fast) {
+            // finite quotients: clamp with v_med3, round to nearest even by adding 1.5 * 2^23,
+            // and the low byte of the sum's mantissa is the two's-complement int8
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float a = __builtin_amdgcn_fmed3f(round_via<VIA>(q[j]), -128.0f, 127.0f);
+                const float b = __builtin_amdgcn_fmed3f(round_via<VIA>(q[4 + j]), -128.0f, 127.0f);
+                lo |= (f2u(a + 12582912.0f) & 0xFFu) << (8 * j);
+                hi |= (f2u(b + 12582912.0f) & 0xFFu) << (8 * j);
+            }
+        } else if constexpr (FMT == 0) {
             lo = f32x2_to_e4m3x2(round_via<VIA>(q[0]), round_via<VIA>(q[1])) |
                  (f32x2_to_e4m3x2(round_via<VIA>(q[2]), round_via<VIA>(q[3])) << 16);
             hi = f32x2_to_e4m3x2(round_via<VIA>(q[4]), round_via<VIA>(q[5])) |
@@ -145,27 +213,23 @@ __global__ __launch_bounds__(256) void real_quantize_tile_kernel(
     }
 }
 
-template <int DT, int FMT, bool UNIFORM>
+template <int DT, int FMT, int SCALES>
 __global__ __launch_bounds__(256) void real_dequantize_tile_kernel(
     const u32x2* __restrict__ q, int64_t chunks, int64_t axis, int64_t inner_chunks,
-    const void* __restrict__ scale, int scale_dtype, void* __restrict__ y) {
-    const int64_t c0 = (int64_t)blockIdx.x * kRealTileChunks + threadIdx.x;
+    int64_t tiles_per_row, const void* __restrict__ scale, int scale_dtype, void* __restrict__ y) {
+    int64_t cs[4];
+    bool ok[4];
+    float sv[4];
+    tile_layout<SCALES>(chunks, axis, inner_chunks, tiles_per_row, scale, scale_dtype, cs, ok, sv);
     u32x2 w[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int64_t c = c0 + u * 256;
-        if (c < chunks) w[u] = __builtin_nontemporal_load(q + c);
-    }
-    float s0 = 1.0f;
-    if (UNIFORM) s0 = round_via<DT>(load_scalar(scale, scale_dtype, 0));
+    for (int u = 0; u < 4; ++u)
+        if (ok[u]) w[u] = __builtin_nontemporal_load(q + cs[u]);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-        const int64_t c = c0 + u * 256;
-        if (c >= chunks) continue;
-        const float s = UNIFORM ? s0
-                                : round_via<DT>(load_scalar(
-                                      scale, scale_dtype,
-                                      chunk_scale_index(c, chunks, inner_chunks, axis)));
+        const int64_t c = cs[u];
+        if (!ok[u]) continue;
+        const float s = round_via<DT>(sv[u]);
         float v[8];
         // every E4M3 value and every int8 value is exact in bf16, fp16 and fp32
         if constexpr (FMT == 0) {
@@ -481,13 +545,21 @@ extern "C" int mo_real_quantize(const void* x, int64_t outer, int64_t axis, int6
     if (tiled) {
         const int64_t chunks = n / 8, ic = axis == 1 ? 1 : inner / 8;
         const unsigned gt = (unsigned)((chunks + mo::kRealTileChunks - 1) / mo::kRealTileChunks);
+        // rows of at least 2048 elements: one row per workgroup, scale math wavefront-uniform
+        const int64_t tpr = (ic + mo::kRealTileChunks - 1) / mo::kRealTileChunks;
+        const int64_t row_tiles = outer * axis * tpr;
+        const bool by_row = axis > 1 && ic >= 256 && row_tiles <= 0x7FFFFFFF;
 #define TILE4(DT, VIA, FMT)                                                                       \
     if (axis == 1)                                                                                \
-        mo::real_quantize_tile_kernel<DT, VIA, FMT, true><<<gt, 256, 0, s>>>(                     \
-            x, chunks, axis, ic, scale, scale_dtype, (mo::u32x2*)out);                            \
+        mo::real_quantize_tile_kernel<DT, VIA, FMT, mo::kScalePerTensor><<<gt, 256, 0, s>>>(      \
+            x, chunks, axis, ic, 1, scale, scale_dtype, (mo::u32x2*)out);                         \
+    else if (by_row)                                                                              \
+        mo::real_quantize_tile_kernel<DT, VIA, FMT, mo::kScalePerRowTile>                         \
+            <<<(unsigned)row_tiles, 256, 0, s>>>(x, chunks, axis, ic, tpr, scale, scale_dtype,    \
+                                                 (mo::u32x2*)out);                                \
     else                                                                                          \
-        mo::real_quantize_tile_kernel<DT, VIA, FMT, false><<<gt, 256, 0, s>>>(                    \
-            x, chunks, axis, ic, scale, scale_dtype, (mo::u32x2*)out)
+        mo::real_quantize_tile_kernel<DT, VIA, FMT, mo::kScalePerChunk><<<gt, 256, 0, s>>>(       \
+            x, chunks, axis, ic, 1, scale, scale_dtype, (mo::u32x2*)out)
 #define TILE3(DT, VIA) \
     if (format == MO_FMT_E4M3) { TILE4(DT, VIA, 0); } else { TILE4(DT, VIA, 1); }
 #define CALL(DT)                                           \
@@ -532,13 +604,20 @@ extern "C" int mo_real_dequantize(const uint8_t* q, int64_t outer, int64_t axis,
     if (tiled) {
         const int64_t chunks = n / 8, ic = axis == 1 ? 1 : inner / 8;
         const unsigned gt = (unsigned)((chunks + mo::kRealTileChunks - 1) / mo::kRealTileChunks);
+        const int64_t tpr = (ic + mo::kRealTileChunks - 1) / mo::kRealTileChunks;
+        const int64_t row_tiles = outer * axis * tpr;
+        const bool by_row = axis > 1 && ic >= 256 && row_tiles <= 0x7FFFFFFF;
 #define TILE3(DT, FMT)                                                                            \
     if (axis == 1)                                                                                \
-        mo::real_dequantize_tile_kernel<DT, FMT, true><<<gt, 256, 0, s>>>(                        \
-            (const mo::u32x2*)q, chunks, axis, ic, scale, scale_dtype, y);                        \
+        mo::real_dequantize_tile_kernel<DT, FMT, mo::kScalePerTensor><<<gt, 256, 0, s>>>(         \
+            (const mo::u32x2*)q, chunks, axis, ic, 1, scale, scale_dtype, y);                     \
+    else if (by_row)                                                                              \
+        mo::real_dequantize_tile_kernel<DT, FMT, mo::kScalePerRowTile>                            \
+            <<<(unsigned)row_tiles, 256, 0, s>>>((const mo::u32x2*)q, chunks, axis, ic, tpr,      \
+                                                 scale, scale_dtype, y);                          \
     else                                                                                          \
-        mo::real_dequantize_tile_kernel<DT, FMT, false><<<gt, 256, 0, s>>>(                       \
-            (const mo::u32x2*)q, chunks, axis, ic, scale, scale_dtype, y)
+        mo::real_dequantize_tile_kernel<DT, FMT, mo::kScalePerChunk><<<gt, 256, 0, s>>>(          \
+            (const mo::u32x2*)q, chunks, axis, ic, 1, scale, scale_dtype, y)
 #define CALL(DT) \
     if (format == MO_FMT_E4M3) { TILE3(DT, 0); } else { TILE3(DT, 1); }
         DISPATCH_DT(dtype, CALL)
