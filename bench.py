@@ -265,10 +265,23 @@ def calib_sweep(torch, layers, n_seqs, batch, seq_len=512):
     torch.cuda.synchronize()
     calib_s = time.perf_counter() - t0
     n_q = sum(1 for m in model.modules() if isinstance(m, mtq.nn.TensorQuantizer) and m.is_enabled)
-    tokens = n_seqs * seq_len
-    act_bytes = tokens * layers * (38912 * 2 + 2 * 1024 * 2)   # inputs of 7 linears + K and V
     w_bytes = sum(m.weight.numel() * 2 for m in model.modules()
                   if hasattr(m, "weight_quantizer") and m.weight_quantizer.is_enabled)
+
+    # the export of the calibrated model, in memory (the reference's export_hf_checkpoint minus the
+    # safetensors write): fusion pre-pass with its two-token forward, one quantize+pack launch for
+    # all NVFP4 linears, scale buffers, state-dict renaming
+    from modelopt_amd.torch.export.unified_export_hf import _export_hf_checkpoint
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    state, _ = _export_hf_checkpoint(model)
+    torch.cuda.synchronize()
+    export_s = time.perf_counter() - t0
+    packed_bytes = sum(v.numel() * v.element_size() for k, v in state.items()
+                       if k.endswith((".weight", ".weight_scale")) and v.dtype in (torch.uint8, torch.float8_e4m3fn))
+    del state
+    tokens = n_seqs * seq_len
+    act_bytes = tokens * layers * (38912 * 2 + 2 * 1024 * 2)   # inputs of 7 linears + K and V
     return {
         "end_to_end_calib_s": round(calib_s, 3),
         "forward_only_s": round(plain_s, 3),
@@ -276,6 +289,8 @@ def calib_sweep(torch, layers, n_seqs, batch, seq_len=512):
         "enabled_quantizers": n_q,
         "tokens": tokens,
         "amax_bytes_read": {"activations_and_kv": act_bytes, "weights_once": w_bytes},
+        "export_in_memory_s": round(export_s, 3),
+        "export_packed_bytes": packed_bytes,
         "config": f"{layers} layers, {n_seqs} seqs x {seq_len} tokens, batch {batch}, NVFP4 W+A, FP8 KV, max",
     }
 

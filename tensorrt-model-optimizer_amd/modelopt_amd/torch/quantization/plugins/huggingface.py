@@ -10,6 +10,7 @@ optional: without it the plugin does nothing.
 """
 
 import inspect
+import sys
 from functools import partial
 
 from torch import nn
@@ -59,9 +60,10 @@ class _QuantHFAttention(QuantAttentionMixin):
 
 
 def _is_hf_model(model: nn.Module) -> bool:
-    try:
-        import transformers
-    except ImportError:
+    # an instance of a transformers class can only exist if transformers is imported already;
+    # importing it here would put its start-up time into the first mtq.quantize of any model
+    transformers = sys.modules.get("transformers")
+    if transformers is None:
         return False
     return isinstance(model, transformers.PreTrainedModel)
 
