@@ -9,7 +9,10 @@ from .compress import compress, is_real_quantized
 from .config import *  # noqa: F401,F403
 from .conversion import (register, replace_quant_module, set_quantizer_attribute,
                          set_quantizer_by_cfg, set_quantizer_by_cfg_context, unregister)
-from .model_quant import (calibrate, disable_quantizer, enable_quantizer, fold_weight,
+from .model_quant import (auto_quantize, calibrate, disable_quantizer, enable_quantizer, fold_weight,
                           postprocess_amax, print_quant_summary, quantize)
+from .nn.modules.quant_module import QuantModuleRegistry
+from . import plugins
 from .plugins import attention as _attention_plugin  # noqa: F401  (registers KV quantizers)
+from .utils import update_quant_cfg_with_kv_cache_quant
 from .tensor_quant import get_fp8_overflow_behavior, set_fp8_overflow_behavior

@@ -21,7 +21,7 @@ from .nn import SequentialQuantizer, TensorQuantizer
 from .utils import all_valid_scales
 
 __all__ = ["quantize", "calibrate", "disable_quantizer", "enable_quantizer", "print_quant_summary",
-           "fold_weight", "postprocess_amax"]
+           "fold_weight", "postprocess_amax", "auto_quantize"]
 
 ForwardLoop = Callable[[nn.Module], None]
 
@@ -104,6 +104,14 @@ def disable_quantizer(model: nn.Module, wildcard_or_filter_func):
 
 def enable_quantizer(model: nn.Module, wildcard_or_filter_func):
     set_quantizer_attribute(model, wildcard_or_filter_func, {"enable": True})
+
+
+def auto_quantize(*args, **kwargs):
+    """Per-layer format search (reference: model_quant.py:236-480, algorithms.py).  Not part of
+    the path built here: it sits on the reference's searcher / mode machinery."""
+    raise NotImplementedError(
+        "auto_quantize (per-layer format search) is not part of this build; quantize with one of "
+        "the named configs or a custom quant_cfg instead")
 
 
 def print_quant_summary(model: nn.Module):

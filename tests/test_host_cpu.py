@@ -360,3 +360,20 @@ def test_mx_quantizer_control_flow(oracle_backend):
     q(x)
     assert q.amax is None
     assert mtq.MXFP8_DEFAULT_CFG["algorithm"] is None
+
+
+def test_public_names_of_the_reference_package():
+    """``modelopt.torch.quantization`` re-exports the ``__all__`` of model_quant.py:40-49,
+    conversion.py:46-53, compress.py:18 and config.py, plus ``QuantModuleRegistry``,
+    ``update_quant_cfg_with_kv_cache_quant`` and the ``plugins`` / ``utils`` modules
+    (__init__.py:19-27)."""
+    names = ["auto_quantize", "calibrate", "disable_quantizer", "enable_quantizer", "fold_weight",
+             "postprocess_amax", "print_quant_summary", "quantize", "register", "replace_quant_module",
+             "set_quantizer_attribute", "set_quantizer_by_cfg", "set_quantizer_by_cfg_context",
+             "unregister", "compress", "QuantModuleRegistry", "update_quant_cfg_with_kv_cache_quant",
+             "plugins", "utils", "QuantizeConfig", "QuantizerAttributeConfig", "CompressConfig", "choices"]
+    for name in names + sorted(mtq.config.choices):
+        assert hasattr(mtq, name), name
+    with pytest.raises(NotImplementedError):
+        mtq.auto_quantize(None)
+    assert torch.nn.Linear in mtq.QuantModuleRegistry
