@@ -57,3 +57,35 @@ def test_cpu_tensor_is_rejected():
 
     with pytest.raises(RuntimeError, match="GPU memory"):
         _hip.absmax_into(torch.zeros(8), torch.zeros(1), 1, 1, 8)
+
+
+def test_argument_checks_that_need_no_gpu():
+    """Entry points validate before they touch the device: empty work is MO_OK, bad enums, sizes
+    and null pointers come back as the documented status codes (no launch happens here)."""
+    lib = _hip.load()
+    OK, ARG, DTYPE, UNSUP = 0, -1, -2, -3
+    null = ctypes.c_void_p(0)
+    buf = (ctypes.c_float * 64)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    # abs-max / qdq: empty tensors
+    assert lib.mo_nvfp4_quantize(null, 0, 0, 2, 16, null, 0, null, null, null, null, null) == OK
+    assert lib.mo_nvfp4_quantize(p, 4, 16, 2, 12, p, 0, null, p, p, p, null) == UNSUP      # block size
+    assert lib.mo_nvfp4_quantize(null, 4, 16, 2, 16, p, 0, null, p, p, p, null) == ARG     # null input
+    assert lib.mo_nvfp4_quantize_multi(null, 0, null, 0, 2, 16, 0, null) == OK
+    assert lib.mo_nvfp4_quantize_multi(null, 1, null, 1, 2, 16, 0, null) == ARG
+    assert lib.mo_nvfp4_quantize_multi(p, 1, null, 1, 0, 16, 0, null) == UNSUP             # fp32 tensors
+    # clip search
+    ratios = (ctypes.c_float * 2)(0.5, 1.0)
+    assert lib.mo_awq_clip_losses(null, 0, null, 0, 0, 2, 128, null, 2, ratios, 2, 4, 0, 0, null, null) == OK
+    assert lib.mo_awq_clip_losses(p, 8, p, 8, 256, 7, 128, p, 2, ratios, 2, 4, 0, 0, p, null) == DTYPE
+    assert lib.mo_awq_clip_losses(p, 8, p, 8, 256, 2, 48, p, 2, ratios, 2, 4, 0, 0, p, null) == UNSUP
+    assert lib.mo_awq_clip_losses(p, 8, p, 8, 200, 2, 128, p, 2, ratios, 2, 4, 0, 0, p, null) == UNSUP  # ragged
+    assert lib.mo_awq_clip_losses(p, 8, p, 8, 256, 2, 128, p, 2, ratios, 33, 4, 0, 0, p, null) == UNSUP
+    assert lib.mo_awq_clip_losses(p, 8, p, 8, 256, 2, 128, null, 2, ratios, 2, 4, 0, 0, p, null) == ARG
+    assert lib.mo_awq_clip_losses(p, 8, p, 8, 256, 2, 128, p, 2, ratios, 2, 1, 0, 0, p, null) == ARG    # 1 bit
+    # storage casts
+    assert lib.mo_real_quantize(null, 0, 1, 0, 2, null, 2, 2, 0, null, null) == OK
+    assert lib.mo_real_quantize(p, 1, 1, 8, 2, p, 2, 2, 5, p, null) == UNSUP               # format
+    assert lib.mo_real_quantize(p, 1, 1, 8, 2, p, 9, 2, 0, p, null) == DTYPE
+    assert lib.mo_int4_pack_rows(p, 1, 3, 16, 16, 2, p, p, null) == ARG                    # odd row count
+    assert b"unsupported" in lib.mo_error_string(UNSUP).lower() or lib.mo_error_string(UNSUP)
