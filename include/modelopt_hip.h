@@ -299,6 +299,15 @@ int mo_scale_block_int_qdq(const void* x, int64_t rows, int64_t k, int dtype, co
 int mo_abs_colsum(const void* x, int64_t rows, int64_t k, int dtype, const float* blk_amax,
                   int64_t block_size, float* acc, void* stream);
 
+/* mo_abs_colsum in two passes without atomics: row slabs sum into `partial` (a caller-provided
+ * workspace of partial_rows x k floats, 16-byte aligned), then the rows of that matrix are added
+ * to acc in a fixed order -- the result does not depend on scheduling.  Returns
+ * MO_ERR_UNSUPPORTED unless k % 8 == 0, x is 16-byte aligned and, with blk_amax, block_size is a
+ * multiple of 8 that divides k.  Same reference call sites as mo_abs_colsum. */
+int mo_abs_colsum_staged(const void* x, int64_t rows, int64_t k, int dtype, const float* blk_amax,
+                         int64_t block_size, float* acc, float* partial, int64_t partial_rows,
+                         void* stream);
+
 /* AWQ-lite search step for a whole grid of alphas in one launch (bf16 only):
  *   q_a = block INT-N quantise-dequantise (blocks of block_size along k, dynamic abs-max) of
  *         bf16(w * s[a]);   out_a = bf16(xs[a] @ q_a^T)   (fp32 accumulation on the matrix cores)

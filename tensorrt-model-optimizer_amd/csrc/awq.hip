@@ -164,6 +164,104 @@ __global__ __launch_bounds__(256) void abs_colsum_kernel(const void* __restrict_
     atomicAdd(acc + c, sum);
 }
 
+// The same sums for k % 8 == 0 (and bs % 8 == 0), without atomics: a lane owns 8 adjacent columns
+// and walks down a slab of rows, four 16-byte loads in flight; the workgroup of slab blockIdx.y
+// stores its sums to row blockIdx.y of partial[slabs, k], and a second pass adds those rows to
+// acc in a fixed order.  The block abs-max of a chunk is one value, so the division becomes one
+// reciprocal per chunk and the exact FMA-corrected quotient per element.
+template <int DT, bool WITH_AMAX>
+__global__ __launch_bounds__(256) void abs_colsum8_kernel(const void* __restrict__ x, int64_t rows,
+                                                          int64_t k, const float* __restrict__ blk_amax,
+                                                          int64_t bs, int64_t slab,
+                                                          float* __restrict__ partial) {
+    const int64_t col = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (col >= k) return;
+    const int64_t r0 = (int64_t)blockIdx.y * slab;
+    int64_t r1 = r0 + slab;
+    if (r1 > rows) r1 = rows;
+    const int64_t nb = WITH_AMAX ? k / bs : 0, cb = WITH_AMAX ? col / bs : 0;
+    const float tiny = DT == MO_F16 ? 6.103515625e-05f : 1.17549435e-38f;
+    float sum[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    auto add_row = [&](const RawChunk<DT>& raw, float amax) {
+        float v[8];
+        unpack_raw<DT>(raw, v);
+        if constexpr (WITH_AMAX) {
+            const float d = round_to<DT>(amax + tiny);
+            const float r = 1.0f / d;
+            if (mid_range(d)) {     // |x| <= amax <= d: the quotient cannot overflow
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float a = __builtin_fabsf(v[j]);
+                    float q = exact_quotient(a, d, r);   // NaN stays NaN
+                    // the correction steps are exact only while nothing underflows
+                    if (q < 1.0e-30f && a > 0.0f) q = a / d;
+                    sum[j] += round_to<DT>(q);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) sum[j] += round_to<DT>(__builtin_fabsf(v[j]) / d);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) sum[j] += __builtin_fabsf(v[j]);
+        }
+    };
+    int64_t r = r0;
+    constexpr int U = DT == MO_F32 ? 4 : 8;   // rows (16- or 32-byte loads) in flight per lane
+    for (; r + U - 1 < r1; r += U) {
+        RawChunk<DT> raw[U];
+        float am[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            load_raw<DT>(x, (r + u) * k + col, raw[u]);
+            am[u] = WITH_AMAX ? blk_amax[(r + u) * nb + cb] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) add_row(raw[u], am[u]);
+    }
+    for (; r < r1; ++r) {
+        RawChunk<DT> raw;
+        load_raw<DT>(x, r * k + col, raw);
+        add_row(raw, WITH_AMAX ? blk_amax[r * nb + cb] : 0.0f);
+    }
+    f32x4* out = (f32x4*)(partial + (int64_t)blockIdx.y * k + col);
+    const f32x4 a = {sum[0], sum[1], sum[2], sum[3]}, b = {sum[4], sum[5], sum[6], sum[7]};
+    out[0] = a;
+    out[1] = b;
+}
+
+// acc[c] += sum over the rows of partial[rows, k] (k % 4 == 0).  A workgroup owns 64 columns:
+// lane = (column quad, one of 16 row groups); a group adds rows g, g + 16, ... in that order,
+// four 16-byte loads in flight, and the groups are combined through LDS in group order -- a
+// fixed order for a given shape, by one writer per column.
+__global__ __launch_bounds__(256) void colsum_fold_partials_kernel(const float* __restrict__ partial,
+                                                                   int64_t rows, int64_t k,
+                                                                   float* __restrict__ acc) {
+    __shared__ f32x4 smem[16][16];
+    const int cq = threadIdx.x & 15, g = threadIdx.x >> 4;
+    const int64_t col = ((int64_t)blockIdx.x * 16 + cq) * 4;
+    f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (col < k) {
+        int64_t r = g;
+        for (; r + 48 < rows; r += 64) {
+            f32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = *(const f32x4*)(partial + (r + 16 * u) * k + col);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) s += v[u];
+        }
+        for (; r < rows; r += 16) s += *(const f32x4*)(partial + r * k + col);
+    }
+    smem[g][cq] = s;
+    __syncthreads();
+    if (g == 0 && col < k) {
+#pragma unroll
+        for (int i = 1; i < 16; ++i) s += smem[i][cq];
+        f32x4* out = (f32x4*)(acc + col);
+        *out = *out + s;
+    }
+}
+
 // acc[0] += sum of f32( T(a[i] - b[i]) )^2.  Lanes sum 8-element chunks in fp32, the grid
 // combines in double (one atomic per workgroup).
 template <int DT>
@@ -325,5 +423,36 @@ extern "C" int mo_sq_diff_sum(const void* a, const void* b, int64_t n, int dtype
 #define CALL(DT) mo::sq_diff_sum_kernel<DT><<<g, 256, 0, st>>>(a, b, n, vec, acc)
     DISPATCH_DT(dtype, CALL)
 #undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+// mo_abs_colsum without atomics (two passes through a caller-provided workspace of
+// partial_rows x k floats); MO_ERR_UNSUPPORTED unless k % 8 == 0, block_size % 8 == 0 (when
+// blk_amax is given, which also needs block_size to divide k) and the buffers are 16-byte aligned.
+extern "C" int mo_abs_colsum_staged(const void* x, int64_t rows, int64_t k, int dtype,
+                                    const float* blk_amax, int64_t block_size, float* acc,
+                                    float* partial, int64_t partial_rows, void* stream) {
+    if (rows < 0 || k < 0 || partial_rows < 1) return MO_ERR_ARG;
+    if (dtype < MO_F32 || dtype > MO_BF16) return MO_ERR_DTYPE;
+    if (rows == 0 || k == 0) return MO_OK;
+    if (!x || !acc || !partial) return MO_ERR_ARG;
+    if (k % 8 || ((((uintptr_t)x | (uintptr_t)partial | (uintptr_t)acc) & 15u) != 0))
+        return MO_ERR_UNSUPPORTED;
+    if (blk_amax && (block_size <= 0 || block_size % 8 || k % block_size)) return MO_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    int64_t slabs = partial_rows < 65535 ? partial_rows : 65535;
+    const int64_t slab = (rows + slabs - 1) / slabs;
+    slabs = (rows + slab - 1) / slab;
+    const dim3 grid((unsigned)((k / 8 + 255) / 256), (unsigned)slabs);
+#define CALL(DT)                                                                                  \
+    if (blk_amax)                                                                                 \
+        mo::abs_colsum8_kernel<DT, true><<<grid, 256, 0, st>>>(x, rows, k, blk_amax, block_size,  \
+                                                               slab, partial);                    \
+    else                                                                                          \
+        mo::abs_colsum8_kernel<DT, false><<<grid, 256, 0, st>>>(x, rows, k, blk_amax, block_size, \
+                                                                slab, partial)
+    DISPATCH_DT(dtype, CALL)
+#undef CALL
+    mo::colsum_fold_partials_kernel<<<(unsigned)((k + 63) / 64), 256, 0, st>>>(partial, slabs, k, acc);
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

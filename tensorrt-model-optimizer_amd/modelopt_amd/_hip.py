@@ -49,6 +49,7 @@ SIGNATURES = {
     "mo_awq_search_losses": [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _INT, _I64, _INT, _INT, _INT, _P, _P],
     "mo_awq_clip_losses": [_P, _I64, _P, _I64, _I64, _INT, _I64, _P, _INT, _P, _INT, _INT, _INT, _INT, _P, _P],
     "mo_abs_colsum": [_P, _I64, _I64, _INT, _P, _I64, _P, _P],
+    "mo_abs_colsum_staged": [_P, _I64, _I64, _INT, _P, _I64, _P, _P, _I64, _P],
     "mo_sq_diff_sum": [_P, _P, _I64, _INT, _P, _P],
 }
 
@@ -433,7 +434,19 @@ def abs_colsum_into(x, acc, blk_amax=None, block_size=0):
     _require_device(x, acc, blk_amax)
     k = x.shape[-1]
     assert x.is_contiguous() and acc.dtype == torch.float32 and acc.numel() == k
-    call("mo_abs_colsum", x, _ptr(x), x.numel() // k if k else 0, k, dtype_code(x.dtype),
+    rows = x.numel() // k if k else 0
+    # below a few million elements the launch of the second pass costs more than it saves
+    big = rows * k >= ((1 << 22) if blk_amax is not None else (1 << 23))
+    if (big and k % 8 == 0 and rows >= 64 and x.data_ptr() % 16 == 0 and acc.data_ptr() % 16 == 0
+            and (blk_amax is None or (block_size > 0 and block_size % 8 == 0 and k % block_size == 0))):
+        # two passes, no atomics: enough row slabs to fill the chip, at least 16 rows each
+        across = -(-k // 2048)
+        slabs = max(1, min(-(-1024 // across), rows // 16))
+        partial = torch.empty((slabs, k), dtype=torch.float32, device=x.device)
+        call("mo_abs_colsum_staged", x, _ptr(x), rows, k, dtype_code(x.dtype), _ptr(blk_amax),
+             block_size, _ptr(acc), _ptr(partial), slabs, _stream(x))
+        return acc
+    call("mo_abs_colsum", x, _ptr(x), rows, k, dtype_code(x.dtype),
          _ptr(blk_amax), block_size, _ptr(acc), _stream(x))
     return acc
 

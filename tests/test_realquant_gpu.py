@@ -332,6 +332,64 @@ def test_awq_column_statistics_close_to_oracle():
     assert (got == want).float().mean() > 0.95
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("rows,k,block", [(1100, 4096, 128), (16384, 512, 64), (300, 4096, 128),
+                                          (64, 256, 8), (33000, 264, 0), (1000, 264, 0)])
+def test_column_sums_two_pass_kernel(dtype, rows, k, block):
+    """The vectorised two-pass path (k % 8 == 0, a few million elements and more; the smaller
+    cases here take the one-pass kernel and are held to the same figures): every term is rounded as the
+    tensor expression rounds it (|x| / T(block amax + tiny) in T), the fp32 sum of the terms is
+    compared with their float64 sum; all-zero blocks, NaN and inf included; results do not depend
+    on scheduling (no atomics) and add to what the accumulator held."""
+    g = torch.Generator().manual_seed(rows + k)
+    x = (torch.randn(rows, k, generator=g) * torch.exp(torch.randn(rows, 1, generator=g))).to(dtype)
+    if block:
+        x[5, :block] = 0                      # an all-zero block: |x| / tiny
+        x[7, block:2 * block] *= 1e-3
+    xd = x.to(DEV)
+    acc = torch.full((k,), 2.5, dtype=torch.float32, device=DEV)
+    if block:
+        blk = torch.zeros(rows * (k // block), dtype=torch.float32, device=DEV)
+        _hip.absmax_into(xd, blk, 1, rows * (k // block), block)
+        _hip.abs_colsum_into(xd, acc, blk, block)
+        tiny = torch.finfo(dtype).tiny
+        peak = x.view(rows, k // block, block).abs().amax(-1, keepdim=True)
+        terms = (x.view(rows, k // block, block).abs() / (peak + tiny)).view(rows, k)
+        assert terms.dtype == dtype
+    else:
+        _hip.abs_colsum_into(xd, acc)
+        terms = x.abs()
+    want = terms.double().sum(0) + 2.5
+    got = acc.cpu().double()
+    assert torch.allclose(got, want, rtol=3e-6, atol=0), float(((got - want).abs() / want).max())
+    again = torch.full((k,), 2.5, dtype=torch.float32, device=DEV)
+    _hip.abs_colsum_into(xd, again, blk if block else None, block)
+    two_pass = rows * k >= ((1 << 22) if block else (1 << 23))
+    if two_pass:          # fixed summation order; the one-pass kernel folds with atomics
+        assert torch.equal(again, acc)
+    else:
+        assert torch.allclose(again, acc, rtol=1e-6)
+    # NaN and inf propagate to their columns only
+    x2 = x.clone()
+    x2[3, 9] = float("nan")
+    x2[4, 17] = float("inf")
+    acc2 = torch.zeros(k, dtype=torch.float32, device=DEV)
+    if block:
+        blk2 = torch.zeros(rows * (k // block), dtype=torch.float32, device=DEV)
+        _hip.absmax_into(x2.to(DEV), blk2, 1, rows * (k // block), block)
+        _hip.abs_colsum_into(x2.to(DEV), acc2, blk2, block)
+        peak = x2.view(rows, k // block, block).abs().amax(-1, keepdim=True)
+        want2 = (x2.view(rows, k // block, block).abs() / (peak + torch.finfo(dtype).tiny)).view(rows, k).double().sum(0)
+    else:
+        _hip.abs_colsum_into(x2.to(DEV), acc2)
+        want2 = x2.abs().double().sum(0)
+    got2 = acc2.cpu().double()
+    assert torch.equal(torch.isnan(got2), torch.isnan(want2))
+    assert torch.equal(torch.isinf(got2), torch.isinf(want2))
+    ok = torch.isfinite(want2)
+    assert torch.allclose(got2[ok], want2[ok], rtol=3e-6, atol=0)
+
+
 def test_sq_diff_loss():
     a, b = _rand((256, 512), torch.bfloat16, 10, 1.0), _rand((256, 512), torch.bfloat16, 11, 1.0)
     acc = torch.zeros(1, dtype=torch.float64, device=DEV)
