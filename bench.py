@@ -265,6 +265,13 @@ def calib_sweep(torch, layers, n_seqs, batch, seq_len=512):
     torch.cuda.synchronize()
     calib_s = time.perf_counter() - t0
     n_q = sum(1 for m in model.modules() if isinstance(m, mtq.nn.TensorQuantizer) and m.is_enabled)
+    # the same data once more through the calibrated model: every forward fake-quantises the
+    # inputs and weights of all 224 linears and K / V (what evaluating a PTQ model costs)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    forward_loop(model)
+    torch.cuda.synchronize()
+    fake_s = time.perf_counter() - t0
     w_bytes = sum(m.weight.numel() * 2 for m in model.modules()
                   if hasattr(m, "weight_quantizer") and m.weight_quantizer.is_enabled)
 
@@ -289,6 +296,7 @@ def calib_sweep(torch, layers, n_seqs, batch, seq_len=512):
         "enabled_quantizers": n_q,
         "tokens": tokens,
         "amax_bytes_read": {"activations_and_kv": act_bytes, "weights_once": w_bytes},
+        "fake_quant_forward_s": round(fake_s, 3),
         "export_in_memory_s": round(export_s, 3),
         "export_packed_bytes": packed_bytes,
         "config": f"{layers} layers, {n_seqs} seqs x {seq_len} tokens, batch {batch}, NVFP4 W+A, FP8 KV, max",
