@@ -89,3 +89,24 @@ def test_argument_checks_that_need_no_gpu():
     assert lib.mo_real_quantize(p, 1, 1, 8, 2, p, 9, 2, 0, p, null) == DTYPE
     assert lib.mo_int4_pack_rows(p, 1, 3, 16, 16, 2, p, p, null) == ARG                    # odd row count
     assert b"unsupported" in lib.mo_error_string(UNSUP).lower() or lib.mo_error_string(UNSUP)
+
+
+def test_product_never_reaches_for_the_oracle_or_scratch_files():
+    """The shipped package must not import, read or run the CPU oracle (test infrastructure) or
+    anything outside itself: checked on the source text and on a fresh interpreter's modules."""
+    import subprocess
+    import sys
+
+    pkg = os.path.join(ROOT, "tensorrt-model-optimizer_amd", "modelopt_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for name in files:
+            if name.endswith(".py"):
+                text = open(os.path.join(dirpath, name)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), name
+                assert "_work" not in text and "oracle/" not in text, name
+    code = ("import sys; sys.path.insert(0, %r); sys.path.insert(0, %r);"
+            "import modelopt_amd.torch.quantization, modelopt_amd.torch.export;"
+            "bad = [m for m in sys.modules if m == 'oracle' or m.startswith('oracle.')];"
+            "print(bad); sys.exit(1 if bad else 0)") % (os.path.join(ROOT, "tensorrt-model-optimizer_amd"), ROOT)
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout + out.stderr
