@@ -414,3 +414,38 @@ def test_awq_full_runs_lite_then_clip():
     assert model.proj.input_quantizer._pre_quant_scale is not None
     assert model.proj.weight_quantizer.amax.shape == (64 * 2, 1)
     assert torch.isfinite(model(batches[0].to(DEV)).float()).all()
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(num_bits=8, axis=None),
+    dict(num_bits=8, axis=0),
+    dict(num_bits=4, block_sizes={-1: 32}),
+    dict(num_bits=(4, 3), axis=None),
+    dict(num_bits=(2, 1), block_sizes={-1: 16, "type": "dynamic", "scale_bits": (4, 3)}),
+    dict(num_bits=(2, 1), block_sizes={-1: 32, "type": "dynamic", "scale_bits": (8, 0)}),
+], ids=["int8", "int8-axis0", "int4-block", "fp8", "nvfp4", "mxfp4"])
+def test_quantizers_on_views_equal_the_contiguous_result(cfg):
+    """tests/gpu/torch/quantization/test_tensor_quantizer_cuda.py:93-107 (non-contiguous FP4
+    input), for every quantizer family: a transposed view, a strided slice and an expanded
+    tensor quantise to what their contiguous copies do, calibration included."""
+    from modelopt_amd.torch.quantization.model_calib import (enable_stats_collection,
+                                                              finish_stats_collection)
+
+    g = torch.Generator().manual_seed(4)
+    base = torch.randn(96, 128, generator=g).to(torch.bfloat16).to(DEV)
+    views = [base.t(), base[::2, 32:96], base[:1].expand(64, 128)]
+    for v in views:
+        assert not v.is_contiguous()
+        results = []
+        for x in (v, v.contiguous()):
+            q = TensorQuantizer(QuantizerAttributeConfig(**cfg)).to(DEV)
+            if not q._dynamic:
+                enable_stats_collection(q)
+                q(x)
+                finish_stats_collection(q)
+            amax = q.amax          # the MX formats and dynamic quantizers keep none
+            results.append((q(x), None if amax is None else amax.clone()))
+        assert results[0][0].shape == v.shape
+        assert_bits_equal(results[0][0].cpu(), results[1][0].cpu(), f"{tuple(v.shape)} {v.stride()}")
+        if results[0][1] is not None:
+            assert_bits_equal(results[0][1].cpu(), results[1][1].cpu(), "amax")
