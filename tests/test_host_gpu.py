@@ -449,3 +449,21 @@ def test_quantizers_on_views_equal_the_contiguous_result(cfg):
         assert_bits_equal(results[0][0].cpu(), results[1][0].cpu(), f"{tuple(v.shape)} {v.stride()}")
         if results[0][1] is not None:
             assert_bits_equal(results[0][1].cpu(), results[1][1].cpu(), "amax")
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(num_bits=8, axis=None),
+    dict(num_bits=(4, 3), axis=None),
+    dict(num_bits=(2, 1), block_sizes={-1: 16, "type": "dynamic", "scale_bits": (4, 3)}),
+], ids=["int8", "fp8", "nvfp4"])
+def test_straight_through_gradient_with_clipping(cfg):
+    """tests/gpu/torch/quantization/test_tensor_quantizer_cuda.py:76-91: with an amax below the
+    data's maximum the gradient of sum(q(x)) is 1 where |x| <= amax and 0 beyond it."""
+    q = TensorQuantizer(QuantizerAttributeConfig(**cfg)).to(DEV)
+    x = torch.rand(2, 1, 16, generator=torch.Generator().manual_seed(0)).to(DEV)
+    with torch.no_grad():
+        q.amax = torch.median(x.abs())
+    x.requires_grad = True
+    q(x).sum().backward()
+    assert torch.allclose(x.grad, torch.ones_like(x.grad) * (x.abs() <= q.amax))
+    assert 0 < float(x.grad.sum()) < x.numel()
