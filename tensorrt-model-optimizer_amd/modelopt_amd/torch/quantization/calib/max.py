@@ -43,13 +43,22 @@ class MaxCalibrator(_Calibrator):
         self._acc = None             # fp32 running max, one element per kept channel
         self._shape = None           # amax shape with the reduced dims kept as 1
         self._dtype = None
-        self._calib_amax = None      # meta-device shortcut only
+        self._meta_amax = None       # meta-device shortcut only
         self._validated = False
         self._seen_parameter = None  # identity of the last nn.Parameter folded in
 
     @property
     def amaxs(self):
         return self._amaxs
+
+    @property
+    def _calib_amax(self):
+        """The running abs-max as the reference keeps it (calib/max.py:45, :86-93): a tensor of the
+        collected dtype and amax shape, None before the first ``collect``.  Subclasses that
+        override ``compute_amax`` read it (tests/unit/torch/quantization/test_quantize_cpu.py:73-75)."""
+        if self._acc is None:
+            return self._meta_amax
+        return self._acc.to(self._dtype).reshape(self._shape)
 
     @staticmethod
     def _amax_shape(x, reduce_axis):
@@ -68,7 +77,7 @@ class MaxCalibrator(_Calibrator):
         reduce_axis = convert_quantization_axis_to_reduce_axis(x, self._axis)
         shape = self._amax_shape(x, reduce_axis)
         if x.device.type == "meta":
-            self._calib_amax = torch.empty(shape, dtype=x.dtype, device="meta")
+            self._meta_amax = torch.empty(shape, dtype=x.dtype, device="meta")
             return
         keep = [] if reduce_axis is None else [d for d in range(x.dim()) if d not in reduce_axis]
         layout = kernels.amax_layout(tuple(x.shape), keep)
@@ -92,13 +101,13 @@ class MaxCalibrator(_Calibrator):
         self._seen_parameter = None
         self._acc = None
         self._shape = None
-        self._calib_amax = None
+        self._meta_amax = None
         self._validated = False
 
     def compute_amax(self):
         """Running abs-max in the dtype of the collected tensors, or None if nothing was seen."""
         if self._acc is None:
-            return self._calib_amax
+            return self._meta_amax
         amax = self._acc.to(self._dtype).reshape(self._shape)
         if not self._validated:
             bad = torch.stack([(self._acc < 0).any(), torch.isinf(self._acc).any(),

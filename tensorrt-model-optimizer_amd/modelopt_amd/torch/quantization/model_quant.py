@@ -8,6 +8,7 @@ mode registry / state manager (``apply_mode``) is not reproduced.
 
 import copy
 import fnmatch
+import inspect
 import warnings
 from collections.abc import Callable
 
@@ -57,6 +58,14 @@ def calibrate(model: nn.Module, algorithm="max", forward_loop: ForwardLoop | Non
     method, kwargs = normalize_algorithm(algorithm)
     if method is None:
         return model
+    if forward_loop is not None and len(inspect.signature(forward_loop).parameters) == 0:
+        # the pre-model-argument calling convention (reference: model_quant.py:81-96)
+        warnings.warn("forward_loop should take model as argument, but got forward_loop without any"
+                      " arguments. This usage will be deprecated in future versions.", DeprecationWarning)
+        no_arg_loop = forward_loop
+
+        def forward_loop(model):
+            return no_arg_loop()
     training = model.training
     model.eval()
     try:
