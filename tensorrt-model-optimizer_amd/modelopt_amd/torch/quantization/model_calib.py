@@ -23,7 +23,8 @@ from .nn import QuantModule, SequentialQuantizer, TensorQuantizer
 from .utils import all_valid_scales, is_quantized_linear
 
 __all__ = ["max_calibrate", "smoothquant", "awq", "awq_lite", "enable_stats_collection",
-           "finish_stats_collection", "apply_pre_quant_scale_and_smooth"]
+           "finish_stats_collection", "apply_pre_quant_scale_and_smooth",
+           "disable_pre_quant_scale_and_resmooth", "awq_clip", "mse_calibrate"]
 
 
 # ----------------------------------------------------------------------------- max
@@ -168,6 +169,26 @@ def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.T
         device, dtype = linear.weight.device, linear.weight.dtype
         smoothing = linear.input_quantizer._amax_for_smoothing.to(device=device, dtype=dtype)
         linear.input_quantizer.amax = (smoothing * pre_quant_scale.to(device)).amax().to(dtype)
+
+
+@torch.no_grad()
+def disable_pre_quant_scale_and_resmooth(linear: nn.Module, delete_pre_quant_scale: bool = False):
+    """Undo the smoothing of one linear: multiply the weight by the input ``pre_quant_scale``
+    again, recalibrate the weight amax, switch the scale off (kept unless asked otherwise) and
+    restore the un-smoothed input amax (reference: model_calib.py:309-339)."""
+    assert is_quantized_linear(linear), "Only quantized linear modules are supported"
+    assert linear.input_quantizer._enable_pre_quant_scale, "pre_quant_scale should be enabled first!"
+    assert hasattr(linear.input_quantizer, "_pre_quant_scale"), "pre_quant_scale should be available"
+    _apply_weight_pre_quant_scale(linear, linear.input_quantizer._pre_quant_scale.to(torch.float32))
+    linear.input_quantizer._enable_pre_quant_scale = False
+    if linear.input_quantizer.amax is not None:
+        assert hasattr(linear.input_quantizer, "_amax_for_smoothing")
+        device, dtype = linear.weight.device, linear.weight.dtype
+        linear.input_quantizer.amax = linear.input_quantizer._amax_for_smoothing.amax().to(
+            device=device, dtype=dtype)
+    if delete_pre_quant_scale:
+        delattr(linear.input_quantizer, "_pre_quant_scale")
+        linear.input_quantizer._enable_pre_quant_scale = False
 
 
 def _pow(t: torch.Tensor, exponent: float) -> torch.Tensor:

@@ -125,3 +125,95 @@ def test_block_sizes_that_name_whole_axes_equal_the_axis_form():
     for (name, a), (_, b) in zip(model_ref.named_modules(), model.named_modules()):
         if getattr(a, "amax", None) is not None:
             assert torch.equal(a.amax, b.amax.reshape(a.amax.shape)), name
+
+
+# ------------------------------------------------------------------ calibration algorithms
+# tests/unit/torch/quantization/test_calib.py:280-359
+class SimpleMLP(torch.nn.Module):
+    def __init__(self, fi=16, f1=32, f2=16, fo=16):
+        super().__init__()
+        self.net = torch.nn.Sequential(torch.nn.Linear(fi, f1, bias=False), torch.nn.ReLU(),
+                                       torch.nn.Linear(f1, f2, bias=False), torch.nn.ReLU(),
+                                       torch.nn.Linear(f2, fo, bias=False))
+
+    def forward(self, x):
+        return self.net(x)
+
+
+def _awq_config(algorithm, block_size=8):
+    cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
+    cfg["quant_cfg"]["*weight_quantizer"]["block_sizes"] = {-1: block_size}
+    cfg["algorithm"] = {"method": algorithm, "debug": True}
+    if algorithm != "awq_clip":
+        cfg["algorithm"]["alpha_step"] = 0.1
+    return cfg
+
+
+def _loop(batches):
+    def run(model):
+        for b in batches:
+            model(b)
+    return run
+
+
+def test_awq_one_batch_equals_the_same_data_in_four():
+    """:280-302: the search sums over batches, so splitting the data must not change the scales"""
+    torch.manual_seed(0)
+    model = SimpleMLP().to(DEV)
+    states = model.state_dict()
+    batches = [torch.randn(2, 16, 16, device=DEV) for _ in range(4)]
+    single = [torch.cat(batches, dim=0)]
+    scales = []
+    for data in (single, batches):
+        m = SimpleMLP().to(DEV)
+        m.load_state_dict(states)
+        mtq.quantize(m, _awq_config("awq_full"), _loop(data))
+        scales.append([m.net[i].awq_lite.best_scale for i in (0, 2, 4)])
+    for a, b in zip(*scales):
+        assert torch.allclose(a, b)
+
+
+def test_awq_with_padded_blocks():
+    """:305-310: feature counts the block size does not divide"""
+    torch.manual_seed(0)
+    model = SimpleMLP(f1=13, f2=19).to(DEV)
+    mtq.quantize(model, _awq_config("awq_full"), _loop([torch.randn(2, 16, 16, device=DEV)]))
+    assert torch.isfinite(model(torch.randn(2, 16, 16, device=DEV))).all()
+
+
+def test_smoothquant_can_be_undone_and_redone():
+    """:313-344: disable_pre_quant_scale_and_resmooth gives the plain INT8 model's outputs,
+    apply_pre_quant_scale_and_smooth brings the smoothed ones back"""
+    from modelopt_amd.torch.quantization.model_calib import (apply_pre_quant_scale_and_smooth,
+                                                              disable_pre_quant_scale_and_resmooth)
+
+    torch.manual_seed(1234)
+    model = SimpleMLP().to(DEV)
+    data = [torch.randn(2, 16, 16, device=DEV)]
+    x = torch.randn(2, 16, 16, device=DEV)
+    plain = SimpleMLP().to(DEV)
+    plain.load_state_dict(model.state_dict())
+    mtq.quantize(model, mtq.INT8_SMOOTHQUANT_CFG, _loop(data))
+    mtq.quantize(plain, mtq.INT8_DEFAULT_CFG, _loop(data))
+    out_sq = model(x)
+    for module in model.modules():
+        if isinstance(module, torch.nn.Linear):
+            disable_pre_quant_scale_and_resmooth(module)
+            assert module.input_quantizer.pre_quant_scale is None
+    assert torch.allclose(model(x), plain(x))
+    for module in model.modules():
+        if isinstance(module, torch.nn.Linear):
+            apply_pre_quant_scale_and_smooth(module)
+            assert module.input_quantizer.pre_quant_scale is not None
+    assert torch.allclose(model(x), out_sq)
+
+
+def test_postprocess_amax():
+    """:347-358"""
+    torch.manual_seed(0)
+    model = SimpleMLP().to(DEV)
+    mtq.quantize(model, mtq.INT8_DEFAULT_CFG, _loop([torch.randn(2, 16, 16, device=DEV)]))
+    mtq.postprocess_amax(model, "*input_quantizer", lambda amax: torch.clamp(amax, max=0.5))
+    for name, module in model.named_modules():
+        if isinstance(module, mtq.nn.TensorQuantizer) and name.endswith("input_quantizer"):
+            assert module.amax.amax() <= 0.5
