@@ -154,7 +154,7 @@ class QuantizerAttributeConfig(_MappingConfig):
             if nb < 1:
                 raise ValueError("num_bits must be a positive integer or a tuple of positive integers.")
             return self
-        if not all(x > 0 for x in nb) and nb not in _FP_FORMATS:
+        if not all(x > 0 for x in nb):
             raise ValueError("num_bits must be a positive integer or a tuple of positive integers.")
         if nb not in _FP_FORMATS:
             raise ValueError(

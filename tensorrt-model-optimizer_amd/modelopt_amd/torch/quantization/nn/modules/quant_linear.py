@@ -7,7 +7,7 @@ from ...config import QuantizerAttributeConfig
 from ...qtensor.base_qtensor import QTensorWrapper
 from .quant_module import QuantLinearConvBase, QuantModule, QuantModuleRegistry
 
-__all__ = ["QuantLinear", "RealQuantLinear"]
+__all__ = ["Linear", "QuantLinear", "RealQuantLinear"]
 
 
 @QuantModuleRegistry.register({nn.Linear: "nn.Linear"})
@@ -23,7 +23,23 @@ class _QuantLinear(QuantLinearConvBase):
         return self.output_quantizer(output)
 
 
-QuantLinear = _QuantLinear
+class QuantLinear(_QuantLinear, nn.Linear):
+    """``nn.Linear`` that is born quantised: ``QuantLinear(in_features, out_features)`` builds the
+    linear layer and attaches its quantizers (reference: nn/modules/quant_linear.py:56-62 with
+    the constructor of nn/modules/quant_module.py:172-196).  ``quant_desc_input`` /
+    ``quant_desc_weight`` override the default quantizer configurations of this instance."""
+
+    def __init__(self, *args, quant_desc_input=None, quant_desc_weight=None, **kwargs):
+        nn.Linear.__init__(self, *args, **kwargs)
+        if quant_desc_input is not None:
+            self.default_quant_desc_input = quant_desc_input
+        if quant_desc_weight is not None:
+            self.default_quant_desc_weight = quant_desc_weight
+        self._original_cls = nn.Linear
+        self._setup()
+
+
+Linear = QuantLinear
 
 
 class RealQuantLinear(QuantModule):

@@ -75,6 +75,11 @@ def fake_quant_impl(inputs, amax, num_bits=8, unsigned=False, narrow_range=True)
 
 
 def _quantize_impl(inputs, amax, num_bits=8, exponent_bits=0, unsigned=False, narrow_range=True):
+    if inputs.dtype == torch.float64:
+        # the reference's kernels read a double and compute in float as well
+        # (src/tensor_quant_gpu.cu:43-71), so the arithmetic is the fp32 kernel's
+        return _quantize_impl(inputs.float(), amax.float(), num_bits, exponent_bits, unsigned,
+                              narrow_range).double()
     if num_bits == 8 and exponent_bits == 4:
         return scaled_e4m3_impl(inputs, amax)
     if isinstance(num_bits, int):

@@ -377,3 +377,34 @@ def test_public_names_of_the_reference_package():
     with pytest.raises(NotImplementedError):
         mtq.auto_quantize(None)
     assert torch.nn.Linear in mtq.QuantModuleRegistry
+
+
+def test_quantizer_attribute_config_validation():
+    """The constructor-time checks of the reference's config
+    (tests/unit/torch/quantization/test_tensor_quant_cpu.py:33-85): defaults, ``dict()`` round
+    trip, ``{"enable": True}`` alone is refused, bit widths must be positive."""
+    cfg = QuantizerAttributeConfig(num_bits=5)
+    assert cfg.num_bits == 5 and cfg.axis is None
+    cfg = QuantizerAttributeConfig(axis=(0, 1, 3))
+    assert cfg.num_bits == 8 and cfg.axis == (0, 1, 3)
+    for kw in ({"num_bits": 2, "fake_quant": True, "axis": (1, 2)}, {"num_bits": 2, "unsigned": True}):
+        cfg = QuantizerAttributeConfig(**kw)
+        assert cfg == QuantizerAttributeConfig(**cfg.dict())
+    with pytest.raises(ValueError, match="Invalid quantizer config: Cannot specify only {'enable': True}. "
+                                         "Additional parameters are required when enabling quantization."):
+        QuantizerAttributeConfig(enable=True)
+    for bits in (0, -1, (0, 3), (-1, 2)):
+        with pytest.raises(ValueError, match="num_bits must be a positive integer or a tuple of positive integers."):
+            QuantizerAttributeConfig(enable=True, num_bits=bits)
+
+
+def test_quant_linear_is_constructible_without_conversion():
+    """``QuantLinear(in, out)`` is an ``nn.Linear`` with its quantizers attached and the same
+    state dict keys (reference: nn/modules/quant_linear.py:56-62)."""
+    from modelopt_amd.torch.quantization.nn import QuantLinear
+    m = QuantLinear(4, 6, bias=False, quant_desc_weight=QuantizerAttributeConfig(num_bits=4, axis=0))
+    assert isinstance(m, nn.Linear) and m.bias is None and m.weight.shape == (6, 4)
+    assert m.weight_quantizer.num_bits == 4 and m.input_quantizer.num_bits == 8
+    assert not m.output_quantizer.is_enabled
+    assert list(m.state_dict()) == ["weight"]
+    assert QuantLinear(4, 6).weight_quantizer.num_bits == 8      # the override stayed on its instance
