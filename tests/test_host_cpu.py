@@ -408,3 +408,65 @@ def test_quant_linear_is_constructible_without_conversion():
     assert not m.output_quantizer.is_enabled
     assert list(m.state_dict()) == ["weight"]
     assert QuantLinear(4, 6).weight_quantizer.num_bits == 8      # the override stayed on its instance
+
+
+class _SdpaAttention(nn.Module):
+    def forward(self, qkv, extra_arg=None):
+        q, k, v = qkv
+        return F.scaled_dot_product_attention(q, k, v)
+
+
+class _MatmulAttention(nn.Module):
+    def forward(self, qkv):
+        q, k, v = qkv
+        w = torch.matmul(q, k.transpose(-1, -2)) * 0.25
+        out = torch.matmul(w.softmax(-1), v)
+        return out
+
+
+class _AtAttention(nn.Module):
+    def forward(self, qkv):
+        q, k, v = qkv
+        w = (q @ k.transpose(-1, -2)) * 0.25
+        out = w.softmax(-1) @ v
+        return out if super().__call__ is not None else None      # a zero-argument super() survives
+
+
+class _NoAttention(nn.Module):
+    def forward(self, x):
+        return x
+
+
+@pytest.mark.parametrize("cls,q_seen", [(_SdpaAttention, (1, 4, 8)), (_MatmulAttention, (1, 8, 4)),
+                                        (_AtAttention, (1, 4, 8))])
+def test_register_attention_for_kv_quant_rewrites_the_products(cls, q_seen):
+    """Three attention spellings (reference: plugins/attention.py:45-216 and
+    tests/unit/torch/quantization/test_quantize_replace.py:34-58): the converted module owns the
+    three quantizers, each sees its operand in the documented layout (the ``matmul`` form hands
+    the query over transposed), and with them disabled the output is the original's."""
+    assert mtq.plugins.register_attention_for_kv_quant(cls) is True
+    try:
+        model = nn.Sequential(cls())
+        mtq.replace_quant_module(model)
+        attn = model[0]
+        assert isinstance(attn, cls) and type(attn).__mro__[1].__name__ == "_Quant" + cls.__name__
+        seen = {}
+        for n in "qkv":
+            quantizer = getattr(attn, f"{n}_bmm_quantizer")
+            assert quantizer.is_enabled and quantizer.num_bits == 8
+            quantizer.register_forward_hook(lambda m, inp, out, n=n: seen.__setitem__(n, tuple(inp[0].shape)))
+        mtq.set_quantizer_attribute(model, "*", {"enable": False})
+        g = torch.Generator().manual_seed(0)
+        qkv = (torch.randn(1, 4, 8, generator=g), torch.randn(1, 6, 8, generator=g), torch.randn(1, 6, 8, generator=g))
+        assert torch.equal(attn(qkv), cls()(qkv))
+        assert seen == {"q": q_seen, "k": (1, 6, 8), "v": (1, 6, 8)}
+        assert "_kvq_original_class_" not in globals()
+    finally:
+        mtq.unregister(cls)
+    assert mtq.QuantModuleRegistry.get(cls) is None
+
+
+def test_register_attention_for_kv_quant_refuses_other_modules(capsys):
+    assert mtq.plugins.register_attention_for_kv_quant(_NoAttention) is False
+    assert "not attached" in capsys.readouterr().out
+    assert mtq.QuantModuleRegistry.get(_NoAttention) is None

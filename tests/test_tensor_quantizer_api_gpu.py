@@ -376,3 +376,31 @@ def test_set_quantizer_by_cfg_context_restores_everything():
     for k, v in model.state_dict().items():
         if "output_quantizer" not in k:
             assert torch.equal(v, before[k]), k
+
+
+class _SdpaAttention(torch.nn.Module):
+    def forward(self, q, k, v):
+        return F.scaled_dot_product_attention(q, k, v)
+
+
+def test_kv_cache_config_on_a_registered_attention():
+    """``register_attention_for_kv_quant`` + ``FP8_KV_CFG`` (reference: plugins/attention.py:45-216,
+    config.py FP8_KV_CFG): keys and values go through per-tensor FP8 fake quantisation with the
+    calibrated amax, the query stays as it is."""
+    import modelopt_amd.torch.quantization as mtq
+
+    assert mtq.plugins.register_attention_for_kv_quant(_SdpaAttention)
+    try:
+        model = torch.nn.Sequential()
+        model.add_module("attn", _SdpaAttention())
+        q, k, v = _randn(2, 4, 16, 32), _randn(2, 4, 16, 32, seed=1) * 3, _randn(2, 4, 16, 32, seed=2) * 0.2
+        mtq.quantize(model, mtq.FP8_KV_CFG, lambda m: m.attn(q, k, v))
+        attn = model.attn
+        assert not attn.q_bmm_quantizer.is_enabled
+        assert torch.equal(attn.k_bmm_quantizer.amax, k.abs().max())
+        assert torch.equal(attn.v_bmm_quantizer.amax, v.abs().max())
+        fq = lambda t: tensor_quant.scaled_e4m3(t, t.abs().max(), None, 4, 3)
+        assert torch.equal(attn(q, k, v), F.scaled_dot_product_attention(q, fq(k), fq(v)))
+        assert not torch.equal(attn(q, k, v), F.scaled_dot_product_attention(q, k, v))
+    finally:
+        mtq.unregister(_SdpaAttention)
