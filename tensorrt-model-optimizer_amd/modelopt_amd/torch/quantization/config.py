@@ -18,7 +18,7 @@ __all__ = [
     "MXFP6_DEFAULT_CFG", "MXFP4_DEFAULT_CFG", "MXINT8_DEFAULT_CFG", "W4A8_MXFP4_FP8_CFG",
     "NVFP4_AWQ_CLIP_CFG", "NVFP4_AWQ_FULL_CFG", "FP8_PER_CHANNEL_PER_TOKEN_CFG",
     "FP8_2D_BLOCKWISE_WEIGHT_ONLY_CFG", "W4A8_NVFP4_FP8_CFG", "MXFP4_MLP_WEIGHT_ONLY_CFG",
-    "NVFP4_MLP_WEIGHT_ONLY_CFG", "NVFP4_MLP_ONLY_CFG", "choices",
+    "NVFP4_MLP_WEIGHT_ONLY_CFG", "NVFP4_MLP_ONLY_CFG", "choices", "need_calibration",
 ]
 
 _SPECIAL_BLOCK_KEYS = ("type", "scale_bits", "scale_block_sizes")
@@ -435,3 +435,24 @@ choices = {
     "FP8_2D_BLOCKWISE_WEIGHT_ONLY_CFG", "W4A8_NVFP4_FP8_CFG", "MXFP4_MLP_WEIGHT_ONLY_CFG",
     "NVFP4_MLP_WEIGHT_ONLY_CFG", "NVFP4_MLP_ONLY_CFG", "FP8_KV_CFG", "NVFP4_KV_CFG",
 }
+
+
+def need_calibration(config) -> bool:
+    """Whether ``mtq.quantize`` needs a forward loop for ``config`` (reference: config.py:1205-1231):
+    any algorithm other than plain max does; otherwise it is needed as soon as one enabled
+    quantizer that is not a weight quantizer is static (``type`` other than ``"dynamic"`` at the top
+    level of its entry; weights are calibrated from the weights themselves)."""
+    if config["algorithm"] not in (None, "max"):
+        return True
+
+    def static_and_enabled(entry):
+        return (entry.get("enable", True) and entry.get("type", "") != "dynamic"
+                and entry.get("*", {}).get("enable", True))
+
+    for pattern, entry in config.get("quant_cfg", {}).items():
+        if "weight_quantizer" in pattern:
+            continue
+        entries = entry if isinstance(entry, list) else [entry]
+        if any(static_and_enabled(e) for e in entries):
+            return True
+    return False

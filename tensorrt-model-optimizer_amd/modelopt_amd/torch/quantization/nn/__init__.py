@@ -1,9 +1,9 @@
 """Quantised modules."""
 
-from .modules.quant_linear import QuantLinear, RealQuantLinear
+from .modules.quant_linear import Linear, QuantLinear, RealQuantLinear
 from .modules.quant_module import (QuantInputBase, QuantLinearConvBase, QuantModule,
                                    QuantModuleRegistry)
 from .modules.tensor_quantizer import SequentialQuantizer, TensorQuantizer
 
-__all__ = ["QuantLinear", "RealQuantLinear", "QuantInputBase", "QuantLinearConvBase", "QuantModule",
+__all__ = ["Linear", "QuantLinear", "RealQuantLinear", "QuantInputBase", "QuantLinearConvBase", "QuantModule",
            "QuantModuleRegistry", "SequentialQuantizer", "TensorQuantizer"]

@@ -1,6 +1,8 @@
 """Quantization utilities with the reference's names (modelopt/torch/quantization/utils.py),
 backed by the HIP abs-max kernels."""
 
+import contextlib
+
 import torch
 import torch.nn.functional as F
 
@@ -10,6 +12,7 @@ __all__ = [
     "true_divide", "convert_quantization_axis_to_reduce_axis", "reduce_amax", "reduce_block_amax",
     "reduce_block_padding", "is_quantized", "is_quantized_linear",
     "update_quant_cfg_with_kv_cache_quant", "quantizer_attr_names", "weight_attr_names",
+    "enable_fake_quant", "enable_quant", "disable_calib", "reduce_sum",
 ]
 
 
@@ -138,3 +141,46 @@ def all_valid_scales(tensors) -> bool:
         v = torch.cat(group)
         flags.append((torch.isfinite(v) & (v >= 0)).all())
     return all(bool(f) for f in flags)
+
+
+@contextlib.contextmanager
+def enable_fake_quant(module):
+    """Within the block every ``weight_quantizer`` under ``module`` fake-quantises, whatever its
+    ``fake_quant`` setting (reference: utils.py:616-630).  A bare quantizer has no
+    ``weight_quantizer`` child and is left as it is, as in the reference."""
+    held = [m.weight_quantizer for m in module.modules() if hasattr(m, "weight_quantizer")]
+    before = [q._fake_quant for q in held]
+    for q in held:
+        q._fake_quant = True
+    try:
+        yield
+    finally:
+        for q, was in zip(held, before):
+            q._fake_quant = was
+
+
+@contextlib.contextmanager
+def enable_quant(quantizer):
+    """Quantisation switched on for the block (reference: utils.py:633-646)."""
+    was, quantizer._if_quant = quantizer._if_quant, True
+    try:
+        yield
+    finally:
+        quantizer._if_quant = was
+
+
+@contextlib.contextmanager
+def disable_calib(quantizer):
+    """Statistics collection switched off for the block (reference: utils.py:649-662)."""
+    was, quantizer._if_calib = quantizer._if_calib, False
+    try:
+        yield
+    finally:
+        quantizer._if_calib = was
+
+
+def reduce_sum(input, axis=None, keepdims=True):
+    """Sum over ``axis`` (None = everything) (reference: utils.py:192-218)."""
+    if axis is None:
+        return torch.sum(input)
+    return torch.sum(input, dim=(axis,) if isinstance(axis, int) else tuple(axis), keepdim=keepdims)

@@ -470,3 +470,27 @@ def test_register_attention_for_kv_quant_refuses_other_modules(capsys):
     assert mtq.plugins.register_attention_for_kv_quant(_NoAttention) is False
     assert "not attached" in capsys.readouterr().out
     assert mtq.QuantModuleRegistry.get(_NoAttention) is None
+
+
+def test_need_calibration():
+    """tests/unit/torch/quantization/test_config_validation.py:29-35"""
+    from modelopt_amd.torch.quantization import config as C
+    assert C.need_calibration(C.FP8_DEFAULT_CFG)
+    assert not C.need_calibration(C.FP8_PER_CHANNEL_PER_TOKEN_CFG)
+    assert not C.need_calibration(C.FP8_2D_BLOCKWISE_WEIGHT_ONLY_CFG)
+    assert C.need_calibration(C.INT4_AWQ_CFG)
+    assert C.need_calibration(C.W4A8_AWQ_BETA_CFG)
+    assert C.need_calibration(C.NVFP4_DEFAULT_CFG)
+    assert not C.need_calibration(C.INT4_BLOCKWISE_WEIGHT_ONLY_CFG)
+    assert not C.need_calibration(C.MXFP4_MLP_WEIGHT_ONLY_CFG)
+
+
+def test_reprs_do_not_raise():
+    """tests/unit/torch/quantization/test_print.py:25-53 (the parts on this path)"""
+    from modelopt_amd.torch.quantization import calib, nn as qnn, tensor_quant
+    assert "num_bits" in repr(tensor_quant.QUANT_DESC_8BIT_LINEAR_WEIGHT_PER_ROW)
+    assert "TensorQuantizer" in repr(TensorQuantizer())
+    holder = nn.Module()
+    holder.linear, holder.quant_linear = nn.Linear(33, 65), qnn.Linear(33, 65)
+    assert "weight_quantizer" in repr(holder)
+    assert "MaxCalibrator" in repr(calib.MaxCalibrator(7, 1, False))

@@ -404,3 +404,81 @@ def test_kv_cache_config_on_a_registered_attention():
         assert not torch.equal(attn(q, k, v), F.scaled_dot_product_attention(q, k, v))
     finally:
         mtq.unregister(_SdpaAttention)
+
+
+# ------------------------------------------------------------------ calibrators used on their own
+def test_max_calibrator_standalone():
+    """tests/unit/torch/quantization/test_calibrator.py:28-91"""
+    import numpy as np
+
+    from modelopt_amd.torch.quantization import calib
+
+    a, b = torch.rand(16, device=DEV), torch.rand(16, device=DEV)
+    c = calib.MaxCalibrator(8, None, False, track_amax=True)
+    c.collect(a)
+    c.collect(b)
+    assert torch.equal(c.compute_amax(), torch.max(a.max(), b.max()))
+    np.testing.assert_array_equal(c.amaxs[0], a.max().cpu().numpy())
+    np.testing.assert_array_equal(c.amaxs[1], b.max().cpu().numpy())
+    c.reset()
+    assert c.compute_amax() is None
+    for axis in (0, -4):
+        c = calib.MaxCalibrator(8, axis, False)
+        a, b = torch.rand(3, 4, 2, 2, device=DEV), torch.rand(3, 4, 2, 2, device=DEV)
+        c.collect(a)
+        c.collect(b)
+        assert torch.equal(c.compute_amax(), torch.max(a, b).amax(dim=(1, 2, 3), keepdim=True))
+    with pytest.raises(RuntimeError, match="shape changed"):
+        c.collect(torch.rand(4, 4, 2, 2, device=DEV))
+
+
+def _swap_amax_quant_func(tq):
+    """the caller-side ``quant_func`` of the reference's MSE tests (test_mse_calibrator.py:51-67)"""
+    from modelopt_amd.torch.quantization.utils import disable_calib, enable_fake_quant, enable_quant
+
+    def quant_func(x, amax):
+        held = tq._amax.clone()
+        tq._amax = amax
+        with enable_quant(tq), disable_calib(tq), enable_fake_quant(tq):
+            xq = tq(x)
+        tq._amax = held
+        return xq
+    return quant_func
+
+
+def test_mse_calibrator_with_a_caller_supplied_quant_func():
+    """test_mse_calibrator.py:40-86, :233-319, :321-370: the search never ends above the bulk-only
+    loss, honours a custom error function, forgets its state on reset and keeps per-channel shape."""
+    from modelopt_amd.torch.quantization import calib
+
+    x = torch.ones(1024, device=DEV)
+    x[0] = 10.0
+    first = x.abs().max()
+    tq = TensorQuantizer(Cfg(num_bits=8, axis=None), amax=first).to(DEV)
+    cal = calib.MseCalibrator(amax=first, num_steps=20, start_multiplier=0.1, stop_multiplier=1.5,
+                              quant_func=_swap_amax_quant_func(tq))
+    cal.collect(x)
+    best = cal.compute_amax()
+    assert torch.isfinite(best) and 0 < best <= first * 1.5 + 1e-6
+    mse = lambda a: ((_ref(x, a, narrow=True) - x) ** 2).mean()
+    assert mse(best) <= mse(torch.tensor(1.0, device=DEV)) + 1e-6
+    assert torch.equal(tq.amax, first)                              # the quantizer's own amax is back
+    cal.reset()
+    assert cal.compute_amax() is None
+
+    cal = calib.MseCalibrator(amax=first, num_steps=15, start_multiplier=0.5, stop_multiplier=1.5,
+                              quant_func=_swap_amax_quant_func(tq),
+                              error_func=lambda t, tq_: (t - tq_).abs().mean())
+    cal.collect(x)
+    best = cal.compute_amax()
+    assert torch.isfinite(best) and 0 < best <= first * 1.5 + 1e-6
+
+    w = torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]], device=DEV)
+    first = torch.tensor([[3.0], [6.0]], device=DEV)
+    tq = TensorQuantizer(Cfg(num_bits=8, axis=0), amax=first).to(DEV)
+    cal = calib.MseCalibrator(amax=first, axis=0, num_steps=10, start_multiplier=0.5, stop_multiplier=2.0,
+                              quant_func=_swap_amax_quant_func(tq))
+    cal.collect(w)
+    cal.collect(w)
+    best = cal.compute_amax()
+    assert best.shape == first.shape and torch.isfinite(best).all() and (best > 0).all()
