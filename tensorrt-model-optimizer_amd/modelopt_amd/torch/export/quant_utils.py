@@ -29,7 +29,8 @@ __all__ = [
     "process_layer_quant_config", "pack_int4_in_uint8", "to_quantized_weight",
     "postprocess_state_dict", "preprocess_linear_fusion", "fuse_prequant_layernorm",
     "fuse_prequant_to_linear",
-    "get_quant_config", "all_items_same",
+    "get_quant_config", "all_items_same", "adjust_attn_amax_values", "get_kv_cache_scaling_factor",
+    "from_quantized_weight",
 ]
 
 
@@ -517,3 +518,47 @@ def get_quant_config(model: nn.Module) -> dict[str, Any]:
     if kv_format is not None:
         config["quantization"]["kv_cache_quant_algo"] = kv_format
     return config
+
+
+def adjust_attn_amax_values(module: nn.Module) -> None:
+    """Give every direct child whose name contains ``q``, ``k`` or ``v`` and whose weight quantizer
+    holds an amax the largest of those amax values, in place (reference: quant_utils.py:185-211).
+    The maximum is taken and written on the device; no scalar comes back to the host."""
+    layers = [child for name, child in module.named_children()
+              if any(p in name for p in "qkv") and hasattr(child, "weight_quantizer")
+              and getattr(child.weight_quantizer, "amax", None) is not None]
+    if not layers:
+        raise ValueError("No projection layers with the specified prefixes ('q', 'k', 'v') have amax attributes")
+    top = torch.stack([layer.weight_quantizer.amax.float().max() for layer in layers]).max()
+    assert top > 0, "max_amax must be positive."
+    for layer in layers:
+        amax = layer.weight_quantizer.amax
+        amax.copy_(top.to(amax.dtype).expand_as(amax))
+
+
+def get_kv_cache_scaling_factor(kv_module: nn.Module) -> list:
+    """``[k_scale, v_scale]`` of an attention module's BMM quantizers, ``[None, None]`` without
+    them; FP8 scales are raised to at least 1 (reference: quant_utils.py:348-370)."""
+    if not hasattr(kv_module, "k_bmm_quantizer") or not hasattr(kv_module, "v_bmm_quantizer"):
+        return [None, None]
+    factors = [get_scaling_factor(getattr(kv_module, name)) for name in ("k_bmm_quantizer", "v_bmm_quantizer")]
+    if get_kv_cache_dtype(kv_module) == KV_CACHE_FP8:
+        for i, factor in enumerate(factors):
+            if factor.item() > 0.5:
+                warnings.warn(f"Warning: Large KV activation detected: {factor.item()}, "
+                              "Quantized KV cache may lead to higher accuracy drop.")
+            factors[i] = torch.clamp(factor.float().reshape(-1)[:1], min=1.0)
+    return factors
+
+
+def from_quantized_weight(weight, weights_scaling_factor, quantization: str, torch_dtype):
+    """Back from the exported 8-bit storage to ``torch_dtype`` (reference: quant_utils.py:837-857):
+    FP8 bytes times the per-tensor scale, INT8 rows times the per-row scale; wider tensors are
+    only cast."""
+    if weight.element_size() >= 2 or weights_scaling_factor is None or not quantization:
+        return weight.to(torch_dtype)
+    if quantization == QUANTIZATION_FP8:
+        return weight.view(torch.float8_e4m3fn).to(torch_dtype) * weights_scaling_factor.to(torch_dtype)
+    if quantization in (QUANTIZATION_INT8_SQ, QUANTIZATION_INT8_WO):
+        return weight.to(torch_dtype) * weights_scaling_factor[:, None].to(torch_dtype)
+    raise NotImplementedError(f"quantization format {quantization} not supported")
