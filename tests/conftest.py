@@ -50,3 +50,25 @@ def assert_bits_equal(actual: torch.Tensor, expected: torch.Tensor, what: str = 
         raise AssertionError(
             f"{what}: {bad.shape[0]} of {ok.numel()} elements differ; first at {first}: "
             f"got {a[first].item()!r} expected {e[first].item()!r}")
+
+
+def load_export_vectors():
+    """tests/golden/export_vectors.json (outputs of the reference's export casts) as tensors."""
+    import json
+
+    bits = {"bfloat16": torch.int16, "float16": torch.int16, "float32": torch.int32,
+            "uint8": torch.uint8, "int8": torch.uint8, "float8_e4m3fn": torch.uint8}
+    with open(os.path.join(GOLDEN, "export_vectors.json")) as f:
+        raw = json.load(f)["cases"]
+    cases = []
+    for c in raw:
+        wd, od = getattr(torch, c["weight_dtype"]), getattr(torch, c["out_dtype"])
+        cases.append({
+            "name": c["name"], "format": c["format"],
+            "weight": torch.tensor(c["weight_bits"], dtype=bits[c["weight_dtype"]]).view(wd)
+            .reshape(c["weight_shape"]),
+            "scale": torch.tensor(c["scale_bits"], dtype=torch.int32).view(torch.float32)
+            .reshape(c["scale_shape"]),
+            "out": torch.tensor(c["out_bits"], dtype=torch.uint8).view(od).reshape(c["out_shape"]),
+        })
+    return cases

@@ -74,3 +74,25 @@ def test_get_kv_cache_scaling_factor():
     with pytest.warns(UserWarning, match="Large KV activation"):
         k_scale, v_scale = Q.get_kv_cache_scaling_factor(attn)
     assert k_scale.tolist() == [2.0] and v_scale.tolist() == [1.0]
+
+
+def _export_cases():
+    from conftest import load_export_vectors
+
+    return load_export_vectors()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", _export_cases(), ids=lambda c: c["name"])
+def test_to_quantized_weight_matches_reference_outputs(case):
+    """The recorded outputs of the reference's to_quantized_weight / pack_int4_in_uint8
+    (export/quant_utils.py:697-774, tests/golden/export_vectors.json) through the kernels."""
+    from conftest import assert_bits_equal
+    from modelopt_amd.torch.export import quant_utils as Q
+
+    w, s = case["weight"].to("cuda:0"), case["scale"].to("cuda:0")
+    got = Q.to_quantized_weight(w, s, case["format"])
+    want = case["out"]
+    if want.dtype == torch.float8_e4m3fn:
+        got = got.view(torch.float8_e4m3fn)
+    assert_bits_equal(got.cpu(), want, case["name"])

@@ -247,3 +247,29 @@ def test_llama3_8b_weight_shapes_against_c_restatement(shape):
     assert torch.equal(packed.cpu(), p_c)
     y_c = cref.nvfp4_dequantize(p_c, w_c, w2_c, 16, torch.bfloat16)
     assert torch.equal(y.cpu().view(torch.int16), y_c.view(torch.int16))
+
+
+LLAMA3_8B_LAYER = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
+                   ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]
+
+
+def test_two_full_llama3_8b_layers_through_the_multi_tensor_launches():
+    """Two complete Llama-3-8B decoder layers (14 weights, all seven shapes) through the
+    multi-tensor abs-max and quantize+pack launches that the benchmark times: per-tensor amax,
+    global scale, every block scale and every packed code bit for bit against the C restatement."""
+    from oracle import cref
+
+    g = torch.Generator(device=DEV).manual_seed(2024)
+    xs = [(torch.randn((n, k), generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+          for _layer in range(2) for _name, n, k in LLAMA3_8B_LAYER]
+    acc = _hip.AbsmaxPlan(xs).run().clone()
+    packed, wsf, wsf2 = _hip.Nvfp4QuantizePlan(xs, acc).run()
+    torch.cuda.synchronize()
+    for i, xd in enumerate(xs):
+        x = xd.cpu()
+        what = f"tensor {i} {tuple(x.shape)}"
+        assert float(acc[i]) == cref.absmax(x), what
+        p_c, w_c, w2_c = cref.nvfp4_quantize(x, 16)
+        assert float(wsf2[i]) == float(w2_c), what
+        assert torch.equal(wsf[i].cpu().view(torch.uint8), w_c.view(torch.uint8)), what
+        assert torch.equal(packed[i].cpu(), p_c), what

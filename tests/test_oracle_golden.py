@@ -6,7 +6,7 @@ import os
 import pytest
 import torch
 
-from conftest import GOLDEN, assert_bits_equal
+from conftest import GOLDEN, assert_bits_equal, load_export_vectors
 from oracle import export, fake_quant, nf4, qtensor, reduce
 
 with open(os.path.join(GOLDEN, "reference_vectors.json")) as f:
@@ -233,8 +233,8 @@ def test_scaling_factor_from_weight_golden(case):
 
 
 def test_pack_int4_brute_force_and_round_trip():
-    """No reference vector exists for this function: checked against a pure-Python loop and the
-    unpack(pack) invariant."""
+    """The byte layout against a pure-Python loop and the unpack(pack) invariant (the reference's
+    own outputs pin it in test_export_casts_match_reference_outputs)."""
     g = torch.Generator().manual_seed(5)
     w = (torch.randn(6, 16, generator=g) * 0.3).to(torch.bfloat16)
     wsf = export.get_scaling_factor_from_weight(w, 8)
@@ -249,6 +249,37 @@ def test_pack_int4_brute_force_and_round_trip():
         for k in range(16):
             assert int(packed[j, k]) == (q[2 * j][k] & 0xF) | ((q[2 * j + 1][k] & 0xF) << 4)
     assert torch.equal(export.unpack_int4_rows(packed), qt)
+
+
+@pytest.mark.parametrize("case", load_export_vectors(), ids=lambda c: c["name"])
+def test_export_casts_match_reference_outputs(case):
+    """Outputs recorded from the reference's pack_int4_in_uint8 / to_quantized_weight
+    (export/quant_utils.py:697-774) by tests/golden/make_export_vectors.py."""
+    w, s, fmt = case["weight"], case["scale"], case["format"]
+    if fmt in ("int4_awq", "w4a8_awq"):
+        got = export.pack_int4_in_uint8(w, s)
+    elif fmt == "fp8":
+        got = export.fp8_export_cast(w, s.unsqueeze(-1) if w.dim() == 3 else s)
+    elif fmt == "fp8_pc_pt":
+        got = export.fp8_export_cast(w, s[:, None])
+    else:
+        got = export.int8_export_cast(w, s)
+    assert_bits_equal(got, case["out"], case["name"])
+
+
+def test_export_vectors_tell_nibble_orders_apart():
+    """The fixture would fail a swapped nibble order and a pairing along K: both variants differ
+    from the recorded bytes on the 2-D cases."""
+    for case in load_export_vectors():
+        if case["format"] not in ("int4_awq", "w4a8_awq") or case["weight"].dim() != 2:
+            continue
+        w, s = case["weight"], case["scale"]
+        bs = w.shape[1] // s.shape[1]
+        q = (w / s[:, torch.arange(w.shape[1]) // bs]).round().clamp(-8, 7).to(torch.int8)
+        swapped = ((q[1::2] & 0xF) | ((q[0::2] & 0xF) << 4)).view(torch.uint8)
+        assert not torch.equal(swapped, case["out"]), case["name"]
+        along_k = ((q[:, 0::2] & 0xF) | ((q[:, 1::2] & 0xF) << 4)).view(torch.uint8)
+        assert along_k.shape != case["out"].shape or not torch.equal(along_k, case["out"])
 
 
 def test_fp8_export_cast_double_rounding_rule():
