@@ -30,7 +30,8 @@ enum mo_status {
     MO_ERR_ARG = -1,      /* null pointer, negative size, inconsistent shape */
     MO_ERR_DTYPE = -2,    /* unsupported element type */
     MO_ERR_UNSUPPORTED = -3, /* valid request the kernels do not cover (e.g. block size) */
-    MO_ERR_LAUNCH = -4    /* the HIP runtime rejected the launch */
+    MO_ERR_LAUNCH = -4,   /* the HIP runtime rejected the launch */
+    MO_ERR_TOO_LARGE = -5 /* input beyond the fixed workspace of an entry point that may not allocate */
 };
 
 int mo_version(void);
@@ -72,6 +73,20 @@ int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dty
  * aligned (use mo_absmax then).  Replaces the same reference code as mo_absmax. */
 int mo_absmax_cols_staged(const void* x, int64_t outer, int64_t axis, int dtype, float* acc,
                           void* partial, int64_t partial_rows, void* stream);
+
+/* mo_absmax_cols_staged for callers that cannot allocate or provide a workspace (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
+ * the reference.  Same arguments minus the workspace, same result: the row-slab maxima go to a
+ * fixed 4 MiB array in the library's device image (MO_ABSMAX_COLS_NOALLOC_WORDS 32-bit words,
+ * one copy per GPU for the life of the process) and the call performs no hipMalloc / hipFree.
+ * axis > MO_ABSMAX_COLS_NOALLOC_WORDS returns MO_ERR_TOO_LARGE; axis % 8 != 0 or a misaligned x
+ * returns MO_ERR_UNSUPPORTED.  Every call on a GPU uses that GPU's one array (its contents are
+ * overwritten, nothing needs clearing), so calls that overlap on one GPU -- different streams or
+ * threads -- race and must be ordered by the caller.  The first call on a device looks the
+ * array's address up (hipGetSymbolAddress); make that call outside any stream capture. */
+#define MO_ABSMAX_COLS_NOALLOC_WORDS (1 << 20)
+int mo_absmax_cols_noalloc(const void* x, int64_t outer, int64_t axis, int dtype, float* acc,
+                           void* stream);
 
 /* Per-tensor abs-max of many tensors in ONE launch.  jobs_dev is a device-resident table sorted
  * by tile_begin; job j owns tiles [tile_begin_j, tile_begin_j + ceil(elems_j /

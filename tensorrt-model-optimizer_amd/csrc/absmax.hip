@@ -6,6 +6,8 @@
 // accumulator the caller owns.
 #include "common.h"
 
+#include <mutex>
+
 namespace mo {
 
 // Running max state of one lane.  16-bit inputs keep two packed 15-bit magnitudes per word.
@@ -507,6 +509,30 @@ static int launch_absmax_cols_staged(const void* x, int64_t outer, int64_t axis,
     return MO_OK;
 }
 
+// Workspace of the entry point that may not allocate: row-slab maxima of the staged per-column
+// reduction.  One copy per GPU, held until the process ends.  In host code the array's name is
+// only a handle for hipGetSymbolAddress; kernels are given the address that call returns.
+static __device__ __align__(256) uint32_t scratch[MO_ABSMAX_COLS_NOALLOC_WORDS];
+
+constexpr int kMaxDevices = 64;
+static uint32_t* g_scratch_ptr[kMaxDevices] = {nullptr};
+static std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (looked up once per device).
+static int scratch_address(uint32_t** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MO_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        uint32_t* ptr = nullptr;
+        if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr)
+            return MO_ERR_LAUNCH;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return MO_OK;
+}
+
 }  // namespace mo
 
 extern "C" int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
@@ -555,6 +581,29 @@ extern "C" int mo_absmax_cols_staged(const void* x, int64_t outer, int64_t axis,
         case MO_F32: rc = mo::launch_absmax_cols_staged<MO_F32>(x, outer, axis, (uint32_t*)acc, (uint32_t*)partial, partial_rows, s); break;
         case MO_F16: rc = mo::launch_absmax_cols_staged<MO_F16>(x, outer, axis, (uint32_t*)acc, (uint32_t*)partial, partial_rows, s); break;
         case MO_BF16: rc = mo::launch_absmax_cols_staged<MO_BF16>(x, outer, axis, (uint32_t*)acc, (uint32_t*)partial, partial_rows, s); break;
+        default: return MO_ERR_DTYPE;
+    }
+    if (rc != MO_OK) return rc;
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_absmax_cols_noalloc(const void* x, int64_t outer, int64_t axis, int dtype,
+                                      float* acc, void* stream) {
+    if (outer < 0 || axis < 0) return MO_ERR_ARG;
+    if (outer == 0 || axis == 0) return MO_OK;
+    if (!x || !acc) return MO_ERR_ARG;
+    if (axis > MO_ABSMAX_COLS_NOALLOC_WORDS) return MO_ERR_TOO_LARGE;
+    // as many row slabs as fit the fixed workspace, up to what fills the chip
+    int64_t slabs = MO_ABSMAX_COLS_NOALLOC_WORDS / axis;
+    if (slabs > 256) slabs = 256;
+    uint32_t* partial = nullptr;
+    int rc = mo::scratch_address(&partial);
+    if (rc != MO_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case MO_F32: rc = mo::launch_absmax_cols_staged<MO_F32>(x, outer, axis, (uint32_t*)acc, partial, slabs, s); break;
+        case MO_F16: rc = mo::launch_absmax_cols_staged<MO_F16>(x, outer, axis, (uint32_t*)acc, partial, slabs, s); break;
+        case MO_BF16: rc = mo::launch_absmax_cols_staged<MO_BF16>(x, outer, axis, (uint32_t*)acc, partial, slabs, s); break;
         default: return MO_ERR_DTYPE;
     }
     if (rc != MO_OK) return rc;

@@ -10,6 +10,7 @@ extern "C" const char* mo_error_string(int status) {
         case MO_ERR_DTYPE: return "unsupported element type";
         case MO_ERR_UNSUPPORTED: return "request not covered by the kernels";
         case MO_ERR_LAUNCH: return "HIP runtime rejected the kernel launch";
+        case MO_ERR_TOO_LARGE: return "input exceeds the fixed workspace of this entry point";
         default: return "unknown status";
     }
 }

@@ -13,7 +13,7 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_PKG_DIR), "libmodelopt_hip.so")
 
 MO_F32, MO_F16, MO_BF16 = 0, 1, 2
-MO_ERR_ARG, MO_ERR_DTYPE, MO_ERR_UNSUPPORTED, MO_ERR_LAUNCH = -1, -2, -3, -4
+MO_ERR_ARG, MO_ERR_DTYPE, MO_ERR_UNSUPPORTED, MO_ERR_LAUNCH, MO_ERR_TOO_LARGE = -1, -2, -3, -4, -5
 _DTYPES = {torch.float32: MO_F32, torch.float16: MO_F16, torch.bfloat16: MO_BF16}
 
 _P, _I64, _INT = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
@@ -26,6 +26,7 @@ SIGNATURES = {
     "mo_get_option": [_INT],
     "mo_absmax": [_P, _I64, _I64, _I64, _INT, _P, _P],
     "mo_absmax_cols_staged": [_P, _I64, _I64, _INT, _P, _P, _I64, _P],
+    "mo_absmax_cols_noalloc": [_P, _I64, _I64, _INT, _P, _P],
     "mo_absmax_multi": [_P, _INT, _P, _I64, _INT, _P],
     "mo_nvfp4_quantize_multi": [_P, _INT, _P, _I64, _INT, _INT, _INT, _P],
     "mo_fp8_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _P],
