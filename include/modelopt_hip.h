@@ -37,18 +37,17 @@ enum mo_status {
 int mo_version(void);
 const char* mo_error_string(int status);
 
-/* Process-wide switches (debug / verification aids; defaults are all 0).
- * MO_OPT_FORCE_EXACT = 1 makes the NVFP4 quantize kernels divide every element by its block
- * scale (the reference's literal arithmetic) instead of the multiply-and-verify fast path; the
- * outputs are identical either way, which is what the switch exists to demonstrate.
- * MO_OPT_SATURATE_BLOCK_SCALE = 1 makes the NVFP4 quantize kernels clamp a block scale at 448
- * before its E4M3 cast.  The reference's cast (TQ/qtensor/nvfp4_tensor.py:84-91) is torch's
- * non-saturating one: a block whose abs-max exceeds the per-tensor amax by more than 448/464
- * (possible once awq_clip has shrunk that amax, TQ/model_calib.py:869-876) gets the NaN byte
- * and dequantises to NaN.  0 keeps that behaviour. */
-enum mo_option { MO_OPT_FORCE_EXACT = 0, MO_OPT_SATURATE_BLOCK_SCALE = 1, MO_OPT_COUNT_ = 2 };
-int mo_set_option(int key, int value);
-int mo_get_option(int key);
+/* Per-call flags of the NVFP4 quantize entry points (there is no process-wide state: two
+ * callers with different policies can use the library at once).
+ * MO_FLAG_FORCE_EXACT makes the kernels divide every element by its block scale (the
+ * reference's literal arithmetic) instead of the reciprocal-and-correct fast path; the outputs
+ * are identical either way, which is what the flag exists to demonstrate.
+ * MO_FLAG_SATURATE_BLOCK_SCALE makes the kernels clamp a block scale at 448 before its E4M3
+ * cast.  The reference's cast (TQ/qtensor/nvfp4_tensor.py:84-91) is torch's non-saturating one:
+ * a block whose abs-max exceeds the per-tensor amax by more than 448/464 (possible once awq_clip
+ * has shrunk that amax, TQ/model_calib.py:869-876) gets the NaN byte and dequantises to NaN.
+ * Without the flag that behaviour is kept.  Unknown bits return MO_ERR_ARG. */
+enum mo_quantize_flags { MO_FLAG_FORCE_EXACT = 1, MO_FLAG_SATURATE_BLOCK_SCALE = 2 };
 
 /* ------------------------------------------------------------------ abs-max reductions
  * Replaces reduce_amax (TQ/utils.py:156-188) as used by MaxCalibrator.collect
@@ -173,6 +172,13 @@ int mo_block_fp_qdq(const void* x, void* y, int64_t rows, int64_t k, int dtype, 
                     int format, int scale_format, const float* global_amax,
                     int64_t n_global_amax, void* stream);
 
+/* y[i] = the value of `format` nearest to x[i] (fp32 in, fp32 out, n elements): the element
+ * conversion of mo_block_fp_qdq without a block scale.  Replaces convert_to_exmy(x, format), the
+ * binding of convert_to_types (TQ/src/tensor_quant_mx.cu:398, TQ/src/tensor_quant_mx.h:163-186):
+ * ties to even (E3M0: away from zero), saturating at the format's maximum, infinities and NaN
+ * to the maximum for the table formats; MO_EF_E8M0 gives 0 as there. */
+int mo_convert_to_format(const float* x, float* y, int64_t n, int format, void* stream);
+
 /* MXFP4 storage format over the n elements of x in flat blocks of block_size (8 << k, n a
  * multiple of it).  Replaces MXFP4QTensor.quantize / dequantize (TQ/qtensor/mxfp4_tensor.py:38-83,
  * :85-144):
@@ -197,10 +203,11 @@ int mo_mxfp4_dequantize(const uint8_t* packed, const uint8_t* scales, int64_t n,
  *       them (NULL to compute).
  * Outputs: packed[rows, kp / 2] (byte i = code[2i] | code[2i+1] << 4, code = sign << 3 |
  * ordinal), wsf_out[rows, kp / block_size] E4M3 bytes (may be NULL when wsf_in is given),
- * wsf2_out (fp32 scalar, may be NULL). */
+ * wsf2_out (fp32 scalar, may be NULL).  flags: bits of mo_quantize_flags, 0 for the reference's
+ * behaviour. */
 int mo_nvfp4_quantize(const void* x, int64_t rows, int64_t k, int dtype, int block_size,
                       const float* amax, int amax_is_wsf2, const uint8_t* wsf_in,
-                      uint8_t* packed, uint8_t* wsf_out, float* wsf2_out, void* stream);
+                      uint8_t* packed, uint8_t* wsf_out, float* wsf2_out, int flags, void* stream);
 
 /* NVFP4 quantize + pack of many tensors in ONE launch (the whole-model export pass of
  * modelopt/torch/export/unified_export_hf.py:233-391, which calls to_quantized_weight once per
@@ -222,7 +229,7 @@ typedef struct mo_nvfp4_job {
 } mo_nvfp4_job;
 int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs, const int32_t* tile_job_dev,
                             int64_t total_tiles, int dtype, int block_size, int amax_is_wsf2,
-                            void* stream);
+                            int flags, void* stream);
 
 /* NVFP4 unpack + rescale.  Replaces NVFP4QTensor.dequantize (TQ/qtensor/nvfp4_tensor.py
  * :234-297) and fp4_dequantize (TQ/triton/fp4_kernel.py:307):
@@ -255,10 +262,12 @@ int mo_real_dequantize(const uint8_t* q, int64_t outer, int64_t axis, int64_t in
  * scales[b] = T(f32(T(1 / amax_b)) * 7) (what torch computes for `7 / amax` in dtype T),
  * q = clamp(rne(T(x * scale)), -8, 7) + 8, packed[i] = q[2i] << 4 | q[2i + 1].
  * scales has ceil(n / block_size) elements of dtype T; packed has ceil(n / block_size) *
- * block_size / 2 bytes.  Replaces INT4_quantize (TQ/src/tensor_quant_gpu.cu:311) with the CPU
+ * block_size / 2 bytes.  scales_given = 1 makes scales an input: the caller's per-block scales
+ * (dtype T) are used as they are and not written, which is the contract of INT4_quantize(input,
+ * scales, block_size).  Replaces INT4_quantize (TQ/src/tensor_quant_gpu.cu:311) with the CPU
  * numerics of INT4QTensor.quantize (TQ/qtensor/int4_tensor.py:40-88). */
 int mo_int4_block_quantize(const void* x, int64_t n, int64_t block_size, int dtype, void* scales,
-                           uint8_t* packed, void* stream);
+                           int scales_given, uint8_t* packed, void* stream);
 
 /* y[2i] = T((packed[i] >> 4) - 8) / scale), y[2i + 1] = T(((packed[i] & 15) - 8) / scale).
  * Replaces INT4_dequantize (TQ/src/tensor_quant_gpu.cu:262) / INT4QTensor.dequantize

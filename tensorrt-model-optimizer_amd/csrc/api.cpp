@@ -14,15 +14,3 @@ extern "C" const char* mo_error_string(int status) {
         default: return "unknown status";
     }
 }
-
-static int g_options[MO_OPT_COUNT_] = {0};
-
-extern "C" int mo_set_option(int key, int value) {
-    if (key < 0 || key >= MO_OPT_COUNT_) return MO_ERR_ARG;
-    g_options[key] = value;
-    return MO_OK;
-}
-
-extern "C" int mo_get_option(int key) {
-    return (key < 0 || key >= MO_OPT_COUNT_) ? 0 : g_options[key];
-}

@@ -226,6 +226,37 @@ extern "C" int mo_block_fp_qdq(const void* x, void* y, int64_t rows, int64_t k, 
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }
 
+// ------------------------------------------------------------------------------ element casts
+// y[i] = nearest value of `fmt` for x[i], sign carried over: the element conversion on its own
+// (no block scale).  E8M0 is a scale-only format and converts to 0, as in the reference.
+namespace mo {
+__global__ __launch_bounds__(256) void convert_to_format_kernel(const float* __restrict__ x,
+                                                                float* __restrict__ y, int64_t n,
+                                                                int fmt) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float v = x[i];
+    float q = 0.0f;
+    if (fmt != MO_EF_E8M0) {
+        q = convert_runtime(__builtin_fabsf(v), fmt);
+        if (fmt == MO_EF_E4M3 || fmt == MO_EF_E5M2) q = __builtin_copysignf(q, v);
+        else if (v < 0.0f) q = -q;
+    }
+    y[i] = q;
+}
+}  // namespace mo
+
+extern "C" int mo_convert_to_format(const float* x, float* y, int64_t n, int format, void* stream) {
+    if (n < 0) return MO_ERR_ARG;
+    if (format < MO_EF_E4M3 || format > MO_EF_E8M0) return MO_ERR_UNSUPPORTED;
+    if (n == 0) return MO_OK;
+    if (!x || !y) return MO_ERR_ARG;
+    const int64_t grid = (n + 255) / 256;
+    if (grid > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+    mo::convert_to_format_kernel<<<(unsigned)grid, 256, 0, (hipStream_t)stream>>>(x, y, n, format);
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
 // ------------------------------------------------------------------------------ MXFP4 storage
 // Packed MXFP4: blocks of `block` elements share the E8M0 byte 127 + ceil(log2(amax / 6))
 // (clamped below at -127); codes are sign << 3 | ordinal with the ordinal = number of E2M1 bounds

@@ -16,7 +16,7 @@ namespace mo {
 // an invalid operation (0/0, inf/inf) the x86 reference produces the negative default NaN and
 // therefore the byte 0xFF; a NaN that comes from a NaN operand keeps that operand's (positive)
 // sign and gives 0x7F.  `cap` is +inf for the reference's cast (a quotient above E4M3's range
-// becomes the NaN byte) or 448 to saturate instead (option MO_OPT_SATURATE_BLOCK_SCALE).
+// becomes the NaN byte) or 448 to saturate instead (flag MO_FLAG_SATURATE_BLOCK_SCALE).
 __device__ __forceinline__ uint32_t block_scale_byte(float bmax, float gs6,
                                                      float cap = __builtin_inff()) {
     float bs = bmax / gs6;
@@ -534,11 +534,9 @@ static void launch_qdq(const void* x, void* y, int64_t rows, int64_t k, int64_t 
 
 }  // namespace mo
 
-// option bits handed to the quantize kernels
-static int quantize_opts() {
-    return (mo_get_option(MO_OPT_FORCE_EXACT) ? mo::kOptForceExact : 0) |
-           (mo_get_option(MO_OPT_SATURATE_BLOCK_SCALE) ? mo::kOptSaturateScale : 0);
-}
+static_assert(mo::kOptForceExact == MO_FLAG_FORCE_EXACT &&
+              mo::kOptSaturateScale == MO_FLAG_SATURATE_BLOCK_SCALE, "flag bits");
+constexpr int kKnownFlags = MO_FLAG_FORCE_EXACT | MO_FLAG_SATURATE_BLOCK_SCALE;
 
 #define MO_DISPATCH_DT_BS(dtype, bs, CALL)                                            \
     switch (dtype) {                                                                  \
@@ -560,8 +558,8 @@ static int quantize_opts() {
 extern "C" int mo_nvfp4_quantize(const void* x, int64_t rows, int64_t k, int dtype, int block_size,
                                  const float* amax, int amax_is_wsf2, const uint8_t* wsf_in,
                                  uint8_t* packed, uint8_t* wsf_out, float* wsf2_out,
-                                 void* stream) {
-    if (rows < 0 || k < 0) return MO_ERR_ARG;
+                                 int flags, void* stream) {
+    if (rows < 0 || k < 0 || (flags & ~kKnownFlags)) return MO_ERR_ARG;
     if (block_size != 8 && block_size != 16 && block_size != 32) return MO_ERR_UNSUPPORTED;
     if (rows == 0 || k == 0) return MO_OK;
     if (!x || !amax || !packed || (!wsf_in && !wsf_out)) return MO_ERR_ARG;
@@ -574,13 +572,13 @@ extern "C" int mo_nvfp4_quantize(const void* x, int64_t rows, int64_t k, int dty
         const int64_t tiles = (nblocks + mo::kTileBlocks - 1) / mo::kTileBlocks;
         if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
         mo::nvfp4_quantize_fast_kernel<<<(unsigned)tiles, 256, 0, s>>>(
-            (const uint16_t*)x, nblocks, tiles, amax, amax_is_wsf2, quantize_opts(),
+            (const uint16_t*)x, nblocks, tiles, amax, amax_is_wsf2, flags,
             (mo::u32x2*)packed, wsf_out, wsf2_out);
         return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
     }
 #define CALL(DT, BS) \
     mo::launch_quantize<DT, BS>(x, rows, k, kp, amax, amax_is_wsf2, wsf_in, packed, wsf_out, wsf2_out, \
-                                quantize_opts(), s)
+                                flags, s)
     MO_DISPATCH_DT_BS(dtype, block_size, CALL)
 #undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
@@ -644,12 +642,13 @@ extern "C" int mo_nvfp4_qdq(const void* x, void* y, int64_t rows, int64_t k, int
 extern "C" int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs,
                                        const int32_t* tile_job_dev, int64_t total_tiles,
                                        int dtype, int block_size, int amax_is_wsf2,
-                                       void* stream) {
-    if (njobs < 0 || total_tiles < 0 || total_tiles > 0x7FFFFFFF) return MO_ERR_ARG;
+                                       int flags, void* stream) {
+    if (njobs < 0 || total_tiles < 0 || total_tiles > 0x7FFFFFFF || (flags & ~kKnownFlags))
+        return MO_ERR_ARG;
     if (dtype != MO_BF16 || block_size != 16) return MO_ERR_UNSUPPORTED;
     if (njobs == 0 || total_tiles == 0) return MO_OK;
     if (!jobs_dev) return MO_ERR_ARG;
     mo::nvfp4_quantize_multi_kernel<<<(unsigned)total_tiles, 256, 0, (hipStream_t)stream>>>(
-        jobs_dev, njobs, tile_job_dev, amax_is_wsf2, quantize_opts());
+        jobs_dev, njobs, tile_job_dev, amax_is_wsf2, flags);
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

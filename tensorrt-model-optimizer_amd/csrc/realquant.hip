@@ -262,6 +262,7 @@ __global__ __launch_bounds__(256) void int4_block_quantize_kernel(const void* __
                                                                   int64_t n, int64_t bs,
                                                                   int64_t nblocks,
                                                                   void* __restrict__ scales,
+                                                                  int scales_given,
                                                                   uint8_t* __restrict__ packed) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; b < nblocks; b += stride) {
@@ -273,8 +274,9 @@ __global__ __launch_bounds__(256) void int4_block_quantize_kernel(const void* __
             m = t > m ? t : m;
         }
         const float amax = u2f(m);
-        const float scale = round_via<DT>(round_via<DT>(1.0f / amax) * 7.0f);
-        store_elem<DT>(scales, b, scale);
+        float scale = round_via<DT>(round_via<DT>(1.0f / amax) * 7.0f);
+        if (scales_given) scale = load_elem<DT>(scales, b);
+        else store_elem<DT>(scales, b, scale);
         for (int64_t j = 0; j < bs; j += 2) {
             uint32_t nib[2];
 #pragma unroll
@@ -350,7 +352,7 @@ constexpr int kInt4QuantRounds = 8;   // chunks (16-byte loads in flight) per la
 template <int DT>
 __global__ __launch_bounds__(256) void int4_block_quantize_tile_kernel(
     const void* __restrict__ x, int64_t chunks, int lanes_per_block, int shift,
-    void* __restrict__ scales, uint32_t* __restrict__ packed) {
+    void* __restrict__ scales, int scales_given, uint32_t* __restrict__ packed) {
     constexpr int U = kInt4QuantRounds;
     const int64_t c0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
     RawChunk<DT> raw[U];
@@ -374,8 +376,9 @@ __global__ __launch_bounds__(256) void int4_block_quantize_tile_kernel(
         // chunks is a multiple of lanes_per_block, so the lanes of a block are all in or all out
         m = group_max_u32(m, shift);
         if (c >= chunks) continue;
-        const float scale = round_via<DT>(round_via<DT>(1.0f / u2f(m)) * 7.0f);
-        if ((threadIdx.x & (lanes_per_block - 1)) == 0) store_elem<DT>(scales, c >> shift, scale);
+        float scale = round_via<DT>(round_via<DT>(1.0f / u2f(m)) * 7.0f);
+        if (scales_given) scale = load_elem<DT>(scales, c >> shift);
+        else if ((threadIdx.x & (lanes_per_block - 1)) == 0) store_elem<DT>(scales, c >> shift, scale);
         // byte = (hi + 8) << 4 | (lo + 8) = 16 * hi + lo + 0x88; the +8s of the four bytes are
         // added once to the assembled word (the borrows of negative bytes cancel exactly)
         int w = 0;
@@ -637,7 +640,8 @@ extern "C" int mo_real_dequantize(const uint8_t* q, int64_t outer, int64_t axis,
 }
 
 extern "C" int mo_int4_block_quantize(const void* x, int64_t n, int64_t block_size, int dtype,
-                                      void* scales, uint8_t* packed, void* stream) {
+                                      void* scales, int scales_given, uint8_t* packed,
+                                      void* stream) {
     if (n < 0 || block_size <= 0 || (block_size & 1)) return MO_ERR_ARG;
     if (n == 0) return MO_OK;
     if (!x || !scales || !packed) return MO_ERR_ARG;
@@ -652,13 +656,13 @@ extern "C" int mo_int4_block_quantize(const void* x, int64_t n, int64_t block_si
         (((uintptr_t)packed & 3u) == 0) && tiles <= 0x7FFFFFFF) {
 #define CALL(DT)                                                                          \
     mo::int4_block_quantize_tile_kernel<DT><<<(unsigned)tiles, 256, 0, s>>>(              \
-        x, n / 8, 1 << shift, shift, scales, (uint32_t*)packed)
+        x, n / 8, 1 << shift, shift, scales, scales_given, (uint32_t*)packed)
         DISPATCH_DT(dtype, CALL)
 #undef CALL
         return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
     }
     const unsigned g = mo::blocks_for(nblocks);
-#define CALL(DT) mo::int4_block_quantize_kernel<DT><<<g, 256, 0, s>>>(x, n, block_size, nblocks, scales, packed)
+#define CALL(DT) mo::int4_block_quantize_kernel<DT><<<g, 256, 0, s>>>(x, n, block_size, nblocks, scales, scales_given, packed)
     DISPATCH_DT(dtype, CALL)
 #undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;

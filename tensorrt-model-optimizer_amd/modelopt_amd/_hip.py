@@ -13,6 +13,8 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_PKG_DIR), "libmodelopt_hip.so")
 
 MO_F32, MO_F16, MO_BF16 = 0, 1, 2
+# per-call flags of the NVFP4 quantize entry points (enum mo_quantize_flags)
+MO_FLAG_FORCE_EXACT, MO_FLAG_SATURATE_BLOCK_SCALE = 1, 2
 MO_ERR_ARG, MO_ERR_DTYPE, MO_ERR_UNSUPPORTED, MO_ERR_LAUNCH, MO_ERR_TOO_LARGE = -1, -2, -3, -4, -5
 _DTYPES = {torch.float32: MO_F32, torch.float16: MO_F16, torch.bfloat16: MO_BF16}
 
@@ -22,13 +24,11 @@ _P, _I64, _INT = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 SIGNATURES = {
     "mo_version": [],
     "mo_error_string": [_INT],
-    "mo_set_option": [_INT, _INT],
-    "mo_get_option": [_INT],
     "mo_absmax": [_P, _I64, _I64, _I64, _INT, _P, _P],
     "mo_absmax_cols_staged": [_P, _I64, _I64, _INT, _P, _P, _I64, _P],
     "mo_absmax_cols_noalloc": [_P, _I64, _I64, _INT, _P, _P],
     "mo_absmax_multi": [_P, _INT, _P, _I64, _INT, _P],
-    "mo_nvfp4_quantize_multi": [_P, _INT, _P, _I64, _INT, _INT, _INT, _P],
+    "mo_nvfp4_quantize_multi": [_P, _INT, _P, _I64, _INT, _INT, _INT, _INT, _P],
     "mo_fp8_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _P],
     "mo_int_qdq": [_P, _P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _INT, _P],
     "mo_nvfp4_qdq": [_P, _P, _I64, _I64, _INT, _P, _INT, _INT, _INT, _P],
@@ -36,11 +36,12 @@ SIGNATURES = {
     "mo_mxfp4_quantize": [_P, _I64, _INT, _INT, _P, _P, _P],
     "mo_mxfp4_dequantize": [_P, _P, _I64, _INT, _P, _INT, _P],
     "mo_block_fp_qdq": [_P, _P, _I64, _I64, _INT, _INT, _INT, _INT, _P, _I64, _P],
-    "mo_nvfp4_quantize": [_P, _I64, _I64, _INT, _INT, _P, _INT, _P, _P, _P, _P, _P],
+    "mo_convert_to_format": [_P, _P, _I64, _INT, _P],
+    "mo_nvfp4_quantize": [_P, _I64, _I64, _INT, _INT, _P, _INT, _P, _P, _P, _P, _INT, _P],
     "mo_nvfp4_dequantize": [_P, _P, _P, _I64, _I64, _INT, _P, _INT, _P],
     "mo_real_quantize": [_P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _P, _P],
     "mo_real_dequantize": [_P, _I64, _I64, _I64, _INT, _P, _INT, _P, _INT, _P],
-    "mo_int4_block_quantize": [_P, _I64, _I64, _INT, _P, _P, _P],
+    "mo_int4_block_quantize": [_P, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_int4_block_dequantize": [_P, _I64, _I64, _P, _P, _INT, _P],
     "mo_int4_pack_rows": [_P, _I64, _I64, _I64, _I64, _INT, _P, _P, _P],
     "mo_nf4_quantize": [_P, _I64, _I64, _INT, _P, _P, _P],
@@ -207,6 +208,17 @@ def block_fp_qdq(x, block_size, fmt, scale_fmt="E8M0", global_amax=None, out=Non
     return y
 
 
+def convert_to_format(x, fmt):
+    """Nearest value of element format ``fmt`` (name or index of ``ELEM_FORMATS``) for every
+    element of the fp32 device tensor ``x``."""
+    _require_device(x)
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    fmt = ELEM_FORMATS.index(fmt) if isinstance(fmt, str) else int(fmt)
+    y = torch.empty_like(x)
+    call("mo_convert_to_format", x, _ptr(x), _ptr(y), x.numel(), fmt, _stream(x))
+    return y
+
+
 def mxfp4_quantize(x, block_size=32):
     """-> (packed uint8 [..., k / 2], E8M0 scale bytes uint8 [numel / block_size, 1])."""
     _require_device(x)
@@ -227,8 +239,9 @@ def mxfp4_dequantize(packed, scales, block_size, dtype):
     return y
 
 
-def nvfp4_quantize(x, amax_f32, block_size=16, amax_is_wsf2=False, wsf_in=None):
-    """Returns (packed uint8 [..., kp/2], wsf float8_e4m3fn [..., kp/bs], wsf2 f32 scalar)."""
+def nvfp4_quantize(x, amax_f32, block_size=16, amax_is_wsf2=False, wsf_in=None, flags=0):
+    """Returns (packed uint8 [..., kp/2], wsf float8_e4m3fn [..., kp/bs], wsf2 f32 scalar).
+    ``flags``: ``MO_FLAG_*`` bits."""
     _require_device(x, amax_f32, wsf_in)
     assert x.is_contiguous() and amax_f32.dtype == torch.float32
     k = x.shape[-1]
@@ -246,7 +259,7 @@ def nvfp4_quantize(x, amax_f32, block_size=16, amax_is_wsf2=False, wsf_in=None):
         wsf_arg = wsf
     call("mo_nvfp4_quantize", x, _ptr(x), rows, k, dtype_code(x.dtype), block_size,
          _ptr(amax_f32), int(amax_is_wsf2), _ptr(wsf_arg), _ptr(packed),
-         None if wsf_in is not None else _ptr(wsf), _ptr(wsf2), _stream(x))
+         None if wsf_in is not None else _ptr(wsf), _ptr(wsf2), int(flags), _stream(x))
     return packed, wsf.view(torch.float8_e4m3fn), wsf2
 
 
@@ -284,16 +297,21 @@ def real_dequantize(q, scale, outer, axis, inner, fmt, dtype):
     return y
 
 
-def int4_block_quantize(x, block_size):
-    """Flat-block INT4 quantize + pack: returns (packed uint8 [padded_numel / 2], scales [nblocks, 1])."""
-    _require_device(x)
+def int4_block_quantize(x, block_size, scales=None):
+    """Flat-block INT4 quantize + pack: returns (packed uint8 [padded_numel / 2], scales [nblocks, 1]).
+    ``scales`` (``7 / amax`` per block, dtype of ``x``) are computed unless given."""
+    _require_device(x, scales)
     assert x.is_contiguous()
     n = x.numel()
     nblocks = -(-n // block_size)
-    scales = torch.empty((nblocks, 1), dtype=x.dtype, device=x.device)
+    given = scales is not None
+    if given:
+        assert scales.is_contiguous() and scales.dtype == x.dtype and scales.numel() == nblocks
+    else:
+        scales = torch.empty((nblocks, 1), dtype=x.dtype, device=x.device)
     packed = torch.empty(nblocks * block_size // 2, dtype=torch.uint8, device=x.device)
     call("mo_int4_block_quantize", x, _ptr(x), n, block_size, dtype_code(x.dtype), _ptr(scales),
-         _ptr(packed), _stream(x))
+         int(given), _ptr(packed), _stream(x))
     return packed, scales
 
 
@@ -460,18 +478,6 @@ def sq_diff_sum_into(a, b, acc):
     return acc
 
 
-# ----------------------------------------------------------------------------- options
-
-MO_OPT_FORCE_EXACT = 0
-MO_OPT_SATURATE_BLOCK_SCALE = 1
-
-
-def set_option(key: int, value: int):
-    rc = load().mo_set_option(key, value)
-    if rc != 0:
-        raise RuntimeError(f"mo_set_option({key}) failed with status {rc}")
-
-
 # ----------------------------------------------------------------------------- multi-tensor plans
 
 ABSMAX_TILE_ELEMS = 32768
@@ -546,10 +552,11 @@ class Nvfp4QuantizePlan:
     float8_e4m3fn [..., K/16], ``wsf2`` float32 [n].
     """
 
-    def __init__(self, tensors, amax, amax_is_wsf2=False):
+    def __init__(self, tensors, amax, amax_is_wsf2=False, flags=0):
         assert len(tensors) > 0 and amax.dtype == torch.float32 and amax.numel() == len(tensors)
         dev = tensors[0].device
         self.tensors, self.amax, self.amax_is_wsf2 = list(tensors), amax, bool(amax_is_wsf2)
+        self.flags = int(flags)
         self.wsf2 = torch.empty(len(tensors), dtype=torch.float32, device=dev)
         self.packed, self._wsf_u8 = [], []
         rows, tile, per_job = [], 0, []
@@ -585,5 +592,5 @@ class Nvfp4QuantizePlan:
     def run(self):
         call("mo_nvfp4_quantize_multi", self.amax, _ptr(self.jobs), len(self.tensors),
              _ptr(self.tile_job), self.total_tiles, MO_BF16, 16, int(self.amax_is_wsf2),
-             _stream(self.amax))
+             self.flags, _stream(self.amax))
         return self.packed, self.wsf, self.wsf2

@@ -17,6 +17,7 @@ from torch import nn
 
 from ... import _hip
 from ..quantization.nn import SequentialQuantizer, TensorQuantizer
+from ..quantization.overflow import nvfp4_quantize_flags
 from ..quantization.qtensor import NVFP4QTensor, QTensorWrapper
 from ..quantization.utils import is_quantized_linear, true_divide
 from .model_config import *  # noqa: F403
@@ -90,7 +91,8 @@ def _export_nvfp4_batched(modules: list[nn.Module], dtype: torch.dtype):
     weights = [m.weight.data for m in modules]
     amax = torch.stack([m.weight_quantizer._amax.reshape(()).float() for m in modules]).to(
         weights[0].device)
-    plan = _hip.Nvfp4QuantizePlan(weights, amax)  # the kernel derives wsf2 = amax / (6 * 448)
+    # the kernel derives wsf2 = amax / (6 * 448)
+    plan = _hip.Nvfp4QuantizePlan(weights, amax, flags=nvfp4_quantize_flags())
     packed, wsf, wsf2 = plan.run()
     for i, m in enumerate(modules):
         _register_input_scale(m, getattr(m, "input_quantizer", None))

@@ -18,6 +18,7 @@ import torch.nn.functional as F
 
 from .... import _hip
 from .. import kernels
+from ..overflow import fp8_saturates
 from ..utils import convert_quantization_axis_to_reduce_axis
 from .max import _Calibrator
 
@@ -65,7 +66,7 @@ class MseCalibrator(_Calibrator):
             return {"kind": "int", "num_bits": q._num_bits, "unsigned": q._unsigned,
                     "narrow_range": q._narrow_range}
         if q._num_bits == (4, 3):
-            return {"kind": "fp8"}
+            return {"kind": "fp8", "saturate": None}  # decided per call from the candidates' shape
         return None
 
     @torch.no_grad()
@@ -100,6 +101,8 @@ class MseCalibrator(_Calibrator):
         x = x if x.is_contiguous() else x.contiguous()
         cand = torch.stack([c.to(torch.float32).reshape(-1).expand(axis) for c in cands]).contiguous()
         loss = torch.zeros_like(cand)
+        if spec.get("saturate", False) is None:
+            spec = dict(spec, saturate=fp8_saturates(cands[0]))
         if not _hip.qdq_sq_err_into(x, cand, loss, outer, axis, inner, **spec):
             return False
         for step in range(self._num_steps):

@@ -37,10 +37,11 @@ class _IntExt:
 
     @staticmethod
     def INT4_quantize(input_flat, scales, block_size):  # noqa: N802
-        """Pack with *given* inverse scales is what the CUDA kernel does; the CPU numerics the
-        build follows derive the scales from the data, so they are recomputed here and must
-        agree with the argument."""
-        packed, _ = _hip.int4_block_quantize(input_flat.contiguous(), block_size)
+        """``clamp(round(input * scales[block]), -8, 7) + 8`` packed two per byte with the
+        caller's per-block scales (rounding follows the reference's tensor expression,
+        qtensor/int4_tensor.py:69-83: product in the input dtype, ties to even)."""
+        scales = scales.to(input_flat.dtype).contiguous()
+        packed, _ = _hip.int4_block_quantize(input_flat.contiguous(), block_size, scales)
         return packed
 
     @staticmethod
@@ -80,6 +81,13 @@ class _MxExt:
             raise ValueError("Blocksize for fused call must be one of {8, 16, 32}")
         return kernels.fake_quant_block_fp(inputs, block_size, _MxExt._names[int(format)],
                                            _MxExt._names[int(scale_format)], global_amax)
+
+    @staticmethod
+    def convert_to_exmy(x, format):
+        """One Python float to the nearest value of ``format`` (the reference's host helper,
+        TQ/src/tensor_quant_mx.cu:398); computed by the device code that the kernels use."""
+        t = torch.tensor([float(x)], dtype=torch.float32, device="cuda")
+        return float(_hip.convert_to_format(t, int(format)).item())
 
 
 def _loaded(raise_if_failed):

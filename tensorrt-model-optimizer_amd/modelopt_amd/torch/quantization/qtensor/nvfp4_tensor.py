@@ -8,7 +8,8 @@ E2M1 ordinal); per-block scales ``float8_e4m3fn`` [..., K/block]; one fp32 globa
 import torch
 
 from .... import _hip
-from ..utils import reduce_amax, reduce_block_amax, true_divide
+from ..overflow import nvfp4_quantize_flags
+from ..utils import reduce_amax, reduce_block_amax, reduce_block_padding, true_divide
 from .base_qtensor import BaseQuantizedTensor
 
 __all__ = ["NVFP4QTensor"]
@@ -49,7 +50,7 @@ class NVFP4QTensor(BaseQuantizedTensor):
             scale[scale == 0] = 1.0
             return scale, weights_scaling_factor_2
         _, wsf, _ = _hip.nvfp4_quantize(input.contiguous(), _f32_scalar(wsf2), block_size,
-                                        amax_is_wsf2=True)
+                                        amax_is_wsf2=True, flags=nvfp4_quantize_flags())
         return wsf, weights_scaling_factor_2
 
     @classmethod
@@ -69,7 +70,18 @@ class NVFP4QTensor(BaseQuantizedTensor):
         """Returns (NVFP4QTensor, per-block E4M3 scales, fp32 global scale) in one kernel pass
         (plus one abs-max pass when the global scale is not given)."""
         if keep_high_precision:
-            raise NotImplementedError("keep_high_precision=True (un-rounded scaled weights) is not built")
+            # the reference returns the scaled weight before the FP4 cast, fp32 and still padded
+            # (qtensor/nvfp4_tensor.py:208-222); a few tensor ops, no caller on the hot path
+            xp = reduce_block_padding(input, {-1: block_size})
+            if weights_scaling_factor_2 is None:
+                weights_scaling_factor_2 = cls.get_weights_scaling_factor_2(xp)
+            if weights_scaling_factor is None:
+                weights_scaling_factor, _ = cls.get_weights_scaling_factor(
+                    xp, block_size, weights_scaling_factor_2)
+            scale = weights_scaling_factor.to(xp.device).to(torch.float32) * \
+                weights_scaling_factor_2.to(xp.device)
+            blocks = xp.reshape(*xp.shape[:-1], -1, block_size)
+            return torch.div(blocks, scale.unsqueeze(-1)).reshape(xp.shape)
         shape, dtype = input.shape, input.dtype
         x = input.contiguous()
         if weights_scaling_factor_2 is None:
@@ -82,7 +94,8 @@ class NVFP4QTensor(BaseQuantizedTensor):
         if weights_scaling_factor is not None:
             wsf_in = weights_scaling_factor.to(x.device).contiguous()
             assert wsf_in.dtype == torch.float8_e4m3fn, "block scales must be float8_e4m3fn"
-        packed, wsf, wsf2 = _hip.nvfp4_quantize(x, scalar, block_size, is_wsf2, wsf_in)
+        packed, wsf, wsf2 = _hip.nvfp4_quantize(x, scalar, block_size, is_wsf2, wsf_in,
+                                                flags=nvfp4_quantize_flags())
         if weights_scaling_factor is not None:
             wsf = weights_scaling_factor
         if weights_scaling_factor_2 is not None:

@@ -13,6 +13,7 @@ from torch.autograd import Function
 from ... import _hip
 from . import kernels
 from .config import QuantizerAttributeConfig
+from .overflow import fp8_saturates, get_fp8_overflow_behavior, set_fp8_overflow_behavior  # noqa: F401
 
 __all__ = [
     "FakeTensorQuantFunction", "ScaledE4M3Function", "DynamicBlockQuantizationFunction",
@@ -28,45 +29,19 @@ mx_format_map = {(4, 3): "E4M3", (5, 2): "E5M2", (3, 2): "E3M2", (2, 3): "E2M3",
 NVFP4_FAKE_QUANT_MODE = 0
 
 
-# What FP8 fake quantisation does with a scaled value beyond the E4M3 range (|x| * 448 / amax
-# > 464, i.e. data above the calibrated amax).  The reference has both behaviours: its eager
-# torch path -- the only one that runs on a CPU -- casts with ``Tensor.to(float8_e4m3fn)``, which
-# gives NaN (tensor_quant.py:45-59), its CUDA kernel clamps to +-448 first
-# (src/tensor_quant_gpu_fp8.cu:43).  "nan" is the default here because results are held to the
-# CPU path bit for bit; "saturate" is what a deployment wants (a KV-cache value a hair above the
-# calibration maximum becomes the maximum instead of poisoning the attention output).
-_FP8_OVERFLOW = "nan"
-
-
-def set_fp8_overflow_behavior(mode: str) -> str:
-    """``"nan"`` (eager / CPU semantics, default) or ``"saturate"`` (the CUDA kernel's).  Returns
-    the previous mode.
-
-    The mode also governs the E4M3 cast of NVFP4 block scales in *real* quantisation (compress,
-    export): the reference casts with torch's non-saturating conversion
-    (qtensor/nvfp4_tensor.py:84-91), so a block whose abs-max lies above the per-tensor amax --
-    which ``awq_clip`` shrinks for NVFP4 (model_calib.py:869-876) -- stores the NaN byte;
-    ``"saturate"`` stores 448 instead, which is what the fake-quant kernel the clip search
-    itself ran on computes with."""
-    global _FP8_OVERFLOW
-    if mode not in ("nan", "saturate"):
-        raise ValueError(f"mode must be 'nan' or 'saturate', got {mode!r}")
-    previous, _FP8_OVERFLOW = _FP8_OVERFLOW, mode
-    _hip.set_option(_hip.MO_OPT_SATURATE_BLOCK_SCALE, int(mode == "saturate"))
-    return previous
-
-
-def get_fp8_overflow_behavior() -> str:
-    return _FP8_OVERFLOW
-
-
 def scaled_e4m3_impl(inputs: torch.Tensor, amax: torch.Tensor | None = None) -> torch.Tensor:
-    """FP8 E4M3 fake quantisation with the numerics of the reference's eager path (or, after
-    ``set_fp8_overflow_behavior("saturate")``, of its CUDA kernel for out-of-range values)."""
-    return kernels.fake_quant_fp8(inputs, amax, saturate=_FP8_OVERFLOW == "saturate")
+    """FP8 E4M3 fake quantisation.  Out-of-range values follow the reference's dispatch
+    (tensor_quant.py:62-90): clamped where its CUDA kernel runs (per-tensor or per-axis amax),
+    NaN where it falls back to the eager cast; see ``overflow.set_fp8_overflow_behavior``."""
+    return kernels.fake_quant_fp8(inputs, amax, saturate=fp8_saturates(amax))
 
 
-fp8_eager = scaled_e4m3_impl
+def fp8_eager(inputs: torch.Tensor, amax: torch.Tensor | None = None) -> torch.Tensor:
+    """The reference's eager expression (tensor_quant.py:45-59): the non-saturating cast, NaN
+    beyond the E4M3 range, whatever the overflow mode."""
+    return kernels.fake_quant_fp8(inputs, amax, saturate=False)
+
+
 
 
 def fake_quant_impl(inputs, amax, num_bits=8, unsigned=False, narrow_range=True):
@@ -108,8 +83,58 @@ def _dynamic_block_quantize_impl(inputs, block_size, amax, num_bits, exponent_bi
                                        mx_format_map[scale_bits], amax)
 
 
-quantize_op = _quantize_impl
-dynamic_block_quantize_op = _dynamic_block_quantize_impl
+def _like_input(inputs, *_args, **_kwargs):
+    """Fake (meta) implementation of both operators: same shape and dtype as the input."""
+    return torch.empty_like(inputs)
+
+
+def _register_operators():
+    """``tensorrt::quantize_op`` and ``tensorrt::dynamic_block_quantize_op`` (+ ``.overload`` for
+    ``amax=None``) with the reference's schemas (tensor_quant.py:221-273), so that a traced or
+    exported graph of a quantised model carries the same operator nodes.  Returns the two
+    callables; the plain Python functions if registration is impossible (e.g. the names are
+    already taken by the reference package loaded in the same process)."""
+    try:
+        torch.library.define(
+            "tensorrt::quantize_op",
+            "(Tensor input, Tensor amax, int num_bits, int exponent_bits, "
+            "bool unsigned, bool narrow_range) -> Tensor")
+        torch.library.define(
+            "tensorrt::dynamic_block_quantize_op",
+            "(Tensor input, int block_size, Tensor amax, int num_bits, int exponent_bits, "
+            "int scale_num_bits, int scale_exponent_bits) -> Tensor")
+        torch.library.define(
+            "tensorrt::dynamic_block_quantize_op.overload",
+            "(Tensor input, int block_size, None amax, int num_bits, int exponent_bits, "
+            "int scale_num_bits, int scale_exponent_bits) -> Tensor")
+        torch.library.impl("tensorrt::quantize_op", ["cpu", "cuda"])(_quantize_impl)
+        torch.library.impl("tensorrt::dynamic_block_quantize_op", ["cpu", "cuda"])(
+            _dynamic_block_quantize_impl)
+        # the reference's implementation of the amax=None overload returns an uninitialised
+        # tensor (tensor_quant.py:241-251); here it quantises (MX formats need no global amax)
+        torch.library.impl("tensorrt::dynamic_block_quantize_op.overload", ["cpu", "cuda"])(
+            _dynamic_block_quantize_impl)
+        for name in ("quantize_op", "dynamic_block_quantize_op", "dynamic_block_quantize_op.overload"):
+            torch.library.register_fake("tensorrt::" + name)(_like_input)
+        return torch.ops.tensorrt.quantize_op, torch.ops.tensorrt.dynamic_block_quantize_op
+    except (AttributeError, RuntimeError) as e:
+        import warnings
+
+        warnings.warn("Unable to register operators with torch.library. Exporting quantized models "
+                      f"with torch.export will not be supported.\n{e}")
+        return _quantize_impl, _dynamic_block_quantize_impl
+
+
+_quantize_operator, dynamic_block_quantize_op = _register_operators()
+
+
+def quantize_op(inputs, amax, num_bits=8, exponent_bits=0, unsigned=False, narrow_range=True):
+    """``tensorrt::quantize_op``; the operator's schema wants a tensor amax and 32-bit floating
+    inputs or narrower, so ``amax=None`` (a plain E4M3 cast) and float64 go to the function."""
+    if amax is None or inputs.dtype == torch.float64 or not isinstance(amax, torch.Tensor):
+        return _quantize_impl(inputs, amax, num_bits, exponent_bits, unsigned, narrow_range)
+    return _quantize_operator(inputs, amax, num_bits, exponent_bits, unsigned, narrow_range)
+
 
 QUANT_DESC_8BIT_PER_TENSOR = QuantizerAttributeConfig(num_bits=8)
 QUANT_DESC_UNSIGNED_8BIT_PER_TENSOR = QuantizerAttributeConfig(num_bits=8, unsigned=True)

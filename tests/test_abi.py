@@ -40,9 +40,7 @@ def test_version_and_error_strings_without_gpu():
     assert lib.mo_version() >= 1
     assert lib.mo_error_string(0) == b"ok"
     assert b"invalid argument" in lib.mo_error_string(-1)
-    assert lib.mo_set_option(99, 1) == -1
-    assert lib.mo_get_option(_hip.MO_OPT_FORCE_EXACT) == 0
-    assert lib.mo_get_option(_hip.MO_OPT_SATURATE_BLOCK_SCALE) == 0
+    assert not hasattr(lib, "mo_set_option")  # no process-wide state: flags travel with each call
 
 
 def test_missing_library_fails_loudly(monkeypatch):
@@ -68,12 +66,17 @@ def test_argument_checks_that_need_no_gpu():
     buf = (ctypes.c_float * 64)()
     p = ctypes.cast(buf, ctypes.c_void_p)
     # abs-max / qdq: empty tensors
-    assert lib.mo_nvfp4_quantize(null, 0, 0, 2, 16, null, 0, null, null, null, null, null) == OK
-    assert lib.mo_nvfp4_quantize(p, 4, 16, 2, 12, p, 0, null, p, p, p, null) == UNSUP      # block size
-    assert lib.mo_nvfp4_quantize(null, 4, 16, 2, 16, p, 0, null, p, p, p, null) == ARG     # null input
-    assert lib.mo_nvfp4_quantize_multi(null, 0, null, 0, 2, 16, 0, null) == OK
-    assert lib.mo_nvfp4_quantize_multi(null, 1, null, 1, 2, 16, 0, null) == ARG
-    assert lib.mo_nvfp4_quantize_multi(p, 1, null, 1, 0, 16, 0, null) == UNSUP             # fp32 tensors
+    assert lib.mo_nvfp4_quantize(null, 0, 0, 2, 16, null, 0, null, null, null, null, 0, null) == OK
+    assert lib.mo_nvfp4_quantize(p, 4, 16, 2, 12, p, 0, null, p, p, p, 0, null) == UNSUP   # block size
+    assert lib.mo_nvfp4_quantize(null, 4, 16, 2, 16, p, 0, null, p, p, p, 0, null) == ARG  # null input
+    assert lib.mo_nvfp4_quantize(null, 0, 0, 2, 16, null, 0, null, null, null, null, 64, null) == ARG  # flag bit
+    assert lib.mo_nvfp4_quantize_multi(null, 0, null, 0, 2, 16, 0, 0, null) == OK
+    assert lib.mo_nvfp4_quantize_multi(null, 1, null, 1, 2, 16, 0, 0, null) == ARG
+    assert lib.mo_nvfp4_quantize_multi(p, 1, null, 1, 0, 16, 0, 0, null) == UNSUP          # fp32 tensors
+    assert lib.mo_nvfp4_quantize_multi(null, 0, null, 0, 2, 16, 0, 4, null) == ARG         # flag bit
+    assert lib.mo_convert_to_format(null, null, 0, 6, null) == OK
+    assert lib.mo_convert_to_format(p, p, 4, 10, null) == UNSUP
+    assert lib.mo_int4_block_quantize(null, 0, 128, 2, null, 1, null, null) == OK
     # clip search
     ratios = (ctypes.c_float * 2)(0.5, 1.0)
     assert lib.mo_awq_clip_losses(null, 0, null, 0, 0, 2, 128, null, 2, ratios, 2, 4, 0, 0, null, null) == OK

@@ -115,14 +115,29 @@ def test_quantize_and_export(tmp_path, name, quant_algo):
 
 
 def test_fp8_overflow_switch():
-    """Values above the amax: NaN with the eager (CPU) semantics, +-amax with the CUDA kernel's."""
-    from modelopt_amd.torch.quantization.tensor_quant import scaled_e4m3_impl
+    """Values above the amax: NaN with the eager (CPU) semantics, +-amax with the CUDA kernel's.
+    The default follows the reference's dispatch on a device tensor (tensor_quant.py:62-90):
+    per-tensor and per-axis amax go to the clamping kernel, amax None or on two dims to the
+    eager cast."""
+    from modelopt_amd.torch.quantization.tensor_quant import fp8_eager, scaled_e4m3_impl
     from oracle import fake_quant
 
     x = torch.tensor([0.5, 1.0, 1.03, 1.04, 2.0, -3.0], dtype=torch.bfloat16)
     amax = torch.tensor(1.0, dtype=torch.bfloat16)
-    assert mtq.get_fp8_overflow_behavior() == "nan"
-    got = scaled_e4m3_impl(x.to(DEV), amax.to(DEV)).cpu()
+    assert mtq.get_fp8_overflow_behavior() == "auto"
+    clamped = torch.tensor([0.5, 1.0, 1.0, 1.0, 1.0, -1.0], dtype=torch.bfloat16)
+    assert torch.equal(scaled_e4m3_impl(x.to(DEV), amax.to(DEV)).cpu(), clamped)
+    per_axis = scaled_e4m3_impl(x.to(DEV).reshape(2, 3), amax.to(DEV).expand(2, 1).contiguous())
+    assert torch.equal(per_axis.cpu().reshape(-1), clamped)
+    assert torch.isnan(scaled_e4m3_impl((x * 300).to(DEV), None)).sum() == 2       # plain cast: eager
+    two_dims = scaled_e4m3_impl(x.to(DEV).reshape(2, 3), amax.to(DEV).expand(2, 3).contiguous())
+    assert torch.isnan(two_dims).sum() == 3                                          # eager fallback
+    assert torch.isnan(fp8_eager(x.to(DEV), amax.to(DEV))).sum() == 3
+    previous = mtq.set_fp8_overflow_behavior("nan")
+    try:
+        got = scaled_e4m3_impl(x.to(DEV), amax.to(DEV)).cpu()
+    finally:
+        mtq.set_fp8_overflow_behavior(previous)
     want = fake_quant.fp8_eager(x, amax)
     assert torch.equal(torch.isnan(got), torch.isnan(want)) and torch.isnan(got).sum() == 3
     assert torch.equal(got[~torch.isnan(got)], want[~torch.isnan(want)])

@@ -494,3 +494,26 @@ def test_reprs_do_not_raise():
     holder.linear, holder.quant_linear = nn.Linear(33, 65), qnn.Linear(33, 65)
     assert "weight_quantizer" in repr(holder)
     assert "MaxCalibrator" in repr(calib.MaxCalibrator(7, 1, False))
+
+
+def test_library_operators_are_registered_with_fake_implementations():
+    """``tensorrt::quantize_op`` / ``tensorrt::dynamic_block_quantize_op`` exist with the
+    reference's schemas (tensor_quant.py:221-273) and trace under fake tensors without a device."""
+    from torch.fx.experimental.proxy_tensor import make_fx
+
+    from modelopt_amd.torch.quantization import tensor_quant as tq
+
+    assert "Tensor amax, int num_bits, int exponent_bits, bool unsigned, bool narrow_range" in str(
+        torch.ops.tensorrt.quantize_op.default._schema)
+    assert "int block_size, Tensor amax" in str(torch.ops.tensorrt.dynamic_block_quantize_op.default._schema)
+    assert hasattr(torch.ops.tensorrt.dynamic_block_quantize_op, "overload")
+
+    def f(x, a):
+        y = tq.quantize_op(x, a, 8, 4, False, False)
+        return tq.dynamic_block_quantize_op(y, 16, a, 4, 2, 8, 4)
+
+    graph = make_fx(f, tracing_mode="fake")(torch.randn(4, 32), torch.tensor(1.0)).graph
+    targets = [str(n.target) for n in graph.nodes if n.op == "call_function"]
+    assert targets == ["tensorrt.quantize_op.default", "tensorrt.dynamic_block_quantize_op.default"]
+    with pytest.raises(RuntimeError, match="GPU memory"):   # the CPU implementation is the loud failure
+        torch.ops.tensorrt.quantize_op(torch.randn(4), torch.tensor(1.0), 8, 0, False, False)

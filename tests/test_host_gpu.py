@@ -83,6 +83,7 @@ def test_quantizer_int8_per_tensor_and_channel(dtype):
     assert_bits_equal(y.cpu(), fake_quant.tensor_quant(x, want_amax, 8, False, False), "per channel")
 
 
+@pytest.mark.usefixtures("cpu_fp8_overflow")
 def test_quantizer_fp8_and_noncontiguous():
     x = _rand((48, 40), torch.bfloat16, 11)
     q = TensorQuantizer(QuantizerAttributeConfig(num_bits=(4, 3)), amax=3.0).to(DEV)
@@ -223,6 +224,25 @@ def test_quantize_max_calibration_amax_matches_oracle(cfg_name):
     assert model.fc2.input_quantizer.amax.numel() == 1 and model.fc2.input_quantizer.amax > 0
     out = model(batches[0].to(DEV))
     assert out.shape == (8, 16, 32) and torch.isfinite(out.float()).all()
+
+
+def test_fp8_model_clamps_an_outlier_above_the_calibrated_amax():
+    """A calibrated FP8_DEFAULT_CFG model (per-tensor amax) and FP8 KV quantizers clamp an input
+    beyond the calibrated range, as the reference's CUDA kernel does (tensor_quant.py:62-90,
+    src/tensor_quant_gpu_fp8.cu:36-47): the output stays finite."""
+    model = _MLP().to(DEV)
+    batches = _batches()
+    mtq.quantize(model, mtq.FP8_DEFAULT_CFG, lambda m: [m(b.to(DEV)) for b in batches])
+    x = batches[0].to(DEV).clone()
+    x[0, 0, 0] = float(model.fc1.input_quantizer.amax) * 4
+    assert torch.isfinite(model(x).float()).all()
+    q = model.fc1.input_quantizer
+    y = q(x)
+    assert torch.isfinite(y.float()).all() and float(y.float().abs().max()) == float(q.amax)
+    kv = TensorQuantizer(QuantizerAttributeConfig(**mtq.FP8_KV_CFG["quant_cfg"]["*[kv]_bmm_quantizer"]),
+                         amax=1.0).to(DEV)
+    t = torch.tensor([[0.5, 1.0, 1.5, -7.0]], dtype=torch.bfloat16, device=DEV)
+    assert torch.equal(kv(t).cpu(), torch.tensor([[0.5, 1.0, 1.0, -1.0]], dtype=torch.bfloat16))
 
 
 def test_quantized_linear_forward_equals_oracle_composition():

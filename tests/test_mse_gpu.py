@@ -59,6 +59,7 @@ CASES = [
 @pytest.mark.parametrize("name,cfg,shape", CASES, ids=[c[0] for c in CASES])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.usefixtures("cpu_fp8_overflow")
 def test_mse_calibrator_against_oracle(name, cfg, shape, dtype, fused, monkeypatch):
     batches = _batches(shape, dtype)
     q = _calibrated_quantizer(cfg, batches)

@@ -131,11 +131,7 @@ def test_fast_path_equals_exact_division_on_large_input():
     x = (0.02 * torch.randn(8192, 8192, generator=g, device=DEV)).to(torch.bfloat16)
     amax = _gpu_amax(x).reshape(())
     p_fast, w_fast, _ = _hip.nvfp4_quantize(x, amax, 16)
-    _hip.set_option(_hip.MO_OPT_FORCE_EXACT, 1)
-    try:
-        p_exact, w_exact, _ = _hip.nvfp4_quantize(x, amax, 16)
-    finally:
-        _hip.set_option(_hip.MO_OPT_FORCE_EXACT, 0)
+    p_exact, w_exact, _ = _hip.nvfp4_quantize(x, amax, 16, flags=_hip.MO_FLAG_FORCE_EXACT)
     assert torch.equal(w_fast.view(torch.uint8), w_exact.view(torch.uint8))
     assert torch.equal(p_fast, p_exact)
     # and against the oracle on a slice the CPU finishes quickly
@@ -145,10 +141,10 @@ def test_fast_path_equals_exact_division_on_large_input():
 
 @pytest.mark.parametrize("dtype,block", [(torch.bfloat16, 16), (torch.bfloat16, 32),
                                          (torch.float16, 16), (torch.float32, 8)])
-def test_block_scale_overflow_follows_the_option(dtype, block):
+def test_block_scale_overflow_follows_the_flag(dtype, block):
     """A per-tensor amax below the real maximum (awq_clip's doing, TQ/model_calib.py:869-876)
     pushes block scales past E4M3's range: by default the scale byte is the NaN that torch's
-    cast gives (TQ/qtensor/nvfp4_tensor.py:84-91); with MO_OPT_SATURATE_BLOCK_SCALE it is 448,
+    cast gives (TQ/qtensor/nvfp4_tensor.py:84-91); with MO_FLAG_SATURATE_BLOCK_SCALE it is 448,
     and the codes follow from that scale.  Single-tensor (tile and generic kernels) and
     multi-tensor launches."""
     x = _rand((256, 512), dtype, 77)
@@ -160,13 +156,10 @@ def test_block_scale_overflow_follows_the_option(dtype, block):
     for saturate in (0, 1):
         wo = (raw.clamp(max=448.0) if saturate else raw).to(torch.float8_e4m3fn)
         po, _, _ = qtensor.nvfp4_quantize(x, block, wo, wsf2)
-        _hip.set_option(_hip.MO_OPT_SATURATE_BLOCK_SCALE, saturate)
-        try:
-            p, w, _ = _hip.nvfp4_quantize(xd, amax.to(DEV), block)
-            if dtype == torch.bfloat16 and block == 16:
-                mp, mw, _ = _hip.Nvfp4QuantizePlan([xd], amax.to(DEV).reshape(1)).run()
-        finally:
-            _hip.set_option(_hip.MO_OPT_SATURATE_BLOCK_SCALE, 0)
+        flags = _hip.MO_FLAG_SATURATE_BLOCK_SCALE if saturate else 0
+        p, w, _ = _hip.nvfp4_quantize(xd, amax.to(DEV), block, flags=flags)
+        if dtype == torch.bfloat16 and block == 16:
+            mp, mw, _ = _hip.Nvfp4QuantizePlan([xd], amax.to(DEV).reshape(1), flags=flags).run()
         assert_bits_equal(w.cpu(), wo, f"wsf saturate={saturate}")
         assert bool(torch.isnan(w.float()).any()) == (not saturate)
         ok = ~torch.isnan(wo.float()).repeat_interleave(block // 2, dim=-1)   # NaN scale: codes of NaN
