@@ -386,7 +386,7 @@ static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
         if (base_ok) {
             const int64_t tiles = (n + MO_ABSMAX_TILE_ELEMS - 1) / MO_ABSMAX_TILE_ELEMS;
             if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
-            absmax_flat_kernel<DT><<<dim3((unsigned)tiles), 256, 0, s>>>(x, n, acc);
+            absmax_flat_kernel<DT><<<dim3((unsigned)tiles), 256, mo::ballast_bytes("absmax_flat_kernel", 36), s>>>(x, n, acc);
             return MO_OK;
         }
         outer = 1; inner = n;  // unaligned base: guarded row path below
@@ -408,9 +408,9 @@ static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
             if (ws < 16) ws = 16;
             wy = (outer + ws - 1) / ws;
             if (wy > 65535) { wy = 65535; ws = (outer + wy - 1) / wy; wy = (outer + ws - 1) / ws; }
-            absmax_cols8_wide_kernel<DT, false><<<dim3((unsigned)wx, (unsigned)wy), 256, 0, s>>>(x, outer, axis, ws, acc);
+            absmax_cols8_wide_kernel<DT, false><<<dim3((unsigned)wx, (unsigned)wy), 256, mo::ballast_bytes("absmax_cols8_wide_kernel", 0), s>>>(x, outer, axis, ws, acc);
         } else if (vec)
-            absmax_cols8_kernel<DT, false><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
+            absmax_cols8_kernel<DT, false><<<dim3((unsigned)gx, (unsigned)gy), 256, mo::ballast_bytes("absmax_cols8_kernel", 0), s>>>(x, outer, axis, slab, acc);
         else
             absmax_cols1_kernel<DT><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, outer, axis, slab, acc);
         return MO_OK;
@@ -423,7 +423,7 @@ static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
         while ((int64_t(1) << lg_l) < row_chunks) ++lg_l;
         const int64_t tiles = (nrows * row_chunks + 1023) / 1024;
         if (tiles <= 0x7FFFFFFF) {
-            absmax_short_rows_kernel<DT><<<dim3((unsigned)tiles), 256, 0, s>>>(
+            absmax_short_rows_kernel<DT><<<dim3((unsigned)tiles), 256, mo::ballast_bytes("absmax_short_rows_kernel", 0), s>>>(
                 x, nrows, axis, lg_l, outer == 1 ? 1 : 0, acc);
             return MO_OK;
         }
@@ -447,9 +447,9 @@ static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
     gy = (row_chunks + seg - 1) / seg;
     const bool aligned = base_ok && (inner % 8 == 0);
     if (aligned)
-        absmax_rows_kernel<DT, true><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, nrows, inner, axis, lg, seg, acc);
+        absmax_rows_kernel<DT, true><<<dim3((unsigned)gx, (unsigned)gy), 256, mo::ballast_bytes("absmax_rows_kernel", 0), s>>>(x, nrows, inner, axis, lg, seg, acc);
     else
-        absmax_rows_kernel<DT, false><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(x, nrows, inner, axis, lg, seg, acc);
+        absmax_rows_kernel<DT, false><<<dim3((unsigned)gx, (unsigned)gy), 256, mo::ballast_bytes("absmax_rows_kernel", 0), s>>>(x, nrows, inner, axis, lg, seg, acc);
     return MO_OK;
 }
 
@@ -498,11 +498,11 @@ static int launch_absmax_cols_staged(const void* x, int64_t outer, int64_t axis,
     slabs = (outer + rows - 1) / rows;
     if (axis >= 2048) {
         const int64_t wx = (axis + 2047) / 2048;
-        absmax_cols8_wide_kernel<DT, true><<<dim3((unsigned)wx, (unsigned)slabs), 256, 0, s>>>(
+        absmax_cols8_wide_kernel<DT, true><<<dim3((unsigned)wx, (unsigned)slabs), 256, mo::ballast_bytes("absmax_cols8_wide_kernel", 0), s>>>(
             x, outer, axis, rows, partial);
     } else {
         const int64_t gx = (axis + 511) / 512;
-        absmax_cols8_kernel<DT, true><<<dim3((unsigned)gx, (unsigned)slabs), 256, 0, s>>>(
+        absmax_cols8_kernel<DT, true><<<dim3((unsigned)gx, (unsigned)slabs), 256, mo::ballast_bytes("absmax_cols8_kernel", 0), s>>>(
             x, outer, axis, rows, partial);
     }
     absmax_fold_partials_kernel<<<dim3((unsigned)((axis + 31) / 32)), 256, 0, s>>>(partial, slabs, axis, acc);
@@ -561,9 +561,9 @@ extern "C" int mo_absmax_multi(const mo_absmax_job* jobs_dev, int njobs,
     const unsigned grid = (unsigned)total_tiles;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case MO_F32: mo::absmax_multi_kernel<MO_F32><<<grid, 256, 0, s>>>(jobs_dev, njobs, tile_job_dev); break;
-        case MO_F16: mo::absmax_multi_kernel<MO_F16><<<grid, 256, 0, s>>>(jobs_dev, njobs, tile_job_dev); break;
-        case MO_BF16: mo::absmax_multi_kernel<MO_BF16><<<grid, 256, 0, s>>>(jobs_dev, njobs, tile_job_dev); break;
+        case MO_F32: mo::absmax_multi_kernel<MO_F32><<<grid, 256, mo::ballast_bytes("absmax_multi_kernel", 0), s>>>(jobs_dev, njobs, tile_job_dev); break;
+        case MO_F16: mo::absmax_multi_kernel<MO_F16><<<grid, 256, mo::ballast_bytes("absmax_multi_kernel", 0), s>>>(jobs_dev, njobs, tile_job_dev); break;
+        case MO_BF16: mo::absmax_multi_kernel<MO_BF16><<<grid, 256, mo::ballast_bytes("absmax_multi_kernel", 0), s>>>(jobs_dev, njobs, tile_job_dev); break;
         default: return MO_ERR_DTYPE;
     }
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;

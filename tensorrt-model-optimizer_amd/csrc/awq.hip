@@ -352,7 +352,7 @@ extern "C" int mo_mul_cols(const void* x, int64_t rows, int64_t k, int dtype, co
         gy = (rows + slab - 1) / slab;
         if (gy > 65535) { gy = 65535; slab = (rows + gy - 1) / gy; gy = (rows + slab - 1) / slab; }
         dim3 grid((unsigned)gx, (unsigned)gy);
-#define CALL(DT) mo::mul_cols8_kernel<DT><<<grid, 256, 0, st>>>(x, rows, k, slab, s, s_dtype, y)
+#define CALL(DT) mo::mul_cols8_kernel<DT><<<grid, 256, mo::ballast_bytes("mul_cols8_kernel", 53), st>>>(x, rows, k, slab, s, s_dtype, y)
         DISPATCH_DT(dtype, CALL)
 #undef CALL
     } else {
@@ -385,8 +385,8 @@ extern "C" int mo_scale_block_int_qdq(const void* x, int64_t rows, int64_t k, in
                      ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)s) & 15u) == 0);
     const unsigned g = (unsigned)blocks;
 #define CALL(DT)                                                                                      \
-    if (vec) mo::scale_block_int_qdq_kernel<DT, true><<<g, 256, 0, st>>>(x, rows, k, s, s_dtype, lg, bound, lo, y); \
-    else mo::scale_block_int_qdq_kernel<DT, false><<<g, 256, 0, st>>>(x, rows, k, s, s_dtype, lg, bound, lo, y)
+    if (vec) mo::scale_block_int_qdq_kernel<DT, true><<<g, 256, mo::ballast_bytes("scale_block_int_qdq_kernel", 0), st>>>(x, rows, k, s, s_dtype, lg, bound, lo, y); \
+    else mo::scale_block_int_qdq_kernel<DT, false><<<g, 256, mo::ballast_bytes("scale_block_int_qdq_kernel", 0), st>>>(x, rows, k, s, s_dtype, lg, bound, lo, y)
     DISPATCH_DT(dtype, CALL)
 #undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
@@ -420,7 +420,7 @@ extern "C" int mo_sq_diff_sum(const void* a, const void* b, int64_t n, int dtype
     // workgroup is worth its atomic, and never more than 1024 of them
     const unsigned g = mo::blocks_for_awq((n + 63) / 64, 1024);
     const int vec = ((((uintptr_t)a | (uintptr_t)b) & 15u) == 0) ? 1 : 0;
-#define CALL(DT) mo::sq_diff_sum_kernel<DT><<<g, 256, 0, st>>>(a, b, n, vec, acc)
+#define CALL(DT) mo::sq_diff_sum_kernel<DT><<<g, 256, mo::ballast_bytes("sq_diff_sum_kernel", 53), st>>>(a, b, n, vec, acc)
     DISPATCH_DT(dtype, CALL)
 #undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
@@ -446,10 +446,10 @@ extern "C" int mo_abs_colsum_staged(const void* x, int64_t rows, int64_t k, int 
     const dim3 grid((unsigned)((k / 8 + 255) / 256), (unsigned)slabs);
 #define CALL(DT)                                                                                  \
     if (blk_amax)                                                                                 \
-        mo::abs_colsum8_kernel<DT, true><<<grid, 256, 0, st>>>(x, rows, k, blk_amax, block_size,  \
+        mo::abs_colsum8_kernel<DT, true><<<grid, 256, mo::ballast_bytes("abs_colsum8_kernel", 0), st>>>(x, rows, k, blk_amax, block_size,  \
                                                                slab, partial);                    \
     else                                                                                          \
-        mo::abs_colsum8_kernel<DT, false><<<grid, 256, 0, st>>>(x, rows, k, blk_amax, block_size, \
+        mo::abs_colsum8_kernel<DT, false><<<grid, 256, mo::ballast_bytes("abs_colsum8_kernel", 0), st>>>(x, rows, k, blk_amax, block_size, \
                                                                 slab, partial)
     DISPATCH_DT(dtype, CALL)
 #undef CALL

@@ -178,10 +178,10 @@ static void launch_block_fp(const void* x, void* y, int64_t rows, int64_t k, int
     const unsigned grid = (unsigned)((total + kBlockFpTileChunks - 1) / kBlockFpTileChunks);
     const bool flat = (k == kp) && ((((uintptr_t)x | (uintptr_t)y) & 15u) == 0);
     if (flat)
-        block_fp_qdq_kernel<DT, FMT, true><<<grid, 256, 0, s>>>(x, y, total, k, cpr, lg_g, scale_fmt,
+        block_fp_qdq_kernel<DT, FMT, true><<<grid, 256, mo::ballast_bytes("block_fp_qdq_kernel", 0), s>>>(x, y, total, k, cpr, lg_g, scale_fmt,
                                                                 global_amax, per_row);
     else
-        block_fp_qdq_kernel<DT, FMT, false><<<grid, 256, 0, s>>>(x, y, total, k, cpr, lg_g, scale_fmt,
+        block_fp_qdq_kernel<DT, FMT, false><<<grid, 256, mo::ballast_bytes("block_fp_qdq_kernel", 0), s>>>(x, y, total, k, cpr, lg_g, scale_fmt,
                                                                  global_amax, per_row);
 }
 
@@ -400,9 +400,9 @@ extern "C" int mo_mxfp4_quantize(const void* x, int64_t n, int dtype, int block_
     const unsigned grid = (unsigned)((chunks + mo::kBlockFpTileChunks - 1) / mo::kBlockFpTileChunks);
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case MO_F32: mo::mxfp4_quantize_kernel<MO_F32><<<grid, 256, 0, s>>>(x, chunks, lg_g, (uint32_t*)packed, scales); break;
-        case MO_F16: mo::mxfp4_quantize_kernel<MO_F16><<<grid, 256, 0, s>>>(x, chunks, lg_g, (uint32_t*)packed, scales); break;
-        case MO_BF16: mo::mxfp4_quantize_kernel<MO_BF16><<<grid, 256, 0, s>>>(x, chunks, lg_g, (uint32_t*)packed, scales); break;
+        case MO_F32: mo::mxfp4_quantize_kernel<MO_F32><<<grid, 256, mo::ballast_bytes("mxfp4_quantize_kernel", 0), s>>>(x, chunks, lg_g, (uint32_t*)packed, scales); break;
+        case MO_F16: mo::mxfp4_quantize_kernel<MO_F16><<<grid, 256, mo::ballast_bytes("mxfp4_quantize_kernel", 0), s>>>(x, chunks, lg_g, (uint32_t*)packed, scales); break;
+        case MO_BF16: mo::mxfp4_quantize_kernel<MO_BF16><<<grid, 256, mo::ballast_bytes("mxfp4_quantize_kernel", 0), s>>>(x, chunks, lg_g, (uint32_t*)packed, scales); break;
         default: return MO_ERR_DTYPE;
     }
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
@@ -420,9 +420,9 @@ extern "C" int mo_mxfp4_dequantize(const uint8_t* packed, const uint8_t* scales,
     const unsigned grid = (unsigned)((chunks + mo::kBlockFpTileChunks - 1) / mo::kBlockFpTileChunks);
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case MO_F32: mo::mxfp4_dequantize_kernel<MO_F32><<<grid, 256, 0, s>>>((const uint32_t*)packed, scales, chunks, lg_g, y); break;
-        case MO_F16: mo::mxfp4_dequantize_kernel<MO_F16><<<grid, 256, 0, s>>>((const uint32_t*)packed, scales, chunks, lg_g, y); break;
-        case MO_BF16: mo::mxfp4_dequantize_kernel<MO_BF16><<<grid, 256, 0, s>>>((const uint32_t*)packed, scales, chunks, lg_g, y); break;
+        case MO_F32: mo::mxfp4_dequantize_kernel<MO_F32><<<grid, 256, mo::ballast_bytes("mxfp4_dequantize_kernel", 0), s>>>((const uint32_t*)packed, scales, chunks, lg_g, y); break;
+        case MO_F16: mo::mxfp4_dequantize_kernel<MO_F16><<<grid, 256, mo::ballast_bytes("mxfp4_dequantize_kernel", 0), s>>>((const uint32_t*)packed, scales, chunks, lg_g, y); break;
+        case MO_BF16: mo::mxfp4_dequantize_kernel<MO_BF16><<<grid, 256, mo::ballast_bytes("mxfp4_dequantize_kernel", 0), s>>>((const uint32_t*)packed, scales, chunks, lg_g, y); break;
         default: return MO_ERR_DTYPE;
     }
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;

@@ -13,6 +13,10 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#ifdef MO_TUNING
+#include <stdio.h>
+#include <stdlib.h>
+#endif
 
 #include "../../include/modelopt_hip.h"
 
@@ -23,6 +27,25 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
+
+// Occupancy cap of the streaming kernels.  A launch asks for `kb` KiB of dynamic LDS that the
+// kernel never touches: a CU has 160 KiB, so floor(160 / kb) workgroups fit on it instead of the
+// 7 or 8 the register budget would allow.  With every lane keeping 4 to 8 16-byte loads in
+// flight, 4 workgroups per CU (about 32 MB in flight over the chip) already cover the memory
+// latency, and more concurrent streams only cost DRAM efficiency: the mixed read/write kernels
+// gain 5 - 11 % from the cap.  0 = no cap.  A build with -DMO_TUNING reads
+// MO_BALLAST_<kernel> / MO_BALLAST_ALL from the environment at every launch (sweeps only).
+inline size_t ballast_bytes(const char* kernel, int kb) {
+#ifdef MO_TUNING
+    char key[160];
+    snprintf(key, sizeof key, "MO_BALLAST_%s", kernel);
+    if (const char* e = getenv(key)) return (size_t)atoi(e) << 10;
+    if (const char* e = getenv("MO_BALLAST_ALL")) return (size_t)atoi(e) << 10;
+#else
+    (void)kernel;
+#endif
+    return (size_t)kb << 10;
+}
 
 __device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
 __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }

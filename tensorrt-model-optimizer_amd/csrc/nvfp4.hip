@@ -571,7 +571,9 @@ extern "C" int mo_nvfp4_quantize(const void* x, int64_t rows, int64_t k, int dty
         const int64_t nblocks = rows * k / 16;
         const int64_t tiles = (nblocks + mo::kTileBlocks - 1) / mo::kTileBlocks;
         if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
-        mo::nvfp4_quantize_fast_kernel<<<(unsigned)tiles, 256, 0, s>>>(
+        // the occupancy cap pays above about a gigabyte; below, the shorter ramp of a full chip wins
+        const int cap_kb = tiles >= 32768 ? 36 : 0;
+        mo::nvfp4_quantize_fast_kernel<<<(unsigned)tiles, 256, mo::ballast_bytes("nvfp4_quantize_fast_kernel", cap_kb), s>>>(
             (const uint16_t*)x, nblocks, tiles, amax, amax_is_wsf2, flags,
             (mo::u32x2*)packed, wsf_out, wsf2_out);
         return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
@@ -598,7 +600,7 @@ extern "C" int mo_nvfp4_dequantize(const uint8_t* packed, const uint8_t* wsf, co
         const int64_t per_tile = 256 * mo::kDequantRounds;
         const int64_t tiles = (total + per_tile - 1) / per_tile;
         if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
-        mo::nvfp4_dequantize_fast_kernel<<<(unsigned)tiles, 256, 0, s>>>(
+        mo::nvfp4_dequantize_fast_kernel<<<(unsigned)tiles, 256, mo::ballast_bytes("nvfp4_dequantize_fast_kernel", 0), s>>>(
             (const uint32_t*)packed, wsf, wsf2, total, (uint16_t*)y);
         return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
     }
@@ -626,10 +628,10 @@ extern "C" int mo_nvfp4_qdq(const void* x, void* y, int64_t rows, int64_t k, int
         const int64_t tiles = (nblocks + mo::kTileBlocks - 1) / mo::kTileBlocks;
         if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
         if (mode == 0)
-            mo::nvfp4_qdq_fast_kernel<0><<<(unsigned)tiles, 256, 0, s>>>(
+            mo::nvfp4_qdq_fast_kernel<0><<<(unsigned)tiles, 256, mo::ballast_bytes("nvfp4_qdq_fast_kernel", 0), s>>>(
                 (const uint16_t*)x, (uint16_t*)y, nblocks, amax, amax_dtype);
         else
-            mo::nvfp4_qdq_fast_kernel<1><<<(unsigned)tiles, 256, 0, s>>>(
+            mo::nvfp4_qdq_fast_kernel<1><<<(unsigned)tiles, 256, mo::ballast_bytes("nvfp4_qdq_fast_kernel", 0), s>>>(
                 (const uint16_t*)x, (uint16_t*)y, nblocks, amax, amax_dtype);
         return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
     }
@@ -648,7 +650,8 @@ extern "C" int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs,
     if (dtype != MO_BF16 || block_size != 16) return MO_ERR_UNSUPPORTED;
     if (njobs == 0 || total_tiles == 0) return MO_OK;
     if (!jobs_dev) return MO_ERR_ARG;
-    mo::nvfp4_quantize_multi_kernel<<<(unsigned)total_tiles, 256, 0, (hipStream_t)stream>>>(
+    const int cap_kb = total_tiles >= 32768 ? 36 : 0;
+    mo::nvfp4_quantize_multi_kernel<<<(unsigned)total_tiles, 256, mo::ballast_bytes("nvfp4_quantize_multi_kernel", cap_kb), (hipStream_t)stream>>>(
         jobs_dev, njobs, tile_job_dev, amax_is_wsf2, flags);
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

@@ -143,7 +143,7 @@ static int launch_qdq(const void* x, void* y, int64_t outer, int64_t axis, int64
         if (slab < 8) slab = 8;
         gy = (outer + slab - 1) / slab;
         if (gy > 65535) { gy = 65535; slab = (outer + gy - 1) / gy; gy = (outer + slab - 1) / slab; }
-        qdq_cols_kernel<DT, FLAG, Op><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, s>>>(
+        qdq_cols_kernel<DT, FLAG, Op><<<dim3((unsigned)gx, (unsigned)gy), 256, mo::ballast_bytes("qdq_cols_kernel", 0), s>>>(
             x, y, outer, axis, slab, amax, amax_dtype, op);
         return MO_OK;
     }
@@ -152,11 +152,11 @@ static int launch_qdq(const void* x, void* y, int64_t outer, int64_t axis, int64
     if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
     const unsigned g = (unsigned)tiles;
     if (axis == 1 || !amax)
-        qdq_kernel<DT, TENSOR, FLAG, Op><<<g, 256, 0, s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
+        qdq_kernel<DT, TENSOR, FLAG, Op><<<g, 256, mo::ballast_bytes("qdq_kernel_tensor", 36), s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
     else if (inner % 8 == 0)
-        qdq_kernel<DT, CHUNK, FLAG, Op><<<g, 256, 0, s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
+        qdq_kernel<DT, CHUNK, FLAG, Op><<<g, 256, mo::ballast_bytes("qdq_kernel", 0), s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
     else
-        qdq_kernel<DT, ELEM, FLAG, Op><<<g, 256, 0, s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
+        qdq_kernel<DT, ELEM, FLAG, Op><<<g, 256, mo::ballast_bytes("qdq_kernel", 0), s>>>(x, y, n, axis, inner, amax, amax_dtype, op);
     return MO_OK;
 }
 

@@ -554,14 +554,14 @@ extern "C" int mo_real_quantize(const void* x, int64_t outer, int64_t axis, int6
         const bool by_row = axis > 1 && ic >= 256 && row_tiles <= 0x7FFFFFFF;
 #define TILE4(DT, VIA, FMT)                                                                       \
     if (axis == 1)                                                                                \
-        mo::real_quantize_tile_kernel<DT, VIA, FMT, mo::kScalePerTensor><<<gt, 256, 0, s>>>(      \
+        mo::real_quantize_tile_kernel<DT, VIA, FMT, mo::kScalePerTensor><<<gt, 256, mo::ballast_bytes("real_quantize_tile_kernel", 0), s>>>(      \
             x, chunks, axis, ic, 1, scale, scale_dtype, (mo::u32x2*)out);                         \
     else if (by_row)                                                                              \
         mo::real_quantize_tile_kernel<DT, VIA, FMT, mo::kScalePerRowTile>                         \
-            <<<(unsigned)row_tiles, 256, 0, s>>>(x, chunks, axis, ic, tpr, scale, scale_dtype,    \
+            <<<(unsigned)row_tiles, 256, mo::ballast_bytes("real_quantize_tile_kernel", 0), s>>>(x, chunks, axis, ic, tpr, scale, scale_dtype,    \
                                                  (mo::u32x2*)out);                                \
     else                                                                                          \
-        mo::real_quantize_tile_kernel<DT, VIA, FMT, mo::kScalePerChunk><<<gt, 256, 0, s>>>(       \
+        mo::real_quantize_tile_kernel<DT, VIA, FMT, mo::kScalePerChunk><<<gt, 256, mo::ballast_bytes("real_quantize_tile_kernel", 0), s>>>(       \
             x, chunks, axis, ic, 1, scale, scale_dtype, (mo::u32x2*)out)
 #define TILE3(DT, VIA) \
     if (format == MO_FMT_E4M3) { TILE4(DT, VIA, 0); } else { TILE4(DT, VIA, 1); }
@@ -612,14 +612,14 @@ extern "C" int mo_real_dequantize(const uint8_t* q, int64_t outer, int64_t axis,
         const bool by_row = axis > 1 && ic >= 256 && row_tiles <= 0x7FFFFFFF;
 #define TILE3(DT, FMT)                                                                            \
     if (axis == 1)                                                                                \
-        mo::real_dequantize_tile_kernel<DT, FMT, mo::kScalePerTensor><<<gt, 256, 0, s>>>(         \
+        mo::real_dequantize_tile_kernel<DT, FMT, mo::kScalePerTensor><<<gt, 256, mo::ballast_bytes("real_dequantize_tile_kernel", 36), s>>>(         \
             (const mo::u32x2*)q, chunks, axis, ic, 1, scale, scale_dtype, y);                     \
     else if (by_row)                                                                              \
         mo::real_dequantize_tile_kernel<DT, FMT, mo::kScalePerRowTile>                            \
-            <<<(unsigned)row_tiles, 256, 0, s>>>((const mo::u32x2*)q, chunks, axis, ic, tpr,      \
+            <<<(unsigned)row_tiles, 256, mo::ballast_bytes("real_dequantize_tile_kernel", 36), s>>>((const mo::u32x2*)q, chunks, axis, ic, tpr,      \
                                                  scale, scale_dtype, y);                          \
     else                                                                                          \
-        mo::real_dequantize_tile_kernel<DT, FMT, mo::kScalePerChunk><<<gt, 256, 0, s>>>(          \
+        mo::real_dequantize_tile_kernel<DT, FMT, mo::kScalePerChunk><<<gt, 256, mo::ballast_bytes("real_dequantize_tile_kernel", 36), s>>>(          \
             (const mo::u32x2*)q, chunks, axis, ic, 1, scale, scale_dtype, y)
 #define CALL(DT) \
     if (format == MO_FMT_E4M3) { TILE3(DT, 0); } else { TILE3(DT, 1); }
@@ -655,7 +655,7 @@ extern "C" int mo_int4_block_quantize(const void* x, int64_t n, int64_t block_si
     if (shift >= 0 && n % block_size == 0 && (((uintptr_t)x & 15u) == 0) &&
         (((uintptr_t)packed & 3u) == 0) && tiles <= 0x7FFFFFFF) {
 #define CALL(DT)                                                                          \
-    mo::int4_block_quantize_tile_kernel<DT><<<(unsigned)tiles, 256, 0, s>>>(              \
+    mo::int4_block_quantize_tile_kernel<DT><<<(unsigned)tiles, 256, mo::ballast_bytes("int4_block_quantize_tile_kernel", 32), s>>>(              \
         x, n / 8, 1 << shift, shift, scales, scales_given, (uint32_t*)packed)
         DISPATCH_DT(dtype, CALL)
 #undef CALL
@@ -682,7 +682,7 @@ extern "C" int mo_int4_block_dequantize(const uint8_t* packed, int64_t nbytes, i
     if (shift >= 0 && nbytes % 4 == 0 && (((uintptr_t)y & 15u) == 0) &&
         (((uintptr_t)packed & 3u) == 0) && tiles <= 0x7FFFFFFF) {
 #define CALL(DT)                                                                          \
-    mo::int4_block_dequantize_tile_kernel<DT><<<(unsigned)tiles, 256, 0, s>>>(            \
+    mo::int4_block_dequantize_tile_kernel<DT><<<(unsigned)tiles, 256, mo::ballast_bytes("int4_block_dequantize_tile_kernel", 0), s>>>(            \
         (const uint32_t*)packed, nbytes / 4, shift, scales, y)
         DISPATCH_DT(dtype, CALL)
 #undef CALL
@@ -711,7 +711,7 @@ extern "C" int mo_int4_pack_rows(const void* w, int64_t batch, int64_t n_rows, i
         const int64_t items = (rows >> 1) * (k / 8), tiles = (items + per_tile - 1) / per_tile;
         if (tiles <= 0x7FFFFFFF) {
 #define CALL(DT)                                                                      \
-    mo::int4_pack_rows_tile_kernel<DT><<<(unsigned)tiles, 256, 0, s>>>(               \
+    mo::int4_pack_rows_tile_kernel<DT><<<(unsigned)tiles, 256, mo::ballast_bytes("int4_pack_rows_tile_kernel", 0), s>>>(               \
         w, rows >> 1, k / 8, block_size / 8, ws, (mo::u32x2*)out)
             DISPATCH_DT(dtype, CALL)
 #undef CALL

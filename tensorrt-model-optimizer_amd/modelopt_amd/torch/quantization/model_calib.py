@@ -20,6 +20,7 @@ from . import calib
 from .calib.max import MaxCalibrator
 from .conversion import set_quantizer_by_cfg_context
 from .nn import QuantModule, SequentialQuantizer, TensorQuantizer
+from .nn.modules.tensor_quantizer import calibration_pass
 from .utils import all_valid_scales, is_quantized_linear
 
 __all__ = ["max_calibrate", "smoothquant", "awq", "awq_lite", "enable_stats_collection",
@@ -82,7 +83,8 @@ def max_calibrate(model: nn.Module, forward_loop=None, distributed_sync=True):
     if forward_loop is None:
         weight_only_quantize(model)
     else:
-        forward_loop(model)
+        with calibration_pass():
+            forward_loop(model)
     finish_stats_collection(model)
 
 
@@ -379,7 +381,8 @@ def awq_clip(model: nn.Module, forward_loop, max_co_batch_size: int = 1024,
             patched.append(module)
     print("awq_clip: Estimating parameters...")
     enable_stats_collection(model)
-    forward_loop(model)
+    with calibration_pass():
+        forward_loop(model)
     max_calibrate(model, lambda m: None)
     for module in patched:
         helper = module.awq_clip
@@ -664,7 +667,8 @@ def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: boo
     _AWQLiteHelper.cache_mode = True
     print("awq_lite: Caching activation statistics...")
     enable_stats_collection(model)
-    forward_loop(model)
+    with calibration_pass():
+        forward_loop(model)
     max_calibrate(model, lambda model: None)
 
     for name, module in model.named_modules():

@@ -24,6 +24,22 @@ from ...tensor_quant import dynamic_block_quant, fake_tensor_quant, scaled_e4m3
 
 __all__ = ["SequentialQuantizer", "TensorQuantizer"]
 
+# [id of the calibration pass in progress, or 0]; the weight abs-max cache is only valid inside one
+_CALIBRATION_PASS = [0]
+_PASS_COUNTER = [0]
+
+
+@contextlib.contextmanager
+def calibration_pass():
+    """Marks one ``forward_loop`` run by the package's calibration drivers: within it a weight
+    that has not changed is reduced once, not once per forward."""
+    _PASS_COUNTER[0] += 1
+    previous, _CALIBRATION_PASS[0] = _CALIBRATION_PASS[0], _PASS_COUNTER[0]
+    try:
+        yield
+    finally:
+        _CALIBRATION_PASS[0] = previous
+
 
 class TensorQuantizer(nn.Module):
     """Quantises (fake or real) and calibrates one tensor.
@@ -535,19 +551,25 @@ class TensorQuantizer(nn.Module):
             outputs = self._reset_to_original_shape(outputs)
         return outputs
 
-    # A weight is shown to its quantizer on every forward of the calibration loop.  Its abs-max
-    # cannot change while the parameter is untouched, so a repeat of the same parameter (same
-    # storage, same version counter, same scale) is not reduced again; the running maximum is
-    # idempotent, so the calibrated amax is identical.  ``reset_amax`` forgets the parameter.
+    # A weight is shown to its quantizer on every forward of a calibration loop.  Inside one
+    # ``forward_loop`` run by this package (``calibration_pass``) its abs-max cannot change while
+    # the parameter is untouched, so a repeat of the same parameter (same storage, same version
+    # counter, same scale) is not reduced again; the running maximum is idempotent, so the
+    # calibrated amax is identical.  Outside such a pass -- a caller driving ``enable_calib`` and
+    # forwards by hand, who may also write ``weight.data`` in place, which no version counter
+    # sees -- every forward reduces again, as the reference does.  Calibrators other than the
+    # plain MaxCalibrator (history tracking, user classes) always collect.
     cache_weight_amax = True
 
     def _seen_this_parameter(self, source) -> bool:
-        if not (self.cache_weight_amax and isinstance(source, nn.Parameter)):
+        if not (self.cache_weight_amax and _CALIBRATION_PASS[0] and isinstance(source, nn.Parameter)):
+            return False
+        cal = self._calibrator
+        if type(cal) is not calib.MaxCalibrator or cal._track_amax:
             return False
         pqs = self.pre_quant_scale
-        key = (source.data_ptr(), source._version, tuple(source.shape), source.dtype,
-               None if pqs is None else (pqs.data_ptr(), pqs._version))
-        cal = self._calibrator
+        key = (_CALIBRATION_PASS[0], source.data_ptr(), source._version, tuple(source.shape),
+               source.dtype, None if pqs is None else (pqs.data_ptr(), pqs._version))
         if getattr(cal, "_seen_parameter", None) == key and getattr(cal, "_acc", None) is not None:
             return True
         cal._seen_parameter = key

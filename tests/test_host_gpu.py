@@ -262,27 +262,58 @@ def test_quantized_linear_forward_equals_oracle_composition():
     assert torch.allclose(y.cpu().float(), F.linear(xq, wq, ref.fc1.bias).float(), rtol=2e-2, atol=2e-2)
 
 
-def test_weight_amax_is_cached_across_forwards():
+def test_weight_amax_is_cached_inside_a_calibration_pass_only():
+    from modelopt_amd.torch.quantization import model_calib
+    from modelopt_amd.torch.quantization.nn.modules.tensor_quantizer import calibration_pass
+
     model = _MLP().to(DEV)
     mtq.replace_quant_module(model)
     mtq.set_quantizer_by_cfg(model, mtq.model_quant._validated(mtq.INT8_DEFAULT_CFG)[0])
-    from modelopt_amd.torch.quantization import model_calib
     model_calib.enable_stats_collection(model)
     calls = []
     cal = model.fc1.weight_quantizer._calibrator
     orig = cal.collect
     cal.collect = lambda x: (calls.append(1), orig(x))[1]
-    for b in _batches(4):
+    with calibration_pass():
+        for b in _batches(4):
+            model(b.to(DEV))
+        assert len(calls) == 1  # the unchanged weight was reduced once, not once per forward
+        with torch.no_grad():
+            model.fc1.weight.mul_(0.5)  # an in-place update bumps the version
+        model(_batches(1)[0].to(DEV))
+        assert len(calls) == 2
+    for b in _batches(2):  # outside a pass every forward reduces, as in the reference
         model(b.to(DEV))
-    assert len(calls) == 1  # the unchanged weight was reduced once, not once per forward
-    model.fc1.weight.data.mul_(2)  # touching .data does not bump the version ...
-    model.fc1.weight_quantizer.reset_amax()  # ... so callers reset, as the reference's folding does
-    model(_batches(1)[0].to(DEV))
-    assert len(calls) == 2
-    with torch.no_grad():
-        model.fc1.weight.mul_(0.5)  # an in-place update bumps the version
-    model(_batches(1)[0].to(DEV))
-    assert len(calls) == 3
+    assert len(calls) == 4
+    model_calib.finish_stats_collection(model)
+
+
+def test_recalibration_after_an_in_place_data_write_sees_the_new_weight():
+    """``weight.data.mul_(2)`` bumps no version counter; a second calibration without
+    ``reset_amax`` still re-reduces the weight and the running maximum doubles, as in the
+    reference (every forward collects, quant_module.py:148-169)."""
+    ref = _MLP()
+    model = copy.deepcopy(ref).to(DEV)
+    batches = _batches(2)
+    loop = lambda m: [m(b.to(DEV)) for b in batches]  # noqa: E731
+    mtq.quantize(model, mtq.FP8_DEFAULT_CFG, loop)
+    first = model.fc1.weight_quantizer.amax.clone()
+    assert_bits_equal(first.cpu().reshape(()), reduce.reduce_amax(ref.fc1.weight.data), "first amax")
+    model.fc1.weight.data.mul_(2)
+    mtq.calibrate(model, "max", loop)
+    assert_bits_equal(model.fc1.weight_quantizer.amax.cpu().reshape(()),
+                      reduce.reduce_amax(ref.fc1.weight.data * 2), "amax after the write")
+    # a history-tracking calibrator sees every forward
+    from modelopt_amd.torch.quantization import calib as calib_mod, model_calib
+    from modelopt_amd.torch.quantization.nn.modules.tensor_quantizer import calibration_pass
+
+    q = model.fc1.weight_quantizer
+    q._calibrator = calib_mod.MaxCalibrator(q._calibrator._num_bits, q._calibrator._axis,
+                                            q._calibrator._unsigned, track_amax=True)
+    model_calib.enable_stats_collection(model)
+    with calibration_pass():
+        loop(model)
+    assert len(q._calibrator.amaxs) == len(batches)
     model_calib.finish_stats_collection(model)
 
 
