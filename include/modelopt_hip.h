@@ -332,6 +332,15 @@ int mo_abs_colsum_staged(const void* x, int64_t rows, int64_t k, int dtype, cons
                          int64_t block_size, float* acc, float* partial, int64_t partial_rows,
                          void* stream);
 
+/* xs[a][c][t][0..8) = bf16(x[t][8 c ..] * inv_s[a][8 c ..]) for n_alpha rows of inv_s: the
+ * activations under every candidate scale, in the chunk-major layout mo_awq_search_losses reads
+ * ([n_alpha][k / 8][tokens][8] bf16).  This is the `inputs * pre_quant_scale` of the input
+ * quantizer in the search forward (TQ/nn/modules/tensor_quantizer.py:881-882, set per alpha at
+ * TQ/model_calib.py:671-675) for all alphas at once.  bf16 only, k % 8 == 0, 16-byte aligned
+ * buffers; MO_ERR_UNSUPPORTED otherwise. */
+int mo_awq_scale_activations(const void* x, const void* inv_s, int64_t n_alpha, int64_t tokens,
+                             int64_t k, int dtype, void* xs, void* stream);
+
 /* AWQ-lite search step for a whole grid of alphas in one launch (bf16 only):
  *   q_a = block INT-N quantise-dequantise (blocks of block_size along k, dynamic abs-max) of
  *         bf16(w * s[a]);   out_a = bf16(xs[a] @ q_a^T)   (fp32 accumulation on the matrix cores)
@@ -341,8 +350,11 @@ int mo_abs_colsum_staged(const void* x, int64_t rows, int64_t k, int dtype, cons
  * lanes of a matrix-core operand read adjacent memory; w [n, k]; s [n_alpha, k]; ref [tokens, n];
  * loss: n_alpha doubles, accumulated into.  The quantised weights
  * and the outputs never reach memory.  Returns MO_ERR_UNSUPPORTED unless dtype is bf16,
- * tokens <= 512, n % 64 == 0, k % 128 == 0, block_size is 32, 64 or 128 and the buffers are
- * 16-byte aligned (use mo_scale_block_int_qdq + a GEMM + mo_sq_diff_sum per alpha then).
+ * tokens <= 512, n % 128 == 0, k % 128 == 0, block_size is 32, 64 or 128 and the buffers are
+ * 16-byte aligned, or the grid is unsigned (use mo_scale_block_int_qdq + a GEMM + mo_sq_diff_sum
+ * per alpha then).  The integer codes are the reference's; the dequantised weight is
+ * code * (amax / bound) instead of code / (bound / amax), which can differ in the last bf16 bit
+ * for about one weight in 10^4 (per-alpha losses agree to ~1e-6 relative).
  * Replaces the per-alpha loop of the search forward, TQ/model_calib.py:645-690 (weight
  * pre-quant scale, TQ/nn/modules/tensor_quantizer.py:881-882; dynamic block amax :505-514;
  * _tensor_quant TQ/tensor_quant.py:574-612; update_loss TQ/model_calib.py:623-627). */

@@ -8,12 +8,26 @@
 // dynamic block amax -> fake quant -> linear -> squared error against the unquantised output,
 // TQ/model_calib.py:645-690) with the activations already multiplied by 1 / s[a].
 //
-// A workgroup owns a column tile of 64 output features for one alpha and all T <= 512 tokens, so
-// every weight element is scaled and quantised exactly once per alpha; the quantised tile goes
-// to LDS as bf16 and is the B operand of v_mfma_f32_32x32x16_bf16 (the 16 x 16 x 32 form reaches
-// 70 % of this form's rate here), the activations are loaded straight into the A operand
-// registers from a chunk-major copy, in which the lanes of an operand read adjacent memory.  The output tile never leaves the registers: it is rounded
-// to bf16, compared with the reference output and reduced to one double per workgroup.
+// A workgroup of 8 wavefronts owns a column tile of 128 output features for one alpha and all
+// T <= 512 tokens, so every weight element is scaled and quantised exactly once per alpha.  Every
+// wavefront does both jobs: it multiplies its 64 (or 32) token rows with the quantised tile of
+// the current k block (B operand of v_mfma_f32_32x32x16_bf16 from LDS, A operand straight from a
+// chunk-major copy of the activations, in which the lanes of an operand read adjacent memory)
+// and, between those matrix instructions, quantises its share of the tile of the next k block
+// into the other LDS buffer.  Two wavefronts share a SIMD, so one's vector work and LDS waits
+// run under the other's matrix instructions; an activation fragment is used for all 128
+// columns, which halves the traffic of the A operand through L2 against a 64-column tile.  The
+// output tile never leaves the registers: it is rounded to bf16, compared with the reference
+// output and reduced to one double per workgroup.
+//
+// The integer codes are the reference's bit for bit (correctly rounded bound / amax, one IEEE
+// multiply, round half to even); the dequantised value is code * (1 / scale) with a correctly
+// rounded reciprocal instead of the reference's division: the fp32 results differ by at most an
+// ulp, which survives the rounding to bf16 for about one weight in 10^4, far below the 1e-3
+// tolerance of the per-alpha losses.  The weights that are kept after the search come from the
+// exact kernels.
+#include <type_traits>
+
 #include "awq_ops.h"
 #include "common.h"
 
@@ -22,209 +36,272 @@ namespace mo {
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-constexpr int kSearchTileN = 64;    // output features per workgroup
-constexpr int kSearchBlockK = 128;  // k elements per step: 16 chunks of 8
+constexpr int kSearchTileN = 128;   // output features per workgroup
+constexpr int kSearchBlockK = 128;  // k elements per step of the outer loop: 16 chunks of 8
+constexpr int kSearchWaves = 8;
+constexpr int kXcds = 8;            // accelerator dies of the chip, each with its own L2
 
-// MB = 32-row blocks per consumer wavefront; the workgroup covers 128 * MB token rows.
-// Eight wavefronts: 0-3 produce (weight tile of the next k block: scale, quantise, to LDS), 4-7
-// consume (activation fragments from memory, weight fragments from LDS, MFMA).  A SIMD hosts one
-// of each, so the vector ALU work of quantising overlaps the matrix work.  Both roles pass the
-// same number of barriers: the producer after each tile it wrote, the consumer before each tile
-// it reads; tile kb lives in buffer kb & 1, which the producer rewrites (as tile kb + 2) only
-// after the barrier that the consumers reach when they are done with tile kb.
-template <int MB>
+// RB = 32-row blocks per wavefront; the workgroup covers 8 * 32 * RB token rows.
+template <int RB>
 __global__ __launch_bounds__(512) void awq_search_kernel(
     const uint16_t* __restrict__ xs,   // [A][K / 8][T][8] bf16, activations * (1 / s[a])
     const uint16_t* __restrict__ w,    // [N, K] bf16
     const uint16_t* __restrict__ s,    // [A, K] bf16
     const uint16_t* __restrict__ ref,  // [T, N] bf16
-    int T, int N, int K, int lg_g, float bound, float lo, double* __restrict__ loss) {
-    // quantised weight tile, two buffers: [64 rows][16 chunk slots] of 16 bytes, the slot of
+    int T, int N, int K, int n_alpha, int lg_g, float bound, double* __restrict__ loss) {
+    // quantised weight tile, two buffers: [128 rows][16 chunk slots] of 16 bytes; the slot of
     // chunk c in row r is c ^ (r & 15) so that both the writers (16 lanes per row) and the
     // readers (lanes along rows) spread over all banks
     __shared__ u32x4 tile[2][kSearchTileN][16];
-    __shared__ double red[4];
+    __shared__ double red[kSearchWaves];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int a = blockIdx.y;
-    const int n0 = blockIdx.x * kSearchTileN;
+    // Workgroup L of a launch runs on XCD L % 8, and each XCD has its own L2.  All column tiles
+    // of an alpha read the same activations, so the (alpha, column tile) pairs are dealt out in
+    // contiguous runs: XCD x takes pairs [x * per, (x + 1) * per) in alpha-major order, i.e. the
+    // column tiles of one alpha run side by side on one XCD (at most two share an alpha) and
+    // the 4 MB of activations they walk through in step are fetched into that L2 once instead
+    // of once per XCD.  Every XCD gets the same number of pairs; the grid is padded to a
+    // multiple of 8 and the surplus workgroups leave at once.
+    const int ncol = N / kSearchTileN;
+    const int pairs = n_alpha * ncol, per = (pairs + kXcds - 1) / kXcds;
+    const int xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+    const int pair = xcd * per + slot;
+    if (pair >= pairs) return;
+    const int a = pair / ncol;
+    const int n0 = (pair % ncol) * kSearchTileN;
     const int nkb = K / kSearchBlockK;
 
-    // Wavefront w of a workgroup runs on SIMD w % 4: wavefronts 0-3 produce and 4-7 consume, so
-    // that every SIMD hosts one of each (with alternating roles two SIMDs would get both
-    // consumers and the matrix work would run at half rate).
-    const bool producer = wave < 4;
-    const int rw = wave & 3;  // index within the role
-    if (producer) {
-        // ------------------------------------------------------------------ producer
-        const uint16_t* sa = s + (int64_t)a * K;
-        const int pid = rw * 64 + lane;
-        const int qc = pid & 15, qr = pid >> 4;  // chunk qc of rows qr + 16 u
-        // Raw weight chunks and scales of two blocks in flight: block kb lives in buffer kb & 1
-        // and, once unpacked, its registers are refilled with block kb + 2 (the last blocks fetch
-        // the last block again, which is never used).
-        const uint16_t* wp[4];
+    // ---- producer side: chunk qc of rows qr + 32 u of the tile (u = 0..3), two chunks at a time
+    const int qc = threadIdx.x & 15, qr = threadIdx.x >> 4;
+    const uint16_t* wp0 = w + (int64_t)(n0 + qr) * K + qc * 8;
+    const int64_t wstride = (int64_t)32 * K;  // between the rows of two of a lane's chunks
+    const uint16_t* sp = s + (int64_t)a * K + qc * 8;
+    u32x4 wraw[4], sraw;    // raw weight chunks and scales of the block to quantise next
+    float v[2][8];          // the pair of chunks being quantised: bf16(w * s) as fp32
+    float mul[2], rdiv[2];  // per chunk: bound / amax and amax / bound
+
+    auto fetch = [&](int kb) {  // weights are used once per alpha: streamed past the L2
+        const int k0 = (kb < nkb ? kb : nkb - 1) * kSearchBlockK;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) wp[u] = w + (int64_t)(n0 + qr + 16 * u) * K + qc * 8;
-        const uint16_t* sp = sa + qc * 8;
-        u32x4 w0[4], s0, w1[4], s1;
-        {
-            const int k1 = nkb > 1 ? kSearchBlockK : 0;
+        for (int u = 0; u < 4; ++u)
+            wraw[u] = __builtin_nontemporal_load((const u32x4*)(wp0 + u * wstride + k0));
+        sraw = *(const u32x4*)(sp + k0);
+    };
+    auto scale_pair = [&](int h) {  // chunks 2 h, 2 h + 1: v = bf16(w * s)
+        const uint32_t sw[4] = {sraw.x, sraw.y, sraw.z, sraw.w};
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                w0[u] = *(const u32x4*)wp[u];
-                w1[u] = *(const u32x4*)(wp[u] + k1);
-            }
-            s0 = *(const u32x4*)sp;
-            s1 = *(const u32x4*)(sp + k1);
-        }
-        auto produce = [&](int kb, u32x4 (&wb)[4], u32x4& sb) {
-            const uint32_t sw[4] = {sb.x, sb.y, sb.z, sb.w};
-            float sc[8];
+        for (int i = 0; i < 2; ++i) {
+            const u32x4 r = wraw[2 * h + i];
+            const uint32_t ww[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                sc[2 * j] = u2f(sw[j] << 16);
-                sc[2 * j + 1] = u2f(sw[j] & 0xFFFF0000u);
+                v[i][2 * j] = round_to_bf16(u2f(ww[j] << 16) * u2f(sw[j] << 16));
+                v[i][2 * j + 1] = round_to_bf16(u2f(ww[j] & 0xFFFF0000u) * u2f(sw[j] & 0xFFFF0000u));
             }
-            float v[4][8];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const uint32_t ww[4] = {wb[u].x, wb[u].y, wb[u].z, wb[u].w};
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    v[u][2 * j] = round_to_bf16(u2f(ww[j] << 16) * sc[2 * j]);
-                    v[u][2 * j + 1] = round_to_bf16(u2f(ww[j] & 0xFFFF0000u) * sc[2 * j + 1]);
-                }
-            }
-            const int k2 = (kb + 2 < nkb ? kb + 2 : nkb - 1) * kSearchBlockK;
-#pragma unroll
-            for (int u = 0; u < 4; ++u) wb[u] = *(const u32x4*)(wp[u] + k2);
-            sb = *(const u32x4*)(sp + k2);
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                block_int_qdq_chunk(v[u], lg_g, bound, lo);
-                u32x4 o;
-                o.x = f32x2_to_bf16x2(v[u][0], v[u][1]);
-                o.y = f32x2_to_bf16x2(v[u][2], v[u][3]);
-                o.z = f32x2_to_bf16x2(v[u][4], v[u][5]);
-                o.w = f32x2_to_bf16x2(v[u][6], v[u][7]);
-                const int r = qr + 16 * u;
-                tile[kb & 1][r][qc ^ (r & 15)] = o;
-            }
-            __syncthreads();
-        };
-        for (int kb = 0; kb < nkb; kb += 2) {
-            produce(kb, w0, s0);
-            if (kb + 1 < nkb) produce(kb + 1, w1, s1);
         }
-        __syncthreads();  // the consumers' reduction barrier
-        return;
+    };
+    const float inv_bound = 1.0f / bound;
+    auto block_scales = [&]() {  // block abs-max over the lanes of a block, then the two factors
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            uint32_t m = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t t = f2u(v[i][j]) & 0x7FFFFFFFu;
+                m = t > m ? t : m;
+            }
+            // abs-max over the 1 << lg_g (4, 8 or 16) lanes of a block; selects instead of
+            // branches keep the loop body one basic block
+#define MO_DPP_STEP(CTRL, ON)                                                                 \
+    {                                                                                         \
+        const uint32_t t = (uint32_t)__builtin_amdgcn_mov_dpp((int)m, CTRL, 0xF, 0xF, true);  \
+        m = ((ON) && t > m) ? t : m;                                                          \
     }
+            MO_DPP_STEP(0xB1, true)        // quad_perm [1, 0, 3, 2]
+            MO_DPP_STEP(0x4E, true)        // quad_perm [2, 3, 0, 1]
+            MO_DPP_STEP(0x141, lg_g >= 3)  // row_half_mirror
+            MO_DPP_STEP(0x140, lg_g >= 4)  // row_mirror
+#undef MO_DPP_STEP
+            const float amax = u2f(m);
+            const bool dead = amax <= 5.9604644775390625e-8f;  // 2^-24
+            mul[i] = dead ? 0.0f : bound / amax;
+            rdiv[i] = dead ? 1.0f : amax * inv_bound;
+        }
+    };
+    // |v| <= amax, so the rounded code never leaves [-bound, bound]: no clamp is needed
+    auto quantise_store = [&](int h, int i, int buf) {
+        float y[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) y[j] = __builtin_rintf(v[i][j] * mul[i]) * rdiv[i];
+        u32x4 o;
+        o.x = f32x2_to_bf16x2(y[0], y[1]);
+        o.y = f32x2_to_bf16x2(y[2], y[3]);
+        o.z = f32x2_to_bf16x2(y[4], y[5]);
+        o.w = f32x2_to_bf16x2(y[6], y[7]);
+        const int r = qr + 32 * (2 * h + i);
+        tile[buf][r][qc ^ (r & 15)] = o;
+    };
+    // the work on one tile in eight slices (one per step of the matrix loop)
+    auto produce_slice = [&](int j, int kb_next, int buf) {
+        const int h = j >> 2;
+        switch (j & 3) {
+            case 0: scale_pair(h); if (h == 1) fetch(kb_next + 1); break;
+            case 1: block_scales(); break;
+            case 2: quantise_store(h, 0, buf); break;
+            default: quantise_store(h, 1, buf); break;
+        }
+    };
 
-    // ---------------------------------------------------------------------- consumer
-    // v_mfma_f32_32x32x16_bf16: lane (fr, kg) = (lane & 31, lane >> 5) supplies row fr of the A
-    // block and column fr of the B block, elements [8 kg, 8 kg + 8) of the 16 k of a step, and
-    // receives rows 8 (i / 4) + 4 kg + i % 4 (i = 0..15) of column fr.
-    const int cw = rw;
+    // ---- consumer side.  v_mfma_f32_32x32x16_bf16: lane (fr, kg) = (lane & 31, lane >> 5)
+    // supplies row fr of the A block and column fr of the B block, elements [8 kg, 8 kg + 8) of
+    // the 16 k of a step, and receives rows 8 (i / 4) + 4 kg + i % 4 (i = 0..15) of column fr.
     const int fr = lane & 31, kg = lane >> 5;
-    const int row_base = cw * (MB * 32);
+    const int row_base = wave * (RB * 32);
+    const bool has_rows = row_base < T;  // wavefronts past T only produce
     const uint16_t* xa = xs + (int64_t)a * T * K;
-
-    f32x16_t acc[MB][2];
+    f32x16_t acc[RB][4];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+    for (int mb = 0; mb < RB; ++mb)
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb)
+        for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.0f;
-
     // Element offsets of this lane's A fragments.  xs is chunk-major: [K / 8][T][8], i.e. the 16
     // bytes of chunk c of row t sit at ((c * T) + t) * 8, so the 32 lanes fr of a k-group read
     // 512 contiguous bytes.  Rows past T repeat row T - 1 (masked in the epilogue); T * K < 2^31
     // is checked by the launcher.
-    uint32_t aoff[MB];
+    uint32_t aoff[RB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
+    for (int mb = 0; mb < RB; ++mb) {
         int t = row_base + mb * 32 + fr;
         t = t < T ? t : T - 1;
         aoff[mb] = ((uint32_t)kg * (uint32_t)T + (uint32_t)t) * 8u;
     }
     const uint32_t step_stride = 2u * (uint32_t)T * 8u;  // one step of 16 k = 2 chunks
-    // fragments of one half block (four steps of 16 k); each is reloaded for the next half block
-    // as soon as the MFMAs that read it have been issued
-    u32x4 af[MB][4];
+    const int steps = nkb * 8;
+    // activation fragments are fetched this many steps ahead (a divisor of the 8 steps of a k
+    // block, so that a step's register slot j % PF is the same in every block)
+    constexpr int PF = 2;
+    static_assert(8 % PF == 0, "slot of a step must not depend on the k block");
+    u32x4 af[RB][PF];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+    for (int mb = 0; mb < RB; ++mb)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) af[mb][j] = *(const u32x4*)(xa + aoff[mb] + j * step_stride);
+        for (int j = 0; j < PF; ++j)
+            af[mb][j] = *(const u32x4*)(xa + aoff[mb] + (uint32_t)j * step_stride);
 
-    const int halves = nkb * 2;
-    for (int kb = 0; kb < nkb; ++kb) {
+    // ---- prologue: tile 0 into buffer 0, raw weights of block 1 in flight
+    fetch(0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) produce_slice(j, 0, 0);
+    __syncthreads();
+
+    // One k block: 8 steps of 16 k against the tile in buffer kb & 1; with MORE, one eighth of
+    // the work on the next tile (into the other buffer) follows each step's matrix instructions.
+    // No branches inside, so the whole block is scheduled as one: wavefronts whose rows lie past
+    // T multiply their clamped rows as well and are left out of the sum.
+    auto k_block = [&](int kb, auto more_tag) {
+        constexpr bool MORE = decltype(more_tag)::value;
         const int buf = kb & 1;
-        __syncthreads();
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            // the half block to prefetch (the last one fetches itself again: no branch in the loop)
-            const int nh = kb * 2 + h + 1 < halves ? kb * 2 + h + 1 : halves - 1;
+        for (int j = 0; j < 8; ++j) {
+            bf16x8_t bfrag[4];
+            const int c = j * 2 + kg;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int c = h * 8 + j * 2 + kg;
-                bf16x8_t bfrag[2];
-#pragma unroll
-                for (int nb = 0; nb < 2; ++nb) {
-                    const int r = nb * 32 + fr;
-                    const u32x4 t = tile[buf][r][c ^ (r & 15)];
-                    __builtin_memcpy(&bfrag[nb], &t, 16);
-                }
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) {
-                    bf16x8_t afrag;
-                    __builtin_memcpy(&afrag, &af[mb][j], 16);
-#pragma unroll
-                    for (int nb = 0; nb < 2; ++nb)
-                        acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[nb],
-                                                                              acc[mb][nb], 0, 0, 0);
-                }
-                // keep the reloads behind the MFMAs that read the old fragments: hoisted above
-                // them they would need a second set of registers
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
-                    af[mb][j] = *(const u32x4*)(xa + aoff[mb] + (uint32_t)(nh * 4 + j) * step_stride);
-                __builtin_amdgcn_sched_barrier(0);
+            for (int nb = 0; nb < 4; ++nb) {
+                const int r = nb * 32 + fr;
+                const u32x4 t = tile[buf][r][c ^ (r & 15)];
+                __builtin_memcpy(&bfrag[nb], &t, 16);
             }
+#pragma unroll
+            for (int mb = 0; mb < RB; ++mb) {
+                bf16x8_t afrag;
+                __builtin_memcpy(&afrag, &af[mb][j % PF], 16);
+#pragma unroll
+                for (int nb = 0; nb < 4; ++nb)
+                    acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[nb],
+                                                                          acc[mb][nb], 0, 0, 0);
+            }
+            int g = kb * 8 + j + PF;
+            g = g < steps ? g : steps - 1;
+#pragma unroll
+            for (int mb = 0; mb < RB; ++mb)
+                af[mb][j % PF] = *(const u32x4*)(xa + aoff[mb] + (uint32_t)g * step_stride);
+            if constexpr (MORE) produce_slice(j, kb + 1, buf ^ 1);
         }
-    }
+        __syncthreads();
+    };
+    for (int kb = 0; kb + 1 < nkb; ++kb) k_block(kb, std::true_type{});
+    k_block(nkb - 1, std::false_type{});
 
     // ---- epilogue: bf16(out) - ref in bf16, squared in fp32 (rows past T read row T - 1 and are
     // masked out of the sum)
     float part = 0.0f;
+    if (has_rows) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+        for (int mb = 0; mb < RB; ++mb)
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-            const uint16_t* rcol = ref + n0 + nb * 32 + fr;
-            uint16_t rv[16];
+            for (int nb = 0; nb < 4; ++nb) {
+                const uint16_t* rcol = ref + n0 + nb * 32 + fr;
+                uint16_t rv[16];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                int t = row_base + mb * 32 + 8 * (i / 4) + 4 * kg + (i % 4);
-                t = t < T ? t : T - 1;
-                rv[i] = rcol[(int64_t)t * N];
+                for (int i = 0; i < 16; ++i) {
+                    int t = row_base + mb * 32 + 8 * (i / 4) + 4 * kg + (i % 4);
+                    t = t < T ? t : T - 1;
+                    rv[i] = rcol[(int64_t)t * N];
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int t = row_base + mb * 32 + 8 * (i / 4) + 4 * kg + (i % 4);
+                    const float o = round_to_bf16(acc[mb][nb][i]);
+                    const float d = round_to_bf16(o - bf16_bits_to_f32(rv[i]));
+                    part += t < T ? d * d : 0.0f;
+                }
             }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int t = row_base + mb * 32 + 8 * (i / 4) + 4 * kg + (i % 4);
-                const float o = round_to_bf16(acc[mb][nb][i]);
-                const float d = round_to_bf16(o - bf16_bits_to_f32(rv[i]));
-                part += t < T ? d * d : 0.0f;
-            }
-        }
+    }
     double sum = (double)part;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
-    if (lane == 0) red[cw] = sum;
+    if (lane == 0) red[wave] = sum;
     __syncthreads();
-    if (cw == 0 && lane == 0) atomicAdd(loss + a, red[0] + red[1] + red[2] + red[3]);
+    if (threadIdx.x == 0) {
+        double total = 0.0;
+#pragma unroll
+        for (int i = 0; i < kSearchWaves; ++i) total += red[i];
+        atomicAdd(loss + a, total);
+    }
+}
+
+// xs[a][c][t][0..8) = bf16(x[t][8 c ..] * inv_s[a][8 c ..]) for every alpha: the activations the
+// search kernel multiplies, in its chunk-major layout.  A wavefront owns one chunk column c and
+// 64 consecutive tokens (its scales are wave-uniform, its stores contiguous: 1 KiB per alpha).
+__global__ __launch_bounds__(256) void awq_scale_activations_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ inv_s, int A, int T, int K,
+    uint16_t* __restrict__ xs) {
+    const int lane = threadIdx.x & 63;
+    const int c = blockIdx.y * 4 + (threadIdx.x >> 6);  // chunk column
+    const int t = blockIdx.x * 64 + lane;
+    const int kc = K >> 3;
+    if (c >= kc || t >= T) return;
+    const u32x4 raw = *(const u32x4*)(x + (int64_t)t * K + c * 8);
+    const uint32_t xw[4] = {raw.x, raw.y, raw.z, raw.w};
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        v[2 * j] = u2f(xw[j] << 16);
+        v[2 * j + 1] = u2f(xw[j] & 0xFFFF0000u);
+    }
+    for (int a = 0; a < A; ++a) {
+        const u32x4 sr = *(const u32x4*)(inv_s + (int64_t)a * K + c * 8);
+        const uint32_t sw[4] = {sr.x, sr.y, sr.z, sr.w};
+        u32x4 o;
+        o.x = f32x2_to_bf16x2(v[0] * u2f(sw[0] << 16), v[1] * u2f(sw[0] & 0xFFFF0000u));
+        o.y = f32x2_to_bf16x2(v[2] * u2f(sw[1] << 16), v[3] * u2f(sw[1] & 0xFFFF0000u));
+        o.z = f32x2_to_bf16x2(v[4] * u2f(sw[2] << 16), v[5] * u2f(sw[2] & 0xFFFF0000u));
+        o.w = f32x2_to_bf16x2(v[6] * u2f(sw[3] << 16), v[7] * u2f(sw[3] & 0xFFFF0000u));
+        *(u32x4*)(xs + (((int64_t)a * kc + c) * T + t) * 8) = o;
+    }
 }
 
 }  // namespace mo
@@ -242,25 +319,42 @@ extern "C" int mo_awq_search_losses(const void* xs, const void* w, const void* s
     else if (block_size == 64) lg_g = 3;
     else if (block_size == 128) lg_g = 4;
     if (lg_g < 0 || tokens > 512 || n % mo::kSearchTileN || k % mo::kSearchBlockK ||
-        n_alpha > 65535 || n > 0x7FFFFFFF || tokens * k > 0x7FFFFFFF)
+        n_alpha > 65535 || n > 0x7FFFFFFF || tokens * k > 0x7FFFFFFF ||
+        (n_alpha + 8) * (n / mo::kSearchTileN) > 0x7FFFFFFF)
         return MO_ERR_UNSUPPORTED;
     if ((((uintptr_t)xs | (uintptr_t)w | (uintptr_t)s) & 15u) || ((uintptr_t)ref & 1u))
         return MO_ERR_UNSUPPORTED;
     const float bound = (float)((1 << (num_bits - 1 + (is_unsigned ? 1 : 0))) - 1);
-    const float lo = is_unsigned ? 0.0f : (narrow_range ? -bound : -bound - 1.0f);
+    // signed grids only: the kernel relies on |w * s| <= block amax keeping every code inside
+    // [-bound, bound] (so narrow_range makes no difference); an unsigned grid would have to clamp
+    // negative weights to 0
+    if (is_unsigned) return MO_ERR_UNSUPPORTED;
+    (void)narrow_range;
     hipStream_t st = (hipStream_t)stream;
-    const dim3 grid((unsigned)(n / mo::kSearchTileN), (unsigned)n_alpha);
-    const int mb = (int)((tokens + 127) / 128);
-#define CALL(MB)                                                                           \
-    mo::awq_search_kernel<MB><<<grid, 512, 0, st>>>(                                       \
+    const int64_t pairs = n_alpha * (n / mo::kSearchTileN);
+    const dim3 grid((unsigned)((pairs + mo::kXcds - 1) / mo::kXcds * mo::kXcds));
+#define CALL(RB)                                                                           \
+    mo::awq_search_kernel<RB><<<grid, 512, 0, st>>>(                                       \
         (const uint16_t*)xs, (const uint16_t*)w, (const uint16_t*)s, (const uint16_t*)ref, \
-        (int)tokens, (int)n, (int)k, lg_g, bound, lo, loss)
-    switch (mb) {
-        case 1: CALL(1); break;
-        case 2: CALL(2); break;
-        case 3: CALL(3); break;
-        default: CALL(4); break;
-    }
+        (int)tokens, (int)n, (int)k, (int)n_alpha, lg_g, bound, loss)
+    if (tokens <= 256) CALL(1);
+    else CALL(2);
 #undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_awq_scale_activations(const void* x, const void* inv_s, int64_t n_alpha,
+                                        int64_t tokens, int64_t k, int dtype, void* xs,
+                                        void* stream) {
+    if (n_alpha < 0 || tokens < 0 || k < 0) return MO_ERR_ARG;
+    if (dtype != MO_BF16 || k % 8) return MO_ERR_UNSUPPORTED;
+    if (n_alpha == 0 || tokens == 0 || k == 0) return MO_OK;
+    if (!x || !inv_s || !xs) return MO_ERR_ARG;
+    if ((((uintptr_t)x | (uintptr_t)inv_s | (uintptr_t)xs) & 15u)) return MO_ERR_UNSUPPORTED;
+    const int64_t gx = (tokens + 63) / 64, gy = (k / 8 + 3) / 4;
+    if (gx > 0x7FFFFFFF || gy > 65535 || tokens * k > 0x7FFFFFFF || n_alpha > 0x7FFFFFFF)
+        return MO_ERR_UNSUPPORTED;
+    mo::awq_scale_activations_kernel<<<dim3((unsigned)gx, (unsigned)gy), 256, 0, (hipStream_t)stream>>>(
+        (const uint16_t*)x, (const uint16_t*)inv_s, (int)n_alpha, (int)tokens, (int)k, (uint16_t*)xs);
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

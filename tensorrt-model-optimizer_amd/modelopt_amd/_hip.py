@@ -48,6 +48,7 @@ SIGNATURES = {
     "mo_nf4_dequantize": [_P, _I64, _I64, _P, _P, _INT, _P],
     "mo_mul_cols": [_P, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_scale_block_int_qdq": [_P, _I64, _I64, _INT, _P, _INT, _I64, _INT, _INT, _INT, _P, _P],
+    "mo_awq_scale_activations": [_P, _P, _I64, _I64, _I64, _INT, _P, _P],
     "mo_awq_search_losses": [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _INT, _I64, _INT, _INT, _INT, _P, _P],
     "mo_awq_clip_losses": [_P, _I64, _P, _I64, _I64, _INT, _I64, _P, _INT, _P, _INT, _INT, _INT, _INT, _P, _P],
     "mo_abs_colsum": [_P, _I64, _I64, _INT, _P, _I64, _P, _P],
@@ -366,10 +367,15 @@ def awq_scaled_activations(x, inv_s):
     """``T(x * inv_s[a])`` for every row a of ``inv_s`` in the layout the search kernel reads:
     [n_alpha, K / 8, tokens, 8] (the 8-element chunks of a column group are contiguous over
     tokens, so that the lanes of a matrix-core operand read adjacent memory)."""
+    _require_device(x, inv_s)
     n_alpha, k = inv_s.shape
     tokens = x.shape[0]
-    xs = x[None] * inv_s[:, None, :]
-    return xs.view(n_alpha, tokens, k // 8, 8).transpose(1, 2).contiguous()
+    assert x.is_contiguous() and inv_s.is_contiguous() and x.shape == (tokens, k) and k % 8 == 0
+    assert x.dtype == inv_s.dtype == torch.bfloat16, "the search kernel takes bf16 activations"
+    xs = torch.empty((n_alpha, k // 8, tokens, 8), dtype=x.dtype, device=x.device)
+    call("mo_awq_scale_activations", x, _ptr(x), _ptr(inv_s), n_alpha, tokens, k, MO_BF16, _ptr(xs),
+         _stream(x))
+    return xs
 
 
 def awq_search_losses_into(xs, w, s, ref, block_size, num_bits, unsigned, narrow_range, loss):

@@ -41,8 +41,9 @@ def _fused_losses(x, w, s, ref, block, bits, unsigned, narrow):
     return out
 
 
-@pytest.mark.parametrize("tokens,n,k", [(512, 256, 512), (128, 64, 128), (100, 128, 256),
-                                        (300, 192, 384), (1, 64, 128), (512, 4096, 4096)])
+@pytest.mark.parametrize("tokens,n,k", [(512, 256, 512), (128, 128, 128), (100, 128, 256),
+                                        (300, 384, 384), (1, 128, 128), (257, 256, 256),
+                                        (512, 4096, 4096)])
 @pytest.mark.parametrize("block,bits,unsigned,narrow", [(128, 4, False, False), (64, 4, False, True),
                                                          (32, 8, False, False)])
 def test_matches_unfused_device_path(tokens, n, k, block, bits, unsigned, narrow):
@@ -57,7 +58,7 @@ def test_matches_unfused_device_path(tokens, n, k, block, bits, unsigned, narrow
 
 
 def test_accumulates_and_rejects_uncovered_shapes():
-    x, w, s = (t.to(DEV) for t in _problem(64, 64, 128, 2, 3))
+    x, w, s = (t.to(DEV) for t in _problem(64, 128, 128, 2, 3))
     ref = F.linear(x, w).contiguous()
     first = _fused_losses(x, w, s, ref, 128, 4, False, False)
     xs = _hip.awq_scaled_activations(x, (1 / s.float()).to(torch.bfloat16))
@@ -68,8 +69,10 @@ def test_accumulates_and_rejects_uncovered_shapes():
     assert not _hip.awq_search_losses_into(xs, w, s, ref, 256, 4, False, False, acc)
     assert not _hip.awq_search_losses_into(xs[:, :8].contiguous(), w[:, :64].contiguous(),
                                            s[:, :64].contiguous(), ref, 32, 4, False, False, acc)
+    assert not _hip.awq_search_losses_into(xs, w[:64].contiguous(), s, ref[:, :64].contiguous(), 128, 4,
+                                           False, False, acc)   # 64 output features
     big = torch.zeros(2, 16, 513, 8, dtype=torch.bfloat16, device=DEV)
-    assert not _hip.awq_search_losses_into(big, w, s, torch.zeros(513, 64, dtype=torch.bfloat16, device=DEV),
+    assert not _hip.awq_search_losses_into(big, w, s, torch.zeros(513, 128, dtype=torch.bfloat16, device=DEV),
                                            128, 4, False, False, acc)
     assert torch.allclose(acc, 2 * first, rtol=1e-12)
 
@@ -86,3 +89,15 @@ def test_matches_cpu_restatement_of_the_search_loop():
     want = torch.stack(want)
     got = _fused_losses(x.to(DEV), w.to(DEV), s.to(DEV), ref.to(DEV).contiguous(), 128, 4, False, False)
     assert torch.allclose(got.cpu(), want, rtol=1e-3), (got, want)
+
+
+@pytest.mark.parametrize("tokens,k,n_alpha", [(512, 4096, 21), (100, 256, 3), (1, 8, 1), (65, 1032, 2)])
+def test_scaled_activations_layout_and_rounding(tokens, k, n_alpha):
+    """``bf16(x * inv_s[a])`` for every alpha, chunk-major: bit for bit the tensor expression
+    (the reference multiplies the input by the bf16 pre-quant scale, tensor_quantizer.py:881-882)."""
+    g = torch.Generator().manual_seed(tokens + k)
+    x = (torch.randn(tokens, k, generator=g) * torch.exp(torch.randn(k, generator=g))).to(torch.bfloat16)
+    inv_s = torch.exp(0.5 * torch.randn(n_alpha, k, generator=g)).to(torch.bfloat16)
+    got = _hip.awq_scaled_activations(x.to(DEV), inv_s.to(DEV)).cpu()
+    want = (x[None] * inv_s[:, None, :]).view(n_alpha, tokens, k // 8, 8).transpose(1, 2).contiguous()
+    assert got.shape == want.shape and torch.equal(got.view(torch.int16), want.view(torch.int16))
