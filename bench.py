@@ -33,6 +33,8 @@ DEQUANT_BYTES_PER_ELEM = 0.5 + 1.0 / 16.0 + 2.0
 # scale factors come from a 1 GiB device copy in the same runs
 # (profiles/nvfp4_quantize_multi_kernel__llama3_8b_weights.txt).
 MEASURED_TRAFFIC_BYTES_32_LAYERS = 17.912e9
+TRAFFIC_SOURCE = ("profiles/nvfp4_quantize_multi_kernel__llama3_8b_weights.txt (rocprofv3 --pmc FETCH_SIZE, "
+                  "WRITE_SIZE of this command, scaled by a device copy of known size)")
 
 
 def make_weights(torch, layers, device):
@@ -42,6 +44,23 @@ def make_weights(torch, layers, device):
         for _, n, k in LAYER_SHAPES:
             ws.append(torch.randn(n, k, generator=g, device=device, dtype=torch.bfloat16).mul_(0.02))
     return ws
+
+
+def verify_against_restatement(torch, weights, amax, qplan, picks=(1, 3, 6)):
+    """What the timed launch wrote for a few tensors (k, o and down of the first layer) against the
+    C restatement of the reference arithmetic on the host: packed codes, block scales, global scale."""
+    from oracle import cref
+
+    packed, wsf, wsf2 = qplan.packed, qplan.wsf, qplan.wsf2
+    torch.cuda.synchronize()
+    for i in picks:
+        if i >= len(weights):
+            continue
+        p_c, s_c, w2_c = cref.nvfp4_quantize(weights[i].cpu(), 16, float(amax[i]))
+        assert torch.equal(packed[i].cpu(), p_c), f"tensor {i}: packed codes differ"
+        assert torch.equal(wsf[i].cpu().view(torch.uint8), s_c.view(torch.uint8)), f"tensor {i}: scales differ"
+        assert float(wsf2[i]) == float(w2_c), f"tensor {i}: global scale differs"
+    return f"outputs of the timed launch for tensors {list(picks)} equal the CPU restatement bit for bit"
 
 
 def timed(torch, fn, steps, warmup):
@@ -63,11 +82,12 @@ def timed(torch, fn, steps, warmup):
     return wall_ms, dev_ms
 
 
-def cpu_baseline(torch, passes=8):
-    """The C restatement of the reference's NVFP4 quantize+pack (oracle/c, OpenMP over blocks) on
-    a bounded sample: the seven weights of one decoder layer, quantised `passes` times from a
-    given global amax.  The first weight is also run through the torch CPU restatement (the
-    reference's own CPU path) and must give the same bytes."""
+def cpu_baseline(torch, passes=3, c_passes=4):
+    """The reference's CPU path for the benchmarked configuration -- NVFP4QTensor.quantize on torch CPU
+    tensors, restated op for op in oracle/ -- on a bounded sample: the seven weights of one
+    decoder layer (all four shapes), one warm-up pass, then `passes` timed passes from a given
+    global amax; the whole model is 32 such layers.  The OpenMP C restatement of the same
+    arithmetic is timed beside it and must give the same bytes."""
     from oracle import cref
     from oracle import export as oexport
 
@@ -75,31 +95,104 @@ def cpu_baseline(torch, passes=8):
     weights = []
     for _, n, k in LAYER_SHAPES:
         w = (0.02 * torch.randn(n, k, generator=g)).to(torch.bfloat16)
-        weights.append((w, float(w.abs().max())))
-    cref.nvfp4_quantize(*weights[0][:1], 16, weights[0][1])  # load the library, warm the threads
-    elems, secs = 0, 0.0
+        weights.append((w, w.abs().max()))
+    elems = sum(w.numel() for w, _ in weights)
+    for w, amax in weights:                      # warm-up pass (threads, allocator), and the check
+        p_t, s_t, _ = oexport.nvfp4_export(w, amax, 16)
+        p_c, s_c, _ = cref.nvfp4_quantize(w, 16, float(amax))
+        assert torch.equal(p_c, p_t) and torch.equal(s_c.view(torch.uint8), s_t.view(torch.uint8))
+    t0 = time.perf_counter()
     for _ in range(passes):
         for w, amax in weights:
-            t0 = time.perf_counter()
-            cref.nvfp4_quantize(w, 16, amax)
-            secs += time.perf_counter() - t0
-            elems += w.numel()
-    w, amax = weights[0]
+            oexport.nvfp4_export(w, amax, 16)
+    secs = time.perf_counter() - t0
     t0 = time.perf_counter()
-    p_t, s_t, _ = oexport.nvfp4_export(w, torch.tensor(amax), 16)
-    torch_secs = time.perf_counter() - t0
-    p_c, s_c, _ = cref.nvfp4_quantize(w, 16, amax)
-    assert torch.equal(p_c, p_t) and torch.equal(s_c.view(torch.uint8), s_t.view(torch.uint8))
-    torch_rate = w.numel() * QUANT_BYTES_PER_ELEM / torch_secs / 1e9
+    for _ in range(c_passes):
+        for w, amax in weights:
+            cref.nvfp4_quantize(w, 16, float(amax))
+    c_secs = time.perf_counter() - t0
+    rate = passes * elems * QUANT_BYTES_PER_ELEM / secs / 1e9
     return {
-        "value": round(elems * QUANT_BYTES_PER_ELEM / secs / 1e9, 4),
+        "value": round(rate, 4),
         "unit": "GB/s",
-        "cores": cref.threads(),
+        "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"7 weights of one layer x {passes} passes ({elems} elements), C restatement with "
-                  f"OpenMP, {secs:.2f} s wall; the torch CPU path does {torch_rate:.3f} GB/s on "
-                  f"{torch.get_num_threads()} threads; host has {os.cpu_count()} logical CPUs",
+        "sample": f"torch CPU restatement of NVFP4QTensor.quantize on the 7 weights of one layer "
+                  f"({elems} elements), {passes} timed passes after one warm-up pass, {secs:.2f} s; "
+                  f"32 layers extrapolate to {32 * secs / passes:.1f} s per model pass; host has "
+                  f"{os.cpu_count()} logical CPUs",
+        "c_port_GBps": round(c_passes * elems * QUANT_BYTES_PER_ELEM / c_secs / 1e9, 3),
+        "c_port_threads": cref.threads(),
     }
+
+
+def cpu_reference_configs(torch):
+    """The other benchmark configurations on the reference's CPU path (torch restatements in oracle/), each
+    run once on the host cores: C1 and C4 in full, C3 in full (21 alphas), C5's quantizer work on one
+    layer and one sequence, extrapolated.  Seconds of wall time; a reported baseline only."""
+    import torch.nn.functional as F  # noqa: F401
+
+    from oracle import awq as oawq
+    from oracle import fake_quant, qtensor, reduce
+
+    out = {"threads": torch.get_num_threads()}
+
+    def clock(fn):
+        t0 = time.perf_counter()
+        fn()
+        return time.perf_counter() - t0
+
+    g = torch.Generator().manual_seed(1)
+    w = 0.02 * torch.randn(4096, 4096, generator=g)
+    w.view(-1)[torch.randperm(w.numel(), generator=g)[:16777]] *= 50
+    w = w.to(torch.bfloat16)
+    clock(lambda: fake_quant.fp8_eager(w[:256], reduce.reduce_amax(w[:256])))  # warm the threads
+    out["c1_fp8_amax_plus_qdq_4096x4096_s"] = round(
+        clock(lambda: fake_quant.fp8_eager(w, reduce.reduce_amax(w))), 4)
+
+    g = torch.Generator().manual_seed(3)
+    w3 = (0.02 * torch.randn(4096, 4096, generator=g)).to(torch.bfloat16)
+    c = torch.exp(torch.randn(4096, generator=g))
+    c[torch.randperm(4096, generator=g)[:41]] *= 20
+    x3 = (torch.randn(512, 4096, generator=g) * c).to(torch.bfloat16)
+    out["c3_awq_lite_21_alphas_4096x4096_s"] = round(
+        clock(lambda: oawq.awq_lite_search(w3, [x3], alpha_step=0.05, block_size=128)), 3)
+
+    g = torch.Generator().manual_seed(4)
+    x = (torch.randn(8192, 8192, generator=g) * torch.exp(1.5 * torch.randn(8192, generator=g))[None, :]
+         ).to(torch.bfloat16)
+
+    def c4_nvfp4():  # the CPU has no fake-quant kernel: quantize + dequantize through the QTensor
+        p, s, s2 = qtensor.nvfp4_quantize(x, 16)
+        qtensor.nvfp4_dequantize(p, s, s2, 16, x.shape, x.dtype)
+    out["c4_nvfp4_amax_plus_qdq_8192x8192_s"] = round(clock(c4_nvfp4), 3)
+    g = torch.Generator().manual_seed(5)
+    w8 = (0.02 * torch.randn(8192, 8192, generator=g)).to(torch.bfloat16)
+
+    def c4_smoothquant():  # quantizer work only: the layer's own GEMM is not part of it
+        act = reduce.reduce_amax(x, axis=[0]).reshape(-1)
+        pqs, w_new, in_amax, w_amax = oawq.smoothquant_linear(w8, act, 0.5)
+        fake_quant.tensor_quant(x * pqs, in_amax, 8, False, False)
+        fake_quant.tensor_quant(w_new, w_amax, 8, False, False)
+    out["c4_smoothquant_int8_8192x8192_quantizer_work_s"] = round(clock(c4_smoothquant), 3)
+    del x, w8
+
+    # C5: per layer and forward the reference reduces the 7 weights (every forward) and, per
+    # sequence, the inputs of the 7 linears and K / V; timed on one layer and one 512-token sequence
+    g = torch.Generator().manual_seed(6)
+    ws = [(0.02 * torch.randn(n, k, generator=g)).to(torch.bfloat16) for _, n, k in LAYER_SHAPES]
+    acts = [torch.randn(512, k, generator=g).to(torch.bfloat16) for _, _, k in LAYER_SHAPES]
+    kv = [torch.randn(8, 512, 128, generator=g).to(torch.bfloat16) for _ in range(2)]
+    t_w = clock(lambda: [reduce.reduce_amax(t) for t in ws])
+    t_a = clock(lambda: [reduce.reduce_amax(t) for t in acts + kv])
+    forwards = 8  # 128 sequences in batches of 16
+    out["c5_quantizer_work_one_layer_s"] = {"weights_one_forward": round(t_w, 4),
+                                            "activations_and_kv_one_sequence": round(t_a, 4)}
+    out["c5_quantizer_work_extrapolated_s"] = round(32 * (forwards * t_w + 128 * t_a), 1)
+    out["note"] = ("reduce_amax / fake quant / QTensor code of the reference restated in torch, default "
+                   "thread count; C5 counts the quantizer reductions only (no decoder GEMMs) and is 32 "
+                   "layers x (8 forwards x weights + 128 sequences x activations) of the one-layer timings")
+    return out
 
 
 def single_tensor_configs(torch, steps, warmup):
@@ -265,6 +358,14 @@ def calib_sweep(torch, layers, n_seqs, batch, seq_len=512):
     torch.cuda.synchronize()
     calib_s = time.perf_counter() - t0
     n_q = sum(1 for m in model.modules() if isinstance(m, mtq.nn.TensorQuantizer) and m.is_enabled)
+    # the quantizer kernels on their own: the same calibration pass once more with an event pair
+    # around every library call (sum of the per-call device times)
+    from modelopt_amd import _hip
+    for m in model.modules():
+        if isinstance(m, mtq.nn.TensorQuantizer):
+            m.reset_amax()
+    with _hip.KernelTimer() as kt:
+        mtq.calibrate(model, "max", forward_loop)
     # the same data once more through the calibrated model: every forward fake-quantises the
     # inputs and weights of all 224 linears and K / V (what evaluating a PTQ model costs)
     torch.cuda.synchronize()
@@ -293,6 +394,8 @@ def calib_sweep(torch, layers, n_seqs, batch, seq_len=512):
         "end_to_end_calib_s": round(calib_s, 3),
         "forward_only_s": round(plain_s, 3),
         "quantizer_overhead_s": round(calib_s - plain_s, 3),
+        "quantizer_kernel_s": round(kt.total_seconds, 4),
+        "quantizer_kernel_calls": dict(kt.calls),
         "enabled_quantizers": n_q,
         "tokens": tokens,
         "amax_bytes_read": {"activations_and_kv": act_bytes, "weights_once": w_bytes},
@@ -342,6 +445,7 @@ def main():
     torch.cuda.synchronize()
 
     wall_ms, dev_ms = timed(torch, qplan.run, a.steps, a.warmup)
+    verified = verify_against_restatement(torch, weights, amax, qplan)
     quant_bytes = elems * QUANT_BYTES_PER_ELEM
     value = quant_bytes / (wall_ms * 1e-3) / 1e9
     achieved = quant_bytes / (dev_ms * 1e-3) / 1e9
@@ -366,6 +470,7 @@ def main():
             "elements": elems,
             "algorithmic_bytes": int(quant_bytes),
             "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+            "verified": verified,
         },
         "roofline": {
             "bound": "hbm",
@@ -375,7 +480,10 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "launch_ms": round(dev_ms, 4),
+            # frac = algorithmic bytes / launch_ms / peak; traffic is NOT measured by this run: it is
+            # the counter reading of the committed profile of this same command
             "traffic": MEASURED_TRAFFIC_BYTES_32_LAYERS if a.layers == 32 else None,
+            "traffic_source": TRAFFIC_SOURCE if a.layers == 32 else None,
         },
     }
 
@@ -456,6 +564,9 @@ def main():
 
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)
+        if not a.no_extras:
+            with contextlib.redirect_stdout(sys.stderr):
+                out.setdefault("extras", {})["cpu_reference_path"] = cpu_reference_configs(torch)
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

@@ -103,11 +103,53 @@ def _require_device(*tensors):
             raise RuntimeError("modelopt_amd kernels need tensors in GPU memory (got a CPU tensor)")
 
 
+_timer = None  # the active KernelTimer, if any
+
+
+class KernelTimer:
+    """Context manager that brackets every library call made through ``call`` with a pair of
+    events on the stream the kernels are launched on, and sums the elapsed device time of those
+    calls per entry point when it exits (one synchronisation, at exit).  Measurement aid: a call
+    costs two extra event records while it is active."""
+
+    def __init__(self):
+        self.pairs = []      # (entry point, start event, end event)
+        self.seconds = {}    # entry point -> summed device seconds
+        self.calls = {}
+
+    def __enter__(self):
+        global _timer
+        self._previous, _timer = _timer, self
+        return self
+
+    def __exit__(self, *exc):
+        global _timer
+        _timer = self._previous
+        torch.cuda.synchronize()
+        for name, start, end in self.pairs:
+            self.seconds[name] = self.seconds.get(name, 0.0) + start.elapsed_time(end) * 1e-3
+            self.calls[name] = self.calls.get(name, 0) + 1
+        self.pairs = []
+        return False
+
+    @property
+    def total_seconds(self):
+        return sum(self.seconds.values())
+
+
 def call(name: str, anchor: torch.Tensor, *args):
     """Invoke ``name`` with the device of ``anchor`` current; raise on a non-zero status."""
     lib = load()
     with torch.cuda.device(anchor.device):
-        rc = getattr(lib, name)(*args)
+        if _timer is None:
+            rc = getattr(lib, name)(*args)
+        else:
+            start = torch.cuda.Event(enable_timing=True)
+            end = torch.cuda.Event(enable_timing=True)
+            start.record()
+            rc = getattr(lib, name)(*args)
+            end.record()
+            _timer.pairs.append((name, start, end))
     if rc != 0:
         msg = lib.mo_error_string(rc).decode()
         raise RuntimeError(f"{name} failed: {msg} (status {rc})")

@@ -7,6 +7,8 @@ reproduced; conversion acts on the model in place.
 """
 
 import fnmatch
+import functools
+import re
 import warnings
 from contextlib import contextmanager
 from typing import Any
@@ -63,9 +65,15 @@ def set_quantizer_by_cfg(quant_model: nn.Module, quant_cfg: dict | QuantizeConfi
         set_quantizer_attribute(quant_model, pattern, cfg, _index=index)
 
 
+@functools.lru_cache(maxsize=512)
+def _compiled(pattern: str):
+    return re.compile(fnmatch.translate(pattern)).match
+
+
 def _matches(name: str, wildcard_or_filter) -> bool:
     if isinstance(wildcard_or_filter, str):
-        return fnmatch.fnmatch(name, wildcard_or_filter)
+        # fnmatch.fnmatch without its per-call normalisation (names are already in posix form)
+        return _compiled(wildcard_or_filter)(name) is not None
     if callable(wildcard_or_filter):
         return bool(wildcard_or_filter(name))
     raise NotImplementedError(f"Unsupported type {type(wildcard_or_filter)}")

@@ -11,7 +11,7 @@ import torch
 from ... import _hip
 
 __all__ = [
-    "amax_layout", "kept_dims_first", "absmax_accumulate", "reduce_amax_gpu", "fake_quant_int", "fake_quant_fp8",
+    "amax_layout", "kept_dims_first", "dense_flat_view", "absmax_accumulate", "reduce_amax_gpu", "fake_quant_int", "fake_quant_fp8",
     "fake_quant_nvfp4", "fake_quant_block_fp", "mul_last_dim",
 ]
 
@@ -77,10 +77,28 @@ def layout_from_amax_shape(x_shape, amax_shape):
     return amax_layout(x_shape, keep)
 
 
+def dense_flat_view(x: torch.Tensor):
+    """A 1-D view over the memory of ``x`` when ``x`` is a permutation of a contiguous block (a
+    transposed K / V view, a channels-last tensor): every element appears exactly once, in memory
+    order.  None when ``x`` has gaps or overlaps."""
+    dims = sorted((d for d in range(x.dim()) if x.shape[d] != 1), key=lambda d: -x.stride(d))
+    expect = 1
+    for d in reversed(dims):
+        if x.stride(d) != expect:
+            return None
+        expect *= x.shape[d]
+    return x.as_strided((x.numel(),), (1,))
+
+
 def absmax_accumulate(x: torch.Tensor, acc: torch.Tensor, layout):
     """acc (fp32, ``axis`` elements) = max(acc, abs-max of x over the reduced dims)."""
     outer, axis, inner = layout
-    return _hip.absmax_into(x if x.is_contiguous() else x.contiguous(), acc, outer, axis, inner)
+    if not x.is_contiguous():
+        # a per-tensor maximum does not care about element order: a permuted dense tensor (the
+        # [B, H, S, D] view of K / V) is reduced where it lies instead of through a copy
+        flat = dense_flat_view(x) if axis == 1 else None
+        x = flat if flat is not None else x.contiguous()
+    return _hip.absmax_into(x, acc, outer, axis, inner)
 
 
 def reduce_amax_gpu(x: torch.Tensor, reduce_dims, keepdims=True):

@@ -62,11 +62,12 @@ class TensorQuantizer(nn.Module):
         if amax is not None:
             self.amax = amax
         self.set_from_attribute_config(cfg)
-        self._if_quant = if_quant
-        self._if_calib = if_calib
-        self._enable_pre_quant_scale = True
-        self._dequantize = False
-        self._input_dtype = None
+        plain = object.__setattr__  # plain python values: skip nn.Module's attribute bookkeeping
+        plain(self, "_if_quant", if_quant)
+        plain(self, "_if_calib", if_calib)
+        plain(self, "_enable_pre_quant_scale", True)
+        plain(self, "_dequantize", False)
+        plain(self, "_input_dtype", None)
 
     # ------------------------------------------------------------------ configuration
     def set_from_attribute_config(self, attribute_cfg: QuantizerAttributeConfig | dict):
@@ -90,7 +91,7 @@ class TensorQuantizer(nn.Module):
                 plain(self, f"_{name}", val)
         for name, val in items:
             if name == "calibrator":
-                self._calibrator = self._make_calibrator(val)
+                plain(self, "_calibrator", self._make_calibrator(val))
         if self.is_mx_format:
             self._pass_through_bwd = True
 

@@ -517,3 +517,15 @@ def test_library_operators_are_registered_with_fake_implementations():
     assert targets == ["tensorrt.quantize_op.default", "tensorrt.dynamic_block_quantize_op.default"]
     with pytest.raises(RuntimeError, match="GPU memory"):   # the CPU implementation is the loud failure
         torch.ops.tensorrt.quantize_op(torch.randn(4), torch.tensor(1.0), 8, 0, False, False)
+
+
+def test_dense_flat_view_covers_permuted_blocks_only():
+    from modelopt_amd.torch.quantization.kernels import dense_flat_view
+
+    x = torch.arange(2 * 3 * 4 * 5, dtype=torch.float32).reshape(2, 3, 4, 5)
+    for t in (x, x.transpose(1, 2), x.permute(3, 0, 2, 1), x.transpose(1, 2)[1:], x.unsqueeze(0).transpose(2, 3),
+              torch.zeros(3, 1, 4).transpose(0, 2)):
+        v = dense_flat_view(t)
+        assert v is not None and v.dim() == 1 and sorted(v.tolist()) == sorted(t.flatten().tolist())
+    for t in (x[:, :2], x[..., ::2], x.transpose(1, 2)[:, :, :2], x[0, 0].expand(3, 4, 5)):
+        assert dense_flat_view(t) is None

@@ -518,3 +518,26 @@ def test_straight_through_gradient_with_clipping(cfg):
     q(x).sum().backward()
     assert torch.allclose(x.grad, torch.ones_like(x.grad) * (x.abs() <= q.amax))
     assert 0 < float(x.grad.sum()) < x.numel()
+
+
+def test_per_tensor_calibration_of_a_permuted_view_makes_no_copy(monkeypatch):
+    """K / V reach their quantizers as [B, H, S, D] views of a [B, S, H, D] projection: the
+    per-tensor abs-max is taken over the memory as it lies and equals the oracle's."""
+    from modelopt_amd import _hip
+    from modelopt_amd.torch.quantization import kernels
+
+    x = _rand((4, 64, 8, 32), seed=31)
+    view = x.to(DEV).transpose(1, 2)
+    assert not view.is_contiguous()
+    seen = []
+    real = _hip.absmax_into
+    monkeypatch.setattr(_hip, "absmax_into", lambda t, *a: (seen.append(t.data_ptr()), real(t, *a))[1])
+    cal = calib.MaxCalibrator(8, None, False)
+    cal.collect(view)
+    assert seen == [view.data_ptr()]                       # reduced in place, not through a copy
+    assert_bits_equal(cal.compute_amax().cpu(), reduce.reduce_amax(x), "amax of the view")
+    sliced = x.to(DEV)[:, :, :4]                           # gaps: falls back to a contiguous copy
+    cal2 = calib.MaxCalibrator(8, None, False)
+    cal2.collect(sliced)
+    assert_bits_equal(cal2.compute_amax().cpu(), reduce.reduce_amax(x[:, :, :4]), "amax of a slice")
+    assert kernels.dense_flat_view(sliced) is None

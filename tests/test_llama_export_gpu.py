@@ -355,3 +355,49 @@ def test_pattern_fuse_prequant(cfg_name, heads):
     # without quantization error only the rounding of the folded weights (and, for grouped
     # heads, of o_proj re-smoothed to the averaged scale) remains
     assert float((after_exact - before_exact).norm() / before_exact.norm()) < 0.03
+
+
+def test_calibration_sweep_on_two_layers_of_the_8b_shape():
+    """The calibration sweep configuration on a two-layer slice at the real layer shape (hidden 4096, FFN 14336,
+    32 query / 8 KV heads; vocabulary cut to 1024): NVFP4 weight + input quantizers and FP8 K / V
+    quantizers.  Every calibrated amax -- 14 weights, 14 linear inputs, 2 x (K, V) -- equals the
+    oracle's reduce_amax over exactly the tensors that reached that quantizer on the device."""
+    import dataclasses
+
+    from modelopt_amd.testing.llama_decoder import LLAMA3_8B
+
+    shape = dataclasses.replace(LLAMA3_8B, num_hidden_layers=2, vocab_size=1024)
+    model = LlamaForCausalLM(shape, device=DEV, seed=9)
+    g = torch.Generator().manual_seed(9)
+    batches = [torch.randint(0, shape.vocab_size, (2, 512), generator=g) for _ in range(3)]
+    cfg = mtq.utils.update_quant_cfg_with_kv_cache_quant(mtq.NVFP4_DEFAULT_CFG, mtq.FP8_KV_CFG["quant_cfg"])
+
+    seen = {}   # quantizer name -> running oracle amax of what it was shown
+
+    def watch(name):
+        def hook(module, args):
+            if module._if_calib:
+                local = reduce.reduce_amax(args[0].detach().cpu())
+                seen[name] = local if name not in seen else torch.maximum(seen[name], local)
+        return hook
+
+    def loop(m):
+        handles = [q.register_forward_pre_hook(watch(n)) for n, q in m.named_modules()
+                   if isinstance(q, TensorQuantizer)]
+        for ids in batches:
+            m(ids.to(DEV))
+        for h in handles:
+            h.remove()
+
+    mtq.quantize(model, cfg, loop)
+    enabled = {n: q for n, q in model.named_modules() if isinstance(q, TensorQuantizer) and q.is_enabled}
+    assert len(enabled) == 2 * (7 * 2 + 2)
+    kinds = {"weight_quantizer": 0, "input_quantizer": 0, "k_bmm_quantizer": 0, "v_bmm_quantizer": 0}
+    for name, q in enabled.items():
+        assert name in seen, name
+        assert_bits_equal(q.amax.cpu().reshape(()), seen[name].reshape(()).to(q.amax.dtype), name)
+        kinds[name.rsplit(".", 1)[1]] += 1
+    assert kinds == {"weight_quantizer": 14, "input_quantizer": 14, "k_bmm_quantizer": 2, "v_bmm_quantizer": 2}
+    assert model.get_submodule("model.layers.1.mlp.down_proj").weight.shape == (4096, 14336)
+    k_seen = model.get_submodule("model.layers.0.self_attn.k_bmm_quantizer")
+    assert k_seen.amax.numel() == 1 and float(k_seen.amax) > 0
