@@ -228,6 +228,29 @@ def single_tensor_configs(torch, steps, warmup):
     _, ms = timed(torch, c1, steps, warmup)
     out["c1_fp8_amax_plus_qdq_4096x4096"] = {"ms": round(ms, 4), "GBps": round(w.numel() * 6 / ms / 1e6, 1)}
 
+    # the same in one launch that reads the tensor once (4 B / element): every workgroup keeps its
+    # share in registers while the workgroups agree on the abs-max
+    def c1_fused():
+        assert _hip.fused_amax_qdq(w, "fp8", out=y) is not None
+    _, ms = timed(torch, c1_fused, max(steps, 50), max(warmup, 10))
+    out["c1_fp8_fused_amax_qdq_4096x4096"] = {"ms": round(ms, 4), "GBps": round(w.numel() * 4 / ms / 1e6, 1),
+                                              "bytes_per_element": 4}
+    wq = (0.02 * torch.randn(4096, 4096, generator=torch.Generator().manual_seed(7))).to(torch.bfloat16).to(dev)
+
+    def nvfp4_two():
+        acc.zero_()
+        _hip.absmax_into(wq, acc, 1, 1, wq.numel())
+        _hip.nvfp4_quantize(wq, acc.reshape(()), 16)
+
+    def nvfp4_fused():
+        assert _hip.nvfp4_quantize_fused(wq) is not None
+    _, ms2 = timed(torch, nvfp4_two, max(steps, 50), max(warmup, 10))
+    _, ms1 = timed(torch, nvfp4_fused, max(steps, 50), max(warmup, 10))
+    out["nvfp4_amax_plus_quantize_one_weight_4096x4096"] = {
+        "two_launches_ms": round(ms2, 4), "fused_one_launch_ms": round(ms1, 4),
+        "fused_GBps": round(wq.numel() * QUANT_BYTES_PER_ELEM / ms1 / 1e6, 1)}
+    assert not _hip.fused_gave_up(dev)
+
     g = torch.Generator().manual_seed(4)
     x = (torch.randn(8192, 8192, generator=g) * torch.exp(1.5 * torch.randn(8192, generator=g))[None, :]
          ).to(torch.bfloat16).to(dev)
@@ -293,7 +316,7 @@ def single_tensor_configs(torch, steps, warmup):
 
     def search():
         _hip.awq_search_losses_into(xs, w3, scales, ref, 128, 4, False, False, loss)
-    _, ms = timed(torch, search, steps, warmup)
+    _, ms = timed(torch, search, max(steps, 50), max(warmup, 20))  # past the clock ramp
     kflops = 2 * 512 * 4096 * 4096 * 21
     out["c3_awq_search_kernel_21_alphas"] = {
         "ms": round(ms, 4), "TFLOPs": round(kflops / ms / 1e9, 1), "bound": "mfma",

@@ -231,6 +231,39 @@ int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs, const int32
                             int64_t total_tiles, int dtype, int block_size, int amax_is_wsf2,
                             int flags, void* stream);
 
+/* ------------------------------------------------------------------ one-launch amax -> quantize
+ * The fused variants compute the per-tensor abs-max and quantise in ONE launch that reads the
+ * tensor once (2 + 2 instead of 2 + 2 + 2 bytes per bf16 element for fake quant, 2.56 instead of
+ * 4.56 for NVFP4 quantize + pack): every workgroup keeps its share of the tensor in registers
+ * while the workgroups agree on the maximum.  All workgroups have to be resident at once, which
+ * bounds the tensor size: MO_ERR_TOO_LARGE beyond 32 MiB (what two workgroups per compute unit
+ * hold in registers), MO_ERR_UNSUPPORTED when the layout is not covered; the two-launch entry
+ * points take over then.  Run one fused call at a time per device (successive calls in one
+ * stream do that); other kernels may share the device.
+ * workspace: MO_FUSED_WS_BYTES of device memory, 128-byte aligned, all zero before the first
+ *   call; it can be reused by calls that follow each other in one stream (calls that overlap
+ *   must not share a workspace).  The 32-bit word at byte MO_FUSED_WS_FAIL_OFFSET is set to 1,
+ *   and the outputs are not written, if a workgroup gave up waiting for the others after
+ *   spin_limit polls (a safety net: no wavefront waits for ever); the caller zeroes the
+ *   workspace after reading that flag.
+ * amax_out (optional): the abs-max that was used, as fp32. */
+
+#define MO_FUSED_WS_BYTES 512
+#define MO_FUSED_WS_FAIL_OFFSET 384
+
+/* mo_absmax (per tensor) followed by mo_nvfp4_quantize with that amax: the same outputs.
+ * bf16, block_size 16, k % 16 == 0, x 16-byte and packed 8-byte aligned. */
+int mo_nvfp4_quantize_fused(const void* x, int64_t rows, int64_t k, int dtype, int block_size,
+                            uint8_t* packed, uint8_t* wsf_out, float* wsf2_out, float* amax_out,
+                            int flags, void* workspace, int64_t spin_limit, void* stream);
+
+/* mo_absmax (per tensor) followed by mo_int_qdq (kind 0) or mo_fp8_qdq (kind 1) with that amax:
+ * dynamic per-tensor fake quantisation, TensorQuantizer._get_amax + _fake_quantize
+ * (TQ/nn/modules/tensor_quantizer.py:505-514, 633-686).  x and y 16-byte aligned; y may alias x. */
+int mo_fused_amax_qdq(const void* x, void* y, int64_t n, int dtype, int kind, int num_bits,
+                      int is_unsigned, int narrow_range, int saturate, float* amax_out,
+                      void* workspace, int64_t spin_limit, void* stream);
+
 /* NVFP4 unpack + rescale.  Replaces NVFP4QTensor.dequantize (TQ/qtensor/nvfp4_tensor.py
  * :234-297) and fp4_dequantize (TQ/triton/fp4_kernel.py:307):
  * y[rows, kp] = T(LUT[code] * (f32(wsf) * wsf2)). */

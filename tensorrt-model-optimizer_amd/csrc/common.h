@@ -388,4 +388,90 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* smem) {
     return v;
 }
 
+
+// ---------------------------------------------------------------- one-launch amax -> quantize
+// The fused kernels read their share of the tensor into registers, agree on the global abs-max
+// and then quantise from the registers: the tensor is read once.  Each workgroup waits here for
+// all the others, so the host launches no more workgroups than the device holds at the same time
+// (resident_grid_limit).  It is an ordinary launch: hipLaunchCooperativeKernel adds about 15 us
+// per call on this device, more than the second launch that the fusion saves.  Workgroups of
+// other kernels that occupy the device only delay the exchange, because they end without help
+// from this kernel; two of THESE kernels running side by side could each hold the compute units
+// the other one waits for, so callers run one fused call at a time per device, and the bounded
+// wait below turns a violation into an error instead of a hang.
+//
+// ws: MO_FUSED_WS_BYTES of device memory, all zero before the first use; one word per 128-byte
+// line, so that the atomics on different words do not queue behind each other:
+//   line 0  workgroups that have delivered their maximum (back to 0 when the exchange is over)
+//   line 1  running maximum, an abs-max bit pattern (back to 0 likewise)
+//   line 2  64-bit {generation, result}: the last workgroup to arrive publishes the maximum
+//           together with a generation one higher than the one every workgroup read on entry
+//   line 3  set to 1 when a wait gave up
+// Only these words cross workgroups and every access to them is a device-scope atomic performed
+// at the memory side, so relaxed ordering is enough (a release / acquire pair would write back
+// and invalidate caches on this multi-die part); program order between two atomics of a thread
+// is kept by waiting for the value the first one returns.
+// The wait is bounded: after `spin_limit` polls (one about every half microsecond) a workgroup
+// sets the flag, returns false and the kernel ends without writing its outputs, so that no
+// wavefront can stay behind for ever.  Calls that share a workspace must follow each other in
+// one stream.
+constexpr int kWsCount = 0, kWsMax = 32, kWsPublished = 64, kWsFail = 96;  // word offsets
+
+__device__ __forceinline__ bool grid_max_exchange(uint32_t* ws, uint32_t local, uint32_t nwg,
+                                                  uint32_t spin_limit, uint32_t* smem /* 8 words */,
+                                                  uint32_t& global) {
+    unsigned long long* published = (unsigned long long*)(ws + kWsPublished);
+    unsigned long long entry = 0;
+    if (threadIdx.x == 0)  // the generation of the previous exchange; issued ahead of the reduction
+        entry = __hip_atomic_load(published, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t m = block_max_u32(local, smem);
+    if (threadIdx.x == 0) {
+        uint32_t old = 0;
+        if (m) old = __hip_atomic_fetch_max(ws + kWsMax, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::"v"(old), "v"(entry) : "memory");
+        const uint32_t before =
+            __hip_atomic_fetch_add(ws + kWsCount, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        bool ok = true;
+        uint32_t g;
+        if (before + 1 == nwg) {
+            // last to arrive: every maximum has been applied.  Clean up, then publish.
+            g = __hip_atomic_load(ws + kWsMax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::"v"(g) : "memory");
+            const uint32_t c0 = __hip_atomic_exchange(ws + kWsCount, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint32_t m0 = __hip_atomic_exchange(ws + kWsMax, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::"v"(c0), "v"(m0) : "memory");
+            const unsigned long long next = (((entry >> 32) + 1ull) << 32) | (unsigned long long)g;
+            __hip_atomic_store(published, next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            uint32_t spins = 0;
+            unsigned long long now;
+            for (;;) {
+                __builtin_amdgcn_s_sleep(16);
+                now = __hip_atomic_load(published, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((now >> 32) != (entry >> 32)) break;
+                if (spins++ >= spin_limit) { ok = false; break; }
+            }
+            g = (uint32_t)now;
+            if (!ok) __hip_atomic_store(ws + kWsFail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        smem[4] = g;
+        smem[5] = ok ? 1u : 0u;
+    }
+    __syncthreads();
+    global = smem[4];
+    return smem[5] != 0u;
+}
+
+// How many workgroups of `kernel` (of `threads` lanes) the current device holds at the same time;
+// cached by the caller; 0 on error.
+template <typename K>
+static int resident_grid_limit(K kernel, int threads) {
+    int dev = 0, cus = 0, per_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess)
+        return 0;
+    return cus * per_cu;
+}
+
 }  // namespace mo

@@ -245,33 +245,41 @@ __device__ __forceinline__ uint32_t swap_adjacent_lanes(uint32_t v) {
     return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);
 }
 
-__device__ __forceinline__ void quantize_tile_bf16(const uint16_t* __restrict__ x,
-                                                   int64_t nblocks, int64_t tile, float wsf2,
-                                                   float gs6, int opts,
-                                                   u32x2* __restrict__ packed,
-                                                   uint8_t* __restrict__ wsf) {
-    constexpr int RP = kTileBlocks / 256;  // round pairs
+constexpr int kTileRoundPairs = kTileBlocks / 256;
+
+// the raw chunks of one tile: lane t holds chunks t + 512 p (a) and t + 256 + 512 p (b)
+struct TileRaw { u32x4 a[kTileRoundPairs], b[kTileRoundPairs]; };
+
+__device__ __forceinline__ void load_tile_bf16(const uint16_t* __restrict__ x, int64_t nblocks,
+                                               int64_t tile, TileRaw& r) {
+    const int64_t nchunks = nblocks * 2;
+    const int64_t c0 = tile * (kTileBlocks * 2) + threadIdx.x;
+#pragma unroll
+    for (int p = 0; p < kTileRoundPairs; ++p) {
+        const int64_t ca = c0 + p * 512, cb = ca + 256;
+        const u32x4 zero = {0, 0, 0, 0};
+        r.a[p] = ca < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + ca * 8)) : zero;
+        r.b[p] = cb < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + cb * 8)) : zero;
+    }
+}
+
+__device__ __forceinline__ void quantize_loaded_tile_bf16(const TileRaw& r, int64_t nblocks,
+                                                          int64_t tile, float wsf2, float gs6,
+                                                          int opts, u32x2* __restrict__ packed,
+                                                          uint8_t* __restrict__ wsf) {
     const int64_t nchunks = nblocks * 2;
     const int64_t c0 = tile * (kTileBlocks * 2) + threadIdx.x;
     const bool odd = threadIdx.x & 1;
-    u32x4 a[RP], b[RP];
 #pragma unroll
-    for (int p = 0; p < RP; ++p) {
+    for (int p = 0; p < kTileRoundPairs; ++p) {
         const int64_t ca = c0 + p * 512, cb = ca + 256;
-        const u32x4 zero = {0, 0, 0, 0};
-        a[p] = ca < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + ca * 8)) : zero;
-        b[p] = cb < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + cb * 8)) : zero;
-    }
-#pragma unroll
-    for (int p = 0; p < RP; ++p) {
-        const int64_t ca = c0 + p * 512, cb = ca + 256;
-        const u32x4 send = odd ? a[p] : b[p];
+        const u32x4 send = odd ? r.a[p] : r.b[p];
         u32x4 recv;
         recv.x = swap_adjacent_lanes(send.x);
         recv.y = swap_adjacent_lanes(send.y);
         recv.z = swap_adjacent_lanes(send.z);
         recv.w = swap_adjacent_lanes(send.w);
-        const u32x4 first = odd ? recv : a[p], second = odd ? b[p] : recv;
+        const u32x4 first = odd ? recv : r.a[p], second = odd ? r.b[p] : recv;
         const uint32_t w[8] = {first.x, first.y, first.z, first.w,
                                second.x, second.y, second.z, second.w};
         uint32_t byte, lo, hi;
@@ -284,6 +292,16 @@ __device__ __forceinline__ void quantize_tile_bf16(const uint16_t* __restrict__ 
             wsf[blk] = (uint8_t)byte;
         }
     }
+}
+
+__device__ __forceinline__ void quantize_tile_bf16(const uint16_t* __restrict__ x,
+                                                   int64_t nblocks, int64_t tile, float wsf2,
+                                                   float gs6, int opts,
+                                                   u32x2* __restrict__ packed,
+                                                   uint8_t* __restrict__ wsf) {
+    TileRaw r;
+    load_tile_bf16(x, nblocks, tile, r);
+    quantize_loaded_tile_bf16(r, nblocks, tile, wsf2, gs6, opts, packed, wsf);
 }
 
 __global__ __launch_bounds__(256) void nvfp4_quantize_fast_kernel(
@@ -321,6 +339,67 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_multi_kernel(
     if (jb.wsf2_out && t == jb.tile_begin && threadIdx.x == 0) jb.wsf2_out[0] = wsf2;
     quantize_tile_bf16((const uint16_t*)jb.x, jb.elems >> 4, t - jb.tile_begin, wsf2, 6.0f * wsf2,
                        opts, (u32x2*)jb.packed, jb.wsf);
+}
+
+// Abs-max and quantize + pack in ONE launch that reads the tensor once: workgroup w loads tiles
+// w, w + G, ... (TP of them) into registers, the workgroups agree on the global abs-max
+// (grid_max_exchange) and each quantises the tiles it holds.
+template <int TP>
+__global__ __launch_bounds__(256) void nvfp4_quantize_fused_kernel(
+    const uint16_t* __restrict__ x, int64_t nblocks, int64_t tiles, int opts,
+    u32x2* __restrict__ packed, uint8_t* __restrict__ wsf_out, float* __restrict__ wsf2_out,
+    float* __restrict__ amax_out, uint32_t* __restrict__ ws, uint32_t spin_limit) {
+    __shared__ uint32_t smem[8];
+    TileRaw r[TP];
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < TP; ++i) {
+        const int64_t t = (int64_t)i * gridDim.x + blockIdx.x;
+        load_tile_bf16(x, nblocks, t < tiles ? t : tiles, r[i]);  // past the end: all zero
+    }
+#pragma unroll
+    for (int i = 0; i < TP; ++i)
+#pragma unroll
+        for (int p = 0; p < kTileRoundPairs; ++p) {
+            const u32x4 a = r[i].a[p], b = r[i].b[p];
+            m = pk_max_u16(m, pk_max_u16(pk_max_u16(a.x & 0x7FFF7FFFu, a.y & 0x7FFF7FFFu),
+                                         pk_max_u16(a.z & 0x7FFF7FFFu, a.w & 0x7FFF7FFFu)));
+            m = pk_max_u16(m, pk_max_u16(pk_max_u16(b.x & 0x7FFF7FFFu, b.y & 0x7FFF7FFFu),
+                                         pk_max_u16(b.z & 0x7FFF7FFFu, b.w & 0x7FFF7FFFu)));
+        }
+    const uint32_t h = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
+    uint32_t gbits;
+    if (!grid_max_exchange(ws, h << 16, gridDim.x, spin_limit, smem, gbits)) return;
+    const float amax = u2f(gbits);
+    const float wsf2 = amax / 2688.0f;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        if (amax_out) amax_out[0] = amax;
+        if (wsf2_out) wsf2_out[0] = wsf2;
+    }
+#pragma unroll
+    for (int i = 0; i < TP; ++i) {
+        const int64_t t = (int64_t)i * gridDim.x + blockIdx.x;
+        if (t < tiles) quantize_loaded_tile_bf16(r[i], nblocks, t, wsf2, 6.0f * wsf2, opts, packed, wsf_out);
+    }
+}
+
+template <int TP>
+static int launch_quantize_fused(const uint16_t* x, int64_t nblocks, int64_t tiles, int opts,
+                                 u32x2* packed, uint8_t* wsf_out, float* wsf2_out, float* amax_out,
+                                 uint32_t* ws, uint32_t spin_limit, hipStream_t s) {
+    static int limit[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MO_ERR_LAUNCH;
+    if (!limit[dev]) {
+        const int l = resident_grid_limit(nvfp4_quantize_fused_kernel<TP>, 256);
+        limit[dev] = l > 0 ? l : -1;
+    }
+    if (limit[dev] < 0) return MO_ERR_UNSUPPORTED;
+    const int64_t grid = (tiles + TP - 1) / TP;
+    if (grid > limit[dev]) return MO_ERR_TOO_LARGE;
+    nvfp4_quantize_fused_kernel<TP><<<dim3((unsigned)grid), 256, 0, s>>>(
+        x, nblocks, tiles, opts, packed, wsf_out, wsf2_out, amax_out, ws, spin_limit);
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }
 
 // ------------------------------------------------------------------------------ fast dequantize
@@ -654,4 +733,33 @@ extern "C" int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs,
     mo::nvfp4_quantize_multi_kernel<<<(unsigned)total_tiles, 256, mo::ballast_bytes("nvfp4_quantize_multi_kernel", cap_kb), (hipStream_t)stream>>>(
         jobs_dev, njobs, tile_job_dev, amax_is_wsf2, flags);
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_nvfp4_quantize_fused(const void* x, int64_t rows, int64_t k, int dtype,
+                                       int block_size, uint8_t* packed, uint8_t* wsf_out,
+                                       float* wsf2_out, float* amax_out, int flags,
+                                       void* workspace, int64_t spin_limit, void* stream) {
+    if (rows < 0 || k < 0 || (flags & ~kKnownFlags) || spin_limit < 0) return MO_ERR_ARG;
+    if (dtype != MO_BF16 || block_size != 16 || k % 16) return MO_ERR_UNSUPPORTED;
+    if (rows == 0 || k == 0) return MO_OK;
+    if (!x || !packed || !wsf_out || !workspace) return MO_ERR_ARG;
+    if (((uintptr_t)x & 15u) || ((uintptr_t)packed & 7u) || ((uintptr_t)workspace & 127u))
+        return MO_ERR_UNSUPPORTED;
+    const int64_t nblocks = rows * k / 16;
+    const int64_t tiles = (nblocks + mo::kTileBlocks - 1) / mo::kTileBlocks;
+    const uint32_t spins = spin_limit > 0xFFFFFFFFll ? 0xFFFFFFFFu : (uint32_t)spin_limit;
+    hipStream_t s = (hipStream_t)stream;
+    // the fewer workgroups meet at the exchange, the cheaper it is: as many tiles per workgroup
+    // (1, 2, 4) as keep the grid at two workgroups per compute unit, more workgroups after that
+    int rc = MO_ERR_TOO_LARGE;
+    if (tiles <= 512)
+        rc = mo::launch_quantize_fused<1>((const uint16_t*)x, nblocks, tiles, flags, (mo::u32x2*)packed,
+                                          wsf_out, wsf2_out, amax_out, (uint32_t*)workspace, spins, s);
+    if (rc == MO_ERR_TOO_LARGE && tiles <= 1024)
+        rc = mo::launch_quantize_fused<2>((const uint16_t*)x, nblocks, tiles, flags, (mo::u32x2*)packed,
+                                          wsf_out, wsf2_out, amax_out, (uint32_t*)workspace, spins, s);
+    if (rc == MO_ERR_TOO_LARGE)
+        rc = mo::launch_quantize_fused<4>((const uint16_t*)x, nblocks, tiles, flags, (mo::u32x2*)packed,
+                                          wsf_out, wsf2_out, amax_out, (uint32_t*)workspace, spins, s);
+    return rc;
 }

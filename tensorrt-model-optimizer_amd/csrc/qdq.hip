@@ -160,6 +160,101 @@ static int launch_qdq(const void* x, void* y, int64_t outer, int64_t axis, int64
     return MO_OK;
 }
 
+// ------------------------------------------------------------------------------ one launch
+// Per-tensor abs-max and quantize-dequantize in ONE launch that reads x once: a lane loads its
+// U chunks into registers, the workgroups agree on the abs-max (grid_max_exchange) and every
+// lane quantises what it holds.  Chunk (u * gridDim.x + blockIdx.x) * 256 + threadIdx.x belongs
+// to round u of a lane, so a round of a workgroup is 4 KiB of contiguous memory.
+template <int DT, int U, bool FLAG, typename Op>
+__global__ __launch_bounds__(256) void fused_amax_qdq_kernel(
+    const void* __restrict__ x, void* __restrict__ y, int64_t n, Op op, uint32_t* __restrict__ ws,
+    uint32_t spin_limit, float* __restrict__ amax_out) {
+    __shared__ uint32_t smem[8];
+    const int64_t chunks = n >> 3;
+    RawChunk<DT> raw[U];
+    uint32_t m = 0;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int64_t c = ((int64_t)u * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
+        zero_raw<DT>(raw[u]);
+        if (c < chunks) load_raw<DT>(x, c << 3, raw[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if constexpr (DT == MO_F32) {
+            const uint32_t w[8] = {raw[u].a.x, raw[u].a.y, raw[u].a.z, raw[u].a.w,
+                                   raw[u].b.x, raw[u].b.y, raw[u].b.z, raw[u].b.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { const uint32_t t = w[j] & 0x7FFFFFFFu; m = t > m ? t : m; }
+        } else {
+            const uint32_t t = pk_max_u16(pk_max_u16(raw[u].a.x & 0x7FFF7FFFu, raw[u].a.y & 0x7FFF7FFFu),
+                                          pk_max_u16(raw[u].a.z & 0x7FFF7FFFu, raw[u].a.w & 0x7FFF7FFFu));
+            m = pk_max_u16(m, t);
+        }
+    }
+    // the tail (n % 8 elements) is handled by the first lanes of workgroup 0
+    float tail = 0.0f;
+    const bool has_tail = blockIdx.x == 0 && threadIdx.x < (n & 7);
+    if (has_tail) tail = load_elem<DT>(x, (chunks << 3) + threadIdx.x);
+    uint32_t bits;
+    if constexpr (DT == MO_F32) bits = m;
+    else {
+        const uint32_t h = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
+        bits = DT == MO_BF16 ? h << 16 : f2u(f16_bits_to_f32(h));
+    }
+    const uint32_t tb = f2u(tail) & 0x7FFFFFFFu;
+    bits = tb > bits ? tb : bits;
+    uint32_t gbits;
+    if (!grid_max_exchange(ws, bits, gridDim.x, spin_limit, smem, gbits)) return;
+    if (amax_out && blockIdx.x == 0 && threadIdx.x == 0) amax_out[0] = u2f(gbits);
+    const typename Op::Scale s0 = op.make(u2f(gbits));
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int64_t c = ((int64_t)u * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
+        if (c >= chunks) continue;
+        float v[8];
+        unpack_raw<DT>(raw[u], v);
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[j], v[j + 1], s0, s0);
+        store_chunk<DT>(y, c << 3, v);
+    }
+    if (has_tail) store_elem<DT>(y, (chunks << 3) + threadIdx.x, op.template apply<FLAG>(tail, s0));
+}
+
+template <int DT, int U, bool FLAG, typename Op>
+static int launch_fused_qdq_u(const void* x, void* y, int64_t n, Op op, uint32_t* ws,
+                              uint32_t spin_limit, float* amax_out, int64_t grid, hipStream_t s) {
+    static int limit[64] = {0};  // per device: workgroups of this instantiation resident at once
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MO_ERR_LAUNCH;
+    if (!limit[dev]) {
+        const int l = resident_grid_limit(fused_amax_qdq_kernel<DT, U, FLAG, Op>, 256);
+        limit[dev] = l > 0 ? l : -1;
+    }
+    if (limit[dev] < 0) return MO_ERR_UNSUPPORTED;
+    if (grid > limit[dev]) return MO_ERR_TOO_LARGE;
+    fused_amax_qdq_kernel<DT, U, FLAG, Op><<<dim3((unsigned)grid), 256, 0, s>>>(x, y, n, op, ws, spin_limit, amax_out);
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+// chunks per lane: the smallest of 4, 8, 16 that covers the tensor with at most 512 workgroups
+// (two per CU: the fewer workgroups meet at the exchange, the cheaper it is)
+template <int DT, bool FLAG, typename Op>
+static int launch_fused_qdq(const void* x, void* y, int64_t n, Op op, uint32_t* ws,
+                            uint32_t spin_limit, float* amax_out, hipStream_t s) {
+    if ((((uintptr_t)x | (uintptr_t)y) & 15u)) return MO_ERR_UNSUPPORTED;
+    const int64_t chunks = n >> 3;
+    const int64_t lanes = 512 * 256;
+    const int64_t need = (chunks + lanes - 1) / lanes;
+    const int u = need <= 4 ? 4 : (need <= 8 ? 8 : 16);
+    if (need > 16) return MO_ERR_TOO_LARGE;
+    int64_t grid = (chunks + 256 * u - 1) / (256 * u);
+    if (grid < 1) grid = 1;
+    if (u == 4) return launch_fused_qdq_u<DT, 4, FLAG, Op>(x, y, n, op, ws, spin_limit, amax_out, grid, s);
+    if (u == 8) return launch_fused_qdq_u<DT, 8, FLAG, Op>(x, y, n, op, ws, spin_limit, amax_out, grid, s);
+    return launch_fused_qdq_u<DT, 16, FLAG, Op>(x, y, n, op, ws, spin_limit, amax_out, grid, s);
+}
+
 }  // namespace mo
 
 static int check_common(const void* x, void* y, int64_t outer, int64_t axis, int64_t inner,
@@ -215,4 +310,41 @@ extern "C" int mo_int_qdq(const void* x, void* y, int64_t outer, int64_t axis, i
     }
     if (rc != MO_OK) return rc;
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_fused_amax_qdq(const void* x, void* y, int64_t n, int dtype, int kind,
+                                 int num_bits, int is_unsigned, int narrow_range, int saturate,
+                                 float* amax_out, void* workspace, int64_t spin_limit,
+                                 void* stream) {
+    if (n < 0 || (kind != 0 && kind != 1) || spin_limit < 0) return MO_ERR_ARG;
+    if (kind == 0 && (num_bits < 1 || num_bits > 24)) return MO_ERR_ARG;
+    if (n == 0) return MO_OK;
+    if (!x || !y || !workspace || ((uintptr_t)workspace & 127u)) return MO_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    uint32_t* ws = (uint32_t*)workspace;
+    const uint32_t spins = spin_limit > 0xFFFFFFFFll ? 0xFFFFFFFFu : (uint32_t)spin_limit;
+    int rc;
+    if (kind == 1) {
+#define CALL(DT)                                                                                   \
+    rc = saturate ? mo::launch_fused_qdq<DT, true>(x, y, n, mo::Fp8Op<true>(), ws, spins, amax_out, s) \
+                  : mo::launch_fused_qdq<DT, false>(x, y, n, mo::Fp8Op<true>(), ws, spins, amax_out, s)
+        switch (dtype) {
+            case MO_F32: CALL(MO_F32); break;
+            case MO_F16: CALL(MO_F16); break;
+            case MO_BF16: CALL(MO_BF16); break;
+            default: return MO_ERR_DTYPE;
+        }
+#undef CALL
+    } else {
+        mo::IntOp op;
+        op.bound = (float)((1 << (num_bits - 1 + (is_unsigned ? 1 : 0))) - 1);
+        op.lo = is_unsigned ? 0.0f : (narrow_range ? -op.bound : -op.bound - 1.0f);
+        switch (dtype) {
+            case MO_F32: rc = mo::launch_fused_qdq<MO_F32, false>(x, y, n, op, ws, spins, amax_out, s); break;
+            case MO_F16: rc = mo::launch_fused_qdq<MO_F16, false>(x, y, n, op, ws, spins, amax_out, s); break;
+            case MO_BF16: rc = mo::launch_fused_qdq<MO_BF16, false>(x, y, n, op, ws, spins, amax_out, s); break;
+            default: return MO_ERR_DTYPE;
+        }
+    }
+    return rc;
 }

@@ -38,6 +38,8 @@ SIGNATURES = {
     "mo_block_fp_qdq": [_P, _P, _I64, _I64, _INT, _INT, _INT, _INT, _P, _I64, _P],
     "mo_convert_to_format": [_P, _P, _I64, _INT, _P],
     "mo_nvfp4_quantize": [_P, _I64, _I64, _INT, _INT, _P, _INT, _P, _P, _P, _P, _INT, _P],
+    "mo_nvfp4_quantize_fused": [_P, _I64, _I64, _INT, _INT, _P, _P, _P, _P, _INT, _P, _I64, _P],
+    "mo_fused_amax_qdq": [_P, _P, _I64, _INT, _INT, _INT, _INT, _INT, _INT, _P, _P, _I64, _P],
     "mo_nvfp4_dequantize": [_P, _P, _P, _I64, _I64, _INT, _P, _INT, _P],
     "mo_real_quantize": [_P, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _P, _P],
     "mo_real_dequantize": [_P, _I64, _I64, _I64, _INT, _P, _INT, _P, _INT, _P],
@@ -304,6 +306,94 @@ def nvfp4_quantize(x, amax_f32, block_size=16, amax_is_wsf2=False, wsf_in=None, 
          _ptr(amax_f32), int(amax_is_wsf2), _ptr(wsf_arg), _ptr(packed),
          None if wsf_in is not None else _ptr(wsf), _ptr(wsf2), int(flags), _stream(x))
     return packed, wsf.view(torch.float8_e4m3fn), wsf2
+
+
+# --------------------------------------------------------------- one-launch amax -> quantize
+FUSED_WS_BYTES, FUSED_WS_FAIL_OFFSET = 512, 384   # MO_FUSED_WS_BYTES, MO_FUSED_WS_FAIL_OFFSET
+FUSED_SPIN_LIMIT = 1 << 22   # polls a workgroup waits for the others before it gives up
+_fused_ws_by_device = {}
+
+
+def fused_scratch(device, stream=None):
+    """The workspace of the fused kernels for ``device`` and ``stream`` (default: torch's current
+    stream there).  Calls in one stream follow each other and can share it; calls in different
+    streams may overlap and get one each."""
+    index = torch.device(device).index
+    index = torch.cuda.current_device() if index is None else index
+    if stream is None:
+        stream = torch.cuda.current_stream(index).cuda_stream
+    ws = _fused_ws_by_device.get((index, stream))
+    if ws is None:
+        ws = torch.zeros(FUSED_WS_BYTES // 4, dtype=torch.int32, device=torch.device("cuda", index))
+        assert ws.data_ptr() % 128 == 0
+        _fused_ws_by_device[(index, stream)] = ws
+    return ws
+
+
+def fused_gave_up(device=None) -> bool:
+    """Whether a fused kernel (on ``device``; default: any device) ended without writing its
+    outputs because a workgroup gave up waiting for the others.  Synchronises; clears the state."""
+    index = None if device is None else torch.device(device).index
+    failed = False
+    for (dev, _), ws in _fused_ws_by_device.items():
+        if index is not None and dev != index:
+            continue
+        if bool(ws[FUSED_WS_FAIL_OFFSET // 4].item()):
+            ws.zero_()
+            failed = True
+    return failed
+
+
+def _fused_rc(name, rc):
+    if rc in (MO_ERR_UNSUPPORTED, MO_ERR_TOO_LARGE):
+        return False
+    if rc != 0:
+        raise RuntimeError(f"{name} failed: {load().mo_error_string(rc).decode()} (status {rc})")
+    return True
+
+
+def nvfp4_quantize_fused(x, flags=0, spin_limit=FUSED_SPIN_LIMIT):
+    """Per-tensor abs-max and NVFP4 quantize + pack of a bf16 tensor in one launch that reads it
+    once.  Returns (packed, wsf, wsf2, amax fp32 scalar), or None when the tensor is too large
+    for the registers of the chip or the layout is not covered (use the two-launch path then)."""
+    _require_device(x)
+    k = x.shape[-1] if x.dim() else 0
+    if x.dtype != torch.bfloat16 or not x.is_contiguous() or k == 0 or k % 16 or x.data_ptr() % 16:
+        return None
+    rows = x.numel() // k
+    lead = tuple(x.shape[:-1])
+    packed = torch.empty(lead + (k // 2,), dtype=torch.uint8, device=x.device)
+    wsf = torch.empty(lead + (k // 16,), dtype=torch.uint8, device=x.device)
+    wsf2 = torch.empty((), dtype=torch.float32, device=x.device)
+    amax = torch.empty((), dtype=torch.float32, device=x.device)
+    ws = fused_scratch(x.device)
+    with torch.cuda.device(x.device):
+        rc = load().mo_nvfp4_quantize_fused(_ptr(x), rows, k, MO_BF16, 16, _ptr(packed), _ptr(wsf),
+                                            _ptr(wsf2), _ptr(amax), int(flags), _ptr(ws),
+                                            int(spin_limit), _stream(x))
+    if not _fused_rc("mo_nvfp4_quantize_fused", rc):
+        return None
+    return packed, wsf.view(torch.float8_e4m3fn), wsf2, amax
+
+
+def fused_amax_qdq(x, kind, num_bits=8, unsigned=False, narrow_range=False, saturate=False,
+                   out=None, spin_limit=FUSED_SPIN_LIMIT):
+    """Dynamic per-tensor fake quantisation in one launch (``kind`` "int" or "fp8"): returns
+    (y, amax fp32 scalar), or None when the tensor does not fit / the layout is not covered."""
+    _require_device(x)
+    if not x.is_contiguous() or x.dtype not in _DTYPES or x.data_ptr() % 16 or x.numel() == 0:
+        return None
+    y = torch.empty_like(x) if out is None else out
+    amax = torch.empty((), dtype=torch.float32, device=x.device)
+    ws = fused_scratch(x.device)
+    with torch.cuda.device(x.device):
+        rc = load().mo_fused_amax_qdq(_ptr(x), _ptr(y), x.numel(), dtype_code(x.dtype),
+                                      0 if kind == "int" else 1, int(num_bits), int(bool(unsigned)),
+                                      int(bool(narrow_range)), int(bool(saturate)), _ptr(amax),
+                                      _ptr(ws), int(spin_limit), _stream(x))
+    if not _fused_rc("mo_fused_amax_qdq", rc):
+        return None
+    return y, amax
 
 
 def nvfp4_dequantize(packed, wsf, wsf2, block_size, dtype):

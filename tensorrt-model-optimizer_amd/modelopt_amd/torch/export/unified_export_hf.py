@@ -195,6 +195,9 @@ def _export_hf_checkpoint(model: nn.Module, dtype: torch.dtype | None = None):
         if id(m) not in done:
             _export_quantized_weight(m, dtype)
     state = postprocess_state_dict(model.state_dict(), kv_bound, kv_format)
+    if _hip.fused_gave_up():
+        raise RuntimeError("a one-launch quantize kernel ended without writing its outputs (its "
+                           "workgroups could not all run at once); export again")
     return state, quant_config
 
 

@@ -7,6 +7,7 @@ The per-element work (abs-max, scaling, quantize-dequantize, column statistics, 
 runs in the HIP kernels; the search GEMM is a plain library GEMM (``F.linear``).
 """
 
+import functools
 import math
 import types
 import warnings
@@ -458,12 +459,18 @@ def get_act_scale(x):
     return (acc / x2.shape[0]).to(x.dtype).to(torch.float32)
 
 
+@functools.lru_cache(maxsize=64)
+def _exponent_columns_cached(alphas: tuple, device):
+    both = torch.tensor([[float(v) for v in alphas], [1 - float(v) for v in alphas]],
+                        dtype=torch.float32).to(device)
+    return both[0][:, None], both[1][:, None]
+
+
 def _exponent_columns(alphas, device):
     """fp32 ``[A, 1]`` device columns of ``alpha`` and ``1 - alpha`` (the difference is taken in
-    double, as the scalar form of ``pow`` does before it narrows the exponent)."""
-    a = torch.tensor([float(v) for v in alphas], dtype=torch.float32)
-    b = torch.tensor([1 - float(v) for v in alphas], dtype=torch.float32)
-    return a.to(device)[:, None], b.to(device)[:, None]
+    double, as the scalar form of ``pow`` does before it narrows the exponent); built once per
+    alpha grid and device."""
+    return _exponent_columns_cached(tuple(float(v) for v in alphas), torch.device(device))
 
 
 def _pow_rows(t, exponents, column):
@@ -641,13 +648,13 @@ def _awq_forward(self, input, *args, **kwargs):
 
 def _finalize_losses(helper):
     """loss[alpha] = sum over search steps of that step's mean squared error.  The kernel leaves
-    per-step sums of squares on the device; this is the one host synchronisation of the search."""
+    per-step sums of squares on the device; fetching them is the one host synchronisation of the
+    search, and the division and the sum over steps happen on the host in double."""
     if not helper.sq_err_steps:
         return {a: 0.0 for a in helper.alphas}
-    sums = torch.stack([s for s, _ in helper.sq_err_steps])
-    sizes = torch.tensor([n for _, n in helper.sq_err_steps], dtype=torch.float64,
-                         device=sums.device)
-    total = (sums / sizes[:, None]).sum(0).cpu().tolist()
+    sums = torch.stack([s for s, _ in helper.sq_err_steps]).cpu()
+    sizes = torch.tensor([n for _, n in helper.sq_err_steps], dtype=torch.float64)
+    total = (sums / sizes[:, None]).sum(0).tolist()
     return dict(zip(helper.alphas, total))
 
 

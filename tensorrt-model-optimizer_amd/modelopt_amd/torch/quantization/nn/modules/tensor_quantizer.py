@@ -20,9 +20,21 @@ from ... import utils as quant_utils
 from ...config import QuantizerAttributeConfig
 from ...qtensor import (BaseQuantizedTensor, FP8QTensor, INT4QTensor, INT8QTensor, MXFP4QTensor,
                         NF4QTensor, NVFP4QTensor, QTensorWrapper)
+from ...overflow import get_fp8_overflow_behavior
 from ...tensor_quant import dynamic_block_quant, fake_tensor_quant, scaled_e4m3
 
 __all__ = ["SequentialQuantizer", "TensorQuantizer"]
+
+_DEFAULT_CONFIG = []
+
+
+def _default_config():
+    """The all-defaults config, built (and validated) once: a model conversion creates three
+    quantizers per layer and only reads it."""
+    if not _DEFAULT_CONFIG:
+        _DEFAULT_CONFIG.append(QuantizerAttributeConfig())
+    return _DEFAULT_CONFIG[0]
+
 
 # [id of the calibration pass in progress, or 0]; the weight abs-max cache is only valid inside one
 _CALIBRATION_PASS = [0]
@@ -58,7 +70,7 @@ class TensorQuantizer(nn.Module):
 
     def __init__(self, quant_attribute_cfg=None, if_quant=True, if_calib=False, amax=None):
         super().__init__()
-        cfg = quant_attribute_cfg if quant_attribute_cfg is not None else QuantizerAttributeConfig()
+        cfg = quant_attribute_cfg if quant_attribute_cfg is not None else _default_config()
         if amax is not None:
             self.amax = amax
         self.set_from_attribute_config(cfg)
@@ -369,7 +381,30 @@ class TensorQuantizer(nn.Module):
         return outputs
 
     # ------------------------------------------------------------------ fake quantisation
+    def _fused_dynamic_per_tensor(self, inputs):
+        """Dynamic per-tensor INT / FP8 fake quantisation (no calibrated ``_amax``, no axis, no
+        blocks) outside autograd: abs-max and quantize-dequantize in one launch that reads the
+        tensor once.  None when that case does not apply or the tensor is too large for it."""
+        if hasattr(self, "_amax") or self._axis is not None or self.block_sizes is not None:
+            return None
+        if not inputs.is_cuda or (inputs.requires_grad and torch.is_grad_enabled()):
+            return None
+        if getattr(self, "_bias_calibrator", None) is not None or self.is_mx_format:
+            return None
+        if isinstance(self._num_bits, tuple):
+            if self._num_bits != (4, 3):
+                return None
+            # a per-tensor amax goes to the reference's clamping kernel unless "nan" is selected
+            done = kernels._hip.fused_amax_qdq(inputs, "fp8", saturate=get_fp8_overflow_behavior() != "nan")
+        else:
+            done = kernels._hip.fused_amax_qdq(inputs, "int", self._num_bits, self._unsigned,
+                                               self._narrow_range)
+        return None if done is None else done[0]
+
     def _fake_quantize(self, inputs):
+        fused = self._fused_dynamic_per_tensor(inputs)
+        if fused is not None:
+            return fused
         amax = None if self.is_mx_format else self._get_amax(inputs)
         bs = self.block_sizes
         if bs is not None and bs.get("type", "static") == "dynamic":

@@ -84,6 +84,13 @@ class NVFP4QTensor(BaseQuantizedTensor):
             return torch.div(blocks, scale.unsqueeze(-1)).reshape(xp.shape)
         shape, dtype = input.shape, input.dtype
         x = input.contiguous()
+        if weights_scaling_factor_2 is None and weights_scaling_factor is None and block_size == 16:
+            # abs-max, scales and codes in one launch that reads the tensor once (tensors that fit
+            # the chip's registers; larger ones take the two launches below)
+            fused = _hip.nvfp4_quantize_fused(x, flags=nvfp4_quantize_flags())
+            if fused is not None:
+                packed, wsf, wsf2, _ = fused
+                return cls(shape, dtype, packed), wsf, wsf2
         if weights_scaling_factor_2 is None:
             acc = torch.zeros(1, dtype=torch.float32, device=x.device)
             _hip.absmax_into(x, acc, 1, 1, x.numel())
