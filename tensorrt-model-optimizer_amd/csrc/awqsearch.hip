@@ -20,11 +20,13 @@
 // output tile never leaves the registers: it is rounded to bf16, compared with the reference
 // output and reduced to one double per workgroup.
 //
-// The integer codes are the reference's bit for bit (correctly rounded bound / amax, one IEEE
-// multiply, round half to even); the dequantised value is code * (1 / scale) with a correctly
-// rounded reciprocal instead of the reference's division: the fp32 results differ by at most an
-// ulp, which survives the rounding to bf16 for about one weight in 10^4, far below the 1e-3
-// tolerance of the per-alpha losses.  The weights that are kept after the search come from the
+// The integer codes follow the reference's arithmetic (bound / amax, one IEEE multiply, round
+// half to even) with bound / amax from the hardware reciprocal and one FMA correction step,
+// which is the correctly rounded quotient except for quotients that lie within about 2^-40 of
+// the midpoint of two floats; the dequantised value is code * (amax / bound) instead of the
+// reference's division by bound / amax: the fp32 results differ by at most an ulp, which
+// survives the rounding to bf16 for about one weight in 10^4, far below the 1e-3 tolerance of
+// the per-alpha losses.  The weights that are kept after the search come from the
 // exact kernels.
 #include <type_traits>
 
@@ -72,45 +74,62 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
     const int n0 = (pair % ncol) * kSearchTileN;
     const int nkb = K / kSearchBlockK;
 
-    // ---- producer side: chunk qc of rows qr + 32 u of the tile (u = 0..3), two chunks at a time
+    // ---- producer side: chunk qc of rows qr + 32 u of the tile (u = 0..3), two chunks at a time.
+    // Addresses are a wave-uniform base plus a 32-bit byte offset per lane (128 rows of K bf16
+    // stay below 4 GiB: K < 2^24 is checked by the launcher), so advancing along k costs no
+    // vector instruction.
     const int qc = threadIdx.x & 15, qr = threadIdx.x >> 4;
-    const uint16_t* wp0 = w + (int64_t)(n0 + qr) * K + qc * 8;
-    const int64_t wstride = (int64_t)32 * K;  // between the rows of two of a lane's chunks
-    const uint16_t* sp = s + (int64_t)a * K + qc * 8;
+    const char* wtile = (const char*)(w + (int64_t)n0 * K);
+    const uint32_t woff = ((uint32_t)qr * (uint32_t)K + (uint32_t)qc * 8u) * 2u;
+    const uint32_t wstride = 32u * (uint32_t)K * 2u;  // between the rows of two of a lane's chunks
+    const char* srow = (const char*)(s + (int64_t)a * K);
+    const uint32_t soff = (uint32_t)qc * 16u;
     u32x4 wraw[4], sraw;    // raw weight chunks and scales of the block to quantise next
-    float v[2][8];          // the pair of chunks being quantised: bf16(w * s) as fp32
+    float sf[8];            // the scales of the block being quantised
+    uint32_t vp[2][4];      // the pair of chunks being quantised: bf16(w * s), packed
     float mul[2], rdiv[2];  // per chunk: bound / amax and amax / bound
 
     auto fetch = [&](int kb) {  // weights are used once per alpha: streamed past the L2
-        const int k0 = (kb < nkb ? kb : nkb - 1) * kSearchBlockK;
+        const uint32_t k0 = (uint32_t)(kb < nkb ? kb : nkb - 1) * (kSearchBlockK * 2);
 #pragma unroll
         for (int u = 0; u < 4; ++u)
-            wraw[u] = __builtin_nontemporal_load((const u32x4*)(wp0 + u * wstride + k0));
-        sraw = *(const u32x4*)(sp + k0);
+            wraw[u] = __builtin_nontemporal_load((const u32x4*)(wtile + k0 + u * wstride + woff));
+        sraw = *(const u32x4*)(srow + k0 + soff);
     };
-    auto scale_pair = [&](int h) {  // chunks 2 h, 2 h + 1: v = bf16(w * s)
-        const uint32_t sw[4] = {sraw.x, sraw.y, sraw.z, sraw.w};
+    auto scale_pair = [&](int h) {  // chunks 2 h, 2 h + 1: bf16(w * s), two values a word
+        if (h == 0) {
+            const uint32_t sw[4] = {sraw.x, sraw.y, sraw.z, sraw.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                sf[2 * j] = u2f(sw[j] << 16);
+                sf[2 * j + 1] = u2f(sw[j] & 0xFFFF0000u);
+            }
+        }
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const u32x4 r = wraw[2 * h + i];
             const uint32_t ww[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                v[i][2 * j] = round_to_bf16(u2f(ww[j] << 16) * u2f(sw[j] << 16));
-                v[i][2 * j + 1] = round_to_bf16(u2f(ww[j] & 0xFFFF0000u) * u2f(sw[j] & 0xFFFF0000u));
-            }
+            for (int j = 0; j < 4; ++j)
+                vp[i][j] = f32x2_to_bf16x2(u2f(ww[j] << 16) * sf[2 * j],
+                                           u2f(ww[j] & 0xFFFF0000u) * sf[2 * j + 1]);
         }
     };
     const float inv_bound = 1.0f / bound;
     auto block_scales = [&]() {  // block abs-max over the lanes of a block, then the two factors
+        typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            uint32_t m = 0;
+            // |bf16| bit patterns order like the magnitudes: 16-bit integer maxima, two a word
+            u16x2 m2 = {0, 0};
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint32_t t = f2u(v[i][j]) & 0x7FFFFFFFu;
-                m = t > m ? t : m;
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t t = vp[i][j] & 0x7FFF7FFFu;
+                u16x2 t2;
+                __builtin_memcpy(&t2, &t, 4);
+                m2 = __builtin_elementwise_max(m2, t2);
             }
+            uint32_t m = (uint32_t)(m2.x > m2.y ? m2.x : m2.y) << 16;   // as fp32 bits
             // abs-max over the 1 << lg_g (4, 8 or 16) lanes of a block; selects instead of
             // branches keep the loop body one basic block
 #define MO_DPP_STEP(CTRL, ON)                                                                 \
@@ -125,7 +144,12 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
 #undef MO_DPP_STEP
             const float amax = u2f(m);
             const bool dead = amax <= 5.9604644775390625e-8f;  // 2^-24
-            mul[i] = dead ? 0.0f : bound / amax;
+            // bound / amax: hardware reciprocal and one FMA correction step, without the
+            // branches of the full division sequence
+            const float r = __builtin_amdgcn_rcpf(amax);
+            const float q0 = bound * r;
+            const float q1 = __builtin_fmaf(__builtin_fmaf(-q0, amax, bound), r, q0);
+            mul[i] = dead ? 0.0f : q1;
             rdiv[i] = dead ? 1.0f : amax * inv_bound;
         }
     };
@@ -133,7 +157,10 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
     auto quantise_store = [&](int h, int i, int buf) {
         float y[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) y[j] = __builtin_rintf(v[i][j] * mul[i]) * rdiv[i];
+        for (int j = 0; j < 4; ++j) {
+            y[2 * j] = __builtin_rintf(u2f(vp[i][j] << 16) * mul[i]) * rdiv[i];
+            y[2 * j + 1] = __builtin_rintf(u2f(vp[i][j] & 0xFFFF0000u) * mul[i]) * rdiv[i];
+        }
         u32x4 o;
         o.x = f32x2_to_bf16x2(y[0], y[1]);
         o.y = f32x2_to_bf16x2(y[2], y[3]);
@@ -171,14 +198,15 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
     // bytes of chunk c of row t sit at ((c * T) + t) * 8, so the 32 lanes fr of a k-group read
     // 512 contiguous bytes.  Rows past T repeat row T - 1 (masked in the epilogue); T * K < 2^31
     // is checked by the launcher.
-    uint32_t aoff[RB];
+    uint32_t aoff[RB];  // in bytes, added to a wave-uniform address of the step
 #pragma unroll
     for (int mb = 0; mb < RB; ++mb) {
         int t = row_base + mb * 32 + fr;
         t = t < T ? t : T - 1;
-        aoff[mb] = ((uint32_t)kg * (uint32_t)T + (uint32_t)t) * 8u;
+        aoff[mb] = ((uint32_t)kg * (uint32_t)T + (uint32_t)t) * 16u;
     }
-    const uint32_t step_stride = 2u * (uint32_t)T * 8u;  // one step of 16 k = 2 chunks
+    const uint32_t step_stride = 2u * (uint32_t)T * 16u;  // one step of 16 k = 2 chunks, in bytes
+    const char* xab = (const char*)xa;
     const int steps = nkb * 8;
     // activation fragments are fetched this many steps ahead (a divisor of the 8 steps of a k
     // block, so that a step's register slot j % PF is the same in every block)
@@ -189,7 +217,7 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
     for (int mb = 0; mb < RB; ++mb)
 #pragma unroll
         for (int j = 0; j < PF; ++j)
-            af[mb][j] = *(const u32x4*)(xa + aoff[mb] + (uint32_t)j * step_stride);
+            af[mb][j] = *(const u32x4*)(xab + (uint32_t)j * step_stride + aoff[mb]);
 
     // ---- prologue: tile 0 into buffer 0, raw weights of block 1 in flight
     fetch(0);
@@ -225,9 +253,10 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
             }
             int g = kb * 8 + j + PF;
             g = g < steps ? g : steps - 1;
+            const char* xstep = xab + (uint32_t)g * step_stride;   // wave-uniform
 #pragma unroll
             for (int mb = 0; mb < RB; ++mb)
-                af[mb][j % PF] = *(const u32x4*)(xa + aoff[mb] + (uint32_t)g * step_stride);
+                af[mb][j % PF] = *(const u32x4*)(xstep + aoff[mb]);
             if constexpr (MORE) produce_slice(j, kb + 1, buf ^ 1);
         }
         __syncthreads();
@@ -319,7 +348,7 @@ extern "C" int mo_awq_search_losses(const void* xs, const void* w, const void* s
     else if (block_size == 64) lg_g = 3;
     else if (block_size == 128) lg_g = 4;
     if (lg_g < 0 || tokens > 512 || n % mo::kSearchTileN || k % mo::kSearchBlockK ||
-        n_alpha > 65535 || n > 0x7FFFFFFF || tokens * k > 0x7FFFFFFF ||
+        n_alpha > 65535 || n > 0x7FFFFFFF || tokens * k > 0x7FFFFFFF || k >= (1 << 24) ||
         (n_alpha + 8) * (n / mo::kSearchTileN) > 0x7FFFFFFF)
         return MO_ERR_UNSUPPORTED;
     if ((((uintptr_t)xs | (uintptr_t)w | (uintptr_t)s) & 15u) || ((uintptr_t)ref & 1u))

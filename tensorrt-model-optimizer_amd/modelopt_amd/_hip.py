@@ -92,7 +92,8 @@ def dtype_code(dt: torch.dtype) -> int:
 
 
 def _stream(t: torch.Tensor):
-    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+    """torch's current stream on the device of ``t`` as the C ABI takes it."""
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(t.device.index))
 
 
 def _ptr(t):
@@ -142,16 +143,19 @@ class KernelTimer:
 def call(name: str, anchor: torch.Tensor, *args):
     """Invoke ``name`` with the device of ``anchor`` current; raise on a non-zero status."""
     lib = load()
-    with torch.cuda.device(anchor.device):
-        if _timer is None:
-            rc = getattr(lib, name)(*args)
-        else:
-            start = torch.cuda.Event(enable_timing=True)
-            end = torch.cuda.Event(enable_timing=True)
-            start.record()
-            rc = getattr(lib, name)(*args)
-            end.record()
-            _timer.pairs.append((name, start, end))
+    if _timer is None and anchor.device.index == torch.cuda.current_device():
+        rc = getattr(lib, name)(*args)   # the common case, without the context manager's cost
+    else:
+        with torch.cuda.device(anchor.device):
+            if _timer is None:
+                rc = getattr(lib, name)(*args)
+            else:
+                start = torch.cuda.Event(enable_timing=True)
+                end = torch.cuda.Event(enable_timing=True)
+                start.record()
+                rc = getattr(lib, name)(*args)
+                end.record()
+                _timer.pairs.append((name, start, end))
     if rc != 0:
         msg = lib.mo_error_string(rc).decode()
         raise RuntimeError(f"{name} failed: {msg} (status {rc})")
@@ -321,7 +325,7 @@ def fused_scratch(device, stream=None):
     index = torch.device(device).index
     index = torch.cuda.current_device() if index is None else index
     if stream is None:
-        stream = torch.cuda.current_stream(index).cuda_stream
+        stream = torch._C._cuda_getCurrentRawStream(index)
     ws = _fused_ws_by_device.get((index, stream))
     if ws is None:
         ws = torch.zeros(FUSED_WS_BYTES // 4, dtype=torch.int32, device=torch.device("cuda", index))

@@ -68,12 +68,17 @@ class MaxCalibrator(_Calibrator):
         # the reference squeezes a one-element result to a scalar
         return torch.Size(()) if shape.numel() == 1 else shape
 
-    @torch.no_grad()
     def collect(self, x):
         """Fold the abs-max of ``x`` (over everything but ``axis``) into the running maximum.
 
         Raises ``RuntimeError`` when the amax shape differs from what was collected before.
         """
+        if torch.is_grad_enabled():
+            with torch.no_grad():
+                return self._collect(x)
+        return self._collect(x)
+
+    def _collect(self, x):
         reduce_axis = convert_quantization_axis_to_reduce_axis(x, self._axis)
         shape = self._amax_shape(x, reduce_axis)
         if x.device.type == "meta":

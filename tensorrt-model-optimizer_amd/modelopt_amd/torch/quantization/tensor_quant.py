@@ -227,6 +227,27 @@ class DynamicBlockQuantizationFunction(Function):
         return _backward(ctx, grad_outputs, 9)
 
 
-fake_tensor_quant = FakeTensorQuantFunction.apply
-scaled_e4m3 = ScaledE4M3Function.apply
-dynamic_block_quant = DynamicBlockQuantizationFunction.apply
+class _NoGraph:
+    """Stands in for the autograd context when nothing will be differentiated."""
+
+    @staticmethod
+    def save_for_backward(*tensors):
+        pass
+
+
+def _entry(function):
+    """``function.apply``, except that a call whose result cannot need a gradient (grad mode off,
+    or an input that does not require one) runs the forward directly: Function.apply costs
+    several microseconds of host time per quantizer call even then."""
+    def run(inputs, *args, **kwargs):
+        if torch.is_grad_enabled() and isinstance(inputs, torch.Tensor) and inputs.requires_grad:
+            return function.apply(inputs, *args, **kwargs)
+        return function.forward(_NoGraph, inputs, *args, **kwargs)
+    run.__name__ = function.__name__
+    run.__doc__ = function.__doc__
+    return run
+
+
+fake_tensor_quant = _entry(FakeTensorQuantFunction)
+scaled_e4m3 = _entry(ScaledE4M3Function)
+dynamic_block_quant = _entry(DynamicBlockQuantizationFunction)
