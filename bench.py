@@ -344,6 +344,71 @@ def single_tensor_configs(torch, steps, warmup):
     return out
 
 
+def secondary_kernels(torch, steps, warmup):
+    """The library's other streaming kernels on the largest weight of a Llama-3-8B layer
+    (14336 x 4096 bf16) and on one calibration batch of activations (8192 x 4096 bf16): device
+    microseconds per launch and algorithmic bytes per second against the 8 TB/s HBM peak."""
+    from modelopt_amd import _hip
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(2)
+    out = {}
+
+    def rec(name, fn, nbytes):
+        # one event pair around a train of launches: these kernels run for 5 - 50 us, which a
+        # pair of events per launch would inflate
+        reps = max(steps, 50)
+        for _ in range(max(warmup, 10)):
+            fn()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(end) / reps
+        out[name] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / ms / 1e6, 1),
+                     "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 3)}
+
+    n_rows, k = 14336, 4096
+    w = torch.randn(n_rows, k, device=dev, generator=g).mul_(0.02).to(torch.bfloat16)
+    n = w.numel()
+    y = torch.empty_like(w)
+    blk = torch.zeros(n // 128, dtype=torch.float32, device=dev)
+    _hip.absmax_into(w, blk, 1, n // 128, 128)
+    ws = blk.reshape(n_rows, k // 128) / 7.0
+    s = torch.rand(k, device=dev, generator=g).add_(0.5).to(torch.bfloat16)
+    amax = w.abs().amax().float()
+    rec("int4_pack_rows_14336x4096", lambda: _hip.int4_pack_rows(w, ws), n * 2.5)
+    rec("int4_block_quantize_14336x4096", lambda: _hip.int4_block_quantize(w, 128), n * 2.5)
+    packed4, sc4 = _hip.int4_block_quantize(w, 128)
+    rec("int4_block_dequantize_14336x4096", lambda: _hip.int4_block_dequantize(packed4, sc4, 128), n * 2.5)
+    rec("scale_block_int_qdq_14336x4096", lambda: _hip.scale_block_int_qdq(w, s, 128, out=y), n * 4)
+    rec("mul_cols_14336x4096", lambda: _hip.mul_cols(w, s, out=y), n * 4)
+    col = torch.zeros(k, dtype=torch.float32, device=dev)
+    rec("abs_colsum_with_block_amax_14336x4096", lambda: _hip.abs_colsum_into(w, col, blk, 128), n * 2)
+    rec("fp8_qdq_14336x4096", lambda: _hip.fp8_qdq(w, amax, 1, 1, n, out=y), n * 4)
+    rec("int8_qdq_14336x4096", lambda: _hip.int_qdq(w, amax, 1, 1, n, 8, False, False, out=y), n * 4)
+    rec("nvfp4_qdq_14336x4096", lambda: _hip.nvfp4_qdq(w, amax, out=y), n * 4)
+    pk, wsf, wsf2 = _hip.nvfp4_quantize(w, amax, 16)
+    rec("nvfp4_dequantize_14336x4096", lambda: _hip.nvfp4_dequantize(pk, wsf, wsf2, 16, torch.bfloat16),
+        n * DEQUANT_BYTES_PER_ELEM)
+    del y, pk, wsf, packed4
+
+    for t in (512, 8192):
+        x = torch.randn(t, k, device=dev, generator=g).to(torch.bfloat16)
+        b = torch.randn(t, k, device=dev, generator=g).to(torch.bfloat16)
+        m = x.numel()
+        a1 = torch.zeros(1, dtype=torch.float32, device=dev)
+        ak = torch.zeros(k, dtype=torch.float32, device=dev)
+        a64 = torch.zeros(1, dtype=torch.float64, device=dev)
+        rec(f"abs_colsum_{t}x4096", lambda: _hip.abs_colsum_into(x, ak), m * 2)
+        rec(f"absmax_per_tensor_{t}x4096", lambda: _hip.absmax_into(x, a1, 1, 1, m), m * 2)
+        rec(f"absmax_per_column_{t}x4096", lambda: _hip.absmax_into(x, ak, t, k, 1), m * 2)
+        rec(f"sq_diff_sum_{t}x4096", lambda: _hip.sq_diff_sum_into(x, b, a64), m * 4)
+    return out
+
+
 def calib_sweep(torch, layers, n_seqs, batch, seq_len=512):
     """Calibration sweep configuration: mtq.quantize (NVFP4 weights + inputs, FP8 KV cache, max calibration) on
     a random-init Llama-3-8B-shaped decoder over n_seqs x 512 uniform-random token ids.  Reports
@@ -535,6 +600,24 @@ def main():
         extras["amax_plus_quantize_pipeline"] = {
             "ms": round(w_ms, 4),
             "GBps": round(elems * (AMAX_BYTES_PER_ELEM + QUANT_BYTES_PER_ELEM) / w_ms / 1e6, 1)}
+        # does a tensor that was just read come back faster (from the 256 MB memory-side cache)?
+        # abs-max of one 117 MB weight over and over, against the same kernel walking through the
+        # same-shaped weight of every layer (each last touched gigabytes ago)
+        big = max(range(len(LAYER_SHAPES)), key=lambda j: weights[j].numel())
+        same = [weights[big]] * a.layers
+        each = [weights[l * len(LAYER_SHAPES) + big] for l in range(a.layers)]
+        acc1 = torch.zeros(1, dtype=torch.float32, device=dev)
+
+        def reread(ts):
+            for t in ts:
+                _hip.absmax_into(t, acc1, 1, 1, t.numel())
+        _, warm_ms = timed(torch, lambda: reread(same), 5, 2)
+        _, cold_ms = timed(torch, lambda: reread(each), 5, 2)
+        extras["reread_of_one_weight"] = {
+            "bytes": weights[big].numel() * 2,
+            "just_read_us": round(warm_ms / a.layers * 1e3, 2),
+            "read_long_ago_us": round(cold_ms / a.layers * 1e3, 2)}
+
         # dequant round trip on the first layer's tensors
         packed, wsf, wsf2 = qplan.run()
         n1 = len(LAYER_SHAPES)
@@ -577,6 +660,7 @@ def main():
 
         with contextlib.redirect_stdout(sys.stderr):   # the calibration algorithms print progress
             extras["single_tensor_configs"] = single_tensor_configs(torch, a.steps, a.warmup)
+        extras["secondary_kernels"] = secondary_kernels(torch, a.steps, a.warmup)
         out["extras"] = extras
 
     if not a.no_calib_sweep:

@@ -1,6 +1,11 @@
 """Build libmodelopt_hip.so for gfx950 with hipcc (in-tree, next to this file).
 
-Usage: ``python build.py [-j N] [--force]``.  Also importable: ``build(force=False)``.
+Usage: ``python build.py [-j N] [--force] [--tuning]``.  Also importable: ``build(force=False)``.
+
+``--tuning`` builds libmodelopt_hip_tuning.so instead, compiled with -DMO_TUNING: in that build
+the per-kernel occupancy caps (unused dynamic LDS) are read from the environment at every launch
+(``MO_BALLAST_<kernel>`` or ``MO_BALLAST_ALL``, in KiB), which is how the caps compiled into the
+product library were chosen.  ``MODELOPT_AMD_LIB=<path>`` makes the Python layer load that file.
 """
 
 import argparse
@@ -37,30 +42,34 @@ def _stale(out, deps):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def _compile(src, force):
-    out = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+def _compile(src, force, obj_dir, extra):
+    out = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
     path = os.path.join(CSRC, src)
     if not force and not _stale(out, [path, *HEADERS]):
         return out
-    cmd = ["hipcc", *FLAGS, "-x", "hip", "-c", path, "-o", out]
+    cmd = ["hipcc", *FLAGS, *extra, "-x", "hip", "-c", path, "-o", out]
     subprocess.run(cmd, check=True)
     return out
 
 
-def build(force=False, jobs=4):
-    os.makedirs(OBJ, exist_ok=True)
+def build(force=False, jobs=4, tuning=False):
+    obj_dir = os.path.join(OBJ, "tuning") if tuning else OBJ
+    lib = LIB.replace(".so", "_tuning.so") if tuning else LIB
+    extra = ["-DMO_TUNING"] if tuning else []
+    os.makedirs(obj_dir, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(lambda s: _compile(s, force), _sources()))
-    if force or _stale(LIB, objs):
-        subprocess.run(["hipcc", "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-o", LIB],
+        objs = list(ex.map(lambda s: _compile(s, force, obj_dir, extra), _sources()))
+    if force or _stale(lib, objs):
+        subprocess.run(["hipcc", "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-o", lib],
                        check=True)
-    return LIB
+    return lib
 
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("-j", type=int, default=4)
     ap.add_argument("--force", action="store_true")
+    ap.add_argument("--tuning", action="store_true")
     a = ap.parse_args()
-    print(build(a.force, a.j))
+    print(build(a.force, a.j, a.tuning))
     sys.exit(0)

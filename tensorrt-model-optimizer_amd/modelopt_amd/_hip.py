@@ -10,7 +10,9 @@ import os
 import torch
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_PKG_DIR), "libmodelopt_hip.so")
+# MODELOPT_AMD_LIB names another build of the same library (e.g. the tuning build of build.py)
+LIB_PATH = os.environ.get("MODELOPT_AMD_LIB") or os.path.join(os.path.dirname(_PKG_DIR),
+                                                              "libmodelopt_hip.so")
 
 MO_F32, MO_F16, MO_BF16 = 0, 1, 2
 # per-call flags of the NVFP4 quantize entry points (enum mo_quantize_flags)
