@@ -36,12 +36,13 @@ qtensor.nvfp4_*                        test_qtensor_cuda.py:287-375 (values/pack
                                        (brute-force twin of the FP4 cast); oracle/c cross-check
 qtensor.int4_* / int8_* / fp8_*        golden bf16 vectors test_qtensor_cuda.py:133-241
 export.get_scaling_factor_from_weight  exact vectors tests/gpu/torch/export/test_export.py:163-197
-export.pack_int4_in_uint8              PARITY UNPINNED by reference tests (no golden vector
-                                       exists); pinned only by brute force on tiny inputs and
-                                       the unpack(pack(q)) == q invariant
-export.fp8_export_cast                 PARITY UNPINNED by reference tests; pinned by the torch
-                                       type-promotion rule probed in tests (bf16 / 0-dim fp32)
-export.int8_export_cast                PARITY UNPINNED by reference tests; float64 closed form
+export.pack_int4_in_uint8 /            no reference test holds a vector for these, so
+export.fp8_export_cast /               tests/golden/export_vectors.json records what the reference's
+export.int8_export_cast                own pack_int4_in_uint8 and to_quantized_weight
+                                       (export/quant_utils.py:697-774) return on seeded inputs (2-D and
+                                       3-D weights, ties, clamped values, asymmetric nibbles that tell the
+                                       two nibble orders apart, bf16 / 0-dim fp32 promotion); written by
+                                       tests/golden/make_export_vectors.py in the build container
 export.nvfp4_export                    composition of the pinned qtensor.nvfp4_* functions
 fake_quant.static_block_fake_quant     float64 closed form (tests/test_oracle_search.py)
 nf4.nf4_quantize / double_quantization golden round trips test_qtensor_cuda.py:111-131 (with and

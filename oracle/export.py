@@ -24,7 +24,7 @@ def get_scaling_factor_from_weight(weight: torch.Tensor, group_size: int):
 def pack_int4_in_uint8(weight: torch.Tensor, wsf: torch.Tensor):
     """INT4-AWQ export pack.  Follows export/quant_utils.py:697-738.
 
-    PARITY UNPINNED by reference tests (no golden vector exists for this function).
+    Pinned by tests/golden/export_vectors.json (outputs of the reference's own function).
     ``q = int8(clamp(round_rne(w / wsf[:, k // bs]), -8, 7))`` (bf16 / fp32 tensor -> fp32
     division); two's-complement nibbles of *adjacent output rows* share a byte:
     ``byte[j, k] = (q[2j, k] & 0xF) | (q[2j+1, k] << 4)``; result uint8 [N/2, K]
@@ -60,7 +60,8 @@ def fp8_export_cast(weight: torch.Tensor, wsf: torch.Tensor):
     """FP8 per-tensor export cast.  Follows export/quant_utils.py:759-771 with the scale of
     export/unified_export_hf.py:260-269 (``f32(amax) / 448``, 0-dim or 1-element fp32).
 
-    PARITY UNPINNED by reference tests.  ``weight / wsf`` follows torch type promotion: a bf16
+    Pinned by tests/golden/export_vectors.json (outputs of the reference's own
+    ``to_quantized_weight``).  ``weight / wsf`` follows torch type promotion: a bf16
     tensor divided by a 0-dim fp32 tensor gives a **bf16** tensor (fp32 quotient rounded to
     bf16), which is then rounded a second time to E4M3; with a dim>=1 fp32 scale the quotient
     stays fp32 and is rounded once.

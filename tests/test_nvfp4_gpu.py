@@ -266,3 +266,34 @@ def test_two_full_llama3_8b_layers_through_the_multi_tensor_launches():
         assert float(wsf2[i]) == float(w2_c), what
         assert torch.equal(wsf[i].cpu().view(torch.uint8), w_c.view(torch.uint8)), what
         assert torch.equal(packed[i].cpu(), p_c), what
+
+
+def test_elements_on_rounding_boundaries_of_e2m1():
+    """Blocks whose quotients x / s sit exactly on, one bf16 step below and one step above every
+    rounding boundary of E2M1 (0.25, 0.75, ..., 5): the quotient has to be the correctly rounded
+    one for these, and ties go to the even code as in the oracle."""
+    bounds = [0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0]
+    rows = []
+    for scale_exp in (-6, -3, 0, 2):
+        for sign in (1.0, -1.0):
+            vals = []
+            for b in bounds:
+                t = torch.tensor(b * 2.0 ** scale_exp, dtype=torch.bfloat16)
+                bits = t.view(torch.int16)
+                vals += [t, (bits - 1).view(torch.bfloat16), (bits + 1).view(torch.bfloat16)]
+            blk = torch.stack(vals[:15] + [torch.tensor(6.0 * 2.0 ** scale_exp, dtype=torch.bfloat16)])
+            rows.append(sign * blk.float())
+            blk2 = torch.stack(vals[6:21] + [torch.tensor(6.0 * 2.0 ** scale_exp, dtype=torch.bfloat16)])
+            rows.append(sign * blk2.float())
+    x = torch.stack(rows).to(torch.bfloat16).reshape(4, -1)          # 16 blocks of 16
+    x = torch.cat([x, _rand((60, x.shape[1]), torch.bfloat16, seed=11)])   # plus ordinary rows
+    # the global scale that puts the values exactly on the boundaries, and one slightly off
+    for w2 in (torch.tensor(24.0 / 2688.0), torch.tensor(0.0091)):
+        w2 = w2.to(torch.float32)
+        po, wo, _ = qtensor.nvfp4_quantize(x, 16, wsf2=w2)
+        packed, wsf, _ = _hip.nvfp4_quantize(x.to(DEV), w2.to(DEV), 16, amax_is_wsf2=True)
+        p_exact, w_exact, _ = _hip.nvfp4_quantize(x.to(DEV), w2.to(DEV), 16, amax_is_wsf2=True,
+                                                  flags=_hip.MO_FLAG_FORCE_EXACT)
+        assert torch.equal(packed, p_exact) and torch.equal(wsf.view(torch.uint8), w_exact.view(torch.uint8))
+        assert_bits_equal(packed.cpu(), po, "codes on rounding boundaries")
+        assert_bits_equal(wsf.cpu(), wo, "scales on rounding boundaries")
