@@ -41,6 +41,10 @@ struct IntOp {
     struct Scale { float mul, div, rdiv; bool fast; };
     __device__ __forceinline__ Scale make(float amax) const {
         Scale s;
+        // the CPU path's rule (tensor_quant.py:574-612): amax <= 2^-24 zeroes the scale and divides
+        // by 1, so a dead channel gives rint(x * 0) -- -0.0 for negative x, NaN for inf / NaN.
+        // (The reference's CUDA kernel uses amax < 2^-24 and returns +0.0; parity here is with
+        // the CPU path.)
         const bool dead = amax <= 5.9604644775390625e-8f;  // 2^-24
         const float sc = bound / amax;
         s.mul = dead ? 0.0f : sc;

@@ -108,6 +108,23 @@ def _require_device(*tensors):
             raise RuntimeError("modelopt_amd kernels need tensors in GPU memory (got a CPU tensor)")
 
 
+_staging = {}  # (device index, raw stream) -> int32 buffer for the two-pass reducers
+
+
+def _staging_words(anchor: torch.Tensor, words: int) -> torch.Tensor:
+    """``words`` 4-byte words of scratch memory on the device of ``anchor`` for a kernel pair that
+    runs on torch's current stream there.  One buffer per (device, stream), grown when needed and
+    reused by later calls: calls in one stream follow each other, so they can share it, and the
+    calibration loop allocates nothing per call."""
+    index = anchor.device.index
+    key = (index, torch._C._cuda_getCurrentRawStream(index))
+    buf = _staging.get(key)
+    if buf is None or buf.numel() < words:
+        buf = torch.empty(max(words, 1 << 18), dtype=torch.int32, device=anchor.device)
+        _staging[key] = buf
+    return buf
+
+
 _timer = None  # the active KernelTimer, if any
 
 
@@ -176,7 +193,7 @@ def absmax_into(x: torch.Tensor, acc: torch.Tensor, outer: int, axis: int, inner
         # accumulator is not hit by one atomic per column from every workgroup
         across = -(-axis // 2048) if axis >= 2048 else -(-axis // 512)
         slabs = max(1, min(-(-1024 // across), outer // 32))
-        partial = torch.empty((slabs, axis), dtype=torch.int32, device=x.device)
+        partial = _staging_words(x, slabs * axis)
         call("mo_absmax_cols_staged", x, _ptr(x), outer, axis, dtype_code(x.dtype), _ptr(acc),
              _ptr(partial), slabs, _stream(x))
         return acc
@@ -605,7 +622,7 @@ def abs_colsum_into(x, acc, blk_amax=None, block_size=0):
         # two passes, no atomics: enough row slabs to fill the chip, at least 16 rows each
         across = -(-k // 2048)
         slabs = max(1, min(-(-1024 // across), rows // 16))
-        partial = torch.empty((slabs, k), dtype=torch.float32, device=x.device)
+        partial = _staging_words(x, slabs * k)
         call("mo_abs_colsum_staged", x, _ptr(x), rows, k, dtype_code(x.dtype), _ptr(blk_amax),
              block_size, _ptr(acc), _ptr(partial), slabs, _stream(x))
         return acc
@@ -639,6 +656,24 @@ def _tile_job_map(tiles_per_job, device):
     return torch.repeat_interleave(torch.arange(len(tiles_per_job), dtype=torch.int32), counts).to(device)
 
 
+class _PinnedInputs:
+    """The input tensors of a multi-tensor plan.  The job table holds raw addresses, so the plan
+    keeps the tensors' storages alive (the addresses can never point at freed memory) and
+    ``verify`` raises when a tensor has been given other memory since the plan was built
+    (``param.data = ...``, ``.to()``): the plan would then read the old contents."""
+
+    def __init__(self, tensors):
+        self.tensors = list(tensors)
+        self._storages = [t.untyped_storage() for t in self.tensors]
+        self._addresses = [t.data_ptr() for t in self.tensors]
+
+    def verify(self):
+        for i, t in enumerate(self.tensors):
+            if t.data_ptr() != self._addresses[i]:
+                raise RuntimeError(f"tensor {i} of the plan was reallocated after the plan was "
+                                   "built; build a new plan")
+
+
 class AbsmaxPlan:
     """Per-tensor abs-max of a fixed list of tensors in one launch.
 
@@ -646,8 +681,9 @@ class AbsmaxPlan:
     Every tile folds into an accumulator with an atomic max, and atomics that hit one cache line
     are served one after the other; so a tensor is cut into spans of ``SPAN_TILES`` tiles, each
     span is a job with an accumulator of its own on a separate 256-byte line, and ``run`` ends
-    with a small reduction over the spans of each tensor.  The plan keeps the tensors alive and
-    must be rebuilt if any is reallocated.
+    with a small reduction over the spans of each tensor.  The plan keeps the tensors' memory
+    alive; ``run`` checks that none has been reallocated (``verify=False`` skips the check of
+    about 0.15 us per tensor, for a caller that has just built or verified the plan).
     """
 
     SPAN_TILES = 64
@@ -656,7 +692,8 @@ class AbsmaxPlan:
     def __init__(self, tensors):
         assert len(tensors) > 0
         dev, dt = tensors[0].device, tensors[0].dtype
-        self.tensors = list(tensors)
+        self._inputs = _PinnedInputs(tensors)
+        self.tensors = self._inputs.tensors
         self.dtype = dtype_code(dt)
         esize = tensors[0].element_size()
         span_elems = self.SPAN_TILES * ABSMAX_TILE_ELEMS
@@ -679,7 +716,12 @@ class AbsmaxPlan:
         self.jobs = _job_table(rows, dev)
         self.tile_job = _tile_job_map(per_job, dev)
 
-    def run(self, zero=True):
+    def verify(self):
+        self._inputs.verify()
+
+    def run(self, zero=True, verify=True):
+        if verify:
+            self._inputs.verify()
         if zero:
             self._lines.zero_()
         call("mo_absmax_multi", self.acc, _ptr(self.jobs), self.njobs, _ptr(self.tile_job),
@@ -693,12 +735,14 @@ class Nvfp4QuantizePlan:
 
     ``amax`` is a float32 device vector (any stride) with one global amax (or wsf2 when
     ``amax_is_wsf2``) per tensor.  Outputs are allocated once here: ``packed[i]`` uint8 [..., K/2], ``wsf[i]``
-    float8_e4m3fn [..., K/16], ``wsf2`` float32 [n].
+    float8_e4m3fn [..., K/16], ``wsf2`` float32 [n].  The plan keeps the inputs' memory alive and
+    ``run`` checks that no input (or the amax vector) has been reallocated (``verify=False`` skips it).
     """
 
     def __init__(self, tensors, amax, amax_is_wsf2=False, flags=0):
         assert len(tensors) > 0 and amax.dtype == torch.float32 and amax.numel() == len(tensors)
         dev = tensors[0].device
+        self._inputs = _PinnedInputs(list(tensors) + [amax])
         self.tensors, self.amax, self.amax_is_wsf2 = list(tensors), amax, bool(amax_is_wsf2)
         self.flags = int(flags)
         self.wsf2 = torch.empty(len(tensors), dtype=torch.float32, device=dev)
@@ -733,7 +777,12 @@ class Nvfp4QuantizePlan:
         self.tile_job = _tile_job_map(per_job, dev)
         self.wsf = [w.view(torch.float8_e4m3fn) for w in self._wsf_u8]
 
-    def run(self):
+    def verify(self):
+        self._inputs.verify()
+
+    def run(self, verify=True):
+        if verify:
+            self._inputs.verify()
         call("mo_nvfp4_quantize_multi", self.amax, _ptr(self.jobs), len(self.tensors),
              _ptr(self.tile_job), self.total_tiles, MO_BF16, 16, int(self.amax_is_wsf2),
              self.flags, _stream(self.amax))

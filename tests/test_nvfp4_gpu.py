@@ -297,3 +297,21 @@ def test_elements_on_rounding_boundaries_of_e2m1():
         assert torch.equal(packed, p_exact) and torch.equal(wsf.view(torch.uint8), w_exact.view(torch.uint8))
         assert_bits_equal(packed.cpu(), po, "codes on rounding boundaries")
         assert_bits_equal(wsf.cpu(), wo, "scales on rounding boundaries")
+
+
+def test_plans_refuse_inputs_that_were_reallocated():
+    """The job tables hold raw addresses: a parameter that is given new memory after the plan was
+    built (``param.data = ...``) makes ``run`` raise instead of reading the old memory, which the
+    plan keeps alive."""
+    ws = [torch.nn.Parameter(_rand((64, 256), torch.bfloat16, seed=i).to(DEV), requires_grad=False) for i in range(3)]
+    aplan = _hip.AbsmaxPlan(ws)
+    acc = aplan.run().clone()
+    qplan = _hip.Nvfp4QuantizePlan(ws, acc)
+    before = [p.clone() for p in qplan.run()[0]]
+    ws[1].data = ws[1].data.clone() * 2
+    with pytest.raises(RuntimeError, match="reallocated"):
+        aplan.run()
+    with pytest.raises(RuntimeError, match="reallocated"):
+        qplan.run()
+    after = qplan.run(verify=False)[0]      # still the old memory, still valid
+    assert all(torch.equal(a, b) for a, b in zip(before, after))

@@ -127,6 +127,19 @@ def test_int_tiny_amax_channel_is_zero():
     assert_bits_equal(y, fake_quant.tensor_quant(x, amax.reshape(1, 3, 1), 8, False, True), "tiny")
 
 
+def test_int_dead_channel_follows_the_cpu_path():
+    """amax exactly 2^-24 counts as dead (``<=``), a dead channel gives ``rint(x * 0) / 1``: -0.0
+    for negative inputs and NaN for infinite ones, as the reference's CPU path does."""
+    x = torch.tensor([[0.5, -0.5, float("inf"), -0.0, 1e-9, -1e-9, float("-inf"), 3.0]] * 3).reshape(1, 3, 8)
+    amax = torch.tensor([2.0 ** -24, 2.0 ** -23, 1.0])
+    want = fake_quant.tensor_quant(x, amax.reshape(1, 3, 1), 8, False, True)
+    got = _hip.int_qdq(x.to(DEV), amax.to(DEV), 1, 3, 8, 8, False, True).cpu()
+    assert_bits_equal(got, want, "dead channel")
+    assert torch.signbit(got[0, 0, 1]) and got[0, 0, 1] == 0      # -0.5 -> -0.0
+    assert torch.isnan(got[0, 0, 2]) and torch.isnan(got[0, 0, 6])   # inf * 0
+    assert got[0, 1, 0] != 0                                       # 2^-23 is alive
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("k", [256, 200])
 def test_int4_static_block128_like_awq_weight(dtype, k):
