@@ -109,11 +109,16 @@ class MaxCalibrator(_Calibrator):
         self._meta_amax = None
         self._validated = False
 
+    def has_amax(self) -> bool:
+        """Whether ``compute_amax`` would return something, without computing it."""
+        return self._acc is not None or self._meta_amax is not None
+
     def compute_amax(self):
         """Running abs-max in the dtype of the collected tensors, or None if nothing was seen."""
         if self._acc is None:
             return self._meta_amax
-        amax = self._acc.to(self._dtype).reshape(self._shape)
+        # always a tensor of its own (never a view of the accumulator)
+        amax = self._acc.to(self._dtype, copy=True).reshape(self._shape)
         if not self._validated:
             bad = torch.stack([(self._acc < 0).any(), torch.isinf(self._acc).any(),
                                torch.isnan(self._acc).any()]).tolist()  # one host sync

@@ -69,9 +69,12 @@ def finish_stats_collection(model: nn.Module, method: str | None = None):
             continue
         cal = getattr(module, "_calibrator", None)
         if cal and not getattr(module, "_dynamic", False):
-            found = cal.compute_amax() if method != "mse" or isinstance(cal, MaxCalibrator) \
-                else cal.compute_amax(False)
-            if found is not None:
+            if type(cal) is MaxCalibrator:
+                found = cal.has_amax()   # load_calib_amax computes it; not twice
+            else:
+                found = (cal.compute_amax() if method != "mse" or isinstance(cal, MaxCalibrator)
+                         else cal.compute_amax(False)) is not None
+            if found:
                 module.load_calib_amax()
         module.enable_quant()
         module.disable_calib()

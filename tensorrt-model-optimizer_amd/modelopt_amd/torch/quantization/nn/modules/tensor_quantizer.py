@@ -298,10 +298,14 @@ class TensorQuantizer(nn.Module):
             warnings.warn(msg)
             warnings.warn("Set amax to NaN!")
             calib_amax = torch.tensor(math.nan)
-        if not hasattr(self, "_amax"):
-            self.register_buffer("_amax", calib_amax.clone().detach())
+        if type(self._calibrator) is calib.MaxCalibrator and calib_amax.device.type != "meta":
+            fresh = calib_amax.detach()          # already a tensor of its own
         else:
-            self._amax.data.copy_(calib_amax.clone().detach())
+            fresh = calib_amax.clone().detach()
+        if not hasattr(self, "_amax"):
+            self.register_buffer("_amax", fresh)
+        else:
+            self._amax.data.copy_(fresh)
 
     def _get_amax(self, inputs):
         """The calibrated ``_amax`` buffer, or the abs-max of ``inputs`` computed now."""

@@ -129,18 +129,24 @@ def update_quant_cfg_with_kv_cache_quant(quant_cfg: dict, kv_cache_quant_cfg: di
 def all_valid_scales(tensors) -> bool:
     """True when every element of every tensor is finite and non-negative -- one device
     reduction and one host synchronisation for the whole list."""
-    flat = [t.detach().reshape(-1).to(torch.float32) for t in tensors
-            if isinstance(t, torch.Tensor) and not t.is_meta and t.numel()]
-    if not flat:
+    groups = {}   # one concatenation per (device, dtype): no per-tensor conversion
+    for t in tensors:
+        if isinstance(t, torch.Tensor) and not t.is_meta and t.numel():
+            t = t.detach()
+            if not t.is_floating_point():
+                t = t.to(torch.float32)
+            groups.setdefault((t.device, t.dtype), []).append(t.reshape(-1))
+    if not groups:
         return True
-    by_device = {}
-    for t in flat:
-        by_device.setdefault(t.device, []).append(t)
     flags = []
-    for group in by_device.values():
-        v = torch.cat(group)
+    for group in groups.values():
+        v = torch.cat(group) if len(group) > 1 else group[0]
         flags.append((torch.isfinite(v) & (v >= 0)).all())
-    return all(bool(f) for f in flags)
+    # one synchronisation per device at most: flags on one device are combined first
+    by_device = {}
+    for f in flags:
+        by_device.setdefault(f.device, []).append(f)
+    return all(bool(torch.stack(fs).all()) if len(fs) > 1 else bool(fs[0]) for fs in by_device.values())
 
 
 @contextlib.contextmanager
