@@ -529,3 +529,30 @@ def test_dense_flat_view_covers_permuted_blocks_only():
         assert v is not None and v.dim() == 1 and sorted(v.tolist()) == sorted(t.flatten().tolist())
     for t in (x[:, :2], x[..., ::2], x.transpose(1, 2)[:, :, :2], x[0, 0].expand(3, 4, 5)):
         assert dense_flat_view(t) is None
+
+
+def test_all_valid_scales_groups_by_dtype_and_skips_what_is_not_a_tensor():
+    from modelopt_amd.torch.quantization.utils import all_valid_scales
+    ok = [torch.ones(3), torch.ones(2, dtype=torch.bfloat16), None, torch.tensor(2), torch.empty(0)]
+    assert all_valid_scales(ok) and all_valid_scales([])
+    assert not all_valid_scales(ok + [torch.tensor([1.0, -1.0], dtype=torch.bfloat16)])
+    assert not all_valid_scales([torch.tensor([float("nan")])])
+    assert not all_valid_scales([torch.tensor([float("inf")], dtype=torch.float16), torch.ones(1)])
+
+
+def test_max_calibrator_reports_whether_it_has_seen_anything_without_computing():
+    from modelopt_amd.torch.quantization import calib
+    c = calib.MaxCalibrator(8, None, False)
+    assert not c.has_amax() and c.compute_amax() is None
+    c.collect(torch.empty(4, 4, device="meta"))
+    assert c.has_amax() and c.compute_amax().is_meta
+
+
+def test_plan_inputs_notice_a_reallocated_tensor():
+    from modelopt_amd import _hip
+    a, b = torch.nn.Parameter(torch.zeros(8)), torch.zeros(8)
+    pinned = _hip._PinnedInputs([a, b])
+    pinned.verify()
+    a.data = torch.ones(8)
+    with pytest.raises(RuntimeError, match="reallocated"):
+        pinned.verify()
