@@ -191,8 +191,10 @@ def absmax_into(x: torch.Tensor, acc: torch.Tensor, outer: int, axis: int, inner
     if inner == 1 and axis % 8 == 0 and outer >= 64 and x.data_ptr() % 16 == 0:
         # per column over many rows: row slabs go to a small workspace first, so that a fresh
         # accumulator is not hit by one atomic per column from every workgroup
+        # about two workgroups per compute unit in all, 32 rows or more per slab (measured best
+        # from 17 MB to 537 MB)
         across = -(-axis // 2048) if axis >= 2048 else -(-axis // 512)
-        slabs = max(1, min(-(-1024 // across), outer // 32))
+        slabs = max(1, min(-(-512 // across), outer // 32))
         partial = _staging_words(x, slabs * axis)
         call("mo_absmax_cols_staged", x, _ptr(x), outer, axis, dtype_code(x.dtype), _ptr(acc),
              _ptr(partial), slabs, _stream(x))
@@ -619,9 +621,10 @@ def abs_colsum_into(x, acc, blk_amax=None, block_size=0):
     big = rows * k >= ((1 << 22) if blk_amax is not None else (1 << 23))
     if (big and k % 8 == 0 and rows >= 64 and x.data_ptr() % 16 == 0 and acc.data_ptr() % 16 == 0
             and (blk_amax is None or (block_size > 0 and block_size % 8 == 0 and k % block_size == 0))):
-        # two passes, no atomics: enough row slabs to fill the chip, at least 16 rows each
+        # two passes, no atomics: about two workgroups per compute unit in all, at least 32 rows
+        # per slab (8192 x 4096: 14.0 us against 18.1 us with twice as many slabs)
         across = -(-k // 2048)
-        slabs = max(1, min(-(-1024 // across), rows // 16))
+        slabs = max(1, min(-(-512 // across), rows // 32))
         partial = _staging_words(x, slabs * k)
         call("mo_abs_colsum_staged", x, _ptr(x), rows, k, dtype_code(x.dtype), _ptr(blk_amax),
              block_size, _ptr(acc), _ptr(partial), slabs, _stream(x))
