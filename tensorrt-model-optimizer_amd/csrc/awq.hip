@@ -80,7 +80,8 @@ __global__ __launch_bounds__(256) void mul_cols_kernel(const void* __restrict__ 
 // y = T( clamp(rne(f32(xs) * scale), lo, bound) / scale ).
 // A lane owns a chunk of 8 columns; the G = bs / 8 lanes of a block share the amax by shuffles.
 // The division is the exact reciprocal-and-FMA quotient whenever the scale is mid-range.
-constexpr int kQdqTileChunks = 1024;
+constexpr int kQdqRounds = 4;          // chunks per lane (2 measures the same, 1 is 10 % slower)
+constexpr int kQdqTileChunks = 256 * kQdqRounds;
 
 template <int DT, bool VEC>
 __global__ __launch_bounds__(256) void scale_block_int_qdq_kernel(
@@ -89,14 +90,14 @@ __global__ __launch_bounds__(256) void scale_block_int_qdq_kernel(
     const int G = 1 << lg_g;
     const int64_t bs = (int64_t)G << 3;
     const int64_t kp = (k + bs - 1) / bs * bs, kc = kp >> 3, total = rows * kc;
-    // one workgroup per tile of 1024 chunks, 4 per lane; total and the tile size are multiples
+    // one workgroup per tile of 256 * kQdqRounds chunks; total and the tile size are multiples
     // of G, so the lanes of a block stay together and are all live or all idle
     const int64_t t0 = (int64_t)blockIdx.x * kQdqTileChunks + threadIdx.x;
-    int64_t r[4], c0[4];
-    RawChunk<DT> raw[4];
-    float v[4][8];
+    int64_t r[kQdqRounds], c0[kQdqRounds];
+    RawChunk<DT> raw[kQdqRounds];
+    float v[kQdqRounds][8];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < kQdqRounds; ++u) {
         const int64_t t = t0 + u * 256;
         r[u] = c0[u] = 0;
         zero_raw<DT>(raw[u]);
@@ -110,7 +111,7 @@ __global__ __launch_bounds__(256) void scale_block_int_qdq_kernel(
         }
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < kQdqRounds; ++u) {
         const bool live = t0 + u * 256 < total;
         if (VEC) unpack_raw<DT>(raw[u], v[u]);
         if (s && live) {
@@ -346,13 +347,16 @@ extern "C" int mo_mul_cols(const void* x, int64_t rows, int64_t k, int dtype, co
     const bool vec = (k % 8 == 0) && ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)s) & 15u) == 0);
     if (vec) {
         const int64_t gx = (k / 8 + 255) / 256;
-        int64_t gy = (4096 + gx - 1) / gx;
+        // about 8192 workgroups in all and 4 per CU resident: 6.0 - 6.2 TB/s from 67 MB to 235 MB
+        // (4096 workgroups lose 5 % on 14336-wide rows, 1024 lose 10 %)
+        const int64_t want = mo::tuned("mul_cols_workgroups", 8192);
+        int64_t gy = (want + gx - 1) / gx;
         int64_t slab = (rows + gy - 1) / gy;
         if (slab < 8) slab = 8;
         gy = (rows + slab - 1) / slab;
         if (gy > 65535) { gy = 65535; slab = (rows + gy - 1) / gy; gy = (rows + slab - 1) / slab; }
         dim3 grid((unsigned)gx, (unsigned)gy);
-#define CALL(DT) mo::mul_cols8_kernel<DT><<<grid, 256, mo::ballast_bytes("mul_cols8_kernel", 53), st>>>(x, rows, k, slab, s, s_dtype, y)
+#define CALL(DT) mo::mul_cols8_kernel<DT><<<grid, 256, mo::ballast_bytes("mul_cols8_kernel", 36), st>>>(x, rows, k, slab, s, s_dtype, y)
         DISPATCH_DT(dtype, CALL)
 #undef CALL
     } else {
@@ -418,7 +422,9 @@ extern "C" int mo_sq_diff_sum(const void* a, const void* b, int64_t n, int dtype
     hipStream_t st = (hipStream_t)stream;
     // every workgroup ends with one atomic on the same double: 8 chunks per lane before a second
     // workgroup is worth its atomic, and never more than 1024 of them
-    const unsigned g = mo::blocks_for_awq((n + 63) / 64, 1024);
+    // a grid-stride pass by two workgroups per CU: 5.5 - 6.7 TB/s from 134 MB to 470 MB of operands
+    // (1024 workgroups: 4.8 - 5.9, 4096: 3.8 - 5.4)
+    const unsigned g = mo::blocks_for_awq((n + 63) / 64, (unsigned)mo::tuned("sq_diff_workgroups", 512));
     const int vec = ((((uintptr_t)a | (uintptr_t)b) & 15u) == 0) ? 1 : 0;
 #define CALL(DT) mo::sq_diff_sum_kernel<DT><<<g, 256, mo::ballast_bytes("sq_diff_sum_kernel", 53), st>>>(a, b, n, vec, acc)
     DISPATCH_DT(dtype, CALL)

@@ -47,6 +47,19 @@ inline size_t ballast_bytes(const char* kernel, int kb) {
     return (size_t)kb << 10;
 }
 
+// A launch parameter (grid size, rows per slab ...): `value` in the product build; a build with
+// -DMO_TUNING reads MO_TUNE_<name> from the environment at every launch (sweeps only).
+inline int64_t tuned(const char* name, int64_t value) {
+#ifdef MO_TUNING
+    char key[160];
+    snprintf(key, sizeof key, "MO_TUNE_%s", name);
+    if (const char* e = getenv(key)) return atoll(e);
+#else
+    (void)name;
+#endif
+    return value;
+}
+
 __device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
 __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 
