@@ -497,8 +497,9 @@ def calib_sweep(torch, layers, n_seqs, batch, seq_len=512):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=15,
+                    help="untimed launches first: the first ten or so run slower (first touch of the outputs, clocks)")
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip amax / dequant side measurements")
