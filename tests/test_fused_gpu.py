@@ -1,4 +1,4 @@
-"""The one-launch abs-max -> quantize kernels (cooperative launch, the tensor read once) against
+"""The one-launch abs-max -> quantize kernels (all workgroups resident, the tensor read once) against
 the two-launch entry points and the CPU oracle, through the C ABI."""
 
 import pytest
@@ -112,7 +112,7 @@ def test_dynamic_quantizer_takes_the_fused_path():
 
 def test_a_wait_that_gives_up_ends_the_kernel_and_raises_the_flag():
     """With a spin limit of zero every workgroup that is not the last to arrive gives up at once:
-    all wavefronts exit, nothing is written, word 3 of the workspace reports it, and the next
+    all wavefronts exit, nothing is written, the flag word of the workspace reports it, and the next
     call works once the workspace has been cleared."""
     x = _rand((4096, 2048), seed=7).to(DEV)
     assert _hip.nvfp4_quantize_fused(x, spin_limit=0) is not None
