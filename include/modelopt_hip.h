@@ -242,10 +242,11 @@ int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs, const int32
  * stream do that); other kernels may share the device.
  * workspace: MO_FUSED_WS_BYTES of device memory, 128-byte aligned, all zero before the first
  *   call; it can be reused by calls that follow each other in one stream (calls that overlap
- *   must not share a workspace).  The 32-bit word at byte MO_FUSED_WS_FAIL_OFFSET is set to 1,
- *   and the outputs are not written, if a workgroup gave up waiting for the others after
- *   spin_limit polls (a safety net: no wavefront waits for ever); the caller zeroes the
- *   workspace after reading that flag.
+ *   must not share a workspace).  The 32-bit word at byte MO_FUSED_WS_FAIL_OFFSET is set to 1
+ *   if a workgroup gave up waiting for the others after spin_limit polls (a safety net: no
+ *   wavefront waits for ever); such a workgroup fills its share of the outputs with NaN (NaN
+ *   block-scale bytes for NVFP4) instead of results.  The caller zeroes the workspace after
+ *   reading that flag.
  * amax_out (optional): the abs-max that was used, as fp32. */
 
 #define MO_FUSED_WS_BYTES 512

@@ -211,7 +211,20 @@ __global__ __launch_bounds__(256) void fused_amax_qdq_kernel(
     const uint32_t tb = f2u(tail) & 0x7FFFFFFFu;
     bits = tb > bits ? tb : bits;
     uint32_t gbits;
-    if (!grid_max_exchange(ws, bits, gridDim.x, spin_limit, smem, gbits)) return;
+    if (!grid_max_exchange(ws, bits, gridDim.x, spin_limit, smem, gbits)) {
+        // gave up waiting: fill this workgroup's share of the output with NaN, so that a caller
+        // who does not look at the flag sees a loud failure instead of uninitialised memory
+        float nan8[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) nan8[j] = __builtin_nanf("");
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t c = ((int64_t)u * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
+            if (c < chunks) store_chunk<DT>(y, c << 3, nan8);
+        }
+        if (has_tail) store_elem<DT>(y, (chunks << 3) + threadIdx.x, __builtin_nanf(""));
+        return;
+    }
     if (amax_out && blockIdx.x == 0 && threadIdx.x == 0) amax_out[0] = u2f(gbits);
     const typename Op::Scale s0 = op.make(u2f(gbits));
 #pragma unroll

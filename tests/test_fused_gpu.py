@@ -115,8 +115,16 @@ def test_a_wait_that_gives_up_ends_the_kernel_and_raises_the_flag():
     all wavefronts exit, nothing is written, the flag word of the workspace reports it, and the next
     call works once the workspace has been cleared."""
     x = _rand((4096, 2048), seed=7).to(DEV)
-    assert _hip.nvfp4_quantize_fused(x, spin_limit=0) is not None
+    got = _hip.nvfp4_quantize_fused(x, spin_limit=0)
+    assert got is not None
     torch.cuda.synchronize()
+    # the workgroups that gave up mark their blocks: NaN scale bytes (only the last one to arrive
+    # can have written real scales)
+    assert int((got[1].view(torch.uint8) == 0x7F).sum()) > 0
+    y = torch.empty_like(x)
+    assert _hip.fused_amax_qdq(x, "fp8", out=y, spin_limit=0) is not None
+    torch.cuda.synchronize()
+    assert int(torch.isnan(y).sum()) > 0
     assert _hip.fused_gave_up(DEV)                 # clears the workspace
     assert int(_hip.fused_scratch(DEV).abs().sum()) == 0
     packed, wsf, wsf2, _ = _hip.nvfp4_quantize_fused(x)
