@@ -419,15 +419,17 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* smem) {
 //   line 1  running maximum, an abs-max bit pattern (back to 0 likewise)
 //   line 2  64-bit {generation, result}: the last workgroup to arrive publishes the maximum
 //           together with a generation one higher than the one every workgroup read on entry
-//   line 3  set to 1 when a wait gave up
+//   line 3  set to 1 when a wait gave up; while it is set every later exchange fails at once
+//           (the count and the maximum of the abandoned exchange may still be in lines 0 and 1),
+//           until the host has cleared the workspace
 // Only these words cross workgroups and every access to them is a device-scope atomic performed
 // at the memory side, so relaxed ordering is enough (a release / acquire pair would write back
 // and invalidate caches on this multi-die part); program order between two atomics of a thread
 // is kept by waiting for the value the first one returns.
 // The wait is bounded: after `spin_limit` polls (one about every half microsecond) a workgroup
-// sets the flag, returns false and the kernel ends without writing its outputs, so that no
-// wavefront can stay behind for ever.  Calls that share a workspace must follow each other in
-// one stream.
+// sets the flag and returns false; the kernel then marks its share of the outputs (NaN) and
+// ends, so that no wavefront can stay behind for ever.  Calls that share a workspace must follow
+// each other in one stream.
 constexpr int kWsCount = 0, kWsMax = 32, kWsPublished = 64, kWsFail = 96;  // word offsets
 
 __device__ __forceinline__ bool grid_max_exchange(uint32_t* ws, uint32_t local, uint32_t nwg,
@@ -435,18 +437,25 @@ __device__ __forceinline__ bool grid_max_exchange(uint32_t* ws, uint32_t local, 
                                                   uint32_t& global) {
     unsigned long long* published = (unsigned long long*)(ws + kWsPublished);
     unsigned long long entry = 0;
-    if (threadIdx.x == 0)  // the generation of the previous exchange; issued ahead of the reduction
-        entry = __hip_atomic_load(published, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t poisoned = 0;
+    if (threadIdx.x == 0) {  // issued ahead of the reduction
+        entry = __hip_atomic_load(published, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // previous generation
+        poisoned = __hip_atomic_load(ws + kWsFail, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     const uint32_t m = block_max_u32(local, smem);
     if (threadIdx.x == 0) {
-        uint32_t old = 0;
-        if (m) old = __hip_atomic_fetch_max(ws + kWsMax, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("s_waitcnt vmcnt(0)" ::"v"(old), "v"(entry) : "memory");
-        const uint32_t before =
-            __hip_atomic_fetch_add(ws + kWsCount, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        bool ok = true;
-        uint32_t g;
-        if (before + 1 == nwg) {
+        asm volatile("s_waitcnt vmcnt(0)" ::"v"(poisoned), "v"(entry) : "memory");
+        bool ok = poisoned == 0;
+        uint32_t g = 0, before = 0;
+        if (ok) {
+            uint32_t old = 0;
+            if (m) old = __hip_atomic_fetch_max(ws + kWsMax, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::"v"(old) : "memory");
+            before = __hip_atomic_fetch_add(ws + kWsCount, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (!ok) {
+            // an earlier exchange on this workspace was abandoned: nothing in it can be trusted
+        } else if (before + 1 == nwg) {
             // last to arrive: every maximum has been applied.  Clean up, then publish.
             g = __hip_atomic_load(ws + kWsMax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::"v"(g) : "memory");

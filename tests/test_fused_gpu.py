@@ -125,6 +125,12 @@ def test_a_wait_that_gives_up_ends_the_kernel_and_raises_the_flag():
     assert _hip.fused_amax_qdq(x, "fp8", out=y, spin_limit=0) is not None
     torch.cuda.synchronize()
     assert int(torch.isnan(y).sum()) > 0
+    # until the host clears the workspace every further call on it fails the same loud way: the
+    # abandoned exchange may have left its count and maximum behind
+    y2 = torch.zeros_like(x)
+    assert _hip.fused_amax_qdq(x, "fp8", out=y2) is not None
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(y2).all())
     assert _hip.fused_gave_up(DEV)                 # clears the workspace
     assert int(_hip.fused_scratch(DEV).abs().sum()) == 0
     packed, wsf, wsf2, _ = _hip.nvfp4_quantize_fused(x)
