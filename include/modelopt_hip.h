@@ -245,8 +245,8 @@ int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs, const int32
  *   must not share a workspace).  The 32-bit word at byte MO_FUSED_WS_FAIL_OFFSET is set to 1
  *   if a workgroup gave up waiting for the others after spin_limit polls (a safety net: no
  *   wavefront waits for ever); such a workgroup fills its share of the outputs with NaN (NaN
- *   block-scale bytes for NVFP4) instead of results.  The caller zeroes the workspace after
- *   reading that flag.
+ *   block-scale bytes for NVFP4) instead of results, and so does every later call on that
+ *   workspace until the caller, having read the flag, has zeroed the workspace.
  * amax_out (optional): the abs-max that was used, as fp32. */
 
 #define MO_FUSED_WS_BYTES 512
