@@ -22,7 +22,7 @@ from .calib.max import MaxCalibrator
 from .conversion import set_quantizer_by_cfg_context
 from .nn import QuantModule, SequentialQuantizer, TensorQuantizer
 from .nn.modules.tensor_quantizer import calibration_pass
-from .utils import all_valid_scales, is_quantized_linear
+from .utils import all_valid_scales, deferred_scale_checks, is_quantized_linear
 
 __all__ = ["max_calibrate", "smoothquant", "awq", "awq_lite", "enable_stats_collection",
            "finish_stats_collection", "apply_pre_quant_scale_and_smooth",
@@ -156,14 +156,20 @@ def _apply_weight_pre_quant_scale(linear, pre_quant_scale):
 
 
 @torch.no_grad()
-def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.Tensor | None = None):
-    """Set the input ``pre_quant_scale`` and fold its inverse into the weight."""
+def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.Tensor | None = None,
+                                     _positive_later: list | None = None):
+    """Set the input ``pre_quant_scale`` and fold its inverse into the weight.  A caller that loops
+    over many layers passes ``_positive_later``: the scale is appended to it instead of being
+    checked for positivity here (a host synchronisation), and the caller checks them all at once."""
     assert is_quantized_linear(linear), "Only quantized linear modules are supported"
     assert linear.input_quantizer.pre_quant_scale is None, "pre_quant_scale should be None first!"
     if pre_quant_scale is None:
         pre_quant_scale = getattr(linear.input_quantizer, "_pre_quant_scale", None)
     assert pre_quant_scale is not None, "pre_quant_scale should be provided or already set"
-    assert torch.all(pre_quant_scale > 0), "pre_quant_scale should be positive"
+    if _positive_later is None:
+        assert torch.all(pre_quant_scale > 0), "pre_quant_scale should be positive"
+    else:
+        _positive_later.append(pre_quant_scale)
     pre_quant_scale = pre_quant_scale.to(torch.float32)  # fp32 keeps the scaling maths safe
 
     linear.input_quantizer._enable_pre_quant_scale = True
@@ -527,6 +533,7 @@ class _AWQLiteHelper:
         self.best_scale = None
         self.best_alpha = None
         self.exponent_columns = None  # device copies of alpha and 1 - alpha, made on first search step
+        self.scale_grid = None        # (fp32 scales [n_alphas, K], weight-dtype copy, inverse) of the search
         self.is_input_quantized = module.input_quantizer.is_enabled
         self.num_tokens = 0
         self.module = module
@@ -620,9 +627,13 @@ def _awq_forward(self, input, *args, **kwargs):
     sq_err = torch.zeros(len(helper.alphas), dtype=torch.float64, device=ref.device)
     if helper.exponent_columns is None or helper.exponent_columns[0].device != ref.device:
         helper.exponent_columns = _exponent_columns(helper.alphas, ref.device)
-    scales = get_scales(helper.act_scale, helper.weight_scale, helper.alphas, helper.exponent_columns)
-    w_scales = scales.to(dtype)
-    x_scales = (1 / scales).to(dtype)
+    # the candidate scales depend on the cached statistics only: built at the first search step,
+    # reused by the later ones, and the best row is folded when the search is over
+    grid = helper.scale_grid
+    if grid is None or grid[1].dtype != dtype or grid[0].device != ref.device:
+        scales = get_scales(helper.act_scale, helper.weight_scale, helper.alphas, helper.exponent_columns)
+        grid = helper.scale_grid = (scales, scales.to(dtype), (1 / scales).to(dtype))
+    _, w_scales, x_scales = grid
     if fused:
         q = self.weight_quantizer
         x_in = input.contiguous()
@@ -649,16 +660,26 @@ def _awq_forward(self, input, *args, **kwargs):
     return out_actual
 
 
-def _finalize_losses(helper):
-    """loss[alpha] = sum over search steps of that step's mean squared error.  The kernel leaves
-    per-step sums of squares on the device; fetching them is the one host synchronisation of the
-    search, and the division and the sum over steps happen on the host in double."""
+def _losses_on_device(helper):
+    """float64 ``[n_alphas]`` on the device: loss[alpha] = sum over search steps of that step's mean
+    squared error (the kernels leave per-step sums of squares there); None without search steps."""
     if not helper.sq_err_steps:
-        return {a: 0.0 for a in helper.alphas}
-    sums = torch.stack([s for s, _ in helper.sq_err_steps]).cpu()
-    sizes = torch.tensor([n for _, n in helper.sq_err_steps], dtype=torch.float64)
-    total = (sums / sizes[:, None]).sum(0).tolist()
-    return dict(zip(helper.alphas, total))
+        return None
+    # the element counts go in as scalars: a host tensor would have to be copied to the device,
+    # which waits for everything queued on the stream
+    total = None
+    for sums, n in helper.sq_err_steps:
+        mean = sums / float(n)
+        total = mean if total is None else total + mean
+    return total
+
+
+def _first_minimum(loss):
+    """Index (0-dim int64 on the device) that ``min(dict, key=dict.get)`` would pick: the first
+    smallest value; a NaN is never smaller than anything, and a NaN in front is never replaced."""
+    key = torch.where(torch.isnan(loss), torch.full_like(loss, float("inf")), loss)
+    idx = torch.argmin(key)
+    return torch.where(torch.isnan(loss[0]), torch.zeros_like(idx), idx)
 
 
 @torch.no_grad()
@@ -681,24 +702,44 @@ def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: boo
         forward_loop(model)
     max_calibrate(model, lambda model: None)
 
+    cached = []
     for name, module in model.named_modules():
         if is_quantized_linear(module) and hasattr(module, "awq_lite") and module.awq_lite.num_cache_steps > 0:
             module._if_calib = True
             h = module.awq_lite
             h.act_scale = h.act_scale / h.num_cache_steps
-            if bool(torch.any(torch.isnan(h.act_scale)) or torch.any(torch.isnan(h.weight_scale))):
+            cached.append(h)
+    if cached:  # one host synchronisation for the NaN checks of all layers
+        flags = torch.stack([torch.isnan(h.act_scale).any() | torch.isnan(h.weight_scale).any()
+                             for h in cached]).tolist()
+        for h, bad in zip(cached, flags):
+            if bad:
                 h.is_enabled = False
 
     _AWQLiteHelper.cache_mode = False
     print("awq_lite: Searching parameters...")
     forward_loop(model)
 
+    # The best alpha is picked on the device and the checks are collected, so that folding the
+    # scales of one layer does not wait for the search kernels of the layers behind it: one host
+    # synchronisation at the end instead of three per layer.
+    positive_later, searched = [], []
+
     def postprocess(module, name):
         h = module.awq_lite
         if h.is_enabled:
-            h.loss = _finalize_losses(h)
-            h.best_alpha = min(h.loss, key=h.loss.get)
-            h.best_scale = get_scale(h.act_scale, h.weight_scale, h.best_alpha)
+            loss = _losses_on_device(h)
+            if loss is None:
+                h.loss = {a: 0.0 for a in h.alphas}
+                h.best_alpha = min(h.loss, key=h.loss.get)
+                h.best_scale = get_scale(h.act_scale, h.weight_scale, h.best_alpha)
+            else:
+                best = _first_minimum(loss)
+                grid = h.scale_grid[0] if h.scale_grid is not None else get_scales(
+                    h.act_scale, h.weight_scale, h.alphas, h.exponent_columns)
+                h.best_scale = grid.index_select(0, best.reshape(1))[0]  # the row the search scored
+                h.scale_grid = None
+                searched.append((h, loss, best))
         for q in (module.weight_quantizer, module.input_quantizer):
             if hasattr(q, "_pre_quant_scale"):
                 delattr(q, "_pre_quant_scale")
@@ -710,23 +751,36 @@ def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: boo
             module.input_quantizer.amax = act_amax.amax()
             module.input_quantizer.enable()
         if h.is_enabled:
-            apply_pre_quant_scale_and_smooth(module, 1.0 / h.best_scale)
+            apply_pre_quant_scale_and_smooth(module, 1.0 / h.best_scale, _positive_later=positive_later)
         else:
             warnings.warn(f"awq_lite: Disabling for {name}, quantizing with max calibration.")
             max_calibrate(module, lambda module: module.weight_quantizer(module.weight))
 
-    for name, module in model.named_modules():
-        if hasattr(module, "awq_lite"):
-            h = module.awq_lite
-            if h.num_cache_steps == 0:
-                h.is_enabled = False
-            elif h.num_search_steps == 0:
-                h.is_enabled = False
-                warnings.warn(
-                    "awq_lite: Calling `forward_loop(model)` the second time did not forward data "
-                    f"through the {name}. Please provide a valid `forward_loop` function that can "
-                    "be used to forward data through the model many times.")
-            postprocess(module, name)
-            h.cleanup()
-            if not debug:
-                delattr(module, "awq_lite")
+    kept = []
+    with deferred_scale_checks():
+        for name, module in model.named_modules():
+            if hasattr(module, "awq_lite"):
+                h = module.awq_lite
+                if h.num_cache_steps == 0:
+                    h.is_enabled = False
+                elif h.num_search_steps == 0:
+                    h.is_enabled = False
+                    warnings.warn(
+                        "awq_lite: Calling `forward_loop(model)` the second time did not forward data "
+                        f"through the {name}. Please provide a valid `forward_loop` function that can "
+                        "be used to forward data through the model many times.")
+                postprocess(module, name)
+                h.cleanup()
+                if debug:
+                    kept.append(h)
+                else:
+                    delattr(module, "awq_lite")
+    if positive_later:
+        assert bool(torch.stack([(p > 0).all() for p in positive_later]).all()), \
+            "pre_quant_scale should be positive"
+    if kept and searched:  # the helpers stay on the modules: give them the numbers as Python values
+        losses = torch.stack([loss for _, loss, _ in searched]).tolist()
+        picks = torch.stack([best for _, _, best in searched]).tolist()
+        for (h, _, _), row, pick in zip(searched, losses, picks):
+            h.loss = dict(zip(h.alphas, row))
+            h.best_alpha = h.alphas[pick]

@@ -126,9 +126,31 @@ def update_quant_cfg_with_kv_cache_quant(quant_cfg: dict, kv_cache_quant_cfg: di
     return quant_cfg
 
 
+_DEFERRED_CHECKS = []   # innermost ``deferred_scale_checks`` block last
+
+
+@contextlib.contextmanager
+def deferred_scale_checks():
+    """Within the block ``all_valid_scales`` only records its tensors and reports True; the one
+    real check -- one host synchronisation -- happens when the block ends and raises
+    ``AssertionError`` if any recorded value is negative, infinite or NaN by then.  For loops
+    over many layers whose per-layer checks would each wait for the device."""
+    pending = []
+    _DEFERRED_CHECKS.append(pending)
+    try:
+        yield pending
+    finally:
+        _DEFERRED_CHECKS.pop()
+    if pending and not all_valid_scales(pending):
+        raise AssertionError("detected negative, inf or nan values in a calibrated amax or scale")
+
+
 def all_valid_scales(tensors) -> bool:
     """True when every element of every tensor is finite and non-negative -- one device
     reduction and one host synchronisation for the whole list."""
+    if _DEFERRED_CHECKS:
+        _DEFERRED_CHECKS[-1].extend(t for t in tensors if isinstance(t, torch.Tensor))
+        return True
     groups = {}   # one concatenation per (device, dtype): no per-tensor conversion
     for t in tensors:
         if isinstance(t, torch.Tensor) and not t.is_meta and t.numel():
