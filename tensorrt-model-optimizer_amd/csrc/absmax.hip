@@ -384,12 +384,14 @@ static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
     if (axis == 1) {  // per tensor
         const int64_t n = outer * inner;
         if (base_ok) {
-            // 16384-element tiles, and the occupancy cap only from 256 MB: 7.4 - 7.5 TB/s on a 67 MB
-            // batch of activations (7.0 with 32768-element tiles and the cap), 7.2 - 7.4 on 0.5 - 2 GB
-            const int64_t tile = mo::tuned("absmax_flat_tile", 16384);
+            // 32768-element tiles under the occupancy cap.  Smaller tiles without the cap read a
+            // 67 MB tensor 6 % faster into a warm accumulator, but with a fresh one (dynamic
+            // quantisation, the first batch of a calibration) twice as many workgroups meet at the
+            // accumulator's atomic and the launch and its successor lose 10 us.
+            const int64_t tile = mo::tuned("absmax_flat_tile", 32768);
             const int64_t tiles = (n + tile - 1) / tile;
             if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
-            const size_t cap = mo::ballast_bytes("absmax_flat_kernel", n >= (1ll << 27) ? 36 : 0);
+            const size_t cap = mo::ballast_bytes("absmax_flat_kernel", 36);
             if (tile == 8192) absmax_flat_kernel<DT, 8192><<<dim3((unsigned)tiles), 256, cap, s>>>(x, n, acc);
             else if (tile == 16384) absmax_flat_kernel<DT, 16384><<<dim3((unsigned)tiles), 256, cap, s>>>(x, n, acc);
             else absmax_flat_kernel<DT, 32768><<<dim3((unsigned)tiles), 256, cap, s>>>(x, n, acc);
