@@ -775,12 +775,12 @@ def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: boo
                     kept.append(h)
                 else:
                     delattr(module, "awq_lite")
-    if positive_later:
-        assert bool(torch.stack([(p > 0).all() for p in positive_later]).all()), \
-            "pre_quant_scale should be positive"
-    if kept and searched:  # the helpers stay on the modules: give them the numbers as Python values
-        losses = torch.stack([loss for _, loss, _ in searched]).tolist()
-        picks = torch.stack([best for _, _, best in searched]).tolist()
-        for (h, _, _), row, pick in zip(searched, losses, picks):
-            h.loss = dict(zip(h.alphas, row))
-            h.best_alpha = h.alphas[pick]
+    by_device = {}
+    for p in positive_later:
+        by_device.setdefault(p.device, []).append((p > 0).all())
+    assert all(bool(torch.stack(flags).all()) for flags in by_device.values()), \
+        "pre_quant_scale should be positive"
+    if kept:  # the helpers stay on the modules: give them the numbers as Python values
+        for h, loss, best in searched:
+            h.loss = dict(zip(h.alphas, loss.tolist()))
+            h.best_alpha = h.alphas[int(best)]

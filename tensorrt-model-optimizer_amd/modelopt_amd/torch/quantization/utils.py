@@ -133,8 +133,9 @@ _DEFERRED_CHECKS = []   # innermost ``deferred_scale_checks`` block last
 def deferred_scale_checks():
     """Within the block ``all_valid_scales`` only records its tensors and reports True; the one
     real check -- one host synchronisation -- happens when the block ends and raises
-    ``AssertionError`` if any recorded value is negative, infinite or NaN by then.  For loops
-    over many layers whose per-layer checks would each wait for the device."""
+    ``AssertionError`` if any recorded value is negative, infinite or NaN by then (a nested block
+    hands its tensors to the enclosing one).  For loops over many layers whose per-layer checks
+    would each wait for the device."""
     pending = []
     _DEFERRED_CHECKS.append(pending)
     try:

@@ -556,3 +556,30 @@ def test_plan_inputs_notice_a_reallocated_tensor():
     a.data = torch.ones(8)
     with pytest.raises(RuntimeError, match="reallocated"):
         pinned.verify()
+
+
+def test_first_minimum_picks_what_min_over_the_loss_dict_picks():
+    """AWQ-lite chooses ``min(loss, key=loss.get)`` in the reference: the first smallest value,
+    where a NaN never replaces the running best and a NaN in front is never replaced."""
+    from modelopt_amd.torch.quantization.model_calib import _first_minimum
+    nan = float("nan")
+    cases = [[3.0, 1.0, 2.0], [1.0, 1.0, 0.5, 0.5], [nan, 1.0, 0.5], [2.0, nan, 1.0], [2.0, nan, 3.0],
+             [nan, nan], [0.0], [5.0, 4.0, nan, 4.0], [float("inf"), float("inf")]]
+    for values in cases:
+        keys = list(range(len(values)))
+        want = min(keys, key=dict(zip(keys, values)).get)
+        got = int(_first_minimum(torch.tensor(values, dtype=torch.float64)))
+        assert got == want, (values, got, want)
+
+
+def test_deferred_scale_checks_make_one_check_at_the_end():
+    from modelopt_amd.torch.quantization.utils import all_valid_scales, deferred_scale_checks
+    with deferred_scale_checks() as pending:
+        assert all_valid_scales([torch.ones(2), None])
+        with deferred_scale_checks():                      # a nested block hands over to the outer one
+            assert all_valid_scales([torch.ones(1)])
+        assert len(pending) == 2
+    with pytest.raises(AssertionError, match="negative, inf or nan"):
+        with deferred_scale_checks():
+            assert all_valid_scales([torch.tensor([1.0, float("nan")])])   # recorded, reported later
+    assert not all_valid_scales([torch.tensor([-1.0])])                  # outside a block: checked at once
