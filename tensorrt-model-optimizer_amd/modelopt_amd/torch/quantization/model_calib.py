@@ -240,27 +240,36 @@ def smoothquant(model: nn.Module, forward_loop=None, alpha=1.0):
         module.input_quantizer.axis = None
         module.input_quantizer.amax = act_amax.amax().to(dtype=dtype, device=device)
         eps = 1.0 / (1 << 31)
-        if scale_a.min() <= eps:  # channels that never fired would make scale_a overflow
-            scale_a[act_amax.reshape(-1) <= eps] = 1
+        # channels that never fired would make scale_a overflow: when the smallest scale is tiny
+        # they are set to 1 -- selected on the device, the host does not wait for the answer
+        dead = (scale_a.min() <= eps) & (act_amax.reshape(-1) <= eps)
+        scale_a = torch.where(dead, torch.ones_like(scale_a), scale_a)
         scale_a = scale_a.clamp(min=1e-4, max=1e4)
-        apply_pre_quant_scale_and_smooth(module, scale_a)
+        apply_pre_quant_scale_and_smooth(module, scale_a, _positive_later=positive_later)
 
     smoothed = 0
-    for name, module in model.named_modules():
-        if not is_quantized_linear(module):
-            continue
-        if not hasattr(module.input_quantizer, "_amax"):
-            warnings.warn(f"{name} is not calibrated, skip smoothing")
-            continue
-        if module.input_quantizer.num_bits != 8 or module.weight_quantizer.num_bits != 8:
-            warnings.warn(f"Only int8 smoothing is supported, skip {name}")
-            continue
-        if module.input_quantizer.axis != -1:
-            warnings.warn(f"Only per-channel smoothing is supported, skip {name}")
-            continue
-        assert module.input_quantizer._amax.numel() > 1, f"Error: {name} has only one channel to smooth"
-        postprocess(module)
-        smoothed += 1
+    positive_later = []   # checked once for all layers below
+    with deferred_scale_checks():   # one synchronisation for the checks of all layers
+        for name, module in model.named_modules():
+            if not is_quantized_linear(module):
+                continue
+            if not hasattr(module.input_quantizer, "_amax"):
+                warnings.warn(f"{name} is not calibrated, skip smoothing")
+                continue
+            if module.input_quantizer.num_bits != 8 or module.weight_quantizer.num_bits != 8:
+                warnings.warn(f"Only int8 smoothing is supported, skip {name}")
+                continue
+            if module.input_quantizer.axis != -1:
+                warnings.warn(f"Only per-channel smoothing is supported, skip {name}")
+                continue
+            assert module.input_quantizer._amax.numel() > 1, f"Error: {name} has only one channel to smooth"
+            postprocess(module)
+            smoothed += 1
+    by_device = {}
+    for p in positive_later:
+        by_device.setdefault(p.device, []).append((p > 0).all())
+    assert all(bool(torch.stack(flags).all()) for flags in by_device.values()), \
+        "pre_quant_scale should be positive"
     print(f"Smoothed {smoothed} modules")
 
 
