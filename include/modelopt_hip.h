@@ -366,6 +366,15 @@ int mo_abs_colsum_staged(const void* x, int64_t rows, int64_t k, int dtype, cons
                          int64_t block_size, float* acc, float* partial, int64_t partial_rows,
                          void* stream);
 
+/* acc[c] += sum over rows of T(|x[r, c]| / T(amax(r, c / block_size) + tiny)), amax being the
+ * abs-max of the row's block of `block_size` columns taken in the same pass: the whole numerator
+ * of get_weight_scale (TQ/model_calib.py:588-603) in one read of the weight, no block-amax
+ * array.  Two passes without atomics like mo_abs_colsum_staged (`partial`: partial_rows x k
+ * floats, 16-byte aligned); same bits as mo_abs_colsum_staged fed the block abs-max.  Returns
+ * MO_ERR_UNSUPPORTED unless block_size is 8, 16, ... 512, divides k, and x is 16-byte aligned. */
+int mo_weight_scale_colsum(const void* x, int64_t rows, int64_t k, int dtype, int64_t block_size,
+                           float* acc, float* partial, int64_t partial_rows, void* stream);
+
 /* xs[a][c][t][0..8) = bf16(x[t][8 c ..] * inv_s[a][8 c ..]) for n_alpha rows of inv_s: the
  * activations under every candidate scale, in the chunk-major layout mo_awq_search_losses reads
  * ([n_alpha][k / 8][tokens][8] bf16).  This is the `inputs * pre_quant_scale` of the input

@@ -195,10 +195,14 @@ __global__ __launch_bounds__(256) void abs_colsum8_kernel(const void* __restrict
                     const float a = __builtin_fabsf(v[j]);
                     float q = exact_quotient(a, d, r);   // NaN stays NaN
                     // the correction steps are exact only while nothing underflows
-                    if (q < 1.0e-30f && a > 0.0f) q = a / d;
+                    if (q < 1.0e-30f && a > 0.0f) {
+                        keep_branch();
+                        q = a / d;
+                    }
                     sum[j] += round_to<DT>(q);
                 }
             } else {
+                keep_branch();
 #pragma unroll
                 for (int j = 0; j < 8; ++j) sum[j] += round_to<DT>(__builtin_fabsf(v[j]) / d);
             }
@@ -224,6 +228,112 @@ __global__ __launch_bounds__(256) void abs_colsum8_kernel(const void* __restrict
         RawChunk<DT> raw;
         load_raw<DT>(x, r * k + col, raw);
         add_row(raw, WITH_AMAX ? blk_amax[r * nb + cb] : 0.0f);
+    }
+    f32x4* out = (f32x4*)(partial + (int64_t)blockIdx.y * k + col);
+    const f32x4 a = {sum[0], sum[1], sum[2], sum[3]}, b = {sum[4], sum[5], sum[6], sum[7]};
+    out[0] = a;
+    out[1] = b;
+}
+
+// abs_colsum8_kernel<DT, true> with the block abs-max taken from x itself: the G = bs / 8 lanes
+// that own a block of a row exchange the maxima of their chunks (bit patterns, so a NaN wins
+// as in torch's amax).  One pass over the weight instead of two and no amax array.
+//
+// bf16: |x| and d = T(amax + tiny) have 8-bit significands, so the exact quotient differs from
+// every rounding boundary of bf16 by at least 1 / (255 * 512) of its value unless it lies on
+// one, which it cannot (the boundary's odd 9-bit numerator would have to divide the 8-bit
+// numerator of |x|).  A quotient good to 2^-22 -- |x| times the hardware reciprocal -- therefore
+// rounds to the same bf16 value as the correctly rounded fp32 quotient does; only quotients in
+// fp32's denormal range, where that error bound does not hold, take the division.
+#ifndef MO_WS_U
+#define MO_WS_U 8
+#endif
+template <int DT>
+__global__ __launch_bounds__(256) void weight_scale_colsum8_kernel(const void* __restrict__ x,
+                                                                   int64_t rows, int64_t k, int lg_g,
+                                                                   int64_t slab,
+                                                                   float* __restrict__ partial) {
+    const int64_t col = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (col >= k) return;   // k is a multiple of the block: its lanes leave together
+    const int64_t r0 = (int64_t)blockIdx.y * slab;
+    int64_t r1 = r0 + slab;
+    if (r1 > rows) r1 = rows;
+    const float tiny = DT == MO_F16 ? 6.103515625e-05f : 1.17549435e-38f;
+    float sum[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    auto add_row = [&](const RawChunk<DT>& raw) {
+        float v[8];
+        unpack_raw<DT>(raw, v);
+        float amax;
+        if constexpr (DT == MO_F32) {
+            uint32_t m = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t b = f2u(v[j]) & 0x7FFFFFFFu;
+                m = b > m ? b : m;
+            }
+            amax = u2f(group_max_u32(m, lg_g));
+        } else {
+            const uint32_t mask = 0x7FFF7FFFu;
+            const uint32_t p = pk_max_u16(pk_max_u16(raw.a.x & mask, raw.a.y & mask),
+                                          pk_max_u16(raw.a.z & mask, raw.a.w & mask));
+            uint32_t m = p & 0xFFFFu;
+            m = (p >> 16) > m ? (p >> 16) : m;
+            m = group_max_u32(m, lg_g);
+            amax = DT == MO_BF16 ? u2f(m << 16) : f16_bits_to_f32(m);
+        }
+        const float d = round_to<DT>(amax + tiny);
+        if (mid_range(d)) {     // |x| <= amax <= d: the quotient cannot overflow
+            if constexpr (DT == MO_BF16) {
+                const float r = __builtin_amdgcn_rcpf(d);
+                float q[8];
+                bool denormal = false;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    q[j] = __builtin_fabsf(v[j]) * r;                  // NaN stays NaN
+                    denormal |= __builtin_amdgcn_classf(q[j], 0x80);   // positive denormal
+                }
+                if (denormal) {     // one branch per chunk; rare
+                    keep_branch();
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (__builtin_amdgcn_classf(q[j], 0x80)) q[j] = __builtin_fabsf(v[j]) / d;
+                }
+                // the pair (0, q) converted leaves bf16(q) as an fp32 bit pattern
+#pragma unroll
+                for (int j = 0; j < 8; ++j) sum[j] += u2f(f32x2_to_bf16x2(0.0f, q[j]));
+            } else {
+                const float r = 1.0f / d;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float a = __builtin_fabsf(v[j]);
+                    float q = exact_quotient(a, d, r);
+                    // the correction steps are exact only while nothing underflows
+                    if (q < 1.0e-30f && a > 0.0f) {
+                        keep_branch();
+                        q = a / d;
+                    }
+                    sum[j] += round_to<DT>(q);
+                }
+            }
+        } else {
+            keep_branch();
+#pragma unroll
+            for (int j = 0; j < 8; ++j) sum[j] += round_to<DT>(__builtin_fabsf(v[j]) / d);
+        }
+    };
+    int64_t r = r0;
+    constexpr int U = DT == MO_F32 ? MO_WS_U / 2 : MO_WS_U;   // rows (16- or 32-byte loads) in flight per lane
+    for (; r + U - 1 < r1; r += U) {
+        RawChunk<DT> raw[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) load_raw<DT>(x, (r + u) * k + col, raw[u]);
+#pragma unroll
+        for (int u = 0; u < U; ++u) add_row(raw[u]);
+    }
+    for (; r < r1; ++r) {
+        RawChunk<DT> raw;
+        load_raw<DT>(x, r * k + col, raw);
+        add_row(raw);
     }
     f32x4* out = (f32x4*)(partial + (int64_t)blockIdx.y * k + col);
     const f32x4 a = {sum[0], sum[1], sum[2], sum[3]}, b = {sum[4], sum[5], sum[6], sum[7]};
@@ -457,6 +567,34 @@ extern "C" int mo_abs_colsum_staged(const void* x, int64_t rows, int64_t k, int 
     else                                                                                          \
         mo::abs_colsum8_kernel<DT, false><<<grid, 256, mo::ballast_bytes("abs_colsum8_kernel", 0), st>>>(x, rows, k, blk_amax, block_size, \
                                                                 slab, partial)
+    DISPATCH_DT(dtype, CALL)
+#undef CALL
+    mo::colsum_fold_partials_kernel<<<(unsigned)((k + 63) / 64), 256, 0, st>>>(partial, slabs, k, acc);
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+// Column sums of |x| / T(block abs-max + tiny) with the block abs-max computed in the same pass
+// (two launches: slab sums, then the fold of the partial rows in a fixed order).
+extern "C" int mo_weight_scale_colsum(const void* x, int64_t rows, int64_t k, int dtype,
+                                      int64_t block_size, float* acc, float* partial,
+                                      int64_t partial_rows, void* stream) {
+    if (rows < 0 || k < 0 || partial_rows < 1 || block_size <= 0) return MO_ERR_ARG;
+    if (dtype < MO_F32 || dtype > MO_BF16) return MO_ERR_DTYPE;
+    int lg_g = 0;
+    while (lg_g < 6 && (8ll << lg_g) < block_size) ++lg_g;
+    if ((8ll << lg_g) != block_size || k % block_size) return MO_ERR_UNSUPPORTED;
+    if (rows == 0 || k == 0) return MO_OK;
+    if (!x || !acc || !partial) return MO_ERR_ARG;
+    if ((((uintptr_t)x | (uintptr_t)partial | (uintptr_t)acc) & 15u) != 0) return MO_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    int64_t slabs = partial_rows < 65535 ? partial_rows : 65535;
+    const int64_t slab = (rows + slabs - 1) / slabs;
+    slabs = (rows + slab - 1) / slab;
+    const dim3 grid((unsigned)((k / 8 + 255) / 256), (unsigned)slabs);
+#define CALL(DT)                                                                              \
+    mo::weight_scale_colsum8_kernel<DT>                                                       \
+        <<<grid, 256, mo::ballast_bytes("weight_scale_colsum8_kernel", 0), st>>>(x, rows, k, lg_g, \
+                                                                                 slab, partial)
     DISPATCH_DT(dtype, CALL)
 #undef CALL
     mo::colsum_fold_partials_kernel<<<(unsigned)((k + 63) / 64), 256, 0, st>>>(partial, slabs, k, acc);

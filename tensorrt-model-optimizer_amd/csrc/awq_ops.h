@@ -27,8 +27,15 @@ __device__ __forceinline__ void block_int_qdq_chunk(float (&v)[8], int lg_g, flo
     for (int j = 0; j < 8; ++j) {
         float q = __builtin_rintf(v[j] * mul);
         q = q < lo ? lo : q;
-        q = q > bound ? bound : q;
-        v[j] = fast ? __builtin_copysignf(exact_quotient(q, div, rdiv), q) : q / div;
+        v[j] = q > bound ? bound : q;
+    }
+    if (fast) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = __builtin_copysignf(exact_quotient(v[j], div, rdiv), v[j]);
+    } else {
+        keep_branch();
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = v[j] / div;
     }
 }
 

@@ -12,14 +12,22 @@
 // lane, so they are read through uniform (scalar) loads and cost the vector ALU nothing.  The
 // org[] values of a lane live in LDS ([token][lane], conflict-free).  VALU-bound: each product
 // is one multiply, one rounding to T (and, for 16-bit T, an unpack) and one add.
+//
+// A weight with few (row, block) pairs does not fill the chip with one wavefront per 64 pairs
+// (1024 x 4096 in blocks of 128 is 512 wavefronts for 1024 SIMDs, and a lone wavefront on a
+// SIMD runs at two thirds of the rate three of them reach together), so a workgroup may hold
+// 2 or 4 wavefronts that own the same 64 pairs and share the tokens of a pass between them;
+// their partial sums meet in LDS and wavefront 0 adds them in wavefront order, so the result
+// does not depend on timing.
 #include "common.h"
 #include "qdq_ops.h"
 
 namespace mo {
 
 constexpr int kClipMaxRatios = 32;
-constexpr int kClipTokens = 64;   // tokens per pass over the ratios (org[] held in LDS)
+constexpr int kClipTokens = 64;   // tokens per wavefront and pass over the ratios (org[] in LDS)
 constexpr int kClipLanes = 64;
+constexpr int kClipMaxSplit = 4;  // wavefronts that may share the tokens of one (row, block) set
 
 struct ClipRatios {
     float r[kClipMaxRatios];
@@ -114,14 +122,22 @@ __device__ __forceinline__ float org_unpack(typename OrgStore<DT>::type v) {
 }
 
 template <int DT, int BS>
-__global__ __launch_bounds__(kClipLanes) void awq_clip_loss_kernel(
+__global__ __launch_bounds__(kClipLanes * kClipMaxSplit) void awq_clip_loss_kernel(
     const void* __restrict__ x, int tokens, const void* __restrict__ w, int n, int k,
     const void* __restrict__ w_amax, int amax_dtype, ClipRatios ratios, IntOp op,
     float* __restrict__ loss) {
     constexpr int NC = BS / 8;
     constexpr int GC = NC < 4 ? NC : 4;   // chunks loaded together
-    __shared__ typename OrgStore<DT>::type org[kClipTokens][kClipLanes];
-    const int lane = threadIdx.x;
+    typedef typename OrgStore<DT>::type org_t;
+    // dynamic LDS: org[pass_tokens][64] in the tensor dtype, then part[2][split][64] fp32
+    extern __shared__ __align__(16) unsigned char clip_smem[];
+    const int split = blockDim.x / kClipLanes;
+    const int pass_tokens = split * kClipTokens;
+    org_t (*org)[kClipLanes] = (org_t (*)[kClipLanes])clip_smem;
+    float (*part)[kClipLanes] =
+        (float (*)[kClipLanes])(clip_smem + (size_t)pass_tokens * kClipLanes * sizeof(org_t));
+    const int lane = threadIdx.x % kClipLanes;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kClipLanes);
     const int nblk = k / BS;
     const int b = blockIdx.y;
     int row = blockIdx.x * kClipLanes + lane;
@@ -153,11 +169,16 @@ __global__ __launch_bounds__(kClipLanes) void awq_clip_loss_kernel(
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    for (int t0 = 0; t0 < tokens; t0 += kClipTokens) {
-        const int tc = tokens - t0 < kClipTokens ? tokens - t0 : kClipTokens;
+    int flip = 0;   // part[] is double-buffered: one barrier per ratio is enough
+    for (int t0 = 0; t0 < tokens; t0 += pass_tokens) {
+        const int tc = tokens - t0 < pass_tokens ? tokens - t0 : pass_tokens;
+        // this wavefront's share of the pass: tokens [lo, lo + mine)
+        const int lo = (int)((int64_t)tc * wave / split);
+        const int mine = (int)((int64_t)tc * (wave + 1) / split) - lo;
+        const int64_t x0 = (int64_t)(t0 + lo) * k + xb;
         refill([](float v) { return v; });
-        token_dots<DT, BS>(x, (int64_t)t0 * k + xb, k, tc, wv,
-                           [&](int t, float v) { org[t][lane] = org_pack<DT>(v); });
+        token_dots<DT, BS>(x, x0, k, mine, wv,
+                           [&](int t, float v) { org[lo + t][lane] = org_pack<DT>(v); });
         for (int r = 0; r < ratios.count; ++r) {
             // `w_amax * ratio` on a tensor: fp32 product rounded to the dtype of the amax
             float clipped = amax * ratios.r[r];
@@ -174,11 +195,20 @@ __global__ __launch_bounds__(kClipLanes) void awq_clip_loss_kernel(
                 refill([&](float v) { return clip_round<DT>(op.apply<false>(v, s)); });
             }
             float sum = 0.0f;
-            token_dots<DT, BS>(x, (int64_t)t0 * k + xb, k, tc, wv, [&](int t, float cur) {
-                const float d = clip_round<DT>(cur - org_unpack<DT>(org[t][lane]));
+            token_dots<DT, BS>(x, x0, k, mine, wv, [&](int t, float cur) {
+                const float d = clip_round<DT>(cur - org_unpack<DT>(org[lo + t][lane]));
                 sum += d * d;
             });
-            if (active) {
+            if (split > 1) {
+                part[flip * split + wave][lane] = sum;
+                __syncthreads();
+                if (wave == 0) {
+                    sum = part[flip * split][lane];
+                    for (int v = 1; v < split; ++v) sum += part[flip * split + v][lane];
+                }
+                flip ^= 1;
+            }
+            if (active && wave == 0) {
                 float* out = loss + ((int64_t)r * n + row) * nblk + b;
                 *out += sum / (float)tokens;
             }
@@ -214,9 +244,23 @@ extern "C" int mo_awq_clip_losses(const void* x, int64_t tokens, const void* w, 
     op.lo = is_unsigned ? 0.0f : (narrow_range ? -op.bound : -op.bound - 1.0f);
     const dim3 grid((unsigned)((n + mo::kClipLanes - 1) / mo::kClipLanes),
                     (unsigned)(k / block_size));
+    // Wavefronts per 64 (row, block) pairs.  Measured on 4096-wide rows, 64 tokens, bf16: up to
+    // about 2048 such sets (two wavefronts per SIMD) a workgroup of four -- one wavefront on
+    // each SIMD of a compute unit -- is faster (1024 rows: 848 -> 406 us, 2048 rows: 870 ->
+    // 729 us, 3072 rows: 1349 -> 1043 us); from 2048 sets on the single wavefront is (4096 rows:
+    // 1359 us either way, 14336 rows: 4017 against 4642 us).  Eight are slower than four
+    // everywhere.  Each wavefront should still get 8 tokens or more.
+    const int64_t sets = (int64_t)grid.x * grid.y;
+    int split = sets < mo::tuned("clip_split_below_sets", 2048) ? mo::kClipMaxSplit : 1;
+    while (split > 1 && tokens < 8 * split) split /= 2;
+    const size_t elem = dtype == MO_F32 ? 4 : 2;
+    if (dtype == MO_F32 && split > 2) split = 2;   // org[] of a pass stays within 64 KB of LDS
+    split = (int)mo::tuned("clip_split", split);
+    const size_t smem = (size_t)split * mo::kClipTokens * mo::kClipLanes * elem +
+                        (split > 1 ? (size_t)2 * split * mo::kClipLanes * sizeof(float) : 0);
     hipStream_t s = (hipStream_t)stream;
 #define CALL(DT, BS)                                                                       \
-    mo::awq_clip_loss_kernel<DT, BS><<<grid, mo::kClipLanes, 0, s>>>(                      \
+    mo::awq_clip_loss_kernel<DT, BS><<<grid, mo::kClipLanes * split, smem, s>>>(           \
         x, (int)tokens, w, (int)n, (int)k, w_amax, amax_dtype, rr, op, loss)
 #define BY_BS(DT)                                                         \
     switch (block_size) {                                                 \

@@ -324,6 +324,11 @@ __device__ __forceinline__ float exact_quotient(float x, float s, float r) {
     return __builtin_fmaf(__builtin_fmaf(-s, q1, x), r, q1);
 }
 
+// Placed at the top of a rarely taken block: an empty statement the optimiser may not move or
+// run speculatively, so the block stays behind a branch (without it a cheap-looking block -- one
+// fp32 division is ten instructions -- is evaluated on every pass and its result selected).
+__device__ __forceinline__ void keep_branch() { asm volatile(""); }
+
 // true when 2^-64 <= s <= 2^64 (normal, and far from the ends of the exponent range)
 __device__ __forceinline__ bool mid_range(float s) {
     const uint32_t b = f2u(s);

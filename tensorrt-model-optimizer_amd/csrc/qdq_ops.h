@@ -60,6 +60,7 @@ struct IntOp {
         q = q < lo ? lo : q;
         q = q > bound ? bound : q;
         if (s.fast) return __builtin_copysignf(exact_quotient(q, s.div, s.rdiv), q);
+        keep_branch();
         return q / s.div;
     }
     template <bool F>

@@ -57,6 +57,7 @@ SIGNATURES = {
     "mo_awq_clip_losses": [_P, _I64, _P, _I64, _I64, _INT, _I64, _P, _INT, _P, _INT, _INT, _INT, _INT, _P, _P],
     "mo_abs_colsum": [_P, _I64, _I64, _INT, _P, _I64, _P, _P],
     "mo_abs_colsum_staged": [_P, _I64, _I64, _INT, _P, _I64, _P, _P, _I64, _P],
+    "mo_weight_scale_colsum": [_P, _I64, _I64, _INT, _I64, _P, _P, _I64, _P],
     "mo_sq_diff_sum": [_P, _P, _I64, _INT, _P, _P],
 }
 
@@ -632,6 +633,29 @@ def abs_colsum_into(x, acc, blk_amax=None, block_size=0):
     call("mo_abs_colsum", x, _ptr(x), rows, k, dtype_code(x.dtype),
          _ptr(blk_amax), block_size, _ptr(acc), _stream(x))
     return acc
+
+
+def weight_scale_colsum_into(x, acc, block_size):
+    """``acc[c] +=`` the column sums of ``T(|x| / T(block abs-max + tiny))`` with the abs-max of
+    every ``block_size`` adjacent columns of a row taken in the same pass over ``x``.  Returns
+    False (nothing written) for block sizes the kernel does not take: anything but 8, 16, ...
+    512 dividing the row length."""
+    _require_device(x, acc)
+    k = x.shape[-1]
+    assert x.is_contiguous() and acc.dtype == torch.float32 and acc.numel() == k
+    rows = x.numel() // k if k else 0
+    bs = int(block_size)
+    if (bs < 8 or bs > 512 or bs & (bs - 1) or k % bs or x.data_ptr() % 16 or acc.data_ptr() % 16):
+        return False
+    # about four workgroups per compute unit in all (the quotients give each wavefront work to
+    # overlap with the loads of the others: 14336 x 4096 takes 27 us with 1024 workgroups, 29 with
+    # 512, 34 with 2048), at least 16 rows per slab
+    across = -(-k // 2048)
+    slabs = max(1, min(-(-1024 // across), rows // 16))
+    partial = _staging_words(x, slabs * k)
+    call("mo_weight_scale_colsum", x, _ptr(x), rows, k, dtype_code(x.dtype), bs, _ptr(acc),
+         _ptr(partial), slabs, _stream(x))
+    return True
 
 
 def sq_diff_sum_into(a, b, acc):

@@ -451,6 +451,11 @@ def get_weight_scale(weight, block_size=None):
     n, k = weight.shape
     w = weight.data.contiguous()
     dev = w.device
+    if block_size and k % block_size == 0:
+        # block abs-max, quotient and column sum in one pass over the weight
+        acc = torch.zeros(k, dtype=torch.float32, device=dev)
+        if _hip.weight_scale_colsum_into(w, acc, block_size):
+            return (acc / n).to(weight.dtype).to(torch.float32)
     if block_size:
         nb = -(-k // block_size)
         if k % block_size:

@@ -62,15 +62,37 @@ def test_losses_match_restatement(dtype, block):
     assert float((best_got == best_want).float().mean()) > 0.97
 
 
-@pytest.mark.parametrize("tokens", [1, 64, 65, 150])
+@pytest.mark.parametrize("tokens", [1, 7, 20, 64, 65, 150, 300])
 def test_token_chunks_and_ragged_rows(tokens):
-    """more tokens than one pass holds, a row count that is not a multiple of the lanes"""
+    """more tokens than one pass holds, a row count that is not a multiple of the lanes; a small
+    weight like this one is given 1, 2 or 4 wavefronts per row set depending on the token count"""
     w, x = _case(70, 128, tokens, torch.bfloat16, tokens)
     ratios, got = _run_kernel(w, x, 64)
     want, _ = oawq.awq_clip_search(w, [x], 64, 4, max_tokens_per_batch=1 << 20)
     for i, r in enumerate(ratios):
         rel = (got[i] - want[r]).abs().sum() / want[r].abs().sum()
         assert float(rel) < 2e-4, (r, float(rel))
+
+
+def test_fp32_passes_shared_by_two_wavefronts():
+    """fp32 keeps its partial outputs in LDS as fp32: two wavefronts per row set, two passes"""
+    w, x = _case(70, 128, 200, torch.float32, 11)
+    ratios, got = _run_kernel(w, x, 32)
+    want, _ = oawq.awq_clip_search(w, [x], 32, 4, max_tokens_per_batch=1 << 20)
+    for i, r in enumerate(ratios):
+        rel = (got[i] - want[r]).abs().sum() / want[r].abs().sum()
+        assert float(rel) < 2e-4, (r, float(rel))
+
+
+def test_large_launch_equals_its_row_slices():
+    """A weight with 2048 row sets or more runs one wavefront per set, a slice of its rows
+    several that share the tokens: same products, sums of the token errors in another order."""
+    w, x = _case(2048, 1024, 150, torch.bfloat16, 12)
+    ratios, whole = _run_kernel(w, x, 16)
+    for r0 in (0, 1024, 1984):
+        rows = slice(r0, r0 + 64)
+        _, part = _run_kernel(w[rows].contiguous(), x, 16)
+        torch.testing.assert_close(part, whole[:, rows], rtol=2e-6, atol=0)
 
 
 def test_accumulates_over_batches_and_special_blocks():

@@ -390,6 +390,95 @@ def test_column_sums_two_pass_kernel(dtype, rows, k, block):
     assert torch.allclose(got2[ok], want2[ok], rtol=3e-6, atol=0)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("rows,k,block", [(1100, 4096, 128), (4100, 1024, 512), (300, 4096, 16),
+                                          (64, 256, 8), (1, 512, 32), (2000, 2560, 256), (257, 192, 64)])
+def test_weight_scale_sums_in_one_pass(dtype, rows, k, block):
+    """Block abs-max, quotient and column sum in one kernel: the same bits as the two-pass
+    column sum fed the block abs-max from its own kernel (same slabs, same order), and the
+    float64 sum of the tensor expression's terms; all-zero blocks, quotients in fp32's denormal
+    range, NaN and inf included."""
+    g = torch.Generator().manual_seed(rows + k + block)
+    x = (torch.randn(rows, k, generator=g) * torch.exp(torch.randn(rows, 1, generator=g))).to(dtype)
+    if rows > 8:
+        x[5, :block] = 0                      # an all-zero block: |x| / tiny
+        x[7, :block] *= 1e-3
+        if dtype != torch.float16:            # tiny elements beside a large one: denormal quotients
+            x[2, :block] = torch.tensor(3e-38, dtype=dtype)
+            x[2, 1] = 2.0 ** 60
+            x[6, :block] = torch.tensor(1e-20, dtype=dtype)
+            x[6, 3] = 2.0 ** 63
+    xd = x.to(DEV)
+    acc = torch.full((k,), 2.5, dtype=torch.float32, device=DEV)
+    assert _hip.weight_scale_colsum_into(xd, acc, block)
+    tiny = torch.finfo(dtype).tiny
+    blocks = x.view(rows, k // block, block)
+    terms = (blocks.abs() / (blocks.abs().amax(-1, keepdim=True) + tiny)).view(rows, k)
+    assert terms.dtype == dtype
+    want = terms.double().sum(0) + 2.5
+    got = acc.cpu().double()
+    assert torch.allclose(got, want, rtol=3e-6, atol=0), float(((got - want).abs() / want).max())
+    if rows == 1:                             # one term per column: exact
+        assert torch.equal(acc.cpu(), terms[0].float() + 2.5)
+    if rows >= 64:      # over the same row slabs: the bits of the column sum fed the block abs-max
+        blk = torch.zeros(rows * (k // block), dtype=torch.float32, device=DEV)
+        _hip.absmax_into(xd, blk, 1, rows * (k // block), block)
+        slabs = 7
+        work = torch.empty(slabs * k, dtype=torch.float32, device=DEV)
+        two, one = (torch.full((k,), 2.5, dtype=torch.float32, device=DEV) for _ in range(2))
+        _hip.call("mo_abs_colsum_staged", xd, xd.data_ptr(), rows, k, _hip.dtype_code(dtype),
+                  blk.data_ptr(), block, two.data_ptr(), work.data_ptr(), slabs, None)
+        torch.cuda.synchronize()
+        _hip.call("mo_weight_scale_colsum", xd, xd.data_ptr(), rows, k, _hip.dtype_code(dtype),
+                  block, one.data_ptr(), work.data_ptr(), slabs, None)
+        assert torch.equal(two, one)
+        assert torch.allclose(one, acc, rtol=2e-6, atol=0)
+    x2 = x.clone()
+    x2[0, 9] = float("nan")
+    x2[rows // 2, k - 3] = float("inf")
+    acc2 = torch.zeros(k, dtype=torch.float32, device=DEV)
+    assert _hip.weight_scale_colsum_into(x2.to(DEV), acc2, block)
+    b2 = x2.view(rows, k // block, block)
+    want2 = (b2.abs() / (b2.abs().amax(-1, keepdim=True) + tiny)).view(rows, k).double().sum(0)
+    got2 = acc2.cpu().double()
+    assert torch.equal(torch.isnan(got2), torch.isnan(want2))
+    ok = torch.isfinite(want2)
+    assert torch.allclose(got2[ok], want2[ok], rtol=3e-6, atol=0)
+
+
+def test_weight_scale_bf16_quotients_term_by_term():
+    """One row, so every column sum is a single term: every pair of bf16 significands at
+    several exponent distances (subnormal numerators too), each quotient rounded exactly as
+    the tensor expression rounds it."""
+    sig = torch.arange(128, 256, dtype=torch.float32)
+    rows = []
+    for shift in (0, 1, 5, 40, 120):
+        for d in sig:
+            # a block of 256: the first 128 hold d (the abs-max), the rest every numerator
+            num = sig * 2.0 ** -shift
+            num = torch.where(num <= d, num, num / 2)
+            rows.append(torch.cat([d.expand(128), num]))
+    x = torch.stack(rows).reshape(1, -1).to(torch.bfloat16)
+    sub = torch.arange(1, 129, dtype=torch.float32) * 2.0 ** -133        # bf16 subnormals
+    x = torch.cat([x, torch.cat([torch.full((128,), 2.0 ** -120), sub]).to(torch.bfloat16).reshape(1, -1),
+                   torch.cat([torch.full((128,), 2.0 ** -126), sub]).to(torch.bfloat16).reshape(1, -1)], 1)
+    k = x.shape[1]
+    acc = torch.zeros(k, dtype=torch.float32, device=DEV)
+    assert _hip.weight_scale_colsum_into(x.to(DEV), acc, 256)
+    blocks = x.view(1, k // 256, 256)
+    want = (blocks.abs() / (blocks.abs().amax(-1, keepdim=True) + torch.finfo(torch.bfloat16).tiny))
+    assert torch.equal(acc.cpu(), want.view(-1).float())
+
+
+def test_weight_scale_one_pass_refuses_other_blocks():
+    x = torch.ones(64, 192, dtype=torch.bfloat16, device=DEV)
+    acc = torch.zeros(192, dtype=torch.float32, device=DEV)
+    assert not _hip.weight_scale_colsum_into(x, acc, 128)      # does not divide 192
+    assert not _hip.weight_scale_colsum_into(x, acc, 24)       # not a power of two
+    assert not _hip.weight_scale_colsum_into(x, acc, 4)
+    assert float(acc.abs().sum()) == 0.0
+
+
 def test_sq_diff_loss():
     a, b = _rand((256, 512), torch.bfloat16, 10, 1.0), _rand((256, 512), torch.bfloat16, 11, 1.0)
     acc = torch.zeros(1, dtype=torch.float64, device=DEV)
