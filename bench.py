@@ -386,7 +386,7 @@ def secondary_kernels(torch, steps, warmup):
     rec("scale_block_int_qdq_14336x4096", lambda: _hip.scale_block_int_qdq(w, s, 128, out=y), n * 4)
     rec("mul_cols_14336x4096", lambda: _hip.mul_cols(w, s, out=y), n * 4)
     col = torch.zeros(k, dtype=torch.float32, device=dev)
-    rec("abs_colsum_with_block_amax_14336x4096", lambda: _hip.abs_colsum_into(w, col, blk, 128), n * 2)
+    rec("weight_scale_colsum_14336x4096", lambda: _hip.weight_scale_colsum_into(w, col, 128), n * 2)
     rec("fp8_qdq_14336x4096", lambda: _hip.fp8_qdq(w, amax, 1, 1, n, out=y), n * 4)
     rec("int8_qdq_14336x4096", lambda: _hip.int_qdq(w, amax, 1, 1, n, 8, False, False, out=y), n * 4)
     rec("nvfp4_qdq_14336x4096", lambda: _hip.nvfp4_qdq(w, amax, out=y), n * 4)

@@ -134,6 +134,53 @@ __global__ __launch_bounds__(256) void scale_block_int_qdq_kernel(
     }
 }
 
+// The same for the aligned case (k a multiple of the block, 16-byte aligned operands), where
+// chunk t of the tensor is elements [8 t, 8 t + 8): all loads of a lane -- its kQdqRounds chunks
+// and their scales -- are issued first, in straight-line code (a lane past the end re-reads the
+// last chunk and does not store), so nothing waits behind a store.  SD is the dtype of the
+// scale vector, -1 without one.
+template <int DT, int SD>
+__global__ __launch_bounds__(256) void scale_block_int_qdq_vec_kernel(
+    const void* __restrict__ x, int64_t total, int64_t kc, const void* __restrict__ s, int lg_g,
+    float bound, float lo, void* __restrict__ y) {
+    constexpr int SDT = SD < 0 ? MO_BF16 : SD;
+    const int64_t t0 = (int64_t)blockIdx.x * kQdqTileChunks + threadIdx.x;
+    const int64_t last = total - 1;
+    RawChunk<DT> raw[kQdqRounds];
+    RawChunk<SDT> sraw[kQdqRounds];
+    // column chunk of the first item by one division, of the others by stepping
+    int64_t cc = 0;
+    if constexpr (SD >= 0) {
+        const int64_t tt = t0 < last ? t0 : last;
+        cc = total <= 0xFFFFFFFFll ? (int64_t)((uint32_t)tt % (uint32_t)kc) : tt % kc;
+    }
+    const int64_t step = 256 % kc;
+#pragma unroll
+    for (int u = 0; u < kQdqRounds; ++u) {
+        const int64_t t = t0 + u * 256;
+        load_raw<DT>(x, (t < last ? t : last) << 3, raw[u]);
+        if constexpr (SD >= 0) {
+            load_raw<SDT>(s, cc << 3, sraw[u]);
+            cc += step;
+            cc = cc >= kc ? cc - kc : cc;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kQdqRounds; ++u) {
+        const int64_t t = t0 + u * 256;
+        float v[8];
+        unpack_raw<DT>(raw[u], v);
+        if constexpr (SD >= 0) {
+            float sc[8];
+            unpack_raw<SDT>(sraw[u], sc);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = round_to<DT>(v[j] * sc[j]);
+        }
+        block_int_qdq_chunk(v, lg_g, bound, lo);
+        if (t <= last) store_chunk<DT>(y, t << 3, v);
+    }
+}
+
 // acc[c] += sum over rows of f32( T( |x[r, c]| / T(f32(blk_amax[r, c / bs]) + tiny) ) ) when
 // blk_amax is given, else of |x[r, c]|.  One thread per column over a slab of rows.
 template <int DT>
@@ -498,9 +545,23 @@ extern "C" int mo_scale_block_int_qdq(const void* x, int64_t rows, int64_t k, in
     const bool vec = (k % block_size == 0) &&
                      ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)s) & 15u) == 0);
     const unsigned g = (unsigned)blocks;
+    const size_t cap = mo::ballast_bytes("scale_block_int_qdq_kernel", 0);
+    if (vec) {
+        const int64_t kc = k >> 3;
+#define CALL_SD(DT, SD)                                                                          \
+    mo::scale_block_int_qdq_vec_kernel<DT, SD><<<g, 256, cap, st>>>(x, total, kc, s, lg, bound, lo, y)
+#define CALL(DT)                                                                                 \
+    if (!s) CALL_SD(DT, -1);                                                                     \
+    else if (s_dtype == MO_F32) CALL_SD(DT, MO_F32);                                             \
+    else if (s_dtype == MO_F16) CALL_SD(DT, MO_F16);                                             \
+    else CALL_SD(DT, MO_BF16)
+        DISPATCH_DT(dtype, CALL)
+#undef CALL
+#undef CALL_SD
+        return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+    }
 #define CALL(DT)                                                                                      \
-    if (vec) mo::scale_block_int_qdq_kernel<DT, true><<<g, 256, mo::ballast_bytes("scale_block_int_qdq_kernel", 0), st>>>(x, rows, k, s, s_dtype, lg, bound, lo, y); \
-    else mo::scale_block_int_qdq_kernel<DT, false><<<g, 256, mo::ballast_bytes("scale_block_int_qdq_kernel", 0), st>>>(x, rows, k, s, s_dtype, lg, bound, lo, y)
+    mo::scale_block_int_qdq_kernel<DT, false><<<g, 256, cap, st>>>(x, rows, k, s, s_dtype, lg, bound, lo, y)
     DISPATCH_DT(dtype, CALL)
 #undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;

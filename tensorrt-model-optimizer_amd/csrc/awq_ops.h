@@ -23,19 +23,33 @@ __device__ __forceinline__ void block_int_qdq_chunk(float (&v)[8], int lg_g, flo
     const float mul = dead ? 0.0f : sc, div = dead ? 1.0f : sc;
     const float rdiv = 1.0f / div;
     const bool fast = mid_range(div);
+    if (fast && lo < 0.0f) {
+        // mid-range scale: the block holds no NaN or inf (either would be its abs-max), so the
+        // clamp is a plain median (signed grids only: with lo = +0 the median of (-0, +0, bound)
+        // need not keep the -0 that the comparison keeps) and the quotient the exact
+        // reciprocal-and-FMA one
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        float q = __builtin_rintf(v[j] * mul);
-        q = q < lo ? lo : q;
-        v[j] = q > bound ? bound : q;
-    }
-    if (fast) {
+        for (int j = 0; j < 8; ++j) {
+            const float q = __builtin_amdgcn_fmed3f(__builtin_rintf(v[j] * mul), lo, bound);
+            v[j] = __builtin_copysignf(exact_quotient(q, div, rdiv), q);
+        }
+    } else if (fast) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = __builtin_copysignf(exact_quotient(v[j], div, rdiv), v[j]);
+        for (int j = 0; j < 8; ++j) {
+            float q = __builtin_rintf(v[j] * mul);
+            q = q < lo ? lo : q;
+            q = q > bound ? bound : q;
+            v[j] = __builtin_copysignf(exact_quotient(q, div, rdiv), q);
+        }
     } else {
         keep_branch();
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = v[j] / div;
+        for (int j = 0; j < 8; ++j) {
+            float q = __builtin_rintf(v[j] * mul);
+            q = q < lo ? lo : q;            // the way torch.clamp does: NaN stays NaN
+            q = q > bound ? bound : q;
+            v[j] = q / div;
+        }
     }
 }
 

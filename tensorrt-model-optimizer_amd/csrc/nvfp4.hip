@@ -442,22 +442,22 @@ __global__ __launch_bounds__(256) void nvfp4_dequantize_fast_kernel(
     const float wsf2 = wsf2p[0];
     const int64_t c0 = (int64_t)blockIdx.x * (256 * R) + threadIdx.x;
     uint32_t c[R], sb[R];
+    // every load in straight-line code (a lane past the end re-reads the last chunk), only the
+    // stores conditional: with the loads inside per-round branches the compiler waits at every
+    // join for all memory operations in flight, the previous round's store among them
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int64_t ch = c0 + r * 256;
-        if (ch < nchunks) {
-            c[r] = __builtin_nontemporal_load(packed + ch);
-            sb[r] = wsf[ch >> 1];
-        }
+        int64_t ch = c0 + r * 256;
+        ch = ch < nchunks ? ch : nchunks - 1;
+        c[r] = __builtin_nontemporal_load(packed + ch);
+        sb[r] = wsf[ch >> 1];
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int64_t ch = c0 + r * 256;
-        if (ch < nchunks) {
-            float v[8];
-            decode8(c[r], e4m3_to_f32(sb[r]) * wsf2, v);
-            store_chunk<MO_BF16>(y, ch * 8, v);
-        }
+        float v[8];
+        decode8(c[r], e4m3_to_f32(sb[r]) * wsf2, v);
+        if (ch < nchunks) store_chunk<MO_BF16>(y, ch * 8, v);
     }
 }
 

@@ -31,39 +31,48 @@ __global__ __launch_bounds__(256) void qdq_kernel(const void* __restrict__ x, vo
     const int64_t c0 = (int64_t)blockIdx.x * kTileChunks + threadIdx.x;
     typename Op::Scale s0 = {};
     if (KIND == TENSOR && amax) s0 = op.make(load_scalar(amax, amax_dtype, 0));
-    RawChunk<DT> raw[kQdqU];
+    if (chunks > 0) {
+        // All loads of the lane (the per-chunk amax too) come first, in straight-line code: a
+        // chunk past the end re-reads the last one and is not stored.  Loads inside per-chunk
+        // branches, or after a store, would make every round wait for the store before it.
+        const int64_t inner_chunks = KIND == CHUNK ? inner >> 3 : 1;
+        RawChunk<DT> raw[kQdqU];
+        float am[kQdqU];
 #pragma unroll
-    for (int u = 0; u < kQdqU; ++u) {
-        const int64_t c = c0 + u * 256;
-        zero_raw<DT>(raw[u]);
-        if (c < chunks) load_raw<DT>(x, c << 3, raw[u]);
-    }
-    const int64_t inner_chunks = KIND == CHUNK ? inner >> 3 : 1;
-    float v[kQdqU][8];
-#pragma unroll
-    for (int u = 0; u < kQdqU; ++u) {
-        const int64_t c = c0 + u * 256;
-        if (c >= chunks) continue;
-        unpack_raw<DT>(raw[u], v[u]);
-        if constexpr (KIND == TENSOR) {
-#pragma unroll
-            for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[u][j], v[u][j + 1], s0, s0);
-        } else if constexpr (KIND == CHUNK) {
-            int64_t row;
-            if (chunks <= 0xFFFFFFFFll) row = (uint32_t)c / (uint32_t)inner_chunks;
-            else row = c / inner_chunks;
-            const int64_t a = row < axis ? row : row % axis;
-            const typename Op::Scale s = op.make(load_scalar(amax, amax_dtype, a));
-#pragma unroll
-            for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[u][j], v[u][j + 1], s, s);
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int64_t a = (((c << 3) + j) / inner) % axis;
-                v[u][j] = op.template apply<FLAG>(v[u][j], op.make(load_scalar(amax, amax_dtype, a)));
+        for (int u = 0; u < kQdqU; ++u) {
+            int64_t c = c0 + u * 256;
+            c = c < chunks ? c : chunks - 1;
+            load_raw<DT>(x, c << 3, raw[u]);
+            am[u] = 0.0f;
+            if constexpr (KIND == CHUNK) {
+                int64_t row;
+                if (chunks <= 0xFFFFFFFFll) row = (uint32_t)c / (uint32_t)inner_chunks;
+                else row = c / inner_chunks;
+                am[u] = load_scalar(amax, amax_dtype, row < axis ? row : row % axis);
             }
         }
-        store_chunk<DT>(y, c << 3, v[u]);
+        float v[kQdqU][8];
+#pragma unroll
+        for (int u = 0; u < kQdqU; ++u) {
+            const int64_t c = c0 + u * 256;
+            unpack_raw<DT>(raw[u], v[u]);
+            if constexpr (KIND == TENSOR) {
+#pragma unroll
+                for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[u][j], v[u][j + 1], s0, s0);
+            } else if constexpr (KIND == CHUNK) {
+                const typename Op::Scale s = op.make(am[u]);
+#pragma unroll
+                for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[u][j], v[u][j + 1], s, s);
+            } else {
+                if (c >= chunks) continue;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int64_t a = (((c << 3) + j) / inner) % axis;
+                    v[u][j] = op.template apply<FLAG>(v[u][j], op.make(load_scalar(amax, amax_dtype, a)));
+                }
+            }
+            if (c < chunks) store_chunk<DT>(y, c << 3, v[u]);
+        }
     }
     // tail (n % 8 elements): the first lanes of the last workgroup
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x < (n & 7)) {

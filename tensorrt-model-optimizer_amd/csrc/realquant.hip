@@ -108,7 +108,10 @@ __device__ __forceinline__ void chunk_scale_indices(int64_t c0, int64_t chunks, 
 //   kScalePerChunk   anything else: each lane finds the rows of its chunks
 constexpr int kScalePerTensor = 0, kScalePerRowTile = 1, kScalePerChunk = 2;
 
-// chunk index, validity and scale of the lane's 4 chunks
+// chunk index, validity and scale of the lane's 4 chunks.  A chunk past the end gets the index
+// of the last valid one and ok = false: the kernels load it like any other (all loads in
+// straight-line code ahead of the first store, so that no round waits behind a store) and skip
+// only its store.
 template <int SCALES>
 __device__ __forceinline__ void tile_layout(int64_t chunks, int64_t axis, int64_t inner_chunks,
                                             int64_t tiles_per_row, const void* scale,
@@ -122,15 +125,15 @@ __device__ __forceinline__ void tile_layout(int64_t chunks, int64_t axis, int64_
         for (int u = 0; u < 4; ++u) {
             const int64_t local = tile * kRealTileChunks + threadIdx.x + u * 256;
             ok[u] = local < inner_chunks;
-            c[u] = row * inner_chunks + local;
+            c[u] = row * inner_chunks + (ok[u] ? local : inner_chunks - 1);
             sv[u] = s0;
         }
     } else {
         const int64_t c0 = (int64_t)blockIdx.x * kRealTileChunks + threadIdx.x;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            c[u] = c0 + u * 256;
-            ok[u] = c[u] < chunks;
+            ok[u] = c0 + u * 256 < chunks;
+            c[u] = ok[u] ? c0 + u * 256 : chunks - 1;
         }
         if constexpr (SCALES == kScalePerTensor) {
             sv[0] = sv[1] = sv[2] = sv[3] = load_scalar(scale, scale_dtype, 0);
@@ -138,7 +141,7 @@ __device__ __forceinline__ void tile_layout(int64_t chunks, int64_t axis, int64_
             int64_t idx[4];
             chunk_scale_indices<4>(c0, chunks, inner_chunks, axis, idx);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) sv[u] = ok[u] ? load_scalar(scale, scale_dtype, idx[u]) : 1.0f;
+            for (int u = 0; u < 4; ++u) sv[u] = load_scalar(scale, scale_dtype, idx[u]);
         }
     }
 }
@@ -154,16 +157,12 @@ __global__ __launch_bounds__(256) void real_quantize_tile_kernel(
     tile_layout<SCALES>(chunks, axis, inner_chunks, tiles_per_row, scale, scale_dtype, cs, ok, sv);
     RawChunk<DT> raw[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        zero_raw<DT>(raw[u]);
-        if (ok[u]) load_raw<DT>(x, cs[u] << 3, raw[u]);
-    }
+    for (int u = 0; u < 4; ++u) load_raw<DT>(x, cs[u] << 3, raw[u]);
     float v[4][8];
     float rv = 1.0f;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int64_t c = cs[u];
-        if (!ok[u]) continue;
         unpack_raw<DT>(raw[u], v[u]);
         const float s = sv[u];
         // the reciprocal (an IEEE division) is taken again only when the scale changes
@@ -182,6 +181,7 @@ __global__ __launch_bounds__(256) void real_quantize_tile_kernel(
             for (int j = 0; j < 8; ++j)
                 q[j] = __builtin_copysignf(exact_quotient(v[u][j], s, r), v[u][j]);
         } else {
+            keep_branch();
 #pragma unroll
             for (int j = 0; j < 8; ++j) q[j] = v[u][j] / s;
         }
@@ -209,7 +209,7 @@ __global__ __launch_bounds__(256) void real_quantize_tile_kernel(
             }
         }
         const u32x2 o = {lo, hi};
-        __builtin_nontemporal_store(o, out + c);
+        if (ok[u]) __builtin_nontemporal_store(o, out + c);
     }
 }
 
@@ -223,12 +223,10 @@ __global__ __launch_bounds__(256) void real_dequantize_tile_kernel(
     tile_layout<SCALES>(chunks, axis, inner_chunks, tiles_per_row, scale, scale_dtype, cs, ok, sv);
     u32x2 w[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
-        if (ok[u]) w[u] = __builtin_nontemporal_load(q + cs[u]);
+    for (int u = 0; u < 4; ++u) w[u] = __builtin_nontemporal_load(q + cs[u]);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int64_t c = cs[u];
-        if (!ok[u]) continue;
         const float s = round_via<DT>(sv[u]);
         float v[8];
         // every E4M3 value and every int8 value is exact in bf16, fp16 and fp32
@@ -248,7 +246,7 @@ __global__ __launch_bounds__(256) void real_dequantize_tile_kernel(
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] *= s;
-        store_chunk<DT>(y, c << 3, v);
+        if (ok[u]) store_chunk<DT>(y, c << 3, v);
     }
 }
 
@@ -359,11 +357,24 @@ __global__ __launch_bounds__(256) void int4_block_quantize_tile_kernel(
     constexpr int U = kInt4QuantRounds;
     const int64_t c0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
     RawChunk<DT> raw[U];
+    float given[U];
+    // every load (the scales too, when the caller gives them) before the first store and in
+    // straight-line code -- a lane past the end re-reads the last chunk and stores nothing --
+    // so that no round waits behind the stores of the one before
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        const int64_t c = c0 + u * 256;
-        zero_raw<DT>(raw[u]);
-        if (c < chunks) load_raw<DT>(x, c << 3, raw[u]);
+        int64_t c = c0 + u * 256;
+        c = c < chunks ? c : chunks - 1;
+        load_raw<DT>(x, c << 3, raw[u]);
+        given[u] = 0.0f;
+    }
+    if (scales_given) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int64_t c = c0 + u * 256;
+            c = c < chunks ? c : chunks - 1;
+            given[u] = load_elem<DT>(scales, c >> shift);
+        }
     }
     float v[U][8];
 #pragma unroll
@@ -378,10 +389,10 @@ __global__ __launch_bounds__(256) void int4_block_quantize_tile_kernel(
         }
         // chunks is a multiple of lanes_per_block, so the lanes of a block are all in or all out
         m = group_max_u32(m, shift);
-        if (c >= chunks) continue;
         float scale = round_via<DT>(round_via<DT>(1.0f / u2f(m)) * 7.0f);
-        if (scales_given) scale = load_elem<DT>(scales, c >> shift);
-        else if ((threadIdx.x & (lanes_per_block - 1)) == 0) store_elem<DT>(scales, c >> shift, scale);
+        if (scales_given) scale = given[u];
+        else if (c < chunks && (threadIdx.x & (lanes_per_block - 1)) == 0)
+            store_elem<DT>(scales, c >> shift, scale);
         // byte = (hi + 8) << 4 | (lo + 8) = 16 * hi + lo + 0x88; the +8s of the four bytes are
         // added once to the assembled word (the borrows of negative bytes cancel exactly)
         int w = 0;
@@ -391,7 +402,7 @@ __global__ __launch_bounds__(256) void int4_block_quantize_tile_kernel(
             const int lo = int4_rne(round_via<DT>(v[u][j + 1] * scale));
             w += (hi * 16 + lo) << (4 * j);
         }
-        __builtin_nontemporal_store((uint32_t)w + 0x88888888u, packed + c);
+        if (c < chunks) __builtin_nontemporal_store((uint32_t)w + 0x88888888u, packed + c);
     }
 }
 
@@ -402,16 +413,22 @@ __global__ __launch_bounds__(256) void int4_block_dequantize_tile_kernel(
     constexpr int U = kInt4DequantRounds;
     const int64_t c0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
     uint32_t w[U];
+    float sc[U];
+    // Codes and scales of all rounds are loaded in straight-line code (a lane past the end
+    // re-reads the last chunk) and only the stores are conditional: loads inside per-round
+    // branches make the compiler wait for everything outstanding, the previous round's store
+    // included, at every join.
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        const int64_t c = c0 + u * 256;
-        if (c < chunks) w[u] = __builtin_nontemporal_load(packed + c);
+        int64_t c = c0 + u * 256;
+        c = c < chunks ? c : chunks - 1;
+        w[u] = __builtin_nontemporal_load(packed + c);
+        sc[u] = load_elem<DT>(scales, c >> shift);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int64_t c = c0 + u * 256;
-        if (c >= chunks) continue;
-        const float s = load_elem<DT>(scales, c >> shift);
+        const float s = sc[u];
         const float r = 1.0f / s;
         const bool fast = mid_range(s);
         float v[8];
@@ -425,10 +442,11 @@ __global__ __launch_bounds__(256) void int4_block_dequantize_tile_kernel(
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = exact_quotient(v[j], s, r);  // 0 / s = +0, s > 0
         } else {
+            keep_branch();
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = v[j] / s;
         }
-        store_chunk<DT>(y, c << 3, v);
+        if (c < chunks) store_chunk<DT>(y, c << 3, v);
     }
 }
 
@@ -455,18 +473,17 @@ __global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
         cc0 = t0 - j0 * kc;
     }
     const int64_t step_j = 256 / kc, step_c = 256 - step_j * kc;   // 256 = step_j * kc + step_c
+    // all loads in straight-line code (an item past the end re-reads the last one and stores
+    // nothing), so that no round waits behind the store of the one before
 #pragma unroll
     for (int u = 0; u < R; ++u) {
         const int64_t t = t0 + u * 256;
-        zero_raw<DT>(ra_[u]);
-        zero_raw<DT>(rb_[u]);
-        sa[u] = sb[u] = 1.0f;
         int64_t j = j0 + u * step_j, c = cc0 + u * step_c;
         // c < kc + u * step_c < (u + 1) * kc: at most u wraps
 #pragma unroll
         for (int i = 0; i < u; ++i)
             if (c >= kc) { c -= kc; ++j; }
-        if (t >= total) continue;
+        if (t >= total) { j = pairs - 1; c = kc - 1; }
         load_raw<DT>(w, ((2 * j) * kc + c) << 3, ra_[u]);
         load_raw<DT>(w, ((2 * j + 1) * kc + c) << 3, rb_[u]);
         const int64_t sc = (uint32_t)c / (uint32_t)chunks_per_scale;  // both below 2^32
@@ -477,7 +494,6 @@ __global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
 #pragma unroll
     for (int u = 0; u < R; ++u) {
         const int64_t t = t0 + u * 256;
-        if (t >= total) continue;
         unpack_raw<DT>(ra_[u], a[u]);
         unpack_raw<DT>(rb_[u], b[u]);
         uint32_t m = 0;
@@ -502,6 +518,7 @@ __global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
                 if (e < 4) lo |= byte << (8 * e); else hi |= byte << (8 * (e - 4));
             }
         } else {
+            keep_branch();
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float qa = a[u][e] / sa[u], qb = b[u][e] / sb[u];
@@ -513,7 +530,7 @@ __global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
             }
         }
         const u32x2 o = {lo, hi};
-        __builtin_nontemporal_store(o, out + t);
+        if (t < total) __builtin_nontemporal_store(o, out + t);
     }
 }
 
