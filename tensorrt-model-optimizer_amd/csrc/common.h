@@ -60,6 +60,14 @@ inline int64_t tuned(const char* name, int64_t value) {
     return value;
 }
 
+// A pointer known to address device (global) memory, as one of that address space: loads and
+// stores through it are global_* instructions.  Kernel arguments are recognised as such by the
+// compiler; pointers read from memory (a job table) are generic and would use flat_* ones.
+template <typename T>
+__device__ __forceinline__ __attribute__((address_space(1))) T* as_global(T* p) {
+    return (__attribute__((address_space(1))) T*)(uintptr_t)p;
+}
+
 __device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
 __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 

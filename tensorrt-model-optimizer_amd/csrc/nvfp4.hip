@@ -258,8 +258,8 @@ __device__ __forceinline__ void load_tile_bf16(const uint16_t* __restrict__ x, i
     for (int p = 0; p < kTileRoundPairs; ++p) {
         const int64_t ca = c0 + p * 512, cb = ca + 256;
         const u32x4 zero = {0, 0, 0, 0};
-        r.a[p] = ca < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + ca * 8)) : zero;
-        r.b[p] = cb < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + cb * 8)) : zero;
+        r.a[p] = ca < nchunks ? __builtin_nontemporal_load(as_global((const u32x4*)(x + ca * 8))) : zero;
+        r.b[p] = cb < nchunks ? __builtin_nontemporal_load(as_global((const u32x4*)(x + cb * 8))) : zero;
     }
 }
 
@@ -288,8 +288,8 @@ __device__ __forceinline__ void quantize_loaded_tile_bf16(const TileRaw& r, int6
         if (mine < nchunks) {
             const int64_t blk = mine >> 1;
             u32x2 o = {lo, hi};
-            __builtin_nontemporal_store(o, packed + blk);
-            wsf[blk] = (uint8_t)byte;
+            __builtin_nontemporal_store(o, as_global(packed + blk));
+            *as_global(wsf + blk) = (uint8_t)byte;
         }
     }
 }
@@ -334,7 +334,10 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_multi_kernel(
         }
     }
     const mo_nvfp4_job jb = jobs[lo];
-    const float a = jb.amax[0];
+    // The amax is fetched, and the global scale stored, before the tile's loads go out.  Issuing
+    // the loads first (they do not depend on the amax) measured 2 % slower at every occupancy
+    // cap: the chip is short of memory bandwidth, not of requests in flight.
+    const float a = *as_global(jb.amax);
     const float wsf2 = amax_is_wsf2 ? a : a / 2688.0f;
     if (jb.wsf2_out && t == jb.tile_begin && threadIdx.x == 0) jb.wsf2_out[0] = wsf2;
     quantize_tile_bf16((const uint16_t*)jb.x, jb.elems >> 4, t - jb.tile_begin, wsf2, 6.0f * wsf2,
