@@ -47,10 +47,20 @@ __global__ __launch_bounds__(256) void sq_err_tensor_kernel(const void* __restri
             for (int k = 0; k < KN; ++k) {
                 if (k < K) {  // uniform
                     float acc = 0.0f;
+                    // one decision per candidate between the branch-free arithmetic and the
+                    // general one, not one per element
+                    if (Op::is_fast(s[k])) {
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const float d = v[j] - op.template apply<SAT>(v[j], s[k]);
-                        acc += d * d;
+                        for (int j = 0; j < 8; ++j) {
+                            const float d = v[j] - op.template apply_fast<SAT>(v[j], s[k]);
+                            acc += d * d;
+                        }
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const float d = v[j] - op.template apply<SAT>(v[j], s[k]);
+                            acc += d * d;
+                        }
                     }
                     part[k] += acc;
                 }
@@ -116,10 +126,18 @@ __global__ __launch_bounds__(256) void sq_err_rows_kernel(const void* __restrict
                 for (int k = 0; k < KN; ++k) {
                     if (k < K) {
                         float acc = 0.0f;
+                        if (Op::is_fast(s[k])) {
 #pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            const float d = v[j] - op.template apply<SAT>(v[j], s[k]);
-                            acc += d * d;
+                            for (int j = 0; j < 8; ++j) {
+                                const float d = v[j] - op.template apply_fast<SAT>(v[j], s[k]);
+                                acc += d * d;
+                            }
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) {
+                                const float d = v[j] - op.template apply<SAT>(v[j], s[k]);
+                                acc += d * d;
+                            }
                         }
                         part[k] += acc;
                     }

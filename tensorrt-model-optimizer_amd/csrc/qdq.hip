@@ -56,13 +56,18 @@ __global__ __launch_bounds__(256) void qdq_kernel(const void* __restrict__ x, vo
         for (int u = 0; u < kQdqU; ++u) {
             const int64_t c = c0 + u * 256;
             unpack_raw<DT>(raw[u], v[u]);
-            if constexpr (KIND == TENSOR) {
+            if constexpr (KIND == TENSOR || KIND == CHUNK) {
+                // one decision per chunk between the branch-free arithmetic and the general one
+                // (a branch per element would end the basic block after every element)
+                typename Op::Scale s = s0;
+                if constexpr (KIND == CHUNK) s = op.make(am[u]);
+                if (Op::is_fast(s)) {
 #pragma unroll
-                for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[u][j], v[u][j + 1], s0, s0);
-            } else if constexpr (KIND == CHUNK) {
-                const typename Op::Scale s = op.make(am[u]);
+                    for (int j = 0; j < 8; j += 2) op.template apply2_fast<FLAG>(v[u][j], v[u][j + 1], s, s);
+                } else {
 #pragma unroll
-                for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[u][j], v[u][j + 1], s, s);
+                    for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[u][j], v[u][j + 1], s, s);
+                }
             } else {
                 if (c >= chunks) continue;
 #pragma unroll
@@ -94,8 +99,12 @@ __global__ __launch_bounds__(256) void qdq_cols_kernel(const void* __restrict__ 
     const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) << 3;
     if (col >= axis) return;
     typename Op::Scale s[8];
+    bool fast = true;   // whether all 8 columns of the lane take the branch-free arithmetic
 #pragma unroll
-    for (int j = 0; j < 8; ++j) s[j] = op.make(load_scalar(amax, amax_dtype, col + j));
+    for (int j = 0; j < 8; ++j) {
+        s[j] = op.make(load_scalar(amax, amax_dtype, col + j));
+        fast = fast && Op::is_fast(s[j]);
+    }
     const int64_t r0 = (int64_t)blockIdx.y * slab;
     int64_t r1 = r0 + slab;
     if (r1 > rows) r1 = rows;
@@ -106,13 +115,22 @@ __global__ __launch_bounds__(256) void qdq_cols_kernel(const void* __restrict__ 
         for (int u = 0; u < 4; ++u) load_raw<DT>(x, (r + u) * axis + col, raw[u]);
         float v[4][8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            unpack_raw<DT>(raw[u], v[u]);
+        for (int u = 0; u < 4; ++u) unpack_raw<DT>(raw[u], v[u]);
+        if (fast) {
 #pragma unroll
-            for (int j = 0; j < 8; j += 2)
-                op.template apply2<FLAG>(v[u][j], v[u][j + 1], s[j], s[j + 1]);
-            store_chunk<DT>(y, (r + u) * axis + col, v[u]);
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int j = 0; j < 8; j += 2)
+                    op.template apply2_fast<FLAG>(v[u][j], v[u][j + 1], s[j], s[j + 1]);
+        } else {
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int j = 0; j < 8; j += 2)
+                    op.template apply2<FLAG>(v[u][j], v[u][j + 1], s[j], s[j + 1]);
         }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) store_chunk<DT>(y, (r + u) * axis + col, v[u]);
     }
     for (; r < r1; ++r) {
         float v[8];
@@ -242,8 +260,13 @@ __global__ __launch_bounds__(256) void fused_amax_qdq_kernel(
         if (c >= chunks) continue;
         float v[8];
         unpack_raw<DT>(raw[u], v);
+        if (Op::is_fast(s0)) {
 #pragma unroll
-        for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[j], v[j + 1], s0, s0);
+            for (int j = 0; j < 8; j += 2) op.template apply2_fast<FLAG>(v[j], v[j + 1], s0, s0);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[j], v[j + 1], s0, s0);
+        }
         store_chunk<DT>(y, c << 3, v);
     }
     if (has_tail) store_elem<DT>(y, (chunks << 3) + threadIdx.x, op.template apply<FLAG>(tail, s0));

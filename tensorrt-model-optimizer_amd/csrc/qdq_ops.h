@@ -22,6 +22,14 @@ struct Fp8Op {
         if (!has_amax) return round_e4m3<SAT>(x);
         return round_e4m3<SAT>(x * s.mul) * s.inv;
     }
+    // every scale takes the same path
+    static __device__ __forceinline__ bool is_fast(const Scale&) { return true; }
+    template <bool SAT>
+    __device__ __forceinline__ float apply_fast(float x, const Scale& s) const { return apply<SAT>(x, s); }
+    template <bool SAT>
+    __device__ __forceinline__ void apply2_fast(float& a, float& b, const Scale& sa, const Scale& sb) const {
+        apply2<SAT>(a, b, sa, sb);
+    }
     // two elements per conversion instruction
     template <bool SAT>
     __device__ __forceinline__ void apply2(float& a, float& b, const Scale& sa, const Scale& sb) const {
@@ -67,6 +75,20 @@ struct IntOp {
     __device__ __forceinline__ void apply2(float& a, float& b, const Scale& sa, const Scale& sb) const {
         a = apply<F>(a, sa);
         b = apply<F>(b, sb);
+    }
+    // for a caller that has checked is_fast() of every scale it holds once, outside its loop
+    static __device__ __forceinline__ bool is_fast(const Scale& s) { return s.fast; }
+    template <bool>
+    __device__ __forceinline__ float apply_fast(float x, const Scale& s) const {
+        float q = __builtin_rintf(x * s.mul);
+        q = q < lo ? lo : q;
+        q = q > bound ? bound : q;
+        return __builtin_copysignf(exact_quotient(q, s.div, s.rdiv), q);
+    }
+    template <bool F>
+    __device__ __forceinline__ void apply2_fast(float& a, float& b, const Scale& sa, const Scale& sb) const {
+        a = apply_fast<F>(a, sa);
+        b = apply_fast<F>(b, sb);
     }
 };
 

@@ -163,6 +163,9 @@ __global__ __launch_bounds__(256) void real_quantize_tile_kernel(
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int64_t c = cs[u];
+        // a row of fewer than 1024 chunks leaves part of its workgroup without work: those
+        // lanes skip the arithmetic too (only the loads are unconditional)
+        if (!ok[u]) continue;
         unpack_raw<DT>(raw[u], v[u]);
         const float s = sv[u];
         // the reciprocal (an IEEE division) is taken again only when the scale changes
@@ -209,7 +212,7 @@ __global__ __launch_bounds__(256) void real_quantize_tile_kernel(
             }
         }
         const u32x2 o = {lo, hi};
-        if (ok[u]) __builtin_nontemporal_store(o, out + c);
+        __builtin_nontemporal_store(o, out + c);
     }
 }
 
@@ -227,6 +230,7 @@ __global__ __launch_bounds__(256) void real_dequantize_tile_kernel(
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int64_t c = cs[u];
+        if (!ok[u]) continue;
         const float s = round_via<DT>(sv[u]);
         float v[8];
         // every E4M3 value and every int8 value is exact in bf16, fp16 and fp32
@@ -246,7 +250,7 @@ __global__ __launch_bounds__(256) void real_dequantize_tile_kernel(
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] *= s;
-        if (ok[u]) store_chunk<DT>(y, c << 3, v);
+        store_chunk<DT>(y, c << 3, v);
     }
 }
 
