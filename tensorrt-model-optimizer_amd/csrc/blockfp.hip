@@ -124,20 +124,40 @@ __global__ __launch_bounds__(256) void block_fp_qdq_kernel(
     float v[4][8];
     int64_t base[4], col[4], row[4];
     RawChunk<DT> raw[4];
+    float gl[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if constexpr (FLAT) {
+        // all loads (the global amax of a chunk's row too) in straight-line code ahead of the
+        // first store; a chunk past the end re-reads the last one and is not stored
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int64_t c = c0 + u * 256;
-        base[u] = col[u] = row[u] = 0;
-        zero_raw<DT>(raw[u]);
+        for (int u = 0; u < 4; ++u) {
+            int64_t c = c0 + u * 256;
+            c = c < total_chunks ? c : total_chunks - 1;
+            col[u] = c << 3;
+            base[u] = row[u] = 0;
+            load_raw<DT>(x, col[u], raw[u]);
+        }
+        if (global_amax) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[u][j] = 0.0f;
-        if (c < total_chunks) {
-            if (total_chunks <= 0xFFFFFFFFll) row[u] = (uint32_t)c / (uint32_t)cpr;
-            else row[u] = c / cpr;
-            if constexpr (FLAT) {
-                col[u] = c << 3;
-                load_raw<DT>(x, col[u], raw[u]);
-            } else {
+            for (int u = 0; u < 4; ++u) {
+                int64_t r = 0;
+                if (per_row) {
+                    const int64_t c = col[u] >> 3;
+                    if (total_chunks <= 0xFFFFFFFFll) r = (uint32_t)c / (uint32_t)cpr;
+                    else r = c / cpr;
+                }
+                gl[u] = global_amax[r];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t c = c0 + u * 256;
+            base[u] = col[u] = row[u] = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[u][j] = 0.0f;
+            if (c < total_chunks) {
+                if (total_chunks <= 0xFFFFFFFFll) row[u] = (uint32_t)c / (uint32_t)cpr;
+                else row[u] = c / cpr;
                 col[u] = (c - row[u] * cpr) << 3;
                 base[u] = row[u] * k;
                 load_chunk_guarded<DT>(x, base[u], col[u], k, v[u]);
@@ -156,9 +176,13 @@ __global__ __launch_bounds__(256) void block_fp_qdq_kernel(
             m = t > m ? t : m;
         }
         m = group_max_u32(m, lg_g);  // total_chunks is a multiple of the group size
-        if (!live) continue;
-        float g = 0.0f;
-        if (global_amax) g = global_amax[per_row ? row[u] : 0];
+        if constexpr (!FLAT) {
+            if (!live) continue;
+        }
+        float g = gl[u];
+        if constexpr (!FLAT) {
+            if (global_amax) g = global_amax[per_row ? row[u] : 0];
+        }
         const BlockScale s = block_scale<FMT>(u2f(m), scale_fmt, global_amax != nullptr, g);
         float o[8];
 #pragma unroll
@@ -166,8 +190,11 @@ __global__ __launch_bounds__(256) void block_fp_qdq_kernel(
             const float q = convert_elem<FMT>(__builtin_fabsf(v[u][j]) * s.scale) * s.unscale;
             o[j] = v[u][j] < 0.0f ? -q : q;
         }
-        if constexpr (FLAT) store_chunk<DT>(y, col[u], o);
-        else store_chunk_guarded<DT>(y, base[u], col[u], k, o);
+        if constexpr (FLAT) {
+            if (live) store_chunk<DT>(y, col[u], o);
+        } else {
+            store_chunk_guarded<DT>(y, base[u], col[u], k, o);
+        }
     }
 }
 
