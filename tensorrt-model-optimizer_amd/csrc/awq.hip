@@ -293,7 +293,7 @@ __global__ __launch_bounds__(256) void abs_colsum8_kernel(const void* __restrict
 // rounds to the same bf16 value as the correctly rounded fp32 quotient does; only quotients in
 // fp32's denormal range, where that error bound does not hold, take the division.
 #ifndef MO_WS_U
-#define MO_WS_U 8
+#define MO_WS_U 4
 #endif
 template <int DT>
 __global__ __launch_bounds__(256) void weight_scale_colsum8_kernel(const void* __restrict__ x,

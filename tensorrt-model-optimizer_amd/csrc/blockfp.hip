@@ -377,19 +377,17 @@ __global__ __launch_bounds__(256) void mxfp4_dequantize_kernel(const uint32_t* _
                                                                void* __restrict__ y) {
     const int64_t c0 = (int64_t)blockIdx.x * kBlockFpTileChunks + threadIdx.x;
     uint32_t w[4], sb[4];
+    // loads in straight-line code (a chunk past the end re-reads the last one), stores conditional
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-        const int64_t c = c0 + u * 256;
-        w[u] = sb[u] = 0;
-        if (c < chunks) {
-            w[u] = __builtin_nontemporal_load(packed + c);
-            sb[u] = scales[c >> lg_g];
-        }
+        int64_t c = c0 + u * 256;
+        c = c < chunks ? c : chunks - 1;
+        w[u] = __builtin_nontemporal_load(packed + c);
+        sb[u] = scales[c >> lg_g];
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int64_t c = c0 + u * 256;
-        if (c >= chunks) continue;
         const float s = __builtin_ldexpf(1.0f, (int)sb[u] - 127);  // exp2(byte - 127) in fp32
         float v[8];
 #pragma unroll
@@ -398,7 +396,7 @@ __global__ __launch_bounds__(256) void mxfp4_dequantize_kernel(const uint32_t* _
             const float mag = e2m1_to_f32(code & 7u);
             v[j] = ((code & 8u) ? -mag : mag) * s;   // code 8 is -0
         }
-        store_chunk<DT>(y, c << 3, v);
+        if (c < chunks) store_chunk<DT>(y, c << 3, v);
     }
 }
 

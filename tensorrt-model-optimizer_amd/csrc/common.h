@@ -95,6 +95,10 @@ __device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {
 }
 
 // fp32 rounded to the nearest bf16 / fp16 value, as fp32
+// (Converting the pair (0, f) would leave bf16(f) as an fp32 bit pattern in one instruction instead
+// of two; kernels that are short of vector-ALU slots do that by hand.  As the general form it
+// made no streaming kernel faster and raised the register count of the clip search kernel from
+// 156 to 278, two wavefronts per SIMD fewer.)
 __device__ __forceinline__ float round_to_bf16(float f) { return u2f(f32_to_bf16_bits(f) << 16); }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
