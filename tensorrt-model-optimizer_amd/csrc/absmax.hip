@@ -116,7 +116,17 @@ __global__ __launch_bounds__(256) void absmax_rows_kernel(const void* __restrict
          r += workers) {
         AbsAcc<DT> a;
         const int64_t base = r * inner;
-        for (int64_t c = c0 + sub; c < c1; c += L) {
+        int64_t c = c0 + sub;
+        if (ALIGNED && (inner & 7) == 0) {
+            // whole chunks only: four loads of the lane in flight at a time
+            for (; c + 3 * L < c1; c += 4 * L) {
+                a.chunk(x, base + (c << 3));
+                a.chunk(x, base + ((c + L) << 3));
+                a.chunk(x, base + ((c + 2 * L) << 3));
+                a.chunk(x, base + ((c + 3 * L) << 3));
+            }
+        }
+        for (; c < c1; c += L) {
             const int64_t col = c << 3;
             if (ALIGNED && col + 8 <= inner) {
                 a.chunk(x, base + col);
@@ -147,11 +157,23 @@ __global__ __launch_bounds__(256) void absmax_short_rows_kernel(const void* __re
     const int64_t chunks = nrows << lg_l;
     const int64_t c0 = (int64_t)blockIdx.x * 1024 + threadIdx.x;
     RawChunk<DT> raw[4];
+    uint32_t old[4] = {0, 0, 0, 0};
+    // all loads first and in straight-line code (a chunk past the end re-reads the last one and
+    // folds nothing): the four chunks, then -- for the plain read-modify-write of an accumulator
+    // that one row feeds -- the four accumulator words, one round trip instead of one per round
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-        const int64_t c = c0 + u * 256;
-        zero_raw<DT>(raw[u]);
-        if (c < chunks) load_raw<DT>(x, c << 3, raw[u]);
+        int64_t c = c0 + u * 256;
+        c = c < chunks ? c : chunks - 1;
+        load_raw<DT>(x, c << 3, raw[u]);
+    }
+    if (exclusive) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            int64_t c = c0 + u * 256;
+            c = c < chunks ? c : chunks - 1;
+            old[u] = acc[c >> lg_l];
+        }
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -161,11 +183,10 @@ __global__ __launch_bounds__(256) void absmax_short_rows_kernel(const void* __re
         const uint32_t v = group_max_u32(a.bits(), lg_l);
         if (c < chunks && (threadIdx.x & ((1 << lg_l) - 1)) == 0) {
             const int64_t r = c >> lg_l;
-            uint32_t* dst = acc + (exclusive ? r : r % axis);
             if (exclusive) {
-                if (v > *dst) *dst = v;
+                if (v > old[u]) acc[r] = v;
             } else {
-                fold_max(dst, v);
+                fold_max(acc + r % axis, v);
             }
         }
     }
