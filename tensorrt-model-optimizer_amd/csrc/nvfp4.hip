@@ -334,10 +334,14 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_multi_kernel(
         }
     }
     const mo_nvfp4_job jb = jobs[lo];
-    // The amax is fetched, and the global scale stored, before the tile's loads go out.  Issuing
-    // the loads first (they do not depend on the amax) measured 2 % slower at every occupancy
-    // cap: the chip is short of memory bandwidth, not of requests in flight.
-    const float a = *as_global(jb.amax);
+    // The amax is fetched with a vector load through the generic pointer, and the global scale
+    // stored, before the tile's loads go out.  Measured against this in alternating runs:
+    // issuing the tile's loads first (they do not depend on the amax) is 2 % slower at every
+    // occupancy cap, and fetching the amax through the scalar cache (a much shorter round trip)
+    // 5 % slower; an explicit sleep of 0.5 us or more at the start is slower too.  The launch is
+    // short of memory bandwidth, not of requests in flight, and the round trip of this one load
+    // happens to space the workgroups' bursts well.
+    const float a = jb.amax[0];
     const float wsf2 = amax_is_wsf2 ? a : a / 2688.0f;
     if (jb.wsf2_out && t == jb.tile_begin && threadIdx.x == 0) jb.wsf2_out[0] = wsf2;
     quantize_tile_bf16((const uint16_t*)jb.x, jb.elems >> 4, t - jb.tile_begin, wsf2, 6.0f * wsf2,
