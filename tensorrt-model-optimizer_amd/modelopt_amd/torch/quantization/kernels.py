@@ -140,6 +140,9 @@ def _qdq(x, amax, run):
     return _undo_permutation(y.view(xp.shape), perm)
 
 
+with_scale_layout = _qdq   # the storage casts place their scales the same way
+
+
 def fake_quant_int(x, amax, num_bits=8, unsigned=False, narrow_range=True):
     return _qdq(x, amax, lambda x2, a, outer, axis, inner: _hip.int_qdq(
         x2, a, outer, axis, inner, num_bits, unsigned, narrow_range))

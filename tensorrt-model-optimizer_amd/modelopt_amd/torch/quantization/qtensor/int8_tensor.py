@@ -22,11 +22,10 @@ class INT8QTensor(BaseQuantizedTensor):
         if scales is None:
             amax = reduce_amax(x, axis=convert_quantization_axis_to_reduce_axis(x, axis))
             scales = true_divide(amax, 127.0)
-        layout = kernels.layout_from_amax_shape(tuple(x.shape), tuple(scales.shape))
-        if layout is None:
-            raise NotImplementedError("scale shape not covered by the kernels")
         via = torch.result_type(x, scales)
-        q = _hip.real_quantize(x, scales.reshape(-1).contiguous(), *layout, via, _hip.MO_FMT_INT8)
+        # scales on two separated runs of dims go through a transposing copy, like fake quant
+        q = kernels.with_scale_layout(x, scales, lambda x2, s, outer, axis, inner: _hip.real_quantize(
+            x2, s, outer, axis, inner, via, _hip.MO_FMT_INT8))
         return cls(input.shape, input.dtype, q), scales
 
     def dequantize(self, dtype: torch.dtype = None, **kwarg):
@@ -39,6 +38,5 @@ class INT8QTensor(BaseQuantizedTensor):
         if block_sizes:
             return _block_dequantize(q, self.metadata["shape"], scales, block_sizes,
                                      _hip.MO_FMT_INT8, dtype)
-        layout = kernels.layout_from_amax_shape(tuple(q.shape), tuple(scales.shape))
-        return _hip.real_dequantize(q.view(torch.uint8), scales.reshape(-1).contiguous(), *layout,
-                                    _hip.MO_FMT_INT8, dtype)
+        return kernels.with_scale_layout(q, scales, lambda q2, s, outer, axis, inner: _hip.real_dequantize(
+            q2.view(torch.uint8), s, outer, axis, inner, _hip.MO_FMT_INT8, dtype))

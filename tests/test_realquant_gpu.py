@@ -144,6 +144,29 @@ def test_int8_quantize_dequantize(dtype):
     assert_bits_equal(y.cpu(), qtensor.int8_dequantize(q_o, s_o, x.shape, dtype), "int8 dequant")
 
 
+@pytest.mark.parametrize("cls_name", ["FP8QTensor", "INT8QTensor"])
+def test_qtensor_scales_on_separated_dims(cls_name):
+    """Scales given on two dims with a reduced dim between them ([a, 1, c]): what the reference
+    computes by broadcasting, (x / scales) cast to the storage type and back."""
+    from modelopt_amd.torch.quantization import qtensor as q_mod
+    cls = getattr(q_mod, cls_name)
+    bound = 448.0 if cls_name == "FP8QTensor" else 127.0
+    x = _rand((6, 10, 16), torch.bfloat16, 21, scale=1.0)
+    scales = (x.abs().amax(dim=1, keepdim=True) / bound).to(torch.bfloat16)
+    assert scales.shape == (6, 1, 16)
+    qt, s_out = cls.quantize(x.to(DEV), scales=scales.to(DEV))
+    q = qt._quantized_data.cpu()
+    if cls_name == "FP8QTensor":
+        q_o, _ = qtensor.fp8_quantize(x, scales=scales)
+        want_y = qtensor.fp8_dequantize(q_o, scales, x.shape, torch.bfloat16)
+    else:
+        q_o, _ = qtensor.int8_quantize(x, scales=scales)
+        want_y = qtensor.int8_dequantize(q_o, scales, x.shape, torch.bfloat16)
+    assert torch.equal(q.view(torch.uint8), q_o.view(torch.uint8))
+    y = qt.dequantize(torch.bfloat16, scale=scales.to(DEV)).cpu()
+    assert_bits_equal(y, want_y, "dequantised")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape,bs", [((64, 256), 128), ((32, 64), 64), ((1, 10), 4), ((16, 48), 32)])
 def test_int4_block_quantize(dtype, shape, bs):
