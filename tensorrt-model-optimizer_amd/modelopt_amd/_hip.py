@@ -347,6 +347,11 @@ def fused_scratch(device, stream=None):
     index = torch.device(device).index
     index = torch.cuda.current_device() if index is None else index
     if stream is None:
+        if torch.cuda.is_current_stream_capturing():
+            # the fill that zeroes a new workspace becomes a node of the graph and does not run
+            # now, so a workspace made here would reach later eager calls unzeroed: each captured
+            # call gets its own, zeroed by its own node on every replay, and none is kept
+            return torch.zeros(FUSED_WS_BYTES // 4, dtype=torch.int32, device=torch.device("cuda", index))
         stream = torch._C._cuda_getCurrentRawStream(index)
     ws = _fused_ws_by_device.get((index, stream))
     if ws is None:
@@ -358,7 +363,8 @@ def fused_scratch(device, stream=None):
 
 def fused_gave_up(device=None) -> bool:
     """Whether a fused kernel (on ``device``; default: any device) ended without writing its
-    outputs because a workgroup gave up waiting for the others.  Synchronises; clears the state."""
+    outputs because a workgroup gave up waiting for the others.  Synchronises; clears the state.
+    Calls recorded into a graph use workspaces of their own that this check does not see."""
     index = None if device is None else torch.device(device).index
     failed = False
     for (dev, _), ws in _fused_ws_by_device.items():
