@@ -179,7 +179,18 @@ __global__ __launch_bounds__(256) void real_quantize_tile_kernel(
         }
         float q[8];
         const bool fast = mid_range(s) && u2f(m) * r < 1.0e38f;  // a NaN element fails the comparison
-        if (fast) {
+        // bf16 / bf16 rounded to bf16: both significands have 8 bits, so the exact quotient stays
+        // 2^-17 of its value away from every rounding boundary of bf16 (and is never on one) and
+        // x times the hardware reciprocal, good to 2^-22, rounds to the same bf16 value as the
+        // correctly rounded fp32 quotient.  Where that product is an fp32 denormal the bound
+        // does not hold, but both roundings are then far below half the smallest E4M3 / INT8
+        // step and give the same (signed) zero.
+        const bool narrow = DT == MO_BF16 && VIA == MO_BF16 && (f2u(s) & 0xFFFFu) == 0u;
+        if (fast && narrow) {
+            const float ra = __builtin_amdgcn_rcpf(s);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[j] = v[u][j] * ra;
+        } else if (fast) {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
                 q[j] = __builtin_copysignf(exact_quotient(v[u][j], s, r), v[u][j]);
@@ -435,20 +446,29 @@ __global__ __launch_bounds__(256) void int4_block_dequantize_tile_kernel(
         const float s = sc[u];
         const float r = 1.0f / s;
         const bool fast = mid_range(s);
-        float v[8];
+        float v[8];   // codes + 8
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const uint32_t b = (w[u] >> (8 * j)) & 0xFFu;
-            v[2 * j] = (float)(int)(b >> 4) - 8.0f;
-            v[2 * j + 1] = (float)(int)(b & 0xFu) - 8.0f;
+            v[2 * j] = (float)((w[u] >> (8 * j + 4)) & 0xFu);
+            v[2 * j + 1] = (float)((w[u] >> (8 * j)) & 0xFu);
         }
-        if (fast) {
+        if (fast && DT == MO_BF16) {
+            // a code has 4 significant bits and a bf16 scale 8: the exact quotient stays at
+            // least 2^-17 of its value away from every rounding boundary of bf16 (it cannot
+            // lie on one: the boundary's odd 9-bit numerator times the scale has more bits than
+            // a code), so code times the reciprocal, good to 2^-22, rounds to the same bf16
+            // value as the correctly rounded fp32 quotient.  (n - 8) * ra in one FMA: 8 * ra is
+            // exact, so the sum is rounded once, and n = 8 gives +0 as 0 / s does.
+            const float ra = __builtin_amdgcn_rcpf(s), off = -8.0f * ra;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = exact_quotient(v[j], s, r);  // 0 / s = +0, s > 0
+            for (int j = 0; j < 8; ++j) v[j] = __builtin_fmaf(v[j], ra, off);
+        } else if (fast) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = exact_quotient(v[j] - 8.0f, s, r);  // 0 / s = +0, s > 0
         } else {
             keep_branch();
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = v[j] / s;
+            for (int j = 0; j < 8; ++j) v[j] = (v[j] - 8.0f) / s;
         }
         if (c < chunks) store_chunk<DT>(y, c << 3, v);
     }

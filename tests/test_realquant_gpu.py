@@ -225,6 +225,39 @@ def test_storage_cast_every_pattern_and_extreme_scales(dtype, fmt):
             assert_bits_equal(got.cpu(), want, f"scale {sv}")
 
 
+@pytest.mark.parametrize("fmt", ["e4m3", "int8"])
+def test_storage_cast_bf16_by_bf16_every_pattern_and_every_scale_significand(fmt):
+    """bf16 / bf16 rounded to bf16 takes x times the reciprocal of the scale when the scale is
+    mid-range: every input pattern under every significand of the scale at several exponents
+    (the outermost ones go through the division), per row, per short row and per tensor."""
+    x = _all_patterns(torch.bfloat16)
+    code = _hip.MO_FMT_E4M3 if fmt == "e4m3" else _hip.MO_FMT_INT8
+    sig = 1.0 + torch.arange(128, dtype=torch.float32) / 128.0
+    s = torch.cat([sig * 2.0**e for e in (-100, -64, -21, -3, 0, 6, 63, 70)]).to(torch.bfloat16)
+    rows = s.numel()
+    xs = x.repeat(rows, 1)                                              # [rows, 65536]
+    q = xs / s[:, None]                                                 # bf16 by type promotion
+
+    def want_of(q):
+        return q.to(torch.float8_e4m3fn) if fmt == "e4m3" else q.round().clamp(-128, 127).to(torch.int8)
+
+    def check(got, q, what):
+        if fmt == "int8":
+            ok = ~torch.isnan(q)      # a NaN quotient has no defined int8 value in the reference
+            assert torch.equal(got.cpu()[ok], want_of(q)[ok]), what
+        else:
+            assert_bits_equal(got.cpu(), want_of(q), what)
+
+    xd, sd = xs.to(DEV), s.to(DEV)
+    check(_hip.real_quantize(xd, sd, 1, rows, 65536, torch.bfloat16, code), q, "one scale per long row")
+    short = sd.repeat_interleave(64)                                    # the same data as rows of 1024
+    check(_hip.real_quantize(xd.view(rows * 64, 1024), short, 1, rows * 64, 1024, torch.bfloat16, code).view(rows, 65536),
+          q, "one scale per short row")
+    for i in (0, 77, 5 * 128 + 127, 3 * 128 + 1, 6 * 128 + 64):
+        got = _hip.real_quantize(xd[i].contiguous(), sd[i].reshape(1), 1, 1, 65536, torch.bfloat16, code)
+        check(got, q[i], f"per tensor, scale {float(s[i])}")
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_storage_cast_row_scales_and_unaligned_views(dtype):
     g = torch.Generator().manual_seed(12)
@@ -272,6 +305,21 @@ def test_int4_block_quantize_special_blocks(dtype, bs):
     y = _hip.int4_block_dequantize(packed, scales, bs).reshape(nblk, bs)
     y_o = qtensor.int4_dequantize(got.reshape(p_o.shape), s_o, bs, x.shape, dtype)
     assert_bits_equal(y.cpu(), y_o, "dequant")
+
+
+def test_int4_dequantize_every_code_under_every_bf16_scale():
+    """bf16 takes code * reciprocal instead of the division when the scale is mid-range: all 16
+    codes under every finite positive and negative bf16 scale (the ends of the exponent range and
+    the negative ones go through the division) against the reference's expression."""
+    bits = torch.arange(0x10000, dtype=torch.int32)
+    scales = bits.to(torch.int16).view(torch.bfloat16)
+    scales = scales[torch.isfinite(scales.float()) & (scales.float() != 0)].contiguous()
+    nblk = scales.numel()
+    codes = torch.arange(16, dtype=torch.uint8)
+    packed = (codes[0::2] << 4 | codes[1::2]).repeat(nblk)          # a block of 16 holds each code once
+    y = _hip.int4_block_dequantize(packed.to(DEV), scales.to(DEV), 16)
+    y_o = qtensor.int4_dequantize(packed, scales.reshape(-1, 1), 16, (nblk, 16), torch.bfloat16)
+    assert_bits_equal(y.cpu().reshape(nblk, 16), y_o, "dequant")
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
