@@ -22,38 +22,49 @@ __device__ __forceinline__ void load_scales8(const void* s, int s_dtype, int64_t
 
 // y[r, c] = T( f32(x[r, c]) * f32(s[c]) )   (bf16 * bf16 -> bf16 and bf16 * fp32 -> fp32 -> bf16
 // both reduce to one fp32 product rounded once to T).
-// Vector path (k % 8 == 0, aligned): a lane keeps the scales of its 8 columns in registers and
-// walks down a slab of rows, 4 rows of loads in flight.
-template <int DT>
+// Vector path (k % 8 == 0, aligned): a workgroup owns kMulRows rows of 256 column chunks; a lane
+// loads its chunk of every row and the scales of its 8 columns first, in straight-line code,
+// then multiplies and stores -- no load is issued behind a store, which it would have to wait
+// for.  (Conditional stores would do for the short last slab, but the compiler then sinks a
+// row's load into the block of its store; the short slab has a path of its own instead.)
+constexpr int kMulRows = 8;
+template <int DT, int SD>
 __global__ __launch_bounds__(256) void mul_cols8_kernel(const void* __restrict__ x, int64_t rows,
-                                                        int64_t k, int64_t slab,
-                                                        const void* __restrict__ s, int s_dtype,
+                                                        int64_t k, int64_t col_groups,
+                                                        const void* __restrict__ s,
                                                         void* __restrict__ y) {
-    const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) << 3;
+    const int64_t slab = (int64_t)blockIdx.x / col_groups;
+    const int64_t group = (int64_t)blockIdx.x - slab * col_groups;
+    const int64_t col = (group * 256 + threadIdx.x) << 3;
     if (col >= k) return;
-    float sc[8];
-    load_scales8(s, s_dtype, col, sc);
-    const int64_t r0 = (int64_t)blockIdx.y * slab;
-    int64_t r1 = r0 + slab;
-    if (r1 > rows) r1 = rows;
-    int64_t r = r0;
-    for (; r + 3 < r1; r += 4) {
-        float v[4][8];
+    const int64_t r0 = slab * kMulRows;
+    RawChunk<SD> sraw;
+    load_raw<SD>(s, col, sraw);
+    if (r0 + kMulRows <= rows) {
+        RawChunk<DT> raw[kMulRows];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) load_chunk<DT>(x, (r + u) * k + col, v[u]);
+        for (int u = 0; u < kMulRows; ++u) load_raw<DT>(x, (r0 + u) * k + col, raw[u]);
+        float sc[8];
+        unpack_raw<SD>(sraw, sc);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < kMulRows; ++u) {
+            float v[8];
+            unpack_raw<DT>(raw[u], v);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[u][j] *= sc[j];
-            store_chunk<DT>(y, (r + u) * k + col, v[u]);
+            for (int j = 0; j < 8; ++j) v[j] *= sc[j];
+            store_chunk<DT>(y, (r0 + u) * k + col, v);
         }
-    }
-    for (; r < r1; ++r) {
-        float v[8];
-        load_chunk<DT>(x, r * k + col, v);
+    } else {
+        // the last, short slab of the tensor: row by row
+        float sc[8];
+        unpack_raw<SD>(sraw, sc);
+        for (int64_t r = r0; r < rows; ++r) {
+            float v[8];
+            load_chunk<DT>(x, r * k + col, v);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] *= sc[j];
-        store_chunk<DT>(y, r * k + col, v);
+            for (int j = 0; j < 8; ++j) v[j] *= sc[j];
+            store_chunk<DT>(y, r * k + col, v);
+        }
     }
 }
 
@@ -504,18 +515,17 @@ extern "C" int mo_mul_cols(const void* x, int64_t rows, int64_t k, int dtype, co
     const bool vec = (k % 8 == 0) && ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)s) & 15u) == 0);
     if (vec) {
         const int64_t gx = (k / 8 + 255) / 256;
-        // about 8192 workgroups in all and 4 per CU resident: 6.0 - 6.2 TB/s from 67 MB to 235 MB
-        // (4096 workgroups lose 5 % on 14336-wide rows, 1024 lose 10 %)
-        const int64_t want = mo::tuned("mul_cols_workgroups", 8192);
-        int64_t gy = (want + gx - 1) / gx;
-        int64_t slab = (rows + gy - 1) / gy;
-        if (slab < 8) slab = 8;
-        gy = (rows + slab - 1) / slab;
-        if (gy > 65535) { gy = 65535; slab = (rows + gy - 1) / gy; gy = (rows + slab - 1) / slab; }
-        dim3 grid((unsigned)gx, (unsigned)gy);
-#define CALL(DT) mo::mul_cols8_kernel<DT><<<grid, 256, mo::ballast_bytes("mul_cols8_kernel", 36), st>>>(x, rows, k, slab, s, s_dtype, y)
+        const int64_t blocks = gx * ((rows + mo::kMulRows - 1) / mo::kMulRows);
+        if (blocks > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+#define CALL_SD(DT, SD) \
+    mo::mul_cols8_kernel<DT, SD><<<(unsigned)blocks, 256, mo::ballast_bytes("mul_cols8_kernel", 36), st>>>(x, rows, k, gx, s, y)
+#define CALL(DT)                                     \
+    if (s_dtype == MO_F32) CALL_SD(DT, MO_F32);      \
+    else if (s_dtype == MO_F16) CALL_SD(DT, MO_F16); \
+    else CALL_SD(DT, MO_BF16)
         DISPATCH_DT(dtype, CALL)
 #undef CALL
+#undef CALL_SD
     } else {
         const unsigned g = mo::blocks_for_awq(rows * ((k + 7) >> 3));
 #define CALL(DT) mo::mul_cols_kernel<DT><<<g, 256, 0, st>>>(x, rows, k, s, s_dtype, y)
