@@ -356,9 +356,10 @@ def secondary_kernels(torch, steps, warmup):
 
     def rec(name, fn, nbytes):
         # one event pair around a train of launches: these kernels run for 5 - 50 us, which a
-        # pair of events per launch would inflate
-        reps = max(steps, 50)
-        for _ in range(max(warmup, 10)):
+        # pair of events per launch would inflate.  An untimed train of the same length goes
+        # first: the first milliseconds after other work run 5 - 10 % slower (clocks, caches)
+        reps = max(steps, 200)
+        for _ in range(max(warmup, reps)):
             fn()
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
