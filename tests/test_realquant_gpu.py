@@ -258,6 +258,33 @@ def test_storage_cast_bf16_by_bf16_every_pattern_and_every_scale_significand(fmt
         check(got, q[i], f"per tensor, scale {float(s[i])}")
 
 
+@pytest.mark.parametrize("k", [2048, 2112, 4096, 6144, 14336])
+@pytest.mark.parametrize("rows", [3, 37])
+def test_storage_cast_row_scales_on_long_rows(rows, k):
+    """One scale per row on rows of 256 chunks and more: widths that are a multiple of 2048 take
+    flat tiles with one scale per round of 256 chunks, the others one row per workgroup; the
+    tensor ends in the middle of a tile either way."""
+    g = torch.Generator().manual_seed(rows * 100003 + k)
+    x = (torch.randn((rows, k), generator=g) * 2).to(torch.bfloat16)
+    x[1, 5] = float("inf"); x[2, :] = 0.0; x[0, 3] = -0.0
+    for sdtype in (torch.float32, torch.bfloat16):
+        s = (x.float().abs().amax(dim=1).clamp(min=1e-3, max=1e30) / 448.0).to(sdtype)
+        quot = x / s[:, None]                 # fp32 scales promote to fp32, bf16 scales stay bf16
+        for fmt, code in (("e4m3", _hip.MO_FMT_E4M3), ("int8", _hip.MO_FMT_INT8)):
+            got = _hip.real_quantize(x.to(DEV), s.to(DEV), 1, rows, k, quot.dtype, code)
+            if fmt == "e4m3":
+                want = quot.to(torch.float8_e4m3fn)
+                assert_bits_equal(got.cpu(), want, f"{fmt}, {sdtype} scales")
+                y = _hip.real_dequantize(got, s.to(DEV), 1, rows, k, code, torch.bfloat16)
+                assert_bits_equal(y.cpu(), want.to(torch.bfloat16) * s[:, None].to(torch.bfloat16), "dequant")
+            else:
+                ok = ~torch.isnan(quot)
+                want = quot.round().clamp(-128, 127).to(torch.int8)
+                assert torch.equal(got.cpu()[ok], want[ok]), f"{fmt}, {sdtype} scales"
+                y = _hip.real_dequantize(got, s.to(DEV), 1, rows, k, code, torch.bfloat16)
+                assert_bits_equal(y.cpu()[ok], (want.to(torch.bfloat16) * s[:, None].to(torch.bfloat16))[ok], "dequant")
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_storage_cast_row_scales_and_unaligned_views(dtype):
     g = torch.Generator().manual_seed(12)
