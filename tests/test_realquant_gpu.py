@@ -285,6 +285,20 @@ def test_storage_cast_row_scales_on_long_rows(rows, k):
                 assert_bits_equal(y.cpu()[ok], (want.to(torch.bfloat16) * s[:, None].to(torch.bfloat16))[ok], "dequant")
 
 
+def test_storage_cast_scales_on_a_middle_dim_of_long_rows():
+    """[outer, axis, inner] with outer > 1 and inner a multiple of 2048: the scale index wraps
+    around after every ``axis`` rows."""
+    g = torch.Generator().manual_seed(21)
+    x = (torch.randn((5, 3, 4096), generator=g) * 2).to(torch.bfloat16)
+    s = torch.tensor([0.011, 0.5, 3.0])
+    quot = x / s[None, :, None]                                    # fp32 by promotion
+    want = quot.to(torch.float8_e4m3fn)
+    got = _hip.real_quantize(x.to(DEV), s.to(DEV), 5, 3, 4096, torch.float32, _hip.MO_FMT_E4M3)
+    assert_bits_equal(got.cpu(), want, "quantize")
+    y = _hip.real_dequantize(got, s.to(DEV), 5, 3, 4096, _hip.MO_FMT_E4M3, torch.bfloat16)
+    assert_bits_equal(y.cpu(), want.to(torch.bfloat16) * s[None, :, None].to(torch.bfloat16), "dequantize")
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_storage_cast_row_scales_and_unaligned_views(dtype):
     g = torch.Generator().manual_seed(12)
