@@ -391,8 +391,8 @@ int mo_awq_scale_activations(const void* x, const void* inv_s, int64_t n_alpha, 
  * xs holds the activations already multiplied by 1 / s[a], chunk-major: [n_alpha][k / 8][tokens][8]
  * (element (t, c) of alpha a at ((a * (k / 8) + c / 8) * tokens + t) * 8 + c % 8), so that the
  * lanes of a matrix-core operand read adjacent memory; w [n, k]; s [n_alpha, k]; ref [tokens, n];
- * loss: n_alpha doubles, accumulated into.  The quantised weights
- * and the outputs never reach memory.  Returns MO_ERR_UNSUPPORTED unless dtype is bf16,
+ * loss: n_alpha doubles, accumulated into (one atomic add per column tile, so the last bits depend
+ * on the order the tiles finish in).  The quantised weights and the outputs never reach memory.  Returns MO_ERR_UNSUPPORTED unless dtype is bf16,
  * tokens <= 512, n % 128 == 0, k % 128 == 0, block_size is 32, 64 or 128 and the buffers are
  * 16-byte aligned, or the grid is unsigned (use mo_scale_block_int_qdq + a GEMM + mo_sq_diff_sum
  * per alpha then).  The integer codes are the reference's; the dequantised weight is

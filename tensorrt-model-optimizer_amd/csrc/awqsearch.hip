@@ -8,8 +8,8 @@
 // dynamic block amax -> fake quant -> linear -> squared error against the unquantised output,
 // TQ/model_calib.py:645-690) with the activations already multiplied by 1 / s[a].
 //
-// A workgroup of 8 wavefronts owns a column tile of 128 output features for one alpha and all
-// T <= 512 tokens, so every weight element is scaled and quantised exactly once per alpha.  Every
+// A workgroup of 8 wavefronts owns a column tile of 128 (or 96) output features for one alpha and
+// all T <= 512 tokens, so every weight element is scaled and quantised exactly once per alpha.  Every
 // wavefront does both jobs: it multiplies its 64 (or 32) token rows with the quantised tile of
 // the current k block (B operand of v_mfma_f32_32x32x16_bf16 from LDS, A operand straight from a
 // chunk-major copy of the activations, in which the lanes of an operand read adjacent memory)
@@ -43,35 +43,17 @@ constexpr int kSearchBlockK = 128;  // k elements per step of the outer loop: 16
 constexpr int kSearchWaves = 8;
 constexpr int kXcds = 8;            // accelerator dies of the chip, each with its own L2
 
+// One column tile of 32 * NG output features (NG = 4 or 3) for alpha `a`, starting at feature n0.
 // RB = 32-row blocks per wavefront; the workgroup covers 8 * 32 * RB token rows.
-template <int RB>
-__global__ __launch_bounds__(512) void awq_search_kernel(
+template <int RB, int NG>
+__device__ __forceinline__ void awq_search_tile(
     const uint16_t* __restrict__ xs,   // [A][K / 8][T][8] bf16, activations * (1 / s[a])
     const uint16_t* __restrict__ w,    // [N, K] bf16
     const uint16_t* __restrict__ s,    // [A, K] bf16
     const uint16_t* __restrict__ ref,  // [T, N] bf16
-    int T, int N, int K, int n_alpha, int lg_g, float bound, double* __restrict__ loss) {
-    // quantised weight tile, two buffers: [128 rows][16 chunk slots] of 16 bytes; the slot of
-    // chunk c in row r is c ^ (r & 15) so that both the writers (16 lanes per row) and the
-    // readers (lanes along rows) spread over all banks
-    __shared__ u32x4 tile[2][kSearchTileN][16];
-    __shared__ double red[kSearchWaves];
-
+    int T, int N, int K, int a, int n0, int lg_g, float bound, double* __restrict__ loss,
+    u32x4 (&tile)[2][kSearchTileN][16], double (&red)[kSearchWaves]) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    // Workgroup L of a launch runs on XCD L % 8, and each XCD has its own L2.  All column tiles
-    // of an alpha read the same activations, so the (alpha, column tile) pairs are dealt out in
-    // contiguous runs: XCD x takes pairs [x * per, (x + 1) * per) in alpha-major order, i.e. the
-    // column tiles of one alpha run side by side on one XCD (at most two share an alpha) and
-    // the 4 MB of activations they walk through in step are fetched into that L2 once instead
-    // of once per XCD.  Every XCD gets the same number of pairs; the grid is padded to a
-    // multiple of 8 and the surplus workgroups leave at once.
-    const int ncol = N / kSearchTileN;
-    const int pairs = n_alpha * ncol, per = (pairs + kXcds - 1) / kXcds;
-    const int xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
-    const int pair = xcd * per + slot;
-    if (pair >= pairs) return;
-    const int a = pair / ncol;
-    const int n0 = (pair % ncol) * kSearchTileN;
     const int nkb = K / kSearchBlockK;
 
     // ---- producer side: chunk qc of rows qr + 32 u of the tile (u = 0..3), two chunks at a time.
@@ -84,7 +66,7 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
     const uint32_t wstride = 32u * (uint32_t)K * 2u;  // between the rows of two of a lane's chunks
     const char* srow = (const char*)(s + (int64_t)a * K);
     const uint32_t soff = (uint32_t)qc * 16u;
-    u32x4 wraw[4], sraw;    // raw weight chunks and scales of the block to quantise next
+    u32x4 wraw[NG], sraw;   // raw weight chunks and scales of the block to quantise next
     float sf[8];            // the scales of the block being quantised
     uint32_t vp[2][4];      // the pair of chunks being quantised: bf16(w * s), packed
     float mul[2], rdiv[2];  // per chunk: bound / amax and amax / bound
@@ -92,7 +74,7 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
     auto fetch = [&](int kb) {  // weights are used once per alpha: streamed past the L2
         const uint32_t k0 = (uint32_t)(kb < nkb ? kb : nkb - 1) * (kSearchBlockK * 2);
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < NG; ++u)
             wraw[u] = __builtin_nontemporal_load((const u32x4*)(wtile + k0 + u * wstride + woff));
         sraw = *(const u32x4*)(srow + k0 + soff);
     };
@@ -107,6 +89,7 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
         }
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
+            if (2 * h + i >= NG) continue;   // a tile of 96 features has three row groups
             const u32x4 r = wraw[2 * h + i];
             const uint32_t ww[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
@@ -116,10 +99,11 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
         }
     };
     const float inv_bound = 1.0f / bound;
-    auto block_scales = [&]() {  // block abs-max over the lanes of a block, then the two factors
+    auto block_scales = [&](int h) {  // block abs-max over the lanes of a block, then the two factors
         typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
+            if (2 * h + i >= NG) continue;
             // |bf16| bit patterns order like the magnitudes: 16-bit integer maxima, two a word
             u16x2 m2 = {0, 0};
 #pragma unroll
@@ -155,6 +139,7 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
     };
     // |v| <= amax, so the rounded code never leaves [-bound, bound]: no clamp is needed
     auto quantise_store = [&](int h, int i, int buf) {
+        if (2 * h + i >= NG) return;
         float y[8];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -174,7 +159,7 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
         const int h = j >> 2;
         switch (j & 3) {
             case 0: scale_pair(h); if (h == 1) fetch(kb_next + 1); break;
-            case 1: block_scales(); break;
+            case 1: block_scales(h); break;
             case 2: quantise_store(h, 0, buf); break;
             default: quantise_store(h, 1, buf); break;
         }
@@ -187,11 +172,11 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
     const int row_base = wave * (RB * 32);
     const bool has_rows = row_base < T;  // wavefronts past T only produce
     const uint16_t* xa = xs + (int64_t)a * T * K;
-    f32x16_t acc[RB][4];
+    f32x16_t acc[RB][NG];
 #pragma unroll
     for (int mb = 0; mb < RB; ++mb)
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb)
+        for (int nb = 0; nb < NG; ++nb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.0f;
     // Element offsets of this lane's A fragments.  xs is chunk-major: [K / 8][T][8], i.e. the 16
@@ -234,10 +219,10 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
         const int buf = kb & 1;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            bf16x8_t bfrag[4];
+            bf16x8_t bfrag[NG];
             const int c = j * 2 + kg;
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
+            for (int nb = 0; nb < NG; ++nb) {
                 const int r = nb * 32 + fr;
                 const u32x4 t = tile[buf][r][c ^ (r & 15)];
                 __builtin_memcpy(&bfrag[nb], &t, 16);
@@ -247,7 +232,7 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
                 bf16x8_t afrag;
                 __builtin_memcpy(&afrag, &af[mb][j % PF], 16);
 #pragma unroll
-                for (int nb = 0; nb < 4; ++nb)
+                for (int nb = 0; nb < NG; ++nb)
                     acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[nb],
                                                                           acc[mb][nb], 0, 0, 0);
             }
@@ -271,7 +256,7 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
 #pragma unroll
         for (int mb = 0; mb < RB; ++mb)
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
+            for (int nb = 0; nb < NG; ++nb) {
                 const uint16_t* rcol = ref + n0 + nb * 32 + fr;
                 uint16_t rv[16];
 #pragma unroll
@@ -300,6 +285,75 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
         for (int i = 0; i < kSearchWaves; ++i) total += red[i];
         atomicAdd(loss + a, total);
     }
+}
+
+// Every alpha's n columns are cut into `wide` tiles of 128 features followed by `narrow` tiles of
+// 96 (128 wide + 96 narrow = n).  A launch whose 128-wide tiles do not fill the chip's last round
+// (21 alphas x 32 tiles = 672 workgroups on 256 compute units that hold one each: 2.6 rounds)
+// trades some wide tiles for narrow ones, so that a unit's last tile is a short one.
+//
+// Workgroup L of a launch runs on XCD L % 8, and each XCD has its own L2.  All column tiles of
+// an alpha read the same activations, so tiles are dealt out in contiguous runs in alpha-major
+// order: XCD x takes wide tiles [x * per_wide, (x + 1) * per_wide) first and then narrow tiles
+// [x * per_narrow, (x + 1) * per_narrow) -- both runs cover about the same alphas, the column
+// tiles of one alpha run side by side on one XCD, and the 4 MB of activations they walk through
+// in step are fetched into that L2 once instead of once per XCD.  The grid is
+// 8 * (per_wide + per_narrow) workgroups; surplus ones leave at once.
+template <int RB>
+__global__ __launch_bounds__(512) void awq_search_kernel(
+    const uint16_t* __restrict__ xs, const uint16_t* __restrict__ w, const uint16_t* __restrict__ s,
+    const uint16_t* __restrict__ ref, int T, int N, int K, int n_alpha, int wide, int narrow,
+    int per_wide, int per_narrow, int lg_g, float bound, double* __restrict__ loss) {
+    // quantised weight tile, two buffers: [128 rows][16 chunk slots] of 16 bytes; the slot of
+    // chunk c in row r is c ^ (r & 15) so that both the writers (16 lanes per row) and the
+    // readers (lanes along rows) spread over all banks
+    __shared__ u32x4 tile[2][kSearchTileN][16];
+    __shared__ double red[kSearchWaves];
+    const int xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+    if (slot < per_wide) {
+        const int i = xcd * per_wide + slot;
+        if (i >= n_alpha * wide) return;
+        awq_search_tile<RB, 4>(xs, w, s, ref, T, N, K, i / wide, (i % wide) * 128, lg_g, bound,
+                               loss, tile, red);
+    } else {
+        const int i = xcd * per_narrow + (slot - per_wide);
+        if (i >= n_alpha * narrow) return;
+        awq_search_tile<RB, 3>(xs, w, s, ref, T, N, K, i / narrow, wide * 128 + (i % narrow) * 96,
+                               lg_g, bound, loss, tile, red);
+    }
+}
+
+// How many 96-wide tiles per alpha (a multiple of 4: four of them replace three 128-wide ones)
+// make the launch end soonest: tiles are handed to the compute units of an XCD in launch order
+// as units fall free, a tile costs its width plus a fixed part (prologue and epilogue, about 10
+// columns' worth), and the launch ends when the slowest XCD does.
+static inline int narrow_tiles_per_alpha(int64_t n_alpha, int64_t n, int units_per_xcd) {
+    int best = 0;
+    double best_end = 0.0;
+    double free_at[64];
+    if (units_per_xcd < 1) units_per_xcd = 1;
+    if (units_per_xcd > 64) units_per_xcd = 64;
+    for (int narrow = 0; narrow * 96ll <= n; narrow += 4) {
+        const int64_t wide = (n - narrow * 96ll) / 128;
+        const int64_t per_wide = (n_alpha * wide + kXcds - 1) / kXcds;
+        const int64_t per_narrow = (n_alpha * narrow + kXcds - 1) / kXcds;
+        for (int u = 0; u < units_per_xcd; ++u) free_at[u] = 0.0;
+        double end = 0.0;
+        for (int64_t t = 0; t < per_wide + per_narrow; ++t) {   // the fullest XCD
+            int first = 0;
+            for (int u = 1; u < units_per_xcd; ++u)
+                if (free_at[u] < free_at[first]) first = u;
+            free_at[first] += (t < per_wide ? 128.0 : 96.0) + 10.0;
+            if (free_at[first] > end) end = free_at[first];
+        }
+        // narrower tiles re-read the activations more often: they must pay for themselves
+        if (narrow == 0 || end < best_end * 0.97) {
+            best = narrow;
+            best_end = end;
+        }
+        if (narrow >= 64) break;
+    }
+    return best;
 }
 
 // xs[a][c][t][0..8) = bf16(x[t][8 c ..] * inv_s[a][8 c ..]) for every alpha: the activations the
@@ -360,12 +414,26 @@ extern "C" int mo_awq_search_losses(const void* xs, const void* w, const void* s
     if (is_unsigned) return MO_ERR_UNSUPPORTED;
     (void)narrow_range;
     hipStream_t st = (hipStream_t)stream;
-    const int64_t pairs = n_alpha * (n / mo::kSearchTileN);
-    const dim3 grid((unsigned)((pairs + mo::kXcds - 1) / mo::kXcds * mo::kXcds));
+    static int units_per_xcd = 0;   // compute units that share an L2 (one workgroup each)
+    if (units_per_xcd == 0) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < mo::kXcds)
+            cus = 256;
+        units_per_xcd = cus / mo::kXcds;
+    }
+    int narrow = (int)mo::tuned("search_narrow_tiles", -1);
+    if (narrow < 0) narrow = mo::narrow_tiles_per_alpha(n_alpha, n, units_per_xcd);
+    if (narrow % 4 || narrow * 96ll > n) return MO_ERR_ARG;
+    const int64_t wide = (n - narrow * 96ll) / 128;
+    const int64_t per_wide = (n_alpha * wide + mo::kXcds - 1) / mo::kXcds;
+    const int64_t per_narrow = (n_alpha * narrow + mo::kXcds - 1) / mo::kXcds;
+    const dim3 grid((unsigned)((per_wide + per_narrow) * mo::kXcds));
 #define CALL(RB)                                                                           \
     mo::awq_search_kernel<RB><<<grid, 512, 0, st>>>(                                       \
         (const uint16_t*)xs, (const uint16_t*)w, (const uint16_t*)s, (const uint16_t*)ref, \
-        (int)tokens, (int)n, (int)k, (int)n_alpha, lg_g, bound, loss)
+        (int)tokens, (int)n, (int)k, (int)n_alpha, (int)wide, narrow, (int)per_wide,       \
+        (int)per_narrow, lg_g, bound, loss)
     if (tokens <= 256) CALL(1);
     else CALL(2);
 #undef CALL

@@ -57,6 +57,20 @@ def test_matches_unfused_device_path(tokens, n, k, block, bits, unsigned, narrow
     assert (got > 0).all()
 
 
+@pytest.mark.parametrize("tokens,n,k,n_alpha", [(300, 2048, 256, 21), (96, 1536, 128, 11),
+                                                (512, 2560, 256, 21), (512, 4096, 4096, 21)])
+def test_column_tiles_of_two_widths(tokens, n, k, n_alpha):
+    """Launches whose 128-wide column tiles would leave the chip's last round part empty (more
+    than 256 tiles, one per compute unit at a time) cut some of every alpha's columns into
+    96-wide tiles: 16 of 20, all 16, 12 of 29 and 12 of 35 tiles per alpha in these cases."""
+    x, w, s = (t.to(DEV) for t in _problem(tokens, n, k, n_alpha, tokens + n))
+    ref = F.linear(x, w).contiguous()
+    got = _fused_losses(x, w, s, ref, 128, 4, False, False)
+    want = _unfused_losses(x, w, s, ref, 128, 4, False, False)
+    assert torch.allclose(got, want, rtol=1e-3, atol=0), (got, want)
+    assert int(got.argmin()) == int(want.argmin())
+
+
 def test_accumulates_and_rejects_uncovered_shapes():
     x, w, s = (t.to(DEV) for t in _problem(64, 128, 128, 2, 3))
     ref = F.linear(x, w).contiguous()
