@@ -62,6 +62,17 @@ enum mo_quantize_flags { MO_FLAG_FORCE_EXACT = 1, MO_FLAG_SATURATE_BLOCK_SCALE =
 int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
               float* acc, void* stream);
 
+/* Per-tensor mo_absmax (outer = axis = 1, inner = n) that also leaves the abs-max of every
+ * 32768-element tile of x in parts[0 .. *parts_written): the maximum of those words is the
+ * abs-max of this tensor alone, whatever acc held before.  For calibration loops that show one
+ * tensor to several calibrators in a row (the input of q_proj / k_proj / v_proj; MaxCalibrator.
+ * collect, TQ/calib/max.py:53-94, reduces it once per quantizer): the first reduction is shared,
+ * the others fold parts into their running maximum later instead of reading the tensor again.
+ * parts_written is a host pointer (set before the call returns).  MO_ERR_TOO_LARGE when the
+ * tiles outnumber parts_capacity, MO_ERR_UNSUPPORTED when x is not 16-byte aligned. */
+int mo_absmax_tensor_parts(const void* x, int64_t n, int dtype, float* acc, uint32_t* parts,
+                           int64_t parts_capacity, int64_t* parts_written, void* stream);
+
 /* The per-column case of mo_absmax (x viewed as [outer, axis], inner == 1) in two passes through
  * a caller-provided workspace: row slabs are reduced to partial[slabs, axis] with plain stores
  * (slabs <= partial_rows, chosen by the library), then the columns of that matrix are folded

@@ -75,7 +75,8 @@ __device__ __forceinline__ void fold_max_coherent(uint32_t* acc, uint32_t v) {
 // One workgroup per tile of TILE_ELEMS elements, dispatched in order.
 template <int DT, int TILE_ELEMS>
 __global__ __launch_bounds__(256) void absmax_flat_kernel(const void* __restrict__ x, int64_t n,
-                                                          uint32_t* __restrict__ acc) {
+                                                          uint32_t* __restrict__ acc,
+                                                          uint32_t* __restrict__ parts = nullptr) {
     __shared__ uint32_t smem[4];
     constexpr int64_t kTileChunks = TILE_ELEMS / 8;
     AbsAcc<DT> a;
@@ -93,7 +94,10 @@ __global__ __launch_bounds__(256) void absmax_flat_kernel(const void* __restrict
     for (; c < c1; c += 256) a.chunk(x, c << 3);
     if (c1 == chunks && threadIdx.x < (n & 7)) a.elem(x, (chunks << 3) + threadIdx.x);
     const uint32_t v = block_max_u32(a.bits(), smem);
-    if (threadIdx.x == 0) fold_max(acc, v);
+    if (threadIdx.x == 0) {
+        fold_max(acc, v);
+        if (parts) parts[blockIdx.x] = v;   // the tile's own maximum, for callers that share a reduction
+    }
 }
 
 // ------------------------------------------------------------------------------ rows
@@ -578,6 +582,30 @@ extern "C" int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
         default: return MO_ERR_DTYPE;
     }
     if (rc != MO_OK) return rc;
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_absmax_tensor_parts(const void* x, int64_t n, int dtype, float* acc,
+                                      uint32_t* parts, int64_t parts_capacity,
+                                      int64_t* parts_written, void* stream) {
+    if (n < 0 || parts_capacity < 0 || !parts_written) return MO_ERR_ARG;
+    *parts_written = 0;
+    if (n == 0) return MO_OK;
+    if (!x || !acc || !parts) return MO_ERR_ARG;
+    if (((uintptr_t)x & 15u) || ((uintptr_t)parts & 3u)) return MO_ERR_UNSUPPORTED;
+    constexpr int64_t kTile = 32768;
+    const int64_t tiles = (n + kTile - 1) / kTile;
+    if (tiles > parts_capacity) return MO_ERR_TOO_LARGE;
+    if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    const size_t cap = mo::ballast_bytes("absmax_flat_kernel", 36);
+    switch (dtype) {
+        case MO_F32: mo::absmax_flat_kernel<MO_F32, kTile><<<dim3((unsigned)tiles), 256, cap, s>>>(x, n, (uint32_t*)acc, parts); break;
+        case MO_F16: mo::absmax_flat_kernel<MO_F16, kTile><<<dim3((unsigned)tiles), 256, cap, s>>>(x, n, (uint32_t*)acc, parts); break;
+        case MO_BF16: mo::absmax_flat_kernel<MO_BF16, kTile><<<dim3((unsigned)tiles), 256, cap, s>>>(x, n, (uint32_t*)acc, parts); break;
+        default: return MO_ERR_DTYPE;
+    }
+    *parts_written = tiles;
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }
 

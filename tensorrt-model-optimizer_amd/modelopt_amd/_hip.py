@@ -27,6 +27,7 @@ SIGNATURES = {
     "mo_version": [],
     "mo_error_string": [_INT],
     "mo_absmax": [_P, _I64, _I64, _I64, _INT, _P, _P],
+    "mo_absmax_tensor_parts": [_P, _I64, _INT, _P, _P, _I64, _P, _P],
     "mo_absmax_cols_staged": [_P, _I64, _I64, _INT, _P, _P, _I64, _P],
     "mo_absmax_cols_noalloc": [_P, _I64, _I64, _INT, _P, _P],
     "mo_absmax_multi": [_P, _INT, _P, _I64, _INT, _P],
@@ -202,6 +203,37 @@ def absmax_into(x: torch.Tensor, acc: torch.Tensor, outer: int, axis: int, inner
         return acc
     call("mo_absmax", x, _ptr(x), outer, axis, inner, dtype_code(x.dtype), _ptr(acc), _stream(x))
     return acc
+
+
+_parts_ring = {}   # device index -> [int32 buffer, words handed out]
+_PARTS_RING_WORDS = 1 << 20
+
+
+def absmax_tensor_parts_into(x: torch.Tensor, acc: torch.Tensor):
+    """Per-tensor ``absmax_into`` that also returns the abs-max of every 32768-element tile of
+    ``x`` (int32 bit patterns of non-negative floats, a slice of a ring buffer that stays alive as
+    long as the slice does): ``parts.max()`` is the abs-max of this tensor alone.  None when the
+    tensor is not covered (the accumulator is untouched then)."""
+    _require_device(x, acc)
+    if not x.is_contiguous() or x.dtype not in _DTYPES or x.data_ptr() % 16 or acc.numel() != 1:
+        return None
+    n = x.numel()
+    tiles = -(-n // 32768)
+    if tiles == 0 or tiles > _PARTS_RING_WORDS:
+        return None
+    index = x.device.index
+    ring = _parts_ring.get(index)
+    if ring is None or ring[1] + tiles > _PARTS_RING_WORDS:
+        # slices handed out earlier keep their buffer alive; a new one starts here
+        ring = [torch.empty(_PARTS_RING_WORDS, dtype=torch.int32, device=x.device), 0]
+        _parts_ring[index] = ring
+    parts = ring[0][ring[1]:ring[1] + tiles]
+    written = ctypes.c_int64(0)
+    call("mo_absmax_tensor_parts", x, _ptr(x), n, dtype_code(x.dtype), _ptr(acc), _ptr(parts), tiles,
+         ctypes.byref(written), _stream(x))
+    assert written.value == tiles
+    ring[1] += tiles
+    return parts
 
 
 def fp8_qdq(x, amax, outer, axis, inner, saturate=False, out=None):

@@ -15,6 +15,30 @@ from ..utils import convert_quantization_axis_to_reduce_axis
 
 __all__ = ["MaxCalibrator"]
 
+# Inside a calibration pass of this package (the flag is raised by ``calibration_pass``) one
+# activation is often shown to several calibrators in a row -- the input of q_proj, k_proj and
+# v_proj, of gate_proj and up_proj.  The first per-tensor reduction then also leaves the abs-max
+# of every tile of the tensor behind, and a calibrator that is shown the *same tensor* next (same
+# memory, shape, strides, dtype and version counter, the tensor object of the first reduction
+# still alive so that its memory cannot have been handed out again) notes those words instead of
+# reading the tensor again; it folds them into its running maximum when that is next looked at.
+SHARE_REDUCTIONS = [False]
+_last_reduction = [None]   # (key, the tensor itself, its tile maxima)
+
+
+def forget_last_reduction():
+    """Drop the reference to the last tensor reduced (end of a calibration pass)."""
+    _last_reduction[0] = None
+
+
+def _sharing_key(x):
+    try:
+        version = x._version
+    except RuntimeError:   # inference tensors keep no version counter
+        return None
+    return (x.data_ptr(), version, tuple(x.shape), x.stride(), x.dtype, x.device.index,
+            torch._C._cuda_getCurrentRawStream(x.device.index))
+
 
 class _Calibrator:
     def __init__(self, num_bits=8, axis=None, unsigned=False):
@@ -46,6 +70,7 @@ class MaxCalibrator(_Calibrator):
         self._meta_amax = None       # meta-device shortcut only
         self._validated = False
         self._seen_parameter = None  # identity of the last nn.Parameter folded in
+        self._pending = []           # tile maxima of shared reductions not yet folded into _acc
 
     @property
     def amaxs(self):
@@ -58,7 +83,16 @@ class MaxCalibrator(_Calibrator):
         override ``compute_amax`` read it (tests/unit/torch/quantization/test_quantize_cpu.py:73-75)."""
         if self._acc is None:
             return self._meta_amax
+        self._fold_pending()
         return self._acc.to(self._dtype).reshape(self._shape)
+
+    def _fold_pending(self):
+        """Fold the tile maxima noted by shared reductions into the running maximum (the bit
+        patterns of non-negative floats order like the values; a NaN pattern is the largest)."""
+        if self._pending:
+            words = self._pending[0] if len(self._pending) == 1 else torch.cat(self._pending)
+            self._pending = []
+            self._acc = torch.maximum(self._acc.view(torch.int32), words.max()).view(torch.float32)
 
     @staticmethod
     def _amax_shape(x, reduce_axis):
@@ -94,7 +128,9 @@ class MaxCalibrator(_Calibrator):
         elif shape != self._shape:
             raise RuntimeError("amax shape changed!")
         if not self._track_amax:
-            kernels.absmax_accumulate(x, self._acc, layout)
+            if not (SHARE_REDUCTIONS[0] and layout[1] == 1 and x.is_cuda and x.is_contiguous()
+                    and not isinstance(x, torch.nn.Parameter)) or not self._collect_shared(x):
+                kernels.absmax_accumulate(x, self._acc, layout)
         else:
             local = torch.zeros_like(self._acc)
             kernels.absmax_accumulate(x, local, layout)
@@ -102,8 +138,28 @@ class MaxCalibrator(_Calibrator):
             self._amaxs.append(local.reshape(shape).to(x.dtype).float().cpu().numpy())
         self._validated = False
 
+    def _collect_shared(self, x) -> bool:
+        """Per-tensor reduction inside a calibration pass: note the tile maxima of the previous
+        reduction when it was of this very tensor, else reduce and leave the tile maxima for
+        the next calibrator.  False when the tensor is not covered (the caller reduces it)."""
+        key = _sharing_key(x)
+        if key is None:
+            return False
+        last = _last_reduction[0]
+        if last is not None and last[0] == key and last[1] is x:
+            self._pending.append(last[2])
+            if len(self._pending) >= 64:
+                self._fold_pending()
+            return True
+        parts = kernels._hip.absmax_tensor_parts_into(x, self._acc)
+        if parts is None:
+            return False
+        _last_reduction[0] = (key, x, parts)
+        return True
+
     def reset(self):
         self._seen_parameter = None
+        self._pending = []
         self._acc = None
         self._shape = None
         self._meta_amax = None
@@ -117,6 +173,7 @@ class MaxCalibrator(_Calibrator):
         """Running abs-max in the dtype of the collected tensors, or None if nothing was seen."""
         if self._acc is None:
             return self._meta_amax
+        self._fold_pending()
         # always a tensor of its own (never a view of the accumulator)
         amax = self._acc.to(self._dtype, copy=True).reshape(self._shape)
         if not self._validated:

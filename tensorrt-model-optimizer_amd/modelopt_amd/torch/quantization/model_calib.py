@@ -61,6 +61,9 @@ def finish_stats_collection(model: nn.Module, method: str | None = None):
                if isinstance(m, TensorQuantizer) and not m._disabled
                and getattr(m._calibrator, "_acc", None) is not None
                and not m._calibrator._validated]
+    for c in pending:
+        if hasattr(c, "_fold_pending"):
+            c._fold_pending()   # tile maxima of reductions shared with another calibrator
     if pending and all_valid_scales([c._acc for c in pending]):
         for c in pending:
             c._validated = True

@@ -47,10 +47,13 @@ def calibration_pass():
     that has not changed is reduced once, not once per forward."""
     _PASS_COUNTER[0] += 1
     previous, _CALIBRATION_PASS[0] = _CALIBRATION_PASS[0], _PASS_COUNTER[0]
+    shared, calib.max.SHARE_REDUCTIONS[0] = calib.max.SHARE_REDUCTIONS[0], True
     try:
         yield
     finally:
         _CALIBRATION_PASS[0] = previous
+        calib.max.SHARE_REDUCTIONS[0] = shared
+        calib.max.forget_last_reduction()
 
 
 class TensorQuantizer(nn.Module):

@@ -541,3 +541,66 @@ def test_per_tensor_calibration_of_a_permuted_view_makes_no_copy(monkeypatch):
     cal2.collect(sliced)
     assert_bits_equal(cal2.compute_amax().cpu(), reduce.reduce_amax(x[:, :, :4]), "amax of a slice")
     assert kernels.dense_flat_view(sliced) is None
+
+
+# ----------------------------------------------------------------------------- shared reductions
+def test_calibrators_shown_one_tensor_in_a_row_share_its_reduction():
+    """Inside a calibration pass the input of q_proj / k_proj / v_proj is read once: the first
+    calibrator's launch leaves the tile maxima behind and the others fold those in later."""
+    from modelopt_amd import _hip as hip
+    from modelopt_amd.torch.quantization.calib import MaxCalibrator
+    from modelopt_amd.torch.quantization.nn.modules.tensor_quantizer import calibration_pass
+
+    cals = [MaxCalibrator(8, None, False) for _ in range(3)]
+    batches = [_rand((16, 512, 256), torch.bfloat16, 300 + i, scale=1.0 + i).to(DEV) for i in range(3)]
+    with calibration_pass(), hip.KernelTimer() as timer:
+        for b in batches:
+            for c in cals:
+                c.collect(b)
+    assert timer.calls == {"mo_absmax_tensor_parts": 3}
+    want = max(float(reduce.reduce_amax(b.cpu(), None)) for b in batches)
+    for c in cals:
+        assert float(c.compute_amax()) == want
+        assert c.compute_amax().dtype == torch.bfloat16
+
+    # a tensor written in place between two calibrators is reduced again; so is an equal copy
+    a, b, c = (MaxCalibrator(8, None, False) for _ in range(3))
+    x = _rand((64, 1024), torch.bfloat16, 310).to(DEV)
+    with calibration_pass(), hip.KernelTimer() as timer:
+        a.collect(x)
+        x.mul_(2)
+        b.collect(x)
+        c.collect(x.clone())
+    assert timer.calls == {"mo_absmax_tensor_parts": 3}
+    assert float(b.compute_amax()) == 2 * float(a.compute_amax()) == float(c.compute_amax())
+
+    # outside a pass of the package every collect reduces, as the reference does
+    a, b = MaxCalibrator(8, None, False), MaxCalibrator(8, None, False)
+    with hip.KernelTimer() as timer:
+        a.collect(x)
+        b.collect(x)
+    assert timer.calls == {"mo_absmax": 2}
+    assert float(a.compute_amax()) == float(b.compute_amax())
+
+
+def test_shared_reductions_fold_after_many_batches_and_keep_nan():
+    from modelopt_amd.torch.quantization.calib import MaxCalibrator
+    from modelopt_amd.torch.quantization.nn.modules.tensor_quantizer import calibration_pass
+
+    lead, follow = MaxCalibrator(8, None, False), MaxCalibrator(8, None, False)
+    g = torch.Generator().manual_seed(320)
+    want = 0.0
+    with calibration_pass():
+        for i in range(150):     # more than one fold of the noted tile maxima
+            x = (torch.randn((8, 4096), generator=g) * (1 + i % 7)).to(torch.float16).to(DEV)
+            want = max(want, float(x.abs().max()))
+            lead.collect(x)
+            follow.collect(x)
+    assert float(lead.compute_amax()) == want == float(follow.compute_amax())
+    with calibration_pass():
+        x = torch.ones((8, 4096), dtype=torch.bfloat16, device=DEV)
+        x[3, 7] = float("nan")
+        lead.collect(x)
+        follow.collect(x)
+    with pytest.raises(AssertionError, match="nan"):
+        follow.compute_amax()
