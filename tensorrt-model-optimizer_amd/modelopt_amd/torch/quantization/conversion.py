@@ -48,6 +48,29 @@ def set_quantizer_by_cfg(quant_model: nn.Module, quant_cfg: dict | QuantizeConfi
     """
     quant_cfg = dict(quant_cfg)
     index = _quantizer_index(quant_model)  # walked once, shared by every pattern below
+    # When every entry is a complete attribute set (what validation makes of a dict), an entry
+    # replaces whatever an earlier one set: each quantizer then takes the last entry that matches
+    # it, once, instead of every matching entry in turn.
+    order = [("*", quant_cfg["default"], None)] if "default" in quant_cfg else []
+    for pattern, cfg in quant_cfg.items():
+        if pattern == "default":
+            continue
+        if isinstance(pattern, str) and pattern.startswith("nn.") and isinstance(cfg, dict) and all(
+                isinstance(v, (dict, list, QuantizerAttributeConfig)) for v in cfg.values()):
+            cls = getattr(nn, pattern[3:], None)
+            if cls is not None:
+                order += [(k, v, cls) for k, v in cfg.items()]
+        else:
+            order.append((pattern, cfg, None))
+    if all(isinstance(k, str) and isinstance(v, QuantizerAttributeConfig) for k, v, _ in order) \
+            and not any(isinstance(e[1], SequentialQuantizer) for e in index):
+        order.reverse()
+        for name, module, parent, _ in index:
+            for pattern, cfg, cls in order:
+                if (cls is None or isinstance(parent, cls)) and _compiled(pattern)(name) is not None:
+                    module.set_from_attribute_config(cfg)
+                    break
+        return
     if "default" in quant_cfg:
         set_quantizer_attribute(quant_model, "*", quant_cfg["default"], _index=index)
     for pattern, cfg in quant_cfg.items():
