@@ -22,13 +22,18 @@ __all__ = ["MaxCalibrator"]
 # memory, shape, strides, dtype and version counter, the tensor object of the first reduction
 # still alive so that its memory cannot have been handed out again) notes those words instead of
 # reading the tensor again; it folds them into its running maximum when that is next looked at.
+# Leaving the tile maxima behind costs the host a few microseconds per reduction, so it starts
+# only once a pass has shown one tensor to two calibrators in a row (the first layer of a model
+# with shared inputs does); a model whose quantizers never share an input pays nothing.
 SHARE_REDUCTIONS = [False]
-_last_reduction = [None]   # (key, the tensor itself, its tile maxima)
+_last_reduction = [None]   # (key, the tensor itself, its tile maxima or None)
+_sharing_seen = [False]
 
 
 def forget_last_reduction():
     """Drop the reference to the last tensor reduced (end of a calibration pass)."""
     _last_reduction[0] = None
+    _sharing_seen[0] = False
 
 
 def _sharing_key(x):
@@ -146,16 +151,17 @@ class MaxCalibrator(_Calibrator):
         if key is None:
             return False
         last = _last_reduction[0]
-        if last is not None and last[0] == key and last[1] is x:
+        if last is not None and last[1] is x and last[0] == key:
+            if last[2] is None:          # the same tensor twice in a row: share from now on
+                _sharing_seen[0] = True
+                return False
             self._pending.append(last[2])
             if len(self._pending) >= 64:
                 self._fold_pending()
             return True
-        parts = kernels._hip.absmax_tensor_parts_into(x, self._acc)
-        if parts is None:
-            return False
+        parts = kernels._hip.absmax_tensor_parts_into(x, self._acc) if _sharing_seen[0] else None
         _last_reduction[0] = (key, x, parts)
-        return True
+        return parts is not None
 
     def reset(self):
         self._seen_parameter = None

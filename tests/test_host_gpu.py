@@ -557,7 +557,9 @@ def test_calibrators_shown_one_tensor_in_a_row_share_its_reduction():
         for b in batches:
             for c in cals:
                 c.collect(b)
-    assert timer.calls == {"mo_absmax_tensor_parts": 3}
+    # the first batch finds out that the tensor is shared (three plain reductions); from the
+    # second on one reduction per batch serves all three calibrators
+    assert timer.calls == {"mo_absmax": 3, "mo_absmax_tensor_parts": 2}
     want = max(float(reduce.reduce_amax(b.cpu(), None)) for b in batches)
     for c in cals:
         assert float(c.compute_amax()) == want
@@ -571,7 +573,7 @@ def test_calibrators_shown_one_tensor_in_a_row_share_its_reduction():
         x.mul_(2)
         b.collect(x)
         c.collect(x.clone())
-    assert timer.calls == {"mo_absmax_tensor_parts": 3}
+    assert timer.calls == {"mo_absmax": 3}
     assert float(b.compute_amax()) == 2 * float(a.compute_amax()) == float(c.compute_amax())
 
     # outside a pass of the package every collect reduces, as the reference does
