@@ -73,6 +73,42 @@ def _converted(cfg):
     return m
 
 
+class _NetWithNorm(_Net):
+    def __init__(self):
+        super().__init__()
+        self.norm = nn.BatchNorm1d(16)      # the named configs carry entries scoped to nn classes
+        self.mlp = nn.Sequential(nn.Linear(16, 16))
+
+
+def _quantizer_state(model):
+    keep = ("_num_bits", "_axis", "_block_sizes", "_disabled", "_dynamic", "_unsigned", "_narrow_range",
+            "_fake_quant", "_learn_amax", "_trt_high_precision_dtype", "_bias", "_rotate", "_pass_through_bwd")
+    out = {}
+    for name, q in model.named_modules():
+        if isinstance(q, TensorQuantizer):
+            out[name] = {k: getattr(q, k, None) for k in keep}
+            out[name]["calibrator"] = type(q._calibrator).__name__
+    return out
+
+
+def test_single_pass_configuration_equals_entry_by_entry():
+    """With complete attribute sets only, each quantizer takes the last entry that matches it;
+    an entry with a filter function in place of a wildcard sends the same config through the
+    entry-by-entry route, and both must leave every quantizer in the same state."""
+    for name in mtq.config.choices:
+        quant_cfg, _ = mtq.model_quant._validated(getattr(mtq, name))
+        if any(isinstance(v, list) for v in quant_cfg.values()):
+            continue     # lists build SequentialQuantizers: entry-by-entry either way
+        a, b = _NetWithNorm(), _NetWithNorm()
+        mtq.replace_quant_module(a)
+        mtq.replace_quant_module(b)
+        mtq.set_quantizer_by_cfg(a, quant_cfg)
+        slow = dict(quant_cfg)
+        slow[lambda n: False] = quant_cfg["default"]       # matches nothing, forces the other route
+        mtq.set_quantizer_by_cfg(b, slow)
+        assert _quantizer_state(a) == _quantizer_state(b), name
+
+
 def test_conversion_adds_quantizers_and_keeps_parameters():
     m = _Net()
     w = m.body[0].weight
