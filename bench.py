@@ -33,6 +33,8 @@ DEQUANT_BYTES_PER_ELEM = 0.5 + 1.0 / 16.0 + 2.0
 # scale factors come from a 1 GiB device copy in the same runs
 # (profiles/nvfp4_quantize_multi_kernel__llama3_8b_weights.txt).
 MEASURED_TRAFFIC_BYTES_32_LAYERS = 17.912e9
+# mean kernel-trace duration of the 30 timed dispatches of the default run in that profile
+PROFILE_TIMED_LAUNCH_US = 2873.0
 TRAFFIC_SOURCE = ("profiles/nvfp4_quantize_multi_kernel__llama3_8b_weights.txt (rocprofv3 --pmc FETCH_SIZE, "
                   "WRITE_SIZE of this command, scaled by a device copy of known size)")
 
@@ -46,21 +48,24 @@ def make_weights(torch, layers, device):
     return ws
 
 
-def verify_against_restatement(torch, weights, amax, qplan, picks=(1, 3, 6)):
-    """What the timed launch wrote for a few tensors (k, o and down of the first layer) against the
-    C restatement of the reference arithmetic on the host: packed codes, block scales, global scale."""
+def verify_against_restatement(torch, weights, amax, qplan):
+    """What the timed launch wrote against the C restatement of the reference arithmetic on the
+    host (packed codes, block scales, global scale), for tensors spread over the whole launch:
+    k, o and down of the first layer, gate of the middle layer, and the three largest tensors
+    of the last layer (the launch's last tiles)."""
     from oracle import cref
 
     packed, wsf, wsf2 = qplan.packed, qplan.wsf, qplan.wsf2
     torch.cuda.synchronize()
+    per, n = len(LAYER_SHAPES), len(weights)
+    picks = sorted({1, 3, 6, (n // per // 2) * per + 4, n - 3, n - 2, n - 1} & set(range(n)))
     for i in picks:
-        if i >= len(weights):
-            continue
         p_c, s_c, w2_c = cref.nvfp4_quantize(weights[i].cpu(), 16, float(amax[i]))
         assert torch.equal(packed[i].cpu(), p_c), f"tensor {i}: packed codes differ"
         assert torch.equal(wsf[i].cpu().view(torch.uint8), s_c.view(torch.uint8)), f"tensor {i}: scales differ"
         assert float(wsf2[i]) == float(w2_c), f"tensor {i}: global scale differs"
-    return f"outputs of the timed launch for tensors {list(picks)} equal the CPU restatement bit for bit"
+    return (f"outputs of the timed launch for tensors {picks} of {n} (first, middle and last layer) "
+            "equal the CPU restatement bit for bit")
 
 
 def timed(torch, fn, steps, warmup):
@@ -580,6 +585,10 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "launch_ms": round(dev_ms, 4),
+            # the same fraction from the committed rocprofv3 kernel trace of the default run (another
+            # session, profiler attached): algorithmic bytes / mean duration of its timed dispatches
+            "frac_from_profile": (round(quant_bytes / (PROFILE_TIMED_LAUNCH_US * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)
+                                  if a.layers == 32 else None),
             # frac = algorithmic bytes / launch_ms / peak; traffic is NOT measured by this run: it is
             # the counter reading of the committed profile of this same command
             "traffic": MEASURED_TRAFFIC_BYTES_32_LAYERS if a.layers == 32 else None,

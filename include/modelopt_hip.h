@@ -249,15 +249,17 @@ int mo_nvfp4_quantize_multi(const mo_nvfp4_job* jobs_dev, int njobs, const int32
  * while the workgroups agree on the maximum.  All workgroups have to be resident at once, which
  * bounds the tensor size: MO_ERR_TOO_LARGE beyond 32 MiB (what two workgroups per compute unit
  * hold in registers), MO_ERR_UNSUPPORTED when the layout is not covered; the two-launch entry
- * points take over then.  Run one fused call at a time per device (successive calls in one
- * stream do that); other kernels may share the device.
+ * points take over then.  Other kernels may share the device.  Two fused calls that overlap
+ * (different streams) or a device that cannot hold the grid at once (masked compute units) do
+ * not break anything, they only make the call slow: see spin_limit.
  * workspace: MO_FUSED_WS_BYTES of device memory, 128-byte aligned, all zero before the first
  *   call; it can be reused by calls that follow each other in one stream (calls that overlap
- *   must not share a workspace).  The 32-bit word at byte MO_FUSED_WS_FAIL_OFFSET is set to 1
- *   if a workgroup gave up waiting for the others after spin_limit polls (a safety net: no
- *   wavefront waits for ever); such a workgroup fills its share of the outputs with NaN (NaN
- *   block-scale bytes for NVFP4) instead of results, and so does every later call on that
- *   workspace until the caller, having read the flag, has zeroed the workspace.
+ *   must not share a workspace).  Every call leaves it ready for the next one.
+ * spin_limit: polls (about half a microsecond each) a workgroup waits for the others.  A
+ *   workgroup whose wait expires computes the abs-max of the whole tensor by itself and goes on,
+ *   so the outputs are the same bits in every case; it also sets the 32-bit word at byte
+ *   MO_FUSED_WS_FAIL_OFFSET to 1, which tells the host that a call took that slow way (no kernel
+ *   reads the word; the host clears it).
  * amax_out (optional): the abs-max that was used, as fp32. */
 
 #define MO_FUSED_WS_BYTES 512
@@ -271,7 +273,8 @@ int mo_nvfp4_quantize_fused(const void* x, int64_t rows, int64_t k, int dtype, i
 
 /* mo_absmax (per tensor) followed by mo_int_qdq (kind 0) or mo_fp8_qdq (kind 1) with that amax:
  * dynamic per-tensor fake quantisation, TensorQuantizer._get_amax + _fake_quantize
- * (TQ/nn/modules/tensor_quantizer.py:505-514, 633-686).  x and y 16-byte aligned; y may alias x. */
+ * (TQ/nn/modules/tensor_quantizer.py:505-514, 633-686).  x and y 16-byte aligned and not
+ * overlapping (MO_ERR_UNSUPPORTED otherwise: a workgroup whose wait expired reads x again). */
 int mo_fused_amax_qdq(const void* x, void* y, int64_t n, int dtype, int kind, int num_bits,
                       int is_unsigned, int narrow_range, int saturate, float* amax_out,
                       void* workspace, int64_t spin_limit, void* stream);

@@ -426,9 +426,11 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* smem) {
 // (resident_grid_limit).  It is an ordinary launch: hipLaunchCooperativeKernel adds about 15 us
 // per call on this device, more than the second launch that the fusion saves.  Workgroups of
 // other kernels that occupy the device only delay the exchange, because they end without help
-// from this kernel; two of THESE kernels running side by side could each hold the compute units
-// the other one waits for, so callers run one fused call at a time per device, and the bounded
-// wait below turns a violation into an error instead of a hang.
+// from this kernel; two of THESE kernels running side by side (or a device on which part of the
+// compute units is masked off) could leave workgroups waiting for others that cannot start.  The
+// wait is therefore bounded, and a workgroup whose wait expires computes the abs-max of the whole
+// tensor by itself (workgroup_absmax_bits) and goes on: the outputs are the same bits either way,
+// only later.
 //
 // ws: MO_FUSED_WS_BYTES of device memory, all zero before the first use; one word per 128-byte
 // line, so that the atomics on different words do not queue behind each other:
@@ -436,17 +438,18 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* smem) {
 //   line 1  running maximum, an abs-max bit pattern (back to 0 likewise)
 //   line 2  64-bit {generation, result}: the last workgroup to arrive publishes the maximum
 //           together with a generation one higher than the one every workgroup read on entry
-//   line 3  set to 1 when a wait gave up; while it is set every later exchange fails at once
-//           (the count and the maximum of the abandoned exchange may still be in lines 0 and 1),
-//           until the host has cleared the workspace
+//   line 3  set to 1 when a wait expired (information for the host: the call took the slow way;
+//           no kernel reads it and the host clears it)
+// EVERY workgroup of a launch delivers its maximum and counts itself before it waits, also one
+// that gives up later, so the count reaches the grid size when the last workgroup of the launch
+// has started, that one cleans lines 0 and 1 and publishes, and the workspace is in order again
+// when the kernel ends -- whatever happened to the waits.
 // Only these words cross workgroups and every access to them is a device-scope atomic performed
 // at the memory side, so relaxed ordering is enough (a release / acquire pair would write back
 // and invalidate caches on this multi-die part); program order between two atomics of a thread
 // is kept by waiting for the value the first one returns.
-// The wait is bounded: after `spin_limit` polls (one about every half microsecond) a workgroup
-// sets the flag and returns false; the kernel then marks its share of the outputs (NaN) and
-// ends, so that no wavefront can stay behind for ever.  Calls that share a workspace must follow
-// each other in one stream.
+// After `spin_limit` polls (one about every half microsecond) a workgroup sets the flag and
+// returns false.  Calls that share a workspace must follow each other in one stream.
 constexpr int kWsCount = 0, kWsMax = 32, kWsPublished = 64, kWsFail = 96;  // word offsets
 
 __device__ __forceinline__ bool grid_max_exchange(uint32_t* ws, uint32_t local, uint32_t nwg,
@@ -454,25 +457,17 @@ __device__ __forceinline__ bool grid_max_exchange(uint32_t* ws, uint32_t local, 
                                                   uint32_t& global) {
     unsigned long long* published = (unsigned long long*)(ws + kWsPublished);
     unsigned long long entry = 0;
-    uint32_t poisoned = 0;
-    if (threadIdx.x == 0) {  // issued ahead of the reduction
-        entry = __hip_atomic_load(published, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // previous generation
-        poisoned = __hip_atomic_load(ws + kWsFail, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    if (threadIdx.x == 0)  // issued ahead of the reduction: the previous generation
+        entry = __hip_atomic_load(published, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const uint32_t m = block_max_u32(local, smem);
     if (threadIdx.x == 0) {
-        asm volatile("s_waitcnt vmcnt(0)" ::"v"(poisoned), "v"(entry) : "memory");
-        bool ok = poisoned == 0;
-        uint32_t g = 0, before = 0;
-        if (ok) {
-            uint32_t old = 0;
-            if (m) old = __hip_atomic_fetch_max(ws + kWsMax, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            asm volatile("s_waitcnt vmcnt(0)" ::"v"(old) : "memory");
-            before = __hip_atomic_fetch_add(ws + kWsCount, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        if (!ok) {
-            // an earlier exchange on this workspace was abandoned: nothing in it can be trusted
-        } else if (before + 1 == nwg) {
+        asm volatile("s_waitcnt vmcnt(0)" ::"v"(entry) : "memory");
+        bool ok = true;
+        uint32_t g = 0, old = 0;
+        if (m) old = __hip_atomic_fetch_max(ws + kWsMax, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::"v"(old) : "memory");
+        const uint32_t before = __hip_atomic_fetch_add(ws + kWsCount, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (before + 1 == nwg) {
             // last to arrive: every maximum has been applied.  Clean up, then publish.
             g = __hip_atomic_load(ws + kWsMax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::"v"(g) : "memory");
@@ -499,6 +494,44 @@ __device__ __forceinline__ bool grid_max_exchange(uint32_t* ws, uint32_t local, 
     __syncthreads();
     global = smem[4];
     return smem[5] != 0u;
+}
+
+// Abs-max of `nbytes / 16` 16-byte units at x (fp32 words when WORDS32, else pairs of 16-bit
+// floats), taken by ONE workgroup of 256 lanes that walks over all of them: the way out for a
+// workgroup of a fused kernel whose wait for the others expired.  Returns the masked maximum in
+// the packed form of the loads (fp32: the bit pattern; 16-bit: max of both halves in the low 16
+// bits), the same in every lane.  `extra`: a lane's share of what the units do not cover, in the
+// returned form.  `smem`: 8 words, free to reuse.
+template <bool WORDS32>
+__device__ __noinline__ uint32_t workgroup_absmax_bits(const void* x, int64_t units, uint32_t extra,
+                                                       uint32_t* smem) {
+    const uint4* p = (const uint4*)x;
+    uint32_t m = 0;
+    auto fold = [&](const uint4 v) {
+        if constexpr (WORDS32) {
+            const uint32_t a = v.x & 0x7FFFFFFFu, b = v.y & 0x7FFFFFFFu, c = v.z & 0x7FFFFFFFu,
+                           d = v.w & 0x7FFFFFFFu;
+            const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+            const uint32_t t = ab > cd ? ab : cd;
+            m = t > m ? t : m;
+        } else {
+            m = pk_max_u16(m, pk_max_u16(pk_max_u16(v.x & 0x7FFF7FFFu, v.y & 0x7FFF7FFFu),
+                                         pk_max_u16(v.z & 0x7FFF7FFFu, v.w & 0x7FFF7FFFu)));
+        }
+    };
+    int64_t u = threadIdx.x;
+    for (; u + 3 * 256 < units; u += 4 * 256) {
+        const uint4 v0 = p[u], v1 = p[u + 256], v2 = p[u + 512], v3 = p[u + 768];
+        fold(v0); fold(v1); fold(v2); fold(v3);
+    }
+    for (; u < units; u += 256) fold(p[u]);
+    if constexpr (!WORDS32) m = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
+    m = extra > m ? extra : m;
+    __syncthreads();  // smem is still being read by the caller's exchange
+    m = block_max_u32(m, smem);
+    if (threadIdx.x == 0) smem[6] = m;
+    __syncthreads();
+    return smem[6];
 }
 
 // How many workgroups of `kernel` (of `threads` lanes) the current device holds at the same time;

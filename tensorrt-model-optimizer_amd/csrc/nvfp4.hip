@@ -377,18 +377,10 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_fused_kernel(
     const uint32_t h = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
     uint32_t gbits;
     if (!grid_max_exchange(ws, h << 16, gridDim.x, spin_limit, smem, gbits)) {
-        // gave up waiting: NaN scale bytes for this workgroup's blocks (and a NaN global scale),
-        // so that a caller who does not look at the flag dequantises NaN instead of whatever
-        // the output memory held
-        for (int i = 0; i < TP; ++i) {
-            const int64_t t = (int64_t)i * gridDim.x + blockIdx.x;
-            if (t >= tiles) continue;
-            int64_t b1 = (t + 1) * kTileBlocks;
-            if (b1 > nblocks) b1 = nblocks;
-            for (int64_t b = t * kTileBlocks + threadIdx.x; b < b1; b += 256) wsf_out[b] = 0x7Fu;
-        }
-        if (blockIdx.x == 0 && threadIdx.x == 0 && wsf2_out) wsf2_out[0] = __builtin_nanf("");
-        return;
+        // the wait for the other workgroups expired: take the abs-max of the whole tensor here
+        // (16-element blocks of bf16 = two 16-byte units each)
+        keep_branch();
+        gbits = workgroup_absmax_bits<false>(x, nblocks * 2, 0u, smem) << 16;
     }
     const float amax = u2f(gbits);
     const float wsf2 = amax / 2688.0f;

@@ -239,18 +239,19 @@ __global__ __launch_bounds__(256) void fused_amax_qdq_kernel(
     bits = tb > bits ? tb : bits;
     uint32_t gbits;
     if (!grid_max_exchange(ws, bits, gridDim.x, spin_limit, smem, gbits)) {
-        // gave up waiting: fill this workgroup's share of the output with NaN, so that a caller
-        // who does not look at the flag sees a loud failure instead of uninitialised memory
-        float nan8[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) nan8[j] = __builtin_nanf("");
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int64_t c = ((int64_t)u * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
-            if (c < chunks) store_chunk<DT>(y, c << 3, nan8);
+        // the wait for the other workgroups expired: take the abs-max of the whole tensor here
+        // (x is not written by this launch: the host refuses overlapping x and y)
+        keep_branch();
+        constexpr int kPerUnit = DT == MO_F32 ? 4 : 8;
+        const int64_t units = n / kPerUnit;
+        uint32_t extra = 0;
+        if ((int64_t)threadIdx.x < n - units * kPerUnit) {
+            const int64_t i = units * kPerUnit + threadIdx.x;
+            extra = DT == MO_F32 ? (((const uint32_t*)x)[i] & 0x7FFFFFFFu)
+                                 : (uint32_t)(((const uint16_t*)x)[i] & 0x7FFFu);
         }
-        if (has_tail) store_elem<DT>(y, (chunks << 3) + threadIdx.x, __builtin_nanf(""));
-        return;
+        const uint32_t h = workgroup_absmax_bits<DT == MO_F32>(x, units, extra, smem);
+        gbits = DT == MO_F32 ? h : (DT == MO_BF16 ? h << 16 : f2u(f16_bits_to_f32(h)));
     }
     if (amax_out && blockIdx.x == 0 && threadIdx.x == 0) amax_out[0] = u2f(gbits);
     const typename Op::Scale s0 = op.make(u2f(gbits));
@@ -371,6 +372,12 @@ extern "C" int mo_fused_amax_qdq(const void* x, void* y, int64_t n, int dtype, i
     if (kind == 0 && (num_bits < 1 || num_bits > 24)) return MO_ERR_ARG;
     if (n == 0) return MO_OK;
     if (!x || !y || !workspace || ((uintptr_t)workspace & 127u)) return MO_ERR_ARG;
+    {
+        // a workgroup whose wait expires reads all of x again while others may be writing y
+        const int64_t bytes = n * (dtype == MO_F32 ? 4 : 2);
+        const uintptr_t x0 = (uintptr_t)x, y0 = (uintptr_t)y;
+        if (x0 < y0 + (uintptr_t)bytes && y0 < x0 + (uintptr_t)bytes) return MO_ERR_UNSUPPORTED;
+    }
     hipStream_t s = (hipStream_t)stream;
     uint32_t* ws = (uint32_t*)workspace;
     const uint32_t spins = spin_limit > 0xFFFFFFFFll ? 0xFFFFFFFFu : (uint32_t)spin_limit;

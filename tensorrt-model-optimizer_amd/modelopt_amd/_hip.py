@@ -368,14 +368,18 @@ def nvfp4_quantize(x, amax_f32, block_size=16, amax_is_wsf2=False, wsf_in=None, 
 
 # --------------------------------------------------------------- one-launch amax -> quantize
 FUSED_WS_BYTES, FUSED_WS_FAIL_OFFSET = 512, 384   # MO_FUSED_WS_BYTES, MO_FUSED_WS_FAIL_OFFSET
-FUSED_SPIN_LIMIT = 1 << 22   # polls a workgroup waits for the others before it gives up
+# polls (about a microsecond each with the round trip of the load) a workgroup waits for the
+# others before it takes the abs-max of the whole tensor by itself: some 20 ms
+FUSED_SPIN_LIMIT = 1 << 14
 _fused_ws_by_device = {}
 
 
 def fused_scratch(device, stream=None):
     """The workspace of the fused kernels for ``device`` and ``stream`` (default: torch's current
     stream there).  Calls in one stream follow each other and can share it; calls in different
-    streams may overlap and get one each."""
+    streams may overlap and get one each (overlapping calls can keep each other's workgroups off
+    the device: each then ends its wait after ``FUSED_SPIN_LIMIT`` polls and finishes on its own,
+    with the same results)."""
     index = torch.device(device).index
     index = torch.cuda.current_device() if index is None else index
     if stream is None:
@@ -394,16 +398,19 @@ def fused_scratch(device, stream=None):
 
 
 def fused_gave_up(device=None) -> bool:
-    """Whether a fused kernel (on ``device``; default: any device) ended without writing its
-    outputs because a workgroup gave up waiting for the others.  Synchronises; clears the state.
-    Calls recorded into a graph use workspaces of their own that this check does not see."""
+    """Whether a workgroup of a fused kernel (on ``device``; default: any device) stopped waiting
+    for the others and took the abs-max of the whole tensor by itself since the last look.  The
+    outputs of such a call are right, but it was slow (the wait plus a pass over the tensor per
+    workgroup): a caller that sees this repeatedly should stay with the two-launch path.
+    Synchronises; clears the flag.  Calls recorded into a graph use workspaces of their own that
+    this check does not see."""
     index = None if device is None else torch.device(device).index
     failed = False
     for (dev, _), ws in _fused_ws_by_device.items():
         if index is not None and dev != index:
             continue
         if bool(ws[FUSED_WS_FAIL_OFFSET // 4].item()):
-            ws.zero_()
+            ws[FUSED_WS_FAIL_OFFSET // 4] = 0
             failed = True
     return failed
 
@@ -443,7 +450,8 @@ def nvfp4_quantize_fused(x, flags=0, spin_limit=FUSED_SPIN_LIMIT):
 def fused_amax_qdq(x, kind, num_bits=8, unsigned=False, narrow_range=False, saturate=False,
                    out=None, spin_limit=FUSED_SPIN_LIMIT):
     """Dynamic per-tensor fake quantisation in one launch (``kind`` "int" or "fp8"): returns
-    (y, amax fp32 scalar), or None when the tensor does not fit / the layout is not covered."""
+    (y, amax fp32 scalar), or None when the tensor does not fit / the layout is not covered
+    (``out`` overlapping ``x`` is not: a workgroup whose wait expired reads ``x`` again)."""
     _require_device(x)
     if not x.is_contiguous() or x.dtype not in _DTYPES or x.data_ptr() % 16 or x.numel() == 0:
         return None

@@ -17,6 +17,7 @@ from torch import nn
 
 from ... import _hip
 from ..quantization.nn import SequentialQuantizer, TensorQuantizer
+from ..quantization import modes
 from ..quantization.overflow import nvfp4_quantize_flags
 from ..quantization.qtensor import NVFP4QTensor, QTensorWrapper
 from ..quantization.utils import is_quantized_linear, true_divide
@@ -195,9 +196,10 @@ def _export_hf_checkpoint(model: nn.Module, dtype: torch.dtype | None = None):
         if id(m) not in done:
             _export_quantized_weight(m, dtype)
     state = postprocess_state_dict(model.state_dict(), kv_bound, kv_format)
-    if _hip.fused_gave_up():
-        raise RuntimeError("a one-launch quantize kernel ended without writing its outputs (its "
-                           "workgroups could not all run at once); export again")
+    if modes.one_launch_dynamic_quant() and _hip.fused_gave_up():
+        warnings.warn("a one-launch quantize kernel could not run all its workgroups at once and "
+                      "finished the slow way (same results); something else holds the device -- "
+                      "consider set_one_launch_dynamic_quant(False)")
     return state, quant_config
 
 

@@ -5,12 +5,14 @@ calib/max.py:26-94).  ``collect`` is one kernel launch that folds |x| into a per
 accumulator with integer atomic max -- no temporaries and no host synchronisation.  The three
 sanity checks the reference runs (and blocks on) at every ``collect`` -- non-negative, no inf, no
 NaN -- are evaluated once, in ``compute_amax``; NaN and inf survive the running max, so nothing
-is lost by deferring them.
+is lost by deferring them.  ``modes.set_strict_checks(True)`` brings the reference's timing back:
+every ``collect`` then reduces the batch on its own, asserts on it (one host synchronisation) and
+only then folds it in.
 """
 
 import torch
 
-from .. import kernels
+from .. import kernels, modes
 from ..utils import convert_quantization_axis_to_reduce_axis
 
 __all__ = ["MaxCalibrator"]
@@ -132,7 +134,9 @@ class MaxCalibrator(_Calibrator):
             self._shape, self._dtype = shape, x.dtype
         elif shape != self._shape:
             raise RuntimeError("amax shape changed!")
-        if not self._track_amax:
+        if modes.strict_checks():
+            self._collect_checked(x, layout)
+        elif not self._track_amax:
             if not (SHARE_REDUCTIONS[0] and layout[1] == 1 and x.is_cuda and x.is_contiguous()
                     and not isinstance(x, torch.nn.Parameter)) or not self._collect_shared(x):
                 kernels.absmax_accumulate(x, self._acc, layout)
@@ -142,6 +146,24 @@ class MaxCalibrator(_Calibrator):
             self._acc = torch.maximum(self._acc, local)
             self._amaxs.append(local.reshape(shape).to(x.dtype).float().cpu().numpy())
         self._validated = False
+
+    def _collect_checked(self, x, layout):
+        """``collect`` as the reference runs it (calib/max.py:62-86): the abs-max of this batch
+        alone, the three assertions on it -- one host synchronisation -- and only then the
+        running maximum, so that a bad batch is reported when it is shown and leaves the
+        calibrator as it was."""
+        local = torch.zeros_like(self._acc)
+        kernels.absmax_accumulate(x, local, layout)
+        bad = torch.stack([(local < 0).any(), torch.isinf(local).any(),
+                           torch.isnan(local).any()]).tolist()
+        assert not bad[0], "detected negative values after abs, could be torch or cuda bug"
+        assert not bad[1], ("detected inf values in amax. inf in original tensor: "
+                            f"{torch.any(torch.isinf(x))}")
+        assert not bad[2], ("detected nan values in amax. nan in original tensor: "
+                            f"{torch.any(torch.isnan(x))}")
+        self._acc = torch.maximum(self._acc, local)
+        if self._track_amax:
+            self._amaxs.append(local.reshape(self._shape).to(x.dtype).float().cpu().numpy())
 
     def _collect_shared(self, x) -> bool:
         """Per-tensor reduction inside a calibration pass: note the tile maxima of the previous

@@ -15,7 +15,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
-from ... import calib, kernels
+from ... import calib, kernels, modes
 from ... import utils as quant_utils
 from ...config import QuantizerAttributeConfig
 from ...qtensor import (BaseQuantizedTensor, FP8QTensor, INT4QTensor, INT8QTensor, MXFP4QTensor,
@@ -391,7 +391,10 @@ class TensorQuantizer(nn.Module):
     def _fused_dynamic_per_tensor(self, inputs):
         """Dynamic per-tensor INT / FP8 fake quantisation (no calibrated ``_amax``, no axis, no
         blocks) outside autograd: abs-max and quantize-dequantize in one launch that reads the
-        tensor once.  None when that case does not apply or the tensor is too large for it."""
+        tensor once, when ``modes.set_one_launch_dynamic_quant(True)`` allows it.  None when that
+        case does not apply or the tensor is too large for it."""
+        if not modes.one_launch_dynamic_quant() or modes.strict_checks():
+            return None
         if hasattr(self, "_amax") or self._axis is not None or self.block_sizes is not None:
             return None
         if not inputs.is_cuda or (inputs.requires_grad and torch.is_grad_enabled()):

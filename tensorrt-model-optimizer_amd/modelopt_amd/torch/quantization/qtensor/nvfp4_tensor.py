@@ -8,6 +8,7 @@ E2M1 ordinal); per-block scales ``float8_e4m3fn`` [..., K/block]; one fp32 globa
 import torch
 
 from .... import _hip
+from .. import modes
 from ..overflow import nvfp4_quantize_flags
 from ..utils import reduce_amax, reduce_block_amax, reduce_block_padding, true_divide
 from .base_qtensor import BaseQuantizedTensor
@@ -84,9 +85,10 @@ class NVFP4QTensor(BaseQuantizedTensor):
             return torch.div(blocks, scale.unsqueeze(-1)).reshape(xp.shape)
         shape, dtype = input.shape, input.dtype
         x = input.contiguous()
-        if weights_scaling_factor_2 is None and weights_scaling_factor is None and block_size == 16:
+        if (weights_scaling_factor_2 is None and weights_scaling_factor is None and block_size == 16
+                and modes.one_launch_dynamic_quant()):
             # abs-max, scales and codes in one launch that reads the tensor once (tensors that fit
-            # the chip's registers; larger ones take the two launches below)
+            # the chip's registers; larger ones take the two launches below); opt-in
             fused = _hip.nvfp4_quantize_fused(x, flags=nvfp4_quantize_flags())
             if fused is not None:
                 packed, wsf, wsf2, _ = fused

@@ -11,7 +11,7 @@ import torch
 from torch.autograd import Function
 
 from ... import _hip
-from . import kernels
+from . import kernels, modes
 from .config import QuantizerAttributeConfig
 from .overflow import fp8_saturates, get_fp8_overflow_behavior, set_fp8_overflow_behavior  # noqa: F401
 
@@ -45,7 +45,18 @@ def fp8_eager(inputs: torch.Tensor, amax: torch.Tensor | None = None) -> torch.T
 
 
 def fake_quant_impl(inputs, amax, num_bits=8, unsigned=False, narrow_range=True):
-    """Integer fake quantisation; ``amax`` per tensor or with one non-unit run of dims."""
+    """Integer fake quantisation; ``amax`` per tensor or with one non-unit run of dims.
+
+    The reference's CPU path first looks at the data on the host (tensor_quant.py:577-587):
+    negative inputs with ``unsigned=True`` raise ``TypeError``, a negative amax raises
+    ``ValueError``.  Its CUDA kernel clamps instead, and so does this function unless
+    ``modes.set_strict_checks(True)`` asks for the CPU path's errors (two host synchronisations
+    per call)."""
+    if modes.strict_checks():
+        if unsigned and inputs.numel() and inputs.min() < 0.0:
+            raise TypeError("Negative values encountered in unsigned quantization.")
+        if amax.numel() and amax.min() < 0:
+            raise ValueError("Negative values in amax")
     return kernels.fake_quant_int(inputs, amax, num_bits, unsigned, narrow_range)
 
 

@@ -47,8 +47,6 @@ def _fused_losses(x, w, s, ref, block, bits, unsigned, narrow):
 @pytest.mark.parametrize("block,bits,unsigned,narrow", [(128, 4, False, False), (64, 4, False, True),
                                                          (32, 8, False, False)])
 def test_matches_unfused_device_path(tokens, n, k, block, bits, unsigned, narrow):
-    if n * k > 1 << 22 and block != 128:
-        pytest.skip("the large case runs once")
     x, w, s = (t.to(DEV) for t in _problem(tokens, n, k, 5, tokens + n))
     ref = F.linear(x, w).contiguous()
     got = _fused_losses(x, w, s, ref, block, bits, unsigned, narrow)
@@ -103,6 +101,31 @@ def test_matches_cpu_restatement_of_the_search_loop():
     want = torch.stack(want)
     got = _fused_losses(x.to(DEV), w.to(DEV), s.to(DEV), ref.to(DEV).contiguous(), 128, 4, False, False)
     assert torch.allclose(got.cpu(), want, rtol=1e-3), (got, want)
+
+
+def _cpu_search_losses(x, w, s, block):
+    """The reference's per-alpha loop body (model_calib.py:645-690 with the weight quantizer of
+    INT4_AWQ_CFG, tensor_quant.py:574-612) on the CPU: sum of f32(bf16(out - ref))^2."""
+    ref = F.linear(x, w)
+    want = []
+    for i in range(s.shape[0]):
+        xs = x * (1 / s[i].float()).to(torch.bfloat16)
+        out = F.linear(xs, oawq.int4_block_qdq(w * s[i], block))
+        want.append((out - ref).float().pow(2).sum().double())
+    return ref, torch.stack(want)
+
+
+@pytest.mark.parametrize("tokens,n,k,n_alpha", [(512, 14336, 4096, 5), (512, 4096, 14336, 5),
+                                                (200, 4096, 4096, 3)])
+def test_llama_8b_layer_shapes_against_the_cpu_restatement(tokens, n, k, n_alpha):
+    """gate / up (14336 x 4096) and down (4096 x 14336) of the 8B shape -- the layers the sweep
+    spends its time on, 112 and 32 column tiles per alpha over 32 and 112 k blocks -- scored by
+    the one-launch kernel and by the CPU restatement: every loss within 1e-3, same best alpha."""
+    x, w, s = _problem(tokens, n, k, n_alpha, n + k)
+    ref, want = _cpu_search_losses(x, w, s, 128)
+    got = _fused_losses(x.to(DEV), w.to(DEV), s.to(DEV), ref.to(DEV).contiguous(), 128, 4, False, False)
+    assert torch.allclose(got.cpu(), want, rtol=1e-3, atol=0), (got, want)
+    assert int(got.argmin()) == int(want.argmin())
 
 
 @pytest.mark.parametrize("tokens,k,n_alpha", [(512, 4096, 21), (100, 256, 3), (1, 8, 1), (65, 1032, 2)])

@@ -77,10 +77,16 @@ def test_static_fp8_and_int8_fake_quant(dtype):
 def test_dynamic_per_tensor_fake_quant_in_one_launch(num_bits):
     """The one-launch abs-max + quantize path waits across workgroups on a workspace; a recorded
     call brings a workspace of its own, zeroed by a node of the graph."""
+    import modelopt_amd.torch.quantization as mtq
+
     q = _quantizer(num_bits=num_bits, axis=None)
-    with torch.no_grad():
-        assert q._fused_dynamic_per_tensor(torch.ones(8, 64, device=DEV, dtype=torch.bfloat16)) is not None
-        _replay_against_eager(q, (512, 2048), torch.bfloat16, seed=1)
+    previous = mtq.set_one_launch_dynamic_quant(True)
+    try:
+        with torch.no_grad():
+            assert q._fused_dynamic_per_tensor(torch.ones(8, 64, device=DEV, dtype=torch.bfloat16)) is not None
+            _replay_against_eager(q, (512, 2048), torch.bfloat16, seed=1)
+    finally:
+        mtq.set_one_launch_dynamic_quant(previous)
     assert not _hip.fused_gave_up(DEV)
 
 

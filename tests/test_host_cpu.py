@@ -619,3 +619,91 @@ def test_deferred_scale_checks_make_one_check_at_the_end():
         with deferred_scale_checks():
             assert all_valid_scales([torch.tensor([1.0, float("nan")])])   # recorded, reported later
     assert not all_valid_scales([torch.tensor([-1.0])])                  # outside a block: checked at once
+
+
+# ----------------------------------------------------------------------------- strict host checks
+@pytest.fixture
+def strict_checks():
+    previous = mtq.set_strict_checks(True)
+    yield
+    mtq.set_strict_checks(previous)
+
+
+@pytest.fixture
+def lenient_int_kernel(oracle_backend, monkeypatch):
+    """An integer kernel stand-in that, like the HIP kernel, never looks at the data on the host
+    (the oracle follows the reference's CPU path and raises by itself): whatever raises in these
+    tests is the product's host layer."""
+    monkeypatch.setattr(kernels, "fake_quant_int", lambda x, amax, *args: x.clone())
+
+
+def test_strict_checks_unsigned_quantization_of_negative_values_raises(oracle_backend, strict_checks, monkeypatch):
+    """tests/_test_utils/torch/quantization/tensor_quant_common.py:86-101 (``test_unsigned``): the
+    accepted case quantises like a signed grid of one more bit, the negative case raises the
+    reference's ``TypeError`` (tensor_quant.py:577-578)."""
+    from modelopt_amd.torch.quantization.tensor_quant import fake_tensor_quant
+
+    torch.manual_seed(0)
+    x = torch.randn(31).abs()
+    got = fake_tensor_quant(x, torch.max(x.abs()), None, 8, True)
+    assert torch.equal(got, fake_quant.tensor_quant(x, torch.max(x.abs()), 9, False, True))
+    monkeypatch.setattr(kernels, "fake_quant_int", lambda x, amax, *args: x.clone())
+    x = torch.randn(3, 7)
+    with pytest.raises(TypeError, match="Negative values encountered"):
+        fake_tensor_quant(x, torch.max(torch.abs(x)), None, 8, True)
+    with pytest.raises(TypeError, match="Negative values encountered"):
+        TensorQuantizer(QuantizerAttributeConfig(num_bits=8, unsigned=True))(x)
+
+
+def test_strict_checks_negative_amax_raises(lenient_int_kernel, strict_checks):
+    """tensor_quant.py:585-587 of the reference: ``ValueError("Negative values in amax")``, also
+    when only one channel's amax is negative."""
+    from modelopt_amd.torch.quantization.tensor_quant import fake_tensor_quant
+
+    x = torch.randn(4, 8)
+    with pytest.raises(ValueError, match="Negative values in amax"):
+        fake_tensor_quant(x, torch.tensor(-1.0))
+    amax = torch.tensor([[1.0], [2.0], [-0.5], [1.0]])
+    with pytest.raises(ValueError, match="Negative values in amax"):
+        fake_tensor_quant(x, amax)
+    assert fake_tensor_quant(x, amax.abs()).shape == x.shape
+
+
+def test_strict_checks_are_off_by_default(lenient_int_kernel):
+    from modelopt_amd.torch.quantization.tensor_quant import fake_tensor_quant
+
+    assert not mtq.strict_checks()
+    x = torch.randn(3, 7)
+    fake_tensor_quant(x, torch.max(torch.abs(x)), None, 8, True)   # no host look at the data
+
+
+def test_strict_checks_max_calibrator_asserts_at_the_batch_that_is_bad(oracle_backend, strict_checks):
+    """calib/max.py:69-77 of the reference: the assertions fire inside ``collect`` on the batch
+    that holds the inf / NaN, and that batch is not folded into the running maximum."""
+    from modelopt_amd.torch.quantization.calib import MaxCalibrator
+
+    cal = MaxCalibrator(8, None, False)
+    cal.collect(torch.tensor([1.0, -3.0, 2.0]))
+    bad = torch.tensor([1.0, float("inf")])
+    with pytest.raises(AssertionError, match="detected inf values in amax. inf in original tensor: True"):
+        cal.collect(bad)
+    with pytest.raises(AssertionError, match="detected nan values in amax. nan in original tensor: True"):
+        cal.collect(torch.tensor([float("nan"), 5.0]))
+    cal.collect(torch.tensor([0.5]))
+    assert float(cal.compute_amax()) == 3.0
+    # per channel, and the history of tracked maxima
+    cal = MaxCalibrator(8, 0, False, track_amax=True)
+    cal.collect(torch.tensor([[1.0, -2.0], [0.5, 0.25]]))
+    with pytest.raises(AssertionError, match="detected nan"):
+        cal.collect(torch.tensor([[1.0, float("nan")], [0.5, 0.25]]))
+    assert torch.equal(cal.compute_amax().flatten(), torch.tensor([2.0, 0.5])) and len(cal.amaxs) == 1
+
+
+def test_default_max_calibrator_reports_a_bad_batch_in_compute_amax(oracle_backend):
+    from modelopt_amd.torch.quantization.calib import MaxCalibrator
+
+    cal = MaxCalibrator(8, None, False)
+    cal.collect(torch.tensor([1.0, float("inf")]))     # no assertion here: no host synchronisation
+    cal.collect(torch.tensor([2.0]))
+    with pytest.raises(AssertionError, match="detected inf values in amax"):
+        cal.compute_amax()

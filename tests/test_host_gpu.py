@@ -606,3 +606,37 @@ def test_shared_reductions_fold_after_many_batches_and_keep_nan():
         follow.collect(x)
     with pytest.raises(AssertionError, match="nan"):
         follow.compute_amax()
+
+
+# ----------------------------------------------------------------------------- strict host checks
+def test_strict_checks_on_the_device():
+    """``mtq.set_strict_checks(True)``: the reference's CPU-path errors (tensor_quant.py:577-587,
+    calib/max.py:69-77) for device tensors, at the reference's moment; without it the kernels
+    clamp like the reference's CUDA kernel and the calibrator reports in ``compute_amax``."""
+    from modelopt_amd.torch.quantization.tensor_quant import fake_tensor_quant
+
+    x = _rand((3, 7), torch.float32, seed=1).to(DEV)
+    amax = x.abs().max()
+    clamped = fake_tensor_quant(x, amax, None, 8, True)          # default: negatives clamp to 0
+    assert float(clamped.min()) == 0.0
+    previous = mtq.set_strict_checks(True)
+    try:
+        with pytest.raises(TypeError, match="Negative values encountered"):
+            fake_tensor_quant(x, amax, None, 8, True)
+        with pytest.raises(ValueError, match="Negative values in amax"):
+            fake_tensor_quant(x, -amax)
+        assert_bits_equal(fake_tensor_quant(x.abs(), amax, None, 8, True).cpu(),
+                          fake_quant.tensor_quant(x.abs().cpu(), amax.cpu(), 8, True, True), "accepted case")
+        c = calib.MaxCalibrator(8, None, False)
+        c.collect(_rand((64, 64), seed=2).to(DEV))
+        good = c.compute_amax().clone()
+        bad = _rand((64, 64), seed=3)
+        bad[5, 5] = float("nan")
+        with pytest.raises(AssertionError, match="detected nan values in amax. nan in original tensor: True"):
+            c.collect(bad.to(DEV))
+        assert_bits_equal(c.compute_amax().cpu(), good.cpu(), "the bad batch was not folded in")
+        q = TensorQuantizer(QuantizerAttributeConfig(num_bits=8, unsigned=True)).to(DEV)
+        with pytest.raises(TypeError, match="Negative values encountered"):
+            q(x)
+    finally:
+        mtq.set_strict_checks(previous)
