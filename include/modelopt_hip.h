@@ -62,6 +62,14 @@ enum mo_quantize_flags { MO_FLAG_FORCE_EXACT = 1, MO_FLAG_SATURATE_BLOCK_SCALE =
 int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
               float* acc, void* stream);
 
+/* Two per-tensor mo_absmax calls (x0 of n0 elements into acc0, x1 of n1 into acc1, one dtype) in
+ * one launch: the key and the value states of an attention layer reach their quantizers
+ * together (k_bmm_quantizer / v_bmm_quantizer, TQ/plugins/huggingface.py:52-69, each a
+ * MaxCalibrator.collect, TQ/calib/max.py:53-94) and are a few megabytes each, so a launch per
+ * tensor is mostly launch latency.  x0 and x1 16-byte aligned (MO_ERR_UNSUPPORTED otherwise). */
+int mo_absmax_pair(const void* x0, int64_t n0, float* acc0, const void* x1, int64_t n1,
+                   float* acc1, int dtype, void* stream);
+
 /* Per-tensor mo_absmax (outer = axis = 1, inner = n) that also leaves the abs-max of every
  * 32768-element tile of x in parts[0 .. *parts_written): the maximum of those words is the
  * abs-max of this tensor alone, whatever acc held before.  For calibration loops that show one

@@ -74,14 +74,13 @@ __device__ __forceinline__ void fold_max_coherent(uint32_t* acc, uint32_t v) {
 // ------------------------------------------------------------------------------ per tensor
 // One workgroup per tile of TILE_ELEMS elements, dispatched in order.
 template <int DT, int TILE_ELEMS>
-__global__ __launch_bounds__(256) void absmax_flat_kernel(const void* __restrict__ x, int64_t n,
-                                                          uint32_t* __restrict__ acc,
-                                                          uint32_t* __restrict__ parts = nullptr) {
-    __shared__ uint32_t smem[4];
+__device__ __forceinline__ void absmax_flat_tile(const void* __restrict__ x, int64_t n, int64_t tile,
+                                                 uint32_t* __restrict__ acc,
+                                                 uint32_t* __restrict__ parts, uint32_t* smem) {
     constexpr int64_t kTileChunks = TILE_ELEMS / 8;
     AbsAcc<DT> a;
     const int64_t chunks = n >> 3;
-    const int64_t c0 = (int64_t)blockIdx.x * kTileChunks;
+    const int64_t c0 = tile * kTileChunks;
     int64_t c1 = c0 + kTileChunks;
     if (c1 > chunks) c1 = chunks;
     int64_t c = c0 + threadIdx.x;
@@ -96,8 +95,28 @@ __global__ __launch_bounds__(256) void absmax_flat_kernel(const void* __restrict
     const uint32_t v = block_max_u32(a.bits(), smem);
     if (threadIdx.x == 0) {
         fold_max(acc, v);
-        if (parts) parts[blockIdx.x] = v;   // the tile's own maximum, for callers that share a reduction
+        if (parts) parts[tile] = v;   // the tile's own maximum, for callers that share a reduction
     }
+}
+
+template <int DT, int TILE_ELEMS>
+__global__ __launch_bounds__(256) void absmax_flat_kernel(const void* __restrict__ x, int64_t n,
+                                                          uint32_t* __restrict__ acc,
+                                                          uint32_t* __restrict__ parts = nullptr) {
+    __shared__ uint32_t smem[4];
+    absmax_flat_tile<DT, TILE_ELEMS>(x, n, blockIdx.x, acc, parts, smem);
+}
+
+// Two tensors, each into its own accumulator, in one launch: workgroups [0, tiles0) take the
+// tiles of the first, the others those of the second.
+template <int DT, int TILE_ELEMS>
+__global__ __launch_bounds__(256) void absmax_pair_kernel(const void* __restrict__ x0, int64_t n0,
+                                                          uint32_t* __restrict__ acc0,
+                                                          const void* __restrict__ x1, int64_t n1,
+                                                          uint32_t* __restrict__ acc1, int tiles0) {
+    __shared__ uint32_t smem[4];
+    if ((int)blockIdx.x < tiles0) absmax_flat_tile<DT, TILE_ELEMS>(x0, n0, blockIdx.x, acc0, nullptr, smem);
+    else absmax_flat_tile<DT, TILE_ELEMS>(x1, n1, (int)blockIdx.x - tiles0, acc1, nullptr, smem);
 }
 
 // ------------------------------------------------------------------------------ rows
@@ -582,6 +601,28 @@ extern "C" int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
         default: return MO_ERR_DTYPE;
     }
     if (rc != MO_OK) return rc;
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_absmax_pair(const void* x0, int64_t n0, float* acc0, const void* x1, int64_t n1,
+                              float* acc1, int dtype, void* stream) {
+    if (n0 < 0 || n1 < 0) return MO_ERR_ARG;
+    if (dtype < MO_F32 || dtype > MO_BF16) return MO_ERR_DTYPE;
+    if ((n0 && (!x0 || !acc0)) || (n1 && (!x1 || !acc1))) return MO_ERR_ARG;
+    if (n0 == 0 && n1 == 0) return MO_OK;
+    if ((((uintptr_t)x0 | (uintptr_t)x1) & 15u)) return MO_ERR_UNSUPPORTED;
+    // 8192-element tiles: the pair is for small tensors (K and V of one batch), which a larger
+    // tile would spread over too few compute units
+    constexpr int64_t kTile = 8192;
+    const int64_t t0 = (n0 + kTile - 1) / kTile, t1 = (n1 + kTile - 1) / kTile;
+    if (t0 + t1 > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((unsigned)(t0 + t1));
+    switch (dtype) {
+        case MO_F32: mo::absmax_pair_kernel<MO_F32, kTile><<<grid, 256, 0, s>>>(x0, n0, (uint32_t*)acc0, x1, n1, (uint32_t*)acc1, (int)t0); break;
+        case MO_F16: mo::absmax_pair_kernel<MO_F16, kTile><<<grid, 256, 0, s>>>(x0, n0, (uint32_t*)acc0, x1, n1, (uint32_t*)acc1, (int)t0); break;
+        default: mo::absmax_pair_kernel<MO_BF16, kTile><<<grid, 256, 0, s>>>(x0, n0, (uint32_t*)acc0, x1, n1, (uint32_t*)acc1, (int)t0); break;
+    }
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }
 

@@ -28,6 +28,8 @@
 // survives the rounding to bf16 for about one weight in 10^4, far below the 1e-3 tolerance of
 // the per-alpha losses.  The weights that are kept after the search come from the
 // exact kernels.
+#include <atomic>
+#include <mutex>
 #include <type_traits>
 
 #include "awq_ops.h"
@@ -327,7 +329,7 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
 // make the launch end soonest: tiles are handed to the compute units of an XCD in launch order
 // as units fall free, a tile costs its width plus a fixed part (prologue and epilogue, about 10
 // columns' worth), and the launch ends when the slowest XCD does.
-static inline int narrow_tiles_per_alpha(int64_t n_alpha, int64_t n, int units_per_xcd) {
+static inline int narrow_tiles_per_alpha_uncached(int64_t n_alpha, int64_t n, int units_per_xcd) {
     int best = 0;
     double best_end = 0.0;
     double free_at[64];
@@ -354,6 +356,28 @@ static inline int narrow_tiles_per_alpha(int64_t n_alpha, int64_t n, int units_p
         if (narrow >= 64) break;
     }
     return best;
+}
+
+// The answer for the last few (alphas, features, units) asked about: a search step of every layer
+// of a model asks the same handful of questions, and the simulation costs as much host time as
+// the kernel it plans takes on the device.
+static inline int narrow_tiles_per_alpha(int64_t n_alpha, int64_t n, int units_per_xcd) {
+    struct Entry { int64_t n_alpha, n; int units, narrow; };
+    static std::mutex lock;
+    static Entry memo[16];
+    static int used = 0, next = 0;
+    {
+        std::lock_guard<std::mutex> hold(lock);
+        for (int i = 0; i < used; ++i)
+            if (memo[i].n_alpha == n_alpha && memo[i].n == n && memo[i].units == units_per_xcd)
+                return memo[i].narrow;
+    }
+    const int narrow = narrow_tiles_per_alpha_uncached(n_alpha, n, units_per_xcd);
+    std::lock_guard<std::mutex> hold(lock);
+    memo[next] = Entry{n_alpha, n, units_per_xcd, narrow};
+    next = (next + 1) % 16;
+    if (used < 16) ++used;
+    return narrow;
 }
 
 // xs[a][c][t][0..8) = bf16(x[t][8 c ..] * inv_s[a][8 c ..]) for every alpha: the activations the
@@ -414,13 +438,17 @@ extern "C" int mo_awq_search_losses(const void* xs, const void* w, const void* s
     if (is_unsigned) return MO_ERR_UNSUPPORTED;
     (void)narrow_range;
     hipStream_t st = (hipStream_t)stream;
-    static int units_per_xcd = 0;   // compute units that share an L2 (one workgroup each)
+    // compute units that share an L2 (one workgroup each), per device
+    static std::atomic<int> units_of_device[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MO_ERR_LAUNCH;
+    int units_per_xcd = units_of_device[dev].load(std::memory_order_relaxed);
     if (units_per_xcd == 0) {
-        int dev = 0, cus = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < mo::kXcds)
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < mo::kXcds)
             cus = 256;
         units_per_xcd = cus / mo::kXcds;
+        units_of_device[dev].store(units_per_xcd, std::memory_order_relaxed);
     }
     int narrow = (int)mo::tuned("search_narrow_tiles", -1);
     if (narrow < 0) narrow = mo::narrow_tiles_per_alpha(n_alpha, n, units_per_xcd);

@@ -27,6 +27,7 @@ SIGNATURES = {
     "mo_version": [],
     "mo_error_string": [_INT],
     "mo_absmax": [_P, _I64, _I64, _I64, _INT, _P, _P],
+    "mo_absmax_pair": [_P, _I64, _P, _P, _I64, _P, _INT, _P],
     "mo_absmax_tensor_parts": [_P, _I64, _INT, _P, _P, _I64, _P, _P],
     "mo_absmax_cols_staged": [_P, _I64, _I64, _INT, _P, _P, _I64, _P],
     "mo_absmax_cols_noalloc": [_P, _I64, _I64, _INT, _P, _P],
@@ -119,6 +120,10 @@ def _staging_words(anchor: torch.Tensor, words: int) -> torch.Tensor:
     reused by later calls: calls in one stream follow each other, so they can share it, and the
     calibration loop allocates nothing per call."""
     index = anchor.device.index
+    if torch.cuda.is_current_stream_capturing():
+        # memory from a graph's private pool belongs to that graph: a buffer made here is not kept
+        # (eager calls and other graphs on this stream would share it with the replays)
+        return torch.empty(words, dtype=torch.int32, device=anchor.device)
     key = (index, torch._C._cuda_getCurrentRawStream(index))
     buf = _staging.get(key)
     if buf is None or buf.numel() < words:
@@ -203,6 +208,20 @@ def absmax_into(x: torch.Tensor, acc: torch.Tensor, outer: int, axis: int, inner
         return acc
     call("mo_absmax", x, _ptr(x), outer, axis, inner, dtype_code(x.dtype), _ptr(acc), _stream(x))
     return acc
+
+
+def absmax_pair_into(x0: torch.Tensor, acc0: torch.Tensor, x1: torch.Tensor, acc1: torch.Tensor):
+    """Per-tensor ``absmax_into`` of two dense tensors of one dtype (each into its own one-element
+    accumulator) in one launch.  False, with nothing launched, when the pair is not covered."""
+    _require_device(x0, acc0, x1, acc1)
+    if (x0.dtype != x1.dtype or x0.dtype not in _DTYPES or x0.device != x1.device
+            or x0.data_ptr() % 16 or x1.data_ptr() % 16 or acc0.numel() != 1 or acc1.numel() != 1):
+        return False
+    assert x0.is_contiguous() and x1.is_contiguous()
+    assert acc0.dtype == torch.float32 and acc1.dtype == torch.float32
+    call("mo_absmax_pair", x0, _ptr(x0), x0.numel(), _ptr(acc0), _ptr(x1), x1.numel(), _ptr(acc1),
+         dtype_code(x0.dtype), _stream(x0))
+    return True
 
 
 _parts_ring = {}   # device index -> [int32 buffer, words handed out]

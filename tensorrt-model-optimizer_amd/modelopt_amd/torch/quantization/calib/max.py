@@ -47,6 +47,32 @@ def _sharing_key(x):
             torch._C._cuda_getCurrentRawStream(x.device.index))
 
 
+def collect_pair(cal0, x0, cal1, x1) -> bool:
+    """``cal0.collect(x0); cal1.collect(x1)`` for two plain per-tensor ``MaxCalibrator``s in one
+    kernel launch (the key and value states of an attention layer).  False, with nothing
+    collected, when the pair is not covered; the caller then collects one by one."""
+    if modes.strict_checks():
+        return False
+    flats = []
+    for cal, x in ((cal0, x0), (cal1, x1)):
+        if (type(cal) is not MaxCalibrator or cal._track_amax or cal._axis is not None
+                or not x.is_cuda or x.numel() == 0 or (cal._acc is not None and cal._shape != torch.Size(()))):
+            return False
+        flat = x if x.is_contiguous() else kernels.dense_flat_view(x)   # order does not matter
+        if flat is None:
+            return False
+        flats.append(flat)
+    for cal, x in ((cal0, x0), (cal1, x1)):
+        if cal._acc is None:
+            cal._acc = torch.zeros(1, dtype=torch.float32, device=x.device)
+            cal._shape, cal._dtype = torch.Size(()), x.dtype
+    with torch.no_grad():
+        if not kernels._hip.absmax_pair_into(flats[0], cal0._acc, flats[1], cal1._acc):
+            return False
+    cal0._validated = cal1._validated = False
+    return True
+
+
 class _Calibrator:
     def __init__(self, num_bits=8, axis=None, unsigned=False):
         self._num_bits = num_bits

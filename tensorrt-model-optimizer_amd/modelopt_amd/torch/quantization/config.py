@@ -6,6 +6,7 @@ reference (modelopt/torch/quantization/config.py:146-440, 661-955, 958-1190) so 
 written for it is accepted unchanged.
 """
 
+import weakref
 from typing import Any, Literal
 
 from pydantic import BaseModel, ConfigDict, ValidationInfo, field_validator, model_validator
@@ -60,6 +61,9 @@ class _MappingConfig(BaseModel):
         return getattr(self, key) if key in self else default
 
 
+_QUANTIZER_ATTRIBUTES: dict = {}   # id(config) -> (weak reference to it, its quantizer_attributes())
+
+
 class QuantizerAttributeConfig(_MappingConfig):
     """Attributes of one ``TensorQuantizer`` (reference: config.py:661-955)."""
 
@@ -77,6 +81,34 @@ class QuantizerAttributeConfig(_MappingConfig):
     calibrator: Any = "max"
     rotate: bool = False
     pass_through_bwd: bool = False
+
+    def __setattr__(self, name, value):
+        super().__setattr__(name, value)
+        _QUANTIZER_ATTRIBUTES.pop(id(self), None)   # a field changed
+
+    def quantizer_attributes(self):
+        """``({"_num_bits": ..., "_disabled": ..., "_dynamic": ...}, calibrator spec)``: the
+        attribute names and values a ``TensorQuantizer`` takes from this config (``enable`` ->
+        ``_disabled``, ``type`` -> ``_dynamic``, every other field ``_<field>``).  Kept until a
+        field is assigned: a model conversion configures hundreds of quantizers from a handful
+        of config objects."""
+        entry = _QUANTIZER_ATTRIBUTES.get(id(self))
+        if entry is not None and entry[0]() is self:
+            return entry[1]
+        plain = {}
+        for name in type(self).model_fields:
+            val = getattr(self, name)
+            if name == "enable":
+                plain["_disabled"] = val is False
+            elif name == "type":
+                plain["_dynamic"] = val == "dynamic"
+            elif name != "calibrator":
+                plain[f"_{name}"] = val
+        made = (plain, self.calibrator)
+        key = id(self)
+        _QUANTIZER_ATTRIBUTES[key] = (weakref.ref(self, lambda _, key=key: _QUANTIZER_ATTRIBUTES.pop(key, None)),
+                                      made)
+        return made
 
     @model_validator(mode="before")
     @classmethod

@@ -90,6 +90,21 @@ def set_quantizer_by_cfg(quant_model: nn.Module, quant_cfg: dict | QuantizeConfi
 
 @functools.lru_cache(maxsize=512)
 def _compiled(pattern: str):
+    """``match(name)`` -> something that is not None when the wildcard matches.  The shapes almost
+    every config uses (``*suffix``, ``*infix*``, ``prefix*``, a literal) become string methods;
+    anything else is fnmatch's regular expression."""
+    body = pattern.strip("*")
+    if not any(c in body for c in "*?[]"):
+        lead, trail = pattern.startswith("*"), pattern.endswith("*") and len(pattern) > 1
+        stars = len(pattern) - len(body)
+        if stars == int(lead) + int(trail):     # no doubled stars to think about
+            if lead and trail:
+                return lambda name: True if body in name else None
+            if lead:
+                return lambda name: True if name.endswith(body) else None
+            if trail:
+                return lambda name: True if name.startswith(body) else None
+            return lambda name: True if name == body else None
     return re.compile(fnmatch.translate(pattern)).match
 
 

@@ -606,11 +606,14 @@ def _one_launch_search(module, x, w, ref, x_scales, w_scales, block, sq_err) -> 
         quantizer = getattr(module, name, None)
         if not isinstance(quantizer, TensorQuantizer) or quantizer.is_enabled:
             return False
-    k = w.shape[1]
+    n, k = w.shape
     tokens = x.numel() // k
-    if tokens > 512 or k % 8:
-        return False
     q = module.weight_quantizer
+    # what mo_awq_search_losses takes, checked before the activations of every alpha are written
+    # out for it (n_alpha x tokens x K values)
+    if (tokens == 0 or tokens > 512 or k % 128 or n % 128 or block not in (32, 64, 128) or q._unsigned
+            or any(t.data_ptr() % 16 for t in (x, w, w_scales, x_scales))):
+        return False
     xs = _hip.awq_scaled_activations(x.view(tokens, k), x_scales)
     return _hip.awq_search_losses_into(xs, w, w_scales, ref.view(tokens, -1), block, q._num_bits,
                                        q._unsigned, q._narrow_range, sq_err)

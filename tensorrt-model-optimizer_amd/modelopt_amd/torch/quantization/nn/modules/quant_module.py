@@ -23,6 +23,7 @@ class _Registry:
 
     def __init__(self):
         self._map: dict[type, type] = {}
+        self._derived: dict[tuple[type, type], type] = {}   # (quantised base, original class) -> class
 
     def register(self, mapping: dict[type, str]):
         def deco(qcls):
@@ -33,6 +34,8 @@ class _Registry:
 
     def unregister(self, orig):
         self._map.pop(orig, None)
+        for key in [k for k in self._derived if k[1] is orig]:
+            del self._derived[key]
 
     def get(self, orig):
         return self._map.get(orig)
@@ -44,9 +47,12 @@ class _Registry:
         """Swap ``module`` to its quantised class in place and create its quantizers."""
         qcls = self._map[type(module)]
         if type(module) is not qcls:
-            module._original_cls = type(module)
-            module.__class__ = type(f"Quant{module._original_cls.__name__}",
-                                    (qcls, module._original_cls), {})
+            orig = type(module)
+            object.__setattr__(module, "_original_cls", orig)
+            derived = self._derived.get((qcls, orig))
+            if derived is None:   # one class per pair, not one per converted instance
+                derived = self._derived[(qcls, orig)] = type(f"Quant{orig.__name__}", (qcls, orig), {})
+            module.__class__ = derived
         module._setup()
         return module
 
@@ -97,9 +103,11 @@ class QuantInputBase(QuantModule):
         return self.output_quantizer(output)
 
     def _setup(self):
-        self.add_module("input_quantizer", TensorQuantizer(self.default_quant_desc_input))
-        self.add_module("output_quantizer", TensorQuantizer(self.default_quant_desc_output))
-        self.output_quantizer.disable()
+        # plain insertion: the names are fixed and the values are modules (add_module's checks
+        # cost as much as building the quantizer)
+        self._modules["input_quantizer"] = TensorQuantizer(self.default_quant_desc_input)
+        out = self._modules["output_quantizer"] = TensorQuantizer(self.default_quant_desc_output)
+        out.disable()
 
 
 class QuantLinearConvBase(QuantInputBase):
@@ -127,5 +135,5 @@ class QuantLinearConvBase(QuantInputBase):
 
     def _setup(self):
         super()._setup()
-        self.add_module("weight_quantizer", TensorQuantizer(self.default_quant_desc_weight))
-        self._enable_weight_quantization = False
+        self._modules["weight_quantizer"] = TensorQuantizer(self.default_quant_desc_weight)
+        object.__setattr__(self, "_enable_weight_quantization", False)

@@ -88,6 +88,17 @@ class TensorQuantizer(nn.Module):
     def set_from_attribute_config(self, attribute_cfg: QuantizerAttributeConfig | dict):
         """Copy config fields onto ``_<field>`` attributes (``enable`` -> ``_disabled``,
         ``type`` -> ``_dynamic``, ``calibrator`` -> a calibrator instance)."""
+        if type(attribute_cfg) is QuantizerAttributeConfig:
+            # a complete, validated config: its attribute set is built once per config object.
+            # The values are plain python objects (never tensors or modules), so they go straight
+            # into the instance dict, past nn.Module's attribute bookkeeping
+            plain, calibrator = attribute_cfg.quantizer_attributes()
+            own = self.__dict__
+            own.update(plain)
+            own["_calibrator"] = self._make_calibrator(calibrator)
+            if self.is_mx_format:
+                self._pass_through_bwd = True
+            return
         items = attribute_cfg.items()
         fields = QuantizerAttributeConfig.model_fields
         for name, val in items:
@@ -625,6 +636,25 @@ class TensorQuantizer(nn.Module):
         if not self._if_calib or self._dynamic:
             return
         self._calibrator.collect(inputs)
+
+    def _only_collects_per_tensor(self) -> bool:
+        """``forward`` would do nothing but show the tensor to a per-tensor calibrator and hand
+        it back (calibration phase of a plain per-tensor quantizer)."""
+        return (type(self) is TensorQuantizer and self._if_calib and not self._if_quant
+                and not self._disabled and not self._dynamic and not self._rotate
+                and self._block_sizes is None and self._axis is None
+                and self.pre_quant_scale is None and self._calibrator is not None)
+
+    @staticmethod
+    def forward_pair(first, x0, second, x1):
+        """``(first(x0), second(x1))``; while both quantizers only collect per-tensor statistics
+        (calibration of the K / V cache quantizers) the two reductions share one launch."""
+        if (first._only_collects_per_tensor() and second._only_collects_per_tensor()
+                and isinstance(x0, torch.Tensor) and isinstance(x1, torch.Tensor)
+                and x0.numel() and x1.numel()
+                and calib.max.collect_pair(first._calibrator, x0, second._calibrator, x1)):
+            return x0, x1
+        return first(x0), second(x1)
 
     # ------------------------------------------------------------------ representation / state
     def _short_amax(self, fmt=".4f"):

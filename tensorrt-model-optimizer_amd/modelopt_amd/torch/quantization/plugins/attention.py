@@ -29,7 +29,9 @@ class QuantAttentionMixin(QuantModule):
             self.add_module(name, q)
 
     def _quantize_qkv(self, query, key, value):
-        return self.q_bmm_quantizer(query), self.k_bmm_quantizer(key), self.v_bmm_quantizer(value)
+        query = self.q_bmm_quantizer(query)
+        key, value = TensorQuantizer.forward_pair(self.k_bmm_quantizer, key, self.v_bmm_quantizer, value)
+        return query, key, value
 
 
 def register_attention_class(attn_cls: type):

@@ -110,3 +110,29 @@ def test_per_column_staged_path(dtype, shape):
     want2 = torch.maximum(want.float(), reduce.reduce_amax(big, axis=[0], keepdims=False).float())
     want2[3] = float("nan")
     assert_bits_equal(acc.cpu(), want2, f"warm, larger {shape}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n0,n1", [(1, 1), (8192 * 3 + 5, 7), (16 * 8 * 512 * 128, 16 * 8 * 512 * 128), (1000, 1 << 20)])
+def test_pair_of_tensors_in_one_launch(dtype, n0, n1):
+    """mo_absmax_pair: each tensor into its own running maximum, NaN propagating like torch.max."""
+    x0, x1 = _rand((n0,), dtype, 5), _rand((n1,), dtype, 6)
+    acc0 = torch.zeros(1, dtype=torch.float32, device=DEV)
+    acc1 = torch.full((1,), 2.5, dtype=torch.float32, device=DEV)          # a running maximum
+    assert _hip.absmax_pair_into(x0.to(DEV), acc0, x1.to(DEV), acc1)
+    assert_bits_equal(acc0.cpu().reshape(()).to(dtype), reduce.reduce_amax(x0), "first")
+    want1 = torch.maximum(reduce.reduce_amax(x1).float(), torch.tensor(2.5))
+    assert float(acc1) == float(want1)
+    if n1 > 3:
+        x1[n1 // 2] = float("nan")
+        assert _hip.absmax_pair_into(x0.to(DEV), acc0, x1.to(DEV), acc1)
+        assert torch.isnan(acc1).all() and not torch.isnan(acc0).any()
+
+
+def test_pair_rejects_what_it_does_not_cover():
+    a = torch.ones(64, dtype=torch.bfloat16, device=DEV)
+    acc = torch.zeros(1, dtype=torch.float32, device=DEV)
+    acc2 = torch.zeros(1, dtype=torch.float32, device=DEV)
+    assert not _hip.absmax_pair_into(a, acc, a.float(), acc2)              # two dtypes
+    assert not _hip.absmax_pair_into(a[1:33], acc, a, acc2)                # misaligned
+    assert float(acc) == 0 and float(acc2) == 0

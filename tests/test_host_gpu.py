@@ -640,3 +640,36 @@ def test_strict_checks_on_the_device():
             q(x)
     finally:
         mtq.set_strict_checks(previous)
+
+
+def test_k_and_v_calibrate_in_one_launch():
+    """The K / V cache quantizers of an attention layer are shown their tensors together: while
+    both only calibrate per tensor, one launch reduces both (same amax as one by one), a
+    transposed dense view included; any other state takes the two ordinary forwards."""
+    from modelopt_amd import _hip
+
+    def fresh():
+        q = TensorQuantizer(QuantizerAttributeConfig(num_bits=(4, 3), axis=None)).to(DEV)
+        q.enable_calib(); q.disable_quant()
+        return q
+
+    k = _rand((4, 8, 96, 128), seed=21).to(DEV)
+    v = _rand((4, 96, 8, 128), seed=22).to(DEV).transpose(1, 2)            # [B, H, S, D] view
+    qk, qv = fresh(), fresh()
+    with _hip.KernelTimer() as timer:
+        for _ in range(2):
+            out_k, out_v = TensorQuantizer.forward_pair(qk, k, qv, v)
+    assert timer.calls == {"mo_absmax_pair": 2}
+    assert out_k is k and out_v is v
+    for q, x in ((qk, k), (qv, v)):
+        q.load_calib_amax()
+        assert_bits_equal(q.amax.cpu().reshape(()), reduce.reduce_amax(x.cpu()).reshape(()), "amax")
+    # a quantizer that also quantises (or is disabled, per channel, ...) takes its own forward
+    qk2, qv2 = fresh(), fresh()
+    qv2.enable_quant(); qv2.amax = torch.tensor(8.0, device=DEV)
+    with _hip.KernelTimer() as timer:
+        out_k, out_v = TensorQuantizer.forward_pair(qk2, k, qv2, v)
+    assert "mo_absmax_pair" not in timer.calls
+    assert_bits_equal(out_v.cpu(), fake_quant.fp8_eager(v.cpu().contiguous(), torch.tensor(8.0)), "v fake quant")
+    qk2.load_calib_amax()
+    assert_bits_equal(qk2.amax.cpu().reshape(()), reduce.reduce_amax(k.cpu()).reshape(()), "k amax")
