@@ -14,6 +14,7 @@ from typing import Any
 import torch
 import torch.nn.functional as F
 from torch import nn
+from torch.nn.modules import module as _module_hooks
 
 from ... import calib, kernels, modes
 from ... import utils as quant_utils
@@ -639,8 +640,11 @@ class TensorQuantizer(nn.Module):
 
     def _only_collects_per_tensor(self) -> bool:
         """``forward`` would do nothing but show the tensor to a per-tensor calibrator and hand
-        it back (calibration phase of a plain per-tensor quantizer)."""
+        it back (calibration phase of a plain per-tensor quantizer; no hooks that a direct call
+        of the calibrator would skip)."""
         return (type(self) is TensorQuantizer and self._if_calib and not self._if_quant
+                and not self._forward_pre_hooks and not self._forward_hooks
+                and not _module_hooks._global_forward_pre_hooks and not _module_hooks._global_forward_hooks
                 and not self._disabled and not self._dynamic and not self._rotate
                 and self._block_sizes is None and self._axis is None
                 and self.pre_quant_scale is None and self._calibrator is not None)

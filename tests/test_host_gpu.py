@@ -664,6 +664,14 @@ def test_k_and_v_calibrate_in_one_launch():
     for q, x in ((qk, k), (qv, v)):
         q.load_calib_amax()
         assert_bits_equal(q.amax.cpu().reshape(()), reduce.reduce_amax(x.cpu()).reshape(()), "amax")
+    # a hook on either quantizer must see its call: the ordinary forwards run
+    qk3, qv3 = fresh(), fresh()
+    calls = []
+    handle = qv3.register_forward_pre_hook(lambda m, a: calls.append(tuple(a[0].shape)))
+    with _hip.KernelTimer() as timer:
+        TensorQuantizer.forward_pair(qk3, k, qv3, v)
+    handle.remove()
+    assert calls == [tuple(v.shape)] and "mo_absmax_pair" not in timer.calls
     # a quantizer that also quantises (or is disabled, per channel, ...) takes its own forward
     qk2, qv2 = fresh(), fresh()
     qv2.enable_quant(); qv2.amax = torch.tensor(8.0, device=DEV)
