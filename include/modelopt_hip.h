@@ -406,6 +406,21 @@ int mo_weight_scale_colsum(const void* x, int64_t rows, int64_t k, int dtype, in
 int mo_awq_scale_activations(const void* x, const void* inv_s, int64_t n_alpha, int64_t tokens,
                              int64_t k, int dtype, void* xs, void* stream);
 
+/* The candidate scales of a whole AWQ-lite alpha grid in one launch: get_scale
+ * (TQ/model_calib.py:608-621) for every alpha a of the grid,
+ *   s[a][c] = clamp(x_max[c]^alpha_a / (w_max[c]^(1 - alpha_a) + FLT_MIN), 1e-4, 1e4)
+ *   s[a]   /= sqrt(max_c s[a][c] * min_c s[a][c])
+ * in fp32 (IEEE division, correctly rounded square root; a NaN anywhere in a row makes the row NaN,
+ * as torch's amax / amin do).  exponents: device fp32 [4][n_alpha] -- alpha, 1 - alpha, and for
+ * each of the two how the power is evaluated: 0 powf, 1 the constant 1 (exponent 0), 2 the base
+ * (exponent 1), 3 the correctly rounded square root (exponent 0.5) -- the cases torch's scalar
+ * pow evaluates without calling pow.  Outputs: scales fp32 [n_alpha, k]; w_scales and x_scales
+ * (each optional) [n_alpha, k] in dtype: T(s), the weight quantizer's pre-quant scale of the
+ * search step, and T(1 / s), the input quantizer's (TQ/model_calib.py:661-664). */
+int mo_awq_scale_grid(const float* x_max, const float* w_max, const float* exponents,
+                      int64_t n_alpha, int64_t k, float* scales, void* w_scales, void* x_scales,
+                      int dtype, void* stream);
+
 /* AWQ-lite search step for a whole grid of alphas in one launch (bf16 only):
  *   q_a = block INT-N quantise-dequantise (blocks of block_size along k, dynamic abs-max) of
  *         bf16(w * s[a]);   out_a = bf16(xs[a] @ q_a^T)   (fp32 accumulation on the matrix cores)

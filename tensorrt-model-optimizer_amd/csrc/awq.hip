@@ -495,6 +495,65 @@ static inline unsigned blocks_for_awq(int64_t items, int64_t cap = 16384) {
     return (unsigned)b;
 }
 
+
+// ------------------------------------------------------------------------------ scale grid
+// The candidate scales of a whole alpha grid: one workgroup per alpha.  Pass 1 writes the clamped
+// quotients to `scales` and reduces their maximum and minimum; pass 2 divides every element
+// (each lane re-reads what it wrote itself) by sqrt(max * min) and writes the two rounded copies.
+__device__ __forceinline__ float grid_power(float base, float exponent, int mode) {
+    if (mode == 1) return 1.0f;                      // exponent 0
+    if (mode == 2) return base;                      // exponent 1
+    if (mode == 3) return __builtin_sqrtf(base);     // exponent 0.5: correctly rounded root
+    return __builtin_powf(base, exponent);
+}
+
+template <int DT>
+__global__ __launch_bounds__(1024) void awq_scale_grid_kernel(
+    const float* __restrict__ x_max, const float* __restrict__ w_max,
+    const float* __restrict__ exponents, int n_alpha, int k, float* __restrict__ scales,
+    void* __restrict__ w_scales, void* __restrict__ x_scales) {
+    __shared__ float red_max[16], red_min[16];
+    __shared__ int red_nan[16];
+    const int a = blockIdx.x;
+    const float ea = exponents[a], eb = exponents[n_alpha + a];
+    const int ma = (int)exponents[2 * n_alpha + a], mb = (int)exponents[3 * n_alpha + a];
+    float* row = scales + (int64_t)a * k;
+    float hi = 0.0f, lo = 3.0e38f;
+    int nan = 0;
+    for (int c = threadIdx.x; c < k; c += blockDim.x) {
+        const float num = grid_power(x_max[c], ea, ma);
+        const float den = grid_power(w_max[c], eb, mb) + 1.17549435e-38f;
+        float v = num / den;
+        v = v < 1e-4f ? 1e-4f : v;
+        v = v > 1e4f ? 1e4f : v;
+        row[c] = v;
+        if (v != v) nan = 1;
+        else { hi = v > hi ? v : hi; lo = v < lo ? v : lo; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float h2 = __shfl_xor(hi, o, kWave), l2 = __shfl_xor(lo, o, kWave);
+        hi = h2 > hi ? h2 : hi;
+        lo = l2 < lo ? l2 : lo;
+        nan |= __shfl_xor(nan, o, kWave);
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    if (lane == 0) { red_max[wave] = hi; red_min[wave] = lo; red_nan[wave] = nan; }
+    __syncthreads();
+    for (int w = 0; w < waves; ++w) {
+        hi = red_max[w] > hi ? red_max[w] : hi;
+        lo = red_min[w] < lo ? red_min[w] : lo;
+        nan |= red_nan[w];
+    }
+    const float norm = nan ? __builtin_nanf("") : __builtin_sqrtf(hi * lo);
+    for (int c = threadIdx.x; c < k; c += blockDim.x) {
+        const float v = row[c] / norm;
+        row[c] = v;
+        if (w_scales) store_elem<DT>(w_scales, (int64_t)a * k + c, v);
+        if (x_scales) store_elem<DT>(x_scales, (int64_t)a * k + c, 1.0f / v);
+    }
+}
+
 }  // namespace mo
 
 #define DISPATCH_DT(dtype, CALL)          \
@@ -669,5 +728,24 @@ extern "C" int mo_weight_scale_colsum(const void* x, int64_t rows, int64_t k, in
     DISPATCH_DT(dtype, CALL)
 #undef CALL
     mo::colsum_fold_partials_kernel<<<(unsigned)((k + 63) / 64), 256, 0, st>>>(partial, slabs, k, acc);
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+// The AWQ-lite candidate scales for every alpha of the search grid in one launch.
+extern "C" int mo_awq_scale_grid(const float* x_max, const float* w_max, const float* exponents,
+                                 int64_t n_alpha, int64_t k, float* scales, void* w_scales,
+                                 void* x_scales, int dtype, void* stream) {
+    if (n_alpha < 0 || k < 0) return MO_ERR_ARG;
+    if (dtype < MO_F32 || dtype > MO_BF16) return MO_ERR_DTYPE;
+    if (n_alpha == 0 || k == 0) return MO_OK;
+    if (!x_max || !w_max || !exponents || !scales) return MO_ERR_ARG;
+    if (n_alpha > 65535 || k > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    const int threads = k >= 4096 ? 1024 : 256;
+#define CALL(DT)                                                                                   \
+    mo::awq_scale_grid_kernel<DT><<<(unsigned)n_alpha, threads, 0, st>>>(                          \
+        x_max, w_max, exponents, (int)n_alpha, (int)k, scales, w_scales, x_scales)
+    DISPATCH_DT(dtype, CALL)
+#undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

@@ -54,6 +54,7 @@ SIGNATURES = {
     "mo_nf4_dequantize": [_P, _I64, _I64, _P, _P, _INT, _P],
     "mo_mul_cols": [_P, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_scale_block_int_qdq": [_P, _I64, _I64, _INT, _P, _INT, _I64, _INT, _INT, _INT, _P, _P],
+    "mo_awq_scale_grid": [_P, _P, _P, _I64, _I64, _P, _P, _P, _INT, _P],
     "mo_awq_scale_activations": [_P, _P, _I64, _I64, _I64, _INT, _P, _P],
     "mo_awq_search_losses": [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _INT, _I64, _INT, _INT, _INT, _P, _P],
     "mo_awq_clip_losses": [_P, _I64, _P, _I64, _I64, _INT, _I64, _P, _INT, _P, _INT, _INT, _INT, _INT, _P, _P],
@@ -584,6 +585,23 @@ def int4_pack_rows(w, ws):
     call("mo_int4_pack_rows", w, _ptr(w), batch, n, k, bs, dtype_code(w.dtype), _ptr(ws), _ptr(out),
          _stream(w))
     return out
+
+
+def awq_scale_grid(x_max, w_max, exponents, dtype):
+    """AWQ-lite candidate scales for every alpha of a grid: (fp32 scales [A, K], ``dtype`` copy,
+    ``dtype`` copy of the reciprocals).  ``exponents``: fp32 device tensor [4, A] (alpha,
+    1 - alpha, and the evaluation mode of each power, see ``mo_awq_scale_grid``)."""
+    _require_device(x_max, w_max, exponents)
+    assert x_max.dtype == w_max.dtype == exponents.dtype == torch.float32
+    assert x_max.is_contiguous() and w_max.is_contiguous() and exponents.is_contiguous()
+    n_alpha, k = exponents.shape[1], x_max.numel()
+    assert exponents.shape[0] == 4 and w_max.numel() == k
+    scales = torch.empty((n_alpha, k), dtype=torch.float32, device=x_max.device)
+    w_scales = torch.empty((n_alpha, k), dtype=dtype, device=x_max.device)
+    x_scales = torch.empty((n_alpha, k), dtype=dtype, device=x_max.device)
+    call("mo_awq_scale_grid", x_max, _ptr(x_max), _ptr(w_max), _ptr(exponents), n_alpha, k,
+         _ptr(scales), _ptr(w_scales), _ptr(x_scales), dtype_code(dtype), _stream(x_max))
+    return scales, w_scales, x_scales
 
 
 def awq_scaled_activations(x, inv_s):

@@ -22,7 +22,7 @@ from .calib.max import MaxCalibrator
 from .conversion import set_quantizer_by_cfg_context
 from .nn import QuantModule, SequentialQuantizer, TensorQuantizer
 from .nn.modules.tensor_quantizer import calibration_pass
-from .utils import all_valid_scales, deferred_scale_checks, is_quantized_linear
+from .utils import all_positive, all_valid_scales, deferred_scale_checks, is_quantized_linear
 
 __all__ = ["max_calibrate", "smoothquant", "awq", "awq_lite", "enable_stats_collection",
            "finish_stats_collection", "apply_pre_quant_scale_and_smooth",
@@ -158,21 +158,40 @@ def _apply_weight_pre_quant_scale(linear, pre_quant_scale):
     max_calibrate(linear, lambda lin: lin.weight_quantizer(lin.weight))
 
 
+def _host_copy_later(t: torch.Tensor) -> torch.Tensor:
+    """``t.cpu()`` without waiting for the device: a copy into pinned host memory queued on the
+    current stream.  The host may read it once that stream has been synchronised -- the
+    calibration algorithms end with a host synchronisation, so what they leave on the modules is
+    complete when they return.  The device tensor rides along (``_device_twin``) for consumers
+    that want the values back on the device."""
+    if not t.is_cuda:
+        return t
+    host = torch.empty(t.shape, dtype=t.dtype, pin_memory=True)
+    host.copy_(t, non_blocking=True)
+    host._device_twin = t
+    return host
+
+
+def _on_device(t: torch.Tensor, device) -> torch.Tensor:
+    """``t.to(device)``; a host copy made by ``_host_copy_later`` hands back the device tensor it
+    was copied from."""
+    twin = getattr(t, "_device_twin", None)
+    if twin is not None and twin.device == torch.device(device):
+        return twin
+    return t.to(device)
+
+
 @torch.no_grad()
-def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.Tensor | None = None,
-                                     _positive_later: list | None = None):
-    """Set the input ``pre_quant_scale`` and fold its inverse into the weight.  A caller that loops
-    over many layers passes ``_positive_later``: the scale is appended to it instead of being
-    checked for positivity here (a host synchronisation), and the caller checks them all at once."""
+def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.Tensor | None = None):
+    """Set the input ``pre_quant_scale`` and fold its inverse into the weight.  Inside a
+    ``deferred_scale_checks`` block (a caller that loops over many layers) the positivity of the
+    scale is checked when the block ends instead of here (a host synchronisation per layer)."""
     assert is_quantized_linear(linear), "Only quantized linear modules are supported"
     assert linear.input_quantizer.pre_quant_scale is None, "pre_quant_scale should be None first!"
     if pre_quant_scale is None:
         pre_quant_scale = getattr(linear.input_quantizer, "_pre_quant_scale", None)
     assert pre_quant_scale is not None, "pre_quant_scale should be provided or already set"
-    if _positive_later is None:
-        assert torch.all(pre_quant_scale > 0), "pre_quant_scale should be positive"
-    else:
-        _positive_later.append(pre_quant_scale)
+    assert all_positive(pre_quant_scale), "pre_quant_scale should be positive"
     pre_quant_scale = pre_quant_scale.to(torch.float32)  # fp32 keeps the scaling maths safe
 
     linear.input_quantizer._enable_pre_quant_scale = True
@@ -182,7 +201,7 @@ def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.T
     if linear.input_quantizer.amax is not None:
         assert hasattr(linear.input_quantizer, "_amax_for_smoothing")
         device, dtype = linear.weight.device, linear.weight.dtype
-        smoothing = linear.input_quantizer._amax_for_smoothing.to(device=device, dtype=dtype)
+        smoothing = _on_device(linear.input_quantizer._amax_for_smoothing, device).to(dtype)
         linear.input_quantizer.amax = (smoothing * pre_quant_scale.to(device)).amax().to(dtype)
 
 
@@ -238,7 +257,7 @@ def smoothquant(model: nn.Module, forward_loop=None, alpha=1.0):
         _hip.absmax_into(w.data.contiguous(), col, w.shape[0], w.shape[1], 1)
         weight_scale = col.to(dtype).reshape(1, -1)  # == w.abs().amax(dim=0, keepdim=True)
         scale_a = (_pow(weight_scale, 1 - alpha) / _pow(act_amax, alpha)).squeeze()
-        module.input_quantizer._amax_for_smoothing = act_amax.cpu()
+        module.input_quantizer._amax_for_smoothing = _host_copy_later(act_amax)
         module.input_quantizer.reset_amax()
         module.input_quantizer.axis = None
         module.input_quantizer.amax = act_amax.amax().to(dtype=dtype, device=device)
@@ -248,10 +267,9 @@ def smoothquant(model: nn.Module, forward_loop=None, alpha=1.0):
         dead = (scale_a.min() <= eps) & (act_amax.reshape(-1) <= eps)
         scale_a = torch.where(dead, torch.ones_like(scale_a), scale_a)
         scale_a = scale_a.clamp(min=1e-4, max=1e4)
-        apply_pre_quant_scale_and_smooth(module, scale_a, _positive_later=positive_later)
+        apply_pre_quant_scale_and_smooth(module, scale_a)
 
     smoothed = 0
-    positive_later = []   # checked once for all layers below
     with deferred_scale_checks():   # one synchronisation for the checks of all layers
         for name, module in model.named_modules():
             if not is_quantized_linear(module):
@@ -268,15 +286,38 @@ def smoothquant(model: nn.Module, forward_loop=None, alpha=1.0):
             assert module.input_quantizer._amax.numel() > 1, f"Error: {name} has only one channel to smooth"
             postprocess(module)
             smoothed += 1
-    by_device = {}
-    for p in positive_later:
-        by_device.setdefault(p.device, []).append((p > 0).all())
-    assert all(bool(torch.stack(flags).all()) for flags in by_device.values()), \
-        "pre_quant_scale should be positive"
     print(f"Smoothed {smoothed} modules")
 
 
 # ----------------------------------------------------------------------------- AWQ-clip
+@functools.lru_cache(maxsize=16)
+def _clip_ratios(min_clip_ratio: float, shrink_step: float) -> tuple:
+    """The clip ratios of the search, smallest first, 1.0 last (reference: model_calib.py:818-821)."""
+    return tuple(round(float(k), 2) for k in torch.arange(min_clip_ratio, 1.0, shrink_step)) + (1.0,)
+
+
+@functools.lru_cache(maxsize=16)
+def _ratio_column(ratios: tuple, device) -> torch.Tensor:
+    """The ratios as an fp32 device vector (built once per ratio list and device)."""
+    return torch.tensor(ratios, dtype=torch.float32).to(device)
+
+
+def _best_clip(helper):
+    """``(best_loss, best_clip_val)`` as the reference's loop over the ratios leaves them
+    (model_calib.py:958-966: a ratio replaces the running best when its loss is strictly smaller,
+    so the first smallest loss wins, a NaN never does, and a block for which no loss is below
+    infinity keeps a clip value of zero) -- from the stacked losses in a handful of launches
+    instead of three per ratio."""
+    ratios = tuple(helper.loss)
+    w_amax = helper.w_amax
+    loss = helper.loss_all.view(len(ratios), *w_amax.shape)
+    inf = torch.full((), float("inf"), dtype=loss.dtype, device=loss.device)
+    best_loss, index = torch.where(torch.isnan(loss), inf, loss).min(dim=0)
+    # amax * python float: one product in fp32, one rounding to the amax dtype
+    clip = (w_amax.float() * _ratio_column(ratios, w_amax.device)[index]).to(w_amax.dtype)
+    return best_loss, torch.where(best_loss < inf, clip, torch.zeros_like(clip))
+
+
 class _AWQClipHelper:
     """Per-linear state of the clip search (reference: model_calib.py:810-850)."""
 
@@ -288,7 +329,7 @@ class _AWQClipHelper:
         max_calibrate(q, lambda quantizer: quantizer(module.weight))
         self.w_amax = q.amax.clone()
         co, ci = module.weight.shape
-        ratios = [round(float(k), 2) for k in torch.arange(min_clip_ratio, 1.0, shrink_step)] + [1.0]
+        ratios = list(_clip_ratios(float(min_clip_ratio), float(shrink_step)))
         dev = module.weight.device
         if self.is_per_tensor_clip(module):
             self.loss = {k: torch.tensor(0.0, device=dev) for k in ratios}
@@ -408,7 +449,9 @@ def awq_clip(model: nn.Module, forward_loop, max_co_batch_size: int = 1024,
     max_calibrate(model, lambda m: None)
     for module in patched:
         helper = module.awq_clip
-        if helper.num_tokens > 0:
+        if helper.num_tokens > 0 and hasattr(helper, "loss_all"):
+            helper.best_loss, helper.best_clip_val = _best_clip(helper)
+        elif helper.num_tokens > 0:
             helper.best_loss = torch.ones_like(helper.w_amax) * float("inf")
             helper.best_clip_val = torch.zeros_like(helper.w_amax)
             for shrink, loss in helper.loss.items():
@@ -416,6 +459,7 @@ def awq_clip(model: nn.Module, forward_loop, max_co_batch_size: int = 1024,
                 better = loss < helper.best_loss
                 helper.best_loss = torch.where(better, loss, helper.best_loss)
                 helper.best_clip_val = torch.where(better, helper.w_amax * shrink, helper.best_clip_val)
+        if helper.num_tokens > 0:
             module.weight_quantizer.amax = helper.best_clip_val
             module.weight_quantizer.enable()
             if helper.is_input_quantized:
@@ -486,45 +530,34 @@ def get_act_scale(x):
 
 
 @functools.lru_cache(maxsize=64)
-def _exponent_columns_cached(alphas: tuple, device):
-    both = torch.tensor([[float(v) for v in alphas], [1 - float(v) for v in alphas]],
-                        dtype=torch.float32).to(device)
-    return both[0][:, None], both[1][:, None]
+def _exponent_table_cached(alphas: tuple, device):
+    """fp32 ``[4, A]`` on the device: alpha, 1 - alpha (the difference taken in double, as the
+    scalar form of ``pow`` does before it narrows the exponent), and for each of the two how the
+    power is evaluated -- 0 ``pow``; the exponents the scalar form of ``pow`` evaluates without
+    calling it: 1 the constant one (exponent 0), 2 the base itself (exponent 1), 3 the correctly
+    rounded square root (exponent 0.5, see ``_pow``)."""
+    def mode(e):
+        return {0.0: 1.0, 1.0: 2.0, 0.5: 3.0}.get(e, 0.0)
+    a = [float(v) for v in alphas]
+    b = [1 - v for v in a]
+    return torch.tensor([a, b, [mode(v) for v in a], [mode(v) for v in b]], dtype=torch.float32).to(device)
 
 
-def _exponent_columns(alphas, device):
-    """fp32 ``[A, 1]`` device columns of ``alpha`` and ``1 - alpha`` (the difference is taken in
-    double, as the scalar form of ``pow`` does before it narrows the exponent); built once per
-    alpha grid and device."""
-    return _exponent_columns_cached(tuple(float(v) for v in alphas), torch.device(device))
+def _exponent_table(alphas, device):
+    """Built once per alpha grid and device."""
+    return _exponent_table_cached(tuple(float(v) for v in alphas), torch.device(device))
 
 
-def _pow_rows(t, exponents, column):
-    """``[A, K]``: row i is ``_pow(t, exponents[i])``.  One broadcast ``pow`` over all rows; the
-    rows whose exponent the scalar form evaluates without calling ``pow`` (0, 1 and 0.5) are
-    then written the way it would write them."""
-    out = torch.pow(t.view(1, -1), column)
-    for i, e in enumerate(exponents):
-        if e == 0.0:
-            out[i].fill_(1.0)
-        elif e == 1.0:
-            out[i].copy_(t.view(-1))
-        elif e == 0.5:
-            out[i].copy_(_pow(t.view(-1), 0.5))
-    return out
-
-
-def get_scales(x_max, w_max, alphas, columns=None):
+def get_scales(x_max, w_max, alphas, table=None, dtype=None):
     """fp32 ``[len(alphas), K]``: row i is the AWQ scale ``x^a / w^(1-a)`` for ``a = alphas[i]``,
-    clamped to [1e-4, 1e4] and normalised by ``sqrt(max * min)`` of its own row.  The whole
-    search grid takes a fixed number of launches instead of a dozen per alpha."""
+    clamped to [1e-4, 1e4] and normalised by ``sqrt(max * min)`` of its own row -- the whole
+    search grid in one launch.  With ``dtype`` also the two rounded copies a search step
+    multiplies with: ``(scales, dtype(scales), dtype(1 / scales))``."""
     dev = x_max.device
-    col_a, col_b = columns if columns is not None else _exponent_columns(alphas, dev)
-    num = _pow_rows(x_max.float(), [float(v) for v in alphas], col_a)
-    den = _pow_rows(w_max.to(dev).float(), [1 - float(v) for v in alphas], col_b)
-    scales = (num / (den + torch.finfo(torch.float32).tiny)).clamp_(min=1e-4, max=1e4)
-    norm = (scales.amax(1, keepdim=True) * scales.amin(1, keepdim=True)).sqrt_()
-    return scales.div_(norm)
+    table = table if table is not None else _exponent_table(alphas, dev)
+    made = _hip.awq_scale_grid(x_max.float().contiguous().view(-1), w_max.to(dev).float().contiguous().view(-1),
+                               table, dtype if dtype is not None else torch.float32)
+    return made if dtype is not None else made[0]
 
 
 def get_scale(x_max, w_max, alpha):
@@ -549,7 +582,7 @@ class _AWQLiteHelper:
         self.loss = {a: 0.0 for a in self.alphas}
         self.best_scale = None
         self.best_alpha = None
-        self.exponent_columns = None  # device copies of alpha and 1 - alpha, made on first search step
+        self.exponent_columns = None  # device table of the exponents, made on first search step
         self.scale_grid = None        # (fp32 scales [n_alphas, K], weight-dtype copy, inverse) of the search
         self.is_input_quantized = module.input_quantizer.is_enabled
         self.num_tokens = 0
@@ -645,14 +678,14 @@ def _awq_forward(self, input, *args, **kwargs):
     dtype = self.weight.dtype
     fused = _fused_weight_path(self) and not args and not kwargs
     sq_err = torch.zeros(len(helper.alphas), dtype=torch.float64, device=ref.device)
-    if helper.exponent_columns is None or helper.exponent_columns[0].device != ref.device:
-        helper.exponent_columns = _exponent_columns(helper.alphas, ref.device)
+    if helper.exponent_columns is None or helper.exponent_columns.device != ref.device:
+        helper.exponent_columns = _exponent_table(helper.alphas, ref.device)
     # the candidate scales depend on the cached statistics only: built at the first search step,
     # reused by the later ones, and the best row is folded when the search is over
     grid = helper.scale_grid
     if grid is None or grid[1].dtype != dtype or grid[0].device != ref.device:
-        scales = get_scales(helper.act_scale, helper.weight_scale, helper.alphas, helper.exponent_columns)
-        grid = helper.scale_grid = (scales, scales.to(dtype), (1 / scales).to(dtype))
+        grid = helper.scale_grid = get_scales(helper.act_scale, helper.weight_scale, helper.alphas,
+                                              helper.exponent_columns, dtype)
     _, w_scales, x_scales = grid
     if fused:
         q = self.weight_quantizer
@@ -743,7 +776,7 @@ def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: boo
     # The best alpha is picked on the device and the checks are collected, so that folding the
     # scales of one layer does not wait for the search kernels of the layers behind it: one host
     # synchronisation at the end instead of three per layer.
-    positive_later, searched = [], []
+    searched = []
 
     def postprocess(module, name):
         h = module.awq_lite
@@ -765,13 +798,13 @@ def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: boo
                 delattr(q, "_pre_quant_scale")
         if h.is_input_quantized and module.input_quantizer.amax is not None:
             act_amax = module.input_quantizer.amax
-            module.input_quantizer._amax_for_smoothing = act_amax.cpu()
+            module.input_quantizer._amax_for_smoothing = _host_copy_later(act_amax)
             module.input_quantizer.reset_amax()
             module.input_quantizer.axis = None
             module.input_quantizer.amax = act_amax.amax()
             module.input_quantizer.enable()
         if h.is_enabled:
-            apply_pre_quant_scale_and_smooth(module, 1.0 / h.best_scale, _positive_later=positive_later)
+            apply_pre_quant_scale_and_smooth(module, 1.0 / h.best_scale)
         else:
             warnings.warn(f"awq_lite: Disabling for {name}, quantizing with max calibration.")
             max_calibrate(module, lambda module: module.weight_quantizer(module.weight))
@@ -795,11 +828,6 @@ def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: boo
                     kept.append(h)
                 else:
                     delattr(module, "awq_lite")
-    by_device = {}
-    for p in positive_later:
-        by_device.setdefault(p.device, []).append((p > 0).all())
-    assert all(bool(torch.stack(flags).all()) for flags in by_device.values()), \
-        "pre_quant_scale should be positive"
     if kept:  # the helpers stay on the modules: give them the numbers as Python values
         for h, loss, best in searched:
             h.loss = dict(zip(h.alphas, loss.tolist()))

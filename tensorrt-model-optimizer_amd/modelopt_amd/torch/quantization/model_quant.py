@@ -19,7 +19,7 @@ from . import model_calib
 from .config import QuantizeConfig, QuantizerAttributeConfig, normalize_algorithm
 from .conversion import is_converted, replace_quant_module, set_quantizer_attribute, set_quantizer_by_cfg
 from .nn import SequentialQuantizer, TensorQuantizer
-from .utils import all_valid_scales
+from .utils import DeferredCheckError, deferred_scale_checks
 
 __all__ = ["quantize", "calibrate", "disable_quantizer", "enable_quantizer", "print_quant_summary",
            "fold_weight", "postprocess_amax", "auto_quantize"]
@@ -69,26 +69,40 @@ def calibrate(model: nn.Module, algorithm="max", forward_loop: ForwardLoop | Non
     training = model.training
     model.eval()
     try:
-        if method == "max":
-            model_calib.max_calibrate(model, forward_loop, kwargs.get("distributed_sync", True))
-        elif method == "mse":
-            model_calib.mse_calibrate(model, forward_loop, kwargs.get("distributed_sync", True),
-                                      kwargs.get("num_steps", 10), kwargs.get("start_multiplier", 0.25),
-                                      kwargs.get("stop_multiplier", 4.0))
-        elif method == "smoothquant":
-            model_calib.smoothquant(model, forward_loop, alpha=kwargs.get("alpha", 1.0))
-        elif method in ("awq_clip", "awq_full"):
-            model_calib.awq(model, forward_loop, method, **kwargs)
-        elif method == "awq_lite":
-            model_calib.awq(model, forward_loop, "awq_lite", alpha_step=kwargs.get("alpha_step", 0.1),
-                            debug=kwargs.get("debug", False))
-        quantizers = [(n, m) for n, m in model.named_modules() if isinstance(m, TensorQuantizer)]
-        attrs = ("_amax", "_pre_quant_scale")
-        # one check for all of them; only a failure is walked through to name the culprit
-        if not all_valid_scales([getattr(m, a, None) for _, m in quantizers for a in attrs]):
+        # every "amax / scale is finite and non-negative" check of the algorithm and the final look at
+        # what it left on the quantizers are one device reduction and one host synchronisation
+        with deferred_scale_checks() as checks:
+            if method == "max":
+                model_calib.max_calibrate(model, forward_loop, kwargs.get("distributed_sync", True))
+            elif method == "mse":
+                model_calib.mse_calibrate(model, forward_loop, kwargs.get("distributed_sync", True),
+                                          kwargs.get("num_steps", 10), kwargs.get("start_multiplier", 0.25),
+                                          kwargs.get("stop_multiplier", 4.0))
+            elif method == "smoothquant":
+                model_calib.smoothquant(model, forward_loop, alpha=kwargs.get("alpha", 1.0))
+            elif method in ("awq_clip", "awq_full"):
+                model_calib.awq(model, forward_loop, method, **kwargs)
+            elif method == "awq_lite":
+                model_calib.awq(model, forward_loop, "awq_lite", alpha_step=kwargs.get("alpha_step", 0.1),
+                                debug=kwargs.get("debug", False))
+            quantizers = [(n, m) for n, m in model.named_modules() if isinstance(m, TensorQuantizer)]
+            attrs = ("_amax", "_pre_quant_scale")
+            checks.report = [t for _, m in quantizers for a in attrs
+                             if isinstance(t := getattr(m, a, None), torch.Tensor)]
+        # only a failure is walked through to name the culprit
+        if not checks.report_ok:
             for name, module in quantizers:
                 for attr in attrs:
                     module.validate_attr(attr_name=attr, warn_error=True, name=name)
+    except DeferredCheckError:
+        # a calibrator whose running maximum is bad says so in its own words (the reference's
+        # per-collect assertions); anything else keeps the message of the deferred check
+        for module in model.modules():
+            cal = getattr(module, "_calibrator", None) if isinstance(module, TensorQuantizer) else None
+            if getattr(cal, "_acc", None) is not None and hasattr(cal, "_validated"):
+                cal._validated = False
+                cal.compute_amax()
+        raise
     finally:
         model.train(training)
     return model

@@ -129,21 +129,83 @@ def update_quant_cfg_with_kv_cache_quant(quant_cfg: dict, kv_cache_quant_cfg: di
 _DEFERRED_CHECKS = []   # innermost ``deferred_scale_checks`` block last
 
 
+class DeferredCheckError(AssertionError):
+    """A check recorded inside a ``deferred_scale_checks`` block failed when the block ended."""
+
+
+class _DeferredChecks(list):
+    """The tensors a ``deferred_scale_checks`` block has recorded: the list itself holds those
+    that must be finite and non-negative, ``positive`` those that must be positive, ``report``
+    those whose validity is only reported (``report_ok`` after the block)."""
+
+    def __init__(self):
+        super().__init__()
+        self.positive = []
+        self.report = []
+        self.report_ok = True
+
+
+def _validity_flags(tensors, strictly_positive=False):
+    """0-dim bool device tensors, one per (device, dtype) group of ``tensors``: every element is
+    finite and non-negative (or positive).  No host synchronisation."""
+    groups = {}   # one concatenation per (device, dtype): no per-tensor conversion
+    for t in tensors:
+        if isinstance(t, torch.Tensor) and not t.is_meta and t.numel():
+            t = t.detach()
+            if not t.is_floating_point():
+                t = t.to(torch.float32)
+            groups.setdefault((t.device, t.dtype), []).append(t.reshape(-1))
+    flags = []
+    for group in groups.values():
+        v = torch.cat(group) if len(group) > 1 else group[0]
+        flags.append((v > 0).all() if strictly_positive else (torch.isfinite(v) & (v >= 0)).all())
+    return flags
+
+
+def _read_flags(flag_lists):
+    """``[all(flags) for flags in flag_lists]`` with one host synchronisation per device."""
+    by_device = {}
+    for i, flags in enumerate(flag_lists):
+        for f in flags:
+            by_device.setdefault(f.device, []).append((i, f))
+    result = [True] * len(flag_lists)
+    for entries in by_device.values():
+        values = torch.stack([f for _, f in entries]).tolist()
+        for (i, _), ok in zip(entries, values):
+            result[i] = result[i] and ok
+    return result
+
+
 @contextlib.contextmanager
 def deferred_scale_checks():
-    """Within the block ``all_valid_scales`` only records its tensors and reports True; the one
-    real check -- one host synchronisation -- happens when the block ends and raises
-    ``AssertionError`` if any recorded value is negative, infinite or NaN by then (a nested block
-    hands its tensors to the enclosing one).  For loops over many layers whose per-layer checks
-    would each wait for the device."""
-    pending = []
+    """Within the block ``all_valid_scales`` and ``all_positive`` only record their tensors and
+    report True; the real checks -- one device reduction per kind and ONE host synchronisation for
+    all of them -- happen when the outermost block ends, which raises ``AssertionError`` if a
+    recorded value is negative, infinite or NaN (not positive, for ``all_positive``) by then.  A
+    nested block hands its tensors to the enclosing one.  Tensors appended to ``report`` of the
+    yielded object are checked in the same synchronisation but only reported (``report_ok``).
+    For loops over many layers whose per-layer checks would each wait for the device."""
+    pending = _DeferredChecks()
     _DEFERRED_CHECKS.append(pending)
     try:
         yield pending
     finally:
         _DEFERRED_CHECKS.pop()
-    if pending and not all_valid_scales(pending):
-        raise AssertionError("detected negative, inf or nan values in a calibrated amax or scale")
+    if _DEFERRED_CHECKS:    # nested: the enclosing block checks
+        outer = _DEFERRED_CHECKS[-1]
+        outer.extend(pending)
+        outer.positive.extend(pending.positive)
+        if pending.report:   # the block's owner wants an answer now
+            pending.report_ok = _read_flags([_validity_flags(pending.report)])[0]
+        return
+    if not (pending or pending.positive or pending.report):
+        return
+    valid, positive, pending.report_ok = _read_flags([
+        _validity_flags(pending), _validity_flags(pending.positive, True), _validity_flags(pending.report)])
+    if not valid:
+        raise DeferredCheckError("detected negative, inf or nan values in a calibrated amax or scale")
+    if not positive:
+        raise DeferredCheckError("pre_quant_scale should be positive")
 
 
 def all_valid_scales(tensors) -> bool:
@@ -152,24 +214,16 @@ def all_valid_scales(tensors) -> bool:
     if _DEFERRED_CHECKS:
         _DEFERRED_CHECKS[-1].extend(t for t in tensors if isinstance(t, torch.Tensor))
         return True
-    groups = {}   # one concatenation per (device, dtype): no per-tensor conversion
-    for t in tensors:
-        if isinstance(t, torch.Tensor) and not t.is_meta and t.numel():
-            t = t.detach()
-            if not t.is_floating_point():
-                t = t.to(torch.float32)
-            groups.setdefault((t.device, t.dtype), []).append(t.reshape(-1))
-    if not groups:
+    return _read_flags([_validity_flags(tensors)])[0]
+
+
+def all_positive(tensor) -> bool:
+    """True when every element is positive; inside a ``deferred_scale_checks`` block the tensor is
+    recorded and the answer comes when the block ends (``AssertionError``)."""
+    if _DEFERRED_CHECKS:
+        _DEFERRED_CHECKS[-1].positive.append(tensor)
         return True
-    flags = []
-    for group in groups.values():
-        v = torch.cat(group) if len(group) > 1 else group[0]
-        flags.append((torch.isfinite(v) & (v >= 0)).all())
-    # one synchronisation per device at most: flags on one device are combined first
-    by_device = {}
-    for f in flags:
-        by_device.setdefault(f.device, []).append(f)
-    return all(bool(torch.stack(fs).all()) if len(fs) > 1 else bool(fs[0]) for fs in by_device.values())
+    return bool(torch.all(tensor > 0))
 
 
 @contextlib.contextmanager

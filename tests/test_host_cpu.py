@@ -621,6 +621,67 @@ def test_deferred_scale_checks_make_one_check_at_the_end():
     assert not all_valid_scales([torch.tensor([-1.0])])                  # outside a block: checked at once
 
 
+def test_best_clip_from_stacked_losses_equals_the_loop_over_ratios():
+    """model_calib.py:958-966 of the reference, ratio by ratio, against the stacked selection:
+    ties (the first smallest wins), NaN losses (never win), blocks with no finite loss (clip 0)."""
+    import types
+
+    from modelopt_amd.torch.quantization.model_calib import _best_clip, _clip_ratios
+
+    ratios = _clip_ratios(0.5, 0.05)
+    assert ratios == (0.5, 0.55, 0.6, 0.65, 0.7, 0.75, 0.8, 0.85, 0.9, 0.95, 1.0)
+    g = torch.Generator().manual_seed(0)
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        w_amax = (torch.rand(40, 1, generator=g) + 0.01).to(dtype)
+        loss_all = torch.rand(len(ratios), 8, 5, generator=g).round(decimals=1)    # many ties
+        loss_all[3, 0, 0] = float("nan")
+        loss_all[:, 1, 1] = float("nan")
+        loss_all[:, 2, 2] = float("inf")
+        loss_all[0, 3, 3] = -1.0
+        helper = types.SimpleNamespace(w_amax=w_amax, loss_all=loss_all,
+                                       loss={r: loss_all[i] for i, r in enumerate(ratios)})
+        best_loss = torch.ones_like(w_amax) * float("inf")
+        best_clip = torch.zeros_like(w_amax)
+        for shrink, loss in helper.loss.items():
+            loss = loss.view_as(w_amax)
+            better = loss < best_loss
+            best_loss = torch.where(better, loss, best_loss)
+            best_clip = torch.where(better, w_amax * shrink, best_clip)
+        got_loss, got_clip = _best_clip(helper)
+        assert got_clip.dtype == dtype and torch.equal(got_clip, best_clip)
+        assert torch.equal(got_loss, best_loss.float())
+        assert float(got_clip.view(8, 5)[1, 1]) == 0 and float(got_clip.view(8, 5)[2, 2]) == 0
+
+
+def test_deferred_checks_of_three_kinds_share_the_block_s_end():
+    from modelopt_amd.torch.quantization.utils import (DeferredCheckError, all_positive, all_valid_scales,
+                                                        deferred_scale_checks)
+    assert all_positive(torch.tensor([1.0, 2.0])) and not all_positive(torch.tensor([1.0, 0.0]))
+    with deferred_scale_checks() as block:
+        assert all_positive(torch.tensor([0.5]))
+        assert all_valid_scales([torch.zeros(3)])
+        block.report = [torch.tensor([1.0, float("inf")])]     # reported, never raised
+    assert block.report_ok is False
+    with pytest.raises(DeferredCheckError, match="pre_quant_scale should be positive"):
+        with deferred_scale_checks():
+            with deferred_scale_checks():                       # handed to the enclosing block
+                assert all_positive(torch.tensor([1.0, -1.0]))
+    with deferred_scale_checks() as outer:
+        with deferred_scale_checks() as inner:
+            inner.report = [torch.tensor([float("nan")])]       # a nested owner gets its answer at once
+        assert inner.report_ok is False and outer.report_ok
+
+
+def test_quantize_reports_a_bad_calibration_batch_in_the_calibrator_s_words(oracle_backend):
+    """Inside mtq.quantize every validity check waits for the end of the algorithm; a NaN that a
+    calibrator has seen is then reported with the reference's message (calib/max.py:74-77)."""
+    model = nn.Sequential(nn.Linear(16, 16))
+    x = torch.randn(4, 16)
+    x[1, 3] = float("nan")
+    with pytest.raises(AssertionError, match="detected nan values in amax"):
+        mtq.quantize(model, mtq.INT8_DEFAULT_CFG, lambda m: m(x))
+
+
 # ----------------------------------------------------------------------------- strict host checks
 @pytest.fixture
 def strict_checks():
