@@ -85,6 +85,19 @@ class TensorQuantizer(nn.Module):
         plain(self, "_dequantize", False)
         plain(self, "_input_dtype", None)
 
+    # Switches and settings (``_if_quant``, ``_disabled``, ``_axis`` ...) are plain python values
+    # written thousands of times while a model is converted and calibrated; nn.Module's
+    # ``__setattr__`` looks every value up as a parameter, module and buffer first.  A plain value
+    # under a name that is none of those goes straight to the instance dict.
+    _PLAIN_VALUE_TYPES = (bool, int, float, str, tuple, type(None))
+
+    def __setattr__(self, name, value):
+        if (type(value) in TensorQuantizer._PLAIN_VALUE_TYPES and name not in self._buffers
+                and name not in self._parameters and name not in self._modules):
+            object.__setattr__(self, name, value)
+        else:
+            super().__setattr__(name, value)
+
     # ------------------------------------------------------------------ configuration
     def set_from_attribute_config(self, attribute_cfg: QuantizerAttributeConfig | dict):
         """Copy config fields onto ``_<field>`` attributes (``enable`` -> ``_disabled``,
