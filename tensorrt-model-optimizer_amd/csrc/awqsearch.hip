@@ -16,8 +16,12 @@
 // and, between those matrix instructions, quantises its share of the tile of the next k block
 // into the other LDS buffer.  Two wavefronts share a SIMD, so one's vector work and LDS waits
 // run under the other's matrix instructions; an activation fragment is used for all 128
-// columns, which halves the traffic of the A operand through L2 against a 64-column tile.  The
-// output tile never leaves the registers: it is rounded to bf16, compared with the reference
+// columns, which halves the traffic of the A operand through L2 against a 64-column tile.  That
+// traffic is what bounds the kernel: the 32 compute units that share an L2 each pull the whole
+// activation matrix of their alpha through it once per column tile (4 MB per tile, 16 KB per
+// step of 16 k), and a wider tile, the only way to spend fewer bytes per matrix instruction, does
+// not fit the registers (512 tokens x 256 columns of fp32 is the whole register file of a
+// compute unit).  The output tile never leaves the registers: it is rounded to bf16, compared with the reference
 // output and reduced to one double per workgroup.
 //
 // The integer codes follow the reference's arithmetic (bound / amax, one IEEE multiply, round
@@ -196,8 +200,11 @@ __device__ __forceinline__ void awq_search_tile(
     const char* xab = (const char*)xa;
     const int steps = nkb * 8;
     // activation fragments are fetched this many steps ahead (a divisor of the 8 steps of a k
-    // block, so that a step's register slot j % PF is the same in every block)
-    constexpr int PF = 2;
+    // block, so that a step's register slot j % PF is the same in every block).  Four steps and
+    // the one-at-a-time B fragments below measure 5 - 6 % faster than two steps with all four B
+    // fragments of a step loaded up front (0.356 against 0.378 ms on the 21-alpha 4096 x 4096
+    // case); eight steps are slower again (255 registers, no room left for the scheduler).
+    constexpr int PF = 4;
     static_assert(8 % PF == 0, "slot of a step must not depend on the k block");
     u32x4 af[RB][PF];
 #pragma unroll
@@ -221,21 +228,25 @@ __device__ __forceinline__ void awq_search_tile(
         const int buf = kb & 1;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            bf16x8_t bfrag[NG];
             const int c = j * 2 + kg;
+            // B fragments one at a time, the next one's LDS read issued ahead of the current
+            // one's matrix instructions: 8 registers of fragments live instead of 16, which is
+            // what lets the activation prefetch above reach four steps without spilling
+            bf16x8_t afrag[RB];
+#pragma unroll
+            for (int mb = 0; mb < RB; ++mb) __builtin_memcpy(&afrag[mb], &af[mb][j % PF], 16);
+            u32x4 bnext = tile[buf][fr][c ^ (fr & 15)];
 #pragma unroll
             for (int nb = 0; nb < NG; ++nb) {
-                const int r = nb * 32 + fr;
-                const u32x4 t = tile[buf][r][c ^ (r & 15)];
-                __builtin_memcpy(&bfrag[nb], &t, 16);
-            }
+                bf16x8_t bcur;
+                __builtin_memcpy(&bcur, &bnext, 16);
+                if (nb + 1 < NG) {
+                    const int r = (nb + 1) * 32 + fr;
+                    bnext = tile[buf][r][c ^ (r & 15)];
+                }
 #pragma unroll
-            for (int mb = 0; mb < RB; ++mb) {
-                bf16x8_t afrag;
-                __builtin_memcpy(&afrag, &af[mb][j % PF], 16);
-#pragma unroll
-                for (int nb = 0; nb < NG; ++nb)
-                    acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[nb],
+                for (int mb = 0; mb < RB; ++mb)
+                    acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag[mb], bcur,
                                                                           acc[mb][nb], 0, 0, 0);
             }
             int g = kb * 8 + j + PF;
