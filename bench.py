@@ -226,18 +226,30 @@ def single_tensor_configs(torch, steps, warmup):
     acc = torch.zeros(1, dtype=torch.float32, device=dev)
     y = torch.empty_like(w)
 
+    def train(fn, reps=200):
+        # one event pair around a train of passes (after an untimed train of the same length): a
+        # pass is 20 - 80 us, which an event pair per pass would inflate by several microseconds
+        for _ in range(reps):
+            fn()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / reps
+
     def c1():
-        acc.zero_()
+        # the calibrator's running maximum (no fill per pass: the accumulator only ever grows,
+        # and a second look at the same tensor leaves it as it is), then the fake quant with it
         _hip.absmax_into(w, acc, 1, 1, w.numel())
         _hip.fp8_qdq(w, acc, 1, 1, w.numel(), out=y)
-    _, ms = timed(torch, c1, steps, warmup)
-    out["c1_fp8_amax_plus_qdq_4096x4096"] = {"ms": round(ms, 4), "GBps": round(w.numel() * 6 / ms / 1e6, 1)}
-
+    ms = train(c1)
     # the same in one launch that reads the tensor once (4 B / element): every workgroup keeps its
     # share in registers while the workgroups agree on the abs-max
     def c1_fused():
         assert _hip.fused_amax_qdq(w, "fp8", out=y) is not None
-    _, ms = timed(torch, c1_fused, max(steps, 50), max(warmup, 10))
+    ms = train(c1_fused)
     out["c1_fp8_fused_amax_qdq_4096x4096"] = {"ms": round(ms, 4), "GBps": round(w.numel() * 4 / ms / 1e6, 1),
                                               "bytes_per_element": 4}
     wq = (0.02 * torch.randn(4096, 4096, generator=torch.Generator().manual_seed(7))).to(torch.bfloat16).to(dev)
@@ -249,8 +261,7 @@ def single_tensor_configs(torch, steps, warmup):
 
     def nvfp4_fused():
         assert _hip.nvfp4_quantize_fused(wq) is not None
-    _, ms2 = timed(torch, nvfp4_two, max(steps, 50), max(warmup, 10))
-    _, ms1 = timed(torch, nvfp4_fused, max(steps, 50), max(warmup, 10))
+    ms2, ms1 = train(nvfp4_two), train(nvfp4_fused)
     out["nvfp4_amax_plus_quantize_one_weight_4096x4096"] = {
         "two_launches_ms": round(ms2, 4), "fused_one_launch_ms": round(ms1, 4),
         "fused_GBps": round(wq.numel() * QUANT_BYTES_PER_ELEM / ms1 / 1e6, 1)}
@@ -261,11 +272,12 @@ def single_tensor_configs(torch, steps, warmup):
          ).to(torch.bfloat16).to(dev)
     y = torch.empty_like(x)
 
+    acc.zero_()
+
     def c4():
-        acc.zero_()
         _hip.absmax_into(x, acc, 1, 1, x.numel())
         _hip.nvfp4_qdq(x, acc, 16, 0, out=y)
-    _, ms = timed(torch, c4, steps, warmup)
+    ms = train(c4)
     out["c4_nvfp4_amax_plus_qdq_8192x8192"] = {"ms": round(ms, 4), "GBps": round(x.numel() * 6 / ms / 1e6, 1)}
 
     class OneLinear(nn.Module):
