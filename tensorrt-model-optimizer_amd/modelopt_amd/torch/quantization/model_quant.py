@@ -46,10 +46,36 @@ def _full_attribute_cfg(cfg):
     raise TypeError(f"unsupported quantizer config entry: {cfg!r}")
 
 
+_VALIDATED = {}   # repr of a plain config -> (validated quant_cfg, algorithm); a handful of entries
+
+
+def _plain(value) -> bool:
+    """Only dicts, lists, tuples and scalars: ``repr`` then says all there is to say about it."""
+    if isinstance(value, dict):
+        return all(isinstance(k, (str, int)) and _plain(v) for k, v in value.items())
+    if isinstance(value, (list, tuple)):
+        return all(_plain(v) for v in value)
+    return value is None or isinstance(value, (bool, int, float, str))
+
+
 def _validated(config):
-    config = config if isinstance(config, QuantizeConfig) else QuantizeConfig(**dict(config))
-    quant_cfg = {k: _full_attribute_cfg(v) for k, v in config.quant_cfg.items()}
-    return quant_cfg, config.algorithm
+    """``(quant_cfg with every entry a complete QuantizerAttributeConfig, algorithm)``.  A config
+    made of plain values only (every named config is) is validated once per distinct content:
+    the validated entries are never handed out or written to -- a quantizer copies what it takes
+    from them -- so calls with an equal config can share them."""
+    key = None
+    if isinstance(config, dict) and _plain(config):
+        key = repr(config)
+        hit = _VALIDATED.get(key)
+        if hit is not None:
+            return dict(hit[0]), copy.deepcopy(hit[1])
+    parsed = config if isinstance(config, QuantizeConfig) else QuantizeConfig(**dict(config))
+    quant_cfg = {k: _full_attribute_cfg(v) for k, v in parsed.quant_cfg.items()}
+    if key is not None:
+        if len(_VALIDATED) >= 32:
+            _VALIDATED.clear()
+        _VALIDATED[key] = (dict(quant_cfg), copy.deepcopy(parsed.algorithm))
+    return quant_cfg, parsed.algorithm
 
 
 def calibrate(model: nn.Module, algorithm="max", forward_loop: ForwardLoop | None = None) -> nn.Module:

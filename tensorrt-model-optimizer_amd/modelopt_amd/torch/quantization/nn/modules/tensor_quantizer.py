@@ -109,6 +109,9 @@ class TensorQuantizer(nn.Module):
             plain, calibrator = attribute_cfg.quantizer_attributes()
             own = self.__dict__
             own.update(plain)
+            for name in ("_block_sizes", "_bias"):   # a quantizer owns its mutable settings
+                if own[name] is not None:
+                    own[name] = dict(own[name])
             own["_calibrator"] = self._make_calibrator(calibrator)
             if self.is_mx_format:
                 self._pass_through_bwd = True

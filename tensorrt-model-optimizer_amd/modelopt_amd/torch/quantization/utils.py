@@ -146,8 +146,10 @@ class _DeferredChecks(list):
 
 
 def _validity_flags(tensors, strictly_positive=False):
-    """0-dim bool device tensors, one per (device, dtype) group of ``tensors``: every element is
-    finite and non-negative (or positive).  No host synchronisation."""
+    """What decides "every element is finite and non-negative (or positive)", one entry per
+    (device, dtype) group of ``tensors``: the group's ``(min, max)`` as a 2-element device tensor
+    from one ``aminmax`` over the concatenation (a NaN anywhere makes both NaN).  No host
+    synchronisation."""
     groups = {}   # one concatenation per (device, dtype): no per-tensor conversion
     for t in tensors:
         if isinstance(t, torch.Tensor) and not t.is_meta and t.numel():
@@ -158,7 +160,7 @@ def _validity_flags(tensors, strictly_positive=False):
     flags = []
     for group in groups.values():
         v = torch.cat(group) if len(group) > 1 else group[0]
-        flags.append((v > 0).all() if strictly_positive else (torch.isfinite(v) & (v >= 0)).all())
+        flags.append((torch.stack(torch.aminmax(v)).float(), strictly_positive))
     return flags
 
 
@@ -166,12 +168,16 @@ def _read_flags(flag_lists):
     """``[all(flags) for flags in flag_lists]`` with one host synchronisation per device."""
     by_device = {}
     for i, flags in enumerate(flag_lists):
-        for f in flags:
-            by_device.setdefault(f.device, []).append((i, f))
+        for pair, positive in flags:
+            by_device.setdefault(pair.device, []).append((i, pair, positive))
     result = [True] * len(flag_lists)
     for entries in by_device.values():
-        values = torch.stack([f for _, f in entries]).tolist()
-        for (i, _), ok in zip(entries, values):
+        pairs = entries[0][1] if len(entries) == 1 else torch.cat([p for _, p, _ in entries])
+        values = pairs.tolist()
+        for n, (i, _, positive) in enumerate(entries):
+            lo, hi = values[2 * n], values[2 * n + 1]
+            # a NaN anywhere makes lo and hi NaN, and every comparison with it false
+            ok = lo > 0 if positive else (lo >= 0 and hi < float("inf"))
             result[i] = result[i] and ok
     return result
 
