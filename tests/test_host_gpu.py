@@ -681,3 +681,27 @@ def test_k_and_v_calibrate_in_one_launch():
     assert_bits_equal(out_v.cpu(), fake_quant.fp8_eager(v.cpu().contiguous(), torch.tensor(8.0)), "v fake quant")
     qk2.load_calib_amax()
     assert_bits_equal(qk2.amax.cpu().reshape(()), reduce.reduce_amax(k.cpu()).reshape(()), "k amax")
+
+
+@pytest.mark.parametrize("seed,n,k,tokens", [(11, 128, 256, 64), (12, 256, 512, 200), (13, 384, 384, 96),
+                                             (14, 128, 1024, 512), (15, 512, 256, 33), (16, 256, 256, 300)])
+def test_awq_lite_selects_the_oracle_s_alpha_on_several_layers(seed, n, k, tokens):
+    """The one-launch search scores the alphas with arithmetic that differs from the CPU path's by
+    an ulp of a rare weight; what matters downstream is which alpha wins.  Several layers and
+    seeds: same best alpha as the CPU restatement of the search loop, losses within 1e-3, and the
+    scale that is folded is the oracle's formula at that alpha."""
+    g = torch.Generator().manual_seed(seed)
+    ref = _OneLinear(n=n, k=k, seed=seed)
+    c = torch.exp(torch.randn(k, generator=g))
+    c[torch.randperm(k, generator=g)[: max(1, k // 64)]] *= 20
+    batches = [(torch.randn(tokens, k, generator=g) * c).to(torch.bfloat16) for _ in range(2)]
+    model = copy.deepcopy(ref).to(DEV)
+    cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
+    cfg["algorithm"] = {"method": "awq_lite", "alpha_step": 0.1, "debug": True}
+    mtq.quantize(model, cfg, lambda m: [m(b.to(DEV)) for b in batches])
+    losses, best_alpha, best_scale, _, _ = oawq.awq_lite_search(ref.proj.weight.data, batches, 0.1, 128)
+    h = model.proj.awq_lite
+    assert h.best_alpha == best_alpha, (h.loss, losses)
+    for a in losses:
+        assert h.loss[a] == pytest.approx(losses[a], rel=1e-3), f"alpha {a}"
+    assert torch.allclose(h.best_scale.cpu(), best_scale, rtol=2 ** -6)
