@@ -534,6 +534,60 @@ def calib_sweep(torch, layers, n_seqs, batch, seq_len=512):
     }
 
 
+def probe_l2(torch):
+    """How fast the compute units pull L2-resident data through L1 misses (the path the A operand of
+    the AWQ-lite search kernel takes: 3.93 GB per launch of the 21-alpha 4096 x 4096 case).  A
+    kernel that only loads, from libmodelopt_probe.so: one workgroup of 8 wavefronts per compute
+    unit as in the search kernel (or four, with no unused LDS), every workgroup of an XCD walking
+    the same region in step ("shared", the search kernel's pattern) or its own slice of it
+    ("distinct"), 4 / 8 / 16 loads of 16 bytes in flight per lane."""
+    import ctypes
+
+    lib = ctypes.CDLL(os.path.join(ROOT, "tensorrt-model-optimizer_amd", "libmodelopt_probe.so"))
+    fn = lib.mo_probe_l2_read
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                   ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    dev = torch.device("cuda:0")
+    units = torch.cuda.get_device_properties(dev).multi_processor_count
+    buf = torch.zeros(8 * (4 << 20), dtype=torch.uint8, device=dev)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = []
+    for per_unit, ballast in ((1, 96 << 10), (4, 0)):
+        wgs = units * per_unit
+        for pattern in ("shared", "distinct"):
+            for region in (2 << 20, 4 << 20):
+                for depth in (4, 8, 16):
+                    step = 512 * depth * 16
+                    span = region if pattern == "shared" else region // (wgs // 8) // step * step
+                    if span == 0:
+                        continue
+                    passes = max(1, (256 << 20) // span // per_unit)   # about 64 GB through L1 misses per launch
+
+                    def launch():
+                        rc = fn(buf.data_ptr(), buf.numel(), region, span, wgs, passes, int(pattern == "distinct"),
+                                depth, ballast, sink.data_ptr(), stream)
+                        assert rc == 0, rc
+
+                    for _ in range(2):
+                        launch()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(5):
+                        launch()
+                    e1.record()
+                    torch.cuda.synchronize()
+                    ms = e0.elapsed_time(e1) / 5
+                    nbytes = wgs * passes * span
+                    rows.append({"workgroups_per_unit": per_unit, "pattern": pattern, "region_mb_per_xcd": region >> 20,
+                                 "loads_in_flight_per_lane": depth, "ms": round(ms, 3),
+                                 "tb_per_s": round(nbytes / ms / 1e9, 2),
+                                 "gb_per_s_per_unit": round(nbytes / ms / 1e6 / units, 1)})
+    assert int(sink.item()) == 0
+    return {"probe": "l2_resident_reads_through_l1_misses", "compute_units": units, "rows": rows}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -550,6 +604,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device copy (a kernel of known traffic for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--probe-l2", action="store_true",
+                    help="only measure the L2 -> compute unit read rate with the load-only probe kernel and exit")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU only: this build has no multi-GPU path (got --gpus {a.gpus}); "
@@ -565,6 +621,9 @@ def main():
     _hip.load()  # fail loudly if the HIP library is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if a.probe_l2:
+        print(json.dumps(probe_l2(torch)))
+        return
 
     weights = make_weights(torch, a.layers, dev)
     elems = sum(w.numel() for w in weights)

@@ -18,6 +18,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmodelopt_hip.so")
+PROBE_SRC = os.path.join(CSRC, "probe", "l2_read_probe.hip")   # measurement aid for bench.py, its own library
+PROBE_LIB = os.path.join(HERE, "libmodelopt_probe.so")
 HEADERS = [os.path.join(CSRC, h) for h in ("common.h", "qdq_ops.h", "awq_ops.h")] + [
     os.path.join(HERE, "..", "include", "modelopt_hip.h")]
 
@@ -62,6 +64,8 @@ def build(force=False, jobs=4, tuning=False):
     if force or _stale(lib, objs):
         subprocess.run(["hipcc", "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-o", lib],
                        check=True)
+    if not tuning and (force or _stale(PROBE_LIB, [PROBE_SRC])):
+        subprocess.run(["hipcc", *FLAGS, "-shared", "-x", "hip", PROBE_SRC, "-o", PROBE_LIB], check=True)
     return lib
 
 
