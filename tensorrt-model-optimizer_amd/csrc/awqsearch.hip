@@ -16,13 +16,18 @@
 // and, between those matrix instructions, quantises its share of the tile of the next k block
 // into the other LDS buffer.  Two wavefronts share a SIMD, so one's vector work and LDS waits
 // run under the other's matrix instructions; an activation fragment is used for all 128
-// columns, which halves the traffic of the A operand through L2 against a 64-column tile.  That
-// traffic is what bounds the kernel: the 32 compute units that share an L2 each pull the whole
-// activation matrix of their alpha through it once per column tile (4 MB per tile, 16 KB per
-// step of 16 k), and a wider tile, the only way to spend fewer bytes per matrix instruction, does
-// not fit the registers (512 tokens x 256 columns of fp32 is the whole register file of a
-// compute unit).  The output tile never leaves the registers: it is rounded to bf16, compared with the reference
-// output and reduced to one double per workgroup.
+// columns, which halves the traffic of the A operand through L2 against a 64-column tile (a
+// wider tile does not fit the registers: 512 tokens x 256 columns of fp32 is the whole register
+// file of a compute unit).  The 32 compute units that share an L2 each pull the whole activation
+// matrix of their alpha through it once per column tile (4 MB per tile, 16 KB per step of 16 k):
+// 11 - 12 TB/s over the chip, a third of what a load-only kernel draws through the same path, so
+// it is the latency of the loads, not their bytes, that the loop has to hide.  Three things do
+// that, each measured: the loads of a step stay in that step (a scheduling barrier per step; the
+// compiler otherwise gathers them and drains the in-order load counter mid-block), the raw
+// weights of the tile after the next are asked for seven steps ahead, as soon as their
+// registers fall free, and they are plain loads so that the next alpha finds them in the
+// last-level cache.  The output tile never leaves the registers: it is rounded to bf16, compared
+// with the reference output and reduced to one double per workgroup.
 //
 // The integer codes follow the reference's arithmetic (bound / amax, one IEEE multiply, round
 // half to even) with bound / amax from the hardware reciprocal and one FMA correction step,
@@ -214,9 +219,9 @@ __device__ __forceinline__ void awq_search_tile(
     const int steps = nkb * 8;
     // activation fragments are fetched this many steps ahead (a divisor of the 8 steps of a k
     // block, so that a step's register slot j % PF is the same in every block).  Four steps and
-    // the one-at-a-time B fragments below measure 5 - 6 % faster than two steps with all four B
-    // fragments of a step loaded up front (0.356 against 0.378 ms on the 21-alpha 4096 x 4096
-    // case); eight steps are slower again (255 registers, no room left for the scheduler).
+    // the one-at-a-time B fragments below measured 5 - 6 % faster than two steps with all four B
+    // fragments of a step loaded up front; eight steps are slower again (255 registers, no room
+    // left for the scheduler).
     constexpr int PF = 4;
     static_assert(8 % PF == 0, "slot of a step must not depend on the k block");
     u32x4 af[RB][PF];
