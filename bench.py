@@ -342,7 +342,7 @@ def single_tensor_configs(torch, steps, warmup):
 
     def search():
         _hip.awq_search_losses_into(xs, w3, scales, ref, 128, 4, False, False, loss)
-    _, ms = timed(torch, search, max(steps, 50), max(warmup, 20))  # past the clock ramp
+    ms = train(search, reps=50)   # 50 untimed launches (past the clock ramp), then 50 under one event pair
     kflops = 2 * 512 * 4096 * 4096 * 21
     out["c3_awq_search_kernel_21_alphas"] = {
         "ms": round(ms, 4), "TFLOPs": round(kflops / ms / 1e9, 1), "bound": "mfma",
@@ -359,7 +359,7 @@ def single_tensor_configs(torch, steps, warmup):
 
     def clip():
         _hip.awq_clip_losses_into(x64, w3, w_amax, ratios, 128, 4, False, False, clip_loss)
-    _, ms = timed(torch, clip, steps, warmup)
+    ms = train(clip, reps=20)
     products = 4096 * 4096 * 64 * (len(ratios) + 1)
     out["awq_clip_search_kernel_11_ratios_4096x4096_64_tokens"] = {
         "ms": round(ms, 4), "rounded_products_per_s": round(products / ms * 1e3, 0), "bound": "valu",
