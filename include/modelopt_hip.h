@@ -70,6 +70,21 @@ int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dty
 int mo_absmax_pair(const void* x0, int64_t n0, float* acc0, const void* x1, int64_t n1,
                    float* acc1, int dtype, void* stream);
 
+/* The smallest and the largest element of each of n <= 32 tensors and whether it holds a NaN, in
+ * one launch.  Tensor i owns max(1, ceil(counts[i] / 4096)) consecutive chunks of out, tensors in
+ * order; chunk c of the launch writes out[3 c] = min, out[3 c + 1] = max (NaN elements ignored;
+ * +inf / -inf for an empty tensor), out[3 c + 2] = 1 if the chunk holds a NaN, else 0, and the
+ * caller folds a tensor's chunks.  xs, counts and dtypes are host arrays of n entries (device
+ * pointers, element counts, MO_F32 / MO_F16 / MO_BF16); out is a device buffer of 3 * out_chunks
+ * floats.  These are the reductions behind the reference's validity checks of calibrated values --
+ * torch.all(amax >= 0) and no inf, no NaN (TensorQuantizer.validate_attr,
+ * TQ/nn/modules/tensor_quantizer.py:516-536) and torch.all(pre_quant_scale > 0)
+ * (TQ/model_calib.py:384) -- which it runs per quantizer with a host synchronisation each; here
+ * the host reads all answers of an algorithm at once.  MO_ERR_TOO_LARGE for n > 32 or more
+ * chunks than out_chunks. */
+int mo_value_ranges(const void* const* xs, const int64_t* counts, const int* dtypes, int n,
+                    float* out, int64_t out_chunks, void* stream);
+
 /* Per-tensor mo_absmax (outer = axis = 1, inner = n) that also leaves the abs-max of every
  * 32768-element tile of x in parts[0 .. *parts_written): the maximum of those words is the
  * abs-max of this tensor alone, whatever acc held before.  For calibration loops that show one
@@ -420,6 +435,19 @@ int mo_awq_scale_activations(const void* x, const void* inv_s, int64_t n_alpha, 
 int mo_awq_scale_grid(const float* x_max, const float* w_max, const float* exponents,
                       int64_t n_alpha, int64_t k, float* scales, void* w_scales, void* x_scales,
                       int dtype, void* stream);
+
+/* The end of an AWQ-lite search for one linear, in one launch: best = the index of the first
+ * smallest of the n_alpha losses -- what min(loss, key=loss.get) picks (TQ/model_calib.py:633): a
+ * NaN is never smaller than anything and a NaN in front is never replaced -- and, from row best
+ * of the fp32 candidate grid scales [n_alpha, k] (mo_awq_scale_grid), the tensors the folding
+ * makes of it (TQ/model_calib.py:764 and 384-393): best_scale[c] = scales[best][c],
+ * pre_quant_scale[c] = 1 / best_scale[c] (fp32, IEEE division), pre_quant_scale_t[c] the same
+ * rounded to dtype (the input quantizer's buffer), fold[c] = 1 / pre_quant_scale[c] (what the
+ * weight is multiplied by).  loss is a device array of doubles; best (one int64) and every output
+ * row are optional device buffers. */
+int mo_awq_pick_scale(const double* loss, int64_t n_alpha, const float* scales, int64_t k,
+                      int64_t* best, float* best_scale, float* pre_quant_scale,
+                      void* pre_quant_scale_t, float* fold, int dtype, void* stream);
 
 /* AWQ-lite search step for a whole grid of alphas in one launch (bf16 only):
  *   q_a = block INT-N quantise-dequantise (blocks of block_size along k, dynamic abs-max) of

@@ -585,6 +585,70 @@ static int scratch_address(uint32_t** out) {
     return MO_OK;
 }
 
+
+// ---------------------------------------------------------------- value ranges of small tensors
+// The smallest and the largest element of each of up to kRangeJobs tensors, and whether it holds
+// a NaN, one launch for all of them: a workgroup per 4096-element chunk of a tensor, three floats
+// per chunk for the host to fold.  The tensors are calibrated amax and scale buffers (a scalar
+// to a few hundred thousand values each), whose "finite, not negative" checks the host wants
+// answered with a single synchronisation.
+constexpr int kRangeJobs = 32;
+constexpr int kRangeChunk = 4096;
+struct RangeJobs {
+    const void* ptr[kRangeJobs];
+    int64_t count[kRangeJobs];
+    int dtype[kRangeJobs];
+    int first[kRangeJobs + 1];   // first workgroup of each tensor; first[n] = the grid
+};
+
+__global__ __launch_bounds__(256) void value_ranges_kernel(RangeJobs jobs, int n, float* __restrict__ out) {
+    int job = 0;
+    while (job + 1 < n && (int)blockIdx.x >= jobs.first[job + 1]) ++job;
+    const void* p = jobs.ptr[job];
+    const int dt = jobs.dtype[job];
+    const int64_t begin = (int64_t)((int)blockIdx.x - jobs.first[job]) * kRangeChunk;
+    const int64_t left = jobs.count[job] - begin;
+    const int here = left < kRangeChunk ? (int)left : kRangeChunk;
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    bool nan = false;
+#pragma unroll
+    for (int u = 0; u < kRangeChunk / 256; ++u) {
+        const int i = u * 256 + (int)threadIdx.x;
+        if (i < here) {
+            const float v = dt == MO_F32 ? load_elem<MO_F32>(p, begin + i)
+                            : dt == MO_F16 ? load_elem<MO_F16>(p, begin + i) : load_elem<MO_BF16>(p, begin + i);
+            nan |= v != v;
+            lo = __builtin_fminf(lo, v);   // a NaN operand is ignored: it is carried by the flag
+            hi = __builtin_fmaxf(hi, v);
+        }
+    }
+    __shared__ float slo[4], shi[4];
+    __shared__ int snan[4];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        lo = __builtin_fminf(lo, __shfl_xor(lo, o, kWave));
+        hi = __builtin_fmaxf(hi, __shfl_xor(hi, o, kWave));
+        nan |= (bool)__shfl_xor((int)nan, o, kWave);
+    }
+    if ((threadIdx.x & 63) == 0) {
+        slo[threadIdx.x >> 6] = lo;
+        shi[threadIdx.x >> 6] = hi;
+        snan[threadIdx.x >> 6] = nan;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            lo = __builtin_fminf(lo, slo[w]);
+            hi = __builtin_fmaxf(hi, shi[w]);
+            nan |= snan[w] != 0;
+        }
+        out[3 * blockIdx.x] = lo;
+        out[3 * blockIdx.x + 1] = hi;
+        out[3 * blockIdx.x + 2] = nan ? 1.0f : 0.0f;
+    }
+}
+
 }  // namespace mo
 
 extern "C" int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
@@ -705,5 +769,34 @@ extern "C" int mo_absmax_cols_noalloc(const void* x, int64_t outer, int64_t axis
         default: return MO_ERR_DTYPE;
     }
     if (rc != MO_OK) return rc;
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_value_ranges(const void* const* xs, const int64_t* counts, const int* dtypes, int n,
+                               float* out, int64_t out_chunks, void* stream) {
+    if (n < 0 || out_chunks < 0) return MO_ERR_ARG;
+    if (n == 0) return MO_OK;
+    if (!xs || !counts || !dtypes || !out) return MO_ERR_ARG;
+    if (n > mo::kRangeJobs) return MO_ERR_TOO_LARGE;
+    mo::RangeJobs jobs;
+    int64_t grid = 0;
+    for (int i = 0; i < mo::kRangeJobs; ++i) {
+        if (i < n) {
+            if (counts[i] < 0 || (counts[i] && !xs[i])) return MO_ERR_ARG;
+            if (dtypes[i] < MO_F32 || dtypes[i] > MO_BF16) return MO_ERR_DTYPE;
+            if ((uintptr_t)xs[i] & (dtypes[i] == MO_F32 ? 3u : 1u)) return MO_ERR_UNSUPPORTED;
+        }
+        jobs.ptr[i] = i < n ? xs[i] : nullptr;
+        jobs.count[i] = i < n ? counts[i] : 0;
+        jobs.dtype[i] = i < n ? dtypes[i] : MO_F32;
+        jobs.first[i] = (int)grid;
+        if (i < n) {
+            const int64_t chunks = (counts[i] + mo::kRangeChunk - 1) / mo::kRangeChunk;
+            grid += chunks > 0 ? chunks : 1;   // an empty tensor still owns one (+inf, -inf, 0) entry
+            if (grid > out_chunks) return MO_ERR_TOO_LARGE;
+        }
+    }
+    jobs.first[mo::kRangeJobs] = (int)grid;
+    mo::value_ranges_kernel<<<dim3((unsigned)grid), 256, 0, (hipStream_t)stream>>>(jobs, n, out);
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

@@ -554,6 +554,35 @@ __global__ __launch_bounds__(1024) void awq_scale_grid_kernel(
     }
 }
 
+// The row of the candidate-scale grid whose loss is the first smallest one (what
+// min(dict, key=dict.get) picks on the host: a NaN is never smaller than anything, and a NaN in
+// front is never replaced), its index, and the three tensors the folding makes of it.  Every
+// thread scans the few losses itself; no exchange between workgroups.
+template <int DT>
+__global__ __launch_bounds__(256) void awq_pick_scale_kernel(
+    const double* __restrict__ loss, int n_alpha, const float* __restrict__ scales, int k,
+    int64_t* __restrict__ best, float* __restrict__ best_scale, float* __restrict__ pre_quant_scale,
+    void* __restrict__ pre_quant_scale_t, float* __restrict__ fold) {
+    int b = 0;
+    double lowest = loss[0];
+    for (int i = 1; i < n_alpha; ++i) {
+        const double v = loss[i];
+        if (v < lowest) {
+            lowest = v;
+            b = i;
+        }
+    }
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c == 0 && best) best[0] = b;
+    if (c >= k) return;
+    const float s = scales[(int64_t)b * k + c];
+    const float p = 1.0f / s;
+    if (best_scale) best_scale[c] = s;
+    if (pre_quant_scale) pre_quant_scale[c] = p;
+    if (pre_quant_scale_t) store_elem<DT>(pre_quant_scale_t, c, p);
+    if (fold) fold[c] = 1.0f / p;
+}
+
 }  // namespace mo
 
 #define DISPATCH_DT(dtype, CALL)          \
@@ -745,6 +774,25 @@ extern "C" int mo_awq_scale_grid(const float* x_max, const float* w_max, const f
 #define CALL(DT)                                                                                   \
     mo::awq_scale_grid_kernel<DT><<<(unsigned)n_alpha, threads, 0, st>>>(                          \
         x_max, w_max, exponents, (int)n_alpha, (int)k, scales, w_scales, x_scales)
+    DISPATCH_DT(dtype, CALL)
+#undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_awq_pick_scale(const double* loss, int64_t n_alpha, const float* scales, int64_t k,
+                                 int64_t* best, float* best_scale, float* pre_quant_scale,
+                                 void* pre_quant_scale_t, float* fold, int dtype, void* stream) {
+    if (n_alpha < 0 || k < 0) return MO_ERR_ARG;
+    if (dtype < MO_F32 || dtype > MO_BF16) return MO_ERR_DTYPE;
+    if (n_alpha == 0) return MO_ERR_ARG;   // nothing to pick from
+    if (!loss || (k && !scales)) return MO_ERR_ARG;
+    if (n_alpha > 65535 || k > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned blocks = k ? (unsigned)((k + 255) / 256) : 1u;
+#define CALL(DT)                                                                          \
+    mo::awq_pick_scale_kernel<DT><<<blocks, 256, 0, st>>>(loss, (int)n_alpha, scales, (int)k, best, \
+                                                          best_scale, pre_quant_scale,   \
+                                                          pre_quant_scale_t, fold)
     DISPATCH_DT(dtype, CALL)
 #undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;

@@ -28,6 +28,8 @@ SIGNATURES = {
     "mo_error_string": [_INT],
     "mo_absmax": [_P, _I64, _I64, _I64, _INT, _P, _P],
     "mo_absmax_pair": [_P, _I64, _P, _P, _I64, _P, _INT, _P],
+    "mo_value_ranges": [_P, _P, _P, _INT, _P, _I64, _P],
+    "mo_awq_pick_scale": [_P, _I64, _P, _I64, _P, _P, _P, _P, _P, _INT, _P],
     "mo_absmax_tensor_parts": [_P, _I64, _INT, _P, _P, _I64, _P, _P],
     "mo_absmax_cols_staged": [_P, _I64, _I64, _INT, _P, _P, _I64, _P],
     "mo_absmax_cols_noalloc": [_P, _I64, _I64, _INT, _P, _P],
@@ -223,6 +225,49 @@ def absmax_pair_into(x0: torch.Tensor, acc0: torch.Tensor, x1: torch.Tensor, acc
     call("mo_absmax_pair", x0, _ptr(x0), x0.numel(), _ptr(acc0), _ptr(x1), x1.numel(), _ptr(acc1),
          dtype_code(x0.dtype), _stream(x0))
     return True
+
+
+VALUE_RANGES_MAX = 32          # tensors per mo_value_ranges launch
+VALUE_RANGES_CHUNK = 4096      # elements per workgroup, as in the kernel
+VALUE_RANGES_MAX_CHUNKS = 1024
+_range_out = {}   # device index -> float32 buffer of 3 * VALUE_RANGES_MAX_CHUNKS
+
+
+def value_ranges(tensors):
+    """``[(min, max, has_nan), ...]`` of the given tensors (floats; NaN elements are left out of
+    min and max) from one launch and ONE host synchronisation; None, with nothing launched, when
+    the list is not covered (more than 32 tensors or 4 M elements in all, several devices, another
+    dtype, a non-contiguous tensor)."""
+    n = len(tensors)
+    if n == 0:
+        return []
+    device = tensors[0].device
+    if n > VALUE_RANGES_MAX or device.type != "cuda":
+        return None
+    chunks = []
+    for t in tensors:
+        if t.device != device or t.dtype not in _DTYPES or not t.is_contiguous():
+            return None
+        chunks.append(max(1, -(-t.numel() // VALUE_RANGES_CHUNK)))
+    total = sum(chunks)
+    if total > VALUE_RANGES_MAX_CHUNKS:
+        return None
+    out = _range_out.get(device.index)
+    if out is None:
+        out = _range_out[device.index] = torch.empty(3 * VALUE_RANGES_MAX_CHUNKS, dtype=torch.float32,
+                                                     device=device)
+    ptrs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in tensors])
+    counts = (ctypes.c_int64 * n)(*[t.numel() for t in tensors])
+    dtypes = (ctypes.c_int * n)(*[dtype_code(t.dtype) for t in tensors])
+    call("mo_value_ranges", tensors[0], ptrs, counts, dtypes, n, _ptr(out), VALUE_RANGES_MAX_CHUNKS,
+         _stream(tensors[0]))
+    flat = out[:3 * total].tolist()
+    result, at = [], 0
+    for c in chunks:
+        part = flat[3 * at:3 * (at + c)]
+        result.append((min(part[0::3]), max(part[1::3]), any(part[2::3])))
+        at += c
+    return result
 
 
 _parts_ring = {}   # device index -> [int32 buffer, words handed out]
@@ -585,6 +630,25 @@ def int4_pack_rows(w, ws):
     call("mo_int4_pack_rows", w, _ptr(w), batch, n, k, bs, dtype_code(w.dtype), _ptr(ws), _ptr(out),
          _stream(w))
     return out
+
+
+def awq_pick_scale(loss: torch.Tensor, scales: torch.Tensor, dtype: torch.dtype):
+    """The end of an AWQ-lite search in one launch: ``(best, best_scale, pre_quant_scale,
+    pre_quant_scale_t, fold)`` for float64 ``loss`` [A] and the fp32 candidate grid ``scales``
+    [A, K]: ``best`` the index of the first smallest loss (0-dim int64 on the device; a NaN is
+    never smaller, a NaN in front stays), ``best_scale = scales[best]``, ``pre_quant_scale =
+    1 / best_scale``, the same rounded to ``dtype``, and ``fold = 1 / pre_quant_scale``."""
+    _require_device(loss, scales)
+    assert loss.dtype == torch.float64 and scales.dtype == torch.float32
+    assert loss.is_contiguous() and scales.is_contiguous() and scales.dim() == 2
+    n_alpha, k = scales.shape
+    assert loss.numel() == n_alpha and n_alpha > 0
+    rows = torch.empty(3, k, dtype=torch.float32, device=scales.device)
+    rounded = torch.empty(k, dtype=dtype, device=scales.device)
+    best = torch.empty((), dtype=torch.int64, device=scales.device)
+    call("mo_awq_pick_scale", scales, _ptr(loss), n_alpha, _ptr(scales), k, _ptr(best), _ptr(rows[0]),
+         _ptr(rows[1]), _ptr(rounded), _ptr(rows[2]), dtype_code(dtype), _stream(scales))
+    return best, rows[0], rows[1], rounded, rows[2]
 
 
 def awq_scale_grid(x_max, w_max, exponents, dtype):

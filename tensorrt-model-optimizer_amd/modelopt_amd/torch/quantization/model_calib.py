@@ -182,10 +182,13 @@ def _on_device(t: torch.Tensor, device) -> torch.Tensor:
 
 
 @torch.no_grad()
-def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.Tensor | None = None):
+def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.Tensor | None = None, *,
+                                     _rounded: torch.Tensor | None = None, _fold: torch.Tensor | None = None):
     """Set the input ``pre_quant_scale`` and fold its inverse into the weight.  Inside a
     ``deferred_scale_checks`` block (a caller that loops over many layers) the positivity of the
-    scale is checked when the block ends instead of here (a host synchronisation per layer)."""
+    scale is checked when the block ends instead of here (a host synchronisation per layer).
+    ``_rounded`` and ``_fold``: ``pre_quant_scale`` in the weight's dtype and ``1 / pre_quant_scale``
+    in fp32, for a caller that has them already (bit for bit what is computed here otherwise)."""
     assert is_quantized_linear(linear), "Only quantized linear modules are supported"
     assert linear.input_quantizer.pre_quant_scale is None, "pre_quant_scale should be None first!"
     if pre_quant_scale is None:
@@ -195,8 +198,9 @@ def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.T
     pre_quant_scale = pre_quant_scale.to(torch.float32)  # fp32 keeps the scaling maths safe
 
     linear.input_quantizer._enable_pre_quant_scale = True
-    linear.input_quantizer.pre_quant_scale = pre_quant_scale.to(linear.weight.dtype)
-    _apply_weight_pre_quant_scale(linear, 1.0 / pre_quant_scale)
+    linear.input_quantizer.pre_quant_scale = (_rounded if _rounded is not None
+                                              else pre_quant_scale.to(linear.weight.dtype))
+    _apply_weight_pre_quant_scale(linear, _fold if _fold is not None else 1.0 / pre_quant_scale)
 
     if linear.input_quantizer.amax is not None:
         assert hasattr(linear.input_quantizer, "_amax_for_smoothing")
@@ -727,6 +731,9 @@ def _losses_on_device(helper):
     return total
 
 
+_PICK_IN_ONE_LAUNCH = True   # False: the tensor expressions below instead (kept for tests that compare the two)
+
+
 def _first_minimum(loss):
     """Index (0-dim int64 on the device) that ``min(dict, key=dict.get)`` would pick: the first
     smallest value; a NaN is never smaller than anything, and a NaN in front is never replaced."""
@@ -780,6 +787,7 @@ def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: boo
 
     def postprocess(module, name):
         h = module.awq_lite
+        folded = None   # (1 / best_scale, the same in the weight's dtype, 1 / (1 / best_scale)) when made on the way
         if h.is_enabled:
             loss = _losses_on_device(h)
             if loss is None:
@@ -787,10 +795,16 @@ def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: boo
                 h.best_alpha = min(h.loss, key=h.loss.get)
                 h.best_scale = get_scale(h.act_scale, h.weight_scale, h.best_alpha)
             else:
-                best = _first_minimum(loss)
                 grid = h.scale_grid[0] if h.scale_grid is not None else get_scales(
                     h.act_scale, h.weight_scale, h.alphas, h.exponent_columns)
-                h.best_scale = grid.index_select(0, best.reshape(1))[0]  # the row the search scored
+                if (_PICK_IN_ONE_LAUNCH and loss.is_cuda and loss.dtype == torch.float64
+                        and grid.dtype == torch.float32 and module.weight.dtype in _hip._DTYPES):
+                    # the row the search scored and what the folding makes of it, in one launch
+                    best, h.best_scale, *folded = _hip.awq_pick_scale(
+                        loss.contiguous(), grid.contiguous(), module.weight.dtype)
+                else:
+                    best = _first_minimum(loss)
+                    h.best_scale = grid.index_select(0, best.reshape(1))[0]
                 h.scale_grid = None
                 searched.append((h, loss, best))
         for q in (module.weight_quantizer, module.input_quantizer):
@@ -804,7 +818,10 @@ def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: boo
             module.input_quantizer.amax = act_amax.amax()
             module.input_quantizer.enable()
         if h.is_enabled:
-            apply_pre_quant_scale_and_smooth(module, 1.0 / h.best_scale)
+            if folded:
+                apply_pre_quant_scale_and_smooth(module, folded[0], _rounded=folded[1], _fold=folded[2])
+            else:
+                apply_pre_quant_scale_and_smooth(module, 1.0 / h.best_scale)
         else:
             warnings.warn(f"awq_lite: Disabling for {name}, quantizing with max calibration.")
             max_calibrate(module, lambda module: module.weight_quantizer(module.weight))

@@ -182,6 +182,29 @@ def _read_flags(flag_lists):
     return result
 
 
+def _checked(kinds):
+    """``[ok, ...]`` for ``kinds`` = [(tensors, strictly_positive), ...]: whether every element of
+    every tensor of a kind is finite and non-negative (or positive).  One launch and one host
+    synchronisation for all kinds when the tensors are few and small (the calibrated values of a
+    handful of layers); one reduction per kind and dtype otherwise."""
+    from modelopt_amd import _hip
+
+    lists = [[t.detach() for t in tensors if isinstance(t, torch.Tensor) and not t.is_meta and t.numel()]
+             for tensors, _ in kinds]
+    flat = [t for ts in lists for t in ts]
+    ranges = _hip.value_ranges(flat) if flat else []
+    if ranges is None:
+        return _read_flags([_validity_flags(ts, positive) for ts, (_, positive) in zip(lists, kinds)])
+    result, at = [], 0
+    for ts, (_, positive) in zip(lists, kinds):
+        ok = True
+        for lo, hi, has_nan in ranges[at:at + len(ts)]:
+            ok = ok and not has_nan and (lo > 0 if positive else (lo >= 0 and hi < float("inf")))
+        at += len(ts)
+        result.append(ok)
+    return result
+
+
 @contextlib.contextmanager
 def deferred_scale_checks():
     """Within the block ``all_valid_scales`` and ``all_positive`` only record their tensors and
@@ -202,12 +225,12 @@ def deferred_scale_checks():
         outer.extend(pending)
         outer.positive.extend(pending.positive)
         if pending.report:   # the block's owner wants an answer now
-            pending.report_ok = _read_flags([_validity_flags(pending.report)])[0]
+            pending.report_ok = _checked([(pending.report, False)])[0]
         return
     if not (pending or pending.positive or pending.report):
         return
-    valid, positive, pending.report_ok = _read_flags([
-        _validity_flags(pending), _validity_flags(pending.positive, True), _validity_flags(pending.report)])
+    valid, positive, pending.report_ok = _checked([
+        (pending, False), (pending.positive, True), (pending.report, False)])
     if not valid:
         raise DeferredCheckError("detected negative, inf or nan values in a calibrated amax or scale")
     if not positive:
@@ -220,7 +243,7 @@ def all_valid_scales(tensors) -> bool:
     if _DEFERRED_CHECKS:
         _DEFERRED_CHECKS[-1].extend(t for t in tensors if isinstance(t, torch.Tensor))
         return True
-    return _read_flags([_validity_flags(tensors)])[0]
+    return _checked([(list(tensors), False)])[0]
 
 
 def all_positive(tensor) -> bool:

@@ -136,3 +136,37 @@ def test_pair_rejects_what_it_does_not_cover():
     assert not _hip.absmax_pair_into(a, acc, a.float(), acc2)              # two dtypes
     assert not _hip.absmax_pair_into(a[1:33], acc, a, acc2)                # misaligned
     assert float(acc) == 0 and float(acc2) == 0
+
+
+def test_value_ranges_of_many_small_tensors_in_one_launch():
+    """mo_value_ranges: min, max (NaN elements left out) and a NaN flag per tensor, dtypes mixed."""
+    g = torch.Generator().manual_seed(9)
+    tensors = [torch.randn(5000, generator=g), torch.rand(1, generator=g).reshape(()),
+               torch.randn(4096, generator=g).to(torch.bfloat16), torch.randn(257, generator=g).to(torch.float16),
+               torch.rand(33, 7, generator=g) + 0.5, torch.randn(1000, generator=g),
+               torch.tensor([1.0, float("inf"), 3.0]), torch.tensor([-2.0, float("-inf")]).to(torch.bfloat16),
+               torch.rand(300001, generator=g), torch.rand(131072, generator=g).to(torch.bfloat16),
+               torch.rand(4096, generator=g), torch.rand(4097, generator=g)]
+    tensors[5][123] = float("nan")
+    tensors[8][200000] = -3.0          # in a chunk of its own, far from the ends
+    tensors[9][131071] = float("nan")  # the last element of the last chunk
+    tensors[11][4096] = 7.0            # a chunk of one element
+    got = _hip.value_ranges([t.to(DEV) for t in tensors])
+    assert len(got) == len(tensors)
+    for t, (lo, hi, has_nan) in zip(tensors, got):
+        f = t.float().reshape(-1)
+        keep = f[~torch.isnan(f)]
+        assert has_nan == bool(torch.isnan(f).any())
+        assert lo == float(keep.min()) and hi == float(keep.max()), (t.dtype, lo, hi)
+
+
+def test_value_ranges_leaves_what_it_does_not_cover():
+    a = torch.ones(8, device=DEV)
+    assert _hip.value_ranges([]) == []
+    assert _hip.value_ranges([a] * 33) is None                                  # more than one launch holds
+    assert _hip.value_ranges([a, a.to(torch.int32)]) is None                     # not a float
+    assert _hip.value_ranges([a, torch.ones(8, 8, device=DEV)[:, ::2]]) is None  # not dense
+    assert _hip.value_ranges([a.cpu()]) is None
+    assert _hip.value_ranges([torch.ones(5 << 20, device=DEV)]) is None             # more chunks than the buffer holds
+    assert _hip.value_ranges([torch.ones(0, device=DEV), a]) == [(float("inf"), float("-inf"), False), (1.0, 1.0, False)]
+    assert _hip.value_ranges([a] * 32) == [(1.0, 1.0, False)] * 32

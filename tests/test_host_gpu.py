@@ -705,3 +705,54 @@ def test_awq_lite_selects_the_oracle_s_alpha_on_several_layers(seed, n, k, token
     for a in losses:
         assert h.loss[a] == pytest.approx(losses[a], rel=1e-3), f"alpha {a}"
     assert torch.allclose(h.best_scale.cpu(), best_scale, rtol=2 ** -6)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("losses", [[3.0, 1.0, 2.0, 1.0], [float("nan"), 1.0, 0.5], [2.0, float("nan"), 1.5, float("inf")],
+                                    [float("inf"), float("inf")], [5.0]])
+def test_pick_scale_equals_the_host_s_min_and_the_tensor_expressions(dtype, losses):
+    """mo_awq_pick_scale against ``min(loss, key=loss.get)`` (model_calib.py:633 of the reference)
+    and the eager ``1.0 / best_scale``, ``.to(dtype)``, ``1.0 / pre_quant_scale`` of its folding."""
+    g = torch.Generator().manual_seed(len(losses))
+    k = 1000
+    grid = torch.exp(torch.randn(len(losses), k, generator=g)).to(DEV)
+    table = dict(enumerate(losses))
+    want = min(table, key=table.get)
+    from modelopt_amd import _hip
+
+    loss = torch.tensor(losses, dtype=torch.float64, device=DEV)
+    best, best_scale, pqs, pqs_t, fold = _hip.awq_pick_scale(loss, grid, dtype)
+    assert int(best) == want
+    assert torch.equal(best_scale, grid[want])
+    eager = 1.0 / grid[want]
+    assert torch.equal(pqs, eager) and pqs_t.dtype == dtype
+    assert torch.equal(pqs_t.view(torch.int16 if dtype != torch.float32 else torch.int32),
+                       eager.to(dtype).view(torch.int16 if dtype != torch.float32 else torch.int32))
+    assert torch.equal(fold, 1.0 / eager)
+
+
+def test_deferred_checks_on_the_device_take_one_launch():
+    """Finite / non-negative / positive checks of a block of device tensors: same verdicts from
+    the one-launch reduction as from the tensor expressions, for good and for bad values."""
+    from modelopt_amd import _hip
+    from modelopt_amd.torch.quantization import utils as qutils
+
+    good = [torch.rand(100, device=DEV), torch.rand(7, device=DEV).to(torch.bfloat16), torch.tensor(3.0, device=DEV)]
+    with _hip.KernelTimer() as timer:
+        with qutils.deferred_scale_checks() as checks:
+            assert qutils.all_valid_scales(good)
+            assert qutils.all_positive(good[0] + 1)
+            checks.report = [good[1]]
+    assert checks.report_ok and timer.calls == {"mo_value_ranges": 1}
+    for bad in (torch.tensor([1.0, -1e-3], device=DEV), torch.tensor([float("inf")], device=DEV),
+                torch.tensor([0.5, float("nan")], device=DEV).to(torch.float16)):
+        assert not qutils.all_valid_scales(good + [bad])
+        with pytest.raises(AssertionError, match="negative, inf or nan"):
+            with qutils.deferred_scale_checks():
+                qutils.all_valid_scales(good + [bad])
+    with pytest.raises(AssertionError, match="should be positive"):
+        with qutils.deferred_scale_checks():
+            qutils.all_positive(torch.tensor([1.0, 0.0], device=DEV))
+    with qutils.deferred_scale_checks() as checks:
+        checks.report = [torch.tensor([-1.0], device=DEV)]
+    assert not checks.report_ok
