@@ -148,7 +148,10 @@ def _apply_weight_pre_quant_scale(linear, pre_quant_scale):
     """``W <- dtype(W * s[None, :])`` with an fp32 ``s`` (one product, one rounding), then
     recalibrate the weight amax."""
     if _ENABLE_FOLDING_PQS_TO_WEIGHTS:
-        s = pre_quant_scale.to(linear.weight.device).squeeze().to(torch.float32).contiguous()
+        s = pre_quant_scale
+        if not (s.dtype == torch.float32 and s.dim() == 1 and s.device == linear.weight.device
+                and s.is_contiguous()):
+            s = s.to(linear.weight.device).squeeze().to(torch.float32).contiguous()
         _hip.mul_cols(linear.weight.data, s, out=linear.weight.data)
     else:
         linear.weight_quantizer._enable_pre_quant_scale = True
@@ -570,6 +573,13 @@ def get_scale(x_max, w_max, alpha):
     return get_scales(x_max, w_max, [alpha])[0]
 
 
+@functools.lru_cache(maxsize=16)
+def _alpha_grid(alpha_step: float):
+    """The alphas of the search grid as the reference builds them (model_calib.py:563: the fp32
+    ``torch.arange`` values read back as Python floats), once per step size."""
+    return tuple(k.item() for k in torch.arange(0, 1.0 + alpha_step, alpha_step))
+
+
 class _AWQLiteHelper:
     cache_mode: bool = False
 
@@ -581,7 +591,7 @@ class _AWQLiteHelper:
         self.block_size = _awq_block_size(module.weight, module.weight_quantizer)
         self.weight_scale = get_weight_scale(module.weight, self.block_size)
         dev = module.weight.device
-        self.alphas = [k.item() for k in torch.arange(0, 1.0 + alpha_step, alpha_step)]
+        self.alphas = list(_alpha_grid(float(alpha_step)))
         self.sq_err_steps = []  # per search step: (float64 [n_alphas] sums of squared error, numel)
         self.loss = {a: 0.0 for a in self.alphas}
         self.best_scale = None
@@ -595,8 +605,10 @@ class _AWQLiteHelper:
 
     def setup(self):
         m = self.module
-        m._forward_no_awq = m.forward
-        m.forward = types.MethodType(_awq_forward, m)
+        # plain values: written past nn.Module.__setattr__, which would look through the
+        # parameters, buffers and submodules for each
+        m.__dict__["_forward_no_awq"] = m.forward
+        m.__dict__["forward"] = types.MethodType(_awq_forward, m)
         if m.input_quantizer.is_enabled:
             m.input_quantizer.disable()
             if m.input_quantizer.axis not in (None, -1):
@@ -661,7 +673,7 @@ def _awq_forward(self, input, *args, **kwargs):
     helper = self.awq_lite
     self.weight_quantizer.disable()
     for q in (self.input_quantizer, self.weight_quantizer):
-        if hasattr(q, "_pre_quant_scale"):
+        if "_pre_quant_scale" in q._buffers or "_pre_quant_scale" in q.__dict__:
             delattr(q, "_pre_quant_scale")
     out_actual = self._forward_no_awq(input, *args, **kwargs)
     self.weight_quantizer.enable()
@@ -752,8 +764,8 @@ def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: boo
 
     for name, module in model.named_modules():
         if is_quantized_linear(module) and module.weight_quantizer.is_enabled:
-            module.awq_lite = _AWQLiteHelper(module, name, alpha_step)
-            module.awq_lite.setup()
+            helper = module.__dict__["awq_lite"] = _AWQLiteHelper(module, name, alpha_step)   # a plain attribute
+            helper.setup()
 
     _AWQLiteHelper.cache_mode = True
     print("awq_lite: Caching activation statistics...")
@@ -764,14 +776,19 @@ def awq_lite(model: nn.Module, forward_loop, alpha_step: float = 0.1, debug: boo
 
     cached = []
     for name, module in model.named_modules():
-        if is_quantized_linear(module) and hasattr(module, "awq_lite") and module.awq_lite.num_cache_steps > 0:
-            module._if_calib = True
+        if "awq_lite" in module.__dict__ and is_quantized_linear(module) and module.awq_lite.num_cache_steps > 0:
+            module.__dict__["_if_calib"] = True
             h = module.awq_lite
             h.act_scale = h.act_scale / h.num_cache_steps
             cached.append(h)
     if cached:  # one host synchronisation for the NaN checks of all layers
-        flags = torch.stack([torch.isnan(h.act_scale).any() | torch.isnan(h.weight_scale).any()
-                             for h in cached]).tolist()
+        stats = [t for h in cached for t in (h.act_scale, h.weight_scale)]
+        ranges = _hip.value_ranges(stats) if all(isinstance(t, torch.Tensor) for t in stats) else None
+        if ranges is not None:   # a handful of layers: one launch as well
+            flags = [ranges[2 * i][2] or ranges[2 * i + 1][2] for i in range(len(cached))]
+        else:
+            flags = torch.stack([torch.isnan(h.act_scale).any() | torch.isnan(h.weight_scale).any()
+                                 for h in cached]).tolist()
         for h, bad in zip(cached, flags):
             if bad:
                 h.is_enabled = False

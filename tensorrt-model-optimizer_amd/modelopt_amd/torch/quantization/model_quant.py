@@ -9,6 +9,7 @@ mode registry / state manager (``apply_mode``) is not reproduced.
 import copy
 import fnmatch
 import inspect
+import marshal
 import warnings
 from collections.abc import Callable
 
@@ -46,36 +47,48 @@ def _full_attribute_cfg(cfg):
     raise TypeError(f"unsupported quantizer config entry: {cfg!r}")
 
 
-_VALIDATED = {}   # repr of a plain config -> (validated quant_cfg, algorithm); a handful of entries
+_VALIDATED = {}   # marshalled plain config -> (validated quant_cfg, marshalled algorithm); a handful of entries
 
 
-def _plain(value) -> bool:
-    """Only dicts, lists, tuples and scalars: ``repr`` then says all there is to say about it."""
-    if isinstance(value, dict):
-        return all(isinstance(k, (str, int)) and _plain(v) for k, v in value.items())
-    if isinstance(value, (list, tuple)):
-        return all(_plain(v) for v in value)
-    return value is None or isinstance(value, (bool, int, float, str))
+def _content_key(config):
+    """The content of a config made of plain values only (exact dicts, lists, tuples, strings,
+    numbers, booleans, None -- every named config is) as bytes; None for anything else.
+    ``marshal`` refuses every other type, subclasses of the plain ones included, and keeps the
+    order of a dict's entries, which decides which pattern wins."""
+    try:
+        return marshal.dumps(config)
+    except ValueError:
+        return None
 
 
 def _validated(config):
     """``(quant_cfg with every entry a complete QuantizerAttributeConfig, algorithm)``.  A config
-    made of plain values only (every named config is) is validated once per distinct content:
-    the validated entries are never handed out or written to -- a quantizer copies what it takes
-    from them -- so calls with an equal config can share them."""
-    key = None
-    if isinstance(config, dict) and _plain(config):
-        key = repr(config)
+    made of plain values only is validated once per distinct content: the validated entries are
+    never handed out or written to -- a quantizer copies what it takes from them -- so calls
+    with an equal config can share them."""
+    key = _content_key(config) if type(config) is dict else None
+    if key is not None:
         hit = _VALIDATED.get(key)
         if hit is not None:
-            return dict(hit[0]), copy.deepcopy(hit[1])
+            return dict(hit[0]), marshal.loads(hit[1])
     parsed = config if isinstance(config, QuantizeConfig) else QuantizeConfig(**dict(config))
     quant_cfg = {k: _full_attribute_cfg(v) for k, v in parsed.quant_cfg.items()}
     if key is not None:
-        if len(_VALIDATED) >= 32:
-            _VALIDATED.clear()
-        _VALIDATED[key] = (dict(quant_cfg), copy.deepcopy(parsed.algorithm))
+        algorithm = _content_key(parsed.algorithm)
+        if algorithm is not None:
+            if len(_VALIDATED) >= 32:
+                _VALIDATED.clear()
+            _VALIDATED[key] = (dict(quant_cfg), algorithm)
     return quant_cfg, parsed.algorithm
+
+
+def _takes_no_argument(fn) -> bool:
+    """``len(inspect.signature(fn).parameters) == 0`` without building the signature for a plain
+    function or lambda."""
+    code = getattr(fn, "__code__", None)
+    if code is not None and type(fn).__name__ == "function" and not hasattr(fn, "__wrapped__"):
+        return code.co_argcount + code.co_kwonlyargcount == 0 and not code.co_flags & 0x0C  # no *args / **kwargs
+    return len(inspect.signature(fn).parameters) == 0
 
 
 def calibrate(model: nn.Module, algorithm="max", forward_loop: ForwardLoop | None = None) -> nn.Module:
@@ -84,7 +97,7 @@ def calibrate(model: nn.Module, algorithm="max", forward_loop: ForwardLoop | Non
     method, kwargs = normalize_algorithm(algorithm)
     if method is None:
         return model
-    if forward_loop is not None and len(inspect.signature(forward_loop).parameters) == 0:
+    if forward_loop is not None and _takes_no_argument(forward_loop):
         # the pre-model-argument calling convention (reference: model_quant.py:81-96)
         warnings.warn("forward_loop should take model as argument, but got forward_loop without any"
                       " arguments. This usage will be deprecated in future versions.", DeprecationWarning)

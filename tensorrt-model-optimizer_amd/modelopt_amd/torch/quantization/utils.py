@@ -88,12 +88,24 @@ def is_quantized_linear(module):
     """A module with input/weight quantizers and a 2-D weight (reference: utils.py:222-232)."""
     from .nn import SequentialQuantizer, TensorQuantizer
 
-    return (
-        hasattr(module, "input_quantizer") and hasattr(module, "weight_quantizer")
-        and isinstance(module.input_quantizer, (TensorQuantizer, SequentialQuantizer))
-        and isinstance(module.weight_quantizer, (TensorQuantizer, SequentialQuantizer))
-        and getattr(module, "weight", None) is not None and module.weight.dim() == 2
-    )
+    children = module.__dict__.get("_modules")
+    if children is not None:
+        # quantizers are child modules: looked up where nn.Module keeps them, since asking a
+        # module for an attribute it does not have costs an exception
+        input_quantizer, weight_quantizer = children.get("input_quantizer"), children.get("weight_quantizer")
+        if input_quantizer is None or weight_quantizer is None:
+            if "input_quantizer" not in module.__dict__ and "weight_quantizer" not in module.__dict__:
+                return False
+            input_quantizer = getattr(module, "input_quantizer", None)
+            weight_quantizer = getattr(module, "weight_quantizer", None)
+    else:
+        input_quantizer = getattr(module, "input_quantizer", None)
+        weight_quantizer = getattr(module, "weight_quantizer", None)
+    if not (isinstance(input_quantizer, (TensorQuantizer, SequentialQuantizer))
+            and isinstance(weight_quantizer, (TensorQuantizer, SequentialQuantizer))):
+        return False
+    weight = getattr(module, "weight", None)
+    return weight is not None and weight.dim() == 2
 
 
 class _QuantizerNames:
