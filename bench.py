@@ -349,9 +349,9 @@ def single_tensor_configs(torch, steps, warmup):
         "peak_TFLOPs": 2500.0, "frac": round(kflops / ms / 1e9 / 2500.0, 4)}
 
     # AWQ clip search on the same weight: 11 clip ratios x every 128-wide block, 64 calibration
-    # tokens, one launch.  Vector-ALU bound: per rounded product one fp32 multiply, one
-    # conversion to bf16 (half rate) and one fp32 add, i.e. 4 slots of the fp32 vector unit whose
-    # peak is 157.3 TFLOP/s / 2 = 78.65 T lane-operations a second
+    # tokens, one launch.  Vector-ALU bound: two vector instructions per rounded product (one
+    # fp32 multiply each; one conversion to bf16 and one v_dot2c_f32_bf16 add per pair), against
+    # an issue peak of one instruction per lane and clock: 256 CUs x 64 lanes x 2.4 GHz
     ratios = [round(float(v), 2) for v in torch.arange(0.5, 1.0, 0.05)] + [1.0]
     x64 = x3[::8].contiguous()
     w_amax = w3.view(-1, 128).abs().amax(1, keepdim=True)
@@ -363,7 +363,8 @@ def single_tensor_configs(torch, steps, warmup):
     products = 4096 * 4096 * 64 * (len(ratios) + 1)
     out["awq_clip_search_kernel_11_ratios_4096x4096_64_tokens"] = {
         "ms": round(ms, 4), "rounded_products_per_s": round(products / ms * 1e3, 0), "bound": "valu",
-        "peak_lane_ops_per_s": 78.65e12, "frac": round(4 * products / ms * 1e3 / 78.65e12, 4)}
+        "vector_instructions_per_product": 2.0, "peak_lane_instructions_per_s": 39.32e12,
+        "frac": round(2.0 * products / ms * 1e3 / 39.32e12, 4)}
     cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
     cfg["algorithm"] = {"method": "awq_clip"}
     out["awq_clip_4096x4096_end_to_end_ms"] = round(end_to_end(w3, x3, cfg) * 1e3, 3)

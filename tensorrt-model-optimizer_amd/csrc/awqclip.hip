@@ -11,7 +11,8 @@
 // stays in the lane's registers as fp32; the activations of a token are the same for every
 // lane, so they are read through uniform (scalar) loads and cost the vector ALU nothing.  The
 // org[] values of a lane live in LDS ([token][lane], conflict-free).  VALU-bound: each product
-// is one multiply, one rounding to T (and, for 16-bit T, an unpack) and one add.
+// is one multiply, one rounding to T and one add (bf16: two products share the rounding and the
+// add, see token_dots).
 //
 // A weight with few (row, block) pairs does not fill the chip with one wavefront per 64 pairs
 // (1024 x 4096 in blocks of 128 is 512 wavefronts for 1024 SIMDs, and a lone wavefront on a
@@ -86,11 +87,17 @@ __device__ __forceinline__ void token_dots(const void* __restrict__ x, int64_t x
 #pragma unroll
             for (int j = 0; j < 16; j += 2) {
                 if constexpr (DT == MO_BF16) {
-                    // converting the pair (0, p) leaves bf16(p) in the upper half of the word
-                    // and zero below it: the rounded product as an fp32 bit pattern, with no
-                    // unpacking (shifts and masks run at half the rate of fp32 arithmetic)
-                    acc[j & 3] += u2f(f32x2_to_bf16x2(0.0f, xs[j] * w[16 * g + j]));
-                    acc[(j + 1) & 3] += u2f(f32x2_to_bf16x2(0.0f, xs[j + 1] * w[16 * g + j + 1]));
+                    // both rounded products in one word (one conversion for the pair), added to
+                    // a running sum by one instruction: v_dot2c_f32_bf16(pair, (1, 1), acc) =
+                    // acc + pair.lo + pair.hi.  Four vector instructions per two products where
+                    // multiply, round and add one by one take six.
+                    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+                    const uint32_t pk = f32x2_to_bf16x2(xs[j] * w[16 * g + j], xs[j + 1] * w[16 * g + j + 1]);
+                    const uint32_t one2 = 0x3F803F80u;   // (1.0, 1.0)
+                    bf16x2_t pv, ov;
+                    __builtin_memcpy(&pv, &pk, 4);
+                    __builtin_memcpy(&ov, &one2, 4);
+                    acc[(j / 2) & 3] = __builtin_amdgcn_fdot2_f32_bf16(pv, ov, acc[(j / 2) & 3], false);
                 } else {
                     acc[j & 3] += clip_round<DT>(xs[j] * w[16 * g + j]);
                     acc[(j + 1) & 3] += clip_round<DT>(xs[j + 1] * w[16 * g + j + 1]);
