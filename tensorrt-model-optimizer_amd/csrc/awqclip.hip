@@ -90,7 +90,11 @@ __device__ __forceinline__ void token_dots(const void* __restrict__ x, int64_t x
                     // both rounded products in one word (one conversion for the pair), added to
                     // a running sum by one instruction: v_dot2c_f32_bf16(pair, (1, 1), acc) =
                     // acc + pair.lo + pair.hi.  Four vector instructions per two products where
-                    // multiply, round and add one by one take six.
+                    // multiply, round and add one by one take six.  The instruction's add is
+                    // not a correctly rounded fp32 add (about 2e-6 relative at worst) and it
+                    // flushes bf16 denormals; the sum is rounded to bf16 below, and measured
+                    // against the CPU's arithmetic the losses come out bit-equal as often as
+                    // with exact adds (the difference that shows is the order of the adds).
                     typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
                     const uint32_t pk = f32x2_to_bf16x2(xs[j] * w[16 * g + j], xs[j + 1] * w[16 * g + j + 1]);
                     const uint32_t one2 = 0x3F803F80u;   // (1.0, 1.0)
