@@ -449,6 +449,27 @@ int mo_awq_pick_scale(const double* loss, int64_t n_alpha, const float* scales, 
                       int64_t* best, float* best_scale, float* pre_quant_scale,
                       void* pre_quant_scale_t, float* fold, int dtype, void* stream);
 
+/* SmoothQuant's per-channel scale for one linear and what the smoothing makes of it, in one
+ * launch (postprocess of smoothquant, TQ/model_calib.py:447-473, and
+ * apply_pre_quant_scale_and_smooth, :384-407).  With T the weight dtype, act_amax the fp32
+ * per-channel input amax and weight_col_amax the fp32 per-column abs-max of the weight (k each):
+ *   ws = T(weight_col_amax[c]);  s[c] = f32(T(ws ^ exp_w)) / act_amax[c] ^ exp_a
+ *   if min_c s[c] <= 2^-31: s[c] = 1 where act_amax[c] <= 2^-31;  s[c] = clamp(s[c], 1e-4, 1e4)
+ * (exp_w = 1 - alpha, exp_a = alpha; mode_w / mode_a say how each power is evaluated: 0 powf,
+ * 1 the constant 1, 2 the base, 3 the correctly rounded square root -- the cases torch's scalar
+ * pow evaluates without calling pow; for a 16-bit T and mode_w 0 the caller passes exp_w rounded
+ * to T, which is what the tensor expression raises a 16-bit tensor to).  Outputs:
+ * pre_quant_scale[c] = s[c] (fp32),
+ * pre_quant_scale_t[c] = T(s[c]), fold[c] = 1 / s[c] (what the weight is multiplied by),
+ * act_amax_max = T(max_c act_amax[c]) (the per-tensor input amax), smoothed_amax =
+ * T(max_c f32(T(act_amax[c])) * s[c]) (the input amax after smoothing); all but pre_quant_scale
+ * optional.  NaNs behave as in the tensor expressions: a NaN scale makes the minimum NaN (no
+ * channel is reset) and passes the clamp, a NaN operand makes a maximum NaN. */
+int mo_smooth_scales(const float* act_amax, const float* weight_col_amax, int64_t k,
+                     float exp_w, int mode_w, float exp_a, int mode_a, int dtype,
+                     float* pre_quant_scale, void* pre_quant_scale_t, float* fold,
+                     void* act_amax_max, void* smoothed_amax, void* stream);
+
 /* AWQ-lite search step for a whole grid of alphas in one launch (bf16 only):
  *   q_a = block INT-N quantise-dequantise (blocks of block_size along k, dynamic abs-max) of
  *         bf16(w * s[a]);   out_a = bf16(xs[a] @ q_a^T)   (fp32 accumulation on the matrix cores)

@@ -504,7 +504,9 @@ __device__ __forceinline__ float grid_power(float base, float exponent, int mode
     if (mode == 1) return 1.0f;                      // exponent 0
     if (mode == 2) return base;                      // exponent 1
     if (mode == 3) return __builtin_sqrtf(base);     // exponent 0.5: correctly rounded root
-    return __builtin_powf(base, exponent);
+    // the device math library's pow, the one the tensor library calls: the compiler builtin's
+    // result differs from it in the last place now and then
+    return powf(base, exponent);
 }
 
 template <int DT>
@@ -581,6 +583,78 @@ __global__ __launch_bounds__(256) void awq_pick_scale_kernel(
     if (pre_quant_scale) pre_quant_scale[c] = p;
     if (pre_quant_scale_t) store_elem<DT>(pre_quant_scale_t, c, p);
     if (fold) fold[c] = 1.0f / p;
+}
+
+// SmoothQuant's per-channel scale and everything the smoothing makes of it, one workgroup:
+//   ws = T(w_col[c]);  s[c] = f32(T(ws ^ (1 - alpha))) / act[c] ^ alpha          (fp32 division)
+//   if min_c s[c] <= 2^-31: s[c] = 1 where act[c] <= 2^-31;  s[c] = clamp(s[c], 1e-4, 1e4)
+//   rounded[c] = T(s[c]);  fold[c] = 1 / s[c]
+//   act_max = T(max_c act[c]);  smoothed_max = T(max_c f32(T(act[c])) * s[c])
+// with the NaN behaviour of the tensor expressions: a NaN scale makes the minimum NaN (no channel
+// is reset), passes the clamp, and a NaN operand makes a maximum NaN.
+template <int DT>
+__global__ __launch_bounds__(1024) void smooth_scales_kernel(
+    const float* __restrict__ act, const float* __restrict__ w_col, int k, float exp_w, int mode_w,
+    float exp_a, int mode_a, float* __restrict__ scale, void* __restrict__ rounded,
+    float* __restrict__ fold, void* __restrict__ act_max, void* __restrict__ smoothed_max) {
+    __shared__ float red_a[16], red_b[16];
+    __shared__ int red_nan[16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    auto to_t = [](float v) {
+        if constexpr (DT == MO_BF16) return round_to_bf16(v);
+        else if constexpr (DT == MO_F16) return f16_bits_to_f32(f32_to_f16_bits(v));
+        else return v;
+    };
+    // a = running minimum of the scales, b = running maximum of act; NaNs are carried by flags
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    int nan_s = 0, nan_a = 0;
+    for (int c = threadIdx.x; c < k; c += blockDim.x) {
+        const float a = act[c];
+        const float num = to_t(grid_power(to_t(w_col[c]), exp_w, mode_w));
+        const float v = num / grid_power(a, exp_a, mode_a);
+        scale[c] = v;
+        if (v != v) nan_s = 1; else lo = v < lo ? v : lo;
+        if (a != a) nan_a = 1; else hi = a > hi ? a : hi;
+    }
+    auto meet = [&](float& x, float& y, int& flags, bool x_is_min) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float x2 = __shfl_xor(x, o, kWave), y2 = __shfl_xor(y, o, kWave);
+            x = x_is_min ? (x2 < x ? x2 : x) : (x2 > x ? x2 : x);
+            y = y2 > y ? y2 : y;
+            flags |= __shfl_xor(flags, o, kWave);
+        }
+        __syncthreads();   // the arrays may still be read from the meeting before
+        if (lane == 0) { red_a[wave] = x; red_b[wave] = y; red_nan[wave] = flags; }
+        __syncthreads();
+        for (int w = 0; w < waves; ++w) {
+            x = x_is_min ? (red_a[w] < x ? red_a[w] : x) : (red_a[w] > x ? red_a[w] : x);
+            y = red_b[w] > y ? red_b[w] : y;
+            flags |= red_nan[w];
+        }
+    };
+    int flags = nan_s | (nan_a << 1);
+    meet(lo, hi, flags, true);
+    const bool reset_dead = !(flags & 1) && lo <= 4.656612873077393e-10f;   // 2^-31
+    if (threadIdx.x == 0 && act_max)
+        store_elem<DT>(act_max, 0, (flags & 2) ? __builtin_nanf("") : hi);
+    float top = -__builtin_inff(), unused = 0.0f;
+    int nan_p = 0;
+    for (int c = threadIdx.x; c < k; c += blockDim.x) {
+        const float a = act[c];
+        float v = scale[c];   // each lane re-reads what it wrote itself
+        if (reset_dead && a <= 4.656612873077393e-10f) v = 1.0f;
+        v = v < 1e-4f ? 1e-4f : v;
+        v = v > 1e4f ? 1e4f : v;
+        scale[c] = v;
+        if (rounded) store_elem<DT>(rounded, c, v);
+        if (fold) fold[c] = 1.0f / v;
+        const float p = to_t(a) * v;
+        if (p != p) nan_p = 1; else top = p > top ? p : top;
+    }
+    meet(top, unused, nan_p, false);
+    if (threadIdx.x == 0 && smoothed_max)
+        store_elem<DT>(smoothed_max, 0, nan_p ? __builtin_nanf("") : top);
 }
 
 }  // namespace mo
@@ -793,6 +867,26 @@ extern "C" int mo_awq_pick_scale(const double* loss, int64_t n_alpha, const floa
     mo::awq_pick_scale_kernel<DT><<<blocks, 256, 0, st>>>(loss, (int)n_alpha, scales, (int)k, best, \
                                                           best_scale, pre_quant_scale,   \
                                                           pre_quant_scale_t, fold)
+    DISPATCH_DT(dtype, CALL)
+#undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_smooth_scales(const float* act_amax, const float* weight_col_amax, int64_t k,
+                                float exp_w, int mode_w, float exp_a, int mode_a, int dtype,
+                                float* pre_quant_scale, void* pre_quant_scale_t, float* fold,
+                                void* act_amax_max, void* smoothed_amax, void* stream) {
+    if (k < 0 || mode_w < 0 || mode_w > 3 || mode_a < 0 || mode_a > 3) return MO_ERR_ARG;
+    if (dtype < MO_F32 || dtype > MO_BF16) return MO_ERR_DTYPE;
+    if (k == 0) return MO_ERR_ARG;   // a maximum over nothing
+    if (!act_amax || !weight_col_amax || !pre_quant_scale) return MO_ERR_ARG;
+    if (k > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    const int threads = k >= 4096 ? 1024 : 256;
+#define CALL(DT)                                                                                    \
+    mo::smooth_scales_kernel<DT><<<1, threads, 0, st>>>(act_amax, weight_col_amax, (int)k, exp_w, mode_w, \
+                                                        exp_a, mode_a, pre_quant_scale, pre_quant_scale_t, \
+                                                        fold, act_amax_max, smoothed_amax)
     DISPATCH_DT(dtype, CALL)
 #undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;

@@ -30,6 +30,7 @@ SIGNATURES = {
     "mo_absmax_pair": [_P, _I64, _P, _P, _I64, _P, _INT, _P],
     "mo_value_ranges": [_P, _P, _P, _INT, _P, _I64, _P],
     "mo_awq_pick_scale": [_P, _I64, _P, _I64, _P, _P, _P, _P, _P, _INT, _P],
+    "mo_smooth_scales": [_P, _P, _I64, ctypes.c_float, _INT, ctypes.c_float, _INT, _INT, _P, _P, _P, _P, _P, _P],
     "mo_absmax_tensor_parts": [_P, _I64, _INT, _P, _P, _I64, _P, _P],
     "mo_absmax_cols_staged": [_P, _I64, _I64, _INT, _P, _P, _I64, _P],
     "mo_absmax_cols_noalloc": [_P, _I64, _I64, _INT, _P, _P],
@@ -649,6 +650,36 @@ def awq_pick_scale(loss: torch.Tensor, scales: torch.Tensor, dtype: torch.dtype)
     call("mo_awq_pick_scale", scales, _ptr(loss), n_alpha, _ptr(scales), k, _ptr(best), _ptr(rows[0]),
          _ptr(rows[1]), _ptr(rounded), _ptr(rows[2]), dtype_code(dtype), _stream(scales))
     return best, rows[0], rows[1], rounded, rows[2]
+
+
+def _power_mode(exponent: float) -> int:
+    """How a scalar power is evaluated: 0 ``pow``, 1 the constant one (exponent 0), 2 the base
+    (exponent 1), 3 the correctly rounded square root (exponent 0.5)."""
+    return {0.0: 1, 1.0: 2, 0.5: 3}.get(float(exponent), 0)
+
+
+def smooth_scales(act_amax: torch.Tensor, weight_col_amax: torch.Tensor, alpha: float, dtype: torch.dtype):
+    """SmoothQuant's scale of one linear and what the smoothing makes of it, in one launch:
+    ``(pre_quant_scale fp32 [K], the same in dtype, 1 / pre_quant_scale fp32, dtype(max act_amax),
+    dtype(max(dtype(act_amax) * pre_quant_scale)))`` from the fp32 per-channel input amax and the
+    fp32 per-column abs-max of the weight."""
+    _require_device(act_amax, weight_col_amax)
+    assert act_amax.dtype == torch.float32 and weight_col_amax.dtype == torch.float32
+    assert act_amax.is_contiguous() and weight_col_amax.is_contiguous()
+    k = act_amax.numel()
+    assert weight_col_amax.numel() == k and k > 0
+    rows = torch.empty(2, k, dtype=torch.float32, device=act_amax.device)
+    rounded = torch.empty(k, dtype=dtype, device=act_amax.device)
+    maxima = torch.empty(2, dtype=dtype, device=act_amax.device)
+    exp_w, exp_a = 1 - alpha, alpha
+    mode_w = _power_mode(exp_w)
+    if mode_w == 0 and dtype != torch.float32:
+        # a power of a 16-bit tensor is taken with the exponent rounded to that dtype
+        exp_w = float(torch.tensor(exp_w, dtype=dtype))
+    call("mo_smooth_scales", act_amax, _ptr(act_amax), _ptr(weight_col_amax), k, exp_w, mode_w,
+         exp_a, _power_mode(exp_a), dtype_code(dtype), _ptr(rows[0]), _ptr(rounded), _ptr(rows[1]),
+         _ptr(maxima[0]), _ptr(maxima[1]), _stream(act_amax))
+    return rows[0], rounded, rows[1], maxima[0], maxima[1]
 
 
 def awq_scale_grid(x_max, w_max, exponents, dtype):

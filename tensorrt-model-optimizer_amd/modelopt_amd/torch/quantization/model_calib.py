@@ -186,12 +186,14 @@ def _on_device(t: torch.Tensor, device) -> torch.Tensor:
 
 @torch.no_grad()
 def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.Tensor | None = None, *,
-                                     _rounded: torch.Tensor | None = None, _fold: torch.Tensor | None = None):
+                                     _rounded: torch.Tensor | None = None, _fold: torch.Tensor | None = None,
+                                     _smoothed_amax: torch.Tensor | None = None):
     """Set the input ``pre_quant_scale`` and fold its inverse into the weight.  Inside a
     ``deferred_scale_checks`` block (a caller that loops over many layers) the positivity of the
     scale is checked when the block ends instead of here (a host synchronisation per layer).
     ``_rounded`` and ``_fold``: ``pre_quant_scale`` in the weight's dtype and ``1 / pre_quant_scale``
-    in fp32, for a caller that has them already (bit for bit what is computed here otherwise)."""
+    in fp32, ``_smoothed_amax``: the input amax after smoothing, for a caller that has them
+    already (bit for bit what is computed here otherwise)."""
     assert is_quantized_linear(linear), "Only quantized linear modules are supported"
     assert linear.input_quantizer.pre_quant_scale is None, "pre_quant_scale should be None first!"
     if pre_quant_scale is None:
@@ -205,7 +207,10 @@ def apply_pre_quant_scale_and_smooth(linear: nn.Module, pre_quant_scale: torch.T
                                               else pre_quant_scale.to(linear.weight.dtype))
     _apply_weight_pre_quant_scale(linear, _fold if _fold is not None else 1.0 / pre_quant_scale)
 
-    if linear.input_quantizer.amax is not None:
+    if linear.input_quantizer.amax is not None and _smoothed_amax is not None:
+        assert hasattr(linear.input_quantizer, "_amax_for_smoothing")
+        linear.input_quantizer.amax = _smoothed_amax
+    elif linear.input_quantizer.amax is not None:
         assert hasattr(linear.input_quantizer, "_amax_for_smoothing")
         device, dtype = linear.weight.device, linear.weight.dtype
         smoothing = _on_device(linear.input_quantizer._amax_for_smoothing, device).to(dtype)
@@ -264,6 +269,18 @@ def smoothquant(model: nn.Module, forward_loop=None, alpha=1.0):
         device, dtype = w.device, w.dtype
         col = torch.zeros(w.shape[1], dtype=torch.float32, device=device)
         _hip.absmax_into(w.data.contiguous(), col, w.shape[0], w.shape[1], 1)
+        if (_SMOOTH_IN_ONE_LAUNCH and w.is_cuda and dtype in _hip._DTYPES and act_amax.device == device
+                and act_amax.numel() == col.numel()):
+            # the scale, its rounded copy, its inverse and both input amax values from one launch
+            # (some twenty tensor operations otherwise, each a launch behind the layer's GEMM)
+            pqs, pqs_t, fold, act_max, smoothed = _hip.smooth_scales(
+                act_amax.contiguous().view(-1), col, float(alpha), dtype)
+            module.input_quantizer._amax_for_smoothing = _host_copy_later(act_amax)
+            module.input_quantizer.reset_amax()
+            module.input_quantizer.axis = None
+            module.input_quantizer.amax = act_max
+            apply_pre_quant_scale_and_smooth(module, pqs, _rounded=pqs_t, _fold=fold, _smoothed_amax=smoothed)
+            return
         weight_scale = col.to(dtype).reshape(1, -1)  # == w.abs().amax(dim=0, keepdim=True)
         # the 16-bit numerator is widened by hand: the same values as type promotion gives, but a
         # binary operation on two dtypes goes through the tensor library's casting kernel,
@@ -748,6 +765,7 @@ def _losses_on_device(helper):
     return total
 
 
+_SMOOTH_IN_ONE_LAUNCH = True   # False: the tensor expressions of smoothquant's postprocess instead
 _PICK_IN_ONE_LAUNCH = True   # False: the tensor expressions below instead (kept for tests that compare the two)
 
 

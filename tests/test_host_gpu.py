@@ -756,3 +756,47 @@ def test_deferred_checks_on_the_device_take_one_launch():
     with qutils.deferred_scale_checks() as checks:
         checks.report = [torch.tensor([-1.0], device=DEV)]
     assert not checks.report_ok
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("alpha", [0.5, 0.3, 1.0, 0.0])
+@pytest.mark.parametrize("case", ["plain", "dead channels", "nan"])
+def test_smoothquant_in_one_launch_equals_the_tensor_expressions(dtype, alpha, case, monkeypatch):
+    """mo_smooth_scales against the eager postprocess of smoothquant (model_calib.py:447-473 and
+    384-407 of the reference): pre-quant scale, input amax and folded weight bit for bit, for the
+    exponents the scalar pow special-cases and one it does not, with channels that never fired
+    (their scale is reset to 1) and with a NaN in the statistics."""
+    from modelopt_amd.torch.quantization import model_calib
+
+    g = torch.Generator().manual_seed(int(alpha * 10) + len(case))
+    k, n = 512, 256
+    w = (0.05 * torch.randn(n, k, generator=g)).to(dtype)
+    x = (torch.randn(64, k, generator=g) * torch.exp(torch.randn(k, generator=g))).to(dtype)
+    if case != "plain":
+        x[:, 5] = 0
+        x[:, 77] = 0
+        w[:, 9] = 0
+    if case == "nan":
+        x[3, 100] = float("nan")
+
+    def run(one_launch):
+        monkeypatch.setattr(model_calib, "_SMOOTH_IN_ONE_LAUNCH", one_launch)
+        model = nn.Sequential(nn.Linear(k, n, bias=False)).to(dtype).to(DEV)
+        model[0].weight.data.copy_(w)
+        cfg = copy.deepcopy(mtq.INT8_SMOOTHQUANT_CFG)
+        cfg["algorithm"] = {"method": "smoothquant", "alpha": alpha}
+        try:
+            mtq.quantize(model, cfg, lambda m: m(x.to(DEV)))
+        except AssertionError as e:   # the deferred checks refuse a NaN scale either way
+            return str(e)
+        q = model[0].input_quantizer
+        return (q.pre_quant_scale.clone(), q.amax.clone(), model[0].weight.data.clone(),
+                model[0].weight_quantizer.amax.clone(), q._amax_for_smoothing.clone())
+
+    eager, fused = run(False), run(True)
+    if isinstance(eager, str):
+        assert eager == fused
+        return
+    for a, b in zip(eager, fused):
+        assert a.dtype == b.dtype and a.shape == b.shape
+        assert_bits_equal(a.cpu(), b.cpu(), f"{dtype} alpha {alpha} {case}")
