@@ -88,13 +88,14 @@ def is_quantized_linear(module):
     """A module with input/weight quantizers and a 2-D weight (reference: utils.py:222-232)."""
     from .nn import SequentialQuantizer, TensorQuantizer
 
-    children = module.__dict__.get("_modules")
+    children = getattr(module, "__dict__", {}).get("_modules")
     if children is not None:
         # quantizers are child modules: looked up where nn.Module keeps them, since asking a
         # module for an attribute it does not have costs an exception
         input_quantizer, weight_quantizer = children.get("input_quantizer"), children.get("weight_quantizer")
         if input_quantizer is None or weight_quantizer is None:
-            if "input_quantizer" not in module.__dict__ and "weight_quantizer" not in module.__dict__:
+            if "input_quantizer" not in module.__dict__ and "weight_quantizer" not in module.__dict__ \
+                    and not hasattr(type(module), "input_quantizer"):
                 return False
             input_quantizer = getattr(module, "input_quantizer", None)
             weight_quantizer = getattr(module, "weight_quantizer", None)

@@ -768,3 +768,82 @@ def test_default_max_calibrator_reports_a_bad_batch_in_compute_amax(oracle_backe
     cal.collect(torch.tensor([2.0]))
     with pytest.raises(AssertionError, match="detected inf values in amax"):
         cal.compute_amax()
+
+
+def test_forward_loop_argument_count_matches_inspect():
+    """The shortcut for plain functions and lambdas gives what inspect.signature gives, and
+    everything else goes through inspect.signature."""
+    import functools
+    import inspect
+
+    from modelopt_amd.torch.quantization.model_quant import _takes_no_argument
+
+    class Callable_:
+        def __call__(self):
+            return None
+
+        def method(self):
+            return None
+
+    def wrapped_inner(model):
+        return None
+
+    @functools.wraps(wrapped_inner)
+    def wrapper():
+        return wrapped_inner(None)
+
+    def star(*args):
+        return None
+
+    def keyword_only(*, model=None):
+        return None
+
+    cases = [lambda: None, lambda m: None, lambda m=None: None, star, keyword_only, Callable_(),
+             Callable_().method, functools.partial(wrapped_inner, None), wrapper, len.__call__]
+    for fn in cases:
+        assert _takes_no_argument(fn) == (len(inspect.signature(fn).parameters) == 0), fn
+
+
+def test_validated_config_is_kept_by_content_for_plain_configs_only():
+    import enum
+
+    from modelopt_amd.torch.quantization import model_quant
+
+    cfg = {"quant_cfg": {"*weight_quantizer": {"num_bits": 4, "block_sizes": {-1: 32}, "enable": True},
+                         "default": {"enable": False}}, "algorithm": {"method": "max"}}
+    model_quant._VALIDATED.clear()
+    first, algo = model_quant._validated(cfg)
+    assert len(model_quant._VALIDATED) == 1
+    second, algo2 = model_quant._validated(copy.deepcopy(cfg))
+    assert len(model_quant._VALIDATED) == 1 and algo == algo2 and algo is not algo2
+    assert second["*weight_quantizer"] is first["*weight_quantizer"]      # shared, never written to
+    # another order of the patterns is another config: later entries win
+    swapped = {"quant_cfg": dict(reversed(list(cfg["quant_cfg"].items()))), "algorithm": {"method": "max"}}
+    model_quant._validated(swapped)
+    assert len(model_quant._VALIDATED) == 2
+
+    class Bits(enum.IntEnum):
+        FOUR = 4
+
+    odd = copy.deepcopy(cfg)
+    odd["quant_cfg"]["*weight_quantizer"]["num_bits"] = Bits.FOUR          # not a plain value
+    assert model_quant._content_key(odd) is None
+    model_quant._validated(odd)
+    assert len(model_quant._VALIDATED) == 2
+
+
+def test_is_quantized_linear_on_modules_and_other_objects():
+    from modelopt_amd.torch.quantization.utils import is_quantized_linear
+
+    lin = nn.Linear(8, 8)
+    assert not is_quantized_linear(lin) and not is_quantized_linear(object()) and not is_quantized_linear(3)
+    mtq.replace_quant_module(seq := nn.Sequential(lin))
+    assert is_quantized_linear(seq[0]) and not is_quantized_linear(seq)
+    conv = nn.Sequential(nn.Conv2d(3, 3, 1))
+    mtq.replace_quant_module(conv)
+    assert not is_quantized_linear(conv[0])                                 # a 4-D weight
+    plain = nn.Module()                                                     # quantizers as plain attributes
+    plain.__dict__["input_quantizer"] = seq[0].input_quantizer
+    plain.__dict__["weight_quantizer"] = seq[0].weight_quantizer
+    plain.weight = nn.Parameter(torch.zeros(4, 4))
+    assert is_quantized_linear(plain)
