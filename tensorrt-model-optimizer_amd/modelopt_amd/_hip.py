@@ -231,7 +231,6 @@ def absmax_pair_into(x0: torch.Tensor, acc0: torch.Tensor, x1: torch.Tensor, acc
 VALUE_RANGES_MAX = 32          # tensors per mo_value_ranges launch
 VALUE_RANGES_CHUNK = 4096      # elements per workgroup, as in the kernel
 VALUE_RANGES_MAX_CHUNKS = 1024
-_range_out = {}   # device index -> float32 buffer of 3 * VALUE_RANGES_MAX_CHUNKS
 
 
 def value_ranges(tensors):
@@ -253,16 +252,14 @@ def value_ranges(tensors):
     total = sum(chunks)
     if total > VALUE_RANGES_MAX_CHUNKS:
         return None
-    out = _range_out.get(device.index)
-    if out is None:
-        out = _range_out[device.index] = torch.empty(3 * VALUE_RANGES_MAX_CHUNKS, dtype=torch.float32,
-                                                     device=device)
+    # a buffer of its own per call (the caching allocator hands it out in microseconds): calls from
+    # two streams must not share one
+    out = torch.empty(3 * total, dtype=torch.float32, device=device)
     ptrs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in tensors])
     counts = (ctypes.c_int64 * n)(*[t.numel() for t in tensors])
     dtypes = (ctypes.c_int * n)(*[dtype_code(t.dtype) for t in tensors])
-    call("mo_value_ranges", tensors[0], ptrs, counts, dtypes, n, _ptr(out), VALUE_RANGES_MAX_CHUNKS,
-         _stream(tensors[0]))
-    flat = out[:3 * total].tolist()
+    call("mo_value_ranges", tensors[0], ptrs, counts, dtypes, n, _ptr(out), total, _stream(tensors[0]))
+    flat = out.tolist()
     result, at = [], 0
     for c in chunks:
         part = flat[3 * at:3 * (at + c)]
