@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmodelopt_hip.so")
-PROBE_SRC = os.path.join(CSRC, "probe", "l2_read_probe.hip")   # measurement aid for bench.py, its own library
+PROBE_SRC = os.path.join(HERE, "probe", "l2_read_probe.hip")   # measurement aid for bench.py: its own library, outside csrc/
 PROBE_LIB = os.path.join(HERE, "libmodelopt_probe.so")
 HEADERS = [os.path.join(CSRC, h) for h in ("common.h", "qdq_ops.h", "awq_ops.h")] + [
     os.path.join(HERE, "..", "include", "modelopt_hip.h")]

@@ -35,8 +35,11 @@ __all__ = ["export_hf_checkpoint", "convert_hf_quant_config_format",
 
 
 def _register_input_scale(module, input_quantizer):
-    if (input_quantizer is not None and "disabled" not in repr(input_quantizer)
-            and input_quantizer.amax is not None):
+    # the reference asks `"disabled" not in repr(input_quantizer)`; a TensorQuantizer prints that word
+    # exactly when it is disabled, and formatting the amax for the repr would wait for the device
+    enabled = (not input_quantizer._disabled if isinstance(input_quantizer, TensorQuantizer)
+               else "disabled" not in repr(input_quantizer)) if input_quantizer is not None else False
+    if enabled and input_quantizer.amax is not None:
         module.register_buffer("input_scale", get_activation_scaling_factor(module).squeeze())
 
 
