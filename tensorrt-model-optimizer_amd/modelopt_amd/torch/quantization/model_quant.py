@@ -6,7 +6,6 @@ swap + quantizer attributes) and runs the configured calibration algorithm; the 
 mode registry / state manager (``apply_mode``) is not reproduced.
 """
 
-import copy
 import fnmatch
 import inspect
 import marshal
@@ -19,7 +18,7 @@ from torch import nn
 from . import model_calib
 from .config import QuantizeConfig, QuantizerAttributeConfig, normalize_algorithm
 from .conversion import is_converted, replace_quant_module, set_quantizer_attribute, set_quantizer_by_cfg
-from .nn import SequentialQuantizer, TensorQuantizer
+from .nn import TensorQuantizer
 from .utils import DeferredCheckError, deferred_scale_checks
 
 __all__ = ["quantize", "calibrate", "disable_quantizer", "enable_quantizer", "print_quant_summary",
