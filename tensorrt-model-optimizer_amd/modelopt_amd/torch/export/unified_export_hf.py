@@ -7,7 +7,6 @@ packed in ONE multi-tensor kernel launch over the whole model instead of module 
 """
 
 import json
-import os
 import warnings
 from pathlib import Path
 from typing import Any
