@@ -248,6 +248,24 @@ def single_tensor_configs(torch, steps, warmup):
     out["c1_fp8_amax_plus_qdq_4096x4096"] = {"ms": round(ms, 4), "GBps": round(w.numel() * 6 / ms / 1e6, 1)}
     # the same in one launch that reads the tensor once (4 B / element): every workgroup keeps its
     # share in registers while the workgroups agree on the abs-max
+    # a dynamic quantizer: the abs-max of this very call, then the fake quant of the same tensor,
+    # on 32 different tensors in turn (1 GiB: none of them is in a cache when its turn comes).
+    # With the hint the reduction uses plain loads and leaves the tensor in the memory-side cache
+    # for the fake quant; without it, streaming loads as in a calibration pass.
+    many = [torch.randn(4096, 4096, device=dev).to(torch.bfloat16) for _ in range(32)]
+    turn = [0]
+
+    def c1_dynamic(reread):
+        x = many[turn[0] % len(many)]
+        turn[0] += 1
+        _hip.absmax_into(x, acc, 1, 1, x.numel(), reread=reread)
+        _hip.fp8_qdq(x, acc.reshape(()), 1, 1, x.numel(), out=y)
+    ms_hint, ms_stream = train(lambda: c1_dynamic(True), reps=128), train(lambda: c1_dynamic(False), reps=128)
+    out["c1_fp8_dynamic_amax_plus_qdq_4096x4096_cold_inputs"] = {
+        "ms": round(ms_hint, 4), "GBps": round(w.numel() * 6 / ms_hint / 1e6, 1),
+        "ms_with_streaming_loads_in_the_reduction": round(ms_stream, 4)}
+    del many
+
     def c1_fused():
         assert _hip.fused_amax_qdq(w, "fp8", out=y) is not None
     ms = train(c1_fused)

@@ -11,17 +11,28 @@
 namespace mo {
 
 // Running max state of one lane.  16-bit inputs keep two packed 15-bit magnitudes per word.
-template <int DT> struct AbsAcc {
+// KEEP: plain loads instead of streaming ones, for a caller that reads the tensor again right
+// away (the fake quant of a dynamic quantizer: MO_ABSMAX_REREAD).  The streaming hint takes the
+// lines out of the memory-side cache under that second reader's feet: with plain loads abs-max
+// + FP8 fake quant of a 33 MB tensor goes from 22.7 to 20.6 us and of a 134 MB one from 66 to
+// 62 us (inputs that were not in any cache before).  The reduction itself is about 12 % slower
+// that way, so passes nobody follows up on (calibration, the multi-tensor pass over a whole
+// model's weights) keep the streaming loads.
+template <int DT, bool KEEP = false> struct AbsAcc {
     uint32_t m = 0;
+    static __device__ __forceinline__ u32x4 load(const u32x4* q) {
+        if constexpr (KEEP) return *q;
+        else return __builtin_nontemporal_load(q);
+    }
     __device__ __forceinline__ void chunk(const void* p, int64_t i) {
         if constexpr (DT == MO_F32) {
             const u32x4* q = (const u32x4*)((const float*)p + i);
-            u32x4 a = __builtin_nontemporal_load(q), b = __builtin_nontemporal_load(q + 1);
+            u32x4 a = load(q), b = load(q + 1);
             uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
             for (int j = 0; j < 8; ++j) { uint32_t t = w[j] & 0x7FFFFFFFu; m = t > m ? t : m; }
         } else {
-            u32x4 a = __builtin_nontemporal_load((const u32x4*)((const uint16_t*)p + i));
+            u32x4 a = load((const u32x4*)((const uint16_t*)p + i));
             uint32_t t = pk_max_u16(pk_max_u16(a.x & 0x7FFF7FFFu, a.y & 0x7FFF7FFFu),
                                     pk_max_u16(a.z & 0x7FFF7FFFu, a.w & 0x7FFF7FFFu));
             m = pk_max_u16(m, t);
@@ -73,12 +84,12 @@ __device__ __forceinline__ void fold_max_coherent(uint32_t* acc, uint32_t v) {
 
 // ------------------------------------------------------------------------------ per tensor
 // One workgroup per tile of TILE_ELEMS elements, dispatched in order.
-template <int DT, int TILE_ELEMS>
+template <int DT, int TILE_ELEMS, bool KEEP = false>
 __device__ __forceinline__ void absmax_flat_tile(const void* __restrict__ x, int64_t n, int64_t tile,
                                                  uint32_t* __restrict__ acc,
                                                  uint32_t* __restrict__ parts, uint32_t* smem) {
     constexpr int64_t kTileChunks = TILE_ELEMS / 8;
-    AbsAcc<DT> a;
+    AbsAcc<DT, KEEP> a;
     const int64_t chunks = n >> 3;
     const int64_t c0 = tile * kTileChunks;
     int64_t c1 = c0 + kTileChunks;
@@ -99,12 +110,12 @@ __device__ __forceinline__ void absmax_flat_tile(const void* __restrict__ x, int
     }
 }
 
-template <int DT, int TILE_ELEMS>
+template <int DT, int TILE_ELEMS, bool KEEP = false>
 __global__ __launch_bounds__(256) void absmax_flat_kernel(const void* __restrict__ x, int64_t n,
                                                           uint32_t* __restrict__ acc,
                                                           uint32_t* __restrict__ parts = nullptr) {
     __shared__ uint32_t smem[4];
-    absmax_flat_tile<DT, TILE_ELEMS>(x, n, blockIdx.x, acc, parts, smem);
+    absmax_flat_tile<DT, TILE_ELEMS, KEEP>(x, n, blockIdx.x, acc, parts, smem);
 }
 
 // Two tensors, each into its own accumulator, in one launch: workgroups [0, tiles0) take the
@@ -423,7 +434,7 @@ __global__ __launch_bounds__(256) void absmax_multi_kernel(const mo_absmax_job* 
 
 template <int DT>
 static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, uint32_t* acc,
-                         hipStream_t s) {
+                         hipStream_t s, bool keep = false) {
     const bool base_ok = ((uintptr_t)x & 15u) == 0;
     if (axis == 1) {  // per tensor
         const int64_t n = outer * inner;
@@ -436,7 +447,8 @@ static int launch_absmax(const void* x, int64_t outer, int64_t axis, int64_t inn
             const int64_t tiles = (n + tile - 1) / tile;
             if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
             const size_t cap = mo::ballast_bytes("absmax_flat_kernel", 36);
-            if (tile == 8192) absmax_flat_kernel<DT, 8192><<<dim3((unsigned)tiles), 256, cap, s>>>(x, n, acc);
+            if (keep) absmax_flat_kernel<DT, 32768, true><<<dim3((unsigned)((n + 32767) / 32768)), 256, cap, s>>>(x, n, acc);
+            else if (tile == 8192) absmax_flat_kernel<DT, 8192><<<dim3((unsigned)tiles), 256, cap, s>>>(x, n, acc);
             else if (tile == 16384) absmax_flat_kernel<DT, 16384><<<dim3((unsigned)tiles), 256, cap, s>>>(x, n, acc);
             else absmax_flat_kernel<DT, 32768><<<dim3((unsigned)tiles), 256, cap, s>>>(x, n, acc);
             return MO_OK;
@@ -651,21 +663,27 @@ __global__ __launch_bounds__(256) void value_ranges_kernel(RangeJobs jobs, int n
 
 }  // namespace mo
 
-extern "C" int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
-                         float* acc, void* stream) {
-    if (outer < 0 || axis < 0 || inner < 0) return MO_ERR_ARG;
+extern "C" int mo_absmax_hinted(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
+                                float* acc, unsigned hints, void* stream) {
+    if (outer < 0 || axis < 0 || inner < 0 || (hints & ~(unsigned)MO_ABSMAX_REREAD)) return MO_ERR_ARG;
     if (outer == 0 || axis == 0 || inner == 0) return MO_OK;
     if (!x || !acc) return MO_ERR_ARG;
     hipStream_t s = (hipStream_t)stream;
+    const bool keep = (hints & MO_ABSMAX_REREAD) != 0;
     int rc;
     switch (dtype) {
-        case MO_F32: rc = mo::launch_absmax<MO_F32>(x, outer, axis, inner, (uint32_t*)acc, s); break;
-        case MO_F16: rc = mo::launch_absmax<MO_F16>(x, outer, axis, inner, (uint32_t*)acc, s); break;
-        case MO_BF16: rc = mo::launch_absmax<MO_BF16>(x, outer, axis, inner, (uint32_t*)acc, s); break;
+        case MO_F32: rc = mo::launch_absmax<MO_F32>(x, outer, axis, inner, (uint32_t*)acc, s, keep); break;
+        case MO_F16: rc = mo::launch_absmax<MO_F16>(x, outer, axis, inner, (uint32_t*)acc, s, keep); break;
+        case MO_BF16: rc = mo::launch_absmax<MO_BF16>(x, outer, axis, inner, (uint32_t*)acc, s, keep); break;
         default: return MO_ERR_DTYPE;
     }
     if (rc != MO_OK) return rc;
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_absmax(const void* x, int64_t outer, int64_t axis, int64_t inner, int dtype,
+                         float* acc, void* stream) {
+    return mo_absmax_hinted(x, outer, axis, inner, dtype, acc, 0u, stream);
 }
 
 extern "C" int mo_absmax_pair(const void* x0, int64_t n0, float* acc0, const void* x1, int64_t n1,

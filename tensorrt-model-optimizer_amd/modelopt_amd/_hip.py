@@ -27,6 +27,7 @@ SIGNATURES = {
     "mo_version": [],
     "mo_error_string": [_INT],
     "mo_absmax": [_P, _I64, _I64, _I64, _INT, _P, _P],
+    "mo_absmax_hinted": [_P, _I64, _I64, _I64, _INT, _P, ctypes.c_uint, _P],
     "mo_absmax_pair": [_P, _I64, _P, _P, _I64, _P, _INT, _P],
     "mo_value_ranges": [_P, _P, _P, _INT, _P, _I64, _P],
     "mo_awq_pick_scale": [_P, _I64, _P, _I64, _P, _P, _P, _P, _P, _INT, _P],
@@ -194,8 +195,13 @@ def call(name: str, anchor: torch.Tensor, *args):
 # ----------------------------------------------------------------------------- thin wrappers
 
 
-def absmax_into(x: torch.Tensor, acc: torch.Tensor, outer: int, axis: int, inner: int):
-    """acc[a] = max(acc[a], max |x[o, a, i]|) for x viewed as [outer, axis, inner]."""
+MO_ABSMAX_REREAD = 1
+
+
+def absmax_into(x: torch.Tensor, acc: torch.Tensor, outer: int, axis: int, inner: int, reread: bool = False):
+    """acc[a] = max(acc[a], max |x[o, a, i]|) for x viewed as [outer, axis, inner].  ``reread``:
+    the caller reads ``x`` again right away (a dynamic quantizer's fake quant), so a per-tensor
+    reduction leaves it in the memory-side cache instead of streaming it past."""
     _require_device(x, acc)
     assert x.is_contiguous() and acc.dtype == torch.float32 and acc.numel() == axis
     assert outer * axis * inner == x.numel()
@@ -209,6 +215,10 @@ def absmax_into(x: torch.Tensor, acc: torch.Tensor, outer: int, axis: int, inner
         partial = _staging_words(x, slabs * axis)
         call("mo_absmax_cols_staged", x, _ptr(x), outer, axis, dtype_code(x.dtype), _ptr(acc),
              _ptr(partial), slabs, _stream(x))
+        return acc
+    if reread and axis == 1:
+        call("mo_absmax_hinted", x, _ptr(x), outer, axis, inner, dtype_code(x.dtype), _ptr(acc),
+             MO_ABSMAX_REREAD, _stream(x))
         return acc
     call("mo_absmax", x, _ptr(x), outer, axis, inner, dtype_code(x.dtype), _ptr(acc), _stream(x))
     return acc

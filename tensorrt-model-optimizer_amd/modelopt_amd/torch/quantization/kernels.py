@@ -90,18 +90,19 @@ def dense_flat_view(x: torch.Tensor):
     return x.as_strided((x.numel(),), (1,))
 
 
-def absmax_accumulate(x: torch.Tensor, acc: torch.Tensor, layout):
-    """acc (fp32, ``axis`` elements) = max(acc, abs-max of x over the reduced dims)."""
+def absmax_accumulate(x: torch.Tensor, acc: torch.Tensor, layout, reread: bool = False):
+    """acc (fp32, ``axis`` elements) = max(acc, abs-max of x over the reduced dims).  ``reread``:
+    the caller reads ``x`` again right away (see ``_hip.absmax_into``)."""
     outer, axis, inner = layout
     if not x.is_contiguous():
         # a per-tensor maximum does not care about element order: a permuted dense tensor (the
         # [B, H, S, D] view of K / V) is reduced where it lies instead of through a copy
         flat = dense_flat_view(x) if axis == 1 else None
         x = flat if flat is not None else x.contiguous()
-    return _hip.absmax_into(x, acc, outer, axis, inner)
+    return _hip.absmax_into(x, acc, outer, axis, inner, reread=reread)
 
 
-def reduce_amax_gpu(x: torch.Tensor, reduce_dims, keepdims=True):
+def reduce_amax_gpu(x: torch.Tensor, reduce_dims, keepdims=True, reread: bool = False):
     """``reduce_amax`` on the device: abs-max over ``reduce_dims`` (None = all) in x.dtype."""
     nd = x.dim()
     if reduce_dims is None:
@@ -116,7 +117,7 @@ def reduce_amax_gpu(x: torch.Tensor, reduce_dims, keepdims=True):
     if layout is None:
         src, _, layout = kept_dims_first(x, keep)
     acc = torch.zeros(layout[1], dtype=torch.float32, device=x.device)
-    absmax_accumulate(src, acc, layout)
+    absmax_accumulate(src, acc, layout, reread=reread)
     return acc.to(x.dtype).reshape(out_shape)
 
 

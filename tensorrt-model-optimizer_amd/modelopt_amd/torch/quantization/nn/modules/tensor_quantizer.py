@@ -345,8 +345,9 @@ class TensorQuantizer(nn.Module):
                 self._amax = self._amax.to(inputs.device)
             return self._amax.data
         reduce_axis = quant_utils.convert_quantization_axis_to_reduce_axis(inputs, self._axis)
+        # dynamic quantisation: the fake quant reads ``inputs`` again as soon as this returns
         return quant_utils.reduce_amax(inputs, axis=reduce_axis, keepdims=True,
-                                       squeeze_scalar=True).detach()
+                                       squeeze_scalar=True, reread=True).detach()
 
     def validate_attr(self, attr_value=None, attr_name="amax", raise_error=False, warn_error=False,
                       name=""):

@@ -95,7 +95,7 @@ class NVFP4QTensor(BaseQuantizedTensor):
                 return cls(shape, dtype, packed), wsf, wsf2
         if weights_scaling_factor_2 is None:
             acc = torch.zeros(1, dtype=torch.float32, device=x.device)
-            _hip.absmax_into(x, acc, 1, 1, x.numel())
+            _hip.absmax_into(x, acc, 1, 1, x.numel(), reread=True)   # the quantize pass reads x next
             scalar, is_wsf2 = acc.reshape(()), False
         else:
             scalar, is_wsf2 = _f32_scalar(weights_scaling_factor_2.to(x.device)), True

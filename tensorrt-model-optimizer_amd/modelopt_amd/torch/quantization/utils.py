@@ -37,14 +37,16 @@ def convert_quantization_axis_to_reduce_axis(input, axis):
 
 
 @torch.no_grad()
-def reduce_amax(input, axis=None, keepdims=True, squeeze_scalar=True):
+def reduce_amax(input, axis=None, keepdims=True, squeeze_scalar=True, *, reread=False):
     """Abs-max over ``axis`` (None = everything) in the input dtype (reference: utils.py:156-188).
 
     One kernel pass (the reference reads the tensor twice: max and min); NaN propagates.
+    ``reread``: the caller reads ``input`` again right away (a dynamic quantizer's fake quant), so
+    a per-tensor reduction leaves it in the memory-side cache.
     """
     if axis is None:
-        return kernels.reduce_amax_gpu(input, None)
-    out = kernels.reduce_amax_gpu(input, axis, keepdims=keepdims)
+        return kernels.reduce_amax_gpu(input, None, reread=reread)
+    out = kernels.reduce_amax_gpu(input, axis, keepdims=keepdims, reread=reread)
     if squeeze_scalar and out.numel() == 1:
         out = out.squeeze()
     return out

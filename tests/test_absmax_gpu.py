@@ -170,3 +170,31 @@ def test_value_ranges_leaves_what_it_does_not_cover():
     assert _hip.value_ranges([torch.ones(5 << 20, device=DEV)]) is None             # more chunks than the buffer holds
     assert _hip.value_ranges([torch.ones(0, device=DEV), a]) == [(float("inf"), float("-inf"), False), (1.0, 1.0, False)]
     assert _hip.value_ranges([a] * 32) == [(1.0, 1.0, False)] * 32
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n", [1, 4097, 32768 * 3 + 5, 1 << 22])
+def test_reread_hint_changes_nothing_but_the_cache_policy(dtype, n):
+    """mo_absmax_hinted(MO_ABSMAX_REREAD): the same maximum as mo_absmax, NaN included."""
+    x = _rand((n,), dtype, 8)
+    plain = torch.zeros(1, dtype=torch.float32, device=DEV)
+    hinted = torch.full((1,), 0.25, dtype=torch.float32, device=DEV)      # a running maximum
+    _hip.absmax_into(x.to(DEV), plain, 1, 1, n)
+    _hip.absmax_into(x.to(DEV), hinted, 1, 1, n, reread=True)
+    assert float(hinted) == max(float(plain), 0.25)
+    assert_bits_equal(plain.cpu().reshape(()).to(dtype), reduce.reduce_amax(x), "plain")
+    if n > 2:
+        x[n // 2] = float("nan")
+        _hip.absmax_into(x.to(DEV), hinted, 1, 1, n, reread=True)
+        assert torch.isnan(hinted).all()
+
+
+def test_unknown_hint_bits_are_refused():
+    import ctypes
+
+    lib = _hip.load()
+    x = torch.ones(64, dtype=torch.bfloat16, device=DEV)
+    acc = torch.zeros(1, dtype=torch.float32, device=DEV)
+    rc = lib.mo_absmax_hinted(ctypes.c_void_p(x.data_ptr()), 1, 1, 64, _hip.dtype_code(x.dtype),
+                              ctypes.c_void_p(acc.data_ptr()), 2, None)
+    assert rc == _hip.MO_ERR_ARG and float(acc) == 0

@@ -236,13 +236,13 @@ def test_layout_helpers():
 @pytest.fixture
 def oracle_backend(monkeypatch):
     """Route the kernel facade to the CPU oracle so host control flow runs without a GPU."""
-    def accumulate(x, acc, layout):
+    def accumulate(x, acc, layout, reread=False):
         outer, axis, inner = layout
         v = x.reshape(outer, axis, inner).abs().float().amax(dim=(0, 2))
         acc.copy_(torch.maximum(acc, v))
         return acc
 
-    def reduce_gpu(x, dims, keepdims=True):
+    def reduce_gpu(x, dims, keepdims=True, reread=False):
         return reduce.reduce_amax(x, axis=dims, keepdims=keepdims, squeeze_scalar=False) if dims is not None \
             else reduce.reduce_amax(x)
 
