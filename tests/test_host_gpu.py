@@ -531,7 +531,7 @@ def test_per_tensor_calibration_of_a_permuted_view_makes_no_copy(monkeypatch):
     assert not view.is_contiguous()
     seen = []
     real = _hip.absmax_into
-    monkeypatch.setattr(_hip, "absmax_into", lambda t, *a: (seen.append(t.data_ptr()), real(t, *a))[1])
+    monkeypatch.setattr(_hip, "absmax_into", lambda t, *a, **k: (seen.append(t.data_ptr()), real(t, *a, **k))[1])
     cal = calib.MaxCalibrator(8, None, False)
     cal.collect(view)
     assert seen == [view.data_ptr()]                       # reduced in place, not through a copy
