@@ -91,6 +91,35 @@ def test_argument_checks_that_need_no_gpu():
     assert lib.mo_real_quantize(p, 1, 1, 8, 2, p, 2, 2, 5, p, null) == UNSUP               # format
     assert lib.mo_real_quantize(p, 1, 1, 8, 2, p, 9, 2, 0, p, null) == DTYPE
     assert lib.mo_int4_pack_rows(p, 1, 3, 16, 16, 2, p, p, null) == ARG                    # odd row count
+    # the one-launch helpers of the calibration algorithms
+    TOO_LARGE = -5
+    assert lib.mo_absmax_hinted(null, 0, 4, 4, 2, null, 1, null) == OK                     # empty
+    assert lib.mo_absmax_hinted(p, 1, 4, 4, 2, p, 2, null) == ARG                          # unknown hint
+    assert lib.mo_absmax_hinted(p, 1, 4, 4, 9, p, 1, null) == DTYPE
+    assert lib.mo_absmax_hinted(null, 1, 4, 4, 2, p, 0, null) == ARG
+    ptrs = (ctypes.c_void_p * 33)(*[ctypes.addressof(buf)] * 33)
+    counts = (ctypes.c_int64 * 33)(*[8] * 33)
+    kinds = (ctypes.c_int * 33)(*[0] * 33)
+    assert lib.mo_value_ranges(null, null, null, 0, null, 0, null) == OK
+    assert lib.mo_value_ranges(ptrs, counts, kinds, 33, p, 64, null) == TOO_LARGE          # > 32 tensors
+    assert lib.mo_value_ranges(ptrs, counts, kinds, 4, p, 3, null) == TOO_LARGE            # output too short
+    assert lib.mo_value_ranges(ptrs, counts, kinds, 4, null, 4, null) == ARG
+    kinds[1] = 7
+    assert lib.mo_value_ranges(ptrs, counts, kinds, 4, p, 4, null) == DTYPE
+    kinds[1] = 0
+    counts[2] = -1
+    assert lib.mo_value_ranges(ptrs, counts, kinds, 4, p, 4, null) == ARG
+    counts[2] = 8
+    ptrs[3] = ctypes.addressof(buf) + 1
+    assert lib.mo_value_ranges(ptrs, counts, kinds, 4, p, 4, null) == UNSUP                # misaligned fp32
+    assert lib.mo_awq_pick_scale(p, 0, p, 8, p, p, p, p, p, 2, null) == ARG                # nothing to pick
+    assert lib.mo_awq_pick_scale(null, 2, p, 8, p, p, p, p, p, 2, null) == ARG
+    assert lib.mo_awq_pick_scale(p, 2, p, 8, p, p, p, p, p, 5, null) == DTYPE
+    assert lib.mo_awq_pick_scale(p, 70000, p, 8, p, p, p, p, p, 2, null) == UNSUP
+    assert lib.mo_smooth_scales(p, p, 0, 0.5, 0, 0.5, 0, 2, p, p, p, p, p, null) == ARG    # max over nothing
+    assert lib.mo_smooth_scales(p, p, 8, 0.5, 4, 0.5, 0, 2, p, p, p, p, p, null) == ARG    # power mode
+    assert lib.mo_smooth_scales(p, p, 8, 0.5, 0, 0.5, 0, 3, p, p, p, p, p, null) == DTYPE
+    assert lib.mo_smooth_scales(p, null, 8, 0.5, 0, 0.5, 0, 2, p, p, p, p, p, null) == ARG
     assert b"unsupported" in lib.mo_error_string(UNSUP).lower() or lib.mo_error_string(UNSUP)
 
 
