@@ -384,6 +384,16 @@ int mo_nf4_dequantize(const uint8_t* packed, int64_t nbytes, int64_t block_size,
 int mo_int4_pack_rows(const void* w, int64_t batch, int64_t n_rows, int64_t k, int64_t block_size,
                       int dtype, const float* ws, uint8_t* out, void* stream);
 
+/* The same with the type the quotient of the reference's tensor division has
+ * (modelopt/torch/export/quant_utils.py:704-706: weight / scales follows type promotion): MO_F32
+ * for fp32 scales -- what get_scaling_factor (export/quant_utils.py:228) hands the exporter, and
+ * what mo_int4_pack_rows computes -- or `dtype` itself when the caller's scales had the weight's
+ * own 16-bit type: the quotient is then rounded to that type before it is rounded to an integer
+ * (about 1 % of the codes differ).  ws holds the scales widened to fp32 either way.  Any other
+ * via_dtype returns MO_ERR_UNSUPPORTED. */
+int mo_int4_pack_rows_via(const void* w, int64_t batch, int64_t n_rows, int64_t k, int64_t block_size,
+                          int dtype, const float* ws, int via_dtype, uint8_t* out, void* stream);
+
 /* ------------------------------------------------------------------ AWQ-lite / SmoothQuant
  * y[r, c] = T(f32(x[r, c]) * f32(s[c])): the pre_quant_scale multiply of
  * TensorQuantizer.forward (TQ/nn/modules/tensor_quantizer.py:881-882) and the weight folding of

@@ -360,7 +360,9 @@ __global__ __launch_bounds__(256) void int4_block_dequantize_kernel(
 // ------------------------------------------------------------------------------ INT4 AWQ export
 // w[N, K], ws[N, K / bs] fp32; q = int8(clamp(rne(f32(w) / ws), -8, 7));
 // out[j, k] = (q[2j, k] & 0xF) | (q[2j + 1, k] << 4).  A lane packs 8 columns of a row pair.
-template <int DT>
+// NARROW: the scales came in the weight's own 16-bit type, so the tensor division of the
+// reference rounds the quotient to that type before it is rounded to an integer.
+template <int DT, bool NARROW>
 __global__ __launch_bounds__(256) void int4_pack_rows_kernel(const void* __restrict__ w,
                                                              int64_t n_rows, int64_t k, int64_t bs,
                                                              const float* __restrict__ ws,
@@ -376,7 +378,9 @@ __global__ __launch_bounds__(256) void int4_pack_rows_kernel(const void* __restr
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const int64_t row = 2 * j + h;
-                float q = __builtin_rintf(load_elem<DT>(w, row * k + col) / ws[row * nsb + col / bs]);
+                float q = load_elem<DT>(w, row * k + col) / ws[row * nsb + col / bs];
+                if constexpr (NARROW) q = round_via<DT>(q);
+                q = __builtin_rintf(q);
                 q = q < -8.0f ? -8.0f : q;
                 q = q > 7.0f ? 7.0f : q;
                 nib[h] = (q == q) ? ((uint32_t)(int)q & 0xFu) : 0u;
@@ -506,7 +510,7 @@ __global__ __launch_bounds__(256) void int4_block_dequantize_tile_kernel(
 // Row-pair pack with k % 8 == 0 and block_size % 8 == 0: a lane loads the same chunk of
 // columns from rows 2j and 2j + 1 and stores 8 bytes.
 constexpr int kInt4PackRounds = 2;   // items per lane (two 16-byte loads in flight each); 4 is 10 % slower at 117 MB
-template <int DT>
+template <int DT, bool NARROW>
 __global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
     const void* __restrict__ w, int64_t pairs, int64_t kc, int64_t chunks_per_scale,
     const float* __restrict__ ws, u32x2* __restrict__ out) {
@@ -583,8 +587,13 @@ __global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
             constexpr uint32_t kLeft = 0x4B000000u + (0x4B000000u << 4);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float qa = __builtin_amdgcn_fmed3f(exact_quotient(a[u][e], sa[u], ra), -8.0f, 7.0f);
-                const float qb = __builtin_amdgcn_fmed3f(exact_quotient(b[u][e], sb[u], rb), -8.0f, 7.0f);
+                float xa = exact_quotient(a[u][e], sa[u], ra), xb = exact_quotient(b[u][e], sb[u], rb);
+                if constexpr (NARROW) {
+                    xa = round_via<DT>(xa);
+                    xb = round_via<DT>(xb);
+                }
+                const float qa = __builtin_amdgcn_fmed3f(xa, -8.0f, 7.0f);
+                const float qb = __builtin_amdgcn_fmed3f(xb, -8.0f, 7.0f);
                 const uint32_t ba = f2u(qa + 8388616.0f), bb = f2u(qb + 8388616.0f);
                 if (e < 4) lo += (ba << (8 * e)) + (bb << (8 * e + 4));
                 else hi += (ba << (8 * (e - 4))) + (bb << (8 * (e - 4) + 4));
@@ -595,7 +604,11 @@ __global__ __launch_bounds__(256) void int4_pack_rows_tile_kernel(
             keep_branch();
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float qa = a[u][e] / sa[u], qb = b[u][e] / sb[u];
+                float qa = a[u][e] / sa[u], qb = b[u][e] / sb[u];
+                if constexpr (NARROW) {
+                    qa = round_via<DT>(qa);
+                    qb = round_via<DT>(qb);
+                }
                 // a NaN quotient packs as 0 here (what the float -> int8 cast of the CPU path yields)
                 const uint32_t na = qa == qa ? (uint32_t)int4_rne(qa) & 0xFu : 0u;
                 const uint32_t nb = qb == qb ? (uint32_t)int4_rne(qb) & 0xFu : 0u;
@@ -799,8 +812,18 @@ extern "C" int mo_int4_block_dequantize(const uint8_t* packed, int64_t nbytes, i
 extern "C" int mo_int4_pack_rows(const void* w, int64_t batch, int64_t n_rows, int64_t k,
                                  int64_t block_size, int dtype, const float* ws, uint8_t* out,
                                  void* stream) {
+    return mo_int4_pack_rows_via(w, batch, n_rows, k, block_size, dtype, ws, MO_F32, out, stream);
+}
+
+extern "C" int mo_int4_pack_rows_via(const void* w, int64_t batch, int64_t n_rows, int64_t k,
+                                     int64_t block_size, int dtype, const float* ws, int via_dtype,
+                                     uint8_t* out, void* stream) {
     if (batch < 0 || n_rows < 0 || k < 0 || block_size <= 0) return MO_ERR_ARG;
     if ((n_rows & 1) || (k % block_size)) return MO_ERR_ARG;
+    if (dtype < MO_F32 || dtype > MO_BF16 || via_dtype < MO_F32 || via_dtype > MO_BF16) return MO_ERR_DTYPE;
+    // the quotient of a tensor division is fp32 or, when both operands share a 16-bit type, that type
+    if (via_dtype != MO_F32 && via_dtype != dtype) return MO_ERR_UNSUPPORTED;
+    const bool narrow = via_dtype != MO_F32;
     if (batch == 0 || n_rows == 0 || k == 0) return MO_OK;
     if (!w || !ws || !out) return MO_ERR_ARG;
     hipStream_t s = (hipStream_t)stream;
@@ -812,15 +835,23 @@ extern "C" int mo_int4_pack_rows(const void* w, int64_t batch, int64_t n_rows, i
         const int64_t items = (rows >> 1) * (k / 8), tiles = (items + per_tile - 1) / per_tile;
         if (tiles <= 0x7FFFFFFF) {
 #define CALL(DT)                                                                      \
-    mo::int4_pack_rows_tile_kernel<DT><<<(unsigned)tiles, 256, mo::ballast_bytes("int4_pack_rows_tile_kernel", 0), s>>>(               \
-        w, rows >> 1, k / 8, block_size / 8, ws, (mo::u32x2*)out)
+    if (narrow && DT != MO_F32)                                                       \
+        mo::int4_pack_rows_tile_kernel<DT, DT != MO_F32><<<(unsigned)tiles, 256, mo::ballast_bytes("int4_pack_rows_tile_kernel", 0), s>>>( \
+            w, rows >> 1, k / 8, block_size / 8, ws, (mo::u32x2*)out);                \
+    else                                                                              \
+        mo::int4_pack_rows_tile_kernel<DT, false><<<(unsigned)tiles, 256, mo::ballast_bytes("int4_pack_rows_tile_kernel", 0), s>>>(        \
+            w, rows >> 1, k / 8, block_size / 8, ws, (mo::u32x2*)out)
             DISPATCH_DT(dtype, CALL)
 #undef CALL
             return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
         }
     }
     const unsigned g = mo::blocks_for((rows >> 1) * ((k + 7) >> 3));
-#define CALL(DT) mo::int4_pack_rows_kernel<DT><<<g, 256, 0, s>>>(w, rows, k, block_size, ws, out)
+#define CALL(DT)                                                                                      \
+    if (narrow && DT != MO_F32)                                                                       \
+        mo::int4_pack_rows_kernel<DT, DT != MO_F32><<<g, 256, 0, s>>>(w, rows, k, block_size, ws, out); \
+    else                                                                                              \
+        mo::int4_pack_rows_kernel<DT, false><<<g, 256, 0, s>>>(w, rows, k, block_size, ws, out)
     DISPATCH_DT(dtype, CALL)
 #undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;

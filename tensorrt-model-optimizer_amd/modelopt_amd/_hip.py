@@ -54,6 +54,7 @@ SIGNATURES = {
     "mo_int4_block_quantize": [_P, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_int4_block_dequantize": [_P, _I64, _I64, _P, _P, _INT, _P],
     "mo_int4_pack_rows": [_P, _I64, _I64, _I64, _I64, _INT, _P, _P, _P],
+    "mo_int4_pack_rows_via": [_P, _I64, _I64, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_nf4_quantize": [_P, _I64, _I64, _INT, _P, _P, _P],
     "mo_nf4_dequantize": [_P, _I64, _I64, _P, _P, _INT, _P],
     "mo_mul_cols": [_P, _I64, _I64, _INT, _P, _INT, _P, _P],
@@ -627,16 +628,18 @@ def nf4_dequantize(packed, scales, block_size):
     return y
 
 
-def int4_pack_rows(w, ws):
-    """INT4-AWQ export pack: w [..., N, K], ws fp32 [..., N, K / bs] -> uint8 [..., N / 2, K]."""
+def int4_pack_rows(w, ws, via_dtype=torch.float32):
+    """INT4-AWQ export pack: w [..., N, K], ws fp32 [..., N, K / bs] -> uint8 [..., N / 2, K].
+    ``via_dtype``: the type the quotient is rounded to before it is rounded to an integer, fp32
+    or ``w.dtype`` (scales that came in the weight's own 16-bit type)."""
     _require_device(w, ws)
     assert w.is_contiguous() and ws.is_contiguous() and ws.dtype == torch.float32
     n, k = w.shape[-2], w.shape[-1]
     batch = w.numel() // (n * k) if n * k else 0
     bs = k // ws.shape[-1]
     out = torch.empty(tuple(w.shape[:-2]) + (n // 2, k), dtype=torch.uint8, device=w.device)
-    call("mo_int4_pack_rows", w, _ptr(w), batch, n, k, bs, dtype_code(w.dtype), _ptr(ws), _ptr(out),
-         _stream(w))
+    call("mo_int4_pack_rows_via", w, _ptr(w), batch, n, k, bs, dtype_code(w.dtype), _ptr(ws),
+         dtype_code(via_dtype), _ptr(out), _stream(w))
     return out
 
 

@@ -288,8 +288,13 @@ def pack_int4_in_uint8(weight, weights_scaling_factor):
         raise IndexError(
             f"cannot pack INT4 weight: {weights_scaling_factor.shape[-1]} scales per row do not tile "
             f"{in_dim} input channels (the last block is padded); the reference's pack fails the same way")
+    # the quotient has the type tensor division gives it (export/quant_utils.py:704-706): fp32 with
+    # the exporter's fp32 scales, the weight's own type when the scales share a 16-bit type with it
+    via = torch.result_type(weight, weights_scaling_factor)
+    if via not in (torch.float16, torch.bfloat16) or via != weight.dtype:
+        via = torch.float32
     return _hip.int4_pack_rows(weight.contiguous(),
-                               weights_scaling_factor.to(torch.float32).contiguous())
+                               weights_scaling_factor.to(torch.float32).contiguous(), via)
 
 
 def to_quantized_weight(weight, weights_scaling_factor, quantization: str,
@@ -322,6 +327,34 @@ def to_quantized_weight(weight, weights_scaling_factor, quantization: str,
         return FP8QTensor.quantize(weight, weights_scaling_factor.squeeze(),
                                    block_sizes={-1: block_size, -2: block_size})[0]._quantized_data
     if quantization == QUANTIZATION_FP8_PC_PT:
+        if weight.dim() == 3:
+            # stacked expert weights (export/quant_utils.py:780-810): one scale per expert, per
+            # (expert, input channel) or per (expert, output channel), told apart by shape
+            s = weights_scaling_factor
+            experts, n, k = w.shape
+            if s.dim() == 1:
+                return _hip.real_quantize(w, s.contiguous(), 1, experts, n * k,
+                                          torch.result_type(w, s[:, None, None]), _hip.MO_FMT_E4M3)
+            if s.dim() == 2:
+                if s.shape[0] != experts:
+                    raise ValueError(
+                        f"First dimension (num_experts) mismatch for FP8_PC_PT quantization. "
+                        f"weight shape: {weight.shape}, scale shape: {s.shape}")
+                if n == k:
+                    raise ValueError(
+                        f"Ambiguous scaling dimension for FP8_PC_PT quantization with square weight matrix. "
+                        f"weight shape: {weight.shape}, scale shape: {s.shape}. "
+                        f"Cannot determine if scaling should be applied to input_dim or output_dim.")
+                via = torch.result_type(w, s.unsqueeze(-1))
+                if s.shape[-1] == k:    # (experts, input_dim): the scale runs along the rows
+                    return torch.stack([_hip.real_quantize(w[i], s[i].contiguous(), n, k, 1, via,
+                                                           _hip.MO_FMT_E4M3) for i in range(experts)])
+                if s.shape[-1] == n:    # (experts, output_dim)
+                    return _hip.real_quantize(w, s.reshape(-1).contiguous(), 1, experts * n, k, via,
+                                              _hip.MO_FMT_E4M3)
+                raise ValueError(
+                    f"Cannot determine correct unsqueeze dimension for FP8_PC_PT quantization. "
+                    f"weight shape: {weight.shape}, scale shape: {s.shape}")
         s = weights_scaling_factor.reshape(-1).contiguous()
         return _hip.real_quantize(w, s, 1, w.shape[0], w.shape[1], torch.result_type(w, s[:, None]),
                                   _hip.MO_FMT_E4M3)

@@ -91,6 +91,10 @@ def test_argument_checks_that_need_no_gpu():
     assert lib.mo_real_quantize(p, 1, 1, 8, 2, p, 2, 2, 5, p, null) == UNSUP               # format
     assert lib.mo_real_quantize(p, 1, 1, 8, 2, p, 9, 2, 0, p, null) == DTYPE
     assert lib.mo_int4_pack_rows(p, 1, 3, 16, 16, 2, p, p, null) == ARG                    # odd row count
+    assert lib.mo_int4_pack_rows_via(p, 1, 4, 16, 16, 2, p, 1, p, null) == UNSUP            # bf16 weight, fp16 quotient
+    assert lib.mo_int4_pack_rows_via(p, 1, 4, 16, 16, 0, p, 2, p, null) == UNSUP            # fp32 weight, bf16 quotient
+    assert lib.mo_int4_pack_rows_via(p, 1, 4, 16, 16, 2, p, 7, p, null) == DTYPE
+    assert lib.mo_int4_pack_rows_via(null, 0, 4, 16, 16, 2, null, 2, null, null) == OK
     # the one-launch helpers of the calibration algorithms
     TOO_LARGE = -5
     assert lib.mo_absmax_hinted(null, 0, 4, 4, 2, null, 1, null) == OK                     # empty

@@ -96,3 +96,34 @@ def test_to_quantized_weight_matches_reference_outputs(case):
     if want.dtype == torch.float8_e4m3fn:
         got = got.view(torch.float8_e4m3fn)
     assert_bits_equal(got.cpu(), want, case["name"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fp8_pc_pt_cast_of_stacked_expert_weights(dtype):
+    """FP8 per-channel casts of a 3-D (experts, output, input) weight: the three scale layouts the
+    reference tells apart by shape and its three errors (export/quant_utils.py:780-810), each
+    against the literal expression on the CPU."""
+    from conftest import assert_bits_equal
+    from modelopt_amd.torch.export import quant_utils as Q
+    from oracle import export
+
+    g = torch.Generator().manual_seed(21)
+    w = (torch.randn((3, 48, 80), generator=g) * 0.05).to(dtype)
+    per_expert = w.abs().amax(dim=(1, 2)).float() / 448.0
+    per_input = w.abs().amax(dim=1).float() / 448.0
+    per_output = w.abs().amax(dim=2).float() / 448.0
+    for name, s, view in (("per expert", per_expert, per_expert[:, None, None]),
+                          ("per input channel", per_input, per_input.unsqueeze(-2)),
+                          ("per output channel", per_output, per_output.unsqueeze(-1)),
+                          ("per output channel, 16-bit scales", per_output.to(dtype),
+                           per_output.to(dtype).unsqueeze(-1))):
+        got = Q.to_quantized_weight(w.to("cuda:0"), s.to("cuda:0"), "fp8_pc_pt")
+        assert_bits_equal(got.view(torch.float8_e4m3fn).cpu(), export.fp8_export_cast(w, view), name)
+    dev = w.to("cuda:0")
+    with pytest.raises(ValueError, match="num_experts"):
+        Q.to_quantized_weight(dev, torch.ones(2, 48, device="cuda:0"), "fp8_pc_pt")
+    with pytest.raises(ValueError, match="Ambiguous"):
+        Q.to_quantized_weight(dev[:, :, :48].contiguous(), torch.ones(3, 48, device="cuda:0"), "fp8_pc_pt")
+    with pytest.raises(ValueError, match="unsqueeze"):
+        Q.to_quantized_weight(dev, torch.ones(3, 7, device="cuda:0"), "fp8_pc_pt")

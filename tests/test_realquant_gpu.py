@@ -382,6 +382,33 @@ def test_int4_awq_export_pack_large_and_special(dtype):
                       export.pack_int4_in_uint8(w2, ws2), "packed rows, block 12")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape,bs", [((256, 1024), 128), ((2, 64, 256), 64), ((66, 1020), 12)])
+def test_int4_awq_export_pack_with_scales_in_the_weight_s_own_type(dtype, shape, bs):
+    """``weight / scales`` of two tensors of one 16-bit type is rounded to that type before
+    ``.round()`` (type promotion in the reference's expression, export/quant_utils.py:704-706): about
+    1 % of the codes differ from the fp32 quotient the exporter's fp32 scales give.  Both routes
+    against the literal expression on the CPU, the second also with scales of the other 16-bit
+    type (promoted to fp32)."""
+    from modelopt_amd.torch.export.quant_utils import pack_int4_in_uint8
+
+    g = torch.Generator().manual_seed(16)
+    w = (torch.randn(shape, generator=g) * 0.05).to(dtype)
+    w[..., 3, 8:24] = 0.0
+    ws = (reduce.reduce_block_amax(w, {-1: bs}).float() / 7.0).to(dtype)
+    ws[..., 5, 0] = 1e-4 if dtype == torch.float16 else 1e-30   # quotients far outside the clamp range
+    if dtype == torch.bfloat16:
+        ws[..., 6, 1] = 2.0**70                                 # scale outside the reciprocal path's range
+    want = export.pack_int4_in_uint8(w, ws)
+    assert not torch.equal(want, export.pack_int4_in_uint8(w, ws.float())), "the case must differ from fp32"
+    assert_bits_equal(pack_int4_in_uint8(w.to(DEV), ws.to(DEV)).cpu(), want, "16-bit quotient")
+    assert_bits_equal(_hip.int4_pack_rows(w.to(DEV), ws.float().to(DEV), dtype).cpu(), want, "binding")
+    other = torch.float16 if dtype == torch.bfloat16 else torch.bfloat16
+    ws_o = (reduce.reduce_block_amax(w, {-1: bs}).float() / 7.0).to(other)
+    assert_bits_equal(pack_int4_in_uint8(w.to(DEV), ws_o.to(DEV)).cpu(), export.pack_int4_in_uint8(w, ws_o),
+                      "mixed 16-bit types promote to fp32")
+
+
 def test_int4_awq_export_pack_with_a_padded_last_block():
     """in_features that the 128-wide blocks do not tile (reference export/quant_utils.py:701-706:
     block size = in_dim // scales per row, scale index = column // that).  192 columns with two
