@@ -364,8 +364,11 @@ def to_quantized_weight(weight, weights_scaling_factor, quantization: str,
         assert block_size is not None, "Block size not passed. Unable to quantize to NVFP4 format."
         assert weights_scaling_factor2 is not None, (
             "Weights scaling factor 2 not passed. Unable to quantize to NVFP4 format")
-        return NVFP4QTensor.quantize(weight, block_size, weights_scaling_factor,
-                                     weights_scaling_factor2)[0]._quantized_data
+        # one global scale per expert of a stacked weight broadcasts over its matrix
+        return NVFP4QTensor.quantize(
+            weight, block_size, weights_scaling_factor,
+            weights_scaling_factor2.view(-1, 1, 1) if weights_scaling_factor2.dim() != 0
+            else weights_scaling_factor2)[0]._quantized_data
     if quantization in _MXFP4_FAMILY:
         return MXFP4QTensor.quantize(weight, block_size=block_size)[0]._quantized_data
     raise NotImplementedError(f"quantization format {quantization} not supported")

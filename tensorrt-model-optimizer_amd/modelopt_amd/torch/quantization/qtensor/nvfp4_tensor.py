@@ -23,6 +23,19 @@ def _f32_scalar(t: torch.Tensor):
     return t.detach().reshape(()).to(torch.float32)
 
 
+def _per_leading_index(scale2, input):
+    """The global scales of a stack of matrices -- one per index of the first dim, shaped to
+    broadcast (``view(-1, 1, 1)`` for stacked expert weights, export/quant_utils.py:822-829) -- as
+    a flat tensor, or None for the usual single scale."""
+    if scale2 is None or scale2.numel() == 1:
+        return None
+    assert input.dim() >= 2 and scale2.numel() == input.shape[0] and (
+        scale2.dim() <= 1 or tuple(scale2.shape[1:]) == (1,) * (scale2.dim() - 1)), (
+        f"global scale of shape {tuple(scale2.shape)} does not broadcast over the first dim of "
+        f"{tuple(input.shape)}")
+    return scale2.reshape(-1)
+
+
 class NVFP4QTensor(BaseQuantizedTensor):
     """Packed NVFP4 tensor."""
 
@@ -45,6 +58,11 @@ class NVFP4QTensor(BaseQuantizedTensor):
         assert input.shape[-1] % block_size == 0, (
             "Weight shape is not divisible for block size for block quantization.")
         wsf2 = weights_scaling_factor_2.to(input.device)
+        each = _per_leading_index(wsf2, input)
+        if each is not None:
+            return torch.stack([cls.get_weights_scaling_factor(input[i], block_size, each[i],
+                                                               keep_high_precision)[0]
+                                for i in range(input.shape[0])]), weights_scaling_factor_2
         if keep_high_precision:
             bamax = reduce_block_amax(input, {-1: block_size}).float()
             scale = bamax / (6.0 * wsf2)
@@ -84,6 +102,15 @@ class NVFP4QTensor(BaseQuantizedTensor):
             blocks = xp.reshape(*xp.shape[:-1], -1, block_size)
             return torch.div(blocks, scale.unsqueeze(-1)).reshape(xp.shape)
         shape, dtype = input.shape, input.dtype
+        each = _per_leading_index(weights_scaling_factor_2, input)
+        if each is not None:
+            parts = [cls.quantize(input[i], block_size,
+                                  None if weights_scaling_factor is None else weights_scaling_factor[i],
+                                  each[i]) for i in range(shape[0])]
+            scales = weights_scaling_factor if weights_scaling_factor is not None else \
+                torch.stack([p[1] for p in parts])
+            return (cls(shape, dtype, torch.stack([p[0]._quantized_data for p in parts])), scales,
+                    weights_scaling_factor_2)
         x = input.contiguous()
         if (weights_scaling_factor_2 is None and weights_scaling_factor is None and block_size == 16
                 and modes.one_launch_dynamic_quant()):
@@ -120,6 +147,12 @@ class NVFP4QTensor(BaseQuantizedTensor):
         if scale.dtype != torch.float8_e4m3fn:
             raise NotImplementedError("NVFP4 dequantize needs float8_e4m3fn block scales")
         packed = self._quantized_data
+        each = _per_leading_index(wsf2, packed)
+        if each is not None:
+            scale = scale.to(packed.device)
+            return torch.stack([_hip.nvfp4_dequantize(
+                packed[i].contiguous(), scale[i].contiguous(), _f32_scalar(each[i].to(packed.device)),
+                block, dtype) for i in range(packed.shape[0])]).reshape(self.metadata["shape"])
         y = _hip.nvfp4_dequantize(packed.contiguous(), scale.to(packed.device).contiguous(),
                                   _f32_scalar(wsf2.to(packed.device)), block, dtype)
         return y.reshape(self.metadata["shape"])

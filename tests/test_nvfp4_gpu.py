@@ -315,3 +315,29 @@ def test_plans_refuse_inputs_that_were_reallocated():
         qplan.run()
     after = qplan.run(verify=False)[0]      # still the old memory, still valid
     assert all(torch.equal(a, b) for a, b in zip(before, after))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_stacked_expert_weights_with_one_global_scale_each(dtype):
+    """A 3-D (experts, output, input) weight whose global scale is given per expert, shaped
+    ``[E, 1, 1]`` so that it broadcasts (qtensor/nvfp4_tensor.py:199-203 with the scales of
+    export/quant_utils.py:822-829): block scales, codes, the dequantised tensor and the export
+    cast against the same expressions on the CPU."""
+    from modelopt_amd.torch.export.quant_utils import to_quantized_weight
+    from modelopt_amd.torch.quantization.qtensor import NVFP4QTensor
+
+    g = torch.Generator().manual_seed(31)
+    w = (torch.randn((3, 32, 80), generator=g) * torch.tensor([0.02, 0.5, 3.0]).view(-1, 1, 1)).to(dtype)
+    wsf2 = (w.abs().amax(dim=(1, 2)).float() / (6.0 * 448.0)).view(-1, 1, 1)
+    want_packed, want_wsf, _ = qtensor.nvfp4_quantize(w, 16, None, wsf2)
+    dev = w.to(DEV)
+    scales, _ = NVFP4QTensor.get_weights_scaling_factor(dev, 16, wsf2.to(DEV))
+    assert_bits_equal(scales.cpu().view(torch.uint8), want_wsf.view(torch.uint8), "block scales")
+    q, got_wsf, got_wsf2 = NVFP4QTensor.quantize(dev, 16, None, wsf2.to(DEV))
+    assert got_wsf2.shape == (3, 1, 1)
+    assert_bits_equal(got_wsf.cpu().view(torch.uint8), want_wsf.view(torch.uint8), "block scales from quantize")
+    assert_bits_equal(q._quantized_data.cpu(), want_packed, "codes")
+    back = q.dequantize(scale=got_wsf, double_scale=got_wsf2, block_sizes={-1: 16})
+    assert_bits_equal(back.cpu(), qtensor.nvfp4_dequantize(want_packed, want_wsf, wsf2, 16, w.shape, dtype), "dequantised")
+    cast = to_quantized_weight(dev, scales, "nvfp4", wsf2.reshape(-1).to(DEV), block_size=16)
+    assert_bits_equal(cast.cpu(), want_packed, "export cast with a 1-D global scale")
