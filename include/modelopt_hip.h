@@ -377,6 +377,12 @@ int mo_nf4_quantize(const void* x, int64_t n, int64_t block_size, int dtype, voi
 int mo_nf4_dequantize(const uint8_t* packed, int64_t nbytes, int64_t block_size,
                       const void* scales, void* y, int dtype, void* stream);
 
+/* codes[i] = (x[i] < 0) << 3 | ordinal of the E2M1 magnitude nearest to |x[i]| (0, .5, 1, 1.5, 2,
+ * 3, 4, 6; ties to the even code, NaN and infinity give ordinal 7, -0.0 gives code 0): one byte
+ * per element, unpacked.  Replaces NVFP4QTensor._cast_fp4 (TQ/qtensor/nvfp4_tensor.py:120-140);
+ * x is left as it is (the reference takes its absolute value in place). */
+int mo_cast_fp4(const void* x, int64_t n, int dtype, uint8_t* codes, void* stream);
+
 /* INT4-AWQ export pack of w[batch, n_rows, k] with fp32 scales ws[batch, n_rows, k/block_size]:
  * q = int8(clamp(rne(f32(w) / ws), -8, 7)); out[b, j, c] = (q[b, 2j, c] & 0xF) |
  * (q[b, 2j+1, c] << 4), out is uint8 [batch, n_rows / 2, k].  Replaces pack_int4_in_uint8

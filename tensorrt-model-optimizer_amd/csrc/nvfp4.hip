@@ -781,3 +781,39 @@ extern "C" int mo_nvfp4_quantize_fused(const void* x, int64_t rows, int64_t k, i
                                           wsf_out, wsf2_out, amax_out, (uint32_t*)workspace, spins, s);
     return rc;
 }
+
+// ------------------------------------------------------------------------------ E2M1 codes
+// One code byte per element: sign << 3 | ordinal of the nearest E2M1 magnitude, ties to the even
+// code (NVFP4QTensor._cast_fp4, TQ/qtensor/nvfp4_tensor.py:120-140).
+namespace mo {
+template <int DT>
+__global__ __launch_bounds__(256) void cast_fp4_kernel(const void* __restrict__ x, int64_t n,
+                                                       uint8_t* __restrict__ codes) {
+    const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i0 >= n) return;
+    if (i0 + 4 <= n && (((uintptr_t)codes) & 3u) == 0) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w |= f32_to_e2m1(load_elem<DT>(x, i0 + j)) << (8 * j);
+        *(uint32_t*)(codes + i0) = w;
+    } else {
+        for (int64_t i = i0; i < n && i < i0 + 4; ++i) codes[i] = (uint8_t)f32_to_e2m1(load_elem<DT>(x, i));
+    }
+}
+}  // namespace mo
+
+extern "C" int mo_cast_fp4(const void* x, int64_t n, int dtype, uint8_t* codes, void* stream) {
+    if (n < 0) return MO_ERR_ARG;
+    if (dtype < MO_F32 || dtype > MO_BF16) return MO_ERR_DTYPE;
+    if (n == 0) return MO_OK;
+    if (!x || !codes) return MO_ERR_ARG;
+    const int64_t grid = (n + 1023) / 1024;
+    if (grid > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case MO_F32: mo::cast_fp4_kernel<MO_F32><<<(unsigned)grid, 256, 0, s>>>(x, n, codes); break;
+        case MO_F16: mo::cast_fp4_kernel<MO_F16><<<(unsigned)grid, 256, 0, s>>>(x, n, codes); break;
+        default: mo::cast_fp4_kernel<MO_BF16><<<(unsigned)grid, 256, 0, s>>>(x, n, codes); break;
+    }
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}

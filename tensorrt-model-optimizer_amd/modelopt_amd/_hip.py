@@ -53,6 +53,7 @@ SIGNATURES = {
     "mo_real_dequantize": [_P, _I64, _I64, _I64, _INT, _P, _INT, _P, _INT, _P],
     "mo_int4_block_quantize": [_P, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_int4_block_dequantize": [_P, _I64, _I64, _P, _P, _INT, _P],
+    "mo_cast_fp4": [_P, _I64, _INT, _P, _P],
     "mo_int4_pack_rows": [_P, _I64, _I64, _I64, _I64, _INT, _P, _P, _P],
     "mo_int4_pack_rows_via": [_P, _I64, _I64, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_nf4_quantize": [_P, _I64, _I64, _INT, _P, _P, _P],
@@ -552,6 +553,15 @@ def nvfp4_dequantize(packed, wsf, wsf2, block_size, dtype):
     call("mo_nvfp4_dequantize", packed, _ptr(packed), _ptr(wsf.view(torch.uint8)), _ptr(wsf2),
          rows, kp, block_size, _ptr(y), dtype_code(dtype), _stream(packed))
     return y
+
+
+def cast_fp4(x):
+    """E2M1 codes (sign << 3 | ordinal, ties to even), one uint8 per element of ``x``."""
+    _require_device(x)
+    assert x.is_contiguous()
+    codes = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    call("mo_cast_fp4", x, _ptr(x), x.numel(), dtype_code(x.dtype), _ptr(codes), _stream(x))
+    return codes
 
 
 MO_FMT_E4M3, MO_FMT_INT8 = 0, 1

@@ -88,6 +88,9 @@ class _Calibrator:
     def compute_amax(self, *args, **kwargs):
         raise NotImplementedError
 
+    def __repr__(self):
+        return f"num_bits={self._num_bits} axis={self._axis} unsigned={self._unsigned}"
+
 
 class MaxCalibrator(_Calibrator):
     """Tracks the running abs-max of every tensor it is shown."""
@@ -241,3 +244,10 @@ class MaxCalibrator(_Calibrator):
 
     def __str__(self):
         return f"MaxCalibrator(track_amax={self._track_amax})"
+
+    def __repr__(self):
+        # the reference's fields in its order (calib/max.py:102-110)
+        s = f"MaxCalibrator({super().__repr__()} calib_amax={self._calib_amax} track_amax={self._track_amax}"
+        if self._track_amax:
+            s += f" amaxs={self._amaxs}"
+        return s + ")"

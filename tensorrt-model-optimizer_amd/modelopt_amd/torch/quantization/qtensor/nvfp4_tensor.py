@@ -39,6 +39,30 @@ def _per_leading_index(scale2, input):
 class NVFP4QTensor(BaseQuantizedTensor):
     """Packed NVFP4 tensor."""
 
+    e2m1_values_on_device = {}
+    e2m1_bounds_on_device = {}
+
+    @classmethod
+    def get_e2m1_values(cls, device):
+        """The 16 values a code stands for, on ``device`` (reference: nvfp4_tensor.py:41-46)."""
+        if device not in cls.e2m1_values_on_device:
+            cls.e2m1_values_on_device[device] = e2m1_values.to(device)
+        return cls.e2m1_values_on_device[device]
+
+    @classmethod
+    def get_e2m1_bounds(cls, device):
+        """The 7 midpoints between adjacent magnitudes, on ``device`` (reference: :48-53)."""
+        if device not in cls.e2m1_bounds_on_device:
+            cls.e2m1_bounds_on_device[device] = e2m1_bounds.to(device)
+        return cls.e2m1_bounds_on_device[device]
+
+    @classmethod
+    def _cast_fp4(cls, weight: torch.Tensor):
+        """``sign << 3 | ordinal`` per element, uint8, ties to the even code (reference:
+        nvfp4_tensor.py:120-140; unlike the reference, ``weight`` is not overwritten with its
+        absolute value)."""
+        return _hip.cast_fp4(weight.contiguous())
+
     @classmethod
     def get_weights_scaling_factor_2_from_quantizer(cls, weight_quantizer):
         assert hasattr(weight_quantizer, "_amax"), "Weight quantizer does not have attribute amax"

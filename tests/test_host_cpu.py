@@ -529,7 +529,12 @@ def test_reprs_do_not_raise():
     holder = nn.Module()
     holder.linear, holder.quant_linear = nn.Linear(33, 65), qnn.Linear(33, 65)
     assert "weight_quantizer" in repr(holder)
-    assert "MaxCalibrator" in repr(calib.MaxCalibrator(7, 1, False))
+    assert repr(calib.MaxCalibrator(7, 1, False)) == (
+        "MaxCalibrator(num_bits=7 axis=1 unsigned=False calib_amax=None track_amax=False)")
+    assert str(calib.MaxCalibrator(7, 1, False, track_amax=True)) == "MaxCalibrator(track_amax=True)"
+    assert "amaxs=[]" in repr(calib.MaxCalibrator(7, 1, False, track_amax=True))
+    from modelopt_amd.torch.quantization.calib.calibrator import _Calibrator
+    assert issubclass(calib.MaxCalibrator, _Calibrator)
 
 
 def test_library_operators_are_registered_with_fake_implementations():

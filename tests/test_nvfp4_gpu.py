@@ -341,3 +341,37 @@ def test_stacked_expert_weights_with_one_global_scale_each(dtype):
     assert_bits_equal(back.cpu(), qtensor.nvfp4_dequantize(want_packed, want_wsf, wsf2, 16, w.shape, dtype), "dequantised")
     cast = to_quantized_weight(dev, scales, "nvfp4", wsf2.reshape(-1).to(DEV), block_size=16)
     assert_bits_equal(cast.cpu(), want_packed, "export cast with a 1-D global scale")
+
+
+@pytest.mark.parametrize("values", [
+    None,
+    [[0.25, 0.75, 1.25], [1.75, 2.5, 3.5]],
+    [[0.1, 2.5, 1.0, 4.8], [1.5, 1.25, 3.25, 5.0]],
+    [[0, 0.75, 1.25], [1.75, 2.5, 5.5]],
+    [[-0.25, -0.75, -1.25], [-1.75, -2.5, -3.5]],
+    [[-0.1, -2.5, -1.0, -4.8], [-1.5, -1.25, -3.25, -5.0]],
+    [[0, -0.75, -1.25], [-1.75, -2.5, -5.5]],
+    [[float("nan"), float("inf"), -float("inf"), -0.0, 1e-30, -1e-30, 6.0, -7.5, 1e30]],
+])
+def test_cast_fp4_codes(values):
+    """``NVFP4QTensor._cast_fp4`` on the inputs of the reference's equivalence test
+    (tests/gpu/torch/quantization/test_qtensor_cuda.py:399-441) plus special values, a ragged
+    length and the 16-bit types, against the CPU restatement of nvfp4_tensor.py:120-140."""
+    from modelopt_amd.torch.quantization.qtensor import NVFP4QTensor
+
+    if values is None:
+        x = torch.randn((32, 16), generator=torch.Generator().manual_seed(0)) * 3
+    else:
+        x = torch.tensor(values, dtype=torch.float32)
+    got = NVFP4QTensor._cast_fp4(x.to(DEV))
+    assert got.dtype == torch.uint8 and got.shape == x.shape
+    assert torch.equal(got.cpu(), qtensor.cast_fp4(x.clone()))
+    flat = torch.randn(1027, generator=torch.Generator().manual_seed(1)) * 4
+    flat[::50] = torch.tensor([0.75, 1.75, 3.5, 0.25, 1.25, 2.5, 5.0]).repeat(3)
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        v = flat.to(dtype)
+        assert torch.equal(NVFP4QTensor._cast_fp4(v.to(DEV)).cpu(), qtensor.cast_fp4(v.float())), dtype
+        odd = v[1:]                                      # byte stores that are not word aligned
+        assert torch.equal(_hip.cast_fp4(odd.to(DEV).contiguous()).cpu(), qtensor.cast_fp4(odd.float()))
+    assert NVFP4QTensor.get_e2m1_bounds(DEV).tolist() == [0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5]
+    assert NVFP4QTensor.get_e2m1_values(DEV)[9].item() == -0.5
