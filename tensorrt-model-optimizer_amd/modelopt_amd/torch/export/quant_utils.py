@@ -51,6 +51,41 @@ def get_scaling_factor_from_weight(weight, group_size) -> torch.Tensor:
     return sf
 
 
+def maybe_transpose_expert_weight_dimensions(weight, weight_scale=None, is_bmm_expert_weight=True):
+    """Swap the last two dims of a stacked expert weight (and of its scale) between the
+    (experts, input, output) and (experts, output, input) layouts; anything else is returned as
+    it is (reference: export/quant_utils.py:94-123)."""
+    if not is_bmm_expert_weight or weight.dim() != 3:
+        return weight, weight_scale
+    return weight.transpose(-2, -1), None if weight_scale is None else weight_scale.transpose(-2, -1)
+
+
+def resmooth_and_get_scale(merged_weights, pre_quant_scales, ranks, group_size, new_pre_quant_scale=None,
+                           quantization=QUANTIZATION_NONE):
+    """Bring the row chunks of ``merged_weights`` (one per rank, each smoothed with its own
+    ``pre_quant_scale``) to one shared scale -- the mean unless given -- and recompute their block
+    scales (reference: export/quant_utils.py:126-185).  Returns (weights, scales, shared scale).
+    ``w * p / p_new`` is two tensor operations in the weight dtype, as in the reference."""
+    if new_pre_quant_scale is None:
+        new_pre_quant_scale = torch.stack(pre_quant_scales).mean(dim=0)
+    assert len(pre_quant_scales) > 0 and new_pre_quant_scale.numel() == merged_weights.shape[1], (
+        "Shape of pre_quant_scales and weights do not match.")
+    chunks = torch.chunk(merged_weights, ranks, dim=0)
+    weights, scales = [], []
+    for chunk, own in zip(chunks, pre_quant_scales):
+        weight = chunk * own.type(chunk.dtype) / new_pre_quant_scale.type(chunk.dtype)
+        weights.append(weight)
+        if quantization == QUANTIZATION_NVFP4_AWQ:
+            # block scales travel as bytes so that they can be concatenated
+            scales.append(NVFP4QTensor.get_weights_scaling_factor(weight, group_size)[0].view(torch.uint8))
+        else:
+            scales.append(get_scaling_factor_from_weight(weight, group_size))
+    scales = torch.cat(scales, dim=0)
+    if quantization == QUANTIZATION_NVFP4_AWQ:
+        scales = scales.view(torch.float8_e4m3fn)
+    return torch.cat(weights, dim=0), scales, new_pre_quant_scale
+
+
 def get_scaling_factor(quantizer: TensorQuantizer) -> torch.Tensor | None:
     if not quantizer.is_enabled:
         return None

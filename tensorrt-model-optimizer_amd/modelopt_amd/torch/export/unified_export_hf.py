@@ -123,6 +123,9 @@ def _quantizer_on(q) -> bool:
     return isinstance(q, TensorQuantizer) and q.is_enabled
 
 
+_is_enabled_quantizer = _quantizer_on   # the reference's name for it (unified_export_hf.py:80-87)
+
+
 def requantize_resmooth_fused_llm_layers(model: nn.Module):
     """Unify what an inference engine will fuse (reference: unified_export_hf.py:90-231).
 

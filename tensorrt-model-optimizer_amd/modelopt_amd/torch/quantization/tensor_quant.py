@@ -42,6 +42,23 @@ def fp8_eager(inputs: torch.Tensor, amax: torch.Tensor | None = None) -> torch.T
     return kernels.fake_quant_fp8(inputs, amax, saturate=False)
 
 
+_fp8_eager = fp8_eager   # the reference keeps the body under this name (tensor_quant.py:45)
+
+# the reference's switch between its two NVFP4 fake-quant kernels (tensor_quant.py:42); there is
+# one kernel here, so the flag is accepted and changes nothing
+DISABLE_TRITON_KERNEL = False
+
+
+def _tensor_quant(inputs, amax, num_bits=8, unsigned=False, narrow_range=True):
+    """The reference's eager body (tensor_quant.py:574-612) by name: its two looks at the data on
+    the host happen here whatever the strict mode -- negative inputs with ``unsigned`` raise
+    ``TypeError``, a negative amax raises ``ValueError`` -- then the kernel."""
+    if unsigned and inputs.numel() and inputs.min() < 0.0:
+        raise TypeError("Negative values encountered in unsigned quantization.")
+    if amax.numel() and amax.min() < 0:
+        raise ValueError("Negative values in amax")
+    return kernels.fake_quant_int(inputs, amax, num_bits, unsigned, narrow_range)
+
 
 
 def fake_quant_impl(inputs, amax, num_bits=8, unsigned=False, narrow_range=True):
@@ -150,6 +167,13 @@ def quantize_op(inputs, amax, num_bits=8, exponent_bits=0, unsigned=False, narro
 QUANT_DESC_8BIT_PER_TENSOR = QuantizerAttributeConfig(num_bits=8)
 QUANT_DESC_UNSIGNED_8BIT_PER_TENSOR = QuantizerAttributeConfig(num_bits=8, unsigned=True)
 QUANT_DESC_8BIT_LINEAR_WEIGHT_PER_ROW = QuantizerAttributeConfig(num_bits=8, axis=(0))
+# the per-output-channel descriptors of the convolution wrappers (tensor_quant.py:286-292): same content
+QUANT_DESC_8BIT_CONV1D_WEIGHT_PER_CHANNEL = QuantizerAttributeConfig(num_bits=8, axis=(0))
+QUANT_DESC_8BIT_CONV2D_WEIGHT_PER_CHANNEL = QuantizerAttributeConfig(num_bits=8, axis=(0))
+QUANT_DESC_8BIT_CONV3D_WEIGHT_PER_CHANNEL = QuantizerAttributeConfig(num_bits=8, axis=(0))
+QUANT_DESC_8BIT_CONVTRANSPOSE1D_WEIGHT_PER_CHANNEL = QuantizerAttributeConfig(num_bits=8, axis=(0))
+QUANT_DESC_8BIT_CONVTRANSPOSE2D_WEIGHT_PER_CHANNEL = QuantizerAttributeConfig(num_bits=8, axis=(0))
+QUANT_DESC_8BIT_CONVTRANSPOSE3D_WEIGHT_PER_CHANNEL = QuantizerAttributeConfig(num_bits=8, axis=(0))
 
 
 def _fake_tensor_quant_backward(inputs, amax, grad_outputs):

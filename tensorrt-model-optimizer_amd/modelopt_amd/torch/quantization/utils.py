@@ -1,6 +1,7 @@
 """Quantization utilities with the reference's names (modelopt/torch/quantization/utils.py),
 backed by the HIP abs-max kernels."""
 
+import collections
 import contextlib
 
 import torch
@@ -111,16 +112,86 @@ def is_quantized_linear(module):
     return weight is not None and weight.dim() == 2
 
 
-class _QuantizerNames:
-    def __init__(self, weight_name="weight"):
-        prefix = "" if weight_name == "weight" else weight_name + "_"
-        self.weight_quantizer = prefix + "weight_quantizer"
-        self.input_quantizer = prefix + "input_quantizer"
-        self.output_quantizer = prefix + "output_quantizer"
+# every quantizer-related attribute name that goes with one weight attribute (reference: utils.py:247-273)
+QuantizerAttrNames = collections.namedtuple(
+    "QuantizerAttrNames", ("weight_quantizer", "input_quantizer", "output_quantizer", "weight_scale",
+                           "weight_scale_2", "input_scale", "output_scale"))
 
 
-def quantizer_attr_names(weight_name="weight"):
-    return _QuantizerNames(weight_name)
+def quantizer_attr_names(weight_name="weight") -> QuantizerAttrNames:
+    """The names for ``weight_name``: plain for ``"weight"``, prefixed ``<weight_name>_`` otherwise."""
+    prefix = "" if weight_name == "weight" else weight_name + "_"
+    return QuantizerAttrNames(*(prefix + field for field in QuantizerAttrNames._fields))
+
+
+def is_pow2(n) -> bool:
+    """True for 1, 2, 4, ... (reference: utils.py:377-379)."""
+    return n != 0 and n & (n - 1) == 0
+
+
+@contextlib.contextmanager
+def replace_function(package, name, new_func):
+    """Within the block ``package.name`` is ``new_func`` and the original is reachable as
+    ``package._name`` (reference: utils.py:339-347)."""
+    original = getattr(package, name)
+    setattr(package, name, new_func)
+    setattr(package, "_" + name, original)
+    try:
+        yield
+    finally:
+        setattr(package, name, original)
+        delattr(package, "_" + name)
+
+
+@contextlib.contextmanager
+def multi_context(*managers):
+    """Enter any number of context managers as one (reference: utils.py:350-354)."""
+    with contextlib.ExitStack() as stack:
+        yield [stack.enter_context(m) for m in managers]
+
+
+EXPORT_MODE: bool = False
+
+
+@contextlib.contextmanager
+def export_torch_mode():
+    """Marks the block as a ``torch.export`` trace (reference: utils.py:357-374)."""
+    global EXPORT_MODE
+    before, EXPORT_MODE = EXPORT_MODE, True
+    try:
+        yield
+    finally:
+        EXPORT_MODE = before
+
+
+def is_torch_export_mode() -> bool:
+    return EXPORT_MODE
+
+
+@contextlib.contextmanager
+def enable_weight_access_and_writeback(module, root_model):
+    """The reference gathers a sharded or off-loaded weight here and writes it back afterwards
+    (utils.py:466-486); weights of this build's modules are whole and resident, so the block runs
+    as it is."""
+    yield
+
+
+def get_quantizer_state_dict(model):
+    """``{quantizer name: its state_dict()}`` without calling ``model.state_dict()``
+    (reference: utils.py:489-500)."""
+    from .nn import TensorQuantizer
+
+    return {name: module.state_dict() for name, module in model.named_modules()
+            if isinstance(module, TensorQuantizer)}
+
+
+def set_quantizer_state_dict(model, quantizer_state_dict: dict):
+    """Load what ``get_quantizer_state_dict`` returned (reference: utils.py:503-511)."""
+    from .nn import TensorQuantizer
+
+    for name, module in model.named_modules():
+        if isinstance(module, TensorQuantizer) and name in quantizer_state_dict:
+            module.load_state_dict(quantizer_state_dict[name])
 
 
 def weight_attr_names(module):

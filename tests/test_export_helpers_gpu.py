@@ -127,3 +127,36 @@ def test_fp8_pc_pt_cast_of_stacked_expert_weights(dtype):
         Q.to_quantized_weight(dev[:, :, :48].contiguous(), torch.ones(3, 48, device="cuda:0"), "fp8_pc_pt")
     with pytest.raises(ValueError, match="unsqueeze"):
         Q.to_quantized_weight(dev, torch.ones(3, 7, device="cuda:0"), "fp8_pc_pt")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("quantization", ["int4_awq", "nvfp4_awq"])
+def test_resmooth_and_get_scale_of_row_chunks(quantization):
+    """Two row chunks smoothed with their own scales brought to the mean scale, block scales
+    recomputed (export/quant_utils.py:126-185), against the same expressions on the CPU."""
+    from conftest import assert_bits_equal
+    from modelopt_amd.torch.export import quant_utils as Q
+    from oracle import export, qtensor
+
+    g = torch.Generator().manual_seed(41)
+    w = (torch.randn((64, 256), generator=g) * 0.05).to(torch.bfloat16)
+    pqs = [torch.rand(256, generator=g) + 0.5 for _ in range(2)]
+    group = 128 if quantization == "int4_awq" else 16
+    weights, scales, shared = Q.resmooth_and_get_scale(w.to("cuda:0"), [p.to("cuda:0") for p in pqs], 2, group,
+                                                       quantization=quantization)
+    mean = torch.stack(pqs).mean(dim=0)
+    assert_bits_equal(shared.cpu(), mean, "shared scale")
+    want_w = torch.cat([c * p.type(c.dtype) / mean.type(c.dtype) for c, p in zip(torch.chunk(w, 2, dim=0), pqs)])
+    assert_bits_equal(weights.cpu(), want_w, "re-smoothed weights")
+    if quantization == "int4_awq":
+        want_s = torch.cat([export.get_scaling_factor_from_weight(c, group) for c in torch.chunk(want_w, 2, dim=0)])
+        assert_bits_equal(scales.cpu(), want_s, "block scales")
+    else:
+        want_s = torch.cat([qtensor.nvfp4_block_scales(c, group)[0].view(torch.uint8)
+                            for c in torch.chunk(want_w, 2, dim=0)])
+        assert scales.dtype == torch.float8_e4m3fn
+        assert torch.equal(scales.cpu().view(torch.uint8), want_s)
+    t, ts = Q.maybe_transpose_expert_weight_dimensions(torch.zeros(2, 3, 4), torch.zeros(2, 3, 1))
+    assert t.shape == (2, 4, 3) and ts.shape == (2, 1, 3)
+    same, none = Q.maybe_transpose_expert_weight_dimensions(torch.zeros(3, 4))
+    assert same.shape == (3, 4) and none is None

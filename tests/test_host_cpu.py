@@ -852,3 +852,62 @@ def test_is_quantized_linear_on_modules_and_other_objects():
     plain.__dict__["weight_quantizer"] = seq[0].weight_quantizer
     plain.weight = nn.Parameter(torch.zeros(4, 4))
     assert is_quantized_linear(plain)
+
+
+def test_small_helpers_of_the_quantization_utils():
+    """reference: utils.py:247-273 (attribute names), :339-379 (replace_function, multi_context,
+    export mode, is_pow2), :489-511 (quantizer state dicts)."""
+    import contextlib
+    import math
+
+    from modelopt_amd.torch.quantization import utils as U
+
+    names = U.quantizer_attr_names()
+    assert names.weight_quantizer == "weight_quantizer" and names.weight_scale_2 == "weight_scale_2"
+    names = U.quantizer_attr_names("gate_up_proj")
+    assert names == U.QuantizerAttrNames(
+        "gate_up_proj_weight_quantizer", "gate_up_proj_input_quantizer", "gate_up_proj_output_quantizer",
+        "gate_up_proj_weight_scale", "gate_up_proj_weight_scale_2", "gate_up_proj_input_scale",
+        "gate_up_proj_output_scale")
+    assert [n for n in range(0, 20) if U.is_pow2(n)] == [1, 2, 4, 8, 16]
+    with U.replace_function(math, "floor", lambda v: "patched"):
+        assert math.floor(1.5) == "patched" and math._floor(1.5) == 1
+    assert math.floor(1.5) == 1 and not hasattr(math, "_floor")
+    seen = []
+
+    @contextlib.contextmanager
+    def tag(t):
+        seen.append(t)
+        yield t
+
+    with U.multi_context(tag("a"), tag("b")) as entered:
+        assert entered == ["a", "b"] and seen == ["a", "b"]
+    assert not U.is_torch_export_mode()
+    with U.export_torch_mode():
+        assert U.is_torch_export_mode()
+    assert not U.is_torch_export_mode()
+    model = nn.Sequential(nn.Linear(8, 8))
+    mtq.replace_quant_module(model)
+    model[0].input_quantizer.amax = torch.tensor(3.0)
+    state = U.get_quantizer_state_dict(model)
+    assert set(state) == {"0.input_quantizer", "0.weight_quantizer", "0.output_quantizer"}
+    state = {name: {k: v.clone() for k, v in entries.items()} for name, entries in state.items()}
+    assert float(state["0.input_quantizer"]["_amax"]) == 3.0
+    model[0].input_quantizer.amax = torch.tensor(5.0)
+    U.set_quantizer_state_dict(model, state)
+    assert float(model[0].input_quantizer.amax) == 3.0
+    with U.enable_weight_access_and_writeback(model[0], model):
+        assert model[0].weight.shape == (8, 8)
+
+
+def test_private_names_of_the_functional_module():
+    """tensor_quant.py:42-59 and :286-292 by name; the eager body's errors need no strict mode
+    (checked before the kernel is reached)."""
+    from modelopt_amd.torch.quantization import tensor_quant as tq
+
+    assert tq._fp8_eager is tq.fp8_eager and tq.DISABLE_TRITON_KERNEL is False
+    assert tq.QUANT_DESC_8BIT_CONV2D_WEIGHT_PER_CHANNEL.axis == 0
+    with pytest.raises(TypeError, match="unsigned"):
+        tq._tensor_quant(torch.tensor([-1.0, 2.0]), torch.tensor(2.0), 8, True)
+    with pytest.raises(ValueError, match="amax"):
+        tq._tensor_quant(torch.tensor([1.0, 2.0]), torch.tensor(-2.0))
