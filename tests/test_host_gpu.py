@@ -800,3 +800,36 @@ def test_smoothquant_in_one_launch_equals_the_tensor_expressions(dtype, alpha, c
     for a, b in zip(eager, fused):
         assert a.dtype == b.dtype and a.shape == b.shape
         assert_bits_equal(a.cpu(), b.cpu(), f"{dtype} alpha {alpha} {case}")
+
+
+def test_work_goes_to_the_caller_s_current_stream():
+    """Kernels are enqueued on the stream that is current when the operator is called: the input
+    here is produced late on a side stream (behind a few milliseconds of GEMMs) and consumed on
+    that stream without a synchronisation; on any other stream the kernels would read it before it
+    exists.  Results against the CPU restatement."""
+    from modelopt_amd import _hip
+    from modelopt_amd.torch.quantization.utils import reduce_amax
+
+    side = torch.cuda.Stream(device=DEV)
+    g = torch.Generator().manual_seed(77)
+    host = (torch.randn(2048, 2048, generator=g) * 0.05).to(torch.bfloat16)
+    staged = host.to(DEV)
+    x = torch.zeros_like(staged)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        busy = torch.randn(8192, 8192, device=DEV, dtype=torch.bfloat16)
+        for _ in range(6):
+            busy = (busy @ busy.T) * 1e-2
+        x.copy_(staged + (busy[:2048, :2048] * 0).nan_to_num(0.0, 0.0, 0.0))   # depends on the GEMMs
+        amax = reduce_amax(x)
+        qt, wsf, wsf2 = NVFP4QTensor.quantize(x, 16)
+        y = _hip.fp8_qdq(x, amax, 1, 1, x.numel())
+        cols = torch.zeros(2048, dtype=torch.float32, device=DEV)
+        _hip.absmax_into(x, cols, 2048, 2048, 1)
+    side.synchronize()
+    assert_bits_equal(amax.cpu(), reduce.reduce_amax(host), "abs-max on the side stream")
+    p_o, w_o, _ = qtensor.nvfp4_quantize(host, 16)
+    assert_bits_equal(qt._quantized_data.cpu(), p_o, "codes on the side stream")
+    assert_bits_equal(wsf.cpu().view(torch.uint8), w_o.view(torch.uint8), "block scales on the side stream")
+    assert_bits_equal(y.cpu(), fake_quant.fp8_eager(host, reduce.reduce_amax(host)), "fp8 fake quant on the side stream")
+    assert_bits_equal(cols.cpu(), host.abs().amax(dim=0).float(), "per-column abs-max on the side stream")
