@@ -15,7 +15,7 @@ from torch import nn
 from ... import __version__, _hip
 from ..quantization.nn import SequentialQuantizer, TensorQuantizer
 from ..quantization.qtensor import FP8QTensor, MXFP4QTensor, NVFP4QTensor, QTensorWrapper
-from ..quantization.utils import (quantizer_attr_names, reduce_block_amax, true_divide,
+from ..quantization.utils import (all_positive, quantizer_attr_names, reduce_block_amax, true_divide,
                                   weight_attr_names)
 from .model_config import *  # noqa: F403
 
@@ -96,7 +96,7 @@ def get_scaling_factor(quantizer: TensorQuantizer) -> torch.Tensor | None:
         sf = NVFP4QTensor.get_weights_scaling_factor_2_from_quantizer(quantizer)
     else:
         sf = true_divide(amax.float(), quantizer.maxbound)
-    assert torch.all(sf > 0), f"scaling factor {sf} not positive."
+    assert all_positive(sf, lambda: f"scaling factor {sf} not positive."), f"scaling factor {sf} not positive."
     return sf
 
 

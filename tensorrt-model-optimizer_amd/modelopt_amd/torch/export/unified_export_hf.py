@@ -6,6 +6,7 @@ Reference: modelopt/torch/export/unified_export_hf.py:233-391 (``_export_quantiz
 packed in ONE multi-tensor kernel launch over the whole model instead of module by module.
 """
 
+import contextlib
 import json
 import warnings
 from pathlib import Path
@@ -19,9 +20,8 @@ from ..quantization.nn import SequentialQuantizer, TensorQuantizer
 from ..quantization import modes
 from ..quantization.overflow import nvfp4_quantize_flags
 from ..quantization.qtensor import NVFP4QTensor, QTensorWrapper
-from ..quantization.utils import is_quantized_linear, true_divide
+from ..quantization.utils import deferred_scale_checks, is_quantized_linear, true_divide
 from .model_config import *  # noqa: F403
-from ..quantization.conversion import set_quantizer_by_cfg_context
 from .quant_utils import (fuse_prequant_layernorm, fuse_prequant_to_linear,
                           get_activation_scaling_factor, get_quant_config,
                           get_quantization_format,
@@ -126,6 +126,21 @@ def _quantizer_on(q) -> bool:
 _is_enabled_quantizer = _quantizer_on   # the reference's name for it (unified_export_hf.py:80-87)
 
 
+@contextlib.contextmanager
+def _every_quantizer_off(model: nn.Module):
+    """What ``set_quantizer_by_cfg_context(model, {"*": {"enable": False}})`` does for the dummy
+    forward below, without saving and restoring the whole state of several hundred quantizers:
+    the enabled ones are switched off and back on."""
+    switched = [m for m in model.modules() if isinstance(m, TensorQuantizer) and not m._disabled]
+    for q in switched:
+        q._disabled = True
+    try:
+        yield
+    finally:
+        for q in switched:
+            q._disabled = False
+
+
 def requantize_resmooth_fused_llm_layers(model: nn.Module):
     """Unify what an inference engine will fuse (reference: unified_export_hf.py:90-231).
 
@@ -158,7 +173,7 @@ def requantize_resmooth_fused_llm_layers(model: nn.Module):
     groups = None
     try:
         device = next(model.parameters()).device
-        with torch.no_grad(), set_quantizer_by_cfg_context(model, {"*": {"enable": False}}):
+        with torch.no_grad(), _every_quantizer_off(model):
             model(torch.ones([1, 2], dtype=torch.long, device=device))
         groups = list(input_to_linear.items())
     except Exception as err:  # noqa: BLE001 -- any failure of a foreign forward means "not an LLM"
@@ -181,6 +196,13 @@ def requantize_resmooth_fused_llm_layers(model: nn.Module):
 
 
 def _export_hf_checkpoint(model: nn.Module, dtype: torch.dtype | None = None):
+    # the "scaling factor is positive" assertions of the per-layer getters are one host
+    # synchronisation each if made on the spot; they are made together when the export ends
+    with deferred_scale_checks():
+        return _export_hf_checkpoint_unchecked(model, dtype)
+
+
+def _export_hf_checkpoint_unchecked(model: nn.Module, dtype: torch.dtype | None = None):
     if dtype is None:
         dtype = next(model.parameters()).dtype
     requantize_resmooth_fused_llm_layers(model)

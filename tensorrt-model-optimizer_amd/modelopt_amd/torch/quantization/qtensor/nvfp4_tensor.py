@@ -10,7 +10,7 @@ import torch
 from .... import _hip
 from .. import modes
 from ..overflow import nvfp4_quantize_flags
-from ..utils import reduce_amax, reduce_block_amax, reduce_block_padding, true_divide
+from ..utils import all_positive, reduce_amax, reduce_block_amax, reduce_block_padding, true_divide
 from .base_qtensor import BaseQuantizedTensor
 
 __all__ = ["NVFP4QTensor"]
@@ -104,7 +104,9 @@ class NVFP4QTensor(BaseQuantizedTensor):
         if amax is None:
             return None
         sf = true_divide(amax.float(), quantizer.maxbound * 448.0)
-        assert torch.all(sf > 0), f" activation scaling factor {sf} not positive."
+        # one host synchronisation per layer if checked here: an export defers it to its end
+        assert all_positive(sf, lambda: f" activation scaling factor {sf} not positive."), (
+            f" activation scaling factor {sf} not positive.")
         return sf
 
     @classmethod

@@ -14,6 +14,7 @@ __all__ = [
     "reduce_block_padding", "is_quantized", "is_quantized_linear",
     "update_quant_cfg_with_kv_cache_quant", "quantizer_attr_names", "weight_attr_names",
     "enable_fake_quant", "enable_quant", "disable_calib", "reduce_sum",
+    "all_positive", "all_valid_scales", "deferred_scale_checks",
 ]
 
 
@@ -227,6 +228,7 @@ class _DeferredChecks(list):
     def __init__(self):
         super().__init__()
         self.positive = []
+        self.positive_messages = []   # one per entry of ``positive``: text, callable or None
         self.report = []
         self.report_ok = True
 
@@ -310,6 +312,7 @@ def deferred_scale_checks():
         outer = _DEFERRED_CHECKS[-1]
         outer.extend(pending)
         outer.positive.extend(pending.positive)
+        outer.positive_messages.extend(pending.positive_messages)
         if pending.report:   # the block's owner wants an answer now
             pending.report_ok = _checked([(pending.report, False)])[0]
         return
@@ -320,7 +323,13 @@ def deferred_scale_checks():
     if not valid:
         raise DeferredCheckError("detected negative, inf or nan values in a calibrated amax or scale")
     if not positive:
-        raise DeferredCheckError("pre_quant_scale should be positive")
+        # only now, on the way to an error, look for the tensor that failed and its own words
+        message = "pre_quant_scale should be positive"
+        for tensor, own in zip(pending.positive, pending.positive_messages):
+            if own is not None and not bool(torch.all(tensor > 0)):
+                message = own() if callable(own) else own
+                break
+        raise DeferredCheckError(message)
 
 
 def all_valid_scales(tensors) -> bool:
@@ -332,11 +341,13 @@ def all_valid_scales(tensors) -> bool:
     return _checked([(list(tensors), False)])[0]
 
 
-def all_positive(tensor) -> bool:
+def all_positive(tensor, message=None) -> bool:
     """True when every element is positive; inside a ``deferred_scale_checks`` block the tensor is
-    recorded and the answer comes when the block ends (``AssertionError``)."""
+    recorded and the answer comes when the block ends (``AssertionError`` with ``message`` -- a
+    text, or a callable that builds it -- if this is the tensor that failed)."""
     if _DEFERRED_CHECKS:
         _DEFERRED_CHECKS[-1].positive.append(tensor)
+        _DEFERRED_CHECKS[-1].positive_messages.append(message)
         return True
     return bool(torch.all(tensor > 0))
 

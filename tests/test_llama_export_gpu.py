@@ -401,3 +401,19 @@ def test_calibration_sweep_on_two_layers_of_the_8b_shape():
     assert model.get_submodule("model.layers.1.mlp.down_proj").weight.shape == (4096, 14336)
     k_seen = model.get_submodule("model.layers.0.self_attn.k_bmm_quantizer")
     assert k_seen.amax.numel() == 1 and float(k_seen.amax) > 0
+
+
+def test_export_reports_a_scale_that_is_not_positive_in_the_getter_s_words(tmp_path):
+    """The "scaling factor is positive" assertions of the per-layer getters (reference:
+    qtensor/nvfp4_tensor.py:112-114, export/quant_utils.py:229) are made together when the export
+    ends -- one host synchronisation instead of one per layer; a failure is an ``AssertionError``
+    with the failing getter's own message.  Outside an export the getter asserts on the spot."""
+    from modelopt_amd.torch.quantization.qtensor import NVFP4QTensor
+
+    model, _ = _quantized(copy.deepcopy(mtq.NVFP4_DEFAULT_CFG))
+    bad = model.get_submodule("model.layers.1.mlp.down_proj").input_quantizer
+    bad.amax = torch.zeros_like(bad.amax)
+    with pytest.raises(AssertionError, match="activation scaling factor .* not positive"):
+        NVFP4QTensor.get_activation_scaling_factor(bad)
+    with pytest.raises(AssertionError, match="activation scaling factor .* not positive"):
+        export_hf_checkpoint(model, export_dir=tmp_path)
