@@ -144,3 +144,24 @@ def test_block_formats_and_packs_past_the_32_bit_range(big):
     _hip.abs_colsum_into(big[HALF:], sums[2])
     assert torch.allclose(sums[0], sums[1] + sums[2], rtol=1e-5)
     assert torch.allclose(sums[0], big.float().abs().sum(dim=0), rtol=1e-4)
+
+
+def test_two_rows_of_a_billion_elements(big):
+    """The same memory seen as two rows of 2^30 + 2^19 elements: per-row reductions and per-row
+    scales with row lengths past 2^30."""
+    n = big.numel() // 2
+    two = big.view(2, n)
+    amax = torch.zeros(2, dtype=torch.float32, device=DEV)
+    _hip.absmax_into(two, amax, 1, 2, n)
+    want = torch.stack([big[:HALF].abs().amax(), big[HALF:].abs().amax()]).float()
+    assert torch.equal(amax, want) and float(amax[1]) == 3.0
+    y = _hip.fp8_qdq(two, amax.to(torch.bfloat16), 1, 2, n)
+    first = _hip.fp8_qdq(big[:HALF], amax[0:1].to(torch.bfloat16), 1, 1, n)
+    second = _hip.fp8_qdq(big[HALF:], amax[1:2].to(torch.bfloat16), 1, 1, n)
+    assert torch.equal(y.view(ROWS, K)[:HALF], first) and torch.equal(y.view(ROWS, K)[HALF:], second)
+    del y, first, second
+    scale = (amax / 127.0).contiguous()
+    q = _hip.real_quantize(two, scale, 1, 2, n, torch.float32, _hip.MO_FMT_INT8)
+    qa = _hip.real_quantize(big[:HALF], scale[0:1], 1, 1, n, torch.float32, _hip.MO_FMT_INT8)
+    qb = _hip.real_quantize(big[HALF:], scale[1:2], 1, 1, n, torch.float32, _hip.MO_FMT_INT8)
+    assert torch.equal(q.view(ROWS, K)[:HALF], qa) and torch.equal(q.view(ROWS, K)[HALF:], qb)
