@@ -165,3 +165,30 @@ def test_two_rows_of_a_billion_elements(big):
     qa = _hip.real_quantize(big[:HALF], scale[0:1], 1, 1, n, torch.float32, _hip.MO_FMT_INT8)
     qb = _hip.real_quantize(big[HALF:], scale[1:2], 1, 1, n, torch.float32, _hip.MO_FMT_INT8)
     assert torch.equal(q.view(ROWS, K)[:HALF], qa) and torch.equal(q.view(ROWS, K)[HALF:], qb)
+
+
+@pytest.mark.parametrize("rows,k", [(1 << 24, 8), (8, 1 << 24), (3, (1 << 23) + 8), ((1 << 22) + 3, 24),
+                                    (1, 1 << 27), (1 << 27, 1)])
+def test_extreme_aspect_ratios(rows, k):
+    """Very tall and very wide matrices through the per-row / per-column reductions, the column
+    scaling and the per-row fake quant, against the same tensor expressions on the device (a
+    maximum and a rounded product have one right answer)."""
+    g = torch.Generator(device=DEV).manual_seed(rows % 1000 + k % 1000)
+    x = (torch.randn(rows, k, generator=g, device=DEV) * 0.05).to(torch.bfloat16)
+    acc = torch.zeros(rows, dtype=torch.float32, device=DEV)
+    _hip.absmax_into(x, acc, 1, rows, k)
+    assert torch.equal(acc, x.abs().amax(dim=1).float())
+    cols = torch.zeros(k, dtype=torch.float32, device=DEV)
+    _hip.absmax_into(x, cols, rows, k, 1)
+    assert torch.equal(cols, x.abs().amax(dim=0).float())
+    s = (torch.rand(k, generator=g, device=DEV) + 0.5).to(torch.bfloat16)
+    assert torch.equal(_hip.mul_cols(x, s), x * s)
+    row_amax = acc.to(torch.bfloat16)
+    row_amax[row_amax == 0] = 1.0
+    y = _hip.int_qdq(x, row_amax, 1, rows, k, 8, False, False)
+    sample = slice(0, rows, max(1, rows // 64))
+    assert_bits_equal(y[sample].cpu(), fake_quant.tensor_quant(x[sample].cpu(), row_amax[sample].cpu().reshape(-1, 1),
+                                                              8, False, False), "per-row INT8")
+    sums = torch.zeros(k, dtype=torch.float32, device=DEV)
+    _hip.abs_colsum_into(x, sums)
+    assert torch.allclose(sums, x.float().abs().sum(dim=0), rtol=2e-4, atol=1e-6)
