@@ -811,7 +811,7 @@ extern "C" int mo_value_ranges(const void* const* xs, const int64_t* counts, con
         if (i < n) {
             const int64_t chunks = (counts[i] + mo::kRangeChunk - 1) / mo::kRangeChunk;
             grid += chunks > 0 ? chunks : 1;   // an empty tensor still owns one (+inf, -inf, 0) entry
-            if (grid > out_chunks) return MO_ERR_TOO_LARGE;
+            if (grid > out_chunks || grid > 0x7FFFFFFF) return MO_ERR_TOO_LARGE;
         }
     }
     jobs.first[mo::kRangeJobs] = (int)grid;
