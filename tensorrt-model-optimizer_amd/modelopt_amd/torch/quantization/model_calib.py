@@ -665,12 +665,17 @@ def _fused_weight_path(module):
         torch.bfloat16, torch.float16, torch.float32)
 
 
+_SEARCH_TOKENS = 512   # token rows one launch of the search kernel takes (mo_awq_search_losses)
+
+
 def _one_launch_search(module, x, w, ref, x_scales, w_scales, block, sq_err) -> bool:
-    """All alphas of a search step in one kernel launch (weights quantised on the fly in front
-    of the matrix cores, the loss reduced in the epilogue): used when the layer is a plain bf16
-    linear without bias whose input and output quantizers are switched off and the batch has at
-    most 512 tokens -- the regime where per-alpha launches and the repeated weight pass dominate.
-    Returns False, with nothing launched and ``sq_err`` untouched, when that is not the case."""
+    """All alphas of a search step in one kernel launch per 512 tokens (weights quantised on the
+    fly in front of the matrix cores, the loss reduced in the epilogue): used when the layer is a
+    plain bf16 linear without bias whose input and output quantizers are switched off.  The loss
+    is a sum over tokens, so a longer batch goes through in slices of 512 rows that add into the
+    same ``sq_err`` (per-alpha launches with a library GEMM cost more at every batch size: they
+    re-scale and re-quantise per alpha and pass over the activations three times).
+    Returns False, with nothing launched and ``sq_err`` untouched, when the layer is not covered."""
     if module.bias is not None or w.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
         return False
     for name in ("input_quantizer", "output_quantizer"):
@@ -682,12 +687,19 @@ def _one_launch_search(module, x, w, ref, x_scales, w_scales, block, sq_err) -> 
     q = module.weight_quantizer
     # what mo_awq_search_losses takes, checked before the activations of every alpha are written
     # out for it (n_alpha x tokens x K values)
-    if (tokens == 0 or tokens > 512 or k % 128 or n % 128 or block not in (32, 64, 128) or q._unsigned
+    if (tokens == 0 or k % 128 or n % 128 or block not in (32, 64, 128) or q._unsigned
             or any(t.data_ptr() % 16 for t in (x, w, w_scales, x_scales))):
         return False
-    xs = _hip.awq_scaled_activations(x.view(tokens, k), x_scales)
-    return _hip.awq_search_losses_into(xs, w, w_scales, ref.view(tokens, -1), block, q._num_bits,
-                                       q._unsigned, q._narrow_range, sq_err)
+    rows, outs = x.view(tokens, k), ref.view(tokens, -1)
+    for t0 in range(0, tokens, _SEARCH_TOKENS):
+        t1 = min(tokens, t0 + _SEARCH_TOKENS)
+        xs = _hip.awq_scaled_activations(rows[t0:t1], x_scales)
+        if not _hip.awq_search_losses_into(xs, w, w_scales, outs[t0:t1], block, q._num_bits, q._unsigned,
+                                           q._narrow_range, sq_err):
+            if t0:   # cannot happen: every slice has the shape the first one was accepted with
+                raise RuntimeError("the search kernel refused a later slice of a batch it had started on")
+            return False
+    return True
 
 
 def _awq_forward(self, input, *args, **kwargs):

@@ -684,8 +684,9 @@ def test_k_and_v_calibrate_in_one_launch():
 
 
 @pytest.mark.parametrize("seed,n,k,tokens", [(11, 128, 256, 64), (12, 256, 512, 200), (13, 384, 384, 96),
-                                             (14, 128, 1024, 512), (15, 512, 256, 33), (16, 256, 256, 300)])
-def test_awq_lite_selects_the_oracle_s_alpha_on_several_layers(seed, n, k, tokens):
+                                             (14, 128, 1024, 512), (15, 512, 256, 33), (16, 256, 256, 300),
+                                             (17, 256, 256, 513), (18, 128, 384, 1300), (19, 256, 128, 2048)])
+def test_awq_lite_selects_the_oracle_s_alpha_on_several_layers(seed, n, k, tokens, monkeypatch):
     """The one-launch search scores the alphas with arithmetic that differs from the CPU path's by
     an ulp of a rare weight; what matters downstream is which alpha wins.  Several layers and
     seeds: same best alpha as the CPU restatement of the search loop, losses within 1e-3, and the
@@ -698,7 +699,14 @@ def test_awq_lite_selects_the_oracle_s_alpha_on_several_layers(seed, n, k, token
     model = copy.deepcopy(ref).to(DEV)
     cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
     cfg["algorithm"] = {"method": "awq_lite", "alpha_step": 0.1, "debug": True}
+    # batches of more than 512 tokens go through the search kernel in slices of 512 rows
+    from modelopt_amd import _hip
+    launches, real = [], _hip.awq_search_losses_into
+    monkeypatch.setattr(_hip, "awq_search_losses_into",
+                        lambda xs, *a: launches.append(xs.shape[2]) or real(xs, *a))
     mtq.quantize(model, cfg, lambda m: [m(b.to(DEV)) for b in batches])
+    per_batch = [min(512, tokens - t) for t in range(0, tokens, 512)]
+    assert launches == per_batch * len(batches)
     losses, best_alpha, best_scale, _, _ = oawq.awq_lite_search(ref.proj.weight.data, batches, 0.1, 128)
     h = model.proj.awq_lite
     assert h.best_alpha == best_alpha, (h.loss, losses)
