@@ -520,6 +520,15 @@ int mo_awq_search_losses(const void* xs, const void* w, const void* s, const voi
                          int64_t block_size, int num_bits, int is_unsigned, int narrow_range,
                          double* loss, void* stream);
 
+/* The same for a linear layer with a bias (the F.linear of nn.Linear.forward under
+ * QuantLinearConvBase.forward, TQ/nn/modules/quant_module.py:148-169, which the search forward
+ * TQ/model_calib.py:645-690 runs once per alpha): bias[n] (dtype of w, or
+ * null for none) is added to the fp32 sums before they are rounded, out_a = bf16(sum + bias). */
+int mo_awq_search_losses_biased(const void* xs, const void* w, const void* s, const void* ref,
+                                const void* bias, int64_t n_alpha, int64_t tokens, int64_t n,
+                                int64_t k, int dtype, int64_t block_size, int num_bits,
+                                int is_unsigned, int narrow_range, double* loss, void* stream);
+
 /* AWQ clip search, all ratios and all weight blocks of one [n, k] weight on one batch of
  * `tokens` activations in one launch.  For block (row, b) of `block_size` input channels and
  * ratio r, with T the weight dtype and every step rounded as the tensor expression rounds it:

@@ -56,12 +56,13 @@ constexpr int kXcds = 8;            // accelerator dies of the chip, each with i
 
 // One column tile of 32 * NG output features (NG = 4 or 3) for alpha `a`, starting at feature n0.
 // RB = 32-row blocks per wavefront; the workgroup covers 8 * 32 * RB token rows.
-template <int RB, int NG>
+template <int RB, int NG, bool BIAS>
 __device__ __forceinline__ void awq_search_tile(
     const uint16_t* __restrict__ xs,   // [A][K / 8][T][8] bf16, activations * (1 / s[a])
     const uint16_t* __restrict__ w,    // [N, K] bf16
     const uint16_t* __restrict__ s,    // [A, K] bf16
     const uint16_t* __restrict__ ref,  // [T, N] bf16
+    const uint16_t* __restrict__ bias, // [N] bf16, read when BIAS: added to the fp32 sums before rounding
     int T, int N, int K, int a, int n0, int lg_g, float bound, double* __restrict__ loss,
     u32x4 (&tile)[2][kSearchTileN][16], double (&red)[kSearchWaves]) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -303,11 +304,17 @@ __device__ __forceinline__ void awq_search_tile(
     // masked out of the sum)
     float part = 0.0f;
     if (has_rows) {
+        // the column's bias is fetched here, behind a statement the compiler may not move work
+        // across: computed any earlier its address would sit in registers through the k loop
+        int col = n0 + fr;
+        if constexpr (BIAS) asm volatile("" : "+v"(col));
 #pragma unroll
         for (int mb = 0; mb < RB; ++mb)
 #pragma unroll
             for (int nb = 0; nb < NG; ++nb) {
                 const uint16_t* rcol = ref + n0 + nb * 32 + fr;
+                float add = 0.0f;
+                if constexpr (BIAS) add = bf16_bits_to_f32(bias[col + nb * 32]);
                 uint16_t rv[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
@@ -318,7 +325,7 @@ __device__ __forceinline__ void awq_search_tile(
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int t = row_base + mb * 32 + 8 * (i / 4) + 4 * kg + (i % 4);
-                    const float o = round_to_bf16(acc[mb][nb][i]);
+                    const float o = round_to_bf16(BIAS ? acc[mb][nb][i] + add : acc[mb][nb][i]);
                     const float d = round_to_bf16(o - bf16_bits_to_f32(rv[i]));
                     part += t < T ? d * d : 0.0f;
                 }
@@ -349,10 +356,11 @@ __device__ __forceinline__ void awq_search_tile(
 // tiles of one alpha run side by side on one XCD, and the 4 MB of activations they walk through
 // in step are fetched into that L2 once instead of once per XCD.  The grid is
 // 8 * (per_wide + per_narrow) workgroups; surplus ones leave at once.
-template <int RB>
+template <int RB, bool BIAS>
 __global__ __launch_bounds__(512) void awq_search_kernel(
     const uint16_t* __restrict__ xs, const uint16_t* __restrict__ w, const uint16_t* __restrict__ s,
-    const uint16_t* __restrict__ ref, int T, int N, int K, int n_alpha, int wide, int narrow,
+    const uint16_t* __restrict__ ref, const uint16_t* __restrict__ bias, int T, int N, int K,
+    int n_alpha, int wide, int narrow,
     int per_wide, int per_narrow, int lg_g, float bound, double* __restrict__ loss) {
     // quantised weight tile, two buffers: [128 rows][16 chunk slots] of 16 bytes; the slot of
     // chunk c in row r is c ^ (r & 15) so that both the writers (16 lanes per row) and the
@@ -363,12 +371,12 @@ __global__ __launch_bounds__(512) void awq_search_kernel(
     if (slot < per_wide) {
         const int i = xcd * per_wide + slot;
         if (i >= n_alpha * wide) return;
-        awq_search_tile<RB, 4>(xs, w, s, ref, T, N, K, i / wide, (i % wide) * 128, lg_g, bound,
+        awq_search_tile<RB, 4, BIAS>(xs, w, s, ref, bias, T, N, K, i / wide, (i % wide) * 128, lg_g, bound,
                                loss, tile, red);
     } else {
         const int i = xcd * per_narrow + (slot - per_wide);
         if (i >= n_alpha * narrow) return;
-        awq_search_tile<RB, 3>(xs, w, s, ref, T, N, K, i / narrow, wide * 128 + (i % narrow) * 96,
+        awq_search_tile<RB, 3, BIAS>(xs, w, s, ref, bias, T, N, K, i / narrow, wide * 128 + (i % narrow) * 96,
                                lg_g, bound, loss, tile, red);
     }
 }
@@ -465,6 +473,14 @@ extern "C" int mo_awq_search_losses(const void* xs, const void* w, const void* s
                                     int64_t n_alpha, int64_t tokens, int64_t n, int64_t k,
                                     int dtype, int64_t block_size, int num_bits, int is_unsigned,
                                     int narrow_range, double* loss, void* stream) {
+    return mo_awq_search_losses_biased(xs, w, s, ref, nullptr, n_alpha, tokens, n, k, dtype, block_size,
+                                       num_bits, is_unsigned, narrow_range, loss, stream);
+}
+
+extern "C" int mo_awq_search_losses_biased(const void* xs, const void* w, const void* s, const void* ref,
+                                           const void* bias, int64_t n_alpha, int64_t tokens, int64_t n,
+                                           int64_t k, int dtype, int64_t block_size, int num_bits,
+                                           int is_unsigned, int narrow_range, double* loss, void* stream) {
     if (n_alpha < 0 || tokens < 0 || n < 0 || k < 0 || num_bits < 2 || num_bits > 16) return MO_ERR_ARG;
     if (dtype != MO_BF16) return MO_ERR_UNSUPPORTED;
     if (n_alpha == 0 || tokens == 0 || n == 0 || k == 0) return MO_OK;
@@ -477,7 +493,7 @@ extern "C" int mo_awq_search_losses(const void* xs, const void* w, const void* s
         n_alpha > 65535 || n > 0x7FFFFFFF || tokens * k > 0x7FFFFFFF || k >= (1 << 24) ||
         (n_alpha + 8) * (n / mo::kSearchTileN) > 0x7FFFFFFF)
         return MO_ERR_UNSUPPORTED;
-    if ((((uintptr_t)xs | (uintptr_t)w | (uintptr_t)s) & 15u) || ((uintptr_t)ref & 1u))
+    if ((((uintptr_t)xs | (uintptr_t)w | (uintptr_t)s) & 15u) || (((uintptr_t)ref | (uintptr_t)bias) & 1u))
         return MO_ERR_UNSUPPORTED;
     const float bound = (float)((1 << (num_bits - 1 + (is_unsigned ? 1 : 0))) - 1);
     // signed grids only: the kernel relies on |w * s| <= block amax keeping every code inside
@@ -505,13 +521,18 @@ extern "C" int mo_awq_search_losses(const void* xs, const void* w, const void* s
     const int64_t per_wide = (n_alpha * wide + mo::kXcds - 1) / mo::kXcds;
     const int64_t per_narrow = (n_alpha * narrow + mo::kXcds - 1) / mo::kXcds;
     const dim3 grid((unsigned)((per_wide + per_narrow) * mo::kXcds));
-#define CALL(RB)                                                                           \
-    mo::awq_search_kernel<RB><<<grid, 512, 0, st>>>(                                       \
+#define CALL(RB, BIAS)                                                                     \
+    mo::awq_search_kernel<RB, BIAS><<<grid, 512, 0, st>>>(                                 \
         (const uint16_t*)xs, (const uint16_t*)w, (const uint16_t*)s, (const uint16_t*)ref, \
-        (int)tokens, (int)n, (int)k, (int)n_alpha, (int)wide, narrow, (int)per_wide,       \
-        (int)per_narrow, lg_g, bound, loss)
-    if (tokens <= 256) CALL(1);
-    else CALL(2);
+        (const uint16_t*)bias, (int)tokens, (int)n, (int)k, (int)n_alpha, (int)wide, narrow, \
+        (int)per_wide, (int)per_narrow, lg_g, bound, loss)
+    if (tokens <= 256) {
+        if (bias) CALL(1, true);
+        else CALL(1, false);
+    } else {
+        if (bias) CALL(2, true);
+        else CALL(2, false);
+    }
 #undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }

@@ -63,6 +63,7 @@ SIGNATURES = {
     "mo_awq_scale_grid": [_P, _P, _P, _I64, _I64, _P, _P, _P, _INT, _P],
     "mo_awq_scale_activations": [_P, _P, _I64, _I64, _I64, _INT, _P, _P],
     "mo_awq_search_losses": [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _INT, _I64, _INT, _INT, _INT, _P, _P],
+    "mo_awq_search_losses_biased": [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _INT, _I64, _INT, _INT, _INT, _P, _P],
     "mo_awq_clip_losses": [_P, _I64, _P, _I64, _I64, _INT, _I64, _P, _INT, _P, _INT, _INT, _INT, _INT, _P, _P],
     "mo_abs_colsum": [_P, _I64, _I64, _INT, _P, _I64, _P, _P],
     "mo_abs_colsum_staged": [_P, _I64, _I64, _INT, _P, _I64, _P, _P, _I64, _P],
@@ -734,11 +735,11 @@ def awq_scaled_activations(x, inv_s):
     return xs
 
 
-def awq_search_losses_into(xs, w, s, ref, block_size, num_bits, unsigned, narrow_range, loss):
-    """loss[a] += squared error of ``bf16(x_a @ qdq(bf16(w * s[a]))^T)`` against ``ref``, all
-    alphas in one launch; ``xs`` = ``awq_scaled_activations(x, 1 / s)``.  Returns False (nothing
-    launched) when the shapes or dtype are outside what the kernel covers."""
-    _require_device(xs, w, s, ref, loss)
+def awq_search_losses_into(xs, w, s, ref, block_size, num_bits, unsigned, narrow_range, loss, bias=None):
+    """loss[a] += squared error of ``bf16(x_a @ qdq(bf16(w * s[a]))^T + bias)`` against ``ref``,
+    all alphas in one launch; ``xs`` = ``awq_scaled_activations(x, 1 / s)``.  Returns False
+    (nothing launched) when the shapes or dtype are outside what the kernel covers."""
+    _require_device(xs, w, s, ref, loss, bias)
     n_alpha, kc, tokens, eight = xs.shape
     k = kc * 8
     n = w.shape[0]
@@ -748,11 +749,14 @@ def awq_search_losses_into(xs, w, s, ref, block_size, num_bits, unsigned, narrow
     assert loss.dtype == torch.float64 and loss.numel() == n_alpha and loss.is_contiguous()
     if not (xs.dtype == w.dtype == s.dtype == ref.dtype == torch.bfloat16):
         return False
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != n or not bias.is_contiguous()):
+        return False
     lib = load()
     with torch.cuda.device(xs.device):
-        rc = lib.mo_awq_search_losses(_ptr(xs), _ptr(w), _ptr(s), _ptr(ref), n_alpha, tokens, n, k,
-                                      MO_BF16, block_size, int(num_bits), int(bool(unsigned)),
-                                      int(bool(narrow_range)), _ptr(loss), _stream(xs))
+        rc = lib.mo_awq_search_losses_biased(_ptr(xs), _ptr(w), _ptr(s), _ptr(ref), _ptr(bias), n_alpha,
+                                             tokens, n, k, MO_BF16, block_size, int(num_bits),
+                                             int(bool(unsigned)), int(bool(narrow_range)), _ptr(loss),
+                                             _stream(xs))
     if rc == MO_ERR_UNSUPPORTED:
         return False
     if rc != 0:

@@ -671,12 +671,13 @@ _SEARCH_TOKENS = 512   # token rows one launch of the search kernel takes (mo_aw
 def _one_launch_search(module, x, w, ref, x_scales, w_scales, block, sq_err) -> bool:
     """All alphas of a search step in one kernel launch per 512 tokens (weights quantised on the
     fly in front of the matrix cores, the loss reduced in the epilogue): used when the layer is a
-    plain bf16 linear without bias whose input and output quantizers are switched off.  The loss
+    plain bf16 linear (with or without bias) whose input and output quantizers are switched off.  The loss
     is a sum over tokens, so a longer batch goes through in slices of 512 rows that add into the
     same ``sq_err`` (per-alpha launches with a library GEMM cost more at every batch size: they
     re-scale and re-quantise per alpha and pass over the activations three times).
     Returns False, with nothing launched and ``sq_err`` untouched, when the layer is not covered."""
-    if module.bias is not None or w.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
+    bias = module.bias
+    if w.dtype != torch.bfloat16 or x.dtype != torch.bfloat16 or (bias is not None and bias.dtype != w.dtype):
         return False
     for name in ("input_quantizer", "output_quantizer"):
         quantizer = getattr(module, name, None)
@@ -695,7 +696,8 @@ def _one_launch_search(module, x, w, ref, x_scales, w_scales, block, sq_err) -> 
         t1 = min(tokens, t0 + _SEARCH_TOKENS)
         xs = _hip.awq_scaled_activations(rows[t0:t1], x_scales)
         if not _hip.awq_search_losses_into(xs, w, w_scales, outs[t0:t1], block, q._num_bits, q._unsigned,
-                                           q._narrow_range, sq_err):
+                                           q._narrow_range, sq_err,
+                                           None if bias is None else bias.data.contiguous()):
             if t0:   # cannot happen: every slice has the shape the first one was accepted with
                 raise RuntimeError("the search kernel refused a later slice of a batch it had started on")
             return False

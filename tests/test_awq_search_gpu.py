@@ -69,6 +69,37 @@ def test_column_tiles_of_two_widths(tokens, n, k, n_alpha):
     assert int(got.argmin()) == int(want.argmin())
 
 
+@pytest.mark.parametrize("tokens,n,k", [(96, 128, 256), (512, 384, 512), (300, 1536, 128)])
+def test_layer_with_a_bias(tokens, n, k):
+    """``bf16(sum + bias)`` in the epilogue: against the same step with a library GEMM that adds
+    the bias on the device, and against the CPU restatement of the loop body with ``F.linear(xs,
+    wq, bias)``."""
+    x, w, s = _problem(tokens, n, k, 4, tokens + k)
+    bias = (0.3 * torch.randn(n, generator=torch.Generator().manual_seed(n))).to(torch.bfloat16)
+    ref = F.linear(x, w, bias)
+    want_cpu = []
+    for i in range(s.shape[0]):
+        xs = x * (1 / s[i].float()).to(torch.bfloat16)
+        out = F.linear(xs, oawq.int4_block_qdq(w * s[i], 128), bias)
+        want_cpu.append((out - ref).float().pow(2).sum().double())
+    want_cpu = torch.stack(want_cpu)
+    xd, wd, sd, bd = (t.to(DEV) for t in (x, w, s, bias))
+    ref_d = ref.to(DEV).contiguous()
+    xs = _hip.awq_scaled_activations(xd, (1 / sd.float()).to(torch.bfloat16))
+    got = torch.zeros(s.shape[0], dtype=torch.float64, device=DEV)
+    assert _hip.awq_search_losses_into(xs, wd, sd.contiguous(), ref_d, 128, 4, False, False, got, bd)
+    want_dev = torch.zeros(s.shape[0], dtype=torch.float64, device=DEV)
+    for i in range(s.shape[0]):
+        xi = _hip.mul_cols(xd, (1 / sd[i].float()).to(torch.bfloat16))
+        wq = _hip.scale_block_int_qdq(wd, sd[i].contiguous(), 128, 4, False, False)
+        _hip.sq_diff_sum_into(F.linear(xi, wq, bd).contiguous(), ref_d, want_dev[i:i + 1])
+    assert torch.allclose(got, want_dev, rtol=1e-3, atol=0), (got, want_dev)
+    assert torch.allclose(got.cpu(), want_cpu, rtol=1e-3, atol=0), (got, want_cpu)
+    without = torch.zeros(s.shape[0], dtype=torch.float64, device=DEV)
+    assert _hip.awq_search_losses_into(xs, wd, sd.contiguous(), ref_d, 128, 4, False, False, without)
+    assert (without > 1.3 * got).all(), "the bias must matter in this case"
+
+
 def test_accumulates_and_rejects_uncovered_shapes():
     x, w, s = (t.to(DEV) for t in _problem(64, 128, 128, 2, 3))
     ref = F.linear(x, w).contiguous()
