@@ -841,3 +841,40 @@ def test_work_goes_to_the_caller_s_current_stream():
     assert_bits_equal(wsf.cpu().view(torch.uint8), w_o.view(torch.uint8), "block scales on the side stream")
     assert_bits_equal(y.cpu(), fake_quant.fp8_eager(host, reduce.reduce_amax(host)), "fp8 fake quant on the side stream")
     assert_bits_equal(cols.cpu(), host.abs().amax(dim=0).float(), "per-column abs-max on the side stream")
+
+
+@pytest.mark.parametrize("tokens", [96, 700])
+def test_awq_lite_on_a_layer_with_a_bias_takes_the_search_kernel(tokens, monkeypatch):
+    """A linear with a bias goes through the one-launch search (its bias added in the kernel's
+    epilogue) and ends where the per-alpha route ends: same alpha, losses within 1e-3, the same
+    folded weight and input scale bit for bit."""
+    from modelopt_amd.torch.quantization import model_calib
+
+    g = torch.Generator().manual_seed(23)
+    ref = _OneLinear(n=256, k=384, seed=23)
+    ref.proj.bias = nn.Parameter((0.2 * torch.randn(256, generator=g)).to(torch.bfloat16))
+    c = torch.exp(torch.randn(384, generator=g))
+    batches = [(torch.randn(tokens, 384, generator=g) * c).to(torch.bfloat16) for _ in range(2)]
+    cfg = copy.deepcopy(mtq.INT4_AWQ_CFG)
+    cfg["algorithm"] = {"method": "awq_lite", "alpha_step": 0.1, "debug": True}
+    results = []
+    for one_launch in (True, False):
+        model = copy.deepcopy(ref).to(DEV)
+        taken = []
+        real = model_calib._one_launch_search
+        if one_launch:
+            monkeypatch.setattr(model_calib, "_one_launch_search",
+                                lambda *a: taken.append(real(*a)) or taken[-1])
+        else:
+            monkeypatch.setattr(model_calib, "_one_launch_search", lambda *a: False)
+        mtq.quantize(model, copy.deepcopy(cfg), lambda m: [m(b.to(DEV)) for b in batches])
+        monkeypatch.setattr(model_calib, "_one_launch_search", real)
+        assert not one_launch or taken == [True, True]
+        results.append((model.proj.awq_lite, model.proj.weight.detach().clone(),
+                        model.proj.input_quantizer.pre_quant_scale.clone()))
+    (fast, w_fast, p_fast), (slow, w_slow, p_slow) = results
+    assert fast.best_alpha == slow.best_alpha
+    for a in slow.loss:
+        assert fast.loss[a] == pytest.approx(slow.loss[a], rel=1e-3), f"alpha {a}"
+    assert_bits_equal(w_fast.cpu(), w_slow.cpu(), "folded weight")
+    assert_bits_equal(p_fast.cpu(), p_slow.cpu(), "input scale")
