@@ -21,6 +21,7 @@ from . import calib
 from .calib.max import MaxCalibrator
 from .conversion import set_quantizer_by_cfg_context
 from .nn import QuantModule, SequentialQuantizer, TensorQuantizer
+from .nn.modules.quant_linear import _QuantLinear
 from .nn.modules.tensor_quantizer import calibration_pass
 from .utils import all_positive, all_valid_scales, deferred_scale_checks, is_quantized_linear
 
@@ -748,11 +749,26 @@ def _awq_forward(self, input, *args, **kwargs):
             helper.sq_err_steps.append((sq_err, ref.numel()))
             helper.num_search_steps += 1
             return out_actual
+    # a plain quantised linear (``F.linear`` between its three quantizers) whose weight
+    # quantizer is of another kind -- NVFP4, a sequential INT4 + FP8 pair -- still needs neither
+    # the scale buffers on the quantizers nor the trip through the module's forward: a
+    # quantizer multiplies by its pre-quant scale before anything else, in the tensor's dtype,
+    # which is the column scaling below
+    plain = (not fused and not args and not kwargs
+             and getattr(self._forward_no_awq, "__func__", None) is _QuantLinear.forward
+             and input.is_cuda and self.weight.dim() == 2)
+    if plain:
+        x_in = input.contiguous()
+        w_in = self.weight.data.contiguous()
     for i in range(len(helper.alphas)):
         if fused:
             xs = self.input_quantizer(_hip.mul_cols(x_in, x_scales[i]))
             wq = _hip.scale_block_int_qdq(w_in, w_scales[i], block, q._num_bits, q._unsigned,
                                           q._narrow_range)
+            out = self.output_quantizer(F.linear(xs, wq, self.bias))
+        elif plain:
+            xs = self.input_quantizer(_hip.mul_cols(x_in, x_scales[i]))
+            wq = self.weight_quantizer(_hip.mul_cols(w_in, w_scales[i]))
             out = self.output_quantizer(F.linear(xs, wq, self.bias))
         else:
             self.input_quantizer.pre_quant_scale = x_scales[i]

@@ -878,3 +878,33 @@ def test_awq_lite_on_a_layer_with_a_bias_takes_the_search_kernel(tokens, monkeyp
         assert fast.loss[a] == pytest.approx(slow.loss[a], rel=1e-3), f"alpha {a}"
     assert_bits_equal(w_fast.cpu(), w_slow.cpu(), "folded weight")
     assert_bits_equal(p_fast.cpu(), p_slow.cpu(), "input scale")
+
+
+@pytest.mark.parametrize("cfg_name", ["NVFP4_AWQ_LITE_CFG", "W4A8_AWQ_BETA_CFG"])
+def test_awq_lite_lean_per_alpha_route_equals_the_route_through_the_module(cfg_name, monkeypatch):
+    """Weight quantizers the search kernel does not cover (NVFP4 blocks, the INT4 + FP8 pair) are
+    scored alpha by alpha; for a plain quantised linear that loop scales the columns itself and
+    calls the three quantizers directly instead of writing pre-quant scales onto them and going
+    through the module's forward.  Same kernels on the same values: every per-alpha loss, the
+    folded weight and the input scale are bit for bit what the route through the module gives."""
+    from modelopt_amd.torch.quantization import model_calib
+
+    g = torch.Generator().manual_seed(29)
+    ref = _OneLinear(n=256, k=384, seed=29)
+    c = torch.exp(torch.randn(384, generator=g))
+    batches = [(torch.randn(70, 384, generator=g) * c).to(torch.bfloat16) for _ in range(2)]
+    cfg = copy.deepcopy(getattr(mtq, cfg_name))
+    algorithm = cfg["algorithm"] if isinstance(cfg["algorithm"], dict) else {"method": cfg["algorithm"]}
+    cfg["algorithm"] = {**algorithm, "debug": True}
+    results = []
+    for lean in (True, False):
+        if not lean:
+            monkeypatch.setattr(model_calib, "_QuantLinear", type("Other", (), {"forward": None}))
+        model = copy.deepcopy(ref).to(DEV)
+        mtq.quantize(model, copy.deepcopy(cfg), lambda m: [m(b.to(DEV)) for b in batches])
+        results.append((model.proj.awq_lite, model.proj.weight.detach().clone(),
+                        model.proj.input_quantizer.pre_quant_scale.clone()))
+    (fast, w_fast, p_fast), (slow, w_slow, p_slow) = results
+    assert fast.loss == slow.loss and fast.best_alpha == slow.best_alpha
+    assert_bits_equal(w_fast.cpu(), w_slow.cpu(), "folded weight")
+    assert_bits_equal(p_fast.cpu(), p_slow.cpu(), "input scale")
