@@ -173,6 +173,27 @@ int mo_int_qdq(const void* x, void* y, int64_t outer, int64_t axis, int64_t inne
                const void* amax, int amax_dtype, int num_bits, int is_unsigned,
                int narrow_range, void* stream);
 
+/* FP8 / integer fake quantisation with one amax per two-dimensional block: x viewed as
+ * [rows, cols], amax[(row / block_rows) * (cols / block_cols) + col / block_cols] -- the layout a
+ * quantizer with block_sizes on the last two dims gives its amax (FP8_2D_BLOCKWISE_WEIGHT_ONLY_CFG,
+ * TQ/config.py; the reshape to [rows / br, br, cols / bc, bc] with the amax on dims 0 and 2 of
+ * TQ/nn/modules/tensor_quantizer.py:755-782, for which the reference's kernels fall back to the
+ * eager expressions, TQ/tensor_quant.py:75).  Same arithmetic as mo_fp8_qdq / mo_int_qdq, no
+ * transposed copy.  rows % block_rows == 0, cols % block_cols == 0 (the caller pads),
+ * block_cols % 8 == 0 and 16-byte aligned tensors, MO_ERR_UNSUPPORTED otherwise.  y may alias x. */
+int mo_fp8_qdq_blocks2d(const void* x, void* y, int64_t rows, int64_t cols, int64_t block_rows,
+                        int64_t block_cols, int dtype, const void* amax, int amax_dtype, int saturate,
+                        void* stream);
+int mo_int_qdq_blocks2d(const void* x, void* y, int64_t rows, int64_t cols, int64_t block_rows,
+                        int64_t block_cols, int dtype, const void* amax, int amax_dtype, int num_bits,
+                        int is_unsigned, int narrow_range, void* stream);
+
+/* acc[b] = max(acc[b], abs-max of block b) for the same blocks (reduce_amax over dims 1 and 3 of
+ * the reshaped tensor, TQ/utils.py:156-188 under TQ/nn/modules/tensor_quantizer.py:505-514): one
+ * workgroup per block.  Same preconditions. */
+int mo_absmax_blocks2d(const void* x, int64_t rows, int64_t cols, int64_t block_rows,
+                       int64_t block_cols, int dtype, float* acc, void* stream);
+
 /* NVFP4 dynamic-block quantize-dequantize of x[rows, k] with blocks of `block_size` (8, 16 or
  * 32) along k (zero padded).  Replaces fp4_fake_quant_block (TQ/triton/fp4_kernel.py:141-208)
  * and fused_amax_convert for (E2M1, E4M3) (TQ/src/tensor_quant_mx.cu:355).

@@ -598,6 +598,43 @@ static int scratch_address(uint32_t** out) {
 }
 
 
+// ---------------------------------------------------------------- two-dimensional blocks
+// acc[b] = max(acc[b], abs-max of tile b) for x viewed as [rows, cols] cut into tiles of
+// block_rows x block_cols elements, b = (row / block_rows) * (cols / block_cols) + col /
+// block_cols: one workgroup per tile (a 128 x 128 tile is 32 KB of bf16), no atomics.
+template <int DT>
+__global__ __launch_bounds__(256) void absmax_blocks2d_kernel(const void* __restrict__ x, int64_t cols,
+                                                              uint32_t block_rows, uint32_t block_chunks,
+                                                              uint32_t blocks_across,
+                                                              uint32_t* __restrict__ acc) {
+    __shared__ uint32_t smem[8];
+    const int64_t tile_row = blockIdx.x / blocks_across;
+    const uint32_t across = blockIdx.x - (uint32_t)tile_row * blocks_across;
+    const int64_t base = tile_row * block_rows * cols + (int64_t)across * block_chunks * 8;
+    const uint32_t total = block_rows * block_chunks;   // 16-byte (fp32: 32-byte) chunks of the tile
+    AbsAcc<DT> a;
+    uint32_t q = threadIdx.x;
+    for (; q + 768 < total; q += 1024) {   // four loads of a lane in flight
+        RawChunk<DT> raw[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t qq = q + u * 256, r = qq / block_chunks;
+            load_raw<DT>(x, base + (int64_t)r * cols + (int64_t)(qq - r * block_chunks) * 8, raw[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) a.raw(raw[u]);
+    }
+    for (; q < total; q += 256) {
+        const uint32_t r = q / block_chunks;
+        a.chunk(x, base + (int64_t)r * cols + (int64_t)(q - r * block_chunks) * 8);
+    }
+    const uint32_t m = block_max_u32(a.bits(), smem);
+    if (threadIdx.x == 0) {
+        const uint32_t old = acc[blockIdx.x];
+        acc[blockIdx.x] = m > old ? m : old;
+    }
+}
+
 // ---------------------------------------------------------------- value ranges of small tensors
 // The smallest and the largest element of each of up to kRangeJobs tensors, and whether it holds
 // a NaN, one launch for all of them: a workgroup per 4096-element chunk of a tensor, three floats
@@ -787,6 +824,30 @@ extern "C" int mo_absmax_cols_noalloc(const void* x, int64_t outer, int64_t axis
         default: return MO_ERR_DTYPE;
     }
     if (rc != MO_OK) return rc;
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_absmax_blocks2d(const void* x, int64_t rows, int64_t cols, int64_t block_rows,
+                                  int64_t block_cols, int dtype, float* acc, void* stream) {
+    if (rows < 0 || cols < 0 || block_rows <= 0 || block_cols <= 0) return MO_ERR_ARG;
+    if (dtype < MO_F32 || dtype > MO_BF16) return MO_ERR_DTYPE;
+    if (rows == 0 || cols == 0) return MO_OK;
+    if (!x || !acc) return MO_ERR_ARG;
+    const int64_t tiles = (rows / block_rows) * (cols / block_cols);
+    if (rows % block_rows || cols % block_cols || block_cols % 8 || ((uintptr_t)x & 15u) ||
+        tiles > 0x7FFFFFFF || block_rows * (block_cols / 8) > 0x7FFFFFFF)
+        return MO_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+#define CALL(DT)                                                                               \
+    mo::absmax_blocks2d_kernel<DT><<<dim3((unsigned)tiles), 256, 0, s>>>(                      \
+        x, cols, (uint32_t)block_rows, (uint32_t)(block_cols / 8), (uint32_t)(cols / block_cols), \
+        (uint32_t*)acc)
+    switch (dtype) {
+        case MO_F32: CALL(MO_F32); break;
+        case MO_F16: CALL(MO_F16); break;
+        default: CALL(MO_BF16); break;
+    }
+#undef CALL
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }
 

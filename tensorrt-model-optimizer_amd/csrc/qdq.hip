@@ -141,6 +141,74 @@ __global__ __launch_bounds__(256) void qdq_cols_kernel(const void* __restrict__ 
     }
 }
 
+// Scales per two-dimensional block: x viewed as [rows, cols] with one amax per tile of
+// block_rows x block_cols elements, amax[(row / block_rows) * (cols / block_cols) + col /
+// block_cols] (block_cols % 8 == 0, so the 8 elements of a lane's chunk share a scale).  The same
+// tile walk as the CHUNK mode above: all loads first, one decision per chunk.
+template <int DT, bool FLAG, typename Op>
+__global__ __launch_bounds__(256) void qdq_blocks2d_kernel(const void* __restrict__ x,
+                                                           void* __restrict__ y, int64_t chunks,
+                                                           uint32_t row_chunks, uint32_t block_rows,
+                                                           uint32_t block_chunks,
+                                                           const void* __restrict__ amax,
+                                                           int amax_dtype, Op op) {
+    const int64_t c0 = (int64_t)blockIdx.x * kTileChunks + threadIdx.x;
+    const uint32_t blocks_across = row_chunks / block_chunks;
+    RawChunk<DT> raw[kQdqU];
+    float am[kQdqU];
+#pragma unroll
+    for (int u = 0; u < kQdqU; ++u) {
+        int64_t c = c0 + u * 256;
+        c = c < chunks ? c : chunks - 1;
+        load_raw<DT>(x, c << 3, raw[u]);
+        const int64_t row = c / row_chunks;
+        const uint32_t across = (uint32_t)(c - row * row_chunks) / block_chunks;
+        am[u] = load_scalar(amax, amax_dtype, (row / block_rows) * blocks_across + across);
+    }
+#pragma unroll
+    for (int u = 0; u < kQdqU; ++u) {
+        const int64_t c = c0 + u * 256;
+        float v[8];
+        unpack_raw<DT>(raw[u], v);
+        const typename Op::Scale s = op.make(am[u]);
+        if (Op::is_fast(s)) {
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) op.template apply2_fast<FLAG>(v[j], v[j + 1], s, s);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) op.template apply2<FLAG>(v[j], v[j + 1], s, s);
+        }
+        if (c < chunks) store_chunk<DT>(y, c << 3, v);
+    }
+}
+
+template <int DT, bool FLAG, typename Op>
+static int launch_qdq_blocks2d(const void* x, void* y, int64_t rows, int64_t cols, int64_t block_rows,
+                               int64_t block_cols, const void* amax, int amax_dtype, Op op,
+                               hipStream_t s) {
+    const int64_t chunks = rows * (cols >> 3);
+    const int64_t tiles = (chunks + kTileChunks - 1) / kTileChunks;
+    if (tiles > 0x7FFFFFFF) return MO_ERR_UNSUPPORTED;
+    qdq_blocks2d_kernel<DT, FLAG, Op><<<dim3((unsigned)tiles), 256, 0, s>>>(
+        x, y, chunks, (uint32_t)(cols >> 3), (uint32_t)block_rows, (uint32_t)(block_cols >> 3), amax,
+        amax_dtype, op);
+    return MO_OK;
+}
+
+// What the two-dimensional entry points accept: whole blocks (the caller pads), chunks of 8 that
+// stay inside a block, 16-byte aligned tensors.
+static int check_blocks2d(const void* x, const void* y, int64_t rows, int64_t cols, int64_t block_rows,
+                          int64_t block_cols, const void* amax, int amax_dtype) {
+    if (rows < 0 || cols < 0 || block_rows <= 0 || block_cols <= 0) return MO_ERR_ARG;
+    if (amax_dtype < MO_F32 || amax_dtype > MO_BF16) return MO_ERR_DTYPE;
+    if (rows == 0 || cols == 0) return MO_OK;
+    if (!x || !y || !amax) return MO_ERR_ARG;
+    if (rows % block_rows || cols % block_cols || block_cols % 8 || cols > 0x7FFFFFFFll ||
+        block_rows > 0x7FFFFFFFll || (((uintptr_t)x | (uintptr_t)y) & 15u))
+        return MO_ERR_UNSUPPORTED;
+    return MO_OK;
+}
+
 // Unaligned base pointers: same math, scalar accesses.
 template <int DT, bool FLAG, typename Op>
 __global__ __launch_bounds__(256) void qdq_scalar_kernel(const void* __restrict__ x,
@@ -358,6 +426,50 @@ extern "C" int mo_int_qdq(const void* x, void* y, int64_t outer, int64_t axis, i
         case MO_F32: rc = mo::launch_qdq<MO_F32, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s); break;
         case MO_F16: rc = mo::launch_qdq<MO_F16, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s); break;
         case MO_BF16: rc = mo::launch_qdq<MO_BF16, false>(x, y, outer, axis, inner, amax, amax_dtype, op, s); break;
+        default: return MO_ERR_DTYPE;
+    }
+    if (rc != MO_OK) return rc;
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_fp8_qdq_blocks2d(const void* x, void* y, int64_t rows, int64_t cols,
+                                   int64_t block_rows, int64_t block_cols, int dtype,
+                                   const void* amax, int amax_dtype, int saturate, void* stream) {
+    int rc = mo::check_blocks2d(x, y, rows, cols, block_rows, block_cols, amax, amax_dtype);
+    if (rc != MO_OK || rows == 0 || cols == 0) return rc;
+    hipStream_t s = (hipStream_t)stream;
+#define CALL(DT)                                                                                  \
+    rc = saturate ? mo::launch_qdq_blocks2d<DT, true>(x, y, rows, cols, block_rows, block_cols, amax, \
+                                                      amax_dtype, mo::Fp8Op<true>(), s)           \
+                  : mo::launch_qdq_blocks2d<DT, false>(x, y, rows, cols, block_rows, block_cols, amax, \
+                                                       amax_dtype, mo::Fp8Op<true>(), s)
+    switch (dtype) {
+        case MO_F32: CALL(MO_F32); break;
+        case MO_F16: CALL(MO_F16); break;
+        case MO_BF16: CALL(MO_BF16); break;
+        default: return MO_ERR_DTYPE;
+    }
+#undef CALL
+    if (rc != MO_OK) return rc;
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_int_qdq_blocks2d(const void* x, void* y, int64_t rows, int64_t cols,
+                                   int64_t block_rows, int64_t block_cols, int dtype,
+                                   const void* amax, int amax_dtype, int num_bits, int is_unsigned,
+                                   int narrow_range, void* stream) {
+    int rc = mo::check_blocks2d(x, y, rows, cols, block_rows, block_cols, amax, amax_dtype);
+    if (rc != MO_OK) return rc;
+    if (num_bits < 1 || num_bits > 24) return MO_ERR_ARG;
+    if (rows == 0 || cols == 0) return MO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    mo::IntOp op;
+    op.bound = (float)((1 << (num_bits - 1 + (is_unsigned ? 1 : 0))) - 1);
+    op.lo = is_unsigned ? 0.0f : (narrow_range ? -op.bound : -op.bound - 1.0f);
+    switch (dtype) {
+        case MO_F32: rc = mo::launch_qdq_blocks2d<MO_F32, false>(x, y, rows, cols, block_rows, block_cols, amax, amax_dtype, op, s); break;
+        case MO_F16: rc = mo::launch_qdq_blocks2d<MO_F16, false>(x, y, rows, cols, block_rows, block_cols, amax, amax_dtype, op, s); break;
+        case MO_BF16: rc = mo::launch_qdq_blocks2d<MO_BF16, false>(x, y, rows, cols, block_rows, block_cols, amax, amax_dtype, op, s); break;
         default: return MO_ERR_DTYPE;
     }
     if (rc != MO_OK) return rc;

@@ -54,6 +54,9 @@ SIGNATURES = {
     "mo_int4_block_quantize": [_P, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_int4_block_dequantize": [_P, _I64, _I64, _P, _P, _INT, _P],
     "mo_cast_fp4": [_P, _I64, _INT, _P, _P],
+    "mo_fp8_qdq_blocks2d": [_P, _P, _I64, _I64, _I64, _I64, _INT, _P, _INT, _INT, _P],
+    "mo_int_qdq_blocks2d": [_P, _P, _I64, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _INT, _P],
+    "mo_absmax_blocks2d": [_P, _I64, _I64, _I64, _I64, _INT, _P, _P],
     "mo_int4_pack_rows": [_P, _I64, _I64, _I64, _I64, _INT, _P, _P, _P],
     "mo_int4_pack_rows_via": [_P, _I64, _I64, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_nf4_quantize": [_P, _I64, _I64, _INT, _P, _P, _P],
@@ -330,6 +333,43 @@ def int_qdq(x, amax, outer, axis, inner, num_bits, unsigned, narrow_range, out=N
          dtype_code(amax.dtype), int(num_bits), int(bool(unsigned)), int(bool(narrow_range)),
          _stream(x))
     return y
+
+
+def blocks2d_covered(x, rows, cols, block_rows, block_cols) -> bool:
+    """Whether the two-dimensional block kernels take ``x`` viewed as [rows, cols]."""
+    return (rows > 0 and cols > 0 and rows % block_rows == 0 and cols % block_cols == 0
+            and block_cols % 8 == 0 and x.data_ptr() % 16 == 0 and x.is_contiguous())
+
+
+def fp8_qdq_blocks2d(x, amax, rows, cols, block_rows, block_cols, saturate=False):
+    """FP8 fake quant of contiguous ``x`` seen as [rows, cols] with one amax per block of
+    ``block_rows x block_cols`` (``amax`` flat, block rows major)."""
+    _require_device(x, amax)
+    assert x.is_contiguous() and amax.is_contiguous() and x.numel() == rows * cols
+    y = torch.empty_like(x)
+    call("mo_fp8_qdq_blocks2d", x, _ptr(x), _ptr(y), rows, cols, block_rows, block_cols,
+         dtype_code(x.dtype), _ptr(amax), dtype_code(amax.dtype), int(saturate), _stream(x))
+    return y
+
+
+def int_qdq_blocks2d(x, amax, rows, cols, block_rows, block_cols, num_bits, unsigned, narrow_range):
+    _require_device(x, amax)
+    assert x.is_contiguous() and amax.is_contiguous() and x.numel() == rows * cols
+    y = torch.empty_like(x)
+    call("mo_int_qdq_blocks2d", x, _ptr(x), _ptr(y), rows, cols, block_rows, block_cols,
+         dtype_code(x.dtype), _ptr(amax), dtype_code(amax.dtype), int(num_bits), int(bool(unsigned)),
+         int(bool(narrow_range)), _stream(x))
+    return y
+
+
+def absmax_blocks2d_into(x, acc, rows, cols, block_rows, block_cols):
+    """``acc[b] = max(acc[b], abs-max of block b)``, fp32 ``acc`` with one element per block."""
+    _require_device(x, acc)
+    assert x.is_contiguous() and acc.dtype == torch.float32 and acc.is_contiguous()
+    assert acc.numel() == (rows // block_rows) * (cols // block_cols)
+    call("mo_absmax_blocks2d", x, _ptr(x), rows, cols, block_rows, block_cols, dtype_code(x.dtype),
+         _ptr(acc), _stream(x))
+    return acc
 
 
 def nvfp4_qdq(x, amax, block_size=16, mode=0, out=None):

@@ -114,6 +114,14 @@ def reduce_amax_gpu(x: torch.Tensor, reduce_dims, keepdims=True, reread: bool = 
             x.shape[d] for d in keep)
     layout = amax_layout(tuple(x.shape), keep)
     src = x
+    if layout is None and x.is_cuda and x.is_contiguous():
+        # one abs-max per two-dimensional block of a matrix: a workgroup per block, no transposed copy
+        blocks = blocks2d_of(tuple(x.shape), keep)
+        if blocks is not None and _hip.blocks2d_covered(x, *blocks):
+            rows, cols, block_rows, block_cols = blocks
+            acc = torch.zeros((rows // block_rows) * (cols // block_cols), dtype=torch.float32, device=x.device)
+            _hip.absmax_blocks2d_into(x, acc, rows, cols, block_rows, block_cols)
+            return acc.to(x.dtype).reshape(out_shape)
     if layout is None:
         src, _, layout = kept_dims_first(x, keep)
     acc = torch.zeros(layout[1], dtype=torch.float32, device=x.device)
@@ -125,9 +133,25 @@ def _qdq_layout(x, amax):
     return layout_from_amax_shape(tuple(x.shape), tuple(amax.shape))
 
 
-def _qdq(x, amax, run):
+def blocks2d_of(shape, kept) -> tuple | None:
+    """``(rows, cols, block_rows, block_cols)`` when a contiguous tensor of ``shape`` whose scale
+    dims are ``kept`` (a sorted list) is a matrix cut into two-dimensional blocks: the reshape
+    ``[..., R, block_rows, C, block_cols]`` of ``[..., R * block_rows, C * block_cols]`` with a
+    scale for every index of all dims but the two block dims (what a quantizer with block sizes
+    on the last two dims sets up).  None otherwise."""
+    nd = len(shape)
+    if nd < 4 or list(kept) != [d for d in range(nd) if d not in (nd - 3, nd - 1)]:
+        return None
+    block_rows, block_cols = shape[nd - 3], shape[nd - 1]
+    rows = math.prod(shape[:nd - 3]) * block_rows
+    return rows, shape[nd - 2] * block_cols, block_rows, block_cols
+
+
+def _qdq(x, amax, run, run2d=None):
     """``run(x2, amax_flat, outer, axis, inner)`` on ``x`` as it is when the amax spans one run
-    of dims, else on a copy with the amax dims moved to the front (and moved back afterwards)."""
+    of dims; ``run2d(x, amax_flat, rows, cols, block_rows, block_cols)`` when the amax is per
+    two-dimensional block of a matrix; else ``run`` on a copy with the amax dims moved to the
+    front (and moved back afterwards)."""
     x = x if x.is_contiguous() else x.contiguous()
     layout = _qdq_layout(x, amax)
     if layout is not None:
@@ -135,6 +159,10 @@ def _qdq(x, amax, run):
     if amax.dim() != x.dim() or any(a not in (1, s) for a, s in zip(amax.shape, x.shape)):
         raise NotImplementedError(
             f"amax of shape {tuple(amax.shape)} does not broadcast against input {tuple(x.shape)}")
+    if run2d is not None and x.is_cuda:
+        blocks = blocks2d_of(tuple(x.shape), [d for d in range(x.dim()) if amax.shape[d] != 1])
+        if blocks is not None and _hip.blocks2d_covered(x, *blocks):
+            return run2d(x, amax.reshape(-1).contiguous(), *blocks)
     keep = [d for d in range(x.dim()) if amax.shape[d] != 1]
     xp, perm, layout = kept_dims_first(x, keep)
     y = run(xp, amax.reshape(-1).contiguous(), *layout)
@@ -146,7 +174,9 @@ with_scale_layout = _qdq   # the storage casts place their scales the same way
 
 def fake_quant_int(x, amax, num_bits=8, unsigned=False, narrow_range=True):
     return _qdq(x, amax, lambda x2, a, outer, axis, inner: _hip.int_qdq(
-        x2, a, outer, axis, inner, num_bits, unsigned, narrow_range))
+        x2, a, outer, axis, inner, num_bits, unsigned, narrow_range),
+        lambda x2, a, rows, cols, br, bc: _hip.int_qdq_blocks2d(
+            x2, a, rows, cols, br, bc, num_bits, unsigned, narrow_range))
 
 
 def fake_quant_fp8(x, amax=None, saturate=False):
@@ -154,7 +184,8 @@ def fake_quant_fp8(x, amax=None, saturate=False):
         x = x if x.is_contiguous() else x.contiguous()
         return _hip.fp8_qdq(x, None, 1, 1, x.numel(), saturate)
     return _qdq(x, amax, lambda x2, a, outer, axis, inner: _hip.fp8_qdq(
-        x2, a, outer, axis, inner, saturate))
+        x2, a, outer, axis, inner, saturate),
+        lambda x2, a, rows, cols, br, bc: _hip.fp8_qdq_blocks2d(x2, a, rows, cols, br, bc, saturate))
 
 
 def fake_quant_nvfp4(x, global_amax, block_size=16, mode=0):

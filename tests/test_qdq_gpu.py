@@ -195,3 +195,48 @@ def test_two_axis_block_fake_quant_through_the_quantizer(num_bits, shape, blocks
         want = fake_quant.fp8_eager(tiles, amax)
     want = want.reshape(pad.shape)[: shape[0], : shape[1]]
     assert_bits_equal(got, want, "2-D block fake quant")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("lead,rows,cols,br,bc", [((), 256, 384, 128, 128), ((), 192, 320, 64, 32),
+                                                   ((), 48, 64, 16, 8), ((3,), 128, 256, 64, 128),
+                                                   ((), 1024, 4096, 128, 128)])
+def test_two_dimensional_blocks(dtype, lead, rows, cols, br, bc, monkeypatch):
+    """An amax per (br x bc) block of a matrix -- the reshape ``[R, br, C, bc]`` with the amax on
+    dims 0 and 2 that block sizes on the last two dims set up (reference: tensor_quantizer.py
+    :755-782) -- through the block abs-max and the FP8 / INT fake quant without a transposed copy:
+    against the CPU restatement on the same 4-D view, and the binding's refusals."""
+    from modelopt_amd.torch.quantization import kernels
+
+    g = torch.Generator().manual_seed(rows + cols + br)
+    x = (torch.randn(*lead, rows, cols, generator=g) * 0.05).to(dtype)
+    x.view(-1)[::97] *= 8
+    x[..., :br, :bc] = 0.0                                     # an all-zero block
+    x4 = x.reshape(*lead, rows // br, br, cols // bc, bc)
+    dims = (x4.dim() - 3, x4.dim() - 1)
+    taken = []
+    for name in ("absmax_blocks2d_into", "fp8_qdq_blocks2d", "int_qdq_blocks2d"):
+        real = getattr(_hip, name)
+        monkeypatch.setattr(_hip, name, lambda *a, _real=real, _name=name: taken.append(_name) or _real(*a))
+    want_amax = reduce.reduce_amax(x4, axis=list(dims))
+    got_amax = kernels.reduce_amax_gpu(x4.to(DEV), dims)
+    assert got_amax.shape == want_amax.shape
+    assert_bits_equal(got_amax.cpu(), want_amax, "block abs-max")
+    amax = want_amax.clone()
+    amax[amax == 0] = 1.0
+    clipped = amax * 0.5                                       # half of the blocks' range clips
+    for a, what in ((amax, "amax"), (clipped, "half the amax")):
+        got = kernels.fake_quant_fp8(x4.to(DEV), a.to(DEV), saturate=True)
+        want = fake_quant.fp8_eager(x4.clamp(-a, a) if a is clipped else x4, a)
+        assert_bits_equal(got.cpu(), want, f"fp8, {what}")
+        for bits, narrow in ((8, False), (4, True)):
+            got = kernels.fake_quant_int(x4.to(DEV), a.to(DEV), bits, False, narrow)
+            assert_bits_equal(got.cpu(), fake_quant.tensor_quant(x4, a, bits, False, narrow), f"int{bits}, {what}")
+    assert taken == ["absmax_blocks2d_into"] + ["fp8_qdq_blocks2d", "int_qdq_blocks2d", "int_qdq_blocks2d"] * 2
+    # what the kernels do not take goes the long way round and gives the same
+    odd = x4[..., 1:].contiguous() if bc > 8 else None
+    if odd is not None:
+        a_odd = reduce.reduce_amax(odd, axis=list(dims))
+        a_odd[a_odd == 0] = 1.0
+        assert_bits_equal(kernels.fake_quant_int(odd.to(DEV), a_odd.to(DEV), 8, False, False).cpu(),
+                          fake_quant.tensor_quant(odd, a_odd, 8, False, False), "block width not a multiple of 8")
