@@ -361,6 +361,20 @@ int mo_real_quantize(const void* x, int64_t outer, int64_t axis, int64_t inner, 
 int mo_real_dequantize(const uint8_t* q, int64_t outer, int64_t axis, int64_t inner, int format,
                        const void* scale, int scale_dtype, void* y, int dtype, void* stream);
 
+/* The two storage casts with one scale per two-dimensional block: x / q / y viewed as [rows, cols],
+ * scale[(row / block_rows) * (cols / block_cols) + col / block_cols] -- FP8QTensor.quantize /
+ * dequantize with block_sizes on two dims (TQ/qtensor/fp8_tensor.py:64-112 expands the scales with
+ * repeat_interleave; :115-151), the weight-compress path of FP8_2D_BLOCKWISE_WEIGHT_ONLY_CFG and its
+ * dequantize-on-forward.  rows % block_rows == 0, cols % block_cols == 0 (the caller pads and
+ * crops), block_cols % 8 == 0, x / y 16-byte and q / out 8-byte aligned: MO_ERR_UNSUPPORTED
+ * otherwise.  Arguments otherwise as in mo_real_quantize / mo_real_dequantize. */
+int mo_real_quantize_blocks2d(const void* x, int64_t rows, int64_t cols, int64_t block_rows,
+                              int64_t block_cols, int dtype, const void* scale, int scale_dtype,
+                              int via_dtype, int format, uint8_t* out, void* stream);
+int mo_real_dequantize_blocks2d(const uint8_t* q, int64_t rows, int64_t cols, int64_t block_rows,
+                                int64_t block_cols, int format, const void* scale, int scale_dtype,
+                                void* y, int dtype, void* stream);
+
 /* ------------------------------------------------------------------ INT4 weight compression
  * Flat blocks of block_size elements over the n elements of x (tail zero padded).
  * scales[b] = T(f32(T(1 / amax_b)) * 7) (what torch computes for `7 / amax` in dtype T),

@@ -110,7 +110,13 @@ __device__ __forceinline__ void chunk_scale_indices(int64_t c0, int64_t chunks, 
 //                    the flat tensor as in the per-tensor case (no half-empty tiles on
 //                    4096-wide rows), and the 256 chunks of a round lie inside one row, so the
 //                    scale of a round is wavefront-uniform
-constexpr int kScalePerTensor = 0, kScalePerRowTile = 1, kScalePerChunk = 2, kScalePerRound = 3;
+//   kScalePerBlock2d one scale per two-dimensional block of a matrix: `inner_chunks` is the
+//                    length of a matrix row in chunks, `axis` the rows of a block and
+//                    `tiles_per_row` the chunks across a block; the scale of the chunk at
+//                    (row, col) is scale[(row / axis) * (inner_chunks / tiles_per_row) + col /
+//                    tiles_per_row]
+constexpr int kScalePerTensor = 0, kScalePerRowTile = 1, kScalePerChunk = 2, kScalePerRound = 3,
+              kScalePerBlock2d = 4;
 
 // chunk index, validity and scale of the lane's 4 chunks.  A chunk past the end gets the index
 // of the last valid one and ok = false: the kernels load it like any other (all loads in
@@ -154,6 +160,13 @@ __device__ __forceinline__ void tile_layout(int64_t chunks, int64_t axis, int64_
                 sv[u] = load_scalar(scale, scale_dtype, row < axis ? row : row % axis);
                 col += 256;
                 if (col >= inner_chunks) { col -= inner_chunks; ++row; }
+            }
+        } else if constexpr (SCALES == kScalePerBlock2d) {
+            const int64_t across = inner_chunks / tiles_per_row;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int64_t row = c[u] / inner_chunks, col = c[u] - row * inner_chunks;
+                sv[u] = load_scalar(scale, scale_dtype, (row / axis) * across + col / tiles_per_row);
             }
         } else {
             int64_t idx[4];
@@ -208,7 +221,7 @@ __global__ __launch_bounds__(256) void real_quantize_tile_kernel(
         } else {
             // the correctly rounded reciprocal (an IEEE division) is taken again only when the
             // scale changes
-            if (SCALES != kScalePerChunk || u == 0 || f2u(s) != f2u(sv[u - 1])) rv = 1.0f / s;
+            if ((SCALES != kScalePerChunk && SCALES != kScalePerBlock2d) || u == 0 || f2u(s) != f2u(sv[u - 1])) rv = 1.0f / s;
             r = rv;
         }
         uint32_t m = 0;
@@ -750,6 +763,68 @@ extern "C" int mo_real_dequantize(const uint8_t* q, int64_t outer, int64_t axis,
         mo::real_dequantize_kernel<DT, 1><<<g, 256, 0, s>>>(q, n, axis, inner, scale, scale_dtype, y)
     DISPATCH_DT(dtype, CALL)
 #undef CALL
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+// Storage casts with one scale per two-dimensional block (block sizes on the last two dims).
+static int check_real_blocks2d(const void* a, const void* b, const void* scale, int64_t rows, int64_t cols,
+                               int64_t block_rows, int64_t block_cols, int format, int scale_dtype) {
+    if (rows < 0 || cols < 0 || block_rows <= 0 || block_cols <= 0) return MO_ERR_ARG;
+    if (format != MO_FMT_E4M3 && format != MO_FMT_INT8) return MO_ERR_UNSUPPORTED;
+    if (scale_dtype < MO_F32 || scale_dtype > MO_BF16) return MO_ERR_DTYPE;
+    if (rows == 0 || cols == 0) return MO_OK;
+    if (!a || !b || !scale) return MO_ERR_ARG;
+    if (rows % block_rows || cols % block_cols || block_cols % 8 ||
+        (rows * (cols / 8) + mo::kRealTileChunks - 1) / mo::kRealTileChunks > 0x7FFFFFFF)
+        return MO_ERR_UNSUPPORTED;
+    return MO_OK;
+}
+
+extern "C" int mo_real_quantize_blocks2d(const void* x, int64_t rows, int64_t cols, int64_t block_rows,
+                                         int64_t block_cols, int dtype, const void* scale,
+                                         int scale_dtype, int via_dtype, int format, uint8_t* out,
+                                         void* stream) {
+    int rc = check_real_blocks2d(x, out, scale, rows, cols, block_rows, block_cols, format, scale_dtype);
+    if (rc != MO_OK || rows == 0 || cols == 0) return rc;
+    if (via_dtype < MO_F32 || via_dtype > MO_BF16) return MO_ERR_DTYPE;
+    if (((uintptr_t)x & 15u) || ((uintptr_t)out & 7u)) return MO_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t chunks = rows * (cols / 8);
+    const unsigned gt = (unsigned)((chunks + mo::kRealTileChunks - 1) / mo::kRealTileChunks);
+#define TILE4(DT, VIA, FMT)                                                                        \
+    mo::real_quantize_tile_kernel<DT, VIA, FMT, mo::kScalePerBlock2d><<<gt, 256, 0, s>>>(          \
+        x, chunks, block_rows, cols / 8, block_cols / 8, scale, scale_dtype, (mo::u32x2*)out)
+#define CALL3(DT, VIA) \
+    if (format == MO_FMT_E4M3) { TILE4(DT, VIA, 0); } else { TILE4(DT, VIA, 1); }
+#define CALL(DT)                                            \
+    if (via_dtype == MO_F32) { CALL3(DT, MO_F32); }         \
+    else if (via_dtype == MO_F16) { CALL3(DT, MO_F16); }    \
+    else { CALL3(DT, MO_BF16); }
+    DISPATCH_DT(dtype, CALL)
+#undef CALL
+#undef CALL3
+#undef TILE4
+    return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
+}
+
+extern "C" int mo_real_dequantize_blocks2d(const uint8_t* q, int64_t rows, int64_t cols,
+                                           int64_t block_rows, int64_t block_cols, int format,
+                                           const void* scale, int scale_dtype, void* y, int dtype,
+                                           void* stream) {
+    int rc = check_real_blocks2d(q, y, scale, rows, cols, block_rows, block_cols, format, scale_dtype);
+    if (rc != MO_OK || rows == 0 || cols == 0) return rc;
+    if (((uintptr_t)y & 15u) || ((uintptr_t)q & 7u)) return MO_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t chunks = rows * (cols / 8);
+    const unsigned gt = (unsigned)((chunks + mo::kRealTileChunks - 1) / mo::kRealTileChunks);
+#define TILE3(DT, FMT)                                                                             \
+    mo::real_dequantize_tile_kernel<DT, FMT, mo::kScalePerBlock2d><<<gt, 256, 0, s>>>(             \
+        (const mo::u32x2*)q, chunks, block_rows, cols / 8, block_cols / 8, scale, scale_dtype, y)
+#define CALL(DT) \
+    if (format == MO_FMT_E4M3) { TILE3(DT, 0); } else { TILE3(DT, 1); }
+    DISPATCH_DT(dtype, CALL)
+#undef CALL
+#undef TILE3
     return hipGetLastError() == hipSuccess ? MO_OK : MO_ERR_LAUNCH;
 }
 

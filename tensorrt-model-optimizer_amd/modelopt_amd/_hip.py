@@ -57,6 +57,8 @@ SIGNATURES = {
     "mo_fp8_qdq_blocks2d": [_P, _P, _I64, _I64, _I64, _I64, _INT, _P, _INT, _INT, _P],
     "mo_int_qdq_blocks2d": [_P, _P, _I64, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _INT, _P],
     "mo_absmax_blocks2d": [_P, _I64, _I64, _I64, _I64, _INT, _P, _P],
+    "mo_real_quantize_blocks2d": [_P, _I64, _I64, _I64, _I64, _INT, _P, _INT, _INT, _INT, _P, _P],
+    "mo_real_dequantize_blocks2d": [_P, _I64, _I64, _I64, _I64, _INT, _P, _INT, _P, _INT, _P],
     "mo_int4_pack_rows": [_P, _I64, _I64, _I64, _I64, _INT, _P, _P, _P],
     "mo_int4_pack_rows_via": [_P, _I64, _I64, _I64, _I64, _INT, _P, _INT, _P, _P],
     "mo_nf4_quantize": [_P, _I64, _I64, _INT, _P, _P, _P],
@@ -616,6 +618,29 @@ def real_quantize(x, scale, outer, axis, inner, via_dtype, fmt):
     call("mo_real_quantize", x, _ptr(x), outer, axis, inner, dtype_code(x.dtype), _ptr(scale),
          dtype_code(scale.dtype), dtype_code(via_dtype), fmt, _ptr(out), _stream(x))
     return out.view(torch.float8_e4m3fn if fmt == MO_FMT_E4M3 else torch.int8)
+
+
+def real_quantize_blocks2d(x, scale, rows, cols, block_rows, block_cols, via_dtype, fmt):
+    """``fmt(via(x / scale[block]))`` for contiguous ``x`` seen as [rows, cols] with one scale per
+    block of ``block_rows x block_cols`` (flat, block rows major); uint8 bytes of x's shape viewed
+    as float8_e4m3fn or int8."""
+    _require_device(x, scale)
+    assert x.is_contiguous() and scale.is_contiguous() and x.numel() == rows * cols
+    assert scale.numel() == (rows // block_rows) * (cols // block_cols)
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    call("mo_real_quantize_blocks2d", x, _ptr(x), rows, cols, block_rows, block_cols, dtype_code(x.dtype),
+         _ptr(scale), dtype_code(scale.dtype), dtype_code(via_dtype), fmt, _ptr(out), _stream(x))
+    return out.view(torch.float8_e4m3fn if fmt == MO_FMT_E4M3 else torch.int8)
+
+
+def real_dequantize_blocks2d(q, scale, rows, cols, block_rows, block_cols, fmt, dtype):
+    _require_device(q, scale)
+    assert q.is_contiguous() and scale.is_contiguous() and q.numel() == rows * cols
+    assert scale.numel() == (rows // block_rows) * (cols // block_cols)
+    y = torch.empty(q.shape, dtype=dtype, device=q.device)
+    call("mo_real_dequantize_blocks2d", q, _ptr(q.view(torch.uint8)), rows, cols, block_rows, block_cols,
+         fmt, _ptr(scale), dtype_code(scale.dtype), _ptr(y), dtype_code(dtype), _stream(q))
+    return y
 
 
 def real_dequantize(q, scale, outer, axis, inner, fmt, dtype):

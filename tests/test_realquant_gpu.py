@@ -111,12 +111,20 @@ def test_qtensor_golden_vectors_through_the_quantizer(case):
 
 @pytest.mark.parametrize("fmt", ["fp8", "int8"])
 @pytest.mark.parametrize("shape,blocks", [((256, 384), {-1: 128, -2: 128}), ((100, 200), {-1: 64, -2: 32}),
-                                           ((3, 40, 96), {-1: 32}), ((130, 70), {-1: 16})])
-def test_block_scales_on_any_dims_match_restatement(fmt, shape, blocks):
+                                           ((3, 40, 96), {-1: 32}), ((130, 70), {-1: 16}),
+                                           ((2, 128, 256), {-1: 128, -2: 64}), ((3, 50, 72), {-1: 24, -2: 16}),
+                                           ((64, 96), {-1: 12, -2: 16})])
+def test_block_scales_on_any_dims_match_restatement(fmt, shape, blocks, monkeypatch):
     """2-D tiles, padding on either dim, 3-D inputs: codes, scales and dequantised values equal
-    the CPU restatement of the reference's pad / repeat_interleave formulation bit for bit."""
+    the CPU restatement of the reference's pad / repeat_interleave formulation bit for bit.
+    Tiles on the last two dims whose width is a multiple of 8 are cast in place (no copy that
+    gathers every tile into a row)."""
     from modelopt_amd.torch.quantization.qtensor import FP8QTensor, INT8QTensor
 
+    in_place = []
+    for name in ("real_quantize_blocks2d", "real_dequantize_blocks2d"):
+        real = getattr(_hip, name)
+        monkeypatch.setattr(_hip, name, lambda *a, _real=real, _name=name: in_place.append(_name) or _real(*a))
     x = _rand(shape, torch.bfloat16, 21, scale=1.0)
     if fmt == "fp8":
         q_o, s_o = qtensor.fp8_quantize(x, block_sizes=blocks)
@@ -130,6 +138,8 @@ def test_block_scales_on_any_dims_match_restatement(fmt, shape, blocks):
     assert_bits_equal(qt._quantized_data.cpu(), q_o, "codes")
     got = qt.dequantize(scale=s, block_sizes=blocks)
     assert_bits_equal(got.cpu(), want, "dequantised")
+    tiled = len(blocks) == 2 and blocks[-1] % 8 == 0
+    assert in_place == (["real_quantize_blocks2d", "real_dequantize_blocks2d"] if tiled else [])
 
 
 # ----------------------------------------------------------------------------- INT8 / INT4
